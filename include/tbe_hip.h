@@ -1,0 +1,189 @@
+/*
+ * tbe_hip.h -- C ABI of the MI355X (gfx950) table-batched embedding-bag library.
+ *
+ * Every entry point takes plain device pointers, sizes and an opaque HIP stream
+ * (a hipStream_t passed as void*; NULL = the default stream).  Nothing here
+ * allocates device memory: scratch is a caller-owned workspace whose size is
+ * reported by the *_workspace_* queries.  No entry point synchronises the host
+ * with the device.
+ *
+ * Return value: 0 (TBE_OK) on success, a TBE_ERR_* code otherwise; the message
+ * of the last failure on the calling thread is returned by tbe_last_error().
+ * This mirrors the reference's AT_ASSERT / AT_CUDA_CHECK -> RuntimeError
+ * behaviour (table_batched_embeddings_cuda.cu:262-273, 314): the Python host
+ * turns a non-zero code into RuntimeError.
+ *
+ * Layout conventions (table_batched_embeddings_cuda.cu:193-222):
+ *   weights        [total_rows][D], row-major, element type `dtype`
+ *   table_offsets  int32 [T]     first row of each table inside `weights`
+ *   indices        int32 [N]     table-major: all bags of table 0, then table 1...
+ *   offsets        int32 [T*B+1] bag (t,b) owns indices[offsets[t*B+b] : offsets[t*B+b+1]]
+ *   output / grad  [B][T][D]     bag-major, element type `dtype`
+ *   D % 4 == 0.
+ */
+#ifndef TBE_HIP_H
+#define TBE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Exported symbols; everything else in the library has hidden visibility. */
+#define TBE_API __attribute__((visibility("default")))
+
+/* element type of weights / outputs / gradients / per-sample weights */
+enum { TBE_DTYPE_F32 = 0, TBE_DTYPE_F16 = 1, TBE_DTYPE_F64 = 2 };
+
+enum {
+  TBE_OK = 0,
+  TBE_ERR_INVALID = 1,     /* a shape / pointer / dtype precondition failed */
+  TBE_ERR_WORKSPACE = 2,   /* workspace pointer NULL or too small           */
+  TBE_ERR_HIP = 3,         /* a HIP runtime call or kernel launch failed    */
+  TBE_ERR_UNSUPPORTED = 4  /* a valid request this library does not serve   */
+};
+
+/* Message of the last error raised on this thread ("" if none). */
+TBE_API const char *tbe_last_error(void);
+
+/* ABI version; bumped whenever a signature below changes. */
+TBE_API int32_t tbe_abi_version(void);
+
+/* ------------------------------------------------------------------ forward
+ * Pooled gather-sum:  output[b][t][:] = sum_{p in bag(t,b)} (psw[p] *) weights[table_offsets[t] + indices[p]][:]
+ * Replaces batched_embedding_forward_cuda (table_batched_embeddings_cuda.cu:253-316,
+ * bound as "forward" in table_batched_embeddings.cpp:58).  `per_sample_weights`
+ * may be NULL (unweighted); otherwise it has `dtype` elements and length N.
+ * Accumulation is fp32 for F16/F32 and fp64 for F64; the result is rounded to
+ * nearest-even once.  An empty bag yields zeros.  The reference's launch knobs
+ * (L_max, BT_block_size, shmem) do not exist here.
+ */
+TBE_API int tbe_forward(const void *weights, int32_t dtype, int32_t D,
+                const int32_t *table_offsets, int32_t T,
+                const int32_t *indices, int64_t num_indices,
+                const int32_t *offsets, int32_t B,
+                const void *per_sample_weights,
+                void *output, void *stream);
+
+/* ----------------------------------------------------------------- backward
+ * Byte offsets of the regions of the backward workspace.  After a backward call
+ * the first five regions hold the intermediate results that the parity gates
+ * inspect (all int32):
+ *   keys              [N]   table_offsets[t] + indices[p]             (tbe.cu:1495)
+ *   keys_sorted       [N]   stable ascending sort of keys             (tbe.cu:1639-1655)
+ *   positions_sorted  [N]   position p of each sorted key (IndexInfo.indices_idx, tbe.cu:1217)
+ *   segment_starts    [U+1] first sorted position of each unique key, then N (tbe.cu:1523-1539)
+ *   num_unique        [1]   U
+ */
+typedef struct tbe_workspace_layout {
+  uint64_t total_bytes;
+  uint64_t keys;
+  uint64_t grad_rows;        /* int32 [N]: b*T + t of the bag owning position p        */
+  uint64_t keys_sorted;
+  uint64_t positions_sorted;
+  uint64_t segment_starts;
+  uint64_t num_unique;       /* int32 [4]: U, #long segments, #long chunks, reserved   */
+  uint64_t sort_scratch;
+  uint64_t segment_scratch;
+  uint64_t long_segments;    /* int32 [2][max_long]: segment id, first chunk           */
+  uint64_t chunk_segments;   /* int32 [max_chunks]: owning long-segment slot           */
+  uint64_t partial_sums;     /* accumulator-typed [max_chunks][D]                       */
+  int64_t max_long_segments;
+  int64_t max_chunks;
+} tbe_workspace_layout_t;
+
+TBE_API int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int32_t dtype,
+                                  tbe_workspace_layout_t *layout);
+
+/* Exact SGD:  weights[r][:] -= lr * sum_{p: key[p]==r} grad_output[b(p)][t(p)][:]
+ * once per distinct row r, with no atomics and a fixed summation order
+ * (ascending position).  Replaces batched_embedding_backward_sgd_cuda
+ * (table_batched_embeddings_cuda.cu:383-435, "backward_sgd" in
+ * table_batched_embeddings.cpp:59), whose per-lookup read-modify-write is only
+ * correct when no row repeats (test_table_batched_embeddings.py:177-193).
+ * `total_rows` is the row count of `weights`; it fixes the number of key bits
+ * sorted, as optimizer_state.numel() does at tbe.cu:1643.
+ */
+TBE_API int tbe_backward_sgd(const void *grad_output, void *weights, int32_t dtype,
+                     int64_t total_rows, int32_t D,
+                     const int32_t *table_offsets, int32_t T,
+                     const int32_t *indices, int64_t num_indices,
+                     const int32_t *offsets, int32_t B,
+                     float learning_rate,
+                     void *workspace, uint64_t workspace_bytes, void *stream);
+
+/* Exact row-wise Adagrad (table_batched_embeddings_cuda.cu:1589-1706 with
+ * AdaGradFunctor, :437-471; "backward_exact_adagrad" in table_batched_embeddings.cpp:61):
+ *   G = sum over the occurrences of row r of (psw[p] *) grad_output[b(p)][t(p)][:]
+ *   state[r] += sum_d G_d^2 ;  weights[r][:] -= lr / (sqrt(state[r]) + eps) * G
+ * `optimizer_state` is float [total_rows] for F16/F32 weights, double for F64.
+ * When `per_sample_weights` is non-NULL, `grad_per_sample_weights` (same dtype,
+ * length N) receives <weights_before_update[row(p)], grad_output[b(p)][t(p)]>,
+ * the quantity the reference's weighted functor accumulates (tbe.cu:529-553);
+ * the reference leaves the weighted exact case unimplemented (tbe.cu:1552, 1678).
+ */
+TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, int32_t dtype,
+                               int64_t total_rows, int32_t D,
+                               const int32_t *table_offsets, int32_t T,
+                               const int32_t *indices, int64_t num_indices,
+                               const int32_t *offsets, int32_t B,
+                               const void *per_sample_weights,
+                               void *optimizer_state,
+                               float learning_rate, float eps,
+                               void *grad_per_sample_weights,
+                               void *workspace, uint64_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------- stages, individually callable
+ * The backward entry points run exactly these stages on the caller's workspace.
+ */
+
+/* keys[p] = table_offsets[t] + indices[p]; grad_rows[p] = b*T + t
+ * (linear_index_weight_offsets_kernel, table_batched_embeddings_cuda.cu:1471-1497;
+ * IndexInfo.b_t = t*B + b is recoverable from grad_rows, indices_idx is p itself). */
+TBE_API int tbe_linearize(const int32_t *table_offsets, int32_t T,
+                  const int32_t *indices, int64_t num_indices,
+                  const int32_t *offsets, int32_t B,
+                  int32_t *keys, int32_t *grad_rows, void *stream);
+
+/* Stable ascending LSD radix sort of (key, value) pairs on key bits [0, end_bit),
+ * the contract of cub::DeviceRadixSort::SortPairs at
+ * table_batched_embeddings_cuda.cu:1639-1655.  values_in == NULL sorts the
+ * identity permutation (values_out = stable argsort).  Inputs are not modified. */
+TBE_API uint64_t tbe_sort_workspace_bytes(int64_t n);
+TBE_API int tbe_sort_pairs(const int32_t *keys_in, const int32_t *values_in,
+                   int32_t *keys_out, int32_t *values_out,
+                   int64_t n, int32_t end_bit,
+                   void *workspace, uint64_t workspace_bytes, void *stream);
+
+/* Run boundaries of a sorted key array: segment_starts[u] = first i with the
+ * u-th distinct key, segment_starts[U] = n, *num_unique = U (device memory).
+ * Same rule as the segment-head test at table_batched_embeddings_cuda.cu:1523-1539. */
+TBE_API uint64_t tbe_segments_workspace_bytes(int64_t n);
+TBE_API int tbe_find_segments(const int32_t *keys_sorted, int64_t n,
+                      int32_t *segment_starts, int32_t *num_unique,
+                      void *workspace, uint64_t workspace_bytes, void *stream);
+
+/* output[0] = 0; output[1 + t*B + b] = length of bag (t,b) given per-table bag
+ * starts [T][B] and per-table totals [T]; the caller cumsums
+ * (construct_offsets, table_batched_embeddings_cuda.cu:1165-1213,
+ * table_batched_embeddings.cpp:67). */
+TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
+                          const int32_t *total_indices_per_table,
+                          int32_t T, int32_t B, int32_t *output, void *stream);
+
+/* ------------------------------------------------------ host-resident tables
+ * Pinned, device-mapped host memory (new_host_mapped_tensor,
+ * table_batched_embeddings_cuda.cu:820-880) and managed memory preferring the
+ * host (new_managed_tensor, :797-871).  *device_ptr is the address kernels use.
+ */
+TBE_API int tbe_host_mapped_alloc(uint64_t bytes, void **host_ptr, void **device_ptr);
+TBE_API int tbe_host_mapped_free(void *host_ptr);
+TBE_API int tbe_managed_alloc(uint64_t bytes, int32_t device, void **ptr);
+TBE_API int tbe_managed_free(void *ptr);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TBE_HIP_H */

@@ -1,0 +1,137 @@
+"""numpy-facing wrapper of the C oracle (oracle/tbe_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py as the checker.  The shipped package never imports it.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtbe_oracle.so")
+_lib = None
+
+F32, F16, F64 = 0, 1, 2
+_CODES = {np.dtype(np.float32): F32, np.dtype(np.float16): F16, np.dtype(np.float64): F64}
+
+
+def build():
+    subprocess.run(["make", "-s", "-B", "-C", _HERE, "libtbe_oracle.so"], check=True)
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.oracle_half_to_float.restype = ctypes.c_float
+        _lib.oracle_half_to_float.argtypes = [ctypes.c_uint16]
+        _lib.oracle_float_to_half.restype = ctypes.c_uint16
+        _lib.oracle_float_to_half.argtypes = [ctypes.c_float]
+        _lib.oracle_segments.restype = ctypes.c_int64
+    return _lib
+
+
+def _p(a):
+    return ctypes.c_void_p(a.ctypes.data) if a is not None else ctypes.c_void_p(0)
+
+
+def _i32(a):
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    return a
+
+
+def forward(weights, table_offsets, indices, offsets, per_sample_weights=None):
+    """-> output [B, T, D] in the weights' dtype."""
+    weights = np.ascontiguousarray(weights)
+    code = _CODES[weights.dtype]
+    table_offsets, indices, offsets = _i32(table_offsets), _i32(indices), _i32(offsets)
+    T = table_offsets.size
+    B = (offsets.size - 1) // T
+    D = weights.shape[1]
+    psw = None if per_sample_weights is None else np.ascontiguousarray(per_sample_weights, dtype=weights.dtype)
+    out = np.empty((B, T, D), dtype=weights.dtype)
+    lib().oracle_forward(_p(weights), code, ctypes.c_int32(D), _p(table_offsets), ctypes.c_int32(T), _p(indices),
+                         _p(offsets), ctypes.c_int32(B), _p(psw), _p(out))
+    return out
+
+
+def linearize(table_offsets, indices, offsets):
+    """-> keys, info_b_t, info_indices_idx (all int32 [N])."""
+    table_offsets, indices, offsets = _i32(table_offsets), _i32(indices), _i32(offsets)
+    T = table_offsets.size
+    B = (offsets.size - 1) // T
+    n = indices.size
+    keys, b_t, idx = (np.empty(n, np.int32) for _ in range(3))
+    lib().oracle_linearize(_p(table_offsets), ctypes.c_int32(T), _p(indices), _p(offsets), ctypes.c_int32(B),
+                           _p(keys), _p(b_t), _p(idx))
+    return keys, b_t, idx
+
+
+def sort_pairs(keys, values, end_bit):
+    keys = _i32(keys)
+    values = None if values is None else _i32(values)
+    ko, vo = np.empty(keys.size, np.int32), np.empty(keys.size, np.int32)
+    lib().oracle_sort_pairs(_p(keys), _p(values), _p(ko), _p(vo), ctypes.c_int64(keys.size), ctypes.c_int32(end_bit))
+    return ko, vo
+
+
+def segments(keys_sorted):
+    keys_sorted = _i32(keys_sorted)
+    starts = np.empty(keys_sorted.size + 1, np.int32)
+    U = lib().oracle_segments(_p(keys_sorted), ctypes.c_int64(keys_sorted.size), _p(starts))
+    return starts[: U + 1].copy()
+
+
+def backward(optimizer, grad_output, weights, table_offsets, indices, offsets, lr, eps=0.0,
+             optimizer_state=None, per_sample_weights=None):
+    """In-place update of `weights` (and `optimizer_state`); optimizer 'sgd' or 'adagrad'.
+
+    Returns dict(keys_sorted, positions_sorted, segment_starts, grad_psw)."""
+    assert weights.flags["C_CONTIGUOUS"] and weights.dtype in _CODES
+    code = _CODES[weights.dtype]
+    grad_output = np.ascontiguousarray(grad_output, dtype=weights.dtype)
+    table_offsets, indices, offsets = _i32(table_offsets), _i32(indices), _i32(offsets)
+    T = table_offsets.size
+    B = (offsets.size - 1) // T
+    D = weights.shape[1]
+    n = indices.size
+    assert grad_output.shape == (B, T, D)
+    psw = gpsw = None
+    if per_sample_weights is not None:
+        psw = np.ascontiguousarray(per_sample_weights, dtype=weights.dtype)
+        gpsw = np.zeros(n, dtype=weights.dtype)
+    opt = {"sgd": 0, "adagrad": 1}[optimizer]
+    if opt == 1:
+        want = np.float64 if weights.dtype == np.float64 else np.float32
+        assert optimizer_state is not None and optimizer_state.dtype == want
+        assert optimizer_state.flags["C_CONTIGUOUS"]
+    ks, ps, ss = np.empty(n, np.int32), np.empty(n, np.int32), np.empty(n + 1, np.int32)
+    U = ctypes.c_int64(0)
+    lib().oracle_backward(ctypes.c_int(opt), _p(grad_output), _p(weights), ctypes.c_int(code),
+                          ctypes.c_int64(weights.shape[0]), ctypes.c_int32(D), _p(table_offsets), ctypes.c_int32(T),
+                          _p(indices), ctypes.c_int64(n), _p(offsets), ctypes.c_int32(B), _p(psw),
+                          _p(optimizer_state), ctypes.c_float(lr), ctypes.c_float(eps), _p(gpsw), _p(ks), _p(ps),
+                          _p(ss), ctypes.byref(U))
+    return {"keys_sorted": ks, "positions_sorted": ps, "segment_starts": ss[: U.value + 1].copy(), "grad_psw": gpsw}
+
+
+def construct_offsets(batch_offsets_per_table, total_indices_per_table):
+    per_table = _i32(batch_offsets_per_table)
+    totals = _i32(total_indices_per_table)
+    T, B = per_table.shape
+    out = np.empty(1 + T * B, np.int32)
+    lib().oracle_construct_offsets(_p(per_table), _p(totals), ctypes.c_int32(T), ctypes.c_int32(B), _p(out))
+    return out
+
+
+def half_to_float(bits):
+    return lib().oracle_half_to_float(int(bits))
+
+
+def float_to_half(value):
+    return lib().oracle_float_to_half(float(value))

@@ -1,0 +1,126 @@
+// Error plumbing, small utility kernels and host-memory allocators of the C ABI.
+
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "tbe_common.h"
+
+namespace tbe {
+
+namespace {
+thread_local char g_last_error[512] = "";
+}
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char *what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TBE_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return TBE_OK;
+}
+
+namespace {
+
+// One thread per bag; same arithmetic as construct_offsets_kernel
+// (table_batched_embeddings_cuda.cu:1165-1188).
+__global__ __launch_bounds__(kBlockThreads) void construct_offsets_kernel(
+    const int32_t *__restrict__ batch_offsets_per_table,
+    const int32_t *__restrict__ total_indices_per_table, int T, int B,
+    int32_t *__restrict__ output) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i == 0) output[0] = 0;
+  if (i >= static_cast<int64_t>(T) * B) return;
+  const int t = static_cast<int>(i / B);
+  const int b = static_cast<int>(i - static_cast<int64_t>(t) * B);
+  const int32_t lower = batch_offsets_per_table[i];
+  const int32_t upper = (b != B - 1) ? batch_offsets_per_table[i + 1] : total_indices_per_table[t];
+  output[1 + i] = upper - lower;
+}
+
+}  // namespace
+}  // namespace tbe
+
+extern "C" const char *tbe_last_error(void) { return tbe::g_last_error; }
+
+extern "C" int32_t tbe_abi_version(void) { return 1; }
+
+extern "C" int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
+                                     const int32_t *total_indices_per_table, int32_t T,
+                                     int32_t B, int32_t *output, void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(T > 0 && B > 0, "tbe_construct_offsets: T and B must be positive (got %d, %d)", T, B);
+  TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "tbe_construct_offsets: T*B out of range");
+  TBE_REQUIRE(batch_offsets_per_table && total_indices_per_table && output,
+              "tbe_construct_offsets: null pointer argument");
+  const int64_t n = static_cast<int64_t>(T) * B;
+  const dim3 grid(static_cast<unsigned>(ceil_div(n, kBlockThreads)));
+  hipLaunchKernelGGL(construct_offsets_kernel, grid, dim3(kBlockThreads), 0,
+                     static_cast<hipStream_t>(stream), batch_offsets_per_table,
+                     total_indices_per_table, T, B, output);
+  return check_launch("tbe_construct_offsets");
+}
+
+extern "C" int tbe_host_mapped_alloc(uint64_t bytes, void **host_ptr, void **device_ptr) {
+  using namespace tbe;
+  TBE_REQUIRE(host_ptr && device_ptr, "tbe_host_mapped_alloc: null output pointer");
+  *host_ptr = nullptr;
+  *device_ptr = nullptr;
+  if (bytes == 0) return TBE_OK;
+  void *h = nullptr;
+  hipError_t e = hipHostMalloc(&h, bytes, hipHostMallocMapped | hipHostMallocPortable);
+  if (e != hipSuccess)
+    return fail(TBE_ERR_HIP, "tbe_host_mapped_alloc(%llu): %s", (unsigned long long)bytes,
+                hipGetErrorString(e));
+  void *d = nullptr;
+  e = hipHostGetDevicePointer(&d, h, 0);
+  if (e != hipSuccess) {
+    (void)hipHostFree(h);
+    return fail(TBE_ERR_HIP, "tbe_host_mapped_alloc: hipHostGetDevicePointer: %s",
+                hipGetErrorString(e));
+  }
+  *host_ptr = h;
+  *device_ptr = d;
+  return TBE_OK;
+}
+
+extern "C" int tbe_host_mapped_free(void *host_ptr) {
+  using namespace tbe;
+  if (!host_ptr) return TBE_OK;
+  const hipError_t e = hipHostFree(host_ptr);
+  if (e != hipSuccess) return fail(TBE_ERR_HIP, "tbe_host_mapped_free: %s", hipGetErrorString(e));
+  return TBE_OK;
+}
+
+extern "C" int tbe_managed_alloc(uint64_t bytes, int32_t device, void **ptr) {
+  using namespace tbe;
+  TBE_REQUIRE(ptr, "tbe_managed_alloc: null output pointer");
+  *ptr = nullptr;
+  if (bytes == 0) return TBE_OK;
+  void *p = nullptr;
+  hipError_t e = hipMallocManaged(&p, bytes, hipMemAttachGlobal);
+  if (e != hipSuccess)
+    return fail(TBE_ERR_HIP, "tbe_managed_alloc(%llu): %s", (unsigned long long)bytes,
+                hipGetErrorString(e));
+  // Same placement advice as the reference's managed allocator
+  // (table_batched_embeddings_cuda.cu:801-804): pages live on the host, the GPU maps them.
+  // Advice is best effort: a platform that rejects it still has a valid allocation.
+  (void)hipMemAdvise(p, bytes, hipMemAdviseSetPreferredLocation, hipCpuDeviceId);
+  (void)hipMemAdvise(p, bytes, hipMemAdviseSetAccessedBy, device);
+  (void)hipGetLastError();
+  *ptr = p;
+  return TBE_OK;
+}
+
+extern "C" int tbe_managed_free(void *ptr) {
+  using namespace tbe;
+  if (!ptr) return TBE_OK;
+  const hipError_t e = hipFree(ptr);
+  if (e != hipSuccess) return fail(TBE_ERR_HIP, "tbe_managed_free: %s", hipGetErrorString(e));
+  return TBE_OK;
+}

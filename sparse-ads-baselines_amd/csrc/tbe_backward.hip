@@ -1,0 +1,172 @@
+// Fused backward entry points: linearize -> stable radix sort -> run boundaries
+// -> per-row gradient reduction + optimizer, all on the caller's stream and
+// workspace, with no host synchronisation.  Pipeline shape follows
+// batched_embedding_backward_adagrad_exact_cuda
+// (table_batched_embeddings_cuda.cu:1589-1706); SGD uses the same pipeline so
+// that repeated rows are updated exactly once.
+
+#include <math.h>
+
+#include "tbe_stages.h"
+
+namespace tbe {
+namespace {
+
+// Number of low key bits that can be set when keys are < total_rows.  The
+// reference sorts int(log2(total_rows) + 1) bits (tbe.cu:1643), which is the
+// same quantity for every total_rows >= 1.
+int key_bits(int64_t total_rows) {
+  int bits = 0;
+  while (bits < 32 && (int64_t{1} << bits) <= total_rows) ++bits;
+  return bits;
+}
+
+void compute_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t *l) {
+  const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
+  const uint64_t ints = align_up(nn * 4, 256);
+  l->max_long_segments = static_cast<int64_t>(nn / kLongSegment + 1);
+  l->max_chunks = static_cast<int64_t>(nn / kChunkLen + nn / kLongSegment + 2);
+  uint64_t off = 0;
+  l->keys = off; off += ints;
+  l->grad_rows = off; off += ints;
+  l->keys_sorted = off; off += ints;
+  l->positions_sorted = off; off += ints;
+  l->segment_starts = off; off += align_up((nn + 1) * 4, 256);
+  l->num_unique = off; off += 256;
+  l->sort_scratch = off; off += align_up(sort_workspace_bytes(n), 256);
+  l->segment_scratch = off; off += align_up(segments_workspace_bytes(n), 256);
+  l->long_segments = off; off += align_up(static_cast<uint64_t>(l->max_long_segments) * 2 * 4, 256);
+  l->chunk_segments = off; off += align_up(static_cast<uint64_t>(l->max_chunks) * 4, 256);
+  l->partial_sums = off;
+  off += align_up(static_cast<uint64_t>(l->max_chunks) * static_cast<uint64_t>(D) * acc_size(dtype), 256);
+  l->total_bytes = off;
+}
+
+struct BackwardCall {
+  const void *grad_output;
+  void *weights;
+  int32_t dtype;
+  int64_t total_rows;
+  int32_t D;
+  const int32_t *table_offsets;
+  int32_t T;
+  const int32_t *indices;
+  int64_t num_indices;
+  const int32_t *offsets;
+  int32_t B;
+  const void *psw;
+  void *state;
+  float lr;
+  float eps;
+  void *grad_psw;
+  void *workspace;
+  uint64_t workspace_bytes;
+  hipStream_t stream;
+  int optimizer;
+};
+
+int run_backward(const char *name, const BackwardCall &c) {
+  TBE_REQUIRE(c.T > 0, "%s: T must be positive (got %d)", name, c.T);
+  TBE_REQUIRE(c.D > 0, "%s: D must be positive (got %d)", name, c.D);
+  TBE_REQUIRE(c.B > 0, "%s: B must be positive (got %d)", name, c.B);
+  TBE_REQUIRE(c.D % 4 == 0, "%s: D must be a multiple of 4 (got %d)", name, c.D);
+  TBE_REQUIRE(c.dtype >= TBE_DTYPE_F32 && c.dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, c.dtype);
+  TBE_REQUIRE(c.total_rows > 0 && c.total_rows < INT32_MAX, "%s: total_rows out of range", name);
+  TBE_REQUIRE(c.num_indices >= 0 && c.num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(static_cast<int64_t>(c.T) * c.B < INT32_MAX, "%s: T*B out of range", name);
+  TBE_REQUIRE(c.grad_output && c.weights && c.table_offsets && c.offsets, "%s: null pointer argument", name);
+  TBE_REQUIRE(c.indices || c.num_indices == 0, "%s: indices is null but num_indices > 0", name);
+  TBE_REQUIRE(c.optimizer == kOptSgd || c.state, "%s: optimizer_state is null", name);
+  TBE_REQUIRE((c.psw == nullptr) == (c.grad_psw == nullptr),
+              "%s: per_sample_weights and grad_per_sample_weights must both be given or both be null", name);
+  if (c.num_indices == 0) return TBE_OK;
+
+  tbe_workspace_layout_t l;
+  compute_layout(c.num_indices, c.D, c.dtype, &l);
+  if (!c.workspace || c.workspace_bytes < l.total_bytes)
+    return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
+                (unsigned long long)l.total_bytes, (unsigned long long)c.workspace_bytes);
+  char *ws = static_cast<char *>(c.workspace);
+  int32_t *keys = reinterpret_cast<int32_t *>(ws + l.keys);
+  int32_t *grad_rows = reinterpret_cast<int32_t *>(ws + l.grad_rows);
+  int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
+  int32_t *positions_sorted = reinterpret_cast<int32_t *>(ws + l.positions_sorted);
+  int32_t *segment_starts = reinterpret_cast<int32_t *>(ws + l.segment_starts);
+  int32_t *counters = reinterpret_cast<int32_t *>(ws + l.num_unique);
+
+  int rc = linearize(c.table_offsets, c.T, c.indices, c.offsets, c.B, keys, grad_rows, c.stream);
+  if (rc) return rc;
+  rc = sort_pairs(keys, nullptr, keys_sorted, positions_sorted, c.num_indices,
+                  key_bits(c.total_rows), ws + l.sort_scratch, c.stream);
+  if (rc) return rc;
+  rc = find_segments(keys_sorted, c.num_indices, segment_starts, counters, ws + l.segment_scratch,
+                     c.stream);
+  if (rc) return rc;
+
+  UpdateArgs a;
+  a.grad_output = c.grad_output;
+  a.weights = c.weights;
+  a.optimizer_state = c.state;
+  a.per_sample_weights = c.psw;
+  a.grad_per_sample_weights = c.grad_psw;
+  a.keys_sorted = keys_sorted;
+  a.positions_sorted = positions_sorted;
+  a.grad_rows = grad_rows;
+  a.segment_starts = segment_starts;
+  a.counters = counters;
+  a.long_segments = reinterpret_cast<int32_t *>(ws + l.long_segments);
+  a.chunk_segments = reinterpret_cast<int32_t *>(ws + l.chunk_segments);
+  a.partial_sums = ws + l.partial_sums;
+  a.num_indices = c.num_indices;
+  a.max_long = l.max_long_segments;
+  a.max_chunks = l.max_chunks;
+  a.dtype = c.dtype;
+  a.D = c.D;
+  a.optimizer = c.optimizer;
+  a.learning_rate = c.lr;
+  a.eps = c.eps;
+  return segment_update(a, c.stream);
+}
+
+}  // namespace
+}  // namespace tbe
+
+extern "C" int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int32_t dtype,
+                                             tbe_workspace_layout_t *layout) {
+  using namespace tbe;
+  TBE_REQUIRE(layout, "tbe_backward_workspace_layout: null layout");
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX,
+              "tbe_backward_workspace_layout: num_indices out of range");
+  TBE_REQUIRE(D > 0 && D % 4 == 0, "tbe_backward_workspace_layout: D must be a positive multiple of 4 (got %d)", D);
+  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64,
+              "tbe_backward_workspace_layout: bad dtype %d", dtype);
+  compute_layout(num_indices, D, dtype, layout);
+  return TBE_OK;
+}
+
+extern "C" int tbe_backward_sgd(const void *grad_output, void *weights, int32_t dtype,
+                                int64_t total_rows, int32_t D, const int32_t *table_offsets,
+                                int32_t T, const int32_t *indices, int64_t num_indices,
+                                const int32_t *offsets, int32_t B, float learning_rate,
+                                void *workspace, uint64_t workspace_bytes, void *stream) {
+  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
+                      num_indices, offsets, B, nullptr, nullptr, learning_rate, 0.0f, nullptr,
+                      workspace, workspace_bytes, static_cast<hipStream_t>(stream), tbe::kOptSgd};
+  return tbe::run_backward("tbe_backward_sgd", c);
+}
+
+extern "C" int tbe_backward_exact_adagrad(const void *grad_output, void *weights, int32_t dtype,
+                                          int64_t total_rows, int32_t D,
+                                          const int32_t *table_offsets, int32_t T,
+                                          const int32_t *indices, int64_t num_indices,
+                                          const int32_t *offsets, int32_t B,
+                                          const void *per_sample_weights, void *optimizer_state,
+                                          float learning_rate, float eps,
+                                          void *grad_per_sample_weights, void *workspace,
+                                          uint64_t workspace_bytes, void *stream) {
+  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
+                      num_indices, offsets, B, per_sample_weights, optimizer_state, learning_rate,
+                      eps, grad_per_sample_weights, workspace, workspace_bytes,
+                      static_cast<hipStream_t>(stream), tbe::kOptAdagrad};
+  return tbe::run_backward("tbe_backward_exact_adagrad", c);
+}

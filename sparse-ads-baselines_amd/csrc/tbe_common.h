@@ -1,0 +1,167 @@
+// Shared device helpers and host-side plumbing for the gfx950 TBE kernels.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tbe_hip.h"
+
+namespace tbe {
+
+constexpr int kWave = 64;          // CDNA wavefront width
+constexpr int kBlockThreads = 256;  // 4 wavefronts per workgroup
+constexpr int kWavesPerBlock = kBlockThreads / kWave;
+constexpr int kNumXcd = 8;          // MI355X: 8 XCDs, workgroups are dealt round-robin
+
+// ---------------------------------------------------------------- host side
+// Records `msg` as this thread's last error and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int check_launch(const char *what);
+
+#define TBE_REQUIRE(cond, ...)                                  \
+  do {                                                          \
+    if (!(cond)) return ::tbe::fail(TBE_ERR_INVALID, __VA_ARGS__); \
+  } while (0)
+
+inline uint64_t align_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Geometry of one embedding row spread over the lanes of a wavefront.
+// A row is `chunks` vectors of VEC elements (16 bytes where alignment allows);
+// `chunks` consecutive lanes form a lane group that owns one row at a time, and
+// a wavefront holds floor(64 / chunks) groups.  Rows wider than 64 vectors are
+// handled by the whole wavefront looping over column blocks.
+struct RowGeometry {
+  int vec;        // elements per lane per access
+  int chunks;     // D / vec
+  int tmpl;       // chunks if it is a power of two <= 64 (compile-time variant), else 0
+  bool wide;      // chunks > 64
+};
+
+inline RowGeometry row_geometry(int32_t dtype, int32_t D) {
+  RowGeometry g;
+  if (dtype == TBE_DTYPE_F16) g.vec = (D % 8 == 0) ? 8 : 4;
+  else if (dtype == TBE_DTYPE_F32) g.vec = 4;
+  else g.vec = 2;
+  g.chunks = D / g.vec;
+  g.wide = g.chunks > kWave;
+  g.tmpl = (!g.wide && (g.chunks & (g.chunks - 1)) == 0) ? g.chunks : 0;
+  return g;
+}
+
+inline size_t dtype_size(int32_t dtype) {
+  return dtype == TBE_DTYPE_F16 ? 2 : dtype == TBE_DTYPE_F32 ? 4 : 8;
+}
+inline size_t acc_size(int32_t dtype) { return dtype == TBE_DTYPE_F64 ? 8 : 4; }
+
+// -------------------------------------------------------------- device side
+template <typename T> struct AccOf { using type = float; };
+template <> struct AccOf<double> { using type = double; };
+
+// Raw storage of VEC consecutive elements, loaded/stored with one instruction.
+template <typename T, int VEC> struct Raw;
+template <> struct Raw<float, 4> { using type = float4; };
+template <> struct Raw<__half, 8> { using type = uint4; };
+template <> struct Raw<__half, 4> { using type = uint2; };
+template <> struct Raw<double, 2> { using type = double2; };
+
+template <typename T, int VEC> struct RowVec {
+  using A = typename AccOf<T>::type;
+  using R = typename Raw<T, VEC>::type;
+  A v[VEC];
+
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = A(0);
+  }
+  __device__ __forceinline__ static R load_raw(const T *p) {
+    return *reinterpret_cast<const R *>(p);
+  }
+  __device__ __forceinline__ void unpack(const R &r);
+  __device__ __forceinline__ R pack() const;
+  __device__ __forceinline__ void load(const T *p) { unpack(load_raw(p)); }
+  __device__ __forceinline__ void store(T *p) const { *reinterpret_cast<R *>(p) = pack(); }
+};
+
+template <> __device__ __forceinline__ void RowVec<float, 4>::unpack(const float4 &r) {
+  v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+}
+template <> __device__ __forceinline__ float4 RowVec<float, 4>::pack() const {
+  return make_float4(v[0], v[1], v[2], v[3]);
+}
+template <> __device__ __forceinline__ void RowVec<double, 2>::unpack(const double2 &r) {
+  v[0] = r.x; v[1] = r.y;
+}
+template <> __device__ __forceinline__ double2 RowVec<double, 2>::pack() const {
+  return make_double2(v[0], v[1]);
+}
+
+__device__ __forceinline__ void half2_to_floats(uint32_t bits, float &lo, float &hi) {
+  __half2 h = *reinterpret_cast<const __half2 *>(&bits);
+  float2 f = __half22float2(h);
+  lo = f.x; hi = f.y;
+}
+// Round-to-nearest-even, the rounding the reference uses when it stores fp16
+// (__float22half2_rn, table_batched_embeddings_cuda.cu:81-82).
+__device__ __forceinline__ uint32_t floats_to_half2(float lo, float hi) {
+  __half2 h = __floats2half2_rn(lo, hi);
+  return *reinterpret_cast<const uint32_t *>(&h);
+}
+template <> __device__ __forceinline__ void RowVec<__half, 8>::unpack(const uint4 &r) {
+  half2_to_floats(r.x, v[0], v[1]); half2_to_floats(r.y, v[2], v[3]);
+  half2_to_floats(r.z, v[4], v[5]); half2_to_floats(r.w, v[6], v[7]);
+}
+template <> __device__ __forceinline__ uint4 RowVec<__half, 8>::pack() const {
+  return make_uint4(floats_to_half2(v[0], v[1]), floats_to_half2(v[2], v[3]),
+                    floats_to_half2(v[4], v[5]), floats_to_half2(v[6], v[7]));
+}
+template <> __device__ __forceinline__ void RowVec<__half, 4>::unpack(const uint2 &r) {
+  half2_to_floats(r.x, v[0], v[1]); half2_to_floats(r.y, v[2], v[3]);
+}
+template <> __device__ __forceinline__ uint2 RowVec<__half, 4>::pack() const {
+  return make_uint2(floats_to_half2(v[0], v[1]), floats_to_half2(v[2], v[3]));
+}
+
+__device__ __forceinline__ float to_acc(float x) { return x; }
+__device__ __forceinline__ float to_acc(__half x) { return __half2float(x); }
+__device__ __forceinline__ double to_acc(double x) { return x; }
+template <typename T, typename A> __device__ __forceinline__ T from_acc(A x);
+template <> __device__ __forceinline__ float from_acc<float, float>(float x) { return x; }
+template <> __device__ __forceinline__ __half from_acc<__half, float>(float x) { return __float2half_rn(x); }
+template <> __device__ __forceinline__ double from_acc<double, double>(double x) { return x; }
+
+__device__ __forceinline__ float shfl_idx(float v, int src) { return __shfl(v, src, kWave); }
+__device__ __forceinline__ int shfl_idx(int v, int src) { return __shfl(v, src, kWave); }
+__device__ __forceinline__ double shfl_idx(double v, int src) { return __shfl(v, src, kWave); }
+__device__ __forceinline__ float shfl_x(float v, int m) { return __shfl_xor(v, m, kWave); }
+__device__ __forceinline__ double shfl_x(double v, int m) { return __shfl_xor(v, m, kWave); }
+
+// Sum of `v` over the `chunks` lanes of the caller's lane group; every lane of
+// the group gets the result.  CHUNKS > 0: power-of-two group, xor butterfly that
+// never leaves the group.  CHUNKS == 0: arbitrary group size, every lane adds the
+// group's values in lane order (`group_base` = first lane of the group).
+template <int CHUNKS, typename A>
+__device__ __forceinline__ A group_sum(A v, int chunks, int group_base) {
+  if constexpr (CHUNKS > 0) {
+#pragma unroll
+    for (int m = CHUNKS / 2; m > 0; m >>= 1) v += shfl_x(v, m);
+    return v;
+  } else {
+    A s = A(0);
+    for (int j = 0; j < chunks; ++j) s += shfl_idx(v, group_base + j);
+    return s;
+  }
+}
+
+// Workgroups are dealt to the 8 XCDs round-robin by blockIdx.  This maps
+// blockIdx to a logical work index so that each XCD walks one contiguous
+// eighth of the work: consecutive bags / segments (same table, neighbouring
+// hot rows) then share one XCD's L2 instead of being replicated in all eight.
+// `per_xcd` = ceil(num_work / 8); the grid must hold 8 * per_xcd workgroups
+// and indices >= num_work are idle.
+__device__ __forceinline__ int64_t xcd_contiguous(int64_t block, int64_t per_xcd) {
+  return (block % kNumXcd) * per_xcd + block / kNumXcd;
+}
+
+}  // namespace tbe

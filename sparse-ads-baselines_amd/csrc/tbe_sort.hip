@@ -1,0 +1,427 @@
+// Integer stages of the backward pass for gfx950:
+//   linearize      (table,row) keys and the gradient row of every lookup
+//   sort_pairs     stable LSD radix sort, 8-bit digits, LDS-staged scatter
+//   find_segments  run boundaries of the sorted keys (one per unique row)
+//
+// The sort is the contract of cub::DeviceRadixSort::SortPairs as the reference
+// calls it (table_batched_embeddings_cuda.cu:1639-1655): ascending, stable,
+// key bits [0, end_bit).  Each pass is three kernels:
+//   histogram  per-tile digit counts (LDS atomics) -> counts[digit][tile], totals[digit]
+//   scan       one workgroup per digit turns counts into global start offsets
+//   scatter    ranks each key inside its tile with wavefront ballots (all lanes
+//              holding the same digit are found with 8 ballots; the lowest lane
+//              reserves the run in a per-wavefront LDS counter), reorders the
+//              tile in LDS so every digit's keys are contiguous, and writes
+//              them out in runs.
+// A tile is 4096 pairs; position order inside a tile is (wavefront, item, lane),
+// which the ranking preserves, so the sort is stable.
+
+#include "tbe_common.h"
+
+namespace tbe {
+namespace {
+
+constexpr int kRadixBits = 8;
+constexpr int kBins = 1 << kRadixBits;            // 256 == kBlockThreads
+constexpr int kItems = 16;                        // pairs per thread per tile
+constexpr int kTile = kBlockThreads * kItems;     // 4096
+constexpr int kWaveTile = kWave * kItems;         // 1024 pairs per wavefront
+static_assert(kBins == kBlockThreads, "one thread per digit");
+
+constexpr int kSegItems = 8;
+constexpr int kSegTile = kBlockThreads * kSegItems;  // 2048
+
+// Inclusive prefix sum over the 256 threads of a workgroup.  `total` receives the
+// workgroup sum.  `s_wave` is 4 words of LDS.  Ends with a barrier-free state:
+// callers that reuse `s_wave` must __syncthreads() first.
+__device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t x, uint32_t *s_wave,
+                                                         uint32_t &total) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t y = __shfl_up(x, d, kWave);
+    if (lane >= d) x += y;
+  }
+  if (lane == kWave - 1) s_wave[wave] = x;
+  __syncthreads();
+  uint32_t base = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) {
+    const uint32_t v = s_wave[w];
+    if (w < wave) base += v;
+    sum += v;
+  }
+  total = sum;
+  return x + base;
+}
+
+// ------------------------------------------------------------------ linearize
+// 16 lanes per bag.  Mirrors linear_index_weight_offsets_kernel
+// (table_batched_embeddings_cuda.cu:1471-1497); instead of the 8-byte
+// IndexInfo{b_t, indices_idx} payload it records the gradient row b*T + t of
+// each position, and the sort carries the position itself.
+constexpr int kLinLanes = 16;
+__global__ __launch_bounds__(kBlockThreads) void linearize_kernel(
+    const int32_t *__restrict__ table_offsets, const int32_t *__restrict__ indices,
+    const int32_t *__restrict__ offsets, int B, int num_tables, int num_bags,
+    int32_t *__restrict__ keys, int32_t *__restrict__ grad_rows) {
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t bag64 = gid / kLinLanes;
+  if (bag64 >= num_bags) return;
+  const int bag = static_cast<int>(bag64);
+  const int sub = static_cast<int>(gid % kLinLanes);
+  const int t = bag / B;
+  const int b = bag - t * B;
+  const int32_t row0 = table_offsets[t];
+  const int32_t grow = b * num_tables + t;
+  const int start = offsets[bag];
+  const int end = offsets[bag + 1];
+  for (int p = start + sub; p < end; p += kLinLanes) {
+    keys[p] = row0 + indices[p];
+    grad_rows[p] = grow;
+  }
+}
+
+// ------------------------------------------------------------------ radix sort
+__global__ __launch_bounds__(kBlockThreads) void radix_zero_totals_kernel(uint32_t *totals, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) totals[i] = 0;
+}
+
+__global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
+    const uint32_t *__restrict__ keys, int64_t n, int shift, uint32_t mask, int num_tiles,
+    uint32_t *__restrict__ counts, uint32_t *__restrict__ totals) {
+  __shared__ uint32_t s_hist[kBins];
+  const int tid = threadIdx.x;
+  s_hist[tid] = 0;
+  __syncthreads();
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kTile;
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = base + k * kBlockThreads + tid;
+    if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & mask], 1u);
+  }
+  __syncthreads();
+  const uint32_t c = s_hist[tid];
+  counts[static_cast<int64_t>(tid) * num_tiles + blockIdx.x] = c;
+  if (c) atomicAdd(&totals[tid], c);
+}
+
+// Workgroup `d` converts counts[d][0..num_tiles) into the global output offset of
+// digit d's keys in each tile: (keys with a smaller digit) + (same digit, earlier tile).
+__global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
+    uint32_t *__restrict__ counts, const uint32_t *__restrict__ totals, int num_tiles) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int tid = threadIdx.x;
+  const int d = blockIdx.x;
+  uint32_t carry;
+  (void)block_inclusive_scan(tid < d ? totals[tid] : 0u, s_wave, carry);
+  __syncthreads();
+  uint32_t *row = counts + static_cast<int64_t>(d) * num_tiles;
+  for (int c0 = 0; c0 < num_tiles; c0 += kBlockThreads) {
+    const int i = c0 + tid;
+    const uint32_t x = i < num_tiles ? row[i] : 0u;
+    uint32_t total;
+    const uint32_t incl = block_inclusive_scan(x, s_wave, total);
+    if (i < num_tiles) row[i] = carry + incl - x;
+    carry += total;
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
+    const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ values_in,
+    uint32_t *__restrict__ keys_out, uint32_t *__restrict__ values_out, int64_t n, int shift,
+    uint32_t mask, int num_tiles, const uint32_t *__restrict__ bases) {
+  __shared__ uint32_t s_keys[kTile];
+  __shared__ uint32_t s_vals[kTile];
+  __shared__ uint32_t s_wave_count[kWavesPerBlock][kBins];
+  __shared__ uint32_t s_bin_start[kBins];
+  __shared__ uint32_t s_dest[kBins];
+  __shared__ uint32_t s_scan[kWavesPerBlock];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int64_t tile_base = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int tile_count = static_cast<int>(min(static_cast<int64_t>(kTile), n - tile_base));
+
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) s_wave_count[w][tid] = 0;
+
+  uint32_t key[kItems], val[kItems];
+  const int64_t wave_base = tile_base + wave * kWaveTile;
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = wave_base + k * kWave + lane;
+    const bool valid = i < n;
+    key[k] = valid ? keys_in[i] : 0xffffffffu;
+    val[k] = valid ? (values_in ? values_in[i] : static_cast<uint32_t>(i)) : 0u;
+  }
+  __syncthreads();
+
+  // Rank of each key among the keys of its wavefront that share its digit.
+  uint32_t rank[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const bool valid = (wave_base + k * kWave + lane) < n;
+    const uint32_t digit = (key[k] >> shift) & mask;
+    unsigned long long peers = __ballot(valid);
+#pragma unroll
+    for (int bit = 0; bit < kRadixBits; ++bit) {
+      const bool set = (digit >> bit) & 1u;
+      const unsigned long long vote = __ballot(set);
+      peers &= set ? vote : ~vote;
+    }
+    const unsigned long long below = peers & ((1ull << lane) - 1ull);
+    uint32_t run_start = 0;
+    if (valid && below == 0ull) {
+      run_start = atomicAdd(&s_wave_count[wave][digit], static_cast<uint32_t>(__popcll(peers)));
+    }
+    const int leader = valid ? (__ffsll(static_cast<long long>(peers)) - 1) : lane;
+    run_start = __shfl(run_start, leader, kWave);
+    rank[k] = run_start + static_cast<uint32_t>(__popcll(below));
+  }
+  __syncthreads();
+
+  // Thread `tid` owns digit `tid`: prefix over wavefronts, then over digits.
+  {
+    uint32_t running = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+      const uint32_t c = s_wave_count[w][tid];
+      s_wave_count[w][tid] = running;
+      running += c;
+    }
+    uint32_t total;
+    const uint32_t incl = block_inclusive_scan(running, s_scan, total);
+    const uint32_t bin_start = incl - running;
+    s_bin_start[tid] = bin_start;
+    s_dest[tid] = bases[static_cast<int64_t>(tid) * num_tiles + blockIdx.x] - bin_start;
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const bool valid = (wave_base + k * kWave + lane) < n;
+    if (valid) {
+      const uint32_t digit = (key[k] >> shift) & mask;
+      const uint32_t local = s_bin_start[digit] + s_wave_count[wave][digit] + rank[k];
+      s_keys[local] = key[k];
+      s_vals[local] = val[k];
+    }
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int local = k * kBlockThreads + tid;
+    if (local < tile_count) {
+      const uint32_t kk = s_keys[local];
+      const uint32_t dst = s_dest[(kk >> shift) & mask] + static_cast<uint32_t>(local);
+      keys_out[dst] = kk;
+      values_out[dst] = s_vals[local];
+    }
+  }
+}
+
+// -------------------------------------------------------------- find segments
+// Thread owns kSegItems consecutive sorted positions.  head(i) = i == 0 || key[i] != key[i-1]
+// (table_batched_embeddings_cuda.cu:1523-1525).
+__device__ __forceinline__ uint32_t segment_head_flags(const uint32_t *__restrict__ keys, int64_t n,
+                                                       int64_t first) {
+  uint32_t flags = 0;
+  if (first >= n) return 0;
+  uint32_t prev = first > 0 ? keys[first - 1] : 0u;
+#pragma unroll
+  for (int k = 0; k < kSegItems; ++k) {
+    const int64_t i = first + k;
+    if (i < n) {
+      const uint32_t cur = keys[i];
+      if (i == 0 || cur != prev) flags |= 1u << k;
+      prev = cur;
+    }
+  }
+  return flags;
+}
+
+__global__ __launch_bounds__(kBlockThreads) void segment_count_kernel(
+    const uint32_t *__restrict__ keys, int64_t n, uint32_t *__restrict__ tile_heads) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int64_t first = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x) * kSegItems;
+  uint32_t total;
+  (void)block_inclusive_scan(__popc(segment_head_flags(keys, n, first)), s_wave, total);
+  if (threadIdx.x == 0) tile_heads[blockIdx.x] = total;
+}
+
+// Single workgroup: exclusive scan of the per-tile head counts; publishes U and
+// the closing boundary segment_starts[U] = n.
+__global__ __launch_bounds__(kBlockThreads) void segment_scan_kernel(
+    uint32_t *__restrict__ tile_heads, int num_tiles, int64_t n,
+    int32_t *__restrict__ segment_starts, int32_t *__restrict__ num_unique) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int tid = threadIdx.x;
+  uint32_t carry = 0;
+  for (int c0 = 0; c0 < num_tiles; c0 += kBlockThreads) {
+    const int i = c0 + tid;
+    const uint32_t x = i < num_tiles ? tile_heads[i] : 0u;
+    uint32_t total;
+    const uint32_t incl = block_inclusive_scan(x, s_wave, total);
+    if (i < num_tiles) tile_heads[i] = carry + incl - x;
+    carry += total;
+    __syncthreads();
+  }
+  if (tid == 0) {
+    num_unique[0] = static_cast<int32_t>(carry);
+    segment_starts[carry] = static_cast<int32_t>(n);
+  }
+}
+
+__global__ __launch_bounds__(kBlockThreads) void segment_write_kernel(
+    const uint32_t *__restrict__ keys, int64_t n, const uint32_t *__restrict__ tile_base,
+    int32_t *__restrict__ segment_starts) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int64_t first = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x) * kSegItems;
+  const uint32_t flags = segment_head_flags(keys, n, first);
+  const uint32_t mine = __popc(flags);
+  uint32_t total;
+  const uint32_t incl = block_inclusive_scan(mine, s_wave, total);
+  uint32_t u = tile_base[blockIdx.x] + incl - mine;
+#pragma unroll
+  for (int k = 0; k < kSegItems; ++k) {
+    if (flags & (1u << k)) segment_starts[u++] = static_cast<int32_t>(first + k);
+  }
+}
+
+inline int num_sort_tiles(int64_t n) { return static_cast<int>(ceil_div(n, kTile)); }
+inline int num_seg_tiles(int64_t n) { return static_cast<int>(ceil_div(n, kSegTile)); }
+
+}  // namespace
+
+// Sort workspace: [tmp keys n][tmp values n][counts 256*tiles][totals 256*passes]
+constexpr int kMaxPasses = 4;
+
+uint64_t sort_workspace_bytes(int64_t n) {
+  const uint64_t tiles = num_sort_tiles(n > 0 ? n : 1);
+  return align_up(static_cast<uint64_t>(n > 0 ? n : 1) * 4, 256) * 2 +
+         align_up(tiles * kBins * 4, 256) + align_up(kMaxPasses * kBins * 4, 256);
+}
+
+int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
+               int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
+               hipStream_t stream) {
+  if (n == 0) return TBE_OK;
+  const int passes = end_bit <= 0 ? 1 : static_cast<int>(ceil_div(end_bit, kRadixBits));
+  const int tiles = num_sort_tiles(n);
+  char *ws = static_cast<char *>(workspace);
+  uint32_t *tmp_keys = reinterpret_cast<uint32_t *>(ws);
+  ws += align_up(static_cast<uint64_t>(n) * 4, 256);
+  uint32_t *tmp_vals = reinterpret_cast<uint32_t *>(ws);
+  ws += align_up(static_cast<uint64_t>(n) * 4, 256);
+  uint32_t *counts = reinterpret_cast<uint32_t *>(ws);
+  ws += align_up(static_cast<uint64_t>(tiles) * kBins * 4, 256);
+  uint32_t *totals = reinterpret_cast<uint32_t *>(ws);
+
+  const dim3 block(kBlockThreads);
+  hipLaunchKernelGGL(radix_zero_totals_kernel, dim3(kMaxPasses), block, 0, stream, totals,
+                     kMaxPasses * kBins);
+  const uint32_t *src_k = reinterpret_cast<const uint32_t *>(keys_in);
+  const uint32_t *src_v = reinterpret_cast<const uint32_t *>(values_in);
+  for (int pass = 0; pass < passes; ++pass) {
+    const int shift = pass * kRadixBits;
+    const int bits = end_bit <= 0 ? 0 : min(kRadixBits, end_bit - shift);
+    const uint32_t mask = (1u << bits) - 1u;
+    const bool to_out = ((passes - 1 - pass) % 2) == 0;
+    uint32_t *dst_k = to_out ? reinterpret_cast<uint32_t *>(keys_out) : tmp_keys;
+    uint32_t *dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
+    uint32_t *pass_totals = totals + pass * kBins;
+    hipLaunchKernelGGL(radix_histogram_kernel, dim3(tiles), block, 0, stream, src_k, n, shift,
+                       mask, tiles, counts, pass_totals);
+    hipLaunchKernelGGL(radix_scan_kernel, dim3(kBins), block, 0, stream, counts, pass_totals, tiles);
+    hipLaunchKernelGGL(radix_scatter_kernel, dim3(tiles), block, 0, stream, src_k, src_v, dst_k,
+                       dst_v, n, shift, mask, tiles, counts);
+    src_k = dst_k;
+    src_v = dst_v;
+  }
+  return check_launch("tbe_sort_pairs");
+}
+
+uint64_t segments_workspace_bytes(int64_t n) {
+  return align_up(static_cast<uint64_t>(num_seg_tiles(n > 0 ? n : 1)) * 4, 256);
+}
+
+int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts,
+                  int32_t *num_unique, void *workspace, hipStream_t stream) {
+  const int tiles = n > 0 ? num_seg_tiles(n) : 0;
+  uint32_t *tile_heads = static_cast<uint32_t *>(workspace);
+  const uint32_t *keys = reinterpret_cast<const uint32_t *>(keys_sorted);
+  const dim3 block(kBlockThreads);
+  if (tiles > 0)
+    hipLaunchKernelGGL(segment_count_kernel, dim3(tiles), block, 0, stream, keys, n, tile_heads);
+  hipLaunchKernelGGL(segment_scan_kernel, dim3(1), block, 0, stream, tile_heads, tiles, n,
+                     segment_starts, num_unique);
+  if (tiles > 0)
+    hipLaunchKernelGGL(segment_write_kernel, dim3(tiles), block, 0, stream, keys, n, tile_heads,
+                       segment_starts);
+  return check_launch("tbe_find_segments");
+}
+
+int linearize(const int32_t *table_offsets, int32_t T, const int32_t *indices,
+              const int32_t *offsets, int32_t B, int32_t *keys, int32_t *grad_rows,
+              hipStream_t stream) {
+  const int64_t num_bags = static_cast<int64_t>(T) * B;
+  const dim3 grid(static_cast<unsigned>(ceil_div(num_bags * kLinLanes, kBlockThreads)));
+  hipLaunchKernelGGL(linearize_kernel, grid, dim3(kBlockThreads), 0, stream, table_offsets,
+                     indices, offsets, B, T, static_cast<int>(num_bags), keys, grad_rows);
+  return check_launch("tbe_linearize");
+}
+
+}  // namespace tbe
+
+extern "C" int tbe_linearize(const int32_t *table_offsets, int32_t T, const int32_t *indices,
+                             int64_t num_indices, const int32_t *offsets, int32_t B,
+                             int32_t *keys, int32_t *grad_rows, void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(T > 0 && B > 0, "tbe_linearize: T and B must be positive (got %d, %d)", T, B);
+  TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "tbe_linearize: T*B out of range");
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "tbe_linearize: num_indices out of range");
+  TBE_REQUIRE(table_offsets && offsets, "tbe_linearize: null pointer argument");
+  if (num_indices == 0) return TBE_OK;
+  TBE_REQUIRE(indices && keys && grad_rows, "tbe_linearize: null pointer argument");
+  return linearize(table_offsets, T, indices, offsets, B, keys, grad_rows,
+                   static_cast<hipStream_t>(stream));
+}
+
+extern "C" uint64_t tbe_sort_workspace_bytes(int64_t n) { return tbe::sort_workspace_bytes(n); }
+
+extern "C" int tbe_sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
+                              int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
+                              uint64_t workspace_bytes, void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(n >= 0 && n < INT32_MAX, "tbe_sort_pairs: n out of range");
+  TBE_REQUIRE(end_bit >= 0 && end_bit <= 32, "tbe_sort_pairs: end_bit must be in [0, 32] (got %d)", end_bit);
+  if (n == 0) return TBE_OK;
+  TBE_REQUIRE(keys_in && keys_out && values_out, "tbe_sort_pairs: null pointer argument");
+  if (!workspace || workspace_bytes < sort_workspace_bytes(n))
+    return fail(TBE_ERR_WORKSPACE, "tbe_sort_pairs: workspace of %llu bytes needed, %llu given",
+                (unsigned long long)sort_workspace_bytes(n), (unsigned long long)workspace_bytes);
+  return sort_pairs(keys_in, values_in, keys_out, values_out, n, end_bit, workspace,
+                    static_cast<hipStream_t>(stream));
+}
+
+extern "C" uint64_t tbe_segments_workspace_bytes(int64_t n) { return tbe::segments_workspace_bytes(n); }
+
+extern "C" int tbe_find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts,
+                                 int32_t *num_unique, void *workspace, uint64_t workspace_bytes,
+                                 void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(n >= 0 && n < INT32_MAX, "tbe_find_segments: n out of range");
+  TBE_REQUIRE(segment_starts && num_unique, "tbe_find_segments: null pointer argument");
+  TBE_REQUIRE(keys_sorted || n == 0, "tbe_find_segments: null keys");
+  if (!workspace || workspace_bytes < segments_workspace_bytes(n))
+    return fail(TBE_ERR_WORKSPACE, "tbe_find_segments: workspace of %llu bytes needed, %llu given",
+                (unsigned long long)segments_workspace_bytes(n), (unsigned long long)workspace_bytes);
+  return find_segments(keys_sorted, n, segment_starts, num_unique, workspace,
+                       static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,55 @@
+// Host-side launchers of the backward stages, shared between the stage entry
+// points and the fused backward entry points.
+#pragma once
+
+#include "tbe_common.h"
+
+namespace tbe {
+
+int linearize(const int32_t *table_offsets, int32_t T, const int32_t *indices,
+              const int32_t *offsets, int32_t B, int32_t *keys, int32_t *grad_rows,
+              hipStream_t stream);
+
+uint64_t sort_workspace_bytes(int64_t n);
+int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
+               int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
+               hipStream_t stream);
+
+uint64_t segments_workspace_bytes(int64_t n);
+int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts,
+                  int32_t *num_unique, void *workspace, hipStream_t stream);
+
+// Segments longer than kLongSegment occurrences are cut into chunks of
+// kChunkLen occurrences that are reduced by separate wavefronts.
+constexpr int kLongSegment = 256;
+constexpr int kChunkLen = 256;
+
+enum { kOptSgd = 0, kOptAdagrad = 1 };
+
+struct UpdateArgs {
+  const void *grad_output;
+  void *weights;
+  void *optimizer_state;        // null for SGD
+  const void *per_sample_weights;  // null when unweighted
+  void *grad_per_sample_weights;
+  const int32_t *keys_sorted;
+  const int32_t *positions_sorted;
+  const int32_t *grad_rows;
+  const int32_t *segment_starts;
+  int32_t *counters;            // [0] = U (input), [1] = #long segments, [2] = #chunks
+  int32_t *long_segments;       // [2][max_long]
+  int32_t *chunk_segments;      // [max_chunks]
+  void *partial_sums;           // acc [max_chunks][D]
+  int64_t num_indices;
+  int64_t max_long;
+  int64_t max_chunks;
+  int32_t dtype;
+  int32_t D;
+  int32_t optimizer;
+  float learning_rate;
+  float eps;
+};
+
+int segment_update(const UpdateArgs &args, hipStream_t stream);
+
+}  // namespace tbe

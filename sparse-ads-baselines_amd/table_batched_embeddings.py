@@ -1,0 +1,248 @@
+"""Drop-in for the reference's `table_batched_embeddings` extension module.
+
+Same ten function names and positional signatures as the pybind11 module in
+table_batched_embeddings.cpp:56-70, taking torch tensors; each call validates
+its tensors, then hands raw device pointers and the current HIP stream to the
+C-ABI library (include/tbe_hip.h).  torch is used for device memory and streams
+only -- no arithmetic happens here.
+"""
+import ctypes
+
+import torch
+
+import tbe_native as _native
+
+_DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F16,
+                torch.float64: _native.DTYPE_F64}
+
+# One grow-only scratch buffer per device for the backward pipeline (keys, sort
+# buffers, segment lists).  The reference allocates these per call
+# (table_batched_embeddings_cuda.cu:1618-1647).
+_workspaces = {}
+# Storage of host-resident tensors handed out by new_*_tensor, keyed by data pointer.
+_host_allocations = {}
+
+
+def _require(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else ctypes.c_void_p(0)
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _check_common(weights, table_offsets, indices, offsets):
+    _require(weights.is_cuda, "weights must be a GPU tensor")
+    _require(weights.dim() == 2 and weights.is_contiguous(), "weights must be a contiguous [rows, D] tensor")
+    _require(weights.dtype in _DTYPE_CODES, "weights must be float16, float32 or float64")
+    for name, t in (("table_offsets", table_offsets), ("indices", indices), ("offsets", offsets)):
+        _require(t.dtype == torch.int32, "%s must be int32 (got %s)" % (name, t.dtype))
+        _require(t.is_cuda and t.device == weights.device, "%s must live on the weights' device" % name)
+        _require(t.dim() == 1 and t.is_contiguous(), "%s must be a contiguous 1-D tensor" % name)
+    T = table_offsets.numel()
+    _require(T > 0, "T must be positive")
+    B = (offsets.numel() - 1) // T  # table_batched_embeddings_cuda.cu:266
+    _require(B > 0, "B must be positive")
+    _require(offsets.numel() == T * B + 1, "offsets must hold T*B+1 entries")
+    return T, B
+
+
+def _workspace(device, nbytes):
+    ws = _workspaces.get(device)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=device)
+        _workspaces[device] = ws
+    return ws
+
+
+def backward_workspace(device):
+    """The scratch buffer last used by a backward call on `device` (for inspection)."""
+    return _workspaces.get(torch.device(device))
+
+
+def forward(weights, table_offsets, indices, offsets, indice_weights, L_max, BT_block_size, shmem):
+    """batched_embedding_forward_cuda (table_batched_embeddings_cuda.cu:253-316).
+
+    L_max, BT_block_size and shmem are the reference's launch knobs; results do
+    not depend on them and they are ignored apart from the BT_block_size != 0 check."""
+    T, B = _check_common(weights, table_offsets, indices, offsets)
+    _require(BT_block_size != 0, "BT_block_size must be non-zero")
+    D = weights.size(1)
+    if indice_weights is not None:
+        _require(indice_weights.dtype == weights.dtype, "indice_weights must have the weights' dtype")
+        _require(indice_weights.is_contiguous() and indice_weights.numel() == indices.numel(),
+                 "indice_weights must be contiguous with one entry per index")
+        _require(indice_weights.device == weights.device, "indice_weights must live on the weights' device")
+    output = torch.empty((B, T, D), dtype=weights.dtype, device=weights.device)
+    with torch.cuda.device(weights.device):
+        _native.check(_native.load().tbe_forward(
+            _ptr(weights), _DTYPE_CODES[weights.dtype], D, _ptr(table_offsets), T, _ptr(indices),
+            indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(output), _stream(weights.device)))
+    return output
+
+
+def _check_grad(grad_output, weights, T, B):
+    _require(grad_output.dtype == weights.dtype, "grad_output must have the weights' dtype")
+    _require(grad_output.device == weights.device, "grad_output must live on the weights' device")
+    _require(tuple(grad_output.shape) == (B, T, weights.size(1)), "grad_output must be [B, T, D]")
+    return grad_output.contiguous()
+
+
+def backward_sgd(grad_output, weights, table_offsets, indices, offsets, learning_rate, L_max,
+                 BT_block_size, shmem):
+    """batched_embedding_backward_sgd_cuda (table_batched_embeddings_cuda.cu:383-435), made
+    exact: every distinct row receives -lr * (sum of its gradients) once."""
+    T, B = _check_common(weights, table_offsets, indices, offsets)
+    _require(BT_block_size > 0, "BT_block_size must be positive")
+    grad_output = _check_grad(grad_output, weights, T, B)
+    D = weights.size(1)
+    code = _DTYPE_CODES[weights.dtype]
+    layout = _native.backward_workspace_layout(indices.numel(), D, code)
+    ws = _workspace(weights.device, layout.total_bytes)
+    with torch.cuda.device(weights.device):
+        _native.check(_native.load().tbe_backward_sgd(
+            _ptr(grad_output), _ptr(weights), code, weights.size(0), D, _ptr(table_offsets), T,
+            _ptr(indices), indices.numel(), _ptr(offsets), B, float(learning_rate), _ptr(ws), ws.numel(),
+            _stream(weights.device)))
+    return None
+
+
+def backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets, indice_weights,
+                           optimizer_state, learning_rate, eps, stochastic_rounding, BT_block_size):
+    """batched_embedding_backward_adagrad_exact_cuda (table_batched_embeddings_cuda.cu:1589-1706).
+
+    Returns the gradient w.r.t. indice_weights ([N], grad_output's dtype) or None when unweighted.
+    The weighted case, which the reference asserts out (:1678-1679), is served."""
+    T, B = _check_common(weights, table_offsets, indices, offsets)
+    _require(BT_block_size > 0, "BT_block_size must be positive")
+    if stochastic_rounding:
+        raise NotImplementedError("stochastic rounding is not implemented")
+    grad_output = _check_grad(grad_output, weights, T, B)
+    D = weights.size(1)
+    code = _DTYPE_CODES[weights.dtype]
+    state_dtype = torch.float64 if weights.dtype == torch.float64 else torch.float32
+    _require(optimizer_state.dtype == state_dtype, "optimizer_state must be %s" % state_dtype)
+    _require(optimizer_state.is_contiguous() and optimizer_state.numel() == weights.size(0),
+             "optimizer_state must be contiguous with one entry per row")
+    _require(optimizer_state.device == weights.device, "optimizer_state must live on the weights' device")
+    grad_indice_weights = None
+    if indice_weights is not None:
+        _require(indice_weights.dtype == weights.dtype, "indice_weights must have the weights' dtype")
+        _require(indice_weights.is_contiguous() and indice_weights.numel() == indices.numel(),
+                 "indice_weights must be contiguous with one entry per index")
+        grad_indice_weights = torch.empty(indices.shape, dtype=grad_output.dtype, device=weights.device)
+    layout = _native.backward_workspace_layout(indices.numel(), D, code)
+    ws = _workspace(weights.device, layout.total_bytes)
+    with torch.cuda.device(weights.device):
+        _native.check(_native.load().tbe_backward_exact_adagrad(
+            _ptr(grad_output), _ptr(weights), code, weights.size(0), D, _ptr(table_offsets), T,
+            _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state),
+            float(learning_rate), float(eps), _ptr(grad_indice_weights), _ptr(ws), ws.numel(),
+            _stream(weights.device)))
+    return grad_indice_weights
+
+
+def backward_approx_adagrad(grad_output, weights, table_offsets, indices, offsets, indice_weights,
+                            optimizer_state, learning_rate, eps, L_max, stochastic_rounding,
+                            BT_block_size):
+    """Signature of batched_embedding_backward_adagrad_approx_cuda
+    (table_batched_embeddings.cpp:17-21).  Served by the exact row-wise update, which coincides
+    with the approximate one whenever no row repeats across bags -- the only case the
+    reference tests (test_table_batched_embeddings.py:244)."""
+    return backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets, indice_weights,
+                                  optimizer_state, learning_rate, eps, stochastic_rounding, BT_block_size)
+
+
+def _mixed_d_unavailable(*args, **kwargs):
+    raise NotImplementedError("mixed-dimension tables are not served by this library")
+
+
+forward_mixed_D = _mixed_d_unavailable
+backward_approx_adagrad_mixed_D = _mixed_d_unavailable
+backward_exact_adagrad_mixed_D = _mixed_d_unavailable
+
+
+def construct_offsets(batch_offsets_per_table, total_indices_per_table):
+    """construct_offsets (table_batched_embeddings_cuda.cu:1190-1213): [T,B] bag starts and [T]
+    totals -> int32 [1+T*B] bag lengths with a leading zero; the caller cumsums."""
+    _require(batch_offsets_per_table.is_cuda, "batch_offsets_per_table must be a GPU tensor")
+    _require(batch_offsets_per_table.dim() == 2, "batch_offsets_per_table must be [T, B]")
+    _require(batch_offsets_per_table.dtype == torch.int32 and total_indices_per_table.dtype == torch.int32,
+             "construct_offsets takes int32 tensors")
+    _require(total_indices_per_table.device == batch_offsets_per_table.device,
+             "both arguments must live on one device")
+    T, B = batch_offsets_per_table.shape
+    _require(total_indices_per_table.numel() == T, "total_indices_per_table must be [T]")
+    per_table = batch_offsets_per_table.contiguous()
+    totals = total_indices_per_table.contiguous()
+    output = torch.empty(1 + T * B, dtype=torch.int32, device=per_table.device)
+    with torch.cuda.device(per_table.device):
+        _native.check(_native.load().tbe_construct_offsets(
+            _ptr(per_table), _ptr(totals), T, B, _ptr(output), _stream(per_table.device)))
+    return output
+
+
+class _DeviceArray:
+    """Exposes a raw device-visible address to torch through __cuda_array_interface__."""
+
+    def __init__(self, ptr, shape, typestr):
+        self.__cuda_array_interface__ = {"shape": tuple(shape), "typestr": typestr, "data": (ptr, False),
+                                         "version": 2, "strides": None}
+
+
+_TYPESTR = {torch.float32: "<f4", torch.float16: "<f2", torch.float64: "<f8"}
+
+
+def _wrap_host_memory(self, sizes, device_ptr, release):
+    numel = 1
+    for s in sizes:
+        numel *= int(s)
+    tensor = torch.as_tensor(_DeviceArray(device_ptr, (numel,), _TYPESTR[self.dtype]), device=self.device)
+    tensor = tensor.view(*[int(s) for s in sizes])
+    _host_allocations[tensor.data_ptr()] = release
+    return tensor
+
+
+def new_managed_tensor(self, sizes):
+    """new_managed_tensor (table_batched_embeddings_cuda.cu:864-871): a tensor tagged with
+    `self`'s device and dtype whose pages are managed memory preferring the host."""
+    _require(self.is_cuda and self.dtype in _TYPESTR, "prototype must be a floating GPU tensor")
+    nbytes = self.element_size()
+    for s in sizes:
+        nbytes *= int(s)
+    lib = _native.load()
+    ptr = ctypes.c_void_p()
+    with torch.cuda.device(self.device):
+        _native.check(lib.tbe_managed_alloc(nbytes, self.device.index or 0, ctypes.byref(ptr)))
+    address = ptr.value
+    return _wrap_host_memory(self, sizes, address, lambda: lib.tbe_managed_free(ctypes.c_void_p(address)))
+
+
+def new_host_mapped_tensor(self, sizes):
+    """new_host_mapped_tensor (table_batched_embeddings_cuda.cu:873-880): pinned host memory
+    mapped into the device's address space, tagged as a tensor on `self`'s device."""
+    _require(self.is_cuda and self.dtype in _TYPESTR, "prototype must be a floating GPU tensor")
+    nbytes = self.element_size()
+    for s in sizes:
+        nbytes *= int(s)
+    lib = _native.load()
+    host, dev = ctypes.c_void_p(), ctypes.c_void_p()
+    with torch.cuda.device(self.device):
+        _native.check(lib.tbe_host_mapped_alloc(nbytes, ctypes.byref(host), ctypes.byref(dev)))
+    host_address = host.value
+    return _wrap_host_memory(self, sizes, dev.value,
+                             lambda: lib.tbe_host_mapped_free(ctypes.c_void_p(host_address)))
+
+
+def free_host_tensor(tensor):
+    """Releases the storage behind a tensor made by new_managed_tensor / new_host_mapped_tensor.
+    The tensor (and every view of it) must not be used afterwards."""
+    release = _host_allocations.pop(tensor.data_ptr(), None)
+    _require(release is not None, "tensor was not allocated by this module")
+    torch.cuda.synchronize(tensor.device)
+    _native.check(release())

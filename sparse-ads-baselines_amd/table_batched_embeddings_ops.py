@@ -1,0 +1,122 @@
+"""Drop-in for the reference's table_batched_embeddings_ops.py (uniform-D part, :1-201).
+
+`TableBatchedEmbeddingBags` keeps the reference's constructor arguments, state-dict
+keys (`embedding_weights`, `table_offsets`, `optimizer_state`), flat `[sum(rows), D]`
+weight layout and `forward(indices, offsets, per_sample_weights)` signature; the
+optimizer is applied inside backward.  Differences, all extensions:
+  * `num_embeddings` may be a list of per-table row counts;
+  * SGD backward is exact (each distinct row updated once with its summed gradient);
+  * EXACT_ROWWISE_ADAGRAD accepts per-sample weights.
+"""
+import enum
+import logging
+
+import numpy as np
+import torch
+from torch import nn
+
+import table_batched_embeddings
+
+
+class Optimizer(enum.Enum):
+    SGD = 1
+    APPROX_ROWWISE_ADAGRAD = 2
+    EXACT_ROWWISE_ADAGRAD = 3
+
+
+class EmbeddingLocation(enum.Enum):
+    DEVICE = 0
+    HOST_MAPPED = 1
+
+
+def _launch_block(D):
+    # the reference's BT_block_size heuristic (table_batched_embeddings_ops.py:38);
+    # forwarded for signature compatibility, the kernels do not use it
+    return int(max(256 / D, 1))
+
+
+class LookupFunction(torch.autograd.Function):
+    """Mirror of LookupFunction (table_batched_embeddings_ops.py:9-121)."""
+
+    @staticmethod
+    def forward(ctx, weights, table_offsets, indices, offsets, per_sample_weights, optimizer,
+                optimizer_state, learning_rate, eps, stochastic_rounding):
+        ctx.optimizer = optimizer
+        ctx.learning_rate = learning_rate
+        ctx.eps = eps
+        ctx.stochastic_rounding = stochastic_rounding
+        ctx.save_for_backward(weights, table_offsets, indices, offsets, per_sample_weights, optimizer_state)
+        L_max = 200
+        return table_batched_embeddings.forward(
+            weights, table_offsets, indices, offsets, per_sample_weights, L_max,
+            _launch_block(weights.shape[1]), False)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (weights, table_offsets, indices, offsets, per_sample_weights, optimizer_state) = ctx.saved_tensors
+        L_max = 200
+        assert ctx.optimizer in (Optimizer.SGD, Optimizer.APPROX_ROWWISE_ADAGRAD,
+                                 Optimizer.EXACT_ROWWISE_ADAGRAD)
+        if ctx.optimizer == Optimizer.SGD:
+            assert per_sample_weights is None
+            grad_per_sample_weight = table_batched_embeddings.backward_sgd(
+                grad_output, weights, table_offsets, indices, offsets, ctx.learning_rate, L_max,
+                _launch_block(weights.shape[1]), False)
+        elif ctx.optimizer == Optimizer.APPROX_ROWWISE_ADAGRAD:
+            grad_per_sample_weight = table_batched_embeddings.backward_approx_adagrad(
+                grad_output, weights, table_offsets, indices, offsets, per_sample_weights,
+                optimizer_state, ctx.learning_rate, ctx.eps, L_max, ctx.stochastic_rounding, 1)
+        else:
+            grad_per_sample_weight = table_batched_embeddings.backward_exact_adagrad(
+                grad_output, weights, table_offsets, indices, offsets, per_sample_weights,
+                optimizer_state, ctx.learning_rate, ctx.eps, ctx.stochastic_rounding, 1)
+        # The update is already applied; autograd receives an empty sparse gradient of the
+        # weights' shape (table_batched_embeddings_ops.py:110-111), here in the weights' dtype.
+        empty_grad = None
+        if ctx.needs_input_grad[0]:
+            empty_grad = torch.sparse_coo_tensor(
+                torch.empty((2, 0), dtype=torch.int64, device=weights.device),
+                torch.empty((0,), dtype=weights.dtype, device=weights.device),
+                size=tuple(weights.shape))
+        return (empty_grad, None, None, None, grad_per_sample_weight, None, None, None, None, None)
+
+
+class TableBatchedEmbeddingBags(nn.Module):
+    """Mirror of TableBatchedEmbeddingBags (table_batched_embeddings_ops.py:135-201)."""
+
+    def __init__(self, num_tables, num_embeddings, embedding_dim, optimizer=Optimizer.SGD,
+                 learning_rate=0.01, eps=None, stochastic_rounding=False, fp16=False,
+                 managed=EmbeddingLocation.DEVICE):
+        super(TableBatchedEmbeddingBags, self).__init__()
+        assert managed in (EmbeddingLocation.DEVICE, EmbeddingLocation.HOST_MAPPED)
+        if isinstance(num_embeddings, (list, tuple, np.ndarray)):
+            rows = [int(r) for r in num_embeddings]
+            assert len(rows) == num_tables
+        else:
+            rows = [int(num_embeddings)] * num_tables
+        total_rows = int(sum(rows))
+        dtype = torch.float16 if fp16 else torch.float32
+        device = torch.device("cuda", torch.cuda.current_device())
+        if managed == EmbeddingLocation.DEVICE:
+            logging.info("Allocating device embedding bag")
+            embedding_data = torch.randn(total_rows, embedding_dim, device=device, dtype=dtype)
+        else:
+            logging.info("Allocating host-mapped embedding bag")
+            embedding_data = table_batched_embeddings.new_managed_tensor(
+                torch.empty(1, device=device, dtype=dtype), (total_rows, embedding_dim))
+            embedding_data.normal_()
+        self.embedding_weights = nn.Parameter(embedding_data)
+        self.register_buffer("table_offsets",
+                             torch.tensor([0] + np.cumsum(rows[:-1]).tolist()).int())
+        # unused by SGD, kept so state dicts interchange (table_batched_embeddings_ops.py:177-180)
+        self.register_buffer("optimizer_state", torch.zeros(total_rows).float())
+        self.optimizer = optimizer
+        self.learning_rate = learning_rate
+        self.eps = eps
+        self.stochastic_rounding = stochastic_rounding
+
+    def forward(self, sharded_sparse_features, sharded_offsets, per_sample_weights=None):
+        return LookupFunction.apply(
+            self.embedding_weights, self.table_offsets, sharded_sparse_features, sharded_offsets,
+            per_sample_weights, self.optimizer, self.optimizer_state, self.learning_rate, self.eps,
+            self.stochastic_rounding)

@@ -1,0 +1,334 @@
+"""GPU parity of the backward pipeline (linearize -> radix sort -> segments -> fused
+update) through the C ABI.  Integer stages are compared bit for bit with the oracle
+(sorted keys, stable positions, segment boundaries, U); updated weights / optimizer state /
+per-sample-weight gradients within the north star's tolerances: fp32 1e-5 relative,
+fp16 1e-2, fp64 1e-7 (the learning rate is a float on both sides, the sums differ in order)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN_CASES, load_golden, make_problem
+from gpu_util import DEV, assert_close, dev, gpu_backward, gpu_forward
+
+import table_batched_embeddings as ext
+import table_batched_embeddings_ops as ops
+import tbe_native
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float16): 1e-2, np.dtype(np.float64): 1e-7}
+
+
+def _sync():
+    torch.cuda.synchronize()
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _vp(t):
+    return ctypes.c_void_p(t.data_ptr() if t is not None and t.numel() else 0)
+
+
+# ------------------------------------------------------- stages, bit-exact
+@pytest.mark.parametrize("n,hi,end_bit", [(0, 10, 4), (1, 10, 4), (63, 2, 1), (64, 300, 9), (4095, 1 << 8, 8),
+                                          (4096, 1 << 16, 16), (4097, 1 << 23, 23), (100000, 7, 3),
+                                          (250001, 1 << 25, 25), (70000, 1 << 30, 31), (5000, 1000, 0)])
+def test_sort_pairs_is_stable_and_bit_exact(oracle, n, hi, end_bit):
+    rs = np.random.RandomState(n % 97)
+    keys = rs.randint(0, hi, size=n).astype(np.int32)
+    if n > 100:
+        keys[rs.randint(0, n, size=n // 3)] = keys[0]  # a hot key
+    lib = tbe_native.load()
+    k_in = dev(keys)
+    k_out = torch.full((max(n, 1),), -1, dtype=torch.int32, device=DEV)
+    v_out = torch.full((max(n, 1),), -1, dtype=torch.int32, device=DEV)
+    ws = torch.empty(lib.tbe_sort_workspace_bytes(n), dtype=torch.uint8, device=DEV)
+    tbe_native.check(lib.tbe_sort_pairs(_vp(k_in), _vp(None), _vp(k_out), _vp(v_out), n, end_bit, _vp(ws),
+                                        ws.numel(), _stream()))
+    _sync()
+    want_k, want_v = oracle.sort_pairs(keys, None, end_bit)
+    np.testing.assert_array_equal(k_out.cpu().numpy()[:n], want_k)
+    np.testing.assert_array_equal(v_out.cpu().numpy()[:n], want_v)
+    assert torch.equal(k_in.cpu(), torch.from_numpy(keys))  # input untouched
+    if end_bit >= 31 or hi <= (1 << end_bit):
+        np.testing.assert_array_equal(want_v, np.argsort(keys, kind="stable"))
+
+
+def test_sort_pairs_carries_arbitrary_values(oracle):
+    rs = np.random.RandomState(3)
+    n = 30000
+    keys = rs.randint(0, 1 << 12, size=n).astype(np.int32)
+    vals = rs.randint(-2 ** 31, 2 ** 31 - 1, size=n).astype(np.int32)
+    lib = tbe_native.load()
+    k_in, v_in = dev(keys), dev(vals)
+    k_out, v_out = (torch.empty(n, dtype=torch.int32, device=DEV) for _ in range(2))
+    ws = torch.empty(lib.tbe_sort_workspace_bytes(n), dtype=torch.uint8, device=DEV)
+    tbe_native.check(lib.tbe_sort_pairs(_vp(k_in), _vp(v_in), _vp(k_out), _vp(v_out), n, 12, _vp(ws),
+                                        ws.numel(), _stream()))
+    _sync()
+    want_k, want_v = oracle.sort_pairs(keys, vals, 12)
+    np.testing.assert_array_equal(k_out.cpu().numpy(), want_k)
+    np.testing.assert_array_equal(v_out.cpu().numpy(), want_v)
+
+
+@pytest.mark.parametrize("n,hi", [(0, 5), (1, 5), (2047, 3), (2048, 100000), (2049, 1), (300000, 120000)])
+def test_find_segments_bit_exact(oracle, n, hi):
+    keys = np.sort(np.random.RandomState(n % 89).randint(0, hi, size=n)).astype(np.int32)
+    lib = tbe_native.load()
+    starts = torch.full((n + 1,), -7, dtype=torch.int32, device=DEV)
+    count = torch.full((4,), -7, dtype=torch.int32, device=DEV)
+    ws = torch.empty(lib.tbe_segments_workspace_bytes(n), dtype=torch.uint8, device=DEV)
+    k_in = dev(keys)
+    tbe_native.check(lib.tbe_find_segments(_vp(k_in), n, _vp(starts), _vp(count), _vp(ws), ws.numel(),
+                                           _stream()))
+    _sync()
+    want = oracle.segments(keys)
+    U = int(count[0])
+    assert U == want.size - 1
+    np.testing.assert_array_equal(starts.cpu().numpy()[:U + 1], want)
+
+
+def test_linearize_and_construct_offsets_bit_exact(oracle):
+    p = make_problem(3, T=5, E=0, D=4, B=37, L=11, dtype=np.float32, rows=[5, 17, 3, 40, 1000])
+    lib = tbe_native.load()
+    keys, grows = (torch.empty(p["n"], dtype=torch.int32, device=DEV) for _ in range(2))
+    d_to, d_idx, d_off = dev(p["table_offsets"]), dev(p["indices"]), dev(p["offsets"])
+    tbe_native.check(lib.tbe_linearize(_vp(d_to), 5, _vp(d_idx), p["n"], _vp(d_off), 37, _vp(keys), _vp(grows),
+                                       _stream()))
+    _sync()
+    want_keys, b_t, _ = oracle.linearize(p["table_offsets"], p["indices"], p["offsets"])
+    np.testing.assert_array_equal(keys.cpu().numpy(), want_keys)
+    np.testing.assert_array_equal(grows.cpu().numpy(), (b_t % 37) * 5 + b_t // 37)
+    # construct_offsets, the check of test_table_batched_embeddings.py:97-105
+    lengths = np.diff(p["offsets"]).reshape(5, 37)
+    starts = np.concatenate([np.zeros((5, 1), int), np.cumsum(lengths, axis=1)[:, :-1]], axis=1).astype(np.int32)
+    totals = lengths.sum(axis=1).astype(np.int32)
+    got = ext.construct_offsets(dev(starts), dev(totals))
+    np.testing.assert_array_equal(got.cpu().numpy(), oracle.construct_offsets(starts, totals))
+    np.testing.assert_array_equal(torch.cumsum(got, 0).cpu().numpy(), p["offsets"])
+
+
+# --------------------------------------------------- fused backward vs oracle
+SHAPES = [(2, 1000, 32, 64, 4), (3, 50, 128, 33, 20), (1, 7, 4, 5, 3), (2, 100, 12, 17, 9), (2, 30, 520, 9, 5),
+          (4, 20, 64, 700, 40), (2, 100, 256, 50, 70), (1, 3, 8, 400, 9), (2, 64, 16, 31, 6)]
+
+
+def _run_both(oracle, p, optimizer, lr, eps):
+    w = p["weights"].copy()
+    st = np.zeros(w.shape[0], np.float64 if w.dtype == np.float64 else np.float32)
+    ref = oracle.backward(optimizer, p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], lr, eps,
+                          st, p.get("per_sample_weights"))
+    got = gpu_backward(p, optimizer, lr, eps)
+    return w, st, ref, got
+
+
+def _check(p, w, st, ref, got, optimizer):
+    tol = TOL[p["weights"].dtype]
+    v = got["views"]
+    if p["n"]:
+        np.testing.assert_array_equal(v["keys_sorted"], ref["keys_sorted"])
+        np.testing.assert_array_equal(v["positions_sorted"], ref["positions_sorted"])
+        np.testing.assert_array_equal(v["segment_starts"], ref["segment_starts"])
+        assert v["num_unique"] == ref["segment_starts"].size - 1
+    assert_close(got["weights"], w, tol, "weights")
+    # rows no lookup touches must keep their bits
+    touched = np.zeros(w.shape[0], bool)
+    touched[ref["keys_sorted"]] = True
+    assert got["weights"][~touched].tobytes() == p["weights"][~touched].tobytes()
+    if optimizer == "adagrad":
+        assert_close(got["state"], st, 1e-3 if p["weights"].dtype == np.float16 else max(tol, 1e-6), "state")
+        assert not got["state"][~touched].any()
+    if ref["grad_psw"] is not None:
+        assert_close(got["grad_psw"], ref["grad_psw"], tol, "grad_psw")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.float64])
+@pytest.mark.parametrize("mode", ["sgd", "adagrad", "adagrad_weighted"])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_backward_matches_oracle(oracle, shape, mode, dtype):
+    T, E, D, B, L = shape
+    p = make_problem(hash(shape) % 1000 + 1, T, E, D, B, L, dtype, ragged=True, weighted=mode.endswith("weighted"),
+                     zipf=1.2)
+    optimizer = "sgd" if mode == "sgd" else "adagrad"
+    w, st, ref, got = _run_both(oracle, p, optimizer, 0.05, 0.1)
+    _check(p, w, st, ref, got, optimizer)
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_backward_matches_embeddingbag_fixture(name):
+    g = load_golden(name)
+    g["table_offsets"] = (np.arange(g["T"]) * g["E"]).astype(np.int32)
+    g["n"] = g["indices"].size
+    got = gpu_backward(g, g["optimizer"], g["lr"], g["eps"])
+    tol = TOL[g["weights"].dtype]
+    assert_close(got["weights"], g["expected_weights"], tol)
+    if g["optimizer"] == "adagrad":
+        assert_close(got["state"], g["expected_state"], 1e-3 if g["weights"].dtype == np.float16 else 1e-5)
+    if "expected_grad_psw" in g:
+        assert_close(got["grad_psw"], g["expected_grad_psw"], tol)
+
+
+@pytest.mark.parametrize("dtype,D", [(np.float32, 128), (np.float16, 64), (np.float32, 12), (np.float64, 8)])
+@pytest.mark.parametrize("mode", ["sgd", "adagrad_weighted"])
+def test_hot_rows_take_the_chunked_path(oracle, dtype, D, mode):
+    """Segments far longer than one lane group handles: one row receives ~70 % of 60 k lookups,
+    others land on both sides of the 256-occurrence threshold."""
+    rs = np.random.RandomState(5)
+    T, E, B, L = 2, 50, 3000, 10
+    p = make_problem(9, T, E, D, B, L, dtype, ragged=False, weighted=mode.endswith("weighted"))
+    n = p["n"]
+    hot = rs.rand(n) < 0.7
+    p["indices"][hot] = 7
+    p["indices"][~hot] = rs.choice([1, 2, 3, 40, 41], size=(~hot).sum(), p=[0.5, 0.3, 0.19, 0.006, 0.004])
+    optimizer = "sgd" if mode == "sgd" else "adagrad"
+    w, st, ref, got = _run_both(oracle, p, optimizer, 0.001, 0.1)
+    lengths = np.diff(ref["segment_starts"])
+    assert lengths.max() > 15000 and (lengths <= 256).any() and ((lengths > 256) & (lengths < 2000)).any()
+    assert got["views"]["counters"][1] == (lengths > 256).sum()
+    assert got["views"]["counters"][2] == np.ceil(lengths[lengths > 256] / 256).sum()
+    # long serial fp32 sums: the oracle itself is ~1e-4 from the fp64 truth here, so compare
+    # both against each other at the accumulated-rounding level
+    tol = {np.dtype(np.float32): 2e-4, np.dtype(np.float16): 1e-2, np.dtype(np.float64): 1e-7}[np.dtype(dtype)]
+    np.testing.assert_array_equal(got["views"]["positions_sorted"], ref["positions_sorted"])
+    np.testing.assert_array_equal(got["views"]["segment_starts"], ref["segment_starts"])
+    assert_close(got["weights"], w, tol)
+    if optimizer == "adagrad":
+        assert_close(got["state"], st, 1e-3)
+        assert_close(got["grad_psw"], ref["grad_psw"], TOL[np.dtype(dtype)])
+
+
+def test_two_backward_runs_are_bit_identical():
+    p = make_problem(12, T=3, E=40, D=128, B=2000, L=12, dtype=np.float32, weighted=True, zipf=1.1)
+    a = gpu_backward(p, "adagrad", 0.05, 0.1)
+    b = gpu_backward(p, "adagrad", 0.05, 0.1)
+    for k in ("weights", "state", "grad_psw"):
+        assert a[k].tobytes() == b[k].tobytes()
+
+
+def test_zero_gradient_and_empty_input_leave_weights_untouched():
+    p = make_problem(13, T=2, E=100, D=64, B=50, L=6, dtype=np.float32)
+    p["grad_output"][:] = 0
+    assert gpu_backward(p, "sgd", 0.5)["weights"].tobytes() == p["weights"].tobytes()
+    p0 = make_problem(14, T=2, E=100, D=64, B=5, L=0, dtype=np.float32)
+    assert gpu_backward(p0, "sgd", 0.5)["weights"].tobytes() == p0["weights"].tobytes()
+
+
+def test_second_adagrad_step_accumulates_state(oracle):
+    p = make_problem(15, T=2, E=30, D=32, B=40, L=5, dtype=np.float32, zipf=1.3)
+    w = p["weights"].copy()
+    st = np.zeros(60, np.float32)
+    for _ in range(2):
+        oracle.backward("adagrad", p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], 0.05, 0.1, st)
+    first = gpu_backward(p, "adagrad", 0.05, 0.1)
+    p2 = dict(p, weights=first["weights"])
+    second = gpu_backward(p2, "adagrad", 0.05, 0.1, state=first["state"])
+    assert_close(second["state"], st, 1e-5)
+    assert_close(second["weights"], w, 1e-5)
+
+
+# ------------------------------------------------------------- module API
+def test_module_backward_sgd_like_the_reference_test(oracle):
+    """test_table_batched_embeddings.py:163-216 through the drop-in module, but with repeated
+    rows (the reference needs sampling without replacement)."""
+    T, E, D, B, L = 3, 200, 64, 32, 8
+    p = make_problem(16, T, E, D, B, L, np.float32, ragged=False, zipf=1.2)
+    cc = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.SGD, learning_rate=0.05).cuda()
+    cc.embedding_weights.data.copy_(dev(p["weights"]))
+    out = cc(dev(p["indices"]), dev(p["offsets"]))
+    out.backward(dev(p["grad_output"]))
+    w = p["weights"].copy()
+    oracle.backward("sgd", p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], 0.05)
+    assert_close(cc.embedding_weights.detach().cpu().numpy(), w, 1e-5)
+    g = cc.embedding_weights.grad
+    assert g is None or (g.is_sparse and g._nnz() == 0 and g.dtype == torch.float32)
+
+
+@pytest.mark.parametrize("fp16", [False, True])
+@pytest.mark.parametrize("optimizer", [ops.Optimizer.EXACT_ROWWISE_ADAGRAD, ops.Optimizer.APPROX_ROWWISE_ADAGRAD])
+def test_module_backward_adagrad_like_the_reference_test(oracle, optimizer, fp16):
+    # test_table_batched_embeddings.py:219-318: lr=0.5, eps=0.2; exact => E=100 with replacement
+    exact = optimizer == ops.Optimizer.EXACT_ROWWISE_ADAGRAD
+    T, E, D, B, L = 4, (100 if exact else 10000), 32, 64, 6
+    dtype = np.float16 if fp16 else np.float32
+    rs = np.random.RandomState(17)
+    p = make_problem(17, T, E, D, B, L, dtype, ragged=False)
+    if not exact:  # the approximate optimizer is only specified when no row repeats (:244)
+        p["indices"] = np.concatenate([rs.choice(E, size=B * L, replace=False) for _ in range(T)]).astype(np.int32)
+    cc = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=optimizer, learning_rate=0.5, eps=0.2, fp16=fp16).cuda()
+    cc.embedding_weights.data.copy_(dev(p["weights"]))
+    cc(dev(p["indices"]), dev(p["offsets"])).backward(dev(p["grad_output"]))
+    w = p["weights"].copy()
+    st = np.zeros(T * E, np.float32)
+    oracle.backward("adagrad", p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], 0.5, 0.2, st)
+    assert_close(cc.optimizer_state.cpu().numpy(), st, 1e-3 if fp16 else 1e-5)
+    assert_close(cc.embedding_weights.detach().cpu().numpy(), w, 1e-2 if fp16 else 1e-5)
+
+
+def test_gradcheck_on_per_sample_weights_in_double():
+    # test_table_batched_embeddings.py:320-340: lr = 0, module in double, gradcheck on per_sample_weights
+    T, E, D, B, L = 2, 50, 8, 5, 3
+    p = make_problem(18, T, E, D, B, L, np.float64, ragged=False, weighted=True)
+    cc = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.EXACT_ROWWISE_ADAGRAD, learning_rate=0.0,
+                                       eps=0.2).cuda().double()
+    cc.embedding_weights.requires_grad = False
+    psw = dev(p["per_sample_weights"]).requires_grad_(True)
+    assert torch.autograd.gradcheck(cc, (dev(p["indices"]), dev(p["offsets"]), psw))
+
+
+def test_full_size_backward_properties():
+    """BASELINE config 3 shape (T=64, E=1e5, D=128 fp32, B=4096, L=20, Zipf(1.05) indices,
+    exact SGD lr=0.01).  Size-independent properties instead of the oracle:
+    sortedness + permutation + stability of the sort, key/position consistency, strict
+    segment boundaries, the column checksum of the update (linearity), untouched rows
+    bit-identical, and the first table against the oracle."""
+    from oracle import tbe_oracle
+    T, E, D, B, L = 64, 100000, 128, 4096, 20
+    rs = np.random.RandomState(0)
+    idx_np = (rs.zipf(1.05, size=T * B * L) % E).astype(np.int32)
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    W = torch.empty(T * E, D, device=DEV).uniform_(-0.01, 0.01, generator=gen)
+    W0 = W.clone()
+    go = torch.randn(B, T, D, device=DEV, generator=gen)
+    idx = torch.from_numpy(idx_np).to(DEV)
+    offsets = torch.arange(0, T * B * L + 1, L, dtype=torch.int32, device=DEV)
+    table_offsets = torch.arange(T, dtype=torch.int32, device=DEV) * E
+    ext.backward_sgd(go, W, table_offsets, idx, offsets, 0.01, 200, 1, False)
+    _sync()
+    n = T * B * L
+    lay = tbe_native.backward_workspace_layout(n, D, tbe_native.DTYPE_F32)
+    ws = ext.backward_workspace(torch.device(DEV))
+    view = lambda off, cnt: ws[off:off + 4 * cnt].view(torch.int32)
+    keys, ks, ps = view(lay.keys, n), view(lay.keys_sorted, n), view(lay.positions_sorted, n)
+    U = int(view(lay.num_unique, 1)[0])
+    ss = view(lay.segment_starts, U + 1).long()
+    want_keys = idx.long() + torch.arange(T, device=DEV).repeat_interleave(B * L) * E
+    assert torch.equal(keys.long(), want_keys)
+    assert bool((ks[1:] >= ks[:-1]).all())                                   # sorted
+    assert torch.equal(torch.sort(ps.long())[0], torch.arange(n, device=DEV))  # permutation
+    assert torch.equal(keys[ps.long()], ks)                                   # pairs stayed together
+    same = ks[1:] == ks[:-1]
+    assert bool((ps[1:][same] > ps[:-1][same]).all())                         # stable
+    assert U == int(torch.unique(want_keys).numel())
+    assert int(ss[0]) == 0 and int(ss[-1]) == n and bool((ss[1:] > ss[:-1]).all())
+    assert bool((ks[ss[1:-1]] != ks[ss[1:-1] - 1]).all())                     # every start is a head
+    heads = torch.ones(n, dtype=torch.bool, device=DEV)
+    heads[1:] = ks[1:] != ks[:-1]
+    assert int(heads.sum()) == U
+    # linearity checksum: sum over rows of (W0 - W) == lr * sum_p go[grad_row(p)]
+    counts = torch.bincount(torch.arange(T * B, device=DEV).repeat_interleave(L), minlength=T * B)
+    bag_weight = counts.view(T, B).t().contiguous().double()                  # [B][T] lookups per bag
+    want_col = 0.01 * (go.double() * bag_weight.unsqueeze(-1)).sum((0, 1))
+    got_col = (W0.double() - W.double()).sum(0)
+    assert_close(got_col.cpu().numpy(), want_col.cpu().numpy(), 1e-5)
+    touched = torch.zeros(T * E, dtype=torch.bool, device=DEV)
+    touched[want_keys] = True
+    assert torch.equal(W[~touched], W0[~touched])
+    # first table against the oracle (81 920 lookups)
+    w_ref = W0[:E].cpu().numpy().copy()
+    tbe_oracle.backward("sgd", go[:, :1, :].contiguous().cpu().numpy(), w_ref, np.zeros(1, np.int32), idx_np[:B * L],
+                        offsets[:B + 1].cpu().numpy(), 0.01)
+    assert_close(W[:E].cpu().numpy(), w_ref, 1e-5)

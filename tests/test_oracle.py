@@ -1,0 +1,238 @@
+"""Pins the CPU oracle (oracle/tbe_oracle.c) before anything is compared with it.
+
+The reference holds no golden vectors for this path (every reference test draws random
+data and compares with torch.nn.EmbeddingBag at run time), so the oracle is pinned by:
+  * committed fixtures produced with the reference test-suite's own oracle -- per-table
+    torch.nn.EmbeddingBag + the Python optimizer (tests/golden/make_golden.py);
+  * library routines: numpy's stable argsort, numpy.unique, numpy.float16 conversion;
+  * closed forms and special cases (single-lookup bags copy rows, unit weights equal the
+    unweighted sum, a row hit once by Adagrad has state |g|^2, untouched rows keep their
+    bits, linearity of the SGD update in the gradient);
+  * brute force on tiny inputs.
+Each check is chosen so that a dropped term, a transposed [B][T] / [T][B] index, a wrong
+sort bit range or a multiplier built from the old state fails it.
+"""
+import numpy as np
+import pytest
+
+from conftest import GOLDEN_CASES, load_golden, make_problem
+
+
+def table_offsets_of(g):
+    return (np.arange(g["T"]) * g["E"]).astype(np.int32)
+
+
+# ------------------------------------------------------------------ fixtures
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_forward_matches_embeddingbag_fixture(oracle, name):
+    g = load_golden(name)
+    out = oracle.forward(g["weights"], table_offsets_of(g), g["indices"], g["offsets"], g.get("per_sample_weights"))
+    assert out.shape == (g["B"], g["T"], g["D"])
+    tol = 2e-3 if g["weights"].dtype == np.float16 else 1e-5
+    scale = np.abs(g["expected_output"]).max()
+    np.testing.assert_allclose(out.astype(np.float64), g["expected_output"], rtol=tol, atol=tol * scale)
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_backward_matches_embeddingbag_fixture(oracle, name):
+    g = load_golden(name)
+    w = g["weights"].copy()
+    state = np.zeros(w.shape[0], np.float64 if w.dtype == np.float64 else np.float32)
+    r = oracle.backward(g["optimizer"], g["grad_output"], w, table_offsets_of(g), g["indices"], g["offsets"],
+                        g["lr"], g["eps"], state, g.get("per_sample_weights"))
+    half = w.dtype == np.float16
+    tol = 1e-2 if half else 1e-5
+    scale = np.abs(g["expected_weights"]).max()
+    np.testing.assert_allclose(w.astype(np.float64), g["expected_weights"], rtol=tol, atol=tol * scale)
+    if g["optimizer"] == "adagrad":
+        np.testing.assert_allclose(state.astype(np.float64), g["expected_state"], rtol=1e-3 if half else 1e-5,
+                                   atol=1e-30)
+    if "expected_grad_psw" in g:
+        gs = np.abs(g["expected_grad_psw"]).max()
+        np.testing.assert_allclose(r["grad_psw"].astype(np.float64), g["expected_grad_psw"], rtol=tol,
+                                   atol=tol * gs)
+
+
+def test_live_embeddingbag_agrees(oracle):
+    """Same comparison against torch.nn.EmbeddingBag computed now (guards a stale fixture)."""
+    torch = pytest.importorskip("torch")
+    p = make_problem(11, T=3, E=40, D=24, B=21, L=7, dtype=np.float32, weighted=True, zipf=1.3)
+    out = oracle.forward(p["weights"], p["table_offsets"], p["indices"], p["offsets"], p["per_sample_weights"])
+    for t in range(p["T"]):
+        lo, hi = p["offsets"][t * p["B"]], p["offsets"][(t + 1) * p["B"]]
+        w = torch.from_numpy(p["weights"][t * 40:(t + 1) * 40].copy())
+        y = torch.nn.functional.embedding_bag(
+            torch.from_numpy(p["indices"][lo:hi].astype(np.int64)), w,
+            torch.from_numpy((p["offsets"][t * p["B"]:(t + 1) * p["B"]] - lo).astype(np.int64)), mode="sum",
+            per_sample_weights=torch.from_numpy(p["per_sample_weights"][lo:hi].copy()))
+        np.testing.assert_allclose(out[:, t, :], y.numpy(), rtol=1e-5, atol=1e-8)
+
+
+# ------------------------------------------------------------- fp16 rounding
+def test_half_conversions_match_numpy(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    as_float = bits.view(np.float16).astype(np.float32)
+    for b in range(0, 65536, 1):
+        f = oracle.half_to_float(b)
+        if np.isnan(as_float[b]):
+            assert np.isnan(f)
+        else:
+            assert f == as_float[b] and np.signbit(f) == np.signbit(as_float[b])
+    rs = np.random.RandomState(0)
+    vals = np.concatenate([rs.randn(20000).astype(np.float32) * 10.0 ** rs.randint(-9, 6, size=20000),
+                           np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8,
+                                     6.1e-5, 6.09e-5, np.inf, -np.inf], dtype=np.float32),
+                           # exact ties between neighbouring halves
+                           ((bits[:0x7bff].view(np.float16).astype(np.float64) +
+                             (bits[:0x7bff] + 1).astype(np.uint16).view(np.float16).astype(np.float64)) / 2)
+                           .astype(np.float32)]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([oracle.float_to_half(v) for v in vals], dtype=np.uint16)
+    np.testing.assert_array_equal(got, want)
+
+
+# ------------------------------------------------------- integer stages, bit-exact
+@pytest.mark.parametrize("seed,n,hi,end_bit", [(0, 0, 10, 4), (1, 1, 10, 4), (2, 5000, 7, 3), (3, 70000, 1 << 23, 23),
+                                               (4, 4097, 300, 9), (5, 33333, 1 << 17, 25)])
+def test_sort_is_stable_argsort(oracle, seed, n, hi, end_bit):
+    rs = np.random.RandomState(seed)
+    keys = rs.randint(0, hi, size=n).astype(np.int32)
+    ks, vs = oracle.sort_pairs(keys, None, end_bit)
+    order = np.argsort(keys, kind="stable")
+    np.testing.assert_array_equal(ks, keys[order])
+    np.testing.assert_array_equal(vs, order.astype(np.int32))
+
+
+def test_sort_ignores_bits_above_end_bit(oracle):
+    # CUB's contract: only bits [0, end_bit) take part; equal low bits keep input order
+    keys = np.array([0x105, 0x003, 0x205, 0x103, 0x001], np.int32)
+    ks, vs = oracle.sort_pairs(keys, None, 8)
+    np.testing.assert_array_equal(vs, [4, 1, 3, 0, 2])
+    np.testing.assert_array_equal(ks, keys[[4, 1, 3, 0, 2]])
+
+
+def test_sort_brute_force_tiny(oracle):
+    rs = np.random.RandomState(7)
+    for _ in range(50):
+        n = rs.randint(0, 12)
+        keys = rs.randint(0, 4, size=n).astype(np.int32)
+        vals = rs.randint(0, 1000, size=n).astype(np.int32)
+        ks, vs = oracle.sort_pairs(keys, vals, 2)
+        want = sorted(zip(keys.tolist(), range(n)), key=lambda kv: kv[0])  # python's sort is stable
+        assert ks.tolist() == [k for k, _ in want]
+        assert vs.tolist() == [int(vals[i]) for _, i in want]
+
+
+@pytest.mark.parametrize("seed,n,hi", [(0, 0, 5), (1, 1, 5), (2, 1000, 3), (3, 50000, 40000), (4, 777, 1)])
+def test_segments_match_numpy_unique(oracle, seed, n, hi):
+    keys = np.sort(np.random.RandomState(seed).randint(0, hi, size=n)).astype(np.int32)
+    starts = oracle.segments(keys)
+    uniq, first = np.unique(keys, return_index=True)
+    np.testing.assert_array_equal(starts[:-1], first.astype(np.int32))
+    assert starts[-1] == n and starts.size == uniq.size + 1
+
+
+def test_linearize_closed_form(oracle):
+    p = make_problem(3, T=4, E=0, D=4, B=9, L=6, dtype=np.float32, rows=[5, 17, 3, 40])
+    keys, b_t, idx = oracle.linearize(p["table_offsets"], p["indices"], p["offsets"])
+    bag = np.repeat(np.arange(p["T"] * p["B"]), np.diff(p["offsets"]))
+    np.testing.assert_array_equal(b_t, bag)
+    np.testing.assert_array_equal(idx, np.arange(p["n"]))
+    np.testing.assert_array_equal(keys, p["table_offsets"][bag // p["B"]] + p["indices"])
+
+
+def test_construct_offsets_closed_form(oracle):
+    # the check of test_table_batched_embeddings.py:97-105
+    rs = np.random.RandomState(5)
+    T, B = 7, 13
+    lengths = rs.randint(1, 20, size=(T, B))
+    starts = np.concatenate([np.zeros((T, 1), int), np.cumsum(lengths, axis=1)[:, :-1]], axis=1).astype(np.int32)
+    totals = lengths.sum(axis=1).astype(np.int32)
+    out = oracle.construct_offsets(starts, totals)
+    assert out[0] == 0
+    np.testing.assert_array_equal(out[1:], lengths.reshape(-1))
+    np.testing.assert_array_equal(np.cumsum(out), np.concatenate([[0], np.cumsum(lengths.reshape(-1))]))
+
+
+# ------------------------------------------------------------- special cases
+def test_single_lookup_bags_copy_rows_bit_exact(oracle):
+    p = make_problem(1, T=3, E=25, D=12, B=10, L=1, dtype=np.float32, ragged=False)
+    out = oracle.forward(p["weights"], p["table_offsets"], p["indices"], p["offsets"])
+    for t in range(3):
+        for b in range(10):
+            row = p["table_offsets"][t] + p["indices"][t * 10 + b]
+            assert out[b, t].tobytes() == p["weights"][row].tobytes()  # [B][T] order, not [T][B]
+
+
+def test_empty_bags_give_zeros_and_unit_weights_equal_unweighted(oracle):
+    p = make_problem(2, T=2, E=30, D=8, B=50, L=3, dtype=np.float32)
+    out = oracle.forward(p["weights"], p["table_offsets"], p["indices"], p["offsets"])
+    empty = np.diff(p["offsets"]) == 0
+    assert empty.any()
+    for bag in np.nonzero(empty)[0]:
+        assert not out[bag % 50, bag // 50].any()
+    ones = np.ones(p["n"], np.float32)
+    out_w = oracle.forward(p["weights"], p["table_offsets"], p["indices"], p["offsets"], ones)
+    assert out_w.tobytes() == out.tobytes()
+
+
+def test_sgd_untouched_rows_keep_bits_and_update_is_linear(oracle):
+    p = make_problem(4, T=2, E=200, D=16, B=12, L=5, dtype=np.float64, zipf=1.1)
+    w1, w2, w12 = p["weights"].copy(), p["weights"].copy(), p["weights"].copy()
+    g1 = p["grad_output"]
+    g2 = np.random.RandomState(9).randn(*g1.shape)
+    for w, g in ((w1, g1), (w2, g2), (w12, g1 + g2)):
+        oracle.backward("sgd", g, w, p["table_offsets"], p["indices"], p["offsets"], 0.25)
+    keys = oracle.linearize(p["table_offsets"], p["indices"], p["offsets"])[0]
+    untouched = np.setdiff1d(np.arange(400), keys)
+    assert untouched.size and w1[untouched].tobytes() == p["weights"][untouched].tobytes()
+    np.testing.assert_allclose((w1 - p["weights"]) + (w2 - p["weights"]), w12 - p["weights"], rtol=1e-12, atol=1e-15)
+    # closed form: w - lr * scatter-add of gradient rows
+    G = np.zeros_like(p["weights"])
+    bag = np.repeat(np.arange(24), np.diff(p["offsets"]))
+    np.add.at(G, keys, g1[bag % 12, bag // 12])
+    np.testing.assert_allclose(w1, p["weights"] - 0.25 * G, rtol=1e-12, atol=1e-15)
+
+
+def test_adagrad_single_hit_closed_form_and_second_step_uses_new_state(oracle):
+    # one table, one bag, one lookup: state = |g|^2, w -= lr / (|g| + eps) * g
+    w = np.full((3, 4), 0.5, np.float64)
+    g = np.array([[[3.0, 0.0, 4.0, 0.0]]])
+    state = np.zeros(3)
+    args = (np.array([0], np.int32), np.array([1], np.int32), np.array([0, 1], np.int32))
+    oracle.backward("adagrad", g, w, *args, lr=0.5, eps=0.2, optimizer_state=state)
+    assert state.tolist() == [0.0, 25.0, 0.0]
+    np.testing.assert_allclose(w[1], 0.5 - 0.5 / (5.0 + float(np.float32(0.2))) * g[0, 0], rtol=1e-15)
+    assert (w[0] == 0.5).all() and (w[2] == 0.5).all()
+    # second step: multiplier is built from old + new (tbe.cu:453-454), i.e. sqrt(50), not sqrt(25)
+    before = w[1].copy()
+    oracle.backward("adagrad", g, w, *args, lr=0.5, eps=0.2, optimizer_state=state)
+    assert state[1] == 50.0
+    np.testing.assert_allclose(w[1], before - 0.5 / (np.sqrt(50.0) + float(np.float32(0.2))) * g[0, 0],
+                               rtol=1e-15)
+
+
+def test_grad_psw_is_dot_with_weights_before_update(oracle):
+    p = make_problem(6, T=2, E=10, D=8, B=6, L=4, dtype=np.float64, weighted=True, zipf=1.5)
+    w = p["weights"].copy()
+    state = np.zeros(20)
+    r = oracle.backward("adagrad", p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], 0.3, 0.1,
+                        state, p["per_sample_weights"])
+    keys = oracle.linearize(p["table_offsets"], p["indices"], p["offsets"])[0]
+    bag = np.repeat(np.arange(12), np.diff(p["offsets"]))
+    want = np.einsum("nd,nd->n", p["weights"][keys], p["grad_output"][bag % 6, bag // 6])
+    np.testing.assert_allclose(r["grad_psw"], want, rtol=1e-12, atol=1e-18)
+    # duplicates make rows change during the pass; the result must still use the old rows
+    assert np.unique(keys).size < keys.size
+
+
+def test_backward_intermediates_are_sort_and_unique_of_keys(oracle):
+    p = make_problem(8, T=3, E=0, D=4, B=20, L=6, dtype=np.float32, zipf=1.2, rows=[7, 300, 41])
+    w = p["weights"].copy()
+    r = oracle.backward("sgd", p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], 0.1)
+    keys = oracle.linearize(p["table_offsets"], p["indices"], p["offsets"])[0]
+    order = np.argsort(keys, kind="stable")
+    np.testing.assert_array_equal(r["keys_sorted"], keys[order])
+    np.testing.assert_array_equal(r["positions_sorted"], order)
+    np.testing.assert_array_equal(r["segment_starts"][:-1], np.unique(keys[order], return_index=True)[1])
