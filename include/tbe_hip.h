@@ -51,6 +51,19 @@ TBE_API const char *tbe_last_error(void);
 /* ABI version; bumped whenever a signature below changes. */
 TBE_API int32_t tbe_abi_version(void);
 
+/* ---------------------------------------------------------- kernel timing
+ * Benchmark aid with no counterpart in the reference (it times whole calls with
+ * CUDA events, table_batched_embeddings_benchmark.py:27-37).  Between
+ * tbe_profile_begin() and tbe_profile_end() every kernel launch of this library
+ * is bracketed by two HIP events recorded on the launch stream.
+ * tbe_profile_end() waits for those events; tbe_profile_get(i, ...) then returns
+ * the kernel's short name and its duration in milliseconds, in launch order.
+ */
+TBE_API int tbe_profile_begin(void);
+TBE_API int tbe_profile_end(void);
+TBE_API int32_t tbe_profile_count(void);
+TBE_API int tbe_profile_get(int32_t i, const char **name, float *milliseconds);
+
 /* ------------------------------------------------------------------ forward
  * Pooled gather-sum:  output[b][t][:] = sum_{p in bag(t,b)} (psw[p] *) weights[table_offsets[t] + indices[p]][:]
  * Replaces batched_embedding_forward_cuda (table_batched_embeddings_cuda.cu:253-316,

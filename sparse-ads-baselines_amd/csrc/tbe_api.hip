@@ -3,6 +3,9 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+#include <vector>
+
 #include "tbe_common.h"
 
 namespace tbe {
@@ -23,6 +26,46 @@ int check_launch(const char *what) {
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TBE_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
   return TBE_OK;
+}
+
+// ------------------------------------------------------------ launch profiling
+namespace {
+struct TimedLaunch {
+  const char *name;
+  hipEvent_t start, stop;
+  float ms;
+};
+std::mutex g_profile_mutex;
+std::vector<TimedLaunch> g_profile;      // launches recorded since tbe_profile_begin
+std::vector<hipEvent_t> g_event_pool;    // events kept for reuse
+bool g_profiling = false;
+
+hipEvent_t take_event() {
+  if (!g_event_pool.empty()) {
+    hipEvent_t e = g_event_pool.back();
+    g_event_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) return nullptr;
+  return e;
+}
+}  // namespace
+
+LaunchTimer::LaunchTimer(const char *name, hipStream_t s) : slot(-1), stream(s) {
+  if (!g_profiling) return;
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  TimedLaunch t{name, take_event(), take_event(), 0.0f};
+  if (!t.start || !t.stop) return;
+  (void)hipEventRecord(t.start, stream);
+  slot = static_cast<int>(g_profile.size());
+  g_profile.push_back(t);
+}
+
+LaunchTimer::~LaunchTimer() {
+  if (slot < 0) return;
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  (void)hipEventRecord(g_profile[slot].stop, stream);
 }
 
 namespace {
@@ -48,7 +91,46 @@ __global__ __launch_bounds__(kBlockThreads) void construct_offsets_kernel(
 
 extern "C" const char *tbe_last_error(void) { return tbe::g_last_error; }
 
-extern "C" int32_t tbe_abi_version(void) { return 1; }
+extern "C" int32_t tbe_abi_version(void) { return 2; }
+
+extern "C" int tbe_profile_begin(void) {
+  using namespace tbe;
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  for (TimedLaunch &t : g_profile) {
+    g_event_pool.push_back(t.start);
+    g_event_pool.push_back(t.stop);
+  }
+  g_profile.clear();
+  g_profiling = true;
+  return TBE_OK;
+}
+
+extern "C" int tbe_profile_end(void) {
+  using namespace tbe;
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  g_profiling = false;
+  for (TimedLaunch &t : g_profile) {
+    hipError_t e = hipEventSynchronize(t.stop);
+    if (e == hipSuccess) e = hipEventElapsedTime(&t.ms, t.start, t.stop);
+    if (e != hipSuccess) return fail(TBE_ERR_HIP, "tbe_profile_end: %s", hipGetErrorString(e));
+  }
+  return TBE_OK;
+}
+
+extern "C" int32_t tbe_profile_count(void) {
+  std::lock_guard<std::mutex> lock(tbe::g_profile_mutex);
+  return static_cast<int32_t>(tbe::g_profile.size());
+}
+
+extern "C" int tbe_profile_get(int32_t i, const char **name, float *milliseconds) {
+  using namespace tbe;
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  TBE_REQUIRE(name && milliseconds, "tbe_profile_get: null output pointer");
+  TBE_REQUIRE(i >= 0 && i < static_cast<int32_t>(g_profile.size()), "tbe_profile_get: index %d out of range", i);
+  *name = g_profile[i].name;
+  *milliseconds = g_profile[i].ms;
+  return TBE_OK;
+}
 
 extern "C" int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
                                      const int32_t *total_indices_per_table, int32_t T,
@@ -60,9 +142,9 @@ extern "C" int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
               "tbe_construct_offsets: null pointer argument");
   const int64_t n = static_cast<int64_t>(T) * B;
   const dim3 grid(static_cast<unsigned>(ceil_div(n, kBlockThreads)));
-  hipLaunchKernelGGL(construct_offsets_kernel, grid, dim3(kBlockThreads), 0,
-                     static_cast<hipStream_t>(stream), batch_offsets_per_table,
-                     total_indices_per_table, T, B, output);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  TBE_LAUNCH("construct_offsets", s, construct_offsets_kernel, grid, dim3(kBlockThreads),
+             batch_offsets_per_table, total_indices_per_table, T, B, output);
   return check_launch("tbe_construct_offsets");
 }
 

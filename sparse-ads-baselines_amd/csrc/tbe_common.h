@@ -24,6 +24,21 @@ int check_launch(const char *what);
     if (!(cond)) return ::tbe::fail(TBE_ERR_INVALID, __VA_ARGS__); \
   } while (0)
 
+// Per-kernel timing for benchmarks: between tbe_profile_begin() and tbe_profile_end()
+// every launch is bracketed by HIP events recorded on the launch stream.
+struct LaunchTimer {
+  LaunchTimer(const char *name, hipStream_t stream);
+  ~LaunchTimer();
+  int slot;
+  hipStream_t stream;
+};
+
+#define TBE_LAUNCH(name, stream, kernel, grid, block, ...)                     \
+  do {                                                                         \
+    ::tbe::LaunchTimer tbe_launch_timer(name, stream);                         \
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, __VA_ARGS__);           \
+  } while (0)
+
 inline uint64_t align_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

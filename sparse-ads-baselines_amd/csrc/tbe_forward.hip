@@ -195,13 +195,12 @@ int launch_forward(const RowGeometry &g, const void *weights, int32_t D,
   T *o = static_cast<T *>(output);
   constexpr int kUnroll = 8;
 #define TBE_FWD(CH)                                                                        \
-  hipLaunchKernelGGL((forward_kernel<T, VEC, CH, WEIGHTED, kUnroll>), grid, block, 0,      \
-                     stream, w, table_offsets, indices, offsets, p, o, B, T_, D, g.chunks, \
-                     num_bags, per_xcd)
+  TBE_LAUNCH("forward", stream, (forward_kernel<T, VEC, CH, WEIGHTED, kUnroll>), grid,   \
+             block, w, table_offsets, indices, offsets, p, o, B, T_, D, g.chunks, num_bags, \
+             per_xcd)
   if (g.wide) {
-    hipLaunchKernelGGL((forward_wide_kernel<T, VEC, WEIGHTED, 4>), grid, block, 0, stream, w,
-                       table_offsets, indices, offsets, p, o, B, T_, D, g.chunks, num_bags,
-                       per_xcd);
+    TBE_LAUNCH("forward_wide", stream, (forward_wide_kernel<T, VEC, WEIGHTED, 4>), grid, block,
+               w, table_offsets, indices, offsets, p, o, B, T_, D, g.chunks, num_bags, per_xcd);
   } else {
     switch (g.tmpl) {
       case 64: TBE_FWD(64); break;

@@ -324,8 +324,8 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   uint32_t *totals = reinterpret_cast<uint32_t *>(ws);
 
   const dim3 block(kBlockThreads);
-  hipLaunchKernelGGL(radix_zero_totals_kernel, dim3(kMaxPasses), block, 0, stream, totals,
-                     kMaxPasses * kBins);
+  TBE_LAUNCH("radix_zero", stream, radix_zero_totals_kernel, dim3(kMaxPasses), block, totals,
+             kMaxPasses * kBins);
   const uint32_t *src_k = reinterpret_cast<const uint32_t *>(keys_in);
   const uint32_t *src_v = reinterpret_cast<const uint32_t *>(values_in);
   for (int pass = 0; pass < passes; ++pass) {
@@ -336,11 +336,12 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
     uint32_t *dst_k = to_out ? reinterpret_cast<uint32_t *>(keys_out) : tmp_keys;
     uint32_t *dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
     uint32_t *pass_totals = totals + pass * kBins;
-    hipLaunchKernelGGL(radix_histogram_kernel, dim3(tiles), block, 0, stream, src_k, n, shift,
-                       mask, tiles, counts, pass_totals);
-    hipLaunchKernelGGL(radix_scan_kernel, dim3(kBins), block, 0, stream, counts, pass_totals, tiles);
-    hipLaunchKernelGGL(radix_scatter_kernel, dim3(tiles), block, 0, stream, src_k, src_v, dst_k,
-                       dst_v, n, shift, mask, tiles, counts);
+    TBE_LAUNCH("radix_histogram", stream, radix_histogram_kernel, dim3(tiles), block, src_k, n,
+               shift, mask, tiles, counts, pass_totals);
+    TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, dim3(kBins), block, counts, pass_totals,
+               tiles);
+    TBE_LAUNCH("radix_scatter", stream, radix_scatter_kernel, dim3(tiles), block, src_k, src_v,
+               dst_k, dst_v, n, shift, mask, tiles, counts);
     src_k = dst_k;
     src_v = dst_v;
   }
@@ -358,12 +359,13 @@ int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts
   const uint32_t *keys = reinterpret_cast<const uint32_t *>(keys_sorted);
   const dim3 block(kBlockThreads);
   if (tiles > 0)
-    hipLaunchKernelGGL(segment_count_kernel, dim3(tiles), block, 0, stream, keys, n, tile_heads);
-  hipLaunchKernelGGL(segment_scan_kernel, dim3(1), block, 0, stream, tile_heads, tiles, n,
-                     segment_starts, num_unique);
+    TBE_LAUNCH("segment_count", stream, segment_count_kernel, dim3(tiles), block, keys, n,
+               tile_heads);
+  TBE_LAUNCH("segment_scan", stream, segment_scan_kernel, dim3(1), block, tile_heads, tiles, n,
+             segment_starts, num_unique);
   if (tiles > 0)
-    hipLaunchKernelGGL(segment_write_kernel, dim3(tiles), block, 0, stream, keys, n, tile_heads,
-                       segment_starts);
+    TBE_LAUNCH("segment_write", stream, segment_write_kernel, dim3(tiles), block, keys, n,
+               tile_heads, segment_starts);
   return check_launch("tbe_find_segments");
 }
 
@@ -372,8 +374,8 @@ int linearize(const int32_t *table_offsets, int32_t T, const int32_t *indices,
               hipStream_t stream) {
   const int64_t num_bags = static_cast<int64_t>(T) * B;
   const dim3 grid(static_cast<unsigned>(ceil_div(num_bags * kLinLanes, kBlockThreads)));
-  hipLaunchKernelGGL(linearize_kernel, grid, dim3(kBlockThreads), 0, stream, table_offsets,
-                     indices, offsets, B, T, static_cast<int>(num_bags), keys, grad_rows);
+  TBE_LAUNCH("linearize", stream, linearize_kernel, grid, dim3(kBlockThreads), table_offsets,
+             indices, offsets, B, T, static_cast<int>(num_bags), keys, grad_rows);
   return check_launch("tbe_linearize");
 }
 

@@ -440,23 +440,25 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   // grid-stride loop amortises launch cost on large inputs.
   const int64_t want = ceil_div(ceil_div(a.num_indices, groups), kWavesPerBlock);
   const dim3 grid_short(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want, 256 * 32))));
-  hipLaunchKernelGGL((update_short_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kShortUnroll>), grid_short,
-                     block, 0, stream, go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted,
-                     a.grad_rows, a.segment_starts, a.counters, a.long_segments,
-                     a.chunk_segments, a.max_long, a.D, g.chunks, a.learning_rate, a.eps);
+  TBE_LAUNCH("update_short", stream,
+             (update_short_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kShortUnroll>), grid_short, block,
+             go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
+             a.segment_starts, a.counters, a.long_segments, a.chunk_segments, a.max_long, a.D,
+             g.chunks, a.learning_rate, a.eps);
 
   const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
   const dim3 grid_partial(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_chunks, 256 * 8))));
-  hipLaunchKernelGGL((update_long_partial_kernel<T, VEC, CHUNKS, WEIGHTED, kLongUnroll>),
-                     grid_partial, block, 0, stream, go, w, psw, gpsw, a.keys_sorted,
-                     a.positions_sorted, a.grad_rows, a.segment_starts, a.counters,
-                     a.long_segments, a.chunk_segments, partial, a.max_long, a.D, g.chunks);
+  TBE_LAUNCH("update_long_partial", stream,
+             (update_long_partial_kernel<T, VEC, CHUNKS, WEIGHTED, kLongUnroll>), grid_partial,
+             block, go, w, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
+             a.segment_starts, a.counters, a.long_segments, a.chunk_segments, partial, a.max_long,
+             a.D, g.chunks);
 
   const int64_t want_long = ceil_div(ceil_div(a.max_long, groups), kWavesPerBlock);
   const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
-  hipLaunchKernelGGL((update_long_finish_kernel<T, VEC, CHUNKS, OPT>), grid_finish, block, 0,
-                     stream, w, st, a.keys_sorted, a.segment_starts, a.counters, a.long_segments,
-                     partial, a.max_long, a.D, g.chunks, a.learning_rate, a.eps);
+  TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, OPT>),
+             grid_finish, block, w, st, a.keys_sorted, a.segment_starts, a.counters,
+             a.long_segments, partial, a.max_long, a.D, g.chunks, a.learning_rate, a.eps);
 }
 
 template <typename T, int VEC, int OPT, bool WEIGHTED>
@@ -465,13 +467,12 @@ void launch_geometry(const UpdateArgs &a, const RowGeometry &g, hipStream_t stre
   if (g.wide) {
     const int64_t want = ceil_div(a.num_indices, kWavesPerBlock);
     const dim3 grid(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want, 256 * 32))));
-    hipLaunchKernelGGL((update_wide_kernel<T, VEC, OPT, WEIGHTED>), grid, dim3(kBlockThreads), 0,
-                       stream, static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),
-                       static_cast<A *>(a.optimizer_state),
-                       static_cast<const T *>(a.per_sample_weights),
-                       static_cast<T *>(a.grad_per_sample_weights), a.keys_sorted,
-                       a.positions_sorted, a.grad_rows, a.segment_starts, a.counters, a.D,
-                       g.chunks, a.learning_rate, a.eps);
+    TBE_LAUNCH("update_wide", stream, (update_wide_kernel<T, VEC, OPT, WEIGHTED>), grid,
+               dim3(kBlockThreads), static_cast<const T *>(a.grad_output),
+               static_cast<T *>(a.weights), static_cast<A *>(a.optimizer_state),
+               static_cast<const T *>(a.per_sample_weights),
+               static_cast<T *>(a.grad_per_sample_weights), a.keys_sorted, a.positions_sorted,
+               a.grad_rows, a.segment_starts, a.counters, a.D, g.chunks, a.learning_rate, a.eps);
     return;
   }
   switch (g.tmpl) {
@@ -501,7 +502,7 @@ void launch_variant(const UpdateArgs &a, const RowGeometry &g, hipStream_t strea
 int segment_update(const UpdateArgs &a, hipStream_t stream) {
   if (a.num_indices == 0) return TBE_OK;
   const RowGeometry g = row_geometry(a.dtype, a.D);
-  hipLaunchKernelGGL(zero_counters_kernel, dim3(1), dim3(kWave), 0, stream, a.counters);
+  TBE_LAUNCH("zero_counters", stream, zero_counters_kernel, dim3(1), dim3(kWave), a.counters);
   switch (a.dtype) {
     case TBE_DTYPE_F32: launch_variant<float, 4>(a, g, stream); break;
     case TBE_DTYPE_F16:

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -45,6 +45,10 @@ class WorkspaceLayout(ctypes.Structure):
 SIGNATURES = {
     "tbe_last_error": (ctypes.c_char_p, []),
     "tbe_abi_version": (_i32, []),
+    "tbe_profile_begin": (ctypes.c_int, []),
+    "tbe_profile_end": (ctypes.c_int, []),
+    "tbe_profile_count": (_i32, []),
+    "tbe_profile_get": (ctypes.c_int, [_i32, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_f32)]),
     "tbe_forward": (ctypes.c_int, [_vp, _i32, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp, _vp, _vp]),
     "tbe_backward_workspace_layout": (ctypes.c_int, [_i64, _i32, _i32, ctypes.POINTER(WorkspaceLayout)]),
     "tbe_backward_sgd": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p,
@@ -103,3 +107,23 @@ def backward_workspace_layout(num_indices, D, dtype_code):
     layout = WorkspaceLayout()
     check(load().tbe_backward_workspace_layout(num_indices, D, dtype_code, ctypes.byref(layout)))
     return layout
+
+
+class profile:
+    """Context manager: times every kernel launched by the library inside the block.
+
+    After the block, `.launches` is a list of (kernel name, milliseconds) in launch order."""
+
+    def __enter__(self):
+        check(load().tbe_profile_begin())
+        self.launches = []
+        return self
+
+    def __exit__(self, *exc):
+        lib = load()
+        check(lib.tbe_profile_end())
+        name, ms = ctypes.c_char_p(), _f32()
+        for i in range(lib.tbe_profile_count()):
+            check(lib.tbe_profile_get(i, ctypes.byref(name), ctypes.byref(ms)))
+            self.launches.append((name.value.decode(), ms.value))
+        return False
