@@ -186,6 +186,103 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
                           const int32_t *total_indices_per_table,
                           int32_t T, int32_t B, int32_t *output, void *stream);
 
+/* ---------------------------------------------------------------- row cache
+ * An HBM-resident set-associative row cache in front of a host-resident table
+ * (pinned, device-mapped memory from tbe_host_mapped_alloc).  The reference has
+ * no cache: its only host-table mechanism is managed / mapped memory read over
+ * the bus on every lookup (table_batched_embeddings_cuda.cu:795-880,
+ * EmbeddingLocation.HOST_MAPPED in table_batched_embeddings_ops.py:130-167).
+ * Semantics are this library's own and are restated by oracle/lxu_cache_model.c.
+ *
+ * Geometry: num_sets sets of TBE_CACHE_WAYS = 64 slots; set = mix(key) scaled to
+ * [0, num_sets) with a fixed 32-bit integer hash; one wavefront probes a set with
+ * one coalesced tag load and a ballot.  All state lives in caller-owned device
+ * arrays.  One call of tbe_cache_prepare per step (steps are numbered from 1):
+ *   1. the batch is linearized, sorted and cut into unique rows (ascending key);
+ *   2. every unique row probes its set; hits record their slot and are marked
+ *      used in this step (last_used = step, use_count += 1);
+ *   3. the missing rows of a set are inserted in ascending key order; the victim
+ *      is the slot with the smallest (priority, way) among slots not used in this
+ *      step, priority = last_used (LRU) or use_count (LFU); empty slots (priority 0)
+ *      go first; if every slot of the set was used in this step the row stays
+ *      uncached for the step and is read / updated in the backing table directly;
+ *   4. on the side stream, evicted rows are written back to the backing table and
+ *      the inserted rows are fetched into their slots (every resident row counts
+ *      as dirty: the optimizer updates each row it looks up); the side stream is
+ *      joined to `stream` by an event before the call returns control of `stream`
+ *      to the caller's next kernel;
+ *   5. unique_slots[u] / lookup_slots[p] tell the forward and backward kernels
+ *      where each row lives (slot >= 0, or -1 = backing table).
+ * The resulting tags / slots are a pure function of the key sequence, so a CPU
+ * model can reproduce them bit for bit.
+ */
+#define TBE_CACHE_WAYS 64
+enum { TBE_CACHE_LRU = 0, TBE_CACHE_LFU = 1 };
+enum { TBE_OPT_SGD = 0, TBE_OPT_ROWWISE_ADAGRAD = 1 };
+
+typedef struct tbe_cache {
+  int32_t *tags;        /* [num_sets * 64] key of the row held by each slot, -1 = empty  */
+  int32_t *last_used;   /* [num_sets * 64] step of the slot's last use, 0 = never        */
+  int32_t *use_count;   /* [num_sets * 64] steps that used the row since it was inserted */
+  void *rows;           /* [num_sets * 64][D] cached rows                                */
+  void *backing_rows;   /* device-visible address of the backing table [total_rows][D]   */
+  int64_t num_sets;
+  int32_t policy;       /* TBE_CACHE_LRU or TBE_CACHE_LFU                                */
+} tbe_cache_t;
+
+/* Byte offsets into the cache workspace (separate from the backward workspace). */
+typedef struct tbe_cache_workspace_layout {
+  uint64_t total_bytes;
+  uint64_t unique_slots;   /* int32 [U]  slot of each unique row, -1 = backing table          */
+  uint64_t lookup_slots;   /* int32 [N]  the same, per lookup position                         */
+  uint64_t evicted_keys;   /* int32 [U]  -2 untouched, -1 filled an empty slot, >= 0 key written back */
+  uint64_t segment_ids;    /* int32 [N]  index of the unique row of each sorted position       */
+  uint64_t miss_sets;      /* int32 [U]  set of each missing row                               */
+  uint64_t miss_list;      /* int32 [U]  missing rows grouped by set                           */
+  uint64_t set_counts;     /* int32 [num_sets] misses per set                                  */
+  uint64_t set_fill;       /* int32 [num_sets]                                                 */
+  uint64_t set_starts;     /* int32 [num_sets + 1]                                             */
+  uint64_t stats;          /* int32 [8]: unique rows, hits, misses, inserted, written back, uncached */
+} tbe_cache_workspace_layout_t;
+
+TBE_API int tbe_cache_workspace_layout(int64_t num_indices, int64_t num_sets,
+                                       tbe_cache_workspace_layout_t *layout);
+
+/* Empties the cache: tags = -1, last_used = use_count = 0. */
+TBE_API int tbe_cache_init(const tbe_cache_t *cache, void *stream);
+
+/* Steps 1-5 above.  `workspace` is a backward workspace (tbe_backward_workspace_layout)
+ * and keeps the batch's plan for tbe_backward_cached; `cache_workspace` follows
+ * tbe_cache_workspace_layout.  `side_stream` must differ from `stream`. */
+TBE_API int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_t total_rows, int32_t D,
+                              const int32_t *table_offsets, int32_t T,
+                              const int32_t *indices, int64_t num_indices,
+                              const int32_t *offsets, int32_t B, int32_t step,
+                              void *workspace, uint64_t workspace_bytes,
+                              void *cache_workspace, uint64_t cache_workspace_bytes,
+                              void *stream, void *side_stream);
+
+/* tbe_forward with every row read through lookup_slots (cache slot or backing table). */
+TBE_API int tbe_forward_cached(const tbe_cache_t *cache, int32_t dtype, int32_t D,
+                               const int32_t *table_offsets, int32_t T,
+                               const int32_t *indices, int64_t num_indices,
+                               const int32_t *offsets, int32_t B,
+                               const void *per_sample_weights, const int32_t *lookup_slots,
+                               void *output, void *stream);
+
+/* The fused update of tbe_backward_sgd / tbe_backward_exact_adagrad on the plan that
+ * tbe_cache_prepare left in `workspace`, updating each row where it lives. */
+TBE_API int tbe_backward_cached(int32_t optimizer, const void *grad_output, const tbe_cache_t *cache,
+                                int32_t dtype, int64_t total_rows, int32_t D, int32_t T, int32_t B,
+                                int64_t num_indices, const void *per_sample_weights,
+                                void *optimizer_state, float learning_rate, float eps,
+                                void *grad_per_sample_weights,
+                                void *workspace, uint64_t workspace_bytes,
+                                const int32_t *unique_slots, void *stream);
+
+/* Writes every resident row back to the backing table (the cache stays valid). */
+TBE_API int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t D, void *stream);
+
 /* ------------------------------------------------------ host-resident tables
  * Pinned, device-mapped host memory (new_host_mapped_tensor,
  * table_batched_embeddings_cuda.cu:820-880) and managed memory preferring the

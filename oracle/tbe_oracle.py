@@ -135,3 +135,40 @@ def half_to_float(bits):
 
 def float_to_half(value):
     return lib().oracle_float_to_half(float(value))
+
+
+# ------------------------------------------------------------------ row cache model
+class CacheModel:
+    """State and step function of the row-cache specification (oracle/lxu_cache_model.c)."""
+
+    WAYS = 64
+
+    def __init__(self, num_sets, policy="lru"):
+        self.num_sets = int(num_sets)
+        self.policy = {"lru": 0, "lfu": 1}[policy]
+        n = self.num_sets * self.WAYS
+        self.tags = np.full(n, -1, np.int32)
+        self.last_used = np.zeros(n, np.int32)
+        self.use_count = np.zeros(n, np.int32)
+        self.step_no = 0
+
+    def step(self, unique_keys):
+        """unique_keys: strictly ascending int32.  -> (unique_slots, evicted_keys, stats[6])"""
+        keys = _i32(unique_keys)
+        self.step_no += 1
+        slots = np.empty(keys.size, np.int32)
+        evicted = np.empty(keys.size, np.int32)
+        stats = np.zeros(6, np.int32)
+        lib().lxu_cache_step(_p(self.tags), _p(self.last_used), _p(self.use_count), ctypes.c_int64(self.num_sets),
+                             ctypes.c_int32(self.policy), ctypes.c_int32(self.step_no), _p(keys),
+                             ctypes.c_int64(keys.size), _p(slots), _p(evicted), _p(stats))
+        return slots, evicted, stats
+
+    def resident(self):
+        return np.sort(self.tags[self.tags >= 0])
+
+
+def cache_set_of(key, num_sets):
+    fn = lib().lxu_set_of
+    fn.restype = ctypes.c_uint32
+    return fn(ctypes.c_uint32(int(key)), ctypes.c_uint32(int(num_sets)))

@@ -42,6 +42,34 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t 
   l->total_bytes = off;
 }
 
+}  // namespace
+
+int key_bits_for(int64_t total_rows) { return key_bits(total_rows); }
+
+void backward_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t *l) {
+  compute_layout(n, D, dtype, l);
+}
+
+// linearize -> sort -> run boundaries into the workspace regions of `l`.
+int build_plan(const tbe_workspace_layout_t &l, void *workspace, const int32_t *table_offsets,
+               int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
+               int64_t total_rows, int32_t *segment_ids, hipStream_t stream) {
+  char *ws = static_cast<char *>(workspace);
+  int32_t *keys = reinterpret_cast<int32_t *>(ws + l.keys);
+  int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
+  int rc = linearize(table_offsets, T, indices, offsets, B, keys,
+                     reinterpret_cast<int32_t *>(ws + l.grad_rows), stream);
+  if (rc) return rc;
+  rc = sort_pairs(keys, nullptr, keys_sorted, reinterpret_cast<int32_t *>(ws + l.positions_sorted),
+                  n, key_bits(total_rows), ws + l.sort_scratch, stream);
+  if (rc) return rc;
+  return find_segments(keys_sorted, n, reinterpret_cast<int32_t *>(ws + l.segment_starts),
+                       reinterpret_cast<int32_t *>(ws + l.num_unique), segment_ids,
+                       ws + l.segment_scratch, stream);
+}
+
+namespace {
+
 struct BackwardCall {
   const void *grad_output;
   void *weights;
@@ -63,6 +91,10 @@ struct BackwardCall {
   uint64_t workspace_bytes;
   hipStream_t stream;
   int optimizer;
+  // cache-fronted tables: the plan already sits in the workspace, rows are resolved through slots
+  bool planned;
+  const int32_t *unique_slots;
+  void *cache_rows;
 };
 
 int run_backward(const char *name, const BackwardCall &c) {
@@ -74,8 +106,9 @@ int run_backward(const char *name, const BackwardCall &c) {
   TBE_REQUIRE(c.total_rows > 0 && c.total_rows < INT32_MAX, "%s: total_rows out of range", name);
   TBE_REQUIRE(c.num_indices >= 0 && c.num_indices < INT32_MAX, "%s: num_indices out of range", name);
   TBE_REQUIRE(static_cast<int64_t>(c.T) * c.B < INT32_MAX, "%s: T*B out of range", name);
-  TBE_REQUIRE(c.grad_output && c.weights && c.table_offsets && c.offsets, "%s: null pointer argument", name);
-  TBE_REQUIRE(c.indices || c.num_indices == 0, "%s: indices is null but num_indices > 0", name);
+  TBE_REQUIRE(c.grad_output && c.weights, "%s: null pointer argument", name);
+  TBE_REQUIRE(c.planned || (c.table_offsets && c.offsets), "%s: null pointer argument", name);
+  TBE_REQUIRE(c.planned || c.indices || c.num_indices == 0, "%s: indices is null but num_indices > 0", name);
   TBE_REQUIRE(c.optimizer == kOptSgd || c.state, "%s: optimizer_state is null", name);
   TBE_REQUIRE((c.psw == nullptr) == (c.grad_psw == nullptr),
               "%s: per_sample_weights and grad_per_sample_weights must both be given or both be null", name);
@@ -87,21 +120,17 @@ int run_backward(const char *name, const BackwardCall &c) {
     return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
                 (unsigned long long)l.total_bytes, (unsigned long long)c.workspace_bytes);
   char *ws = static_cast<char *>(c.workspace);
-  int32_t *keys = reinterpret_cast<int32_t *>(ws + l.keys);
   int32_t *grad_rows = reinterpret_cast<int32_t *>(ws + l.grad_rows);
   int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
   int32_t *positions_sorted = reinterpret_cast<int32_t *>(ws + l.positions_sorted);
   int32_t *segment_starts = reinterpret_cast<int32_t *>(ws + l.segment_starts);
   int32_t *counters = reinterpret_cast<int32_t *>(ws + l.num_unique);
 
-  int rc = linearize(c.table_offsets, c.T, c.indices, c.offsets, c.B, keys, grad_rows, c.stream);
-  if (rc) return rc;
-  rc = sort_pairs(keys, nullptr, keys_sorted, positions_sorted, c.num_indices,
-                  key_bits(c.total_rows), ws + l.sort_scratch, c.stream);
-  if (rc) return rc;
-  rc = find_segments(keys_sorted, c.num_indices, segment_starts, counters, ws + l.segment_scratch,
-                     c.stream);
-  if (rc) return rc;
+  if (!c.planned) {
+    const int rc = build_plan(l, c.workspace, c.table_offsets, c.T, c.indices, c.num_indices,
+                              c.offsets, c.B, c.total_rows, nullptr, c.stream);
+    if (rc) return rc;
+  }
 
   UpdateArgs a;
   a.grad_output = c.grad_output;
@@ -117,6 +146,8 @@ int run_backward(const char *name, const BackwardCall &c) {
   a.long_segments = reinterpret_cast<int32_t *>(ws + l.long_segments);
   a.chunk_segments = reinterpret_cast<int32_t *>(ws + l.chunk_segments);
   a.partial_sums = ws + l.partial_sums;
+  a.unique_slots = c.unique_slots;
+  a.cache_rows = c.cache_rows;
   a.num_indices = c.num_indices;
   a.max_long = l.max_long_segments;
   a.max_chunks = l.max_chunks;
@@ -151,7 +182,8 @@ extern "C" int tbe_backward_sgd(const void *grad_output, void *weights, int32_t 
                                 void *workspace, uint64_t workspace_bytes, void *stream) {
   tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
                       num_indices, offsets, B, nullptr, nullptr, learning_rate, 0.0f, nullptr,
-                      workspace, workspace_bytes, static_cast<hipStream_t>(stream), tbe::kOptSgd};
+                      workspace, workspace_bytes, static_cast<hipStream_t>(stream), tbe::kOptSgd,
+                      false, nullptr, nullptr};
   return tbe::run_backward("tbe_backward_sgd", c);
 }
 
@@ -167,6 +199,28 @@ extern "C" int tbe_backward_exact_adagrad(const void *grad_output, void *weights
   tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
                       num_indices, offsets, B, per_sample_weights, optimizer_state, learning_rate,
                       eps, grad_per_sample_weights, workspace, workspace_bytes,
-                      static_cast<hipStream_t>(stream), tbe::kOptAdagrad};
+                      static_cast<hipStream_t>(stream), tbe::kOptAdagrad, false, nullptr, nullptr};
   return tbe::run_backward("tbe_backward_exact_adagrad", c);
+}
+
+extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
+                                   const tbe_cache_t *cache, int32_t dtype, int64_t total_rows,
+                                   int32_t D, int32_t T, int32_t B, int64_t num_indices,
+                                   const void *per_sample_weights, void *optimizer_state,
+                                   float learning_rate, float eps, void *grad_per_sample_weights,
+                                   void *workspace, uint64_t workspace_bytes,
+                                   const int32_t *unique_slots, void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(cache && cache->rows && cache->backing_rows, "tbe_backward_cached: null cache");
+  TBE_REQUIRE(optimizer == TBE_OPT_SGD || optimizer == TBE_OPT_ROWWISE_ADAGRAD,
+              "tbe_backward_cached: bad optimizer %d", optimizer);
+  TBE_REQUIRE(unique_slots || num_indices == 0, "tbe_backward_cached: null unique_slots");
+  TBE_REQUIRE(optimizer != TBE_OPT_SGD || !per_sample_weights,
+              "tbe_backward_cached: SGD takes no per-sample weights");
+  BackwardCall c{grad_output, cache->backing_rows, dtype, total_rows, D, nullptr, T, nullptr,
+                 num_indices, nullptr, B, per_sample_weights, optimizer_state, learning_rate, eps,
+                 grad_per_sample_weights, workspace, workspace_bytes,
+                 static_cast<hipStream_t>(stream),
+                 optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad, true, unique_slots, cache->rows};
+  return run_backward("tbe_backward_cached", c);
 }

@@ -19,12 +19,16 @@
 namespace tbe {
 namespace {
 
-template <typename T, int VEC, int CHUNKS, bool WEIGHTED, int UNROLL>
+// CACHED: every lookup carries a location (lookup_slots[p]); a non-negative value is a slot of
+// the HBM row cache (row at cache_rows + slot * D), a negative one means the row is read from
+// `weights` (the host-resident backing table) directly.
+template <typename T, int VEC, int CHUNKS, bool WEIGHTED, bool CACHED, int UNROLL>
 __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
     const T *__restrict__ weights, const int32_t *__restrict__ table_offsets,
     const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
     const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D,
-    int chunks_rt, int num_bags, int64_t blocks_per_xcd) {
+    int chunks_rt, int num_bags, int64_t blocks_per_xcd,
+    const int32_t *__restrict__ lookup_slots, const T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -54,10 +58,12 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
   for (int base = start; base < end; base += kWave) {
     const int n = min(kWave, end - base);
     int my_idx = 0;
+    int my_slot = -1;
     A my_w = A(0);
     if (lane < n) {
       my_idx = __builtin_nontemporal_load(indices + base + lane);
       if constexpr (WEIGHTED) my_w = to_acc(psw[base + lane]);
+      if constexpr (CACHED) my_slot = __builtin_nontemporal_load(lookup_slots + base + lane);
     }
     for (int j0 = 0; j0 < n; j0 += groups * UNROLL) {
       R raw[UNROLL];
@@ -70,7 +76,12 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
         const int src = ok[u] ? j : 0;
         const int idx = shfl_idx(my_idx, src);
         if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, src);
-        if (ok[u]) raw[u] = V::load_raw(col + (table_row0 + idx) * D);
+        const T *row = col + (table_row0 + idx) * D;
+        if constexpr (CACHED) {
+          const int slot = shfl_idx(my_slot, src);
+          if (slot >= 0) row = cache_rows + static_cast<int64_t>(slot) * D + static_cast<int64_t>(c) * VEC;
+        }
+        if (ok[u]) raw[u] = V::load_raw(row);
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
@@ -116,12 +127,13 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
 
 // Rows wider than 64 vectors: the wavefront walks the row in blocks of 64
 // vectors and sums the bag serially per block.
-template <typename T, int VEC, bool WEIGHTED, int UNROLL>
+template <typename T, int VEC, bool WEIGHTED, bool CACHED, int UNROLL>
 __global__ __launch_bounds__(kBlockThreads) void forward_wide_kernel(
     const T *__restrict__ weights, const int32_t *__restrict__ table_offsets,
     const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
     const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D,
-    int chunks, int num_bags, int64_t blocks_per_xcd) {
+    int chunks, int num_bags, int64_t blocks_per_xcd,
+    const int32_t *__restrict__ lookup_slots, const T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -147,10 +159,12 @@ __global__ __launch_bounds__(kBlockThreads) void forward_wide_kernel(
     for (int base = start; base < end; base += kWave) {
       const int n = min(kWave, end - base);
       int my_idx = 0;
+      int my_slot = -1;
       A my_w = A(0);
       if (lane < n) {
         my_idx = indices[base + lane];
         if constexpr (WEIGHTED) my_w = to_acc(psw[base + lane]);
+        if constexpr (CACHED) my_slot = lookup_slots[base + lane];
       }
       for (int j0 = 0; j0 < n; j0 += UNROLL) {
         R raw[UNROLL];
@@ -160,7 +174,12 @@ __global__ __launch_bounds__(kBlockThreads) void forward_wide_kernel(
           const int j = min(j0 + u, n - 1);
           const int idx = shfl_idx(my_idx, j);
           if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, j);
-          if (ok_c && j0 + u < n) raw[u] = V::load_raw(col + (table_row0 + idx) * D);
+          const T *row = col + (table_row0 + idx) * D;
+          if constexpr (CACHED) {
+            const int slot = shfl_idx(my_slot, j);
+            if (slot >= 0) row = cache_rows + static_cast<int64_t>(slot) * D + static_cast<int64_t>(c) * VEC;
+          }
+          if (ok_c && j0 + u < n) raw[u] = V::load_raw(row);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
@@ -180,27 +199,41 @@ __global__ __launch_bounds__(kBlockThreads) void forward_wide_kernel(
   }
 }
 
-template <typename T, int VEC, bool WEIGHTED>
-int launch_forward(const RowGeometry &g, const void *weights, int32_t D,
-                   const int32_t *table_offsets, int32_t T_, const int32_t *indices,
-                   const int32_t *offsets, int32_t B, const void *psw, void *output,
-                   hipStream_t stream) {
-  const int num_bags = T_ * B;
+struct ForwardArgs {
+  const void *weights;
+  int32_t dtype;
+  int32_t D;
+  const int32_t *table_offsets;
+  int32_t T;
+  const int32_t *indices;
+  const int32_t *offsets;
+  int32_t B;
+  const void *psw;
+  void *output;
+  const int32_t *lookup_slots;  // null unless the rows are fronted by the HBM row cache
+  const void *cache_rows;
+};
+
+template <typename T, int VEC, bool WEIGHTED, bool CACHED>
+void launch_forward(const ForwardArgs &a, const RowGeometry &g, hipStream_t stream) {
+  const int num_bags = a.T * a.B;
   const int64_t nblocks = ceil_div(num_bags, kWavesPerBlock);
   const int64_t per_xcd = ceil_div(nblocks, kNumXcd);
   const dim3 grid(static_cast<unsigned>(per_xcd * kNumXcd));
   const dim3 block(kBlockThreads);
-  const T *w = static_cast<const T *>(weights);
-  const T *p = static_cast<const T *>(psw);
-  T *o = static_cast<T *>(output);
+  const T *w = static_cast<const T *>(a.weights);
+  const T *p = static_cast<const T *>(a.psw);
+  const T *cr = static_cast<const T *>(a.cache_rows);
+  T *o = static_cast<T *>(a.output);
   constexpr int kUnroll = 8;
-#define TBE_FWD(CH)                                                                        \
-  TBE_LAUNCH("forward", stream, (forward_kernel<T, VEC, CH, WEIGHTED, kUnroll>), grid,   \
-             block, w, table_offsets, indices, offsets, p, o, B, T_, D, g.chunks, num_bags, \
-             per_xcd)
+#define TBE_FWD(CH)                                                                            \
+  TBE_LAUNCH("forward", stream, (forward_kernel<T, VEC, CH, WEIGHTED, CACHED, kUnroll>), grid, \
+             block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, g.chunks,   \
+             num_bags, per_xcd, a.lookup_slots, cr)
   if (g.wide) {
-    TBE_LAUNCH("forward_wide", stream, (forward_wide_kernel<T, VEC, WEIGHTED, 4>), grid, block,
-               w, table_offsets, indices, offsets, p, o, B, T_, D, g.chunks, num_bags, per_xcd);
+    TBE_LAUNCH("forward_wide", stream, (forward_wide_kernel<T, VEC, WEIGHTED, CACHED, 4>), grid,
+               block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, g.chunks,
+               num_bags, per_xcd, a.lookup_slots, cr);
   } else {
     switch (g.tmpl) {
       case 64: TBE_FWD(64); break;
@@ -212,21 +245,49 @@ int launch_forward(const RowGeometry &g, const void *weights, int32_t D,
     }
   }
 #undef TBE_FWD
-  return check_launch("tbe_forward");
 }
 
 template <typename T, int VEC>
-int launch_forward_w(bool weighted, const RowGeometry &g, const void *weights, int32_t D,
-                     const int32_t *table_offsets, int32_t T_, const int32_t *indices,
-                     const int32_t *offsets, int32_t B, const void *psw, void *output,
-                     hipStream_t stream) {
-  return weighted ? launch_forward<T, VEC, true>(g, weights, D, table_offsets, T_, indices,
-                                                 offsets, B, psw, output, stream)
-                  : launch_forward<T, VEC, false>(g, weights, D, table_offsets, T_, indices,
-                                                  offsets, B, psw, output, stream);
+void launch_forward_variant(const ForwardArgs &a, const RowGeometry &g, hipStream_t stream) {
+  const bool weighted = a.psw != nullptr;
+  const bool cached = a.lookup_slots != nullptr;
+  if (cached) {
+    if (weighted) launch_forward<T, VEC, true, true>(a, g, stream);
+    else launch_forward<T, VEC, false, true>(a, g, stream);
+  } else {
+    if (weighted) launch_forward<T, VEC, true, false>(a, g, stream);
+    else launch_forward<T, VEC, false, false>(a, g, stream);
+  }
+}
+
+int validate_forward(const char *name, const ForwardArgs &a, int64_t num_indices) {
+  TBE_REQUIRE(a.T > 0, "%s: T must be positive (got %d)", name, a.T);
+  TBE_REQUIRE(a.D > 0, "%s: D must be positive (got %d)", name, a.D);
+  TBE_REQUIRE(a.B > 0, "%s: B must be positive (got %d)", name, a.B);
+  TBE_REQUIRE(a.D % 4 == 0, "%s: D must be a multiple of 4 (got %d)", name, a.D);
+  TBE_REQUIRE(a.dtype >= TBE_DTYPE_F32 && a.dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, a.dtype);
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(static_cast<int64_t>(a.T) * a.B < INT32_MAX, "%s: T*B out of range", name);
+  TBE_REQUIRE(a.weights && a.table_offsets && a.offsets && a.output, "%s: null pointer argument", name);
+  TBE_REQUIRE(a.indices || num_indices == 0, "%s: indices is null but num_indices > 0", name);
+  return TBE_OK;
 }
 
 }  // namespace
+
+int run_forward(const ForwardArgs &a, hipStream_t stream) {
+  const RowGeometry g = row_geometry(a.dtype, a.D);
+  switch (a.dtype) {
+    case TBE_DTYPE_F32: launch_forward_variant<float, 4>(a, g, stream); break;
+    case TBE_DTYPE_F16:
+      if (g.vec == 8) launch_forward_variant<__half, 8>(a, g, stream);
+      else launch_forward_variant<__half, 4>(a, g, stream);
+      break;
+    default: launch_forward_variant<double, 2>(a, g, stream); break;
+  }
+  return check_launch("tbe_forward");
+}
+
 }  // namespace tbe
 
 extern "C" int tbe_forward(const void *weights, int32_t dtype, int32_t D,
@@ -234,30 +295,28 @@ extern "C" int tbe_forward(const void *weights, int32_t dtype, int32_t D,
                            int64_t num_indices, const int32_t *offsets, int32_t B,
                            const void *per_sample_weights, void *output, void *stream) {
   using namespace tbe;
-  TBE_REQUIRE(T > 0, "tbe_forward: T must be positive (got %d)", T);
-  TBE_REQUIRE(D > 0, "tbe_forward: D must be positive (got %d)", D);
-  TBE_REQUIRE(B > 0, "tbe_forward: B must be positive (got %d)", B);
-  TBE_REQUIRE(D % 4 == 0, "tbe_forward: D must be a multiple of 4 (got %d)", D);
-  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "tbe_forward: bad dtype %d", dtype);
-  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "tbe_forward: num_indices out of range");
-  TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "tbe_forward: T*B out of range");
-  TBE_REQUIRE(weights && table_offsets && offsets && output, "tbe_forward: null pointer argument");
-  TBE_REQUIRE(indices || num_indices == 0, "tbe_forward: indices is null but num_indices > 0");
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const RowGeometry g = row_geometry(dtype, D);
-  const bool weighted = per_sample_weights != nullptr;
-  switch (dtype) {
-    case TBE_DTYPE_F32:
-      return launch_forward_w<float, 4>(weighted, g, weights, D, table_offsets, T, indices,
-                                        offsets, B, per_sample_weights, output, s);
-    case TBE_DTYPE_F16:
-      if (g.vec == 8)
-        return launch_forward_w<__half, 8>(weighted, g, weights, D, table_offsets, T, indices,
-                                           offsets, B, per_sample_weights, output, s);
-      return launch_forward_w<__half, 4>(weighted, g, weights, D, table_offsets, T, indices,
-                                         offsets, B, per_sample_weights, output, s);
-    default:
-      return launch_forward_w<double, 2>(weighted, g, weights, D, table_offsets, T, indices,
-                                         offsets, B, per_sample_weights, output, s);
+  const ForwardArgs a{weights, dtype, D, table_offsets, T, indices, offsets, B,
+                      per_sample_weights, output, nullptr, nullptr};
+  if (int rc = validate_forward("tbe_forward", a, num_indices)) return rc;
+  return run_forward(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tbe_forward_cached(const tbe_cache_t *cache, int32_t dtype, int32_t D,
+                                  const int32_t *table_offsets, int32_t T,
+                                  const int32_t *indices, int64_t num_indices,
+                                  const int32_t *offsets, int32_t B,
+                                  const void *per_sample_weights, const int32_t *lookup_slots,
+                                  void *output, void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(cache && cache->rows && cache->backing_rows, "tbe_forward_cached: null cache");
+  TBE_REQUIRE(lookup_slots || num_indices == 0, "tbe_forward_cached: null lookup_slots");
+  const ForwardArgs a{cache->backing_rows, dtype, D, table_offsets, T, indices, offsets, B,
+                      per_sample_weights, output, lookup_slots, cache->rows};
+  if (int rc = validate_forward("tbe_forward_cached", a, num_indices)) return rc;
+  if (num_indices == 0) {
+    const ForwardArgs plain{cache->backing_rows, dtype, D, table_offsets, T, indices, offsets, B,
+                            per_sample_weights, output, nullptr, nullptr};
+    return run_forward(plain, static_cast<hipStream_t>(stream));
   }
+  return run_forward(a, static_cast<hipStream_t>(stream));
 }

@@ -280,7 +280,7 @@ __global__ __launch_bounds__(kBlockThreads) void segment_scan_kernel(
 
 __global__ __launch_bounds__(kBlockThreads) void segment_write_kernel(
     const uint32_t *__restrict__ keys, int64_t n, const uint32_t *__restrict__ tile_base,
-    int32_t *__restrict__ segment_starts) {
+    int32_t *__restrict__ segment_starts, int32_t *__restrict__ segment_ids) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   const int64_t first = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x) * kSegItems;
   const uint32_t flags = segment_head_flags(keys, n, first);
@@ -291,6 +291,8 @@ __global__ __launch_bounds__(kBlockThreads) void segment_write_kernel(
 #pragma unroll
   for (int k = 0; k < kSegItems; ++k) {
     if (flags & (1u << k)) segment_starts[u++] = static_cast<int32_t>(first + k);
+    // u now counts the heads at or before this position: its segment is u - 1
+    if (segment_ids && first + k < n) segment_ids[first + k] = static_cast<int32_t>(u) - 1;
   }
 }
 
@@ -353,7 +355,7 @@ uint64_t segments_workspace_bytes(int64_t n) {
 }
 
 int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts,
-                  int32_t *num_unique, void *workspace, hipStream_t stream) {
+                  int32_t *num_unique, int32_t *segment_ids, void *workspace, hipStream_t stream) {
   const int tiles = n > 0 ? num_seg_tiles(n) : 0;
   uint32_t *tile_heads = static_cast<uint32_t *>(workspace);
   const uint32_t *keys = reinterpret_cast<const uint32_t *>(keys_sorted);
@@ -365,7 +367,7 @@ int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts
              segment_starts, num_unique);
   if (tiles > 0)
     TBE_LAUNCH("segment_write", stream, segment_write_kernel, dim3(tiles), block, keys, n,
-               tile_heads, segment_starts);
+               tile_heads, segment_starts, segment_ids);
   return check_launch("tbe_find_segments");
 }
 
@@ -424,6 +426,6 @@ extern "C" int tbe_find_segments(const int32_t *keys_sorted, int64_t n, int32_t 
   if (!workspace || workspace_bytes < segments_workspace_bytes(n))
     return fail(TBE_ERR_WORKSPACE, "tbe_find_segments: workspace of %llu bytes needed, %llu given",
                 (unsigned long long)segments_workspace_bytes(n), (unsigned long long)workspace_bytes);
-  return find_segments(keys_sorted, n, segment_starts, num_unique, workspace,
+  return find_segments(keys_sorted, n, segment_starts, num_unique, nullptr, workspace,
                        static_cast<hipStream_t>(stream));
 }

@@ -16,8 +16,9 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
                hipStream_t stream);
 
 uint64_t segments_workspace_bytes(int64_t n);
+// segment_ids (nullable): receives, for every sorted position, the index of its segment.
 int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts,
-                  int32_t *num_unique, void *workspace, hipStream_t stream);
+                  int32_t *num_unique, int32_t *segment_ids, void *workspace, hipStream_t stream);
 
 // Segments longer than kLongSegment occurrences are cut into chunks of
 // kChunkLen occurrences that are reduced by separate wavefronts.
@@ -40,6 +41,8 @@ struct UpdateArgs {
   int32_t *long_segments;       // [2][max_long]
   int32_t *chunk_segments;      // [max_chunks]
   void *partial_sums;           // acc [max_chunks][D]
+  const int32_t *unique_slots;  // cache-fronted tables: slot of each unique row (-1 = not resident)
+  void *cache_rows;             // cache-fronted tables: [slots][D] rows in HBM
   int64_t num_indices;
   int64_t max_long;
   int64_t max_chunks;
@@ -51,5 +54,11 @@ struct UpdateArgs {
 };
 
 int segment_update(const UpdateArgs &args, hipStream_t stream);
+
+int key_bits_for(int64_t total_rows);
+void backward_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t *layout);
+int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int32_t *table_offsets,
+               int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
+               int64_t total_rows, int32_t *segment_ids, hipStream_t stream);
 
 }  // namespace tbe

@@ -39,6 +39,19 @@ template <> __device__ __forceinline__ double adagrad_multiplier<double>(double 
   return static_cast<double>(lr) * (1.0 / (sqrt(s) + static_cast<double>(eps)));
 }
 
+// Address of the row behind the u-th unique key: its slot in the HBM row cache when the
+// tables are cache-fronted and the row is resident, else its row in `weights`.
+template <typename T>
+__device__ __forceinline__ T *resolve_row(T *weights, T *cache_rows,
+                                          const int32_t *__restrict__ unique_slots, int64_t u,
+                                          int64_t row, int D) {
+  if (unique_slots) {
+    const int slot = unique_slots[u];
+    if (slot >= 0) return cache_rows + static_cast<int64_t>(slot) * D;
+  }
+  return weights + row * D;
+}
+
 // Applies the optimizer to one row held by a lane group.  `w_old` and `G` are
 // this lane's vector of the row.
 template <typename T, int VEC, int CHUNKS, int OPT>
@@ -74,7 +87,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
     const int32_t *__restrict__ segment_starts, int32_t *__restrict__ counters,
     int32_t *__restrict__ long_segments, int32_t *__restrict__ chunk_segments, int64_t max_long,
-    int D, int chunks_rt, float lr, float eps) {
+    int D, int chunks_rt, float lr, float eps, const int32_t *__restrict__ unique_slots,
+    T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -110,7 +124,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
       continue;
     }
     const int64_t row = keys_sorted[seg_begin];
-    T *wrow = weights + row * D + col;
+    T *wrow = resolve_row(weights, cache_rows, unique_slots, u, row, D) + col;
     V w_old;
     w_old.load(wrow);
     V G;
@@ -174,7 +188,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_partial_kernel(
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
     const int32_t *__restrict__ long_segments, const int32_t *__restrict__ chunk_segments,
-    typename AccOf<T>::type *__restrict__ partial_sums, int64_t max_long, int D, int chunks_rt) {
+    typename AccOf<T>::type *__restrict__ partial_sums, int64_t max_long, int D, int chunks_rt,
+    const int32_t *__restrict__ unique_slots, const T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -203,7 +218,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_partial_kernel(
     w_old.zero();
     if constexpr (WEIGHTED) {
       const int64_t row = keys_sorted[seg_begin];
-      if (active) w_old.load(weights + row * D + col);
+      if (active)
+        w_old.load(resolve_row<const T>(weights, cache_rows, unique_slots, u, row, D) + col);
     }
     V G;
     G.zero();
@@ -290,7 +306,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
     const int32_t *__restrict__ counters, const int32_t *__restrict__ long_segments,
     const typename AccOf<T>::type *__restrict__ partial_sums, int64_t max_long, int D,
-    int chunks_rt, float lr, float eps) {
+    int chunks_rt, float lr, float eps, const int32_t *__restrict__ unique_slots,
+    T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
 
@@ -313,7 +330,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     const int len = segment_starts[u + 1] - seg_begin;
     const int nch = (len + kChunkLen - 1) / kChunkLen;
     const int64_t row = keys_sorted[seg_begin];
-    T *wrow = weights + row * D + col;
+    T *wrow = resolve_row(weights, cache_rows, unique_slots, u, row, D) + col;
     V w_old;
     w_old.load(wrow);
     V G;
@@ -340,7 +357,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_wide_kernel(
     T *__restrict__ grad_psw, const int32_t *__restrict__ keys_sorted,
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters, int D,
-    int chunks, float lr, float eps) {
+    int chunks, float lr, float eps, const int32_t *__restrict__ unique_slots,
+    T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
 
@@ -353,7 +371,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_wide_kernel(
     const int seg_begin = segment_starts[u];
     const int seg_end = segment_starts[u + 1];
     const int64_t row = keys_sorted[seg_begin];
-    T *wrow = weights + row * D;
+    T *wrow = resolve_row(weights, cache_rows, unique_slots, u, row, D);
 
     if constexpr (WEIGHTED) {
       for (int i = seg_begin; i < seg_end; ++i) {
@@ -433,6 +451,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   const T *psw = static_cast<const T *>(a.per_sample_weights);
   T *gpsw = static_cast<T *>(a.grad_per_sample_weights);
   A *partial = static_cast<A *>(a.partial_sums);
+  T *cr = static_cast<T *>(a.cache_rows);
   const int groups = kWave / g.chunks;
   const dim3 block(kBlockThreads);
 
@@ -444,7 +463,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
              (update_short_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kShortUnroll>), grid_short, block,
              go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
              a.segment_starts, a.counters, a.long_segments, a.chunk_segments, a.max_long, a.D,
-             g.chunks, a.learning_rate, a.eps);
+             g.chunks, a.learning_rate, a.eps, a.unique_slots, cr);
 
   const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
   const dim3 grid_partial(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_chunks, 256 * 8))));
@@ -452,13 +471,14 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
              (update_long_partial_kernel<T, VEC, CHUNKS, WEIGHTED, kLongUnroll>), grid_partial,
              block, go, w, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
              a.segment_starts, a.counters, a.long_segments, a.chunk_segments, partial, a.max_long,
-             a.D, g.chunks);
+             a.D, g.chunks, a.unique_slots, cr);
 
   const int64_t want_long = ceil_div(ceil_div(a.max_long, groups), kWavesPerBlock);
   const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
   TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, OPT>),
              grid_finish, block, w, st, a.keys_sorted, a.segment_starts, a.counters,
-             a.long_segments, partial, a.max_long, a.D, g.chunks, a.learning_rate, a.eps);
+             a.long_segments, partial, a.max_long, a.D, g.chunks, a.learning_rate, a.eps,
+             a.unique_slots, cr);
 }
 
 template <typename T, int VEC, int OPT, bool WEIGHTED>
@@ -472,7 +492,8 @@ void launch_geometry(const UpdateArgs &a, const RowGeometry &g, hipStream_t stre
                static_cast<T *>(a.weights), static_cast<A *>(a.optimizer_state),
                static_cast<const T *>(a.per_sample_weights),
                static_cast<T *>(a.grad_per_sample_weights), a.keys_sorted, a.positions_sorted,
-               a.grad_rows, a.segment_starts, a.counters, a.D, g.chunks, a.learning_rate, a.eps);
+               a.grad_rows, a.segment_starts, a.counters, a.D, g.chunks, a.learning_rate, a.eps,
+               a.unique_slots, static_cast<T *>(a.cache_rows));
     return;
   }
   switch (g.tmpl) {

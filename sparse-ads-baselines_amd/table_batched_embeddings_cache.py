@@ -1,0 +1,145 @@
+"""Host side of the HBM row cache that fronts a host-resident embedding table.
+
+`RowCache` owns the cache state in device memory (tags, recency / frequency words, the
+cached rows), two scratch workspaces and a side stream, and drives the C-ABI cache entry
+points of include/tbe_hip.h.  The reference has no cache: its HOST_MAPPED location reads
+every row over the bus (table_batched_embeddings_ops.py:159-167).
+"""
+import ctypes
+
+import torch
+
+import tbe_native as _native
+
+_DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F16,
+                torch.float64: _native.DTYPE_F64}
+_POLICIES = {"lru": _native.CACHE_LRU, "lfu": _native.CACHE_LFU}
+STAT_NAMES = ("unique_rows", "hits", "misses", "inserted", "written_back", "uncached")
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr() if t is not None and t.numel() > 0 else 0)
+
+
+class RowCache:
+    def __init__(self, backing_weights, cache_slots, policy="lru"):
+        """backing_weights: [rows, D] tensor whose storage is device-visible host memory
+        (table_batched_embeddings.new_host_mapped_tensor) -- or plain device memory, which is
+        useful for tests.  cache_slots is rounded down to a multiple of 64 (one set)."""
+        if policy not in _POLICIES:
+            raise ValueError("cache policy must be 'lru' or 'lfu'")
+        if not backing_weights.is_cuda or backing_weights.dim() != 2 or not backing_weights.is_contiguous():
+            raise RuntimeError("backing_weights must be a contiguous [rows, D] GPU-visible tensor")
+        self.device = backing_weights.device
+        self.backing = backing_weights
+        self.D = backing_weights.size(1)
+        self.dtype_code = _DTYPE_CODES[backing_weights.dtype]
+        self.num_sets = int(cache_slots) // _native.CACHE_WAYS
+        if self.num_sets < 1:
+            raise ValueError("cache_slots must be at least %d" % _native.CACHE_WAYS)
+        slots = self.num_sets * _native.CACHE_WAYS
+        self.tags = torch.empty(slots, dtype=torch.int32, device=self.device)
+        self.last_used = torch.empty(slots, dtype=torch.int32, device=self.device)
+        self.use_count = torch.empty(slots, dtype=torch.int32, device=self.device)
+        self.rows = torch.empty(slots, self.D, dtype=backing_weights.dtype, device=self.device)
+        self.handle = _native.Cache(_ptr(self.tags), _ptr(self.last_used), _ptr(self.use_count), _ptr(self.rows),
+                                    _ptr(self.backing), self.num_sets, _POLICIES[policy])
+        self.side_stream = torch.cuda.Stream(device=self.device)  # default priority
+        self.step = 0
+        self._plan_ws = None
+        self._cache_ws = None
+        self._layout = None
+        self._plan_layout = None
+        self._n = 0
+        with torch.cuda.device(self.device):
+            _native.check(_native.load().tbe_cache_init(ctypes.byref(self.handle), self._stream()))
+
+    def _stream(self):
+        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _grow(self, current, nbytes):
+        if current is None or current.numel() < nbytes:
+            return torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=self.device)
+        return current
+
+    def _view(self, ws, offset, count):
+        return ws[offset:offset + 4 * count].view(torch.int32)
+
+    def prepare(self, table_offsets, indices, offsets):
+        """Sorts the batch, probes / fills the cache for its unique rows and builds the
+        per-lookup slot table.  Must precede forward() and backward() of the same batch."""
+        T = table_offsets.numel()
+        B = (offsets.numel() - 1) // T
+        n = indices.numel()
+        self.step += 1
+        self._n, self._T, self._B = n, T, B
+        self._plan_layout = _native.backward_workspace_layout(n, self.D, self.dtype_code)
+        self._layout = _native.cache_workspace_layout(n, self.num_sets)
+        self._plan_ws = self._grow(self._plan_ws, self._plan_layout.total_bytes)
+        self._cache_ws = self._grow(self._cache_ws, self._layout.total_bytes)
+        with torch.cuda.device(self.device):
+            _native.check(_native.load().tbe_cache_prepare(
+                ctypes.byref(self.handle), self.dtype_code, self.backing.size(0), self.D, _ptr(table_offsets), T,
+                _ptr(indices), n, _ptr(offsets), B, self.step, _ptr(self._plan_ws), self._plan_ws.numel(),
+                _ptr(self._cache_ws), self._cache_ws.numel(), self._stream(),
+                ctypes.c_void_p(self.side_stream.cuda_stream)))
+
+    @property
+    def lookup_slots(self):
+        return self._view(self._cache_ws, self._layout.lookup_slots, self._n)
+
+    def unique_slots(self):
+        U = int(self._view(self._plan_ws, self._plan_layout.num_unique, 1)[0])
+        return self._view(self._cache_ws, self._layout.unique_slots, U)
+
+    def unique_keys(self):
+        U = int(self._view(self._plan_ws, self._plan_layout.num_unique, 1)[0])
+        starts = self._view(self._plan_ws, self._plan_layout.segment_starts, U).long()
+        return self._view(self._plan_ws, self._plan_layout.keys_sorted, self._n)[starts]
+
+    def evicted_keys(self):
+        U = int(self._view(self._plan_ws, self._plan_layout.num_unique, 1)[0])
+        return self._view(self._cache_ws, self._layout.evicted_keys, U)
+
+    def stats(self):
+        """Counters of the last prepare() (synchronises)."""
+        values = self._view(self._cache_ws, self._layout.stats, 8).tolist()
+        return dict(zip(STAT_NAMES, values))
+
+    def forward(self, table_offsets, indices, offsets, per_sample_weights=None):
+        T, B = self._T, self._B
+        output = torch.empty((B, T, self.D), dtype=self.backing.dtype, device=self.device)
+        slots = self.lookup_slots if self._n else None
+        with torch.cuda.device(self.device):
+            _native.check(_native.load().tbe_forward_cached(
+                ctypes.byref(self.handle), self.dtype_code, self.D, _ptr(table_offsets), T, _ptr(indices), self._n,
+                _ptr(offsets), B, _ptr(per_sample_weights), _ptr(slots), _ptr(output), self._stream()))
+        return output
+
+    def backward(self, optimizer, grad_output, per_sample_weights, optimizer_state, learning_rate, eps):
+        """optimizer: 'sgd' or 'adagrad'.  Updates rows where they live; returns the gradient
+        w.r.t. per_sample_weights or None."""
+        grad_output = grad_output.contiguous()
+        grad_psw = None
+        if per_sample_weights is not None:
+            grad_psw = torch.empty(self._n, dtype=grad_output.dtype, device=self.device)
+        code = _native.OPT_SGD if optimizer == "sgd" else _native.OPT_ROWWISE_ADAGRAD
+        unique = self._view(self._cache_ws, self._layout.unique_slots, max(self._n, 1))
+        with torch.cuda.device(self.device):
+            _native.check(_native.load().tbe_backward_cached(
+                code, _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.backing.size(0), self.D,
+                self._T, self._B, self._n, _ptr(per_sample_weights),
+                _ptr(optimizer_state) if optimizer != "sgd" else ctypes.c_void_p(0), float(learning_rate),
+                float(eps or 0.0), _ptr(grad_psw), _ptr(self._plan_ws), self._plan_ws.numel(), _ptr(unique),
+                self._stream()))
+        return grad_psw
+
+    def flush(self):
+        """Writes every resident row back to the backing table."""
+        with torch.cuda.device(self.device):
+            _native.check(_native.load().tbe_cache_flush(ctypes.byref(self.handle), self.dtype_code, self.D,
+                                                         self._stream()))
+
+    def resident_keys(self):
+        """Sorted keys of the rows currently held (synchronises)."""
+        return torch.sort(self.tags[self.tags >= 0])[0]

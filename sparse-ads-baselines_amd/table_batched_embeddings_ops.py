@@ -16,6 +16,7 @@ import torch
 from torch import nn
 
 import table_batched_embeddings
+import table_batched_embeddings_cache
 
 
 class Optimizer(enum.Enum):
@@ -27,6 +28,7 @@ class Optimizer(enum.Enum):
 class EmbeddingLocation(enum.Enum):
     DEVICE = 0
     HOST_MAPPED = 1
+    HOST_CACHED = 2  # extension: pinned host table fronted by an HBM row cache
 
 
 def _launch_block(D):
@@ -81,14 +83,47 @@ class LookupFunction(torch.autograd.Function):
         return (empty_grad, None, None, None, grad_per_sample_weight, None, None, None, None, None)
 
 
+class CachedLookupFunction(torch.autograd.Function):
+    """LookupFunction for tables that live in host memory behind an HBM row cache: the batch
+    is planned (sorted, cut into unique rows) once, the cache is probed / filled for those
+    rows, and forward and backward address every row where it lives."""
+
+    @staticmethod
+    def forward(ctx, weights, module, indices, offsets, per_sample_weights):
+        cache = module.row_cache
+        cache.prepare(module.table_offsets, indices, offsets)
+        ctx.module = module
+        ctx.save_for_backward(weights, per_sample_weights)
+        return cache.forward(module.table_offsets, indices, offsets, per_sample_weights)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        weights, per_sample_weights = ctx.saved_tensors
+        module = ctx.module
+        if module.optimizer == Optimizer.SGD:
+            assert per_sample_weights is None
+            kind = "sgd"
+        else:
+            kind = "adagrad"
+        grad_per_sample_weight = module.row_cache.backward(
+            kind, grad_output, per_sample_weights, module.optimizer_state, module.learning_rate, module.eps)
+        empty_grad = None
+        if ctx.needs_input_grad[0]:
+            empty_grad = torch.sparse_coo_tensor(
+                torch.empty((2, 0), dtype=torch.int64, device=weights.device),
+                torch.empty((0,), dtype=weights.dtype, device=weights.device), size=tuple(weights.shape))
+        return (empty_grad, None, None, None, grad_per_sample_weight)
+
+
 class TableBatchedEmbeddingBags(nn.Module):
     """Mirror of TableBatchedEmbeddingBags (table_batched_embeddings_ops.py:135-201)."""
 
     def __init__(self, num_tables, num_embeddings, embedding_dim, optimizer=Optimizer.SGD,
                  learning_rate=0.01, eps=None, stochastic_rounding=False, fp16=False,
-                 managed=EmbeddingLocation.DEVICE):
+                 managed=EmbeddingLocation.DEVICE, cache_slots=None, cache_policy="lru"):
         super(TableBatchedEmbeddingBags, self).__init__()
-        assert managed in (EmbeddingLocation.DEVICE, EmbeddingLocation.HOST_MAPPED)
+        assert managed in (EmbeddingLocation.DEVICE, EmbeddingLocation.HOST_MAPPED,
+                           EmbeddingLocation.HOST_CACHED)
         if isinstance(num_embeddings, (list, tuple, np.ndarray)):
             rows = [int(r) for r in num_embeddings]
             assert len(rows) == num_tables
@@ -100,12 +135,24 @@ class TableBatchedEmbeddingBags(nn.Module):
         if managed == EmbeddingLocation.DEVICE:
             logging.info("Allocating device embedding bag")
             embedding_data = torch.randn(total_rows, embedding_dim, device=device, dtype=dtype)
-        else:
+        elif managed == EmbeddingLocation.HOST_MAPPED:
             logging.info("Allocating host-mapped embedding bag")
             embedding_data = table_batched_embeddings.new_managed_tensor(
                 torch.empty(1, device=device, dtype=dtype), (total_rows, embedding_dim))
             embedding_data.normal_()
+        else:
+            logging.info("Allocating pinned host embedding bag behind an HBM row cache")
+            embedding_data = table_batched_embeddings.new_host_mapped_tensor(
+                torch.empty(1, device=device, dtype=dtype), (total_rows, embedding_dim))
+            embedding_data.normal_()
         self.embedding_weights = nn.Parameter(embedding_data)
+        self.row_cache = None
+        if managed == EmbeddingLocation.HOST_CACHED:
+            assert cache_slots is not None, "HOST_CACHED needs cache_slots"
+            self.row_cache = table_batched_embeddings_cache.RowCache(self.embedding_weights.data, cache_slots,
+                                                                     cache_policy)
+            # checkpoints must see the rows the cache holds
+            self.register_state_dict_pre_hook(lambda module, prefix, keep_vars: module.flush_cache())
         self.register_buffer("table_offsets",
                              torch.tensor([0] + np.cumsum(rows[:-1]).tolist()).int())
         # unused by SGD, kept so state dicts interchange (table_batched_embeddings_ops.py:177-180)
@@ -115,7 +162,15 @@ class TableBatchedEmbeddingBags(nn.Module):
         self.eps = eps
         self.stochastic_rounding = stochastic_rounding
 
+    def flush_cache(self):
+        """Writes the rows held by the HBM cache back to embedding_weights (no-op without a cache)."""
+        if self.row_cache is not None:
+            self.row_cache.flush()
+
     def forward(self, sharded_sparse_features, sharded_offsets, per_sample_weights=None):
+        if self.row_cache is not None:
+            return CachedLookupFunction.apply(self.embedding_weights, self, sharded_sparse_features,
+                                              sharded_offsets, per_sample_weights)
         return LookupFunction.apply(
             self.embedding_weights, self.table_offsets, sharded_sparse_features, sharded_offsets,
             per_sample_weights, self.optimizer, self.optimizer_state, self.learning_rate, self.eps,

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -41,6 +41,33 @@ class WorkspaceLayout(ctypes.Structure):
     ]
 
 
+class Cache(ctypes.Structure):
+    """Mirror of tbe_cache_t."""
+
+    _fields_ = [
+        ("tags", _vp),
+        ("last_used", _vp),
+        ("use_count", _vp),
+        ("rows", _vp),
+        ("backing_rows", _vp),
+        ("num_sets", _i64),
+        ("policy", _i32),
+    ]
+
+
+class CacheWorkspaceLayout(ctypes.Structure):
+    """Mirror of tbe_cache_workspace_layout_t."""
+
+    _fields_ = [(name, _u64) for name in (
+        "total_bytes", "unique_slots", "lookup_slots", "evicted_keys", "segment_ids", "miss_sets", "miss_list",
+        "set_counts", "set_fill", "set_starts", "stats")]
+
+
+CACHE_WAYS = 64
+CACHE_LRU, CACHE_LFU = 0, 1
+OPT_SGD, OPT_ROWWISE_ADAGRAD = 0, 1
+_cache_p = ctypes.POINTER(Cache)
+
 # name -> (restype, argtypes); exactly the declarations of include/tbe_hip.h
 SIGNATURES = {
     "tbe_last_error": (ctypes.c_char_p, []),
@@ -61,6 +88,15 @@ SIGNATURES = {
     "tbe_segments_workspace_bytes": (_u64, [_i64]),
     "tbe_find_segments": (ctypes.c_int, [_c_i32p, _i64, _c_i32p, _c_i32p, _vp, _u64, _vp]),
     "tbe_construct_offsets": (ctypes.c_int, [_c_i32p, _c_i32p, _i32, _i32, _c_i32p, _vp]),
+    "tbe_cache_workspace_layout": (ctypes.c_int, [_i64, _i64, ctypes.POINTER(CacheWorkspaceLayout)]),
+    "tbe_cache_init": (ctypes.c_int, [_cache_p, _vp]),
+    "tbe_cache_prepare": (ctypes.c_int, [_cache_p, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32,
+                                         _i32, _vp, _u64, _vp, _u64, _vp, _vp]),
+    "tbe_forward_cached": (ctypes.c_int, [_cache_p, _i32, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp,
+                                          _c_i32p, _vp, _vp]),
+    "tbe_backward_cached": (ctypes.c_int, [_i32, _vp, _cache_p, _i32, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _f32,
+                                           _f32, _vp, _vp, _u64, _c_i32p, _vp]),
+    "tbe_cache_flush": (ctypes.c_int, [_cache_p, _i32, _i32, _vp]),
     "tbe_host_mapped_alloc": (ctypes.c_int, [_u64, ctypes.POINTER(_vp), ctypes.POINTER(_vp)]),
     "tbe_host_mapped_free": (ctypes.c_int, [_vp]),
     "tbe_managed_alloc": (ctypes.c_int, [_u64, _i32, ctypes.POINTER(_vp)]),
@@ -106,6 +142,12 @@ def check(code):
 def backward_workspace_layout(num_indices, D, dtype_code):
     layout = WorkspaceLayout()
     check(load().tbe_backward_workspace_layout(num_indices, D, dtype_code, ctypes.byref(layout)))
+    return layout
+
+
+def cache_workspace_layout(num_indices, num_sets):
+    layout = CacheWorkspaceLayout()
+    check(load().tbe_cache_workspace_layout(num_indices, num_sets, ctypes.byref(layout)))
     return layout
 
 

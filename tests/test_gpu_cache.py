@@ -1,0 +1,174 @@
+"""GPU parity of the HBM row cache (tbe_cache_* through the C ABI).
+
+The reference has no cache, so the checker is the CPU model of this repository's own
+specification (oracle/lxu_cache_model.c) plus the property that ties the cache back to the
+reference's semantics: a run through the cache equals, bit for bit, a run with the tables
+fully in HBM, because the arithmetic kernels are the same and only row addresses differ."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_problem
+from gpu_util import DEV, dev
+
+import table_batched_embeddings as ext
+import table_batched_embeddings_cache as tc
+import table_batched_embeddings_ops as ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _draw_batch(rs, T, rows, B, L, zipf):
+    lengths = rs.randint(0, L + 1, size=(T, B))
+    offsets = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
+    per_table = lengths.sum(axis=1)
+    indices = np.concatenate([(rs.zipf(zipf, size=int(per_table[t])) % rows[t]) for t in range(T)]).astype(np.int32)
+    return indices, offsets
+
+
+@pytest.mark.parametrize("policy", ["lru", "lfu"])
+@pytest.mark.parametrize("num_sets", [1, 5, 64])
+def test_cache_state_matches_model_bit_exact(oracle, policy, num_sets):
+    """tags / recency / frequency words, slot of every unique row, evicted keys and counters
+    after every step equal the CPU model's."""
+    rs = np.random.RandomState(num_sets * 7 + len(policy))
+    T, rows, B, L, D = 3, [300, 5000, 40], 64, 12, 32
+    table_offsets = np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32)
+    backing = torch.randn(sum(rows), D, device=DEV)
+    cache = tc.RowCache(backing, num_sets * 64, policy)
+    model = oracle.CacheModel(num_sets, policy)
+    for step in range(8):
+        indices, offsets = _draw_batch(rs, T, rows, B, L, 1.15)
+        cache.prepare(dev(table_offsets), dev(indices), dev(offsets))
+        keys = np.unique(table_offsets[np.repeat(np.arange(T * B), np.diff(offsets)) // B] + indices)
+        slots, evicted, stats = model.step(keys)
+        np.testing.assert_array_equal(cache.unique_keys().cpu().numpy(), keys)
+        np.testing.assert_array_equal(cache.unique_slots().cpu().numpy(), slots)
+        np.testing.assert_array_equal(cache.evicted_keys().cpu().numpy(), evicted)
+        np.testing.assert_array_equal(cache.tags.cpu().numpy(), model.tags)
+        np.testing.assert_array_equal(cache.last_used.cpu().numpy(), model.last_used)
+        np.testing.assert_array_equal(cache.use_count.cpu().numpy(), model.use_count)
+        np.testing.assert_array_equal(cache.resident_keys().cpu().numpy(), model.resident())
+        assert list(cache.stats().values()) == stats.tolist()
+        # per-lookup slots agree with per-unique slots
+        all_keys = table_offsets[np.repeat(np.arange(T * B), np.diff(offsets)) // B] + indices
+        np.testing.assert_array_equal(cache.lookup_slots.cpu().numpy(), slots[np.searchsorted(keys, all_keys)])
+
+
+@pytest.mark.parametrize("mode,dtype,D", [("sgd", torch.float32, 128), ("adagrad", torch.float32, 64),
+                                          ("adagrad_weighted", torch.float16, 64), ("sgd", torch.float32, 520),
+                                          ("sgd", torch.float64, 12)])
+@pytest.mark.parametrize("num_sets", [2, 40])
+def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets):
+    """Several forward + backward steps through the cache, then a flush: outputs of every step,
+    the final table, optimizer state and per-sample-weight gradients are bit-identical to the
+    same steps on a table that lives entirely in device memory.  With 2 sets most rows are
+    served straight from the backing table; with 40 most are cached."""
+    rs = np.random.RandomState(3)
+    T, rows, B, L = 3, [700, 90, 3000], 48, 9
+    table_offsets = dev(np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
+    total = sum(rows)
+    start = (torch.rand(total, D, device=DEV, dtype=torch.float64) * 0.02 - 0.01).to(dtype)
+    plain_w = start.clone()
+    cached_w = ext.new_host_mapped_tensor(torch.empty(1, device=DEV, dtype=dtype), (total, D))
+    cached_w.copy_(start)
+    st_dtype = torch.float64 if dtype == torch.float64 else torch.float32
+    plain_state = torch.zeros(total, device=DEV, dtype=st_dtype)
+    cached_state = torch.zeros(total, device=DEV, dtype=st_dtype)
+    cache = tc.RowCache(cached_w, num_sets * 64, "lru")
+    weighted = mode.endswith("weighted")
+    opt = "sgd" if mode == "sgd" else "adagrad"
+    served_uncached = 0
+    for step in range(6):
+        indices, offsets = _draw_batch(rs, T, rows, B, L, 1.2)
+        idx, off = dev(indices), dev(offsets)
+        go = torch.randn(B, T, D, device=DEV, dtype=torch.float64).to(dtype)
+        psw = torch.rand(indices.size, device=DEV, dtype=torch.float64).to(dtype) if weighted else None
+        want = ext.forward(plain_w, table_offsets, idx, off, psw, 200, 1, False)
+        if opt == "sgd":
+            ext.backward_sgd(go, plain_w, table_offsets, idx, off, 0.05, 200, 1, False)
+            want_g = None
+        else:
+            want_g = ext.backward_exact_adagrad(go, plain_w, table_offsets, idx, off, psw, plain_state, 0.05, 0.1,
+                                                False, 1)
+        cache.prepare(table_offsets, idx, off)
+        got = cache.forward(table_offsets, idx, off, psw)
+        got_g = cache.backward(opt, go, psw, cached_state, 0.05, 0.1)
+        assert torch.equal(got, want), "forward output differs at step %d" % step
+        if weighted:
+            assert torch.equal(got_g, want_g)
+        served_uncached += cache.stats()["uncached"]
+    cache.flush()
+    torch.cuda.synchronize()
+    assert torch.equal(cached_w, plain_w)
+    assert torch.equal(cached_state, plain_state)
+    assert (served_uncached > 0) == (num_sets == 2)
+    ext.free_host_tensor(cached_w)
+
+
+def test_flush_before_any_step_and_empty_batch():
+    backing = torch.randn(100, 16, device=DEV)
+    before = backing.clone()
+    cache = tc.RowCache(backing, 64)
+    cache.flush()
+    torch.cuda.synchronize()
+    assert torch.equal(backing, before)
+    to = dev(np.zeros(1, np.int32))
+    cache.prepare(to, torch.zeros(0, dtype=torch.int32, device=DEV), dev(np.zeros(5, np.int32)))
+    out = cache.forward(to, torch.zeros(0, dtype=torch.int32, device=DEV), dev(np.zeros(5, np.int32)))
+    assert out.shape == (4, 1, 16) and not out.any()
+    assert cache.stats()["unique_rows"] == 0
+
+
+def test_module_host_cached_trains_like_device_module():
+    """The drop-in module with managed=HOST_CACHED follows the same trajectory as the plain
+    device module, and state_dict() sees the rows the cache holds."""
+    T, E, D, B, L = 4, 500, 64, 32, 6
+    torch.manual_seed(0)
+    plain = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.EXACT_ROWWISE_ADAGRAD, learning_rate=0.1,
+                                          eps=0.1).cuda()
+    cached = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.EXACT_ROWWISE_ADAGRAD,
+                                           learning_rate=0.1, eps=0.1, managed=ops.EmbeddingLocation.HOST_CACHED,
+                                           cache_slots=256).cuda()
+    cached.embedding_weights.data.copy_(plain.embedding_weights.data)
+    assert set(cached.state_dict()) == {"embedding_weights", "table_offsets", "optimizer_state"}
+    rs = np.random.RandomState(1)
+    for _ in range(5):
+        p = make_problem(rs.randint(1 << 30), T, E, D, B, L, np.float32, zipf=1.2)
+        idx, off, go = dev(p["indices"]), dev(p["offsets"]), dev(p["grad_output"])
+        a = plain(idx, off)
+        a.backward(go)
+        b = cached(idx, off)
+        b.backward(go)
+        assert torch.equal(a, b)
+    sd = cached.state_dict()
+    torch.cuda.synchronize()
+    assert torch.equal(sd["embedding_weights"], plain.embedding_weights.data)
+    assert torch.equal(sd["optimizer_state"], plain.optimizer_state)
+    hit_rate = cached.row_cache.stats()
+    assert hit_rate["hits"] > 0 and hit_rate["unique_rows"] == hit_rate["hits"] + hit_rate["misses"]
+
+
+def test_host_tensors_behave_like_device_tensors():
+    """new_managed_tensor / new_host_mapped_tensor (table_batched_embeddings_cuda.cu:864-880):
+    tagged as GPU tensors, usable by torch ops and by the kernels."""
+    proto = torch.empty(1, device=DEV)
+    for make in (ext.new_host_mapped_tensor, ext.new_managed_tensor):
+        t = make(proto, (300, 32))
+        assert t.is_cuda and t.dtype == torch.float32 and tuple(t.shape) == (300, 32)
+        t.normal_()
+        ref = t.clone()
+        to = dev(np.zeros(1, np.int32))
+        idx = torch.randint(0, 300, (20 * 5,), dtype=torch.int32, device=DEV)
+        off = torch.arange(0, 101, 5, dtype=torch.int32, device=DEV)
+        assert torch.equal(ext.forward(t, to, idx, off, None, 200, 1, False),
+                           ext.forward(ref, to, idx, off, None, 200, 1, False))
+        go = torch.randn(20, 1, 32, device=DEV)
+        ext.backward_sgd(go, t, to, idx, off, 0.1, 200, 1, False)
+        ext.backward_sgd(go, ref, to, idx, off, 0.1, 200, 1, False)
+        torch.cuda.synchronize()
+        assert torch.equal(t, ref)
+        ext.free_host_tensor(t)
+    half = ext.new_host_mapped_tensor(torch.empty(1, device=DEV, dtype=torch.float16), (8, 4))
+    assert half.dtype == torch.float16
+    ext.free_host_tensor(half)

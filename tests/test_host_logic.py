@@ -13,7 +13,9 @@ def test_enums_keep_reference_values():
     # table_batched_embeddings_ops.py:124-132
     assert [(e.name, e.value) for e in ops.Optimizer] == [("SGD", 1), ("APPROX_ROWWISE_ADAGRAD", 2),
                                                           ("EXACT_ROWWISE_ADAGRAD", 3)]
-    assert [(e.name, e.value) for e in ops.EmbeddingLocation] == [("DEVICE", 0), ("HOST_MAPPED", 1)]
+    # DEVICE / HOST_MAPPED as in the reference; HOST_CACHED is this library's extension
+    assert [(e.name, e.value) for e in ops.EmbeddingLocation] == [("DEVICE", 0), ("HOST_MAPPED", 1),
+                                                                   ("HOST_CACHED", 2)]
 
 
 def test_extension_module_exports_the_ten_reference_functions():
@@ -41,8 +43,9 @@ def test_positional_signatures_match_the_pybind_declarations():
 def test_module_constructor_signature_matches_reference():
     # table_batched_embeddings_ops.py:136-147
     params = inspect.signature(ops.TableBatchedEmbeddingBags.__init__).parameters
+    # the reference's nine arguments in order, then the cache extension
     assert list(params)[1:] == ["num_tables", "num_embeddings", "embedding_dim", "optimizer", "learning_rate", "eps",
-                                "stochastic_rounding", "fp16", "managed"]
+                                "stochastic_rounding", "fp16", "managed", "cache_slots", "cache_policy"]
     assert params["optimizer"].default is ops.Optimizer.SGD
     assert params["learning_rate"].default == 0.01
     assert params["managed"].default is ops.EmbeddingLocation.DEVICE

@@ -236,3 +236,88 @@ def test_backward_intermediates_are_sort_and_unique_of_keys(oracle):
     np.testing.assert_array_equal(r["keys_sorted"], keys[order])
     np.testing.assert_array_equal(r["positions_sorted"], order)
     np.testing.assert_array_equal(r["segment_starts"][:-1], np.unique(keys[order], return_index=True)[1])
+
+
+# ------------------------------------------------------------------ row cache model
+# The reference has no cache; these pin oracle/lxu_cache_model.c to this repository's own
+# specification (include/tbe_hip.h, above tbe_cache_t).  Parity with the reference is unpinned.
+def _brute_force_cache_step(state, num_sets, policy, step, keys, set_of):
+    """Direct transcription of the specification with Python lists."""
+    tags, used, count = state
+    slots, evicted = [-1] * len(keys), [-2] * len(keys)
+    for u, key in enumerate(keys):                      # phase 1: hits
+        base = set_of(key, num_sets) * 64
+        for w in range(64):
+            if tags[base + w] == key:
+                slots[u] = base + w
+                used[base + w] = step
+                count[base + w] += 1
+    for u, key in enumerate(keys):                      # phase 2: inserts, ascending key order
+        if slots[u] >= 0:
+            continue
+        base = set_of(key, num_sets) * 64
+        free = [(count[base + w] if policy == "lfu" else used[base + w], w) for w in range(64)
+                if used[base + w] < step]
+        if not free:
+            continue
+        _, w = min(free)
+        evicted[u] = tags[base + w] if tags[base + w] >= 0 else -1
+        tags[base + w], used[base + w], count[base + w] = key, step, 1
+        slots[u] = base + w
+    return slots, evicted
+
+
+@pytest.mark.parametrize("policy", ["lru", "lfu"])
+@pytest.mark.parametrize("num_sets,universe", [(1, 150), (3, 400), (8, 600)])
+def test_cache_model_matches_brute_force(oracle, policy, num_sets, universe):
+    rs = np.random.RandomState(num_sets)
+    model = oracle.CacheModel(num_sets, policy)
+    state = ([-1] * (64 * num_sets), [0] * (64 * num_sets), [0] * (64 * num_sets))
+    for step in range(1, 9):
+        keys = np.unique((rs.zipf(1.3, size=rs.randint(1, 300)) % universe).astype(np.int32))
+        slots, evicted, stats = model.step(keys)
+        want_slots, want_evicted = _brute_force_cache_step(state, num_sets, policy, step, keys.tolist(),
+                                                           oracle.cache_set_of)
+        assert slots.tolist() == want_slots and evicted.tolist() == want_evicted
+        assert model.tags.tolist() == state[0] and model.last_used.tolist() == state[1]
+        assert model.use_count.tolist() == state[2]
+        # invariants
+        resident = model.tags[model.tags >= 0]
+        assert np.unique(resident).size == resident.size <= 64 * num_sets
+        assert stats[0] == keys.size and stats[1] + stats[2] == keys.size
+        assert stats[3] + stats[5] == stats[2] and stats[4] == (evicted >= 0).sum()
+        assert ((slots >= 0) | (evicted == -2)).all()
+        assert np.isin(keys[slots >= 0], resident).all()          # used this step => still resident
+        assert (model.tags[slots[slots >= 0]] == keys[slots >= 0]).all()
+
+
+def test_cache_hash_spreads_and_is_in_range(oracle):
+    sets = np.array([oracle.cache_set_of(k, 1000) for k in range(20000)])
+    assert sets.min() >= 0 and sets.max() < 1000
+    assert np.bincount(sets, minlength=1000).max() < 60       # 20 expected per set
+    assert oracle.cache_set_of(12345, 1) == 0
+
+
+def test_cache_lru_and_lfu_pick_different_victims(oracle):
+    # one set: fill it with 64 keys, use key A often and long ago, key B once and recently
+    for policy, expect_gone in (("lru", 0), ("lfu", 1)):
+        m = oracle.CacheModel(1, policy)
+        m.step(np.arange(64, dtype=np.int32))                     # step 1: all inserted
+        for _ in range(3):
+            m.step(np.array([0], np.int32))                       # steps 2-4: key 0 used 3 more times
+        m.step(np.arange(1, 64, dtype=np.int32))                  # step 5: everything but key 0
+        m.step(np.arange(2, 64, dtype=np.int32))                  # step 6: everything but keys 0, 1
+        m.step(np.arange(2, 64, dtype=np.int32))                  # step 7: same (their counts pass key 0's)
+        slots, evicted, _ = m.step(np.array([1000], np.int32))    # step 8: one new key needs a victim
+        # LRU evicts key 0 (last used in step 4, key 1 in step 5); LFU evicts key 1 (2 uses < key 0's 4)
+        assert evicted.tolist() == [expect_gone]
+        assert 1000 in m.resident() and expect_gone not in m.resident()
+
+
+def test_cache_rows_used_in_a_step_are_never_evicted_in_it(oracle):
+    m = oracle.CacheModel(1, "lru")
+    m.step(np.arange(64, dtype=np.int32))
+    slots, evicted, stats = m.step(np.arange(0, 100, dtype=np.int32))   # 64 hits, 36 misses, no free way
+    assert stats.tolist() == [100, 64, 36, 0, 0, 36]
+    assert (slots[64:] == -1).all() and (evicted == -2).all()
+    assert m.resident().tolist() == list(range(64))
