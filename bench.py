@@ -11,7 +11,8 @@ region.  Prints ONE JSON line.  Everything runs on one GPU.
 Default workload = BASELINE config 3 (the shape the target is quoted on):
 T=64 tables x 100k rows x D=128 fp32, B=4096 bags per table, L=20, Zipf(1.05) indices,
 exact SGD lr=0.01.  --config 2 times the forward alone on uniform indices; --config 4 the
-fp16 / weighted / exact row-wise Adagrad shape.
+fp16 / weighted / exact row-wise Adagrad shape; --config 5 the DLRM-style shape whose tables
+live in pinned host memory behind the HBM row cache (indices re-drawn every step).
 """
 import argparse
 import json
@@ -59,14 +60,64 @@ def make_workload(config, seed=0):
         name = ("cfg4 fwd + weighted exact row-wise Adagrad: T=32 E=1M D=64 fp16 B=8192 L~U[0,40] Zipf(1.2) "
                 "lr=0.01 eps=1e-8")
         w = dict(T=T, E=E, D=D, B=B, fp16=True, weighted=True, optimizer="adagrad", lr=0.01, eps=1e-8)
+    elif config == 5:
+        T, D, B = 26, 128, 65536
+        rows = np.floor(np.exp(rs.uniform(np.log(1e3), np.log(2e7), size=T))).astype(np.int64)
+        w = dict(T=T, E=[int(r) for r in rows], D=D, B=B, fp16=False, weighted=False, optimizer="sgd", lr=0.01,
+                 eps=0.0, cache_slots=1 << 22, n=0, seed=seed, indices=None, offsets=None,
+                 name="cfg5 DLRM-style + row cache: T=26 rows log-uniform [1e3,2e7] (sum %d) D=128 fp32 in pinned host "
+                      "memory, 2^22-slot LRU cache, B=65536 L=clip(Poisson(30),1,100) Zipf(1.1) per-table hot set, "
+                      "fwd + exact SGD lr=0.01, indices re-drawn every step" % int(rows.sum()))
+        return w
     else:
-        raise SystemExit("bench.py: --config must be 2, 3 or 4")
+        raise SystemExit("bench.py: --config must be 2, 3, 4 or 5")
     w["name"] = name
     w["indices"] = indices.astype(np.int32)
     w["offsets"] = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
     w["n"] = n
     w["seed"] = seed
     return w
+
+
+def zipf_on_device(torch, a, n, gen, dev):
+    """n samples of Zipf(a) as int64, by the rejection method numpy.random.zipf uses
+    (Devroye, "Non-Uniform Random Variate Generation", p. 551), vectorised on the GPU."""
+    am1 = a - 1.0
+    b = 2.0 ** am1
+    out = []
+    have = 0
+    while have < n:
+        m = int((n - have) * 1.3) + 1024
+        U = 1.0 - torch.rand(m, dtype=torch.float64, device=dev, generator=gen)
+        V = torch.rand(m, dtype=torch.float64, device=dev, generator=gen)
+        X = torch.floor(U.pow(-1.0 / am1))
+        ok = (X >= 1.0) & (X < 9.0e18)
+        Tt = (1.0 + 1.0 / X.clamp(min=1.0)).pow(am1)
+        ok &= V * X * (Tt - 1.0) / (b - 1.0) <= Tt / b
+        acc = X[ok].to(torch.int64)
+        out.append(acc)
+        have += acc.numel()
+    return torch.cat(out)[:n]
+
+
+def draw_cfg5_batch(torch, w, step, dev):
+    """One batch of config 5: lengths clip(Poisson(30), 1, 100); per table Zipf(1.1) mod rows,
+    pushed through a per-table affine bijection so that every table has its own hot set."""
+    T, B = w["T"], w["B"]
+    gen = torch.Generator(device=dev).manual_seed(w["seed"] * 1000003 + step)
+    lengths = torch.poisson(torch.full((T * B,), 30.0, device=dev), generator=gen).clamp_(1, 100).to(torch.int64)
+    offsets = torch.zeros(T * B + 1, dtype=torch.int64, device=dev)
+    offsets[1:] = torch.cumsum(lengths, 0)
+    per_table = lengths.view(T, B).sum(1).tolist()
+    parts = []
+    for t in range(T):
+        rows = w["E"][t]
+        x = zipf_on_device(torch, 1.1, int(per_table[t]), gen, dev) % rows
+        mult = 2 * (7919 * (t + 1)) + 1
+        while np.gcd(mult, rows) != 1:
+            mult += 2
+        parts.append(((x * (mult % rows)) % rows + (104729 * t) % rows) % rows)
+    return torch.cat(parts).to(torch.int32), offsets.to(torch.int32)
 
 
 def algorithmic_bytes(w, U):
@@ -112,6 +163,87 @@ def cpu_baseline(w, torch, tables=8, iters=3):
             "ms_per_step": sec * 1e3}
 
 
+def run_cached(args, w):
+    """Config 5: tables in pinned host memory behind the HBM row cache; one batch per step,
+    all batches resident in HBM before the timed region; cold cache included."""
+    import torch
+
+    import table_batched_embeddings_ops as ops
+    import tbe_native
+
+    dev = torch.device("cuda:0")
+    T, D, B = w["T"], w["D"], w["B"]
+    t0 = time.perf_counter()
+    module = ops.TableBatchedEmbeddingBags(T, w["E"], D, optimizer=ops.Optimizer.SGD, learning_rate=w["lr"],
+                                           managed=ops.EmbeddingLocation.HOST_CACHED,
+                                           cache_slots=w["cache_slots"]).cuda()
+    module.embedding_weights.data.mul_(0.01)
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t0
+    total = args.warmup + args.steps
+    batches = [draw_cfg5_batch(torch, w, s, dev) for s in range(total)]
+    gen = torch.Generator(device=dev).manual_seed(w["seed"])
+    grad_output = torch.randn(B, T, D, device=dev, generator=gen)
+    torch.cuda.synchronize()
+    stats = []
+
+    def step(i):
+        indices, offsets = batches[i]
+        module(indices, offsets).backward(grad_output)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.warmup, total):
+        step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    # a second, untimed pass over fresh batches collects per-step cache counters and kernel times
+    per_kernel = {}
+    lookups = 0
+    bytes_alg = 0
+    extra = [draw_cfg5_batch(torch, w, total + s, dev) for s in range(min(3, args.steps))]
+    with tbe_native.profile() as prof:
+        for indices, offsets in extra:
+            module(indices, offsets).backward(grad_output)
+            st = module.row_cache.stats()
+            stats.append(st)
+            w["n"] = indices.numel()
+            a_fwd, a_bwd, _ = algorithmic_bytes(w, st["unique_rows"])
+            bytes_alg += a_fwd + a_bwd
+            lookups += indices.numel()
+    for name, ms in prof.launches:
+        per_kernel.setdefault(name, []).append(ms)
+    kernels = {k: {"launches_per_step": len(v) / len(extra), "avg_us": 1e3 * sum(v) / len(v)}
+               for k, v in per_kernel.items()}
+    row_bytes = D * 4
+    link_bytes = [(st["inserted"] + st["written_back"] + 3 * st["uncached"]) * row_bytes for st in stats]
+    mean_lookups = sum(b[0].numel() for b in batches[args.warmup:]) / args.steps
+    sec = elapsed / args.steps
+    dominant = max(kernels, key=lambda k: kernels[k]["avg_us"] * kernels[k]["launches_per_step"])
+    result = {
+        "metric": "tbe_fwd_bwd_bags_per_sec", "value": T * B / sec, "unit": "bags/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w["name"], "T": T, "D": D, "B": B, "mean_lookups_per_step": mean_lookups,
+                   "cache_slots": w["cache_slots"], "seed": w["seed"], "host_table_GB": sum(w["E"]) * row_bytes / 1e9,
+                   "setup_seconds": setup_s},
+        "effective_GBps": (bytes_alg / len(extra)) / sec / 1e9,
+        "effective_frac_of_hbm_peak": (bytes_alg / len(extra)) / sec / HBM_PEAK,
+        "cache": {"per_step": stats,
+                  "hit_rate_unique_rows": [st["hits"] / max(st["unique_rows"], 1) for st in stats],
+                  "host_link_bytes_per_step": link_bytes},
+        "roofline": {"bound": "host-link", "kernel": dominant, "achieved": None, "peak": None, "unit": "GB/s",
+                     "frac": None, "traffic": None,
+                     "note": "misses and uncached rows cross the host link; see cache.host_link_bytes_per_step"},
+        "kernels": kernels,
+        "cpu_baseline": None,
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -139,6 +271,8 @@ def main():
         raise SystemExit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     w = make_workload(args.config)
+    if args.config == 5:
+        return run_cached(args, w)
     T, E, D, B = w["T"], w["E"], w["D"], w["B"]
     optimizer = {"sgd": ops.Optimizer.SGD, "adagrad": ops.Optimizer.EXACT_ROWWISE_ADAGRAD,
                  None: ops.Optimizer.SGD}[w["optimizer"]]
