@@ -42,6 +42,7 @@ def make_workload(config, seed=0):
     rs = np.random.RandomState(seed)
     if config in (2, 3):
         T, E, D, B, L = 64, 100000, 128, 4096, 20
+        T = int(os.environ.get("TBE_BENCH_TABLES", T))  # experiments only; the default is the BASELINE shape
         lengths = np.full(T * B, L, dtype=np.int64)
         n = T * B * L
         if config == 2:

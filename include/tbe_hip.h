@@ -97,14 +97,16 @@ typedef struct tbe_workspace_layout {
   uint64_t keys_sorted;
   uint64_t positions_sorted;
   uint64_t segment_starts;
-  uint64_t num_unique;       /* int32 [4]: U, #long segments, #long chunks, reserved   */
+  uint64_t num_unique;       /* int32 [4]: U, #long rows, #chunks, #partial rows        */
   uint64_t sort_scratch;
   uint64_t segment_scratch;
-  uint64_t long_segments;    /* int32 [2][max_long]: segment id, first chunk           */
-  uint64_t chunk_segments;   /* int32 [max_chunks]: owning long-segment slot           */
-  uint64_t partial_sums;     /* accumulator-typed [max_chunks][D]                       */
+  uint64_t segment_ids;      /* int32 [N]: index of the unique row of each sorted position */
+  uint64_t long_segments;    /* 16-byte records [max_long_segments]: rows reduced in several chunks */
+  uint64_t chunk_segments;   /* 32-byte records [max_chunks]: queue of occurrence chunks        */
+  uint64_t partial_sums;     /* accumulator-typed [max_partial_rows][D]                         */
   int64_t max_long_segments;
   int64_t max_chunks;
+  int64_t max_partial_rows;
 } tbe_workspace_layout_t;
 
 TBE_API int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int32_t dtype,
@@ -236,7 +238,6 @@ typedef struct tbe_cache_workspace_layout {
   uint64_t unique_slots;   /* int32 [U]  slot of each unique row, -1 = backing table          */
   uint64_t lookup_slots;   /* int32 [N]  the same, per lookup position                         */
   uint64_t evicted_keys;   /* int32 [U]  -2 untouched, -1 filled an empty slot, >= 0 key written back */
-  uint64_t segment_ids;    /* int32 [N]  index of the unique row of each sorted position       */
   uint64_t miss_sets;      /* int32 [U]  set of each missing row                               */
   uint64_t miss_list;      /* int32 [U]  missing rows grouped by set                           */
   uint64_t set_counts;     /* int32 [num_sets] misses per set                                  */

@@ -24,8 +24,11 @@ int key_bits(int64_t total_rows) {
 void compute_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t *l) {
   const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
   const uint64_t ints = align_up(nn * 4, 256);
-  l->max_long_segments = static_cast<int64_t>(nn / kLongSegment + 1);
-  l->max_chunks = static_cast<int64_t>(nn / kChunkLen + nn / kLongSegment + 2);
+  // a segment enters the chunk queue when it has more than kShortSegment occurrences and owns
+  // partial rows when it has more than kChunkLen
+  l->max_long_segments = static_cast<int64_t>(nn / (kChunkLen + 1) + 1);
+  l->max_chunks = static_cast<int64_t>(nn / kChunkLen + nn / (kShortSegment + 1) + 2);
+  l->max_partial_rows = static_cast<int64_t>(nn / kChunkLen + nn / (kChunkLen + 1) + 2);
   uint64_t off = 0;
   l->keys = off; off += ints;
   l->grad_rows = off; off += ints;
@@ -35,10 +38,11 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t 
   l->num_unique = off; off += 256;
   l->sort_scratch = off; off += align_up(sort_workspace_bytes(n), 256);
   l->segment_scratch = off; off += align_up(segments_workspace_bytes(n), 256);
-  l->long_segments = off; off += align_up(static_cast<uint64_t>(l->max_long_segments) * 2 * 4, 256);
-  l->chunk_segments = off; off += align_up(static_cast<uint64_t>(l->max_chunks) * 4, 256);
+  l->segment_ids = off; off += ints;
+  l->long_segments = off; off += align_up(static_cast<uint64_t>(l->max_long_segments) * 16, 256);
+  l->chunk_segments = off; off += align_up(static_cast<uint64_t>(l->max_chunks) * 32, 256);
   l->partial_sums = off;
-  off += align_up(static_cast<uint64_t>(l->max_chunks) * static_cast<uint64_t>(D) * acc_size(dtype), 256);
+  off += align_up(static_cast<uint64_t>(l->max_partial_rows) * static_cast<uint64_t>(D) * acc_size(dtype), 256);
   l->total_bytes = off;
 }
 
@@ -50,10 +54,11 @@ void backward_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t
   compute_layout(n, D, dtype, l);
 }
 
-// linearize -> sort -> run boundaries into the workspace regions of `l`.
+// linearize -> sort -> run boundaries (and the segment of every sorted position) into the
+// workspace regions of `l`.
 int build_plan(const tbe_workspace_layout_t &l, void *workspace, const int32_t *table_offsets,
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
-               int64_t total_rows, int32_t *segment_ids, hipStream_t stream) {
+               int64_t total_rows, hipStream_t stream) {
   char *ws = static_cast<char *>(workspace);
   int32_t *keys = reinterpret_cast<int32_t *>(ws + l.keys);
   int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
@@ -64,8 +69,9 @@ int build_plan(const tbe_workspace_layout_t &l, void *workspace, const int32_t *
                   n, key_bits(total_rows), ws + l.sort_scratch, stream);
   if (rc) return rc;
   return find_segments(keys_sorted, n, reinterpret_cast<int32_t *>(ws + l.segment_starts),
-                       reinterpret_cast<int32_t *>(ws + l.num_unique), segment_ids,
-                       ws + l.segment_scratch, stream);
+                       reinterpret_cast<int32_t *>(ws + l.num_unique),
+                       reinterpret_cast<int32_t *>(ws + l.segment_ids), ws + l.segment_scratch,
+                       stream);
 }
 
 namespace {
@@ -128,7 +134,7 @@ int run_backward(const char *name, const BackwardCall &c) {
 
   if (!c.planned) {
     const int rc = build_plan(l, c.workspace, c.table_offsets, c.T, c.indices, c.num_indices,
-                              c.offsets, c.B, c.total_rows, nullptr, c.stream);
+                              c.offsets, c.B, c.total_rows, c.stream);
     if (rc) return rc;
   }
 
@@ -143,8 +149,9 @@ int run_backward(const char *name, const BackwardCall &c) {
   a.grad_rows = grad_rows;
   a.segment_starts = segment_starts;
   a.counters = counters;
-  a.long_segments = reinterpret_cast<int32_t *>(ws + l.long_segments);
-  a.chunk_segments = reinterpret_cast<int32_t *>(ws + l.chunk_segments);
+  a.segment_ids = reinterpret_cast<int32_t *>(ws + l.segment_ids);
+  a.long_segments = ws + l.long_segments;
+  a.chunk_segments = ws + l.chunk_segments;
   a.partial_sums = ws + l.partial_sums;
   a.unique_slots = c.unique_slots;
   a.cache_rows = c.cache_rows;

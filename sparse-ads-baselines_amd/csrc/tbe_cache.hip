@@ -265,7 +265,6 @@ void cache_layout(int64_t n, int64_t num_sets, tbe_cache_workspace_layout_t *l) 
   l->unique_slots = off; off += ints;
   l->lookup_slots = off; off += ints;
   l->evicted_keys = off; off += ints;
-  l->segment_ids = off; off += ints;
   l->miss_sets = off; off += ints;
   l->miss_list = off; off += ints;
   l->set_counts = off; off += sets;
@@ -361,8 +360,7 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
   TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(1), block, stats, static_cast<int64_t>(8), 0);
   if (num_indices == 0) return check_launch(name);
 
-  int rc = build_plan(l, workspace, table_offsets, T, indices, num_indices, offsets, B, total_rows,
-                      i32(cw, cl.segment_ids), s);
+  int rc = build_plan(l, workspace, table_offsets, T, indices, num_indices, offsets, B, total_rows, s);
   if (rc) return rc;
   const int32_t *keys_sorted = i32(ws, l.keys_sorted);
   const int32_t *segment_starts = i32(ws, l.segment_starts);
@@ -398,7 +396,7 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
              row_units, keys_sorted, segment_starts, counters, i32(cw, cl.unique_slots),
              i32(cw, cl.evicted_keys));
   TBE_LAUNCH("cache_locate", s, cache_locate_kernel, dim3(grid_for(num_indices, kBlockThreads, 256 * 16)), block,
-             i32(ws, l.positions_sorted), i32(cw, cl.segment_ids), i32(cw, cl.unique_slots), num_indices,
+             i32(ws, l.positions_sorted), i32(ws, l.segment_ids), i32(cw, cl.unique_slots), num_indices,
              i32(cw, cl.lookup_slots));
   e = hipEventRecord(filled, side);
   if (e == hipSuccess) e = hipStreamWaitEvent(s, filled, 0);

@@ -93,6 +93,22 @@ template <typename T, int VEC> struct RowVec {
   __device__ __forceinline__ static R load_raw(const T *p) {
     return *reinterpret_cast<const R *>(p);
   }
+  // Streaming variants: the data is touched once, so it should not displace reusable lines.
+  __device__ __forceinline__ static R load_raw_streaming(const T *p) {
+    using Words = uint32_t __attribute__((ext_vector_type(sizeof(R) / 4)));
+    const Words w = __builtin_nontemporal_load(reinterpret_cast<const Words *>(p));
+    R r;
+    __builtin_memcpy(&r, &w, sizeof(R));
+    return r;
+  }
+  __device__ __forceinline__ void load_streaming(const T *p) { unpack(load_raw_streaming(p)); }
+  __device__ __forceinline__ void store_streaming(T *p) const {
+    using Words = uint32_t __attribute__((ext_vector_type(sizeof(R) / 4)));
+    const R r = pack();
+    Words w;
+    __builtin_memcpy(&w, &r, sizeof(R));
+    __builtin_nontemporal_store(w, reinterpret_cast<Words *>(p));
+  }
   __device__ __forceinline__ void unpack(const R &r);
   __device__ __forceinline__ R pack() const;
   __device__ __forceinline__ void load(const T *p) { unpack(load_raw(p)); }

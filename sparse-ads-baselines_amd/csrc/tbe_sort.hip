@@ -6,8 +6,8 @@
 // The sort is the contract of cub::DeviceRadixSort::SortPairs as the reference
 // calls it (table_batched_embeddings_cuda.cu:1639-1655): ascending, stable,
 // key bits [0, end_bit).  Each pass is three kernels:
-//   histogram  per-tile digit counts (LDS atomics) -> counts[digit][tile], totals[digit]
-//   scan       one workgroup per digit turns counts into global start offsets
+//   histogram  per-tile digit counts (LDS atomics) -> counts[digit][tile]
+//   scan       one workgroup per digit: exclusive prefix over tiles, and the digit's total
 //   scatter    ranks each key inside its tile with wavefront ballots (all lanes
 //              holding the same digit are found with 8 ballots; the lowest lane
 //              reserves the run in a per-wavefront LDS counter), reorders the
@@ -84,14 +84,9 @@ __global__ __launch_bounds__(kBlockThreads) void linearize_kernel(
 }
 
 // ------------------------------------------------------------------ radix sort
-__global__ __launch_bounds__(kBlockThreads) void radix_zero_totals_kernel(uint32_t *totals, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) totals[i] = 0;
-}
-
 __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     const uint32_t *__restrict__ keys, int64_t n, int shift, uint32_t mask, int num_tiles,
-    uint32_t *__restrict__ counts, uint32_t *__restrict__ totals) {
+    uint32_t *__restrict__ counts) {
   __shared__ uint32_t s_hist[kBins];
   const int tid = threadIdx.x;
   s_hist[tid] = 0;
@@ -103,21 +98,18 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & mask], 1u);
   }
   __syncthreads();
-  const uint32_t c = s_hist[tid];
-  counts[static_cast<int64_t>(tid) * num_tiles + blockIdx.x] = c;
-  if (c) atomicAdd(&totals[tid], c);
+  counts[static_cast<int64_t>(tid) * num_tiles + blockIdx.x] = s_hist[tid];
 }
 
-// Workgroup `d` converts counts[d][0..num_tiles) into the global output offset of
-// digit d's keys in each tile: (keys with a smaller digit) + (same digit, earlier tile).
+// Workgroup `d` turns counts[d][0..num_tiles) into an exclusive prefix over tiles (keys with
+// digit d in earlier tiles) and publishes the row total; the scatter kernel adds the number
+// of keys with a smaller digit, which it gets from a scan of the 256 totals.
 __global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
-    uint32_t *__restrict__ counts, const uint32_t *__restrict__ totals, int num_tiles) {
+    uint32_t *__restrict__ counts, uint32_t *__restrict__ totals, int num_tiles) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   const int tid = threadIdx.x;
   const int d = blockIdx.x;
-  uint32_t carry;
-  (void)block_inclusive_scan(tid < d ? totals[tid] : 0u, s_wave, carry);
-  __syncthreads();
+  uint32_t carry = 0;
   uint32_t *row = counts + static_cast<int64_t>(d) * num_tiles;
   for (int c0 = 0; c0 < num_tiles; c0 += kBlockThreads) {
     const int i = c0 + tid;
@@ -128,12 +120,14 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
     carry += total;
     __syncthreads();
   }
+  if (tid == 0) totals[d] = carry;
 }
 
 __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ values_in,
     uint32_t *__restrict__ keys_out, uint32_t *__restrict__ values_out, int64_t n, int shift,
-    uint32_t mask, int num_tiles, const uint32_t *__restrict__ bases) {
+    uint32_t mask, int num_tiles, const uint32_t *__restrict__ bases,
+    const uint32_t *__restrict__ totals) {
   __shared__ uint32_t s_keys[kTile];
   __shared__ uint32_t s_vals[kTile];
   __shared__ uint32_t s_wave_count[kWavesPerBlock][kBins];
@@ -198,7 +192,10 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t incl = block_inclusive_scan(running, s_scan, total);
     const uint32_t bin_start = incl - running;
     s_bin_start[tid] = bin_start;
-    s_dest[tid] = bases[static_cast<int64_t>(tid) * num_tiles + blockIdx.x] - bin_start;
+    __syncthreads();
+    const uint32_t digit_total = totals[tid];
+    const uint32_t smaller = block_inclusive_scan(digit_total, s_scan, total) - digit_total;
+    s_dest[tid] = smaller + bases[static_cast<int64_t>(tid) * num_tiles + blockIdx.x] - bin_start;
   }
   __syncthreads();
 
@@ -326,8 +323,6 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   uint32_t *totals = reinterpret_cast<uint32_t *>(ws);
 
   const dim3 block(kBlockThreads);
-  TBE_LAUNCH("radix_zero", stream, radix_zero_totals_kernel, dim3(kMaxPasses), block, totals,
-             kMaxPasses * kBins);
   const uint32_t *src_k = reinterpret_cast<const uint32_t *>(keys_in);
   const uint32_t *src_v = reinterpret_cast<const uint32_t *>(values_in);
   for (int pass = 0; pass < passes; ++pass) {
@@ -339,11 +334,11 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
     uint32_t *dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
     uint32_t *pass_totals = totals + pass * kBins;
     TBE_LAUNCH("radix_histogram", stream, radix_histogram_kernel, dim3(tiles), block, src_k, n,
-               shift, mask, tiles, counts, pass_totals);
+               shift, mask, tiles, counts);
     TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, dim3(kBins), block, counts, pass_totals,
                tiles);
     TBE_LAUNCH("radix_scatter", stream, radix_scatter_kernel, dim3(tiles), block, src_k, src_v,
-               dst_k, dst_v, n, shift, mask, tiles, counts);
+               dst_k, dst_v, n, shift, mask, tiles, counts, pass_totals);
     src_k = dst_k;
     src_v = dst_v;
   }

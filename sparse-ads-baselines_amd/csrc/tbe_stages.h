@@ -20,9 +20,9 @@ uint64_t segments_workspace_bytes(int64_t n);
 int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts,
                   int32_t *num_unique, int32_t *segment_ids, void *workspace, hipStream_t stream);
 
-// Segments longer than kLongSegment occurrences are cut into chunks of
-// kChunkLen occurrences that are reduced by separate wavefronts.
-constexpr int kLongSegment = 256;
+// Segments of more than kShortSegment occurrences leave the lane-group path and are reduced by
+// whole wavefronts in chunks of at most kChunkLen occurrences.
+constexpr int kShortSegment = 16;
 constexpr int kChunkLen = 256;
 
 enum { kOptSgd = 0, kOptAdagrad = 1 };
@@ -37,10 +37,11 @@ struct UpdateArgs {
   const int32_t *positions_sorted;
   const int32_t *grad_rows;
   const int32_t *segment_starts;
-  int32_t *counters;            // [0] = U (input), [1] = #long segments, [2] = #chunks
-  int32_t *long_segments;       // [2][max_long]
-  int32_t *chunk_segments;      // [max_chunks]
-  void *partial_sums;           // acc [max_chunks][D]
+  int32_t *counters;            // [0] = U (input), [1] = #long records, [2] = #chunk records, [3] = #partial rows
+  const int32_t *segment_ids;   // [N] segment of every sorted position
+  void *long_segments;          // 16-byte records [max_long]: segments cut into several chunks
+  void *chunk_segments;         // 32-byte records [max_chunks]: the chunk queue
+  void *partial_sums;           // acc [max_partial][D]
   const int32_t *unique_slots;  // cache-fronted tables: slot of each unique row (-1 = not resident)
   void *cache_rows;             // cache-fronted tables: [slots][D] rows in HBM
   int64_t num_indices;
@@ -59,6 +60,6 @@ int key_bits_for(int64_t total_rows);
 void backward_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t *layout);
 int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int32_t *table_offsets,
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
-               int64_t total_rows, int32_t *segment_ids, hipStream_t stream);
+               int64_t total_rows, hipStream_t stream);
 
 }  // namespace tbe

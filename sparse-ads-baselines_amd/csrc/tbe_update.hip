@@ -11,16 +11,15 @@
 // (tbe.cu = table_batched_embeddings_cuda.cu.)  The reference gathers every
 // gradient row twice (tbe.cu:1548-1585); here G stays in registers.
 //
-// Work decomposition.  `chunks` lanes (one 16-byte vector each) own a row, a
-// wavefront holds 64/chunks such lane groups, each group takes one segment at a
-// time (grid-stride).  A group first loads the bookkeeping of up to `chunks`
-// occurrences with one coalesced load, then streams the gradient rows with
-// several loads in flight.  Segments longer than kLongSegment are not reduced
-// by one group: they are registered in a list, cut into chunks of kChunkLen
-// occurrences, each chunk is reduced by a whole wavefront into an fp32 partial
-// row, and a last kernel adds a segment's partials in chunk order and applies
-// the update.  Rows wider than 64 vectors take a multi-pass wavefront-per-
-// segment path.
+// Work decomposition.  `chunks` lanes (one 16-byte vector each) own a row and a
+// wavefront holds 64/chunks such lane groups.  Three classes of segment:
+//   short  (<= kShortSegment occurrences)  reduced serially by one lane group inside a
+//          position-balanced tile (update_short_kernel);
+//   medium (<= kChunkLen)  one wavefront, lane groups split the occurrences, update applied
+//          at once (update_chunks_kernel);
+//   long   cut into kChunkLen-occurrence chunks reduced by separate wavefronts into partial
+//          rows, added in chunk order and applied by update_long_finish_kernel.
+// Rows wider than 64 vectors take a multi-pass wavefront-per-segment path.
 
 #include <algorithm>
 
@@ -54,7 +53,7 @@ __device__ __forceinline__ T *resolve_row(T *weights, T *cache_rows,
 
 // Applies the optimizer to one row held by a lane group.  `w_old` and `G` are
 // this lane's vector of the row.
-template <typename T, int VEC, int CHUNKS, int OPT>
+template <typename T, int VEC, int CHUNKS, int OPT, bool STREAMING = false>
 __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_old,
                                              const RowVec<T, VEC> &G,
                                              typename AccOf<T>::type *state_row, float lr,
@@ -75,121 +74,192 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 #pragma unroll
     for (int i = 0; i < VEC; ++i) w_new.v[i] = w_old.v[i] - G.v[i] * mult;
   }
-  w_new.store(wrow);
+  if constexpr (STREAMING) w_new.store_streaming(wrow);
+  else w_new.store(wrow);
 }
 
 // ------------------------------------------------------------ short segments
+// Work is cut by sorted position, not by segment: a wavefront takes a tile of kTilePositions
+// consecutive sorted positions and owns every segment that STARTS inside it, so each tile costs
+// about the same however skewed the keys are.  The tile's bookkeeping is fetched 64 wide into
+// LDS (segment bounds, keys, and the gradient row of every occurrence; positions too when
+// weighted), after which the only global loads on a segment's critical path are rows.  Lane
+// group r walks segments r, r + groups, ...  Segments longer than kShortSegment are not
+// reduced here: the owning group appends chunk records (at most kChunkLen occurrences each)
+// to a queue that update_chunks_kernel drains with one wavefront per chunk.
+constexpr int kTilePositions = 64;
+constexpr int kStageCap = kTilePositions + 64;  // occurrences staged in LDS per wavefront
+
+struct ChunkRecord {   // 32 bytes
+  int32_t begin, end;  // sorted positions [begin, end)
+  int32_t key;         // row
+  int32_t u;           // index of the unique row (for the cache slot table)
+  int32_t partial;     // index of the partial row to write, -1 = the chunk is the whole segment
+  int32_t pad[3];
+};
+struct LongRecord {    // 16 bytes: a segment cut into several chunks
+  int32_t u, key, first_partial, num_chunks;
+};
+
 template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL>
 __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
     T *__restrict__ grad_psw, const int32_t *__restrict__ keys_sorted,
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
-    const int32_t *__restrict__ segment_starts, int32_t *__restrict__ counters,
-    int32_t *__restrict__ long_segments, int32_t *__restrict__ chunk_segments, int64_t max_long,
+    const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ segment_ids,
+    int32_t *__restrict__ counters, LongRecord *__restrict__ long_records,
+    ChunkRecord *__restrict__ chunk_records, int64_t n, int64_t num_tiles, int64_t tiles_per_xcd,
     int D, int chunks_rt, float lr, float eps, const int32_t *__restrict__ unique_slots,
     T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
 
+  __shared__ int32_t s_bounds[kWavesPerBlock][kTilePositions + 1];
+  __shared__ int32_t s_keys[kWavesPerBlock][kTilePositions];
+  __shared__ int32_t s_grow[kWavesPerBlock][kStageCap];
+  __shared__ int32_t s_pos[WEIGHTED ? kWavesPerBlock : 1][WEIGHTED ? kStageCap : 1];
+
   const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int64_t tile = xcd_contiguous(blockIdx.x, tiles_per_xcd) * kWavesPerBlock + wave;
+  if (tile >= num_tiles) return;
   const int chunks = CHUNKS > 0 ? CHUNKS : chunks_rt;
   const int groups = kWave / chunks;
   const int r = lane / chunks;
   const int c = lane - r * chunks;
   const int group_base = r * chunks;
-  const int U = counters[0];
-  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock * groups;
   const int64_t col = static_cast<int64_t>(c) * VEC;
 
-  for (int64_t u = (r < groups) ? wave_id * groups + r : U; u < U; u += stride) {
-    const int seg_begin = segment_starts[u];
-    const int seg_end = segment_starts[u + 1];
+  // Segments that start in [p0, p1): the segment containing p0 belongs to this tile only if
+  // p0 is its head.
+  const int64_t p0 = tile * kTilePositions;
+  const int64_t p1 = min(n, p0 + kTilePositions);
+  int u_first = segment_ids[p0];
+  if (segment_starts[u_first] != p0) ++u_first;
+  int u_limit;
+  if (p1 < n) {
+    u_limit = segment_ids[p1];
+    if (segment_starts[u_limit] != p1) ++u_limit;
+  } else {
+    u_limit = counters[0];
+  }
+  const int nseg = u_limit - u_first;  // <= kTilePositions
+  if (nseg <= 0) return;
+
+  for (int k = lane; k <= nseg; k += kWave) {
+    const int sb = segment_starts[u_first + k];
+    s_bounds[wave][k] = sb;
+    if (k < nseg) s_keys[wave][k] = keys_sorted[sb];
+  }
+  __builtin_amdgcn_wave_barrier();
+  const int tile_begin = s_bounds[wave][0];
+  const int staged = min(s_bounds[wave][nseg] - tile_begin, kStageCap);
+  for (int i = lane; i < staged; i += kWave) {
+    const int pos = positions_sorted[tile_begin + i];
+    s_grow[wave][i] = grad_rows[pos];
+    if constexpr (WEIGHTED) s_pos[wave][i] = pos;
+  }
+  __builtin_amdgcn_wave_barrier();
+
+  for (int j = (r < groups) ? r : nseg; j < nseg; j += groups) {
+    const int u = u_first + j;
+    const int seg_begin = s_bounds[wave][j];
+    const int seg_end = s_bounds[wave][j + 1];
     const int len = seg_end - seg_begin;
-    if (len > kLongSegment) {
-      // Register the segment for the chunked path.
+    const int32_t key = s_keys[wave][j];
+    if (len > kShortSegment) {
+      // Hand the segment to the chunk queue.
       const int nch = (len + kChunkLen - 1) / kChunkLen;
-      int slot = 0, first_chunk = 0;
+      int first_chunk = 0, first_partial = -1;
       if (c == 0) {
-        slot = atomicAdd(&counters[1], 1);
         first_chunk = atomicAdd(&counters[2], nch);
-        long_segments[slot] = static_cast<int32_t>(u);
-        long_segments[max_long + slot] = first_chunk;
+        if (nch > 1) {
+          first_partial = atomicAdd(&counters[3], nch);
+          long_records[atomicAdd(&counters[1], 1)] = LongRecord{u, key, first_partial, nch};
+        }
       }
-      slot = shfl_idx(slot, group_base);
       first_chunk = shfl_idx(first_chunk, group_base);
-      for (int k = c; k < nch; k += chunks) chunk_segments[first_chunk + k] = slot;
+      first_partial = shfl_idx(first_partial, group_base);
+      for (int k = c; k < nch; k += chunks) {
+        ChunkRecord rec;
+        rec.begin = seg_begin + k * kChunkLen;
+        rec.end = min(seg_end, rec.begin + kChunkLen);
+        rec.key = key;
+        rec.u = u;
+        rec.partial = nch > 1 ? first_partial + k : -1;
+        rec.pad[0] = rec.pad[1] = rec.pad[2] = 0;
+        chunk_records[first_chunk + k] = rec;
+      }
       continue;
     }
-    const int64_t row = keys_sorted[seg_begin];
-    T *wrow = resolve_row(weights, cache_rows, unique_slots, u, row, D) + col;
+    T *wrow = resolve_row(weights, cache_rows, unique_slots, u, static_cast<int64_t>(key), D) + col;
     V w_old;
-    w_old.load(wrow);
+    w_old.load_streaming(wrow);  // each row is touched once per step: keep L2 for gradient rows
     V G;
     G.zero();
-    for (int base = seg_begin; base < seg_end; base += chunks) {
-      const int n = min(chunks, seg_end - base);
-      int my_pos = 0, my_grow = 0;
-      A my_w = A(0);
-      if (c < n) {
-        my_pos = positions_sorted[base + c];
-        my_grow = grad_rows[my_pos];
-        if constexpr (WEIGHTED) my_w = to_acc(psw[my_pos]);
-      }
-      for (int j0 = 0; j0 < n; j0 += UNROLL) {
-        R raw[UNROLL];
+    for (int i0 = seg_begin; i0 < seg_end; i0 += UNROLL) {
+      R raw[UNROLL];
+      int pos[UNROLL];
+      A pw[UNROLL];
 #pragma unroll
-        for (int q = 0; q < UNROLL; ++q) {
-          const int j = j0 + q;
-          const int src = group_base + (j < n ? j : 0);
-          const int64_t grow = shfl_idx(my_grow, src);
-          if (j < n) raw[q] = V::load_raw(grad_output + grow * D + col);
+      for (int q = 0; q < UNROLL; ++q) {
+        const int i = i0 + q;
+        if (i < seg_end) {
+          const int rel = i - tile_begin;
+          int64_t grow;
+          if (rel < kStageCap) {
+            grow = s_grow[wave][rel];
+            if constexpr (WEIGHTED) pos[q] = s_pos[wave][rel];
+          } else {
+            const int p = positions_sorted[i];
+            grow = grad_rows[p];
+            if constexpr (WEIGHTED) pos[q] = p;
+          }
+          raw[q] = V::load_raw(grad_output + grow * D + col);
+          if constexpr (WEIGHTED) pw[q] = to_acc(psw[pos[q]]);
         }
+      }
 #pragma unroll
-        for (int q = 0; q < UNROLL; ++q) {
-          const int j = j0 + q;
-          if (j < n) {
-            V x;
-            x.unpack(raw[q]);
-            if constexpr (WEIGHTED) {
-              const int src = group_base + j;
-              const A pw = shfl_idx(my_w, src);
-              const int pos = shfl_idx(my_pos, src);
-              A dot = A(0);
+      for (int q = 0; q < UNROLL; ++q) {
+        if (i0 + q < seg_end) {
+          V x;
+          x.unpack(raw[q]);
+          if constexpr (WEIGHTED) {
+            A dot = A(0);
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
-              dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
-              if (c == 0) grad_psw[pos] = from_acc<T, A>(dot);
+            for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
+            dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
+            if (c == 0) grad_psw[pos[q]] = from_acc<T, A>(dot);
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * pw;
-            } else {
+            for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * pw[q];
+          } else {
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i];
-            }
+            for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i];
           }
         }
       }
     }
-    apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + row : nullptr, lr, eps,
-                                      chunks, group_base, c);
+    apply_update<T, VEC, CHUNKS, OPT, true>(wrow, w_old, G, state ? state + key : nullptr, lr, eps,
+                                            chunks, group_base, c);
   }
 }
 
-// ------------------------------------------------- long segments: chunk sums
-// One wavefront per chunk of at most kChunkLen occurrences.  Lane group r adds
-// occurrences r, r+groups, ... of the chunk; the groups are then combined in a
-// fixed tree and group 0 stores the partial row.
-template <typename T, int VEC, int CHUNKS, bool WEIGHTED, int UNROLL>
-__global__ __launch_bounds__(kBlockThreads) void update_long_partial_kernel(
-    const T *__restrict__ grad_output, const T *__restrict__ weights, const T *__restrict__ psw,
-    T *__restrict__ grad_psw, const int32_t *__restrict__ keys_sorted,
-    const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
-    const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
-    const int32_t *__restrict__ long_segments, const int32_t *__restrict__ chunk_segments,
-    typename AccOf<T>::type *__restrict__ partial_sums, int64_t max_long, int D, int chunks_rt,
-    const int32_t *__restrict__ unique_slots, const T *__restrict__ cache_rows) {
+// ------------------------------------------------ medium / long segments: chunks
+// One wavefront per chunk record (grid-stride over the queue).  Lane group r adds
+// occurrences r, r + groups, ... of the chunk; the groups are combined in a fixed tree.
+// A chunk that is a whole segment is applied to its row at once; a chunk of a longer
+// segment stores its sum as a partial row for update_long_finish_kernel.
+template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL>
+__global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
+    const T *__restrict__ grad_output, T *__restrict__ weights,
+    typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
+    T *__restrict__ grad_psw, const int32_t *__restrict__ positions_sorted,
+    const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ counters,
+    const ChunkRecord *__restrict__ chunk_records,
+    typename AccOf<T>::type *__restrict__ partial_sums, int D, int chunks_rt, float lr, float eps,
+    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -207,24 +277,15 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_partial_kernel(
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
 
   for (int64_t q = wave_id; q < num_chunks; q += stride) {
-    const int slot = chunk_segments[q];
-    const int u = long_segments[slot];
-    const int first_chunk = long_segments[max_long + slot];
-    const int seg_begin = segment_starts[u];
-    const int seg_end = segment_starts[u + 1];
-    const int begin = seg_begin + static_cast<int>(q - first_chunk) * kChunkLen;
-    const int end = min(seg_end, begin + kChunkLen);
+    const ChunkRecord rec = chunk_records[q];
+    T *wrow = resolve_row(weights, cache_rows, unique_slots, rec.u, static_cast<int64_t>(rec.key), D) + col;
     V w_old;
     w_old.zero();
-    if constexpr (WEIGHTED) {
-      const int64_t row = keys_sorted[seg_begin];
-      if (active)
-        w_old.load(resolve_row<const T>(weights, cache_rows, unique_slots, u, row, D) + col);
-    }
+    if (active && (WEIGHTED || rec.partial < 0)) w_old.load(wrow);
     V G;
     G.zero();
-    for (int base = begin; base < end; base += kWave) {
-      const int n = min(kWave, end - base);
+    for (int base = rec.begin; base < rec.end; base += kWave) {
+      const int n = min(kWave, rec.end - base);
       int my_pos = 0, my_grow = 0;
       A my_w = A(0);
       if (lane < n) {
@@ -292,9 +353,14 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_partial_kernel(
       }
     }
     if (r == 0) {
-      A *dst = partial_sums + q * D + col;
+      if (rec.partial >= 0) {
+        A *dst = partial_sums + static_cast<int64_t>(rec.partial) * D + col;
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) dst[i] = G.v[i];
+        for (int i = 0; i < VEC; ++i) dst[i] = G.v[i];
+      } else {
+        apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, lr,
+                                          eps, chunks, 0, c);
+      }
     }
   }
 }
@@ -303,11 +369,9 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_partial_kernel(
 template <typename T, int VEC, int CHUNKS, int OPT>
 __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     T *__restrict__ weights, typename AccOf<T>::type *__restrict__ state,
-    const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
-    const int32_t *__restrict__ counters, const int32_t *__restrict__ long_segments,
-    const typename AccOf<T>::type *__restrict__ partial_sums, int64_t max_long, int D,
-    int chunks_rt, float lr, float eps, const int32_t *__restrict__ unique_slots,
-    T *__restrict__ cache_rows) {
+    const int32_t *__restrict__ counters, const LongRecord *__restrict__ long_records,
+    const typename AccOf<T>::type *__restrict__ partial_sums, int D, int chunks_rt, float lr,
+    float eps, const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
 
@@ -324,23 +388,18 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
 
   for (int64_t slot = (r < groups) ? wave_id * groups + r : num_long; slot < num_long;
        slot += stride) {
-    const int u = long_segments[slot];
-    const int first_chunk = long_segments[max_long + slot];
-    const int seg_begin = segment_starts[u];
-    const int len = segment_starts[u + 1] - seg_begin;
-    const int nch = (len + kChunkLen - 1) / kChunkLen;
-    const int64_t row = keys_sorted[seg_begin];
-    T *wrow = resolve_row(weights, cache_rows, unique_slots, u, row, D) + col;
+    const LongRecord rec = long_records[slot];
+    T *wrow = resolve_row(weights, cache_rows, unique_slots, rec.u, static_cast<int64_t>(rec.key), D) + col;
     V w_old;
     w_old.load(wrow);
     V G;
     G.zero();
-    for (int k = 0; k < nch; ++k) {
-      const A *src = partial_sums + static_cast<int64_t>(first_chunk + k) * D + col;
+    for (int k = 0; k < rec.num_chunks; ++k) {
+      const A *src = partial_sums + static_cast<int64_t>(rec.first_partial + k) * D + col;
 #pragma unroll
       for (int i = 0; i < VEC; ++i) G.v[i] += src[i];
     }
-    apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + row : nullptr, lr, eps,
+    apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, lr, eps,
                                       chunks, group_base, c);
   }
 }
@@ -436,7 +495,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_wide_kernel(
 }
 
 __global__ void zero_counters_kernel(int32_t *counters) {
-  if (threadIdx.x == 1 || threadIdx.x == 2) counters[threadIdx.x] = 0;
+  if (threadIdx.x >= 1 && threadIdx.x <= 3) counters[threadIdx.x] = 0;
 }
 
 constexpr int kShortUnroll = 4;
@@ -452,33 +511,33 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   T *gpsw = static_cast<T *>(a.grad_per_sample_weights);
   A *partial = static_cast<A *>(a.partial_sums);
   T *cr = static_cast<T *>(a.cache_rows);
+  LongRecord *long_records = reinterpret_cast<LongRecord *>(a.long_segments);
+  ChunkRecord *chunk_records = reinterpret_cast<ChunkRecord *>(a.chunk_segments);
   const int groups = kWave / g.chunks;
   const dim3 block(kBlockThreads);
 
-  // Enough wavefronts to cover the worst case U == N once, capped so that the
-  // grid-stride loop amortises launch cost on large inputs.
-  const int64_t want = ceil_div(ceil_div(a.num_indices, groups), kWavesPerBlock);
-  const dim3 grid_short(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want, 256 * 32))));
+  const int64_t num_tiles = ceil_div(a.num_indices, kTilePositions);
+  const int64_t tiles_per_xcd = ceil_div(ceil_div(num_tiles, kWavesPerBlock), kNumXcd);
+  const dim3 grid_short(static_cast<unsigned>(tiles_per_xcd * kNumXcd));
   TBE_LAUNCH("update_short", stream,
              (update_short_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kShortUnroll>), grid_short, block,
              go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
-             a.segment_starts, a.counters, a.long_segments, a.chunk_segments, a.max_long, a.D,
-             g.chunks, a.learning_rate, a.eps, a.unique_slots, cr);
+             a.segment_starts, a.segment_ids, a.counters, long_records, chunk_records,
+             a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,
+             a.unique_slots, cr);
 
   const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
-  const dim3 grid_partial(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_chunks, 256 * 8))));
-  TBE_LAUNCH("update_long_partial", stream,
-             (update_long_partial_kernel<T, VEC, CHUNKS, WEIGHTED, kLongUnroll>), grid_partial,
-             block, go, w, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
-             a.segment_starts, a.counters, a.long_segments, a.chunk_segments, partial, a.max_long,
-             a.D, g.chunks, a.unique_slots, cr);
+  const dim3 grid_chunks(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_chunks, 256 * 8))));
+  TBE_LAUNCH("update_chunks", stream,
+             (update_chunks_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kLongUnroll>), grid_chunks, block,
+             go, w, st, psw, gpsw, a.positions_sorted, a.grad_rows, a.counters, chunk_records,
+             partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr);
 
   const int64_t want_long = ceil_div(ceil_div(a.max_long, groups), kWavesPerBlock);
   const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
   TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, OPT>),
-             grid_finish, block, w, st, a.keys_sorted, a.segment_starts, a.counters,
-             a.long_segments, partial, a.max_long, a.D, g.chunks, a.learning_rate, a.eps,
-             a.unique_slots, cr);
+             grid_finish, block, w, st, a.counters, long_records, partial, a.D, g.chunks,
+             a.learning_rate, a.eps, a.unique_slots, cr);
 }
 
 template <typename T, int VEC, int OPT, bool WEIGHTED>

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -33,11 +33,13 @@ class WorkspaceLayout(ctypes.Structure):
         ("num_unique", _u64),
         ("sort_scratch", _u64),
         ("segment_scratch", _u64),
+        ("segment_ids", _u64),
         ("long_segments", _u64),
         ("chunk_segments", _u64),
         ("partial_sums", _u64),
         ("max_long_segments", _i64),
         ("max_chunks", _i64),
+        ("max_partial_rows", _i64),
     ]
 
 
@@ -59,7 +61,7 @@ class CacheWorkspaceLayout(ctypes.Structure):
     """Mirror of tbe_cache_workspace_layout_t."""
 
     _fields_ = [(name, _u64) for name in (
-        "total_bytes", "unique_slots", "lookup_slots", "evicted_keys", "segment_ids", "miss_sets", "miss_list",
+        "total_bytes", "unique_slots", "lookup_slots", "evicted_keys", "miss_sets", "miss_list",
         "set_counts", "set_fill", "set_starts", "stats")]
 
 

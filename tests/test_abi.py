@@ -43,11 +43,13 @@ def test_abi_version_matches_binding():
 def test_workspace_layout_is_ordered_and_sized():
     lay = tbe_native.backward_workspace_layout(5242880, 128, tbe_native.DTYPE_F32)
     offs = [lay.keys, lay.grad_rows, lay.keys_sorted, lay.positions_sorted, lay.segment_starts, lay.num_unique,
-            lay.sort_scratch, lay.segment_scratch, lay.long_segments, lay.chunk_segments, lay.partial_sums]
+            lay.sort_scratch, lay.segment_scratch, lay.segment_ids, lay.long_segments, lay.chunk_segments,
+            lay.partial_sums]
     assert offs == sorted(offs) and len(set(offs)) == len(offs)
     assert all(o % 256 == 0 for o in offs)
     assert lay.grad_rows - lay.keys >= 5242880 * 4
-    assert lay.total_bytes >= lay.partial_sums + lay.max_chunks * 128 * 4
+    assert lay.total_bytes >= lay.partial_sums + lay.max_partial_rows * 128 * 4
+    assert lay.partial_sums - lay.chunk_segments >= lay.max_chunks * 32
     assert lay.total_bytes < 512 << 20
     half = tbe_native.backward_workspace_layout(1000, 64, tbe_native.DTYPE_F16)
     dbl = tbe_native.backward_workspace_layout(1000, 64, tbe_native.DTYPE_F64)
