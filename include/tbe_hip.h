@@ -37,6 +37,9 @@ extern "C" {
 /* element type of weights / outputs / gradients / per-sample weights */
 enum { TBE_DTYPE_F32 = 0, TBE_DTYPE_F16 = 1, TBE_DTYPE_F64 = 2 };
 
+/* optimizer selector of the entry points that serve several optimizers */
+enum { TBE_OPT_SGD = 0, TBE_OPT_ROWWISE_ADAGRAD = 1 };
+
 enum {
   TBE_OK = 0,
   TBE_ERR_INVALID = 1,     /* a shape / pointer / dtype precondition failed */
@@ -188,6 +191,39 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
                           const int32_t *total_indices_per_table,
                           int32_t T, int32_t B, int32_t *output, void *stream);
 
+/* ---------------------------------------------- per-table embedding dimension
+ * The reference's MixedDim path (table_batched_embeddings_ops.py:204-435):
+ *   weights            1-D; table t occupies elements [table_offsets[t], table_offsets[t+1]),
+ *                      row-major [rows_t][D_t]                         int64 [T+1]
+ *   table_dim_offsets  first global row id of each table (cumulative ROW counts) int32 [T+1]
+ *   dim_offsets        first output column of each table, D_t % 4 == 0  int32 [T+1]
+ *   output / grad      [B][total_D]
+ * `fp16_vector_width` is 8 when every D_t of an fp16 table set is a multiple of 8, else 4
+ * (ignored for other dtypes).
+ * tbe_forward_mixed replaces batched_embedding_forward_mixed_D_cuda
+ * (table_batched_embeddings_cuda.cu:945-1004, "forward_mixed_D" in table_batched_embeddings.cpp:66);
+ * tbe_backward_mixed replaces batched_embedding_backward_adagrad_exact_mixed_D_cuda
+ * (:1350-1469, "backward_exact_adagrad_mixed_D", .cpp:64), serves the approximate variant
+ * (.cpp:63) and adds exact SGD; per-sample weights as in tbe_backward_exact_adagrad.  The
+ * workspace is a backward workspace sized with tbe_backward_workspace_layout(N, 4, dtype).
+ */
+TBE_API int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp16_vector_width,
+                              const int64_t *table_offsets, const int32_t *dim_offsets,
+                              int32_t total_D, int32_t T,
+                              const int32_t *indices, int64_t num_indices,
+                              const int32_t *offsets, int32_t B,
+                              const void *per_sample_weights, void *output, void *stream);
+
+TBE_API int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void *weights, int32_t dtype,
+                               int32_t fp16_vector_width, int64_t total_rows,
+                               const int64_t *table_offsets, const int32_t *table_dim_offsets,
+                               const int32_t *dim_offsets, int32_t total_D, int32_t T,
+                               const int32_t *indices, int64_t num_indices,
+                               const int32_t *offsets, int32_t B,
+                               const void *per_sample_weights, void *optimizer_state,
+                               float learning_rate, float eps, void *grad_per_sample_weights,
+                               void *workspace, uint64_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------- row cache
  * An HBM-resident set-associative row cache in front of a host-resident table
  * (pinned, device-mapped memory from tbe_host_mapped_alloc).  The reference has
@@ -220,7 +256,6 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
  */
 #define TBE_CACHE_WAYS 64
 enum { TBE_CACHE_LRU = 0, TBE_CACHE_LFU = 1 };
-enum { TBE_OPT_SGD = 0, TBE_OPT_ROWWISE_ADAGRAD = 1 };
 
 typedef struct tbe_cache {
   int32_t *tags;        /* [num_sets * 64] key of the row held by each slot, -1 = empty  */

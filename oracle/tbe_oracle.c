@@ -337,3 +337,128 @@ void oracle_construct_offsets(const int32_t *batch_offsets_per_table,
     output[1 + t * B + b] = upper - batch_offsets_per_table[t * B + b];
   }
 }
+
+/* ======================================================= per-table dimension
+ * Mixed-D layout of table_batched_embeddings_ops.py:324-379: weights 1-D with int64
+ * element offsets table_offsets[T+1], global row ids from table_dim_offsets[T+1]
+ * (cumulative row counts), output columns from dim_offsets[T+1], output [B][total_D].
+ */
+
+/* batched_embedding_forward_kernel_mixed_D_1 (tbe.cu:882-943) */
+void oracle_forward_mixed(const void *weights, int dtype, const int64_t *table_offsets,
+                          const int32_t *dim_offsets, int32_t total_D, int32_t T,
+                          const int32_t *indices, const int32_t *offsets, int32_t B,
+                          const void *psw, void *output) {
+  for (int32_t b_t = 0; b_t < T * B; ++b_t) {
+    const int32_t t = b_t / B, b = b_t % B;
+    const int32_t dim_start = dim_offsets[t], D = dim_offsets[t + 1] - dim_start;
+    const int64_t table_offset = table_offsets[t];
+    const int32_t start = offsets[t * B + b], end = offsets[t * B + b + 1];
+    const int64_t out0 = (int64_t)b * total_D + dim_start;
+    for (int32_t d = 0; d < D; ++d) {
+      if (dtype == F64) {
+        double sum = 0;
+        for (int32_t l = start; l < end; ++l) {
+          const double w = ((const double *)weights)[table_offset + (int64_t)indices[l] * D + d];
+          if (psw) sum += w * ((const double *)psw)[l];
+          else sum += w;
+        }
+        ((double *)output)[out0 + d] = sum;
+      } else {
+        float sum = 0;
+        for (int32_t l = start; l < end; ++l) {
+          const float w = load_f(weights, dtype, table_offset + (int64_t)indices[l] * D + d);
+          if (psw) sum += w * load_f(psw, dtype, l);
+          else sum += w;
+        }
+        store_f(output, dtype, out0 + d, sum);
+      }
+    }
+  }
+}
+
+/* linear_index_weight_offsets_mixed_D_kernel (tbe.cu:1220-1247), the sort (tbe.cu:1400-1416)
+ * and batched_embedding_backward_adagrad_exact_kernel_mixed_D_1 (tbe.cu:1249-1348); optimizer
+ * and weighting as in oracle_backward. */
+int oracle_backward_mixed(int optimizer, const void *grad_output, void *weights, int dtype,
+                          int64_t total_rows, const int64_t *table_offsets,
+                          const int32_t *table_dim_offsets, const int32_t *dim_offsets,
+                          int32_t total_D, int32_t T, const int32_t *indices, int64_t n,
+                          const int32_t *offsets, int32_t B, const void *psw,
+                          void *optimizer_state, float lr, float eps, void *grad_psw) {
+  const size_t nn = (size_t)(n > 0 ? n : 1);
+  int32_t *keys = (int32_t *)malloc(nn * 4), *b_ts = (int32_t *)malloc(nn * 4);
+  int32_t *pos = (int32_t *)malloc(nn * 4), *keys_s = (int32_t *)malloc(nn * 4);
+  int32_t *pos_s = (int32_t *)malloc(nn * 4), *seg = (int32_t *)malloc((nn + 1) * 4);
+  oracle_linearize(table_dim_offsets, T, indices, offsets, B, keys, b_ts, pos);
+  oracle_sort_pairs(keys, pos, keys_s, pos_s, n, (int)(log2((double)total_rows) + 1));
+  const int64_t U = oracle_segments(keys_s, n, seg);
+  double *G = (double *)malloc((size_t)total_D * 8);
+  for (int64_t u = 0; u < U; ++u) {
+    const int32_t s0 = seg[u], s1 = seg[u + 1];
+    const int32_t t = b_ts[pos_s[s0]] / B;
+    const int32_t dim_start = dim_offsets[t], D = dim_offsets[t + 1] - dim_start;
+    const int64_t row = keys_s[s0];
+    const int64_t w0 = table_offsets[t] + (row - table_dim_offsets[t]) * D;
+    for (int32_t d = 0; d < D; ++d) G[d] = 0;
+    for (int32_t i = s0; i < s1; ++i) {
+      const int32_t p = pos_s[i], b = b_ts[p] % B;
+      const int64_t g0 = (int64_t)b * total_D + dim_start;
+      if (dtype == F64) {
+        const double *g = (const double *)grad_output + g0;
+        const double *w = (const double *)weights + w0;
+        double pw = 1;
+        if (psw) {
+          double dot = 0;
+          for (int32_t d = 0; d < D; ++d) dot += w[d] * g[d];
+          ((double *)grad_psw)[p] = dot;
+          pw = ((const double *)psw)[p];
+        }
+        for (int32_t d = 0; d < D; ++d) G[d] += psw ? g[d] * pw : g[d];
+      } else {
+        float pw = 1;
+        if (psw) {
+          float dot = 0;
+          for (int32_t d = 0; d < D; ++d) dot += load_f(weights, dtype, w0 + d) * load_f(grad_output, dtype, g0 + d);
+          store_f(grad_psw, dtype, p, dot);
+          pw = load_f(psw, dtype, p);
+        }
+        for (int32_t d = 0; d < D; ++d) {
+          const float g = load_f(grad_output, dtype, g0 + d);
+          G[d] = (double)((float)G[d] + (psw ? g * pw : g));
+        }
+      }
+    }
+    if (dtype == F64) {
+      double mult = lr;
+      if (optimizer == 1) {
+        double gss = 0;
+        for (int32_t d = 0; d < D; ++d) gss += G[d] * G[d];
+        double *st = (double *)optimizer_state + row;
+        const double old = *st;
+        *st = old + gss;
+        mult = lr * (1.0 / (sqrt(old + gss) + eps));
+      }
+      double *w = (double *)weights + w0;
+      for (int32_t d = 0; d < D; ++d) w[d] -= G[d] * mult;
+    } else {
+      float mult = lr;
+      if (optimizer == 1) {
+        float gss = 0;
+        for (int32_t d = 0; d < D; ++d) gss += (float)G[d] * (float)G[d];
+        float *st = (float *)optimizer_state + row;
+        const float old = *st;
+        *st = old + gss;
+        mult = (float)(lr * (1.0 / (sqrtf(old + gss) + eps)));
+      }
+      for (int32_t d = 0; d < D; ++d) {
+        float w = load_f(weights, dtype, w0 + d);
+        w -= (float)G[d] * mult;
+        store_f(weights, dtype, w0 + d, w);
+      }
+    }
+  }
+  free(G);
+  free(keys); free(b_ts); free(pos); free(keys_s); free(pos_s); free(seg);
+  return 0;
+}

@@ -172,3 +172,47 @@ def cache_set_of(key, num_sets):
     fn = lib().lxu_set_of
     fn.restype = ctypes.c_uint32
     return fn(ctypes.c_uint32(int(key)), ctypes.c_uint32(int(num_sets)))
+
+
+# ------------------------------------------------------------ per-table dimension
+def forward_mixed(weights, table_offsets, dim_offsets, indices, offsets, per_sample_weights=None):
+    """weights 1-D; table_offsets int64 [T+1]; dim_offsets int32 [T+1] -> output [B, total_D]."""
+    weights = np.ascontiguousarray(weights)
+    code = _CODES[weights.dtype]
+    table_offsets = np.ascontiguousarray(table_offsets, dtype=np.int64)
+    dim_offsets, indices, offsets = _i32(dim_offsets), _i32(indices), _i32(offsets)
+    T = table_offsets.size - 1
+    B = (offsets.size - 1) // T
+    total_D = int(dim_offsets[-1])
+    psw = None if per_sample_weights is None else np.ascontiguousarray(per_sample_weights, dtype=weights.dtype)
+    out = np.empty((B, total_D), dtype=weights.dtype)
+    lib().oracle_forward_mixed(_p(weights), ctypes.c_int(code), _p(table_offsets), _p(dim_offsets),
+                               ctypes.c_int32(total_D), ctypes.c_int32(T), _p(indices), _p(offsets),
+                               ctypes.c_int32(B), _p(psw), _p(out))
+    return out
+
+
+def backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, indices, offsets,
+                   lr, eps=0.0, optimizer_state=None, per_sample_weights=None):
+    """In-place on `weights` (1-D) and `optimizer_state`; returns grad_psw or None."""
+    assert weights.flags["C_CONTIGUOUS"] and weights.ndim == 1
+    code = _CODES[weights.dtype]
+    grad_output = np.ascontiguousarray(grad_output, dtype=weights.dtype)
+    table_offsets = np.ascontiguousarray(table_offsets, dtype=np.int64)
+    table_dim_offsets, dim_offsets = _i32(table_dim_offsets), _i32(dim_offsets)
+    indices, offsets = _i32(indices), _i32(offsets)
+    T = table_offsets.size - 1
+    B = (offsets.size - 1) // T
+    total_D = int(dim_offsets[-1])
+    assert grad_output.shape == (B, total_D)
+    psw = gpsw = None
+    if per_sample_weights is not None:
+        psw = np.ascontiguousarray(per_sample_weights, dtype=weights.dtype)
+        gpsw = np.zeros(indices.size, dtype=weights.dtype)
+    opt = {"sgd": 0, "adagrad": 1}[optimizer]
+    lib().oracle_backward_mixed(ctypes.c_int(opt), _p(grad_output), _p(weights), ctypes.c_int(code),
+                                ctypes.c_int64(int(table_dim_offsets[-1])), _p(table_offsets), _p(table_dim_offsets),
+                                _p(dim_offsets), ctypes.c_int32(total_D), ctypes.c_int32(T), _p(indices),
+                                ctypes.c_int64(indices.size), _p(offsets), ctypes.c_int32(B), _p(psw),
+                                _p(optimizer_state), ctypes.c_float(lr), ctypes.c_float(eps), _p(gpsw))
+    return gpsw

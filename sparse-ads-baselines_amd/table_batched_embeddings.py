@@ -158,13 +158,118 @@ def backward_approx_adagrad(grad_output, weights, table_offsets, indices, offset
                                   optimizer_state, learning_rate, eps, stochastic_rounding, BT_block_size)
 
 
-def _mixed_d_unavailable(*args, **kwargs):
-    raise NotImplementedError("mixed-dimension tables are not served by this library")
+def _check_mixed(weights, table_offsets, dim_offsets, indices, offsets):
+    _require(weights.is_cuda and weights.dim() == 1 and weights.is_contiguous(),
+             "weights must be a contiguous 1-D GPU tensor")
+    _require(weights.dtype in _DTYPE_CODES, "weights must be float16, float32 or float64")
+    _require(table_offsets.dtype == torch.int64, "table_offsets must be int64 (got %s)" % table_offsets.dtype)
+    for name, t in (("dim_offsets", dim_offsets), ("indices", indices), ("offsets", offsets)):
+        _require(t.dtype == torch.int32, "%s must be int32 (got %s)" % (name, t.dtype))
+    for name, t in (("table_offsets", table_offsets), ("dim_offsets", dim_offsets), ("indices", indices),
+                    ("offsets", offsets)):
+        _require(t.is_cuda and t.device == weights.device, "%s must live on the weights' device" % name)
+        _require(t.dim() == 1 and t.is_contiguous(), "%s must be a contiguous 1-D tensor" % name)
+    T = table_offsets.numel() - 1  # table_batched_embeddings_cuda.cu:952
+    _require(T > 0, "T must be positive")
+    _require(dim_offsets.numel() == T + 1, "dim_offsets must hold T+1 entries")
+    B = (offsets.numel() - 1) // T
+    _require(B > 0, "B must be positive")
+    _require(offsets.numel() == T * B + 1, "offsets must hold T*B+1 entries")
+    return T, B
 
 
-forward_mixed_D = _mixed_d_unavailable
-backward_approx_adagrad_mixed_D = _mixed_d_unavailable
-backward_exact_adagrad_mixed_D = _mixed_d_unavailable
+# fp16 rows are moved 16 bytes at a time when every table's D allows it, else 8 bytes.  The choice
+# needs the per-table dims on the host; it is cached per dim_offsets tensor.
+_fp16_width = {}
+
+
+def _fp16_vector_width(dim_offsets):
+    key = (dim_offsets.data_ptr(), dim_offsets.numel())
+    if key not in _fp16_width:
+        dims = torch.diff(dim_offsets).cpu()
+        _require(bool((dims % 4 == 0).all()) and bool((dims > 0).all()), "every D_t must be a positive multiple of 4")
+        _fp16_width[key] = 8 if bool((dims % 8 == 0).all()) else 4
+    return _fp16_width[key]
+
+
+def forward_mixed_D(weights, table_offsets, dim_offsets, total_D, indices, offsets, indice_weights, L_max,
+                    BT_block_size, shmem):
+    """batched_embedding_forward_mixed_D_cuda (table_batched_embeddings_cuda.cu:945-1004):
+    output [B, total_D], table t in columns dim_offsets[t]:dim_offsets[t+1]."""
+    T, B = _check_mixed(weights, table_offsets, dim_offsets, indices, offsets)
+    _require(BT_block_size != 0, "BT_block_size must be non-zero")
+    if indice_weights is not None:
+        _require(indice_weights.dtype == weights.dtype and indice_weights.is_contiguous()
+                 and indice_weights.numel() == indices.numel(),
+                 "indice_weights must be contiguous, of the weights' dtype, with one entry per index")
+    output = torch.empty((B, int(total_D)), dtype=weights.dtype, device=weights.device)
+    with torch.cuda.device(weights.device):
+        _native.check(_native.load().tbe_forward_mixed(
+            _ptr(weights), _DTYPE_CODES[weights.dtype], _fp16_vector_width(dim_offsets), _ptr(table_offsets),
+            _ptr(dim_offsets), int(total_D), T, _ptr(indices), indices.numel(), _ptr(offsets), B,
+            _ptr(indice_weights), _ptr(output), _stream(weights.device)))
+    return output
+
+
+def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, total_D, indices,
+                    offsets, indice_weights, optimizer_state, learning_rate, eps, stochastic_rounding):
+    T, B = _check_mixed(weights, table_offsets, dim_offsets, indices, offsets)
+    if stochastic_rounding:
+        raise NotImplementedError("stochastic rounding is not implemented")
+    _require(table_dim_offsets.dtype == torch.int32 and table_dim_offsets.numel() == T + 1,
+             "table_dim_offsets must be int32 with T+1 entries")
+    _require(grad_output.dtype == weights.dtype and tuple(grad_output.shape) == (B, int(total_D)),
+             "grad_output must be [B, total_D] of the weights' dtype")
+    grad_output = grad_output.contiguous()
+    code = _DTYPE_CODES[weights.dtype]
+    total_rows = optimizer_state.numel()  # table_batched_embeddings_cuda.cu:1404
+    grad_indice_weights = None
+    if indice_weights is not None:
+        _require(indice_weights.dtype == weights.dtype and indice_weights.is_contiguous()
+                 and indice_weights.numel() == indices.numel(),
+                 "indice_weights must be contiguous, of the weights' dtype, with one entry per index")
+        grad_indice_weights = torch.empty(indices.shape, dtype=grad_output.dtype, device=weights.device)
+    state_dtype = torch.float64 if weights.dtype == torch.float64 else torch.float32
+    _require(optimizer_state.dtype == state_dtype and optimizer_state.is_contiguous(),
+             "optimizer_state must be contiguous %s" % state_dtype)
+    layout = _native.backward_workspace_layout(indices.numel(), 4, code)
+    ws = _workspace(weights.device, layout.total_bytes)
+    with torch.cuda.device(weights.device):
+        _native.check(_native.load().tbe_backward_mixed(
+            optimizer, _ptr(grad_output), _ptr(weights), code, _fp16_vector_width(dim_offsets), total_rows,
+            _ptr(table_offsets), _ptr(table_dim_offsets), _ptr(dim_offsets), int(total_D), T, _ptr(indices),
+            indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state), float(learning_rate),
+            float(eps or 0.0), _ptr(grad_indice_weights), _ptr(ws), ws.numel(), _stream(weights.device)))
+    return grad_indice_weights
+
+
+def backward_exact_adagrad_mixed_D(grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, total_D,
+                                   indices, offsets, indice_weights, optimizer_state, learning_rate, eps,
+                                   stochastic_rounding, BT_block_size):
+    """batched_embedding_backward_adagrad_exact_mixed_D_cuda (table_batched_embeddings_cuda.cu:1350-1469)."""
+    _require(BT_block_size > 0, "BT_block_size must be positive")
+    return _backward_mixed(_native.OPT_ROWWISE_ADAGRAD, grad_output, weights, table_offsets, table_dim_offsets,
+                           dim_offsets, total_D, indices, offsets, indice_weights, optimizer_state, learning_rate,
+                           eps, stochastic_rounding)
+
+
+def backward_approx_adagrad_mixed_D(grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, total_D,
+                                    indices, offsets, indice_weights, optimizer_state, learning_rate, eps, L_max,
+                                    stochastic_rounding, BT_block_size):
+    """Signature of batched_embedding_backward_adagrad_approx_mixed_D_cuda
+    (table_batched_embeddings.cpp:38-43), served by the exact row-wise update."""
+    _require(BT_block_size > 0, "BT_block_size must be positive")
+    return _backward_mixed(_native.OPT_ROWWISE_ADAGRAD, grad_output, weights, table_offsets, table_dim_offsets,
+                           dim_offsets, total_D, indices, offsets, indice_weights, optimizer_state, learning_rate,
+                           eps, stochastic_rounding)
+
+
+def backward_sgd_mixed_D(grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, total_D, indices,
+                         offsets, optimizer_state, learning_rate):
+    """Exact SGD for mixed-dimension tables (no counterpart in the reference, whose mixed module
+    only accepts the Adagrad optimizers, table_batched_embeddings_ops.py:269)."""
+    return _backward_mixed(_native.OPT_SGD, grad_output, weights, table_offsets, table_dim_offsets, dim_offsets,
+                           total_D, indices, offsets, None, optimizer_state, learning_rate, 0.0, False)
 
 
 def construct_offsets(batch_offsets_per_table, total_indices_per_table):

@@ -175,3 +175,107 @@ class TableBatchedEmbeddingBags(nn.Module):
             self.embedding_weights, self.table_offsets, sharded_sparse_features, sharded_offsets,
             per_sample_weights, self.optimizer, self.optimizer_state, self.learning_rate, self.eps,
             self.stochastic_rounding)
+
+
+class MixedDimLookupFunction(torch.autograd.Function):
+    """Mirror of MixedDimLookupFunction (table_batched_embeddings_ops.py:204-321)."""
+
+    @staticmethod
+    def forward(ctx, weights, table_offsets, table_dim_offsets, dim_offsets, total_D, indices, offsets,
+                per_sample_weights, optimizer, optimizer_state, learning_rate, eps, stochastic_rounding):
+        ctx.optimizer = optimizer
+        ctx.learning_rate = learning_rate
+        ctx.eps = eps
+        ctx.stochastic_rounding = stochastic_rounding
+        ctx.total_D = total_D
+        ctx.save_for_backward(weights, table_offsets, table_dim_offsets, dim_offsets, indices, offsets,
+                              per_sample_weights, optimizer_state)
+        return table_batched_embeddings.forward_mixed_D(
+            weights, table_offsets, dim_offsets, total_D, indices, offsets, per_sample_weights, 200, 1, False)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (weights, table_offsets, table_dim_offsets, dim_offsets, indices, offsets, per_sample_weights,
+         optimizer_state) = ctx.saved_tensors
+        L_max = 200
+        if ctx.optimizer == Optimizer.SGD:  # extension: the reference asserts Adagrad here (:269)
+            assert per_sample_weights is None
+            grad_per_sample_weight = table_batched_embeddings.backward_sgd_mixed_D(
+                grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, ctx.total_D, indices, offsets,
+                optimizer_state, ctx.learning_rate)
+        elif ctx.optimizer == Optimizer.APPROX_ROWWISE_ADAGRAD:
+            grad_per_sample_weight = table_batched_embeddings.backward_approx_adagrad_mixed_D(
+                grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, ctx.total_D, indices, offsets,
+                per_sample_weights, optimizer_state, ctx.learning_rate, ctx.eps, L_max, ctx.stochastic_rounding, 1)
+        else:
+            grad_per_sample_weight = table_batched_embeddings.backward_exact_adagrad_mixed_D(
+                grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, ctx.total_D, indices, offsets,
+                per_sample_weights, optimizer_state, ctx.learning_rate, ctx.eps, ctx.stochastic_rounding, 1)
+        empty_grad = None
+        if ctx.needs_input_grad[0]:
+            empty_grad = torch.sparse_coo_tensor(
+                torch.empty((1, 0), dtype=torch.int64, device=weights.device),
+                torch.empty((0,), dtype=weights.dtype, device=weights.device), size=tuple(weights.shape))
+        return (empty_grad, None, None, None, None, None, None, grad_per_sample_weight, None, None, None, None,
+                None)
+
+
+class MixedDimTableBatchedEmbeddingBags(nn.Module):
+    """Mirror of MixedDimTableBatchedEmbeddingBags (table_batched_embeddings_ops.py:324-435):
+    `embeddings` is a list of (rows, dim) per table; weights are one flat 1-D parameter."""
+
+    def __init__(self, embeddings, optimizer=Optimizer.SGD, learning_rate=0.01, eps=None,
+                 stochastic_rounding=False, fp16=False, managed=EmbeddingLocation.DEVICE):
+        super(MixedDimTableBatchedEmbeddingBags, self).__init__()
+        assert managed in (EmbeddingLocation.DEVICE, EmbeddingLocation.HOST_MAPPED)
+        rows, dims = zip(*embeddings)
+        assert all(d > 0 and d % 4 == 0 for d in dims), "every embedding dimension must be a multiple of 4"
+        numel = sum(row * dim for (row, dim) in embeddings)
+        dtype = torch.float16 if fp16 else torch.float32
+        device = torch.device("cuda", torch.cuda.current_device())
+        if managed == EmbeddingLocation.DEVICE:
+            logging.info("Allocating device embedding bag")
+            embedding_data = torch.randn(size=(numel,), device=device, dtype=dtype)
+        else:
+            logging.info("Allocating host-mapped embedding bag")
+            embedding_data = table_batched_embeddings.new_managed_tensor(
+                torch.empty(1, device=device, dtype=dtype), (numel,))
+            embedding_data.normal_()
+        self.embedding_weights = nn.Parameter(embedding_data)
+        self.register_buffer("table_dim_offsets", torch.tensor([0] + np.cumsum(rows).tolist()).int())
+        self.register_buffer("table_offsets",
+                             torch.tensor([0] + np.cumsum([r * d for r, d in zip(rows, dims)]).tolist()).long())
+        self.register_buffer("dim_offsets", torch.tensor([0] + np.cumsum(dims).tolist()).int())
+        self.register_buffer("optimizer_state", torch.zeros(sum(rows)).float())
+        self.total_D = sum(dims)
+        self.optimizer = optimizer
+        self.learning_rate = learning_rate
+        self.eps = eps
+        self.stochastic_rounding = stochastic_rounding
+
+    def forward(self, sharded_sparse_features, sharded_offsets, per_sample_weights=None):
+        return MixedDimLookupFunction.apply(
+            self.embedding_weights, self.table_offsets, self.table_dim_offsets, self.dim_offsets, self.total_D,
+            sharded_sparse_features, sharded_offsets, per_sample_weights, self.optimizer, self.optimizer_state,
+            self.learning_rate, self.eps, self.stochastic_rounding)
+
+    def split_embedding_weights(self):
+        """Returns a list of weights, split by table."""
+        T = self.table_offsets.size(0) - 1
+        return [
+            self.embedding_weights.detach()[self.table_offsets[i]:self.table_offsets[i + 1]].view(
+                self.table_dim_offsets[i + 1] - self.table_dim_offsets[i],
+                self.dim_offsets[i + 1] - self.dim_offsets[i])
+            for i in range(T)
+        ]
+
+    def split_optimizer_state(self):
+        """Returns a list of optimizer states, split by table."""
+        T = self.table_offsets.size(0) - 1
+        return [self.optimizer_state.detach()[self.table_dim_offsets[i]:self.table_dim_offsets[i + 1]]
+                for i in range(T)]
+
+    def split_output(self, output):
+        """Returns a list of outputs, split by table."""
+        T = self.table_offsets.size(0) - 1
+        return [output[:, self.dim_offsets[i]:self.dim_offsets[i + 1]] for i in range(T)]

@@ -61,3 +61,23 @@ def oracle():
     from oracle import tbe_oracle
     tbe_oracle.lib()
     return tbe_oracle
+
+
+def make_mixed_problem(seed, embeddings, B, L, dtype, weighted=False, zipf=1.2):
+    """Seeded problem for tables with per-table (rows, dim): flat 1-D weights and the three offset
+    arrays of MixedDimTableBatchedEmbeddingBags (table_batched_embeddings_ops.py:356-369)."""
+    rs = np.random.RandomState(seed)
+    rows, dims = zip(*embeddings)
+    T = len(embeddings)
+    lengths = rs.randint(0, L + 1, size=(T, B))
+    offsets = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
+    per_table = lengths.sum(axis=1)
+    indices = np.concatenate([(rs.zipf(zipf, size=int(per_table[t])) % rows[t]) for t in range(T)]).astype(np.int32)
+    n = indices.size
+    return dict(T=T, B=B, rows=list(rows), dims=list(dims), n=n, offsets=offsets, indices=indices,
+                table_offsets=np.concatenate([[0], np.cumsum([r * d for r, d in embeddings])]).astype(np.int64),
+                table_dim_offsets=np.concatenate([[0], np.cumsum(rows)]).astype(np.int32),
+                dim_offsets=np.concatenate([[0], np.cumsum(dims)]).astype(np.int32),
+                weights=rs.uniform(-0.01, 0.01, size=sum(r * d for r, d in embeddings)).astype(dtype),
+                grad_output=rs.randn(B, sum(dims)).astype(dtype),
+                per_sample_weights=rs.uniform(0, 1, size=n).astype(dtype) if weighted else None)

@@ -1,0 +1,130 @@
+"""GPU parity of the per-table-dimension path (tbe_forward_mixed / tbe_backward_mixed through
+the C ABI and the MixedDimTableBatchedEmbeddingBags mirror) against the CPU oracle.
+Tolerances as for the uniform path: fp32 1e-5, fp16 1e-2, fp64 1e-7."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_mixed_problem
+from gpu_util import DEV, assert_close, dev
+
+import table_batched_embeddings as ext
+import table_batched_embeddings_ops as ops
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float16): 1e-2, np.dtype(np.float64): 1e-7}
+TABLE_SETS = [
+    [(30, 8), (7, 32), (100, 4), (16, 12)],
+    [(50, 128), (1000, 64), (3, 520)],          # includes a row wider than one wavefront pass
+    [(20, 16)],
+    [(11, 24), (13, 40), (5, 8), (900, 256), (64, 4)],
+]
+
+
+def _gpu_forward(p):
+    return ext.forward_mixed_D(dev(p["weights"]), dev(p["table_offsets"]), dev(p["dim_offsets"]),
+                               int(p["dim_offsets"][-1]), dev(p["indices"]), dev(p["offsets"]),
+                               dev(p["per_sample_weights"]), 200, 1, False).cpu().numpy()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.float64])
+@pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("tables", TABLE_SETS)
+def test_forward_mixed_matches_oracle(oracle, tables, weighted, dtype):
+    p = make_mixed_problem(len(tables), tables, B=19, L=9, dtype=dtype, weighted=weighted)
+    want = oracle.forward_mixed(p["weights"], p["table_offsets"], p["dim_offsets"], p["indices"], p["offsets"],
+                                p["per_sample_weights"])
+    got = _gpu_forward(p)
+    assert got.shape == want.shape and got.dtype == want.dtype
+    assert_close(got, want, TOL[np.dtype(dtype)])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.float64])
+@pytest.mark.parametrize("mode", ["sgd", "adagrad", "adagrad_weighted"])
+@pytest.mark.parametrize("tables", TABLE_SETS)
+def test_backward_mixed_matches_oracle(oracle, tables, mode, dtype):
+    weighted = mode.endswith("weighted")
+    p = make_mixed_problem(len(tables) + 7, tables, B=23, L=8, dtype=dtype, weighted=weighted)
+    optimizer = "sgd" if mode == "sgd" else "adagrad"
+    w_ref = p["weights"].copy()
+    st_dtype = np.float64 if dtype == np.float64 else np.float32
+    st_ref = np.zeros(sum(p["rows"]), st_dtype)
+    gpsw_ref = oracle.backward_mixed(optimizer, p["grad_output"], w_ref, p["table_offsets"], p["table_dim_offsets"],
+                                     p["dim_offsets"], p["indices"], p["offsets"], 0.05, 0.1, st_ref,
+                                     p["per_sample_weights"])
+    w = dev(p["weights"])
+    st = torch.zeros(sum(p["rows"]), device=DEV, dtype=torch.float64 if dtype == np.float64 else torch.float32)
+    args = (dev(p["table_offsets"]), dev(p["table_dim_offsets"]), dev(p["dim_offsets"]), int(p["dim_offsets"][-1]),
+            dev(p["indices"]), dev(p["offsets"]))
+    if optimizer == "sgd":
+        gpsw = ext.backward_sgd_mixed_D(dev(p["grad_output"]), w, *args, st, 0.05)
+    else:
+        gpsw = ext.backward_exact_adagrad_mixed_D(dev(p["grad_output"]), w, *args, dev(p["per_sample_weights"]), st,
+                                                  0.05, 0.1, False, 1)
+    torch.cuda.synchronize()
+    tol = TOL[np.dtype(dtype)]
+    assert_close(w.cpu().numpy(), w_ref, tol)
+    if optimizer == "adagrad":
+        assert_close(st.cpu().numpy(), st_ref, 1e-3 if dtype == np.float16 else max(tol, 1e-6))
+    if weighted:
+        assert_close(gpsw.cpu().numpy(), gpsw_ref, tol)
+    # rows no lookup touches keep their bits
+    keys = p["table_dim_offsets"][np.repeat(np.arange(p["T"] * p["B"]), np.diff(p["offsets"])) // p["B"]] + \
+        p["indices"]
+    touched = np.zeros(sum(p["rows"]), bool)
+    touched[keys] = True
+    for t, (E, D) in enumerate(tables):
+        sl = slice(int(p["table_offsets"][t]), int(p["table_offsets"][t + 1]))
+        rows_t = ~touched[p["table_dim_offsets"][t]:p["table_dim_offsets"][t + 1]]
+        assert w.cpu().numpy()[sl].reshape(E, D)[rows_t].tobytes() == p["weights"][sl].reshape(E, D)[rows_t].tobytes()
+
+
+def test_equal_dims_reproduce_the_uniform_kernels():
+    """With every D_t equal the mixed path computes the same sums as the uniform-D path; the
+    forward outputs agree to rounding and the layouts map onto each other ([B, T*D] == [B, T, D])."""
+    tables = [(200, 64)] * 4
+    p = make_mixed_problem(5, tables, B=40, L=10, dtype=np.float32)
+    got = _gpu_forward(p)
+    uni = ext.forward(dev(p["weights"].reshape(800, 64)), dev(p["table_dim_offsets"][:-1].copy()),
+                      dev(p["indices"]), dev(p["offsets"]), None, 200, 1, False).cpu().numpy()
+    assert_close(got, uni.reshape(40, 256), 1e-6)
+
+
+def test_module_mixed_like_the_reference_test(oracle):
+    """test_backward_adagrad_mixed (test_table_batched_embeddings.py:395-521) through the module:
+    weights set per table via split_embedding_weights, outputs read via split_output, state via
+    split_optimizer_state."""
+    embeddings = [(100, 16), (100, 64), (100, 8)]
+    B, L = 32, 5
+    cc = ops.MixedDimTableBatchedEmbeddingBags(embeddings, optimizer=ops.Optimizer.EXACT_ROWWISE_ADAGRAD,
+                                               learning_rate=0.5, eps=0.2).cuda()
+    assert cc.total_D == 88 and cc.table_offsets.dtype == torch.int64 and cc.dim_offsets.tolist() == [0, 16, 80, 88]
+    assert cc.table_dim_offsets.tolist() == [0, 100, 200, 300] and cc.optimizer_state.shape == (300,)
+    p = make_mixed_problem(9, embeddings, B, L, np.float32, zipf=1.1)
+    for t, w_t in enumerate(cc.split_embedding_weights()):
+        lo, hi = int(p["table_offsets"][t]), int(p["table_offsets"][t + 1])
+        w_t.copy_(dev(p["weights"][lo:hi].reshape(embeddings[t])))
+    out = cc(dev(p["indices"]), dev(p["offsets"]))
+    want = oracle.forward_mixed(p["weights"], p["table_offsets"], p["dim_offsets"], p["indices"], p["offsets"])
+    for t, o_t in enumerate(cc.split_output(out)):
+        assert_close(o_t.detach().cpu().numpy(), want[:, p["dim_offsets"][t]:p["dim_offsets"][t + 1]], 1e-5)
+    out.backward(dev(p["grad_output"]))
+    w_ref = p["weights"].copy()
+    st_ref = np.zeros(300, np.float32)
+    oracle.backward_mixed("adagrad", p["grad_output"], w_ref, p["table_offsets"], p["table_dim_offsets"],
+                          p["dim_offsets"], p["indices"], p["offsets"], 0.5, 0.2, st_ref)
+    for t, (w_t, s_t) in enumerate(zip(cc.split_embedding_weights(), cc.split_optimizer_state())):
+        lo, hi = int(p["table_offsets"][t]), int(p["table_offsets"][t + 1])
+        assert_close(w_t.cpu().numpy(), w_ref[lo:hi].reshape(embeddings[t]), 1e-5)
+        assert_close(s_t.cpu().numpy(), st_ref[p["table_dim_offsets"][t]:p["table_dim_offsets"][t + 1]], 1e-5)
+
+
+def test_mixed_bad_arguments():
+    w = torch.zeros(64, device=DEV)
+    i32 = torch.zeros(3, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="int64"):
+        ext.forward_mixed_D(w, i32[:2], i32[:2], 4, i32[:1], i32[:2], None, 200, 1, False)
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        ext.forward_mixed_D(w, torch.tensor([0, 6], device=DEV), torch.tensor([0, 6], dtype=torch.int32, device=DEV),
+                            6, i32[:1], i32[:2], None, 200, 1, False)

@@ -60,6 +60,21 @@ def test_cpu_tensors_are_rejected_not_silently_computed():
         ext.forward(w, i32[:1], i32, i32, None, 200, 1, False)
 
 
-def test_mixed_d_entry_points_raise():
-    with pytest.raises(NotImplementedError):
-        ext.forward_mixed_D()
+def test_mixed_d_signatures_match_the_pybind_declarations():
+    # table_batched_embeddings.cpp:32-50
+    assert list(inspect.signature(ext.forward_mixed_D).parameters) == [
+        "weights", "table_offsets", "dim_offsets", "total_D", "indices", "offsets", "indice_weights", "L_max",
+        "BT_block_size", "shmem"]
+    assert list(inspect.signature(ext.backward_exact_adagrad_mixed_D).parameters) == [
+        "grad_output", "weights", "table_offsets", "table_dim_offsets", "dim_offsets", "total_D", "indices",
+        "offsets", "indice_weights", "optimizer_state", "learning_rate", "eps", "stochastic_rounding",
+        "BT_block_size"]
+    assert list(inspect.signature(ext.backward_approx_adagrad_mixed_D).parameters) == [
+        "grad_output", "weights", "table_offsets", "table_dim_offsets", "dim_offsets", "total_D", "indices",
+        "offsets", "indice_weights", "optimizer_state", "learning_rate", "eps", "L_max", "stochastic_rounding",
+        "BT_block_size"]
+    params = inspect.signature(ops.MixedDimTableBatchedEmbeddingBags.__init__).parameters
+    assert list(params)[1:] == ["embeddings", "optimizer", "learning_rate", "eps", "stochastic_rounding", "fp16",
+                                "managed"]
+    for helper in ("split_embedding_weights", "split_optimizer_state", "split_output"):
+        assert callable(getattr(ops.MixedDimTableBatchedEmbeddingBags, helper))

@@ -321,3 +321,59 @@ def test_cache_rows_used_in_a_step_are_never_evicted_in_it(oracle):
     assert stats.tolist() == [100, 64, 36, 0, 0, 36]
     assert (slots[64:] == -1).all() and (evicted == -2).all()
     assert m.resident().tolist() == list(range(64))
+
+
+# ------------------------------------------------------------ per-table dimension
+@pytest.mark.parametrize("weighted", [False, True])
+def test_mixed_dim_matches_embeddingbag(oracle, weighted):
+    """The check of test_table_batched_embeddings.py:395-521: one torch.nn.EmbeddingBag per
+    table with its own (rows, dim); forward, Adagrad state and weights."""
+    torch = pytest.importorskip("torch")
+    from conftest import make_mixed_problem
+    embeddings = [(30, 8), (7, 32), (100, 4), (16, 12)]
+    p = make_mixed_problem(21, embeddings, B=11, L=6, dtype=np.float32, weighted=weighted, zipf=1.3)
+    out = oracle.forward_mixed(p["weights"], p["table_offsets"], p["dim_offsets"], p["indices"], p["offsets"],
+                               p["per_sample_weights"])
+    w = p["weights"].copy()
+    state = np.zeros(sum(p["rows"]), np.float32)
+    lr, eps = 0.5, 0.2
+    gpsw = oracle.backward_mixed("adagrad", p["grad_output"], w, p["table_offsets"], p["table_dim_offsets"],
+                                 p["dim_offsets"], p["indices"], p["offsets"], lr, eps, state,
+                                 p["per_sample_weights"])
+    for t, (E, D) in enumerate(embeddings):
+        lo, hi = p["offsets"][t * p["B"]], p["offsets"][(t + 1) * p["B"]]
+        bag = torch.nn.EmbeddingBag(E, D, mode="sum", sparse=True)
+        w_t = p["weights"][p["table_offsets"][t]:p["table_offsets"][t + 1]].reshape(E, D)
+        bag.weight.data.copy_(torch.from_numpy(w_t))
+        kw = {}
+        if weighted:
+            psw_t = torch.from_numpy(p["per_sample_weights"][lo:hi].copy()).requires_grad_(True)
+            kw["per_sample_weights"] = psw_t
+        y = bag(torch.from_numpy(p["indices"][lo:hi].astype(np.int64)),
+                torch.from_numpy((p["offsets"][t * p["B"]:(t + 1) * p["B"]] - lo).astype(np.int64)), **kw)
+        d0, d1 = p["dim_offsets"][t], p["dim_offsets"][t + 1]
+        np.testing.assert_allclose(out[:, d0:d1], y.detach().numpy(), rtol=1e-5, atol=1e-8)
+        y.backward(torch.from_numpy(p["grad_output"][:, d0:d1].copy()))
+        grad = bag.weight.grad.to_dense()
+        st = grad.pow(2).sum(1)
+        r0, r1 = p["table_dim_offsets"][t], p["table_dim_offsets"][t + 1]
+        np.testing.assert_allclose(state[r0:r1], st.numpy(), rtol=1e-5, atol=1e-12)
+        want_w = torch.addcdiv(bag.weight.detach(), grad, (st.sqrt() + eps).view(E, 1), value=-lr)
+        got_w = w[p["table_offsets"][t]:p["table_offsets"][t + 1]].reshape(E, D)
+        np.testing.assert_allclose(got_w, want_w.numpy(), rtol=1e-5, atol=1e-7)
+        if weighted:
+            np.testing.assert_allclose(gpsw[lo:hi], psw_t.grad.numpy(), rtol=1e-5, atol=1e-8)
+
+
+def test_mixed_dim_with_equal_dims_equals_uniform_path(oracle):
+    from conftest import make_mixed_problem
+    p = make_mixed_problem(22, [(40, 16)] * 3, B=9, L=5, dtype=np.float64)
+    out = oracle.forward_mixed(p["weights"], p["table_offsets"], p["dim_offsets"], p["indices"], p["offsets"])
+    uni = oracle.forward(p["weights"].reshape(120, 16), p["table_dim_offsets"][:-1], p["indices"], p["offsets"])
+    assert out.tobytes() == np.ascontiguousarray(uni.reshape(9, 48)).tobytes()
+    w1, w2 = p["weights"].copy(), p["weights"].copy().reshape(120, 16)
+    oracle.backward_mixed("sgd", p["grad_output"], w1, p["table_offsets"], p["table_dim_offsets"], p["dim_offsets"],
+                          p["indices"], p["offsets"], 0.1)
+    oracle.backward("sgd", p["grad_output"].reshape(9, 3, 16), w2, p["table_dim_offsets"][:-1], p["indices"],
+                    p["offsets"], 0.1)
+    assert w1.tobytes() == w2.tobytes()
