@@ -1,0 +1,130 @@
+"""Micro-benchmark CLI with the flags of the reference's table_batched_embeddings_benchmark.py
+(:360-370): --num-tables 64 --num-embeddings 10000 --embedding-dim 32 --batch-size 128
+--bag-size 32 --iters 100 [--fp16] [--managed] [--mixed] [--remote], plus --alpha / --seed.
+
+Each operator is called directly on the extension-module mirror (not through autograd), after
+one warm-up call, `iters` times between two events on the current stream
+(table_batched_embeddings_benchmark.py:27-37).  "BW" is the reference's figure:
+elem * B * T * L * D / time for forward (:240) and twice that for backward (:356).  One JSON
+object per measurement goes to stdout.
+"""
+import json
+import logging
+import sys
+
+import click
+import numpy as np
+import torch
+
+import table_batched_embeddings
+import table_batched_embeddings_ops as ops
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def time_calls(iters, fn):
+    fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1.0e-3 / iters
+
+
+def draw_indices(rs, T, B, L, rows, alpha):
+    if alpha and alpha > 1.0:
+        cols = [rs.zipf(alpha, size=(B, L)) % rows[t] for t in range(T)]
+    else:
+        cols = [rs.randint(0, rows[t], size=(B, L)) for t in range(T)]
+    merged = np.stack(cols).astype(np.int32)  # [T][B][L], table-major as the kernels expect
+    offsets = np.arange(0, T * B * L + 1, L, dtype=np.int32)
+    return torch.from_numpy(merged.reshape(-1)).cuda(), torch.from_numpy(offsets).cuda()
+
+
+def report(name, seconds, bytes_moved, shape):
+    record = dict(shape, op=name, time_us=seconds * 1e6, BW_GBps=bytes_moved / seconds / 1e9,
+                  frac_of_hbm_peak=bytes_moved / seconds / 1e9 / HBM_PEAK_GBPS)
+    logging.info("%s, B: %d, E: %s, T: %d, D: %s, L: %d, BW: %.2fGB/s, T: %.0fus", name, shape["B"], shape["E"],
+                 shape["T"], shape["D"], shape["L"], record["BW_GBps"], record["time_us"])
+    print(json.dumps(record))
+
+
+def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
+    rs = np.random.RandomState(seed)
+    location = ops.EmbeddingLocation.HOST_MAPPED if managed else ops.EmbeddingLocation.DEVICE
+    elem = 2 if fp16 else 4
+    if mixed:
+        dims = [int((rs.randint(int(0.5 * D), int(1.5 * D) + 1) + 3) // 4 * 4) for _ in range(T)]
+        cc = ops.MixedDimTableBatchedEmbeddingBags([(E, d) for d in dims], optimizer=ops.Optimizer.EXACT_ROWWISE_ADAGRAD,
+                                                   learning_rate=0.1, eps=0.1, fp16=fp16, managed=location).cuda()
+        D_eff = float(np.mean(dims))
+    else:
+        cc = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.EXACT_ROWWISE_ADAGRAD, learning_rate=0.1,
+                                           eps=0.1, fp16=fp16, managed=location).cuda()
+        D_eff = D
+    logging.info("Embedding parameters: %.2fGParam", cc.embedding_weights.numel() / 1.0e9)
+    indices, offsets = draw_indices(rs, T, B, L, [E] * T, alpha)
+    unique = np.unique(indices.cpu().numpy().astype(np.int64) + np.repeat(np.arange(T), B * L) * E).size
+    logging.info("Duplicate proportion: %.3f", 1.0 - unique / indices.numel())
+    shape = dict(B=B, E=E, T=T, D=D_eff, L=L, fp16=fp16, managed=managed, mixed=mixed, alpha=alpha)
+    w = cc.embedding_weights.data
+    fwd_bytes = elem * B * T * L * D_eff
+
+    if mixed:
+        fwd = lambda: table_batched_embeddings.forward_mixed_D(
+            w, cc.table_offsets, cc.dim_offsets, cc.total_D, indices, offsets, None, L, 1, False)
+    else:
+        fwd = lambda: table_batched_embeddings.forward(w, cc.table_offsets, indices, offsets, None, L, 1, False)
+    y0 = fwd()
+    if not mixed:  # the launch knobs of the reference must not change results (:179-206)
+        for bt in (1, 2, 4, 8, 16, 32, 64, 128):
+            for shmem in (True, False):
+                assert torch.equal(table_batched_embeddings.forward(w, cc.table_offsets, indices, offsets, None, L,
+                                                                    bt, shmem), y0)
+    report("Forward", time_calls(iters, fwd), fwd_bytes, shape)
+
+    go = torch.randn_like(y0)
+    lr, eps = 0.05, 0.01
+    if mixed:
+        sgd = lambda: table_batched_embeddings.backward_sgd_mixed_D(
+            go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets,
+            cc.optimizer_state, lr)
+        ada = lambda: table_batched_embeddings.backward_exact_adagrad_mixed_D(
+            go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets, None,
+            cc.optimizer_state, lr, eps, False, 1)
+    else:
+        sgd = lambda: table_batched_embeddings.backward_sgd(go, w, cc.table_offsets, indices, offsets, lr, L, 1,
+                                                            False)
+        ada = lambda: table_batched_embeddings.backward_exact_adagrad(
+            go, w, cc.table_offsets, indices, offsets, None, cc.optimizer_state, lr, eps, False, 1)
+    report("Backward-SGD-EXACT", time_calls(iters, sgd), 2 * fwd_bytes, shape)
+    report("Backward-ADAGRAD-nonstochastic-EXACT", time_calls(iters, ada), 2 * fwd_bytes, shape)
+
+
+@click.command()
+@click.option("--num-tables", default=64)
+@click.option("--num-embeddings", default=int(1e4))
+@click.option("--embedding-dim", default=32)
+@click.option("--batch-size", default=128)
+@click.option("--bag-size", default=32)
+@click.option("--iters", default=100)
+@click.option("--remote", is_flag=True, default=False)
+@click.option("--fp16", is_flag=True, default=False)
+@click.option("--managed", is_flag=True, default=False)
+@click.option("--mixed", is_flag=True, default=False)
+@click.option("--alpha", default=0.0, help="Zipf exponent of the indices (0 = uniform)")
+@click.option("--seed", default=42)
+def cli(num_tables, num_embeddings, embedding_dim, batch_size, bag_size, iters, remote, fp16, managed, mixed, alpha,
+        seed):
+    logging.basicConfig(level=logging.INFO, stream=sys.stderr)
+    if remote:
+        raise click.UsageError("--remote (cluster submission) is not available; run the benchmark locally")
+    run(batch_size, num_embeddings, num_tables, bag_size, embedding_dim, iters, fp16, managed, mixed, alpha, seed)
+
+
+if __name__ == "__main__":
+    cli()

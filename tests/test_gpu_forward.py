@@ -150,3 +150,20 @@ def test_full_size_forward_properties():
     out = ext.forward(W, table_offsets, idx, offsets, None, 200, 1, False)
     want_c = ((torch.arange(T, device=DEV, dtype=torch.float32) + 1) / 64 * L).view(1, T, 1).expand(B, T, D)
     assert torch.equal(out, want_c)
+
+
+def test_benchmark_cli_runs_with_reference_flags():
+    """The micro-benchmark keeps the reference's flag names (table_batched_embeddings_benchmark.py:360-370)."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from conftest import PACKAGE
+    cmd = [sys.executable, os.path.join(PACKAGE, "table_batched_embeddings_benchmark.py"), "--num-tables", "4",
+           "--num-embeddings", "1000", "--embedding-dim", "32", "--batch-size", "64", "--bag-size", "8", "--iters",
+           "3", "--fp16"]
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=280)
+    assert out.returncode == 0, out.stderr[-2000:]
+    records = [json.loads(line) for line in out.stdout.splitlines() if line.startswith("{")]
+    assert [r["op"] for r in records] == ["Forward", "Backward-SGD-EXACT", "Backward-ADAGRAD-nonstochastic-EXACT"]
+    assert all(r["BW_GBps"] > 0 for r in records)
