@@ -153,6 +153,23 @@ TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, i
                                void *grad_per_sample_weights,
                                void *workspace, uint64_t workspace_bytes, void *stream);
 
+/* tbe_backward_exact_adagrad with fp16 stochastic rounding of the updated weights
+ * (StochasticRoundingAdaGradFunctor, table_batched_embeddings_cuda.cu:618-646, and
+ * stochastic_rounding_vector, :557-578: 13 random bits added to the fp32 pattern, then
+ * truncation to fp16).  The reference draws its bits from cuRAND's Philox4_32_10 seeded from
+ * PyTorch's generator per thread (:1685-1691); here element e of the table takes word e % 4 of
+ * Philox4x32-10(counter = {e / 4, offset}, key = seed), so results are reproducible for a
+ * given (seed, offset) and independent of launch geometry.  The two random streams differ,
+ * so only the distribution -- not the bits -- matches the reference.  For dtypes other than
+ * F16 the call equals tbe_backward_exact_adagrad.
+ */
+TBE_API int tbe_backward_exact_adagrad_stochastic(
+    const void *grad_output, void *weights, int32_t dtype, int64_t total_rows, int32_t D,
+    const int32_t *table_offsets, int32_t T, const int32_t *indices, int64_t num_indices,
+    const int32_t *offsets, int32_t B, const void *per_sample_weights, void *optimizer_state,
+    float learning_rate, float eps, void *grad_per_sample_weights, uint64_t seed, uint64_t offset,
+    void *workspace, uint64_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------- stages, individually callable
  * The backward entry points run exactly these stages on the caller's workspace.
  */
@@ -204,7 +221,8 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
  * (table_batched_embeddings_cuda.cu:945-1004, "forward_mixed_D" in table_batched_embeddings.cpp:66);
  * tbe_backward_mixed replaces batched_embedding_backward_adagrad_exact_mixed_D_cuda
  * (:1350-1469, "backward_exact_adagrad_mixed_D", .cpp:64), serves the approximate variant
- * (.cpp:63) and adds exact SGD; per-sample weights as in tbe_backward_exact_adagrad.  The
+ * (.cpp:63) and adds exact SGD; per-sample weights as in tbe_backward_exact_adagrad;
+ * stochastic_rounding / seed / offset as in tbe_backward_exact_adagrad_stochastic.  The
  * workspace is a backward workspace sized with tbe_backward_workspace_layout(N, 4, dtype).
  */
 TBE_API int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp16_vector_width,
@@ -222,6 +240,7 @@ TBE_API int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void 
                                const int32_t *offsets, int32_t B,
                                const void *per_sample_weights, void *optimizer_state,
                                float learning_rate, float eps, void *grad_per_sample_weights,
+                               int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
                                void *workspace, uint64_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- row cache

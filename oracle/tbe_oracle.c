@@ -100,6 +100,69 @@ static inline void store_f(void *p, int dtype, int64_t i, float v) {
   else ((uint16_t *)p)[i] = oracle_float_to_half(v);
 }
 
+/* -------------------------------------------------------- stochastic rounding
+ * Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3",
+ * SC'11) -- the generator behind curandStatePhilox4_32_10_t, which the reference draws its
+ * rounding bits from (tbe.cu:595-599, 627-631).  cuRAND is not part of the reference tree and
+ * its per-thread stream layout cannot be reproduced, so the BITS of a stochastically rounded
+ * result are PARITY UNPINNED against the reference; the rounding rule itself
+ * (stochastic_rounding_vector, tbe.cu:564-578: add 13 random bits to the fp32 pattern, truncate
+ * toward zero) is restated exactly.  Pinned by the Random123 known-answer vectors and by
+ * statistical tests (unbiased, within one fp16 ulp, exact values unchanged).
+ */
+void oracle_philox4x32_10(const uint32_t ctr_in[4], const uint32_t key_in[2], uint32_t out[4]) {
+  uint32_t c0 = ctr_in[0], c1 = ctr_in[1], c2 = ctr_in[2], c3 = ctr_in[3];
+  uint32_t k0 = key_in[0], k1 = key_in[1];
+  for (int round = 0; round < 10; ++round) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* __float2half_rz */
+static uint16_t float_to_half_rz(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  const uint32_t ax = x & 0x7fffffffu;
+  if (ax >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | ((ax > 0x7f800000u) ? 0x200u : 0u));
+  if (ax >= 0x47800000u) return (uint16_t)(sign | 0x7bffu); /* >= 65536: truncates to the largest finite half */
+  const int32_t e = (int32_t)(ax >> 23) - 127;
+  if (e < -24) return sign;
+  const uint32_t m = (ax & 0x7fffffu) | 0x800000u;
+  if (e < -14) return (uint16_t)(sign | (m >> (13 + (-14 - e))));
+  return (uint16_t)(sign | (((uint32_t)(e + 15) << 10) | ((m >> 13) & 0x3ffu)));
+}
+
+/* one element: stochastic_rounding_vector (tbe.cu:569-576) */
+uint16_t oracle_stochastic_round(float value, uint32_t random_bits) {
+  uint32_t x;
+  memcpy(&x, &value, 4);
+  x += random_bits >> 19;
+  float f;
+  memcpy(&f, &x, 4);
+  return float_to_half_rz(f);
+}
+
+/* Stores `count` (a multiple of 4) fp16 values starting at table element `element` (a multiple
+ * of 4): element e takes word e % 4 of Philox(counter = {e / 4, offset}, key = seed). */
+static void store_row_stochastic(uint16_t *dst, const float *values, int32_t count, int64_t element,
+                                 uint64_t seed, uint64_t offset) {
+  for (int32_t q = 0; q < count; q += 4) {
+    const uint64_t group = (uint64_t)(element + q) / 4;
+    const uint32_t ctr[4] = {(uint32_t)group, (uint32_t)(group >> 32), (uint32_t)offset, (uint32_t)(offset >> 32)};
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    uint32_t r[4];
+    oracle_philox4x32_10(ctr, key, r);
+    for (int k = 0; k < 4; ++k) dst[q + k] = oracle_stochastic_round(values[q + k], r[k]);
+  }
+}
+
 /* ------------------------------------------------------------------ forward
  * batched_embedding_forward_kernel_1 (tbe.cu:193-251) with UnweightedForward /
  * WeightedForward (tbe.cu:166-191): b_t = t*B + b; serial sum over the bag in
@@ -229,14 +292,16 @@ int64_t oracle_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_
  *   leaves as a TODO (tbe.cu:1552, 1678-1679).
  * `total_rows` sets the sorted bit range int(log2(total_rows) + 1) (tbe.cu:1643).
  * keys_sorted / positions_sorted / segment_starts may be NULL or receive the
- * intermediate results; *num_unique receives U.
+ * intermediate results; *num_unique receives U.  With stochastic_rounding (fp16 only) the
+ * updated row is rounded by store_row_stochastic (StochasticRoundingAdaGradFunctor, tbe.cu:618-646).
  */
 int oracle_backward(int optimizer, const void *grad_output, void *weights, int dtype,
                     int64_t total_rows, int32_t D, const int32_t *table_offsets, int32_t T,
                     const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
                     const void *psw, void *optimizer_state, float lr, float eps, void *grad_psw,
                     int32_t *keys_sorted_out, int32_t *positions_sorted_out,
-                    int32_t *segment_starts_out, int64_t *num_unique) {
+                    int32_t *segment_starts_out, int64_t *num_unique, int32_t stochastic_rounding,
+                    uint64_t sr_seed, uint64_t sr_offset) {
   const size_t nn = (size_t)(n > 0 ? n : 1);
   int32_t *keys = (int32_t *)malloc(nn * 4), *b_ts = (int32_t *)malloc(nn * 4);
   int32_t *pos = (int32_t *)malloc(nn * 4), *keys_s = (int32_t *)malloc(nn * 4);
@@ -309,10 +374,15 @@ int oracle_backward(int optimizer, const void *grad_output, void *weights, int d
         *st = old + gss;
         mult = (float)(lr * (1.0 / (sqrtf(old + gss) + eps)));
       }
-      for (int32_t d = 0; d < D; ++d) {
-        float w = load_f(weights, dtype, row * D + d);
-        w -= Gf[d] * mult;
-        store_f(weights, dtype, row * D + d, w);
+      if (stochastic_rounding && dtype == F16) {
+        for (int32_t d = 0; d < D; ++d) Gf[d] = load_f(weights, dtype, row * D + d) - Gf[d] * mult;
+        store_row_stochastic((uint16_t *)weights + row * D, Gf, D, row * D, sr_seed, sr_offset);
+      } else {
+        for (int32_t d = 0; d < D; ++d) {
+          float w = load_f(weights, dtype, row * D + d);
+          w -= Gf[d] * mult;
+          store_f(weights, dtype, row * D + d, w);
+        }
       }
     }
   }

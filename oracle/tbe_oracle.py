@@ -88,9 +88,10 @@ def segments(keys_sorted):
 
 
 def backward(optimizer, grad_output, weights, table_offsets, indices, offsets, lr, eps=0.0,
-             optimizer_state=None, per_sample_weights=None):
+             optimizer_state=None, per_sample_weights=None, stochastic_rounding=None):
     """In-place update of `weights` (and `optimizer_state`); optimizer 'sgd' or 'adagrad'.
 
+    stochastic_rounding: None or (seed, offset) for fp16 weights.
     Returns dict(keys_sorted, positions_sorted, segment_starts, grad_psw)."""
     assert weights.flags["C_CONTIGUOUS"] and weights.dtype in _CODES
     code = _CODES[weights.dtype]
@@ -116,7 +117,9 @@ def backward(optimizer, grad_output, weights, table_offsets, indices, offsets, l
                           ctypes.c_int64(weights.shape[0]), ctypes.c_int32(D), _p(table_offsets), ctypes.c_int32(T),
                           _p(indices), ctypes.c_int64(n), _p(offsets), ctypes.c_int32(B), _p(psw),
                           _p(optimizer_state), ctypes.c_float(lr), ctypes.c_float(eps), _p(gpsw), _p(ks), _p(ps),
-                          _p(ss), ctypes.byref(U))
+                          _p(ss), ctypes.byref(U), ctypes.c_int32(0 if stochastic_rounding is None else 1),
+                          ctypes.c_uint64(0 if stochastic_rounding is None else stochastic_rounding[0]),
+                          ctypes.c_uint64(0 if stochastic_rounding is None else stochastic_rounding[1]))
     return {"keys_sorted": ks, "positions_sorted": ps, "segment_starts": ss[: U.value + 1].copy(), "grad_psw": gpsw}
 
 
@@ -216,3 +219,18 @@ def backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_off
                                 ctypes.c_int64(indices.size), _p(offsets), ctypes.c_int32(B), _p(psw),
                                 _p(optimizer_state), ctypes.c_float(lr), ctypes.c_float(eps), _p(gpsw))
     return gpsw
+
+
+def philox4x32_10(counter, key):
+    ctr = (ctypes.c_uint32 * 4)(*counter)
+    k = (ctypes.c_uint32 * 2)(*key)
+    out = (ctypes.c_uint32 * 4)()
+    lib().oracle_philox4x32_10(ctr, k, out)
+    return list(out)
+
+
+def stochastic_round(value, random_bits):
+    fn = lib().oracle_stochastic_round
+    fn.restype = ctypes.c_uint16
+    fn.argtypes = [ctypes.c_float, ctypes.c_uint32]
+    return fn(float(value), int(random_bits))

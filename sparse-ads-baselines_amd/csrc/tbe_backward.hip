@@ -101,6 +101,7 @@ struct BackwardCall {
   bool planned;
   const int32_t *unique_slots;
   void *cache_rows;
+  StochasticRounding stochastic_rounding;
 };
 
 int run_backward(const char *name, const BackwardCall &c) {
@@ -163,6 +164,7 @@ int run_backward(const char *name, const BackwardCall &c) {
   a.optimizer = c.optimizer;
   a.learning_rate = c.lr;
   a.eps = c.eps;
+  a.stochastic_rounding = c.stochastic_rounding;
   return segment_update(a, c.stream);
 }
 
@@ -190,7 +192,7 @@ extern "C" int tbe_backward_sgd(const void *grad_output, void *weights, int32_t 
   tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
                       num_indices, offsets, B, nullptr, nullptr, learning_rate, 0.0f, nullptr,
                       workspace, workspace_bytes, static_cast<hipStream_t>(stream), tbe::kOptSgd,
-                      false, nullptr, nullptr};
+                      false, nullptr, nullptr, tbe::StochasticRounding{0, 0, 0}};
   return tbe::run_backward("tbe_backward_sgd", c);
 }
 
@@ -206,8 +208,23 @@ extern "C" int tbe_backward_exact_adagrad(const void *grad_output, void *weights
   tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
                       num_indices, offsets, B, per_sample_weights, optimizer_state, learning_rate,
                       eps, grad_per_sample_weights, workspace, workspace_bytes,
-                      static_cast<hipStream_t>(stream), tbe::kOptAdagrad, false, nullptr, nullptr};
+                      static_cast<hipStream_t>(stream), tbe::kOptAdagrad, false, nullptr, nullptr,
+                      tbe::StochasticRounding{0, 0, 0}};
   return tbe::run_backward("tbe_backward_exact_adagrad", c);
+}
+
+extern "C" int tbe_backward_exact_adagrad_stochastic(
+    const void *grad_output, void *weights, int32_t dtype, int64_t total_rows, int32_t D,
+    const int32_t *table_offsets, int32_t T, const int32_t *indices, int64_t num_indices,
+    const int32_t *offsets, int32_t B, const void *per_sample_weights, void *optimizer_state,
+    float learning_rate, float eps, void *grad_per_sample_weights, uint64_t seed, uint64_t offset,
+    void *workspace, uint64_t workspace_bytes, void *stream) {
+  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
+                      num_indices, offsets, B, per_sample_weights, optimizer_state, learning_rate,
+                      eps, grad_per_sample_weights, workspace, workspace_bytes,
+                      static_cast<hipStream_t>(stream), tbe::kOptAdagrad, false, nullptr, nullptr,
+                      tbe::StochasticRounding{seed, offset, dtype == TBE_DTYPE_F16 ? 1 : 0}};
+  return tbe::run_backward("tbe_backward_exact_adagrad_stochastic", c);
 }
 
 extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
@@ -228,6 +245,7 @@ extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
                  num_indices, nullptr, B, per_sample_weights, optimizer_state, learning_rate, eps,
                  grad_per_sample_weights, workspace, workspace_bytes,
                  static_cast<hipStream_t>(stream),
-                 optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad, true, unique_slots, cache->rows};
+                 optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad, true, unique_slots, cache->rows,
+                 StochasticRounding{0, 0, 0}};
   return run_backward("tbe_backward_cached", c);
 }

@@ -154,6 +154,67 @@ template <> __device__ __forceinline__ uint2 RowVec<__half, 4>::pack() const {
   return make_uint2(floats_to_half2(v[0], v[1]), floats_to_half2(v[2], v[3]));
 }
 
+// ------------------------------------------------------------ stochastic rounding
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11), the
+// generator behind curandStatePhilox4_32_10_t that the reference draws its rounding bits from
+// (table_batched_embeddings_cuda.cu:595-599, 627-631).
+__device__ __forceinline__ uint4 philox4x32_10(uint4 ctr, uint2 key) {
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, ctr.x), lo0 = 0xD2511F53u * ctr.x;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, ctr.z), lo1 = 0xCD9E8D57u * ctr.z;
+    ctr = make_uint4(hi1 ^ ctr.y ^ key.x, lo1, hi0 ^ ctr.w ^ key.y, lo0);
+    key.x += 0x9E3779B9u;
+    key.y += 0xBB67AE85u;
+  }
+  return ctr;
+}
+
+struct StochasticRounding {
+  uint64_t seed;     // Philox key
+  uint64_t offset;   // high half of the Philox counter: one value per backward call
+  int32_t enabled;
+};
+
+// fp32 -> fp16 with stochastic rounding as in stochastic_rounding_vector
+// (table_batched_embeddings_cuda.cu:564-578): 13 random bits are added to the fp32 pattern,
+// then the value is truncated toward zero.
+__device__ __forceinline__ uint32_t floats_to_half2_stochastic(float lo, float hi, uint32_t r0, uint32_t r1) {
+  const __half a = __float2half_rz(__uint_as_float(__float_as_uint(lo) + (r0 >> 19)));
+  const __half b = __float2half_rz(__uint_as_float(__float_as_uint(hi) + (r1 >> 19)));
+  return static_cast<uint32_t>(__half_as_ushort(a)) | (static_cast<uint32_t>(__half_as_ushort(b)) << 16);
+}
+
+// Stores VEC accumulator values at p.  For fp16 with stochastic rounding enabled, element e of
+// the table (e = row * D + column, a multiple of 4) takes word (e % 4) of
+// Philox(counter = {e / 4, offset}, key = seed), so the bits depend on the element and the
+// call, not on the launch geometry.
+template <typename T, int VEC, bool STREAMING>
+__device__ __forceinline__ void store_row(T *p, const RowVec<T, VEC> &v, const StochasticRounding &sr,
+                                          int64_t element) {
+  if constexpr (sizeof(T) == 2) {
+    if (sr.enabled) {
+      uint32_t words[VEC / 2];
+#pragma unroll
+      for (int q = 0; q < VEC / 4; ++q) {
+        const uint64_t group = static_cast<uint64_t>(element) / 4 + q;
+        const uint4 r = philox4x32_10(
+            make_uint4(static_cast<uint32_t>(group), static_cast<uint32_t>(group >> 32),
+                       static_cast<uint32_t>(sr.offset), static_cast<uint32_t>(sr.offset >> 32)),
+            make_uint2(static_cast<uint32_t>(sr.seed), static_cast<uint32_t>(sr.seed >> 32)));
+        words[2 * q] = floats_to_half2_stochastic(v.v[4 * q], v.v[4 * q + 1], r.x, r.y);
+        words[2 * q + 1] = floats_to_half2_stochastic(v.v[4 * q + 2], v.v[4 * q + 3], r.z, r.w);
+      }
+      typename RowVec<T, VEC>::R raw;
+      __builtin_memcpy(&raw, words, sizeof(raw));
+      *reinterpret_cast<typename RowVec<T, VEC>::R *>(p) = raw;
+      return;
+    }
+  }
+  if constexpr (STREAMING) v.store_streaming(p);
+  else v.store(p);
+}
+
 __device__ __forceinline__ float to_acc(float x) { return x; }
 __device__ __forceinline__ float to_acc(__half x) { return __half2float(x); }
 __device__ __forceinline__ double to_acc(double x) { return x; }

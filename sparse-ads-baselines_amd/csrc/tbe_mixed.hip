@@ -128,7 +128,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_mixed_kernel(
     int num_tables, int total_D, const int32_t *__restrict__ keys_sorted,
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters, float lr,
-    float eps) {
+    float eps, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
 
@@ -152,7 +152,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_mixed_kernel(
     const int dim_start = dim_offsets[t];
     const int D = dim_offsets[t + 1] - dim_start;
     const int chunks = D / VEC;
-    T *wrow = weights + table_offsets[t] + static_cast<int64_t>(key - table_dim_offsets[t]) * D;
+    const int64_t row_element = table_offsets[t] + static_cast<int64_t>(key - table_dim_offsets[t]) * D;
+    T *wrow = weights + row_element;
     const T *gcol = grad_output + dim_start;
 
     if constexpr (WEIGHTED) {
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_mixed_kernel(
       w.load(wrow + static_cast<int64_t>(cb) * VEC);
 #pragma unroll
       for (int k = 0; k < VEC; ++k) w.v[k] = w.v[k] - G.v[k] * mult;
-      w.store(wrow + static_cast<int64_t>(cb) * VEC);
+      store_row<T, VEC, false>(wrow + static_cast<int64_t>(cb) * VEC, w, sr, row_element + static_cast<int64_t>(cb) * VEC);
     }
   }
 }
@@ -237,6 +238,7 @@ struct MixedArgs {
   void *grad_psw;
   float lr, eps;
   int optimizer;
+  StochasticRounding sr;
 };
 
 template <typename T, int VEC>
@@ -265,7 +267,7 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
              static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights), static_cast<A *>(a.state),
              static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw), a.table_offsets, a.table_dim_offsets,
              a.dim_offsets, a.T, a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows),
-             i32(l.segment_starts), i32(l.num_unique), a.lr, a.eps);
+             i32(l.segment_starts), i32(l.num_unique), a.lr, a.eps, a.sr);
 }
 
 template <typename T, int VEC>
@@ -340,6 +342,7 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
                                   const int32_t *offsets, int32_t B,
                                   const void *per_sample_weights, void *optimizer_state,
                                   float learning_rate, float eps, void *grad_per_sample_weights,
+                                  int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
                                   void *workspace, uint64_t workspace_bytes, void *stream) {
   using namespace tbe;
   const char *name = "tbe_backward_mixed";
@@ -362,6 +365,7 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   a.grad_psw = grad_per_sample_weights;
   a.lr = learning_rate;
   a.eps = eps;
+  a.sr = StochasticRounding{seed, offset, (stochastic_rounding && dtype == TBE_DTYPE_F16) ? 1 : 0};
   TBE_REQUIRE(optimizer == TBE_OPT_SGD || optimizer == TBE_OPT_ROWWISE_ADAGRAD, "%s: bad optimizer %d", name,
               optimizer);
   a.optimizer = optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad;

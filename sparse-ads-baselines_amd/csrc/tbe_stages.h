@@ -52,6 +52,7 @@ struct UpdateArgs {
   int32_t optimizer;
   float learning_rate;
   float eps;
+  StochasticRounding stochastic_rounding;  // fp16 weights only
 };
 
 int segment_update(const UpdateArgs &args, hipStream_t stream);

@@ -57,7 +57,8 @@ template <typename T, int VEC, int CHUNKS, int OPT, bool STREAMING = false>
 __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_old,
                                              const RowVec<T, VEC> &G,
                                              typename AccOf<T>::type *state_row, float lr,
-                                             float eps, int chunks, int group_base, int c) {
+                                             float eps, int chunks, int group_base, int c,
+                                             const StochasticRounding &sr, int64_t element) {
   using A = typename AccOf<T>::type;
   RowVec<T, VEC> w_new;
   if constexpr (OPT == kOptSgd) {
@@ -74,8 +75,7 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 #pragma unroll
     for (int i = 0; i < VEC; ++i) w_new.v[i] = w_old.v[i] - G.v[i] * mult;
   }
-  if constexpr (STREAMING) w_new.store_streaming(wrow);
-  else w_new.store(wrow);
+  store_row<T, VEC, STREAMING>(wrow, w_new, sr, element);
 }
 
 // ------------------------------------------------------------ short segments
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     int32_t *__restrict__ counters, LongRecord *__restrict__ long_records,
     ChunkRecord *__restrict__ chunk_records, int64_t n, int64_t num_tiles, int64_t tiles_per_xcd,
     int D, int chunks_rt, float lr, float eps, const int32_t *__restrict__ unique_slots,
-    T *__restrict__ cache_rows) {
+    T *__restrict__ cache_rows, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -242,7 +242,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
       }
     }
     apply_update<T, VEC, CHUNKS, OPT, true>(wrow, w_old, G, state ? state + key : nullptr, lr, eps,
-                                            chunks, group_base, c);
+                                            chunks, group_base, c, sr, static_cast<int64_t>(key) * D + col);
   }
 }
 
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ counters,
     const ChunkRecord *__restrict__ chunk_records,
     typename AccOf<T>::type *__restrict__ partial_sums, int D, int chunks_rt, float lr, float eps,
-    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows) {
+    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
         for (int i = 0; i < VEC; ++i) dst[i] = G.v[i];
       } else {
         apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, lr,
-                                          eps, chunks, 0, c);
+                                          eps, chunks, 0, c, sr, static_cast<int64_t>(rec.key) * D + col);
       }
     }
   }
@@ -371,7 +371,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     T *__restrict__ weights, typename AccOf<T>::type *__restrict__ state,
     const int32_t *__restrict__ counters, const LongRecord *__restrict__ long_records,
     const typename AccOf<T>::type *__restrict__ partial_sums, int D, int chunks_rt, float lr,
-    float eps, const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows) {
+    float eps, const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows,
+    StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
 
@@ -400,7 +401,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
       for (int i = 0; i < VEC; ++i) G.v[i] += src[i];
     }
     apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, lr, eps,
-                                      chunks, group_base, c);
+                                      chunks, group_base, c, sr, static_cast<int64_t>(rec.key) * D + col);
   }
 }
 
@@ -417,7 +418,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_wide_kernel(
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters, int D,
     int chunks, float lr, float eps, const int32_t *__restrict__ unique_slots,
-    T *__restrict__ cache_rows) {
+    T *__restrict__ cache_rows, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
 
@@ -489,7 +490,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_wide_kernel(
       w.load(wrow + static_cast<int64_t>(cb) * VEC);
 #pragma unroll
       for (int k = 0; k < VEC; ++k) w.v[k] = w.v[k] - G.v[k] * mult;
-      w.store(wrow + static_cast<int64_t>(cb) * VEC);
+      store_row<T, VEC, false>(wrow + static_cast<int64_t>(cb) * VEC, w, sr, row * D + static_cast<int64_t>(cb) * VEC);
     }
   }
 }
@@ -524,20 +525,21 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
              go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
              a.segment_starts, a.segment_ids, a.counters, long_records, chunk_records,
              a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,
-             a.unique_slots, cr);
+             a.unique_slots, cr, a.stochastic_rounding);
 
   const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
   const dim3 grid_chunks(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_chunks, 256 * 8))));
   TBE_LAUNCH("update_chunks", stream,
              (update_chunks_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kLongUnroll>), grid_chunks, block,
              go, w, st, psw, gpsw, a.positions_sorted, a.grad_rows, a.counters, chunk_records,
-             partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr);
+             partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr,
+             a.stochastic_rounding);
 
   const int64_t want_long = ceil_div(ceil_div(a.max_long, groups), kWavesPerBlock);
   const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
   TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, OPT>),
              grid_finish, block, w, st, a.counters, long_records, partial, a.D, g.chunks,
-             a.learning_rate, a.eps, a.unique_slots, cr);
+             a.learning_rate, a.eps, a.unique_slots, cr, a.stochastic_rounding);
 }
 
 template <typename T, int VEC, int OPT, bool WEIGHTED>
@@ -552,7 +554,7 @@ void launch_geometry(const UpdateArgs &a, const RowGeometry &g, hipStream_t stre
                static_cast<const T *>(a.per_sample_weights),
                static_cast<T *>(a.grad_per_sample_weights), a.keys_sorted, a.positions_sorted,
                a.grad_rows, a.segment_starts, a.counters, a.D, g.chunks, a.learning_rate, a.eps,
-               a.unique_slots, static_cast<T *>(a.cache_rows));
+               a.unique_slots, static_cast<T *>(a.cache_rows), a.stochastic_rounding);
     return;
   }
   switch (g.tmpl) {

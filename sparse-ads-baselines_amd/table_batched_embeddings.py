@@ -52,6 +52,16 @@ def _check_common(weights, table_offsets, indices, offsets):
     return T, B
 
 
+def _rounding_stream(device):
+    """(seed, offset) for one stochastically rounded backward call, taken from PyTorch's
+    generator of `device` the way the reference reserves Philox offsets
+    (table_batched_embeddings_cuda.cu:1685-1691); every call gets a fresh offset."""
+    gen = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
+    seed, offset = gen.initial_seed(), gen.get_offset()
+    gen.set_offset(offset + 4)
+    return seed & 0xFFFFFFFFFFFFFFFF, offset
+
+
 def _workspace(device, nbytes):
     ws = _workspaces.get(device)
     if ws is None or ws.numel() < nbytes:
@@ -120,8 +130,6 @@ def backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets
     The weighted case, which the reference asserts out (:1678-1679), is served."""
     T, B = _check_common(weights, table_offsets, indices, offsets)
     _require(BT_block_size > 0, "BT_block_size must be positive")
-    if stochastic_rounding:
-        raise NotImplementedError("stochastic rounding is not implemented")
     grad_output = _check_grad(grad_output, weights, T, B)
     D = weights.size(1)
     code = _DTYPE_CODES[weights.dtype]
@@ -139,11 +147,19 @@ def backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets
     layout = _native.backward_workspace_layout(indices.numel(), D, code)
     ws = _workspace(weights.device, layout.total_bytes)
     with torch.cuda.device(weights.device):
-        _native.check(_native.load().tbe_backward_exact_adagrad(
-            _ptr(grad_output), _ptr(weights), code, weights.size(0), D, _ptr(table_offsets), T,
-            _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state),
-            float(learning_rate), float(eps), _ptr(grad_indice_weights), _ptr(ws), ws.numel(),
-            _stream(weights.device)))
+        if stochastic_rounding and weights.dtype == torch.float16:
+            seed, offset = _rounding_stream(weights.device)
+            _native.check(_native.load().tbe_backward_exact_adagrad_stochastic(
+                _ptr(grad_output), _ptr(weights), code, weights.size(0), D, _ptr(table_offsets), T,
+                _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state),
+                float(learning_rate), float(eps), _ptr(grad_indice_weights), seed, offset, _ptr(ws), ws.numel(),
+                _stream(weights.device)))
+        else:  # rounding to nearest; stochastic rounding only exists for fp16 (tbe.cu:557-578)
+            _native.check(_native.load().tbe_backward_exact_adagrad(
+                _ptr(grad_output), _ptr(weights), code, weights.size(0), D, _ptr(table_offsets), T,
+                _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state),
+                float(learning_rate), float(eps), _ptr(grad_indice_weights), _ptr(ws), ws.numel(),
+                _stream(weights.device)))
     return grad_indice_weights
 
 
@@ -214,8 +230,6 @@ def forward_mixed_D(weights, table_offsets, dim_offsets, total_D, indices, offse
 def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, total_D, indices,
                     offsets, indice_weights, optimizer_state, learning_rate, eps, stochastic_rounding):
     T, B = _check_mixed(weights, table_offsets, dim_offsets, indices, offsets)
-    if stochastic_rounding:
-        raise NotImplementedError("stochastic rounding is not implemented")
     _require(table_dim_offsets.dtype == torch.int32 and table_dim_offsets.numel() == T + 1,
              "table_dim_offsets must be int32 with T+1 entries")
     _require(grad_output.dtype == weights.dtype and tuple(grad_output.shape) == (B, int(total_D)),
@@ -234,12 +248,15 @@ def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_of
              "optimizer_state must be contiguous %s" % state_dtype)
     layout = _native.backward_workspace_layout(indices.numel(), 4, code)
     ws = _workspace(weights.device, layout.total_bytes)
+    stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
+    seed, offset = _rounding_stream(weights.device) if stochastic else (0, 0)
     with torch.cuda.device(weights.device):
         _native.check(_native.load().tbe_backward_mixed(
             optimizer, _ptr(grad_output), _ptr(weights), code, _fp16_vector_width(dim_offsets), total_rows,
             _ptr(table_offsets), _ptr(table_dim_offsets), _ptr(dim_offsets), int(total_D), T, _ptr(indices),
             indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state), float(learning_rate),
-            float(eps or 0.0), _ptr(grad_indice_weights), _ptr(ws), ws.numel(), _stream(weights.device)))
+            float(eps or 0.0), _ptr(grad_indice_weights), int(stochastic), seed, offset, _ptr(ws), ws.numel(),
+            _stream(weights.device)))
     return grad_indice_weights
 
 

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -93,7 +93,11 @@ SIGNATURES = {
     "tbe_forward_mixed": (ctypes.c_int, [_vp, _i32, _i32, _vp, _c_i32p, _i32, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp,
                                          _vp, _vp]),
     "tbe_backward_mixed": (ctypes.c_int, [_i32, _vp, _vp, _i32, _i32, _i64, _vp, _c_i32p, _c_i32p, _i32, _i32,
-                                          _c_i32p, _i64, _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _vp, _u64, _vp]),
+                                          _c_i32p, _i64, _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _i32, _u64, _u64,
+                                          _vp, _u64, _vp]),
+    "tbe_backward_exact_adagrad_stochastic": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p,
+                                                             _i64, _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _u64,
+                                                             _u64, _vp, _u64, _vp]),
     "tbe_cache_workspace_layout": (ctypes.c_int, [_i64, _i64, ctypes.POINTER(CacheWorkspaceLayout)]),
     "tbe_cache_init": (ctypes.c_int, [_cache_p, _vp]),
     "tbe_cache_prepare": (ctypes.c_int, [_cache_p, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32,

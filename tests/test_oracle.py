@@ -377,3 +377,53 @@ def test_mixed_dim_with_equal_dims_equals_uniform_path(oracle):
     oracle.backward("sgd", p["grad_output"].reshape(9, 3, 16), w2, p["table_dim_offsets"][:-1], p["indices"],
                     p["offsets"], 0.1)
     assert w1.tobytes() == w2.tobytes()
+
+
+# -------------------------------------------------------- stochastic rounding
+def test_philox_known_answers(oracle):
+    """Known-answer vectors of Philox4x32-10 from the Random123 distribution (kat_vectors)."""
+    assert oracle.philox4x32_10([0, 0, 0, 0], [0, 0]) == [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]
+    assert oracle.philox4x32_10([0xffffffff] * 4, [0xffffffff] * 2) == [0x408f276d, 0x41c83b0e, 0xa20bc7c6,
+                                                                         0x6d5451fd]
+    assert oracle.philox4x32_10([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0]) == \
+        [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]
+
+
+def test_stochastic_round_rule(oracle):
+    """stochastic_rounding_vector (tbe.cu:569-576): add the top 13 random bits to the fp32
+    pattern, truncate toward zero.  Values representable in fp16 never move; others land on one
+    of their two fp16 neighbours with probability proportional to proximity (unbiased)."""
+    half = lambda bits: float(np.array([bits], np.uint16).view(np.float16)[0])
+    for x in (0.0, 1.0, -2.5, 0.000123, 65504.0, 6.1035e-05):
+        exact = float(np.float16(x))
+        for r in (0, 1 << 19, 0xffffffff, 0x80000000):
+            assert half(oracle.stochastic_round(exact, r)) == exact
+    x = 1.0 + 0.3 * 2.0 ** -10                                    # 30 % of the way from 1.0 to its successor
+    lo, hi = 1.0, 1.0 + 2.0 ** -10
+    rs = np.random.RandomState(0)
+    draws = np.array([half(oracle.stochastic_round(x, int(r))) for r in rs.randint(0, 2 ** 32, size=20000,
+                                                                                      dtype=np.uint64)])
+    assert set(np.unique(draws)) == {lo, hi}
+    assert abs(draws.mean() - np.float32(x)) < 3e-6             # unbiased: 0.3 +- 0.01 of the draws go up
+    assert abs((draws == hi).mean() - 0.3) < 0.01
+    assert half(oracle.stochastic_round(x, 0)) == lo and half(oracle.stochastic_round(x, 0xffffffff)) == hi
+    # negative values move away from zero with the same rule
+    assert half(oracle.stochastic_round(-x, 0)) == -lo and half(oracle.stochastic_round(-x, 0xffffffff)) == -hi
+
+
+def test_stochastic_backward_is_within_one_ulp_and_reproducible(oracle):
+    p = make_problem(31, T=2, E=40, D=16, B=30, L=6, dtype=np.float16, zipf=1.3)
+    runs = []
+    for stream in ((7, 0), (7, 0), (7, 4), None):
+        w = p["weights"].copy()
+        st = np.zeros(80, np.float32)
+        oracle.backward("adagrad", p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], 0.05, 0.1, st,
+                        stochastic_rounding=stream)
+        runs.append(w)
+    same_a, same_b, other, nearest = runs
+    assert same_a.tobytes() == same_b.tobytes()                  # same (seed, offset) -> same bits
+    assert same_a.tobytes() != other.tobytes()                   # another offset -> another draw
+    ulp = np.abs(np.spacing(nearest.astype(np.float16))).astype(np.float32)
+    assert (np.abs(same_a.astype(np.float32) - nearest.astype(np.float32)) <= ulp).all()
+    untouched = np.setdiff1d(np.arange(80), oracle.linearize(p["table_offsets"], p["indices"], p["offsets"])[0])
+    assert same_a[untouched].tobytes() == p["weights"][untouched].tobytes()
