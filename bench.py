@@ -325,6 +325,21 @@ def main():
         ws = ext.backward_workspace(dev)
         U = int(ws[lay.num_unique:lay.num_unique + 4].view(torch.int32)[0])
     a_fwd, a_bwd, a_update = algorithmic_bytes(w, U)
+    # The update is split over two kernels by segment length: rows with at most 16 occurrences go
+    # to update_short, the others to update_chunks.  Each kernel is credited with the gradient rows
+    # it gathers and the weight rows it reads and writes.
+    short_share = {"lookups": w["n"], "rows": U}
+    if w["optimizer"] and U:
+        starts = ws[lay.segment_starts:lay.segment_starts + 4 * (U + 1)].view(torch.int32).long()
+        lengths = starts[1:] - starts[:-1]
+        short = lengths <= 16
+        short_share = {"lookups": int(lengths[short].sum()), "rows": int(short.sum())}
+    S = 2 if w["fp16"] else 4
+    extra_per_row = 8 if w["optimizer"] == "adagrad" else 0
+    extra_per_lookup = 2 * S if w["weighted"] else 0
+    a_update_short = (short_share["lookups"] * (D * S + extra_per_lookup) +
+                      short_share["rows"] * (2 * D * S + extra_per_row))
+    a_update_chunks = a_update - a_update_short
 
     # per-kernel durations from HIP events recorded by the library on the launch stream
     per_kernel = {}
@@ -336,7 +351,7 @@ def main():
             per_kernel.setdefault(name, []).append(ms)
     kernels = {k: {"launches_per_step": len(v) / max(args.profile_steps, 1), "avg_us": 1e3 * sum(v) / len(v)}
                for k, v in per_kernel.items()}
-    kernel_bytes = {"forward": a_fwd, "update_short": a_update}
+    kernel_bytes = {"forward": a_fwd, "update_short": a_update_short, "update_chunks": a_update_chunks}
     roofline = None
     if kernels:
         dominant = max((k for k in kernels if k in kernel_bytes and kernel_bytes[k]),
@@ -365,7 +380,9 @@ def main():
                    "unique_rows": U, "seed": w["seed"]},
         "effective_GBps": (a_fwd + a_bwd) / (elapsed / args.steps) / 1e9,
         "effective_frac_of_hbm_peak": (a_fwd + a_bwd) / (elapsed / args.steps) / HBM_PEAK,
-        "algorithmic_bytes": {"forward": a_fwd, "backward": a_bwd},
+        "algorithmic_bytes": {"forward": a_fwd, "backward": a_bwd, "update_short": a_update_short,
+                              "update_chunks": a_update_chunks,
+                              "short_segments": short_share},
         "roofline": roofline,
         "kernels": kernels,
     }

@@ -338,6 +338,17 @@ TBE_API int tbe_backward_cached(int32_t optimizer, const void *grad_output, cons
 /* Writes every resident row back to the backing table (the cache stays valid). */
 TBE_API int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t D, void *stream);
 
+/* ------------------------------------------------- interleaved [E][T][D] tables
+ * The older sparse_embedding_cuda kernels keep all tables in one [E][T][D] array and number
+ * bags bag-major, b*T + t (sparse_embedding_cuda_kernel.cu:221-284, 349-379).  Viewed as an
+ * [E*T][D] matrix this is a single table whose row for (ind, t) is ind*T + t; this entry point
+ * writes those row numbers, after which tbe_forward / tbe_backward_sgd run with T = 1,
+ * B = (real B)*(real T), table_offsets = {0}: output [B*T][1][D] is the [B][T][D] layout.
+ * `offsets` is the flattened [B*T+1] array of bag starts.
+ */
+TBE_API int tbe_interleaved_rows(const int32_t *indices, int64_t num_indices, const int32_t *offsets,
+                                 int32_t T, int32_t B, int32_t *rows, void *stream);
+
 /* ------------------------------------------------------ host-resident tables
  * Pinned, device-mapped host memory (new_host_mapped_tensor,
  * table_batched_embeddings_cuda.cu:820-880) and managed memory preferring the

@@ -532,3 +532,41 @@ int oracle_backward_mixed(int optimizer, const void *grad_output, void *weights,
   free(keys); free(b_ts); free(pos); free(keys_s); free(pos_s); free(seg);
   return 0;
 }
+
+/* ================================================== interleaved [E][T][D] tables
+ * The older kernels: sparse_embedding_cuda_forward_offsets_kernel_impl
+ * (sparse_embedding_cuda_kernel.cu:221-284; the dense variant :349-379 is the special case of
+ * equal bag lengths) and the fused update (:464-499), the latter made exact: each distinct
+ * (row, table) gets -lr * (sum of its bags' gradients) once.  fp32 only (what the tests use).
+ * offsets is the flattened [B*T+1] array, bag (b,t) = offsets[b*T+t] .. offsets[b*T+t+1].
+ */
+void oracle_forward_etd(const float *weights, int32_t E, int32_t T, int32_t D, const int32_t *indices,
+                        const int32_t *offsets, int32_t B, float *output) {
+  (void)E;
+  for (int32_t b = 0; b < B; ++b)
+    for (int32_t t = 0; t < T; ++t)
+      for (int32_t d = 0; d < D; ++d) {
+        float sum = 0.0f;
+        for (int32_t l = offsets[b * T + t]; l < offsets[b * T + t + 1]; ++l)
+          sum += weights[((int64_t)indices[l] * T + t) * D + d];
+        output[((int64_t)b * T + t) * D + d] = sum;
+      }
+}
+
+void oracle_backward_etd(const float *grad_output, float *weights, int32_t E, int32_t T, int32_t D,
+                         const int32_t *indices, const int32_t *offsets, int32_t B, float lr) {
+  float *G = (float *)calloc((size_t)E * T * D, sizeof(float));
+  uint8_t *hit = (uint8_t *)calloc((size_t)E * T, 1);
+  for (int32_t b = 0; b < B; ++b)
+    for (int32_t t = 0; t < T; ++t)
+      for (int32_t l = offsets[b * T + t]; l < offsets[b * T + t + 1]; ++l) {
+        const int64_t row = (int64_t)indices[l] * T + t;
+        hit[row] = 1;
+        for (int32_t d = 0; d < D; ++d) G[row * D + d] += grad_output[((int64_t)b * T + t) * D + d];
+      }
+  for (int64_t row = 0; row < (int64_t)E * T; ++row)
+    if (hit[row])
+      for (int32_t d = 0; d < D; ++d) weights[row * D + d] -= G[row * D + d] * lr;
+  free(G);
+  free(hit);
+}

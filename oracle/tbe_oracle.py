@@ -234,3 +234,27 @@ def stochastic_round(value, random_bits):
     fn.restype = ctypes.c_uint16
     fn.argtypes = [ctypes.c_float, ctypes.c_uint32]
     return fn(float(value), int(random_bits))
+
+
+# ------------------------------------------------------ interleaved [E][T][D] tables
+def forward_etd(weights, indices, offsets):
+    """weights float32 [E, T, D]; offsets flattened [B*T+1] -> output [B, T, D]."""
+    weights = np.ascontiguousarray(weights, dtype=np.float32)
+    E, T, D = weights.shape
+    indices, offsets = _i32(indices), _i32(offsets)
+    B = (offsets.size - 1) // T
+    out = np.empty((B, T, D), np.float32)
+    lib().oracle_forward_etd(_p(weights), ctypes.c_int32(E), ctypes.c_int32(T), ctypes.c_int32(D), _p(indices),
+                             _p(offsets), ctypes.c_int32(B), _p(out))
+    return out
+
+
+def backward_etd(grad_output, weights, indices, offsets, lr):
+    """In-place exact SGD on weights float32 [E, T, D]."""
+    assert weights.dtype == np.float32 and weights.flags["C_CONTIGUOUS"]
+    E, T, D = weights.shape
+    indices, offsets = _i32(indices), _i32(offsets)
+    B = (offsets.size - 1) // T
+    grad_output = np.ascontiguousarray(grad_output, dtype=np.float32)
+    lib().oracle_backward_etd(_p(grad_output), _p(weights), ctypes.c_int32(E), ctypes.c_int32(T), ctypes.c_int32(D),
+                              _p(indices), _p(offsets), ctypes.c_int32(B), ctypes.c_float(lr))

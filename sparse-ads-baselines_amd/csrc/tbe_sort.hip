@@ -83,6 +83,22 @@ __global__ __launch_bounds__(kBlockThreads) void linearize_kernel(
   }
 }
 
+// Row numbers for tables stored interleaved, weights[row][table][D] (the layout of the older
+// sparse_embedding_cuda kernels, sparse_embedding_cuda_kernel.cu:349-379: weights[ind][t][d]).
+// Viewed as a [E*T][D] matrix, row `ind` of table t is matrix row ind*T + t; bags are numbered
+// bag-major (b*T + t), so the table of a bag is bag % T.
+__global__ __launch_bounds__(kBlockThreads) void interleaved_rows_kernel(
+    const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets, int num_tables,
+    int num_bags, int32_t *__restrict__ rows) {
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t bag = gid / kLinLanes;
+  if (bag >= num_bags) return;
+  const int t = static_cast<int>(bag % num_tables);
+  const int end = offsets[bag + 1];
+  for (int p = offsets[bag] + static_cast<int>(gid % kLinLanes); p < end; p += kLinLanes)
+    rows[p] = indices[p] * num_tables + t;
+}
+
 // ------------------------------------------------------------------ radix sort
 __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     const uint32_t *__restrict__ keys, int64_t n, int shift, uint32_t mask, int num_tiles,
@@ -390,6 +406,24 @@ extern "C" int tbe_linearize(const int32_t *table_offsets, int32_t T, const int3
   TBE_REQUIRE(indices && keys && grad_rows, "tbe_linearize: null pointer argument");
   return linearize(table_offsets, T, indices, offsets, B, keys, grad_rows,
                    static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tbe_interleaved_rows(const int32_t *indices, int64_t num_indices,
+                                    const int32_t *offsets, int32_t T, int32_t B, int32_t *rows,
+                                    void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(T > 0 && B > 0, "tbe_interleaved_rows: T and B must be positive (got %d, %d)", T, B);
+  TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "tbe_interleaved_rows: T*B out of range");
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "tbe_interleaved_rows: num_indices out of range");
+  TBE_REQUIRE(offsets, "tbe_interleaved_rows: null offsets");
+  if (num_indices == 0) return TBE_OK;
+  TBE_REQUIRE(indices && rows, "tbe_interleaved_rows: null pointer argument");
+  const int64_t num_bags = static_cast<int64_t>(T) * B;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  TBE_LAUNCH("interleaved_rows", s, interleaved_rows_kernel,
+             dim3(static_cast<unsigned>(ceil_div(num_bags * kLinLanes, kBlockThreads))), dim3(kBlockThreads),
+             indices, offsets, T, static_cast<int>(num_bags), rows);
+  return check_launch("tbe_interleaved_rows");
 }
 
 extern "C" uint64_t tbe_sort_workspace_bytes(int64_t n) { return tbe::sort_workspace_bytes(n); }

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -85,6 +85,7 @@ SIGNATURES = {
     "tbe_backward_exact_adagrad": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
                                                   _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _vp, _u64, _vp]),
     "tbe_linearize": (ctypes.c_int, [_c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _c_i32p, _c_i32p, _vp]),
+    "tbe_interleaved_rows": (ctypes.c_int, [_c_i32p, _i64, _c_i32p, _i32, _i32, _c_i32p, _vp]),
     "tbe_sort_workspace_bytes": (_u64, [_i64]),
     "tbe_sort_pairs": (ctypes.c_int, [_c_i32p, _c_i32p, _c_i32p, _c_i32p, _i64, _i32, _vp, _u64, _vp]),
     "tbe_segments_workspace_bytes": (_u64, [_i64]),

@@ -1,0 +1,63 @@
+"""GPU parity of the interleaved [E][T][D] layout (the older sparse_embedding_cuda interface)
+against the CPU oracle, through the module mirror as in test_sparse_embedding_cuda.py:12-135."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import DEV, assert_close, dev
+
+import sparse_embedding_cuda as se
+import sparse_embedding_cuda_ops as se_ops
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("E,T,D,B,L", [(1000, 4, 32, 16, 7), (50, 1, 4, 3, 2), (300, 3, 128, 33, 20),
+                                       (64, 5, 12, 9, 4)])
+def test_dense_and_offsets_variants_match_oracle(oracle, E, T, D, B, L):
+    rs = np.random.RandomState(E + T)
+    weights = rs.randn(E, T, D).astype(np.float32)
+    dense = (rs.zipf(1.2, size=(B, T, L)) % E).astype(np.int32)
+    offsets = np.arange(0, B * T * L + 1, L, dtype=np.int32)
+    go = rs.randn(B, T, D).astype(np.float32)
+    want = oracle.forward_etd(weights, dense.reshape(-1), offsets)
+    w_ref = weights.copy()
+    oracle.backward_etd(go, w_ref, dense.reshape(-1), offsets, 0.05)
+
+    cc = se_ops.UniformShardedEmbeddingBags(T, E, D).cuda()
+    cc.embedding_weights.data.copy_(dev(weights))
+    out = cc(dev(dense))
+    assert tuple(out.shape) == (B, T, D)
+    assert_close(out.detach().cpu().numpy(), want, 1e-5)
+    out.backward(dev(go))
+    assert_close(cc.embedding_weights.detach().cpu().numpy(), w_ref, 1e-5)
+
+    # merged offsets [B][T+1] as get_merged_offsets_from_dense builds them (:61-72)
+    merged = np.fromfunction(lambda b, t: (b * T + t) * L, (B, T + 1), dtype=np.int32).astype(np.int32)
+    cc2 = se_ops.UniformShardedEmbeddingBags(T, E, D).cuda()
+    cc2.embedding_weights.data.copy_(dev(weights))
+    out2 = cc2(dev(dense.reshape(-1)), dev(merged))
+    assert torch.equal(out2, out)
+    out2.backward(dev(go))
+    assert torch.equal(cc2.embedding_weights, cc.embedding_weights)
+
+
+def test_ragged_offsets_and_function_level_calls(oracle):
+    rs = np.random.RandomState(2)
+    E, T, D, B = 200, 3, 64, 11
+    weights = rs.randn(E, T, D).astype(np.float32)
+    lengths = rs.randint(0, 9, size=B * T)
+    flat = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    indices = (rs.zipf(1.3, size=int(flat[-1])) % E).astype(np.int32)
+    merged = np.stack([flat[b * T:b * T + T + 1] for b in range(B)]).astype(np.int32)
+    go = rs.randn(B, T, D).astype(np.float32)
+    w = dev(weights)
+    got = se.forward_offsets(w, dev(indices), dev(merged))
+    assert_close(got.cpu().numpy(), oracle.forward_etd(weights, indices, flat), 1e-5)
+    se.backward_update_offsets(dev(go), w, dev(indices), dev(merged), 0.1)
+    w_ref = weights.copy()
+    oracle.backward_etd(go, w_ref, indices, flat, 0.1)
+    torch.cuda.synchronize()
+    assert_close(w.cpu().numpy(), w_ref, 1e-5)
+    with pytest.raises(NotImplementedError):
+        se.forward_all2all(w, w)

@@ -427,3 +427,31 @@ def test_stochastic_backward_is_within_one_ulp_and_reproducible(oracle):
     assert (np.abs(same_a.astype(np.float32) - nearest.astype(np.float32)) <= ulp).all()
     untouched = np.setdiff1d(np.arange(80), oracle.linearize(p["table_offsets"], p["indices"], p["offsets"])[0])
     assert same_a[untouched].tobytes() == p["weights"][untouched].tobytes()
+
+
+# ------------------------------------------------------ interleaved [E][T][D] tables
+def test_interleaved_layout_matches_embeddingbag(oracle):
+    """The check of test_sparse_embedding_cuda.py:12-135: per table torch.nn.EmbeddingBag on
+    weights[:, t, :], forward and w - lr * grad (with repeated rows, exact)."""
+    torch = pytest.importorskip("torch")
+    rs = np.random.RandomState(33)
+    E, T, D, B, L = 50, 3, 8, 9, 5
+    weights = rs.randn(E, T, D).astype(np.float32)
+    lengths = rs.randint(0, L + 1, size=B * T)
+    offsets = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    indices = (rs.zipf(1.3, size=int(offsets[-1])) % E).astype(np.int32)
+    go = rs.randn(B, T, D).astype(np.float32)
+    out = oracle.forward_etd(weights, indices, offsets)
+    w = weights.copy()
+    oracle.backward_etd(go, w, indices, offsets, 0.05)
+    for t in range(T):
+        bag = torch.nn.EmbeddingBag(E, D, mode="sum", sparse=True)
+        bag.weight.data.copy_(torch.from_numpy(weights[:, t, :].copy()))
+        sel = [np.arange(offsets[b * T + t], offsets[b * T + t + 1]) for b in range(B)]
+        idx_t = torch.from_numpy(indices[np.concatenate(sel)].astype(np.int64))
+        off_t = torch.from_numpy(np.concatenate([[0], np.cumsum([len(s) for s in sel])[:-1]]).astype(np.int64))
+        y = bag(idx_t, off_t)
+        np.testing.assert_allclose(out[:, t, :], y.detach().numpy(), rtol=1e-5, atol=1e-6)
+        y.backward(torch.from_numpy(go[:, t, :].copy()))
+        want = bag.weight.detach() - bag.weight.grad.to_dense() * 0.05
+        np.testing.assert_allclose(w[:, t, :], want.numpy(), rtol=1e-5, atol=1e-6)
