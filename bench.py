@@ -33,8 +33,10 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 # this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
 # reads for a plain 1 GiB device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Keyed by (kernel, config).
 MEASURED_TRAFFIC = {
-    ("update_short", 3): int((1901850.8 * 2.0 + 1283608.9) * 1024),
-    ("forward", 3): int((836316.6 * 2.0 + 131072.0) * 1024),
+    ("update_short", 3): int((1274951.8 * 2.0 + 1278122.7) * 1024),
+    ("update_chunks", 3): int((390560.0 * 2.0 + 8343.4) * 1024),
+    ("forward", 3): int((836363.5 * 2.0 + 131072.0) * 1024),
+    ("forward", 2): int((1227779.4 * 2.0 + 131072.0) * 1024),
 }
 
 

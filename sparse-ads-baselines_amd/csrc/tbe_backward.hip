@@ -71,7 +71,7 @@ int build_plan(const tbe_workspace_layout_t &l, void *workspace, const int32_t *
   return find_segments(keys_sorted, n, reinterpret_cast<int32_t *>(ws + l.segment_starts),
                        reinterpret_cast<int32_t *>(ws + l.num_unique),
                        reinterpret_cast<int32_t *>(ws + l.segment_ids), ws + l.segment_scratch,
-                       stream);
+                       stream, /*clear_queue_counters=*/true);
 }
 
 namespace {

@@ -272,7 +272,7 @@ __global__ __launch_bounds__(kBlockThreads) void segment_count_kernel(
 // the closing boundary segment_starts[U] = n.
 __global__ __launch_bounds__(kBlockThreads) void segment_scan_kernel(
     uint32_t *__restrict__ tile_heads, int num_tiles, int64_t n,
-    int32_t *__restrict__ segment_starts, int32_t *__restrict__ num_unique) {
+    int32_t *__restrict__ segment_starts, int32_t *__restrict__ num_unique, int clear_queue_counters) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   const int tid = threadIdx.x;
   uint32_t carry = 0;
@@ -289,6 +289,8 @@ __global__ __launch_bounds__(kBlockThreads) void segment_scan_kernel(
     num_unique[0] = static_cast<int32_t>(carry);
     segment_starts[carry] = static_cast<int32_t>(n);
   }
+  // the update stage keeps three queue counters next to U; starting them at zero here saves a launch
+  if (clear_queue_counters && tid >= 1 && tid <= 3) num_unique[tid] = 0;
 }
 
 __global__ __launch_bounds__(kBlockThreads) void segment_write_kernel(
@@ -366,7 +368,8 @@ uint64_t segments_workspace_bytes(int64_t n) {
 }
 
 int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts,
-                  int32_t *num_unique, int32_t *segment_ids, void *workspace, hipStream_t stream) {
+                  int32_t *num_unique, int32_t *segment_ids, void *workspace, hipStream_t stream,
+                  bool clear_queue_counters) {
   const int tiles = n > 0 ? num_seg_tiles(n) : 0;
   uint32_t *tile_heads = static_cast<uint32_t *>(workspace);
   const uint32_t *keys = reinterpret_cast<const uint32_t *>(keys_sorted);
@@ -375,7 +378,7 @@ int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts
     TBE_LAUNCH("segment_count", stream, segment_count_kernel, dim3(tiles), block, keys, n,
                tile_heads);
   TBE_LAUNCH("segment_scan", stream, segment_scan_kernel, dim3(1), block, tile_heads, tiles, n,
-             segment_starts, num_unique);
+             segment_starts, num_unique, clear_queue_counters ? 1 : 0);
   if (tiles > 0)
     TBE_LAUNCH("segment_write", stream, segment_write_kernel, dim3(tiles), block, keys, n,
                tile_heads, segment_starts, segment_ids);
@@ -456,5 +459,5 @@ extern "C" int tbe_find_segments(const int32_t *keys_sorted, int64_t n, int32_t 
     return fail(TBE_ERR_WORKSPACE, "tbe_find_segments: workspace of %llu bytes needed, %llu given",
                 (unsigned long long)segments_workspace_bytes(n), (unsigned long long)workspace_bytes);
   return find_segments(keys_sorted, n, segment_starts, num_unique, nullptr, workspace,
-                       static_cast<hipStream_t>(stream));
+                       static_cast<hipStream_t>(stream), /*clear_queue_counters=*/false);
 }

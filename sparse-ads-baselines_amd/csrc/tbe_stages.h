@@ -17,8 +17,11 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
 
 uint64_t segments_workspace_bytes(int64_t n);
 // segment_ids (nullable): receives, for every sorted position, the index of its segment.
+// clear_queue_counters: num_unique points at the 4-word counter block of a backward workspace;
+// words 1..3 (the update stage's queue counters) are set to zero as well.
 int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts,
-                  int32_t *num_unique, int32_t *segment_ids, void *workspace, hipStream_t stream);
+                  int32_t *num_unique, int32_t *segment_ids, void *workspace, hipStream_t stream,
+                  bool clear_queue_counters = false);
 
 // Segments of more than kShortSegment occurrences leave the lane-group path and are reduced by
 // whole wavefronts in chunks of at most kChunkLen occurrences.

@@ -79,7 +79,7 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 }
 
 // ------------------------------------------------------------ short segments
-// Work is cut by sorted position, not by segment: a wavefront takes a tile of kTilePositions
+// Work is cut by sorted position, not by segment: a wavefront takes a tile of tile_positions()
 // consecutive sorted positions and owns every segment that STARTS inside it, so each tile costs
 // about the same however skewed the keys are.  The tile's bookkeeping is fetched 64 wide into
 // LDS (segment bounds, keys, and the gradient row of every occurrence; positions too when
@@ -87,8 +87,11 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 // group r walks segments r, r + groups, ...  Segments longer than kShortSegment are not
 // reduced here: the owning group appends chunk records (at most kChunkLen occurrences each)
 // to a queue that update_chunks_kernel drains with one wavefront per chunk.
-constexpr int kTilePositions = 64;
-constexpr int kStageCap = kTilePositions + 64;  // occurrences staged in LDS per wavefront
+// Tile size in sorted positions: 32 per lane group, so narrow rows (many groups per wavefront)
+// get larger tiles and the per-tile bookkeeping is amortised over the same number of rows.
+constexpr int tile_positions(int chunks_template) {
+  return chunks_template == 0 ? 64 : (32 * (kWave / chunks_template) > 256 ? 256 : 32 * (kWave / chunks_template));
+}
 
 struct ChunkRecord {   // 32 bytes
   int32_t begin, end;  // sorted positions [begin, end)
@@ -116,6 +119,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
   using A = typename V::A;
   using R = typename V::R;
 
+  constexpr int kTilePositions = tile_positions(CHUNKS);
+  constexpr int kStageCap = kTilePositions + 64;  // occurrences staged in LDS per wavefront
   __shared__ int32_t s_bounds[kWavesPerBlock][kTilePositions + 1];
   __shared__ int32_t s_keys[kWavesPerBlock][kTilePositions];
   __shared__ int32_t s_grow[kWavesPerBlock][kStageCap];
@@ -366,6 +371,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
 }
 
 // --------------------------------------------- long segments: combine + update
+// One wavefront per long row: lane group r adds partial rows r, r + groups, ..., the groups are
+// combined in a fixed tree and group 0 applies the update.
 template <typename T, int VEC, int CHUNKS, int OPT>
 __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     T *__restrict__ weights, typename AccOf<T>::type *__restrict__ state,
@@ -381,27 +388,51 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
   const int groups = kWave / chunks;
   const int r = lane / chunks;
   const int c = lane - r * chunks;
-  const int group_base = r * chunks;
+  const bool active = r < groups;
   const int num_long = counters[1];
   const int64_t col = static_cast<int64_t>(c) * VEC;
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock * groups;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
 
-  for (int64_t slot = (r < groups) ? wave_id * groups + r : num_long; slot < num_long;
-       slot += stride) {
+  for (int64_t slot = wave_id; slot < num_long; slot += stride) {
     const LongRecord rec = long_records[slot];
     T *wrow = resolve_row(weights, cache_rows, unique_slots, rec.u, static_cast<int64_t>(rec.key), D) + col;
     V w_old;
-    w_old.load(wrow);
+    w_old.zero();
+    if (r == 0) w_old.load(wrow);
     V G;
     G.zero();
-    for (int k = 0; k < rec.num_chunks; ++k) {
-      const A *src = partial_sums + static_cast<int64_t>(rec.first_partial + k) * D + col;
+    if (active) {
+      for (int k = r; k < rec.num_chunks; k += groups) {
+        const A *src = partial_sums + static_cast<int64_t>(rec.first_partial + k) * D + col;
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) G.v[i] += src[i];
+        for (int i = 0; i < VEC; ++i) G.v[i] += src[i];
+      }
     }
-    apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, lr, eps,
-                                      chunks, group_base, c, sr, static_cast<int64_t>(rec.key) * D + col);
+    if constexpr (CHUNKS > 0) {
+#pragma unroll
+      for (int m = kWave / 2; m >= CHUNKS; m >>= 1) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) G.v[i] += shfl_x(G.v[i], m);
+      }
+    } else {
+      int live = groups;
+      while (live > 1) {
+        const int s = (live + 1) / 2;
+        const int from = min(lane + s * chunks, kWave - 1);
+        const bool take = active && (r + s < live);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          const A o = shfl_idx(G.v[i], from);
+          if (take) G.v[i] += o;
+        }
+        live = s;
+      }
+    }
+    if (r == 0) {
+      apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, lr, eps,
+                                        chunks, 0, c, sr, static_cast<int64_t>(rec.key) * D + col);
+    }
   }
 }
 
@@ -495,10 +526,6 @@ __global__ __launch_bounds__(kBlockThreads) void update_wide_kernel(
   }
 }
 
-__global__ void zero_counters_kernel(int32_t *counters) {
-  if (threadIdx.x >= 1 && threadIdx.x <= 3) counters[threadIdx.x] = 0;
-}
-
 constexpr int kShortUnroll = 4;
 constexpr int kLongUnroll = 4;
 
@@ -517,7 +544,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   const int groups = kWave / g.chunks;
   const dim3 block(kBlockThreads);
 
-  const int64_t num_tiles = ceil_div(a.num_indices, kTilePositions);
+  const int64_t num_tiles = ceil_div(a.num_indices, tile_positions(CHUNKS));
   const int64_t tiles_per_xcd = ceil_div(ceil_div(num_tiles, kWavesPerBlock), kNumXcd);
   const dim3 grid_short(static_cast<unsigned>(tiles_per_xcd * kNumXcd));
   TBE_LAUNCH("update_short", stream,
@@ -535,7 +562,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
              partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr,
              a.stochastic_rounding);
 
-  const int64_t want_long = ceil_div(ceil_div(a.max_long, groups), kWavesPerBlock);
+  const int64_t want_long = ceil_div(a.max_long, kWavesPerBlock);
   const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
   TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, OPT>),
              grid_finish, block, w, st, a.counters, long_records, partial, a.D, g.chunks,
@@ -584,7 +611,7 @@ void launch_variant(const UpdateArgs &a, const RowGeometry &g, hipStream_t strea
 int segment_update(const UpdateArgs &a, hipStream_t stream) {
   if (a.num_indices == 0) return TBE_OK;
   const RowGeometry g = row_geometry(a.dtype, a.D);
-  TBE_LAUNCH("zero_counters", stream, zero_counters_kernel, dim3(1), dim3(kWave), a.counters);
+  // counters[1..3] were zeroed when the plan's segments were found
   switch (a.dtype) {
     case TBE_DTYPE_F32: launch_variant<float, 4>(a, g, stream); break;
     case TBE_DTYPE_F16:

@@ -78,3 +78,13 @@ def test_mixed_d_signatures_match_the_pybind_declarations():
                                 "managed"]
     for helper in ("split_embedding_weights", "split_optimizer_state", "split_output"):
         assert callable(getattr(ops.MixedDimTableBatchedEmbeddingBags, helper))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import os
+    import subprocess
+    import sys
+    from conftest import ROOT
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True,
+                         text=True, timeout=120)
+    assert out.returncode != 0 and "one GPU" in out.stderr and out.stdout.strip() == ""
