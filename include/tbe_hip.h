@@ -153,6 +153,28 @@ TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, i
                                void *grad_per_sample_weights,
                                void *workspace, uint64_t workspace_bytes, void *stream);
 
+/* The backward in two calls, so that the integer half can overlap other work.
+ * tbe_plan_batch runs the stages that depend on the indices only -- linearize, sort, run
+ * boundaries (table_batched_embeddings_cuda.cu:1618-1655 and the head test :1523-1539) -- and
+ * leaves the result in `workspace`; it may run on another stream than the forward, while the
+ * forward gathers.  tbe_backward_planned runs the gradient reduction and the optimizer
+ * (kernel :1499-1587) on that workspace once `grad_output` exists; `stream` must be ordered
+ * after the plan (e.g. by an event).  Together they equal tbe_backward_sgd /
+ * tbe_backward_exact_adagrad(_stochastic); optimizer is TBE_OPT_SGD or TBE_OPT_ROWWISE_ADAGRAD.
+ */
+TBE_API int tbe_plan_batch(const int32_t *table_offsets, int32_t T,
+                           const int32_t *indices, int64_t num_indices,
+                           const int32_t *offsets, int32_t B, int64_t total_rows,
+                           int32_t D, int32_t dtype,
+                           void *workspace, uint64_t workspace_bytes, void *stream);
+
+TBE_API int tbe_backward_planned(int32_t optimizer, const void *grad_output, void *weights, int32_t dtype,
+                                 int64_t total_rows, int32_t D, int32_t T, int32_t B, int64_t num_indices,
+                                 const void *per_sample_weights, void *optimizer_state,
+                                 float learning_rate, float eps, void *grad_per_sample_weights,
+                                 int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
+                                 void *workspace, uint64_t workspace_bytes, void *stream);
+
 /* tbe_backward_exact_adagrad with fp16 stochastic rounding of the updated weights
  * (StochasticRoundingAdaGradFunctor, table_batched_embeddings_cuda.cu:618-646, and
  * stochastic_rounding_vector, :557-578: 13 random bits added to the fp32 pattern, then

@@ -249,3 +249,47 @@ extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
                  StochasticRounding{0, 0, 0}};
   return run_backward("tbe_backward_cached", c);
 }
+
+extern "C" int tbe_plan_batch(const int32_t *table_offsets, int32_t T, const int32_t *indices,
+                              int64_t num_indices, const int32_t *offsets, int32_t B,
+                              int64_t total_rows, int32_t D, int32_t dtype, void *workspace,
+                              uint64_t workspace_bytes, void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_plan_batch";
+  TBE_REQUIRE(T > 0 && B > 0, "%s: T and B must be positive (got %d, %d)", name, T, B);
+  TBE_REQUIRE(D > 0 && D % 4 == 0, "%s: D must be a positive multiple of 4 (got %d)", name, D);
+  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
+  TBE_REQUIRE(total_rows > 0 && total_rows < INT32_MAX, "%s: total_rows out of range", name);
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "%s: T*B out of range", name);
+  TBE_REQUIRE(table_offsets && offsets && (indices || num_indices == 0), "%s: null pointer argument", name);
+  if (num_indices == 0) return TBE_OK;
+  tbe_workspace_layout_t l;
+  compute_layout(num_indices, D, dtype, &l);
+  if (!workspace || workspace_bytes < l.total_bytes)
+    return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
+                (unsigned long long)l.total_bytes, (unsigned long long)workspace_bytes);
+  return build_plan(l, workspace, table_offsets, T, indices, num_indices, offsets, B, total_rows,
+                    static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tbe_backward_planned(int32_t optimizer, const void *grad_output, void *weights,
+                                    int32_t dtype, int64_t total_rows, int32_t D, int32_t T,
+                                    int32_t B, int64_t num_indices,
+                                    const void *per_sample_weights, void *optimizer_state,
+                                    float learning_rate, float eps, void *grad_per_sample_weights,
+                                    int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
+                                    void *workspace, uint64_t workspace_bytes, void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(optimizer == TBE_OPT_SGD || optimizer == TBE_OPT_ROWWISE_ADAGRAD,
+              "tbe_backward_planned: bad optimizer %d", optimizer);
+  TBE_REQUIRE(optimizer != TBE_OPT_SGD || !per_sample_weights,
+              "tbe_backward_planned: SGD takes no per-sample weights");
+  BackwardCall c{grad_output, weights, dtype, total_rows, D, nullptr, T, nullptr, num_indices,
+                 nullptr, B, per_sample_weights, optimizer_state, learning_rate, eps,
+                 grad_per_sample_weights, workspace, workspace_bytes,
+                 static_cast<hipStream_t>(stream),
+                 optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad, true, nullptr, nullptr,
+                 StochasticRounding{seed, offset, (stochastic_rounding && dtype == TBE_DTYPE_F16) ? 1 : 0}};
+  return run_backward("tbe_backward_planned", c);
+}

@@ -75,6 +75,65 @@ def backward_workspace(device):
     return _workspaces.get(torch.device(device))
 
 
+class BackwardPlan:
+    """The index-only half of a backward pass (keys, stable sort, run boundaries), computed
+    ahead of time on a side stream so that it overlaps the forward gather."""
+
+    _side_streams = {}
+
+    def __init__(self, weights, table_offsets, indices, offsets):
+        T, B = _check_common(weights, table_offsets, indices, offsets)
+        self.T, self.B, self.n = T, B, indices.numel()
+        self.D = weights.size(1)
+        self.code = _DTYPE_CODES[weights.dtype]
+        self.total_rows = weights.size(0)
+        self.device = weights.device
+        layout = _native.backward_workspace_layout(self.n, self.D, self.code)
+        # one buffer per call: it lives from the forward to the backward of the same step
+        self.workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=self.device)
+        side = BackwardPlan._side_streams.get(self.device)
+        if side is None:
+            side = BackwardPlan._side_streams[self.device] = torch.cuda.Stream(device=self.device)
+        # the buffer is written on the side stream: the allocator must not recycle it (e.g. when a
+        # forward is never followed by its backward) before that stream is done with it
+        self.workspace.record_stream(side)
+        for t in (table_offsets, indices, offsets):
+            t.record_stream(side)
+        main = torch.cuda.current_stream(self.device)
+        side.wait_stream(main)  # indices / offsets may still be in flight on the caller's stream
+        with torch.cuda.device(self.device):
+            _native.check(_native.load().tbe_plan_batch(
+                _ptr(table_offsets), T, _ptr(indices), self.n, _ptr(offsets), B, self.total_rows, self.D, self.code,
+                _ptr(self.workspace), self.workspace.numel(), ctypes.c_void_p(side.cuda_stream)))
+        self.ready = torch.cuda.Event()
+        self.ready.record(side)
+
+    def apply(self, optimizer, grad_output, weights, indice_weights, optimizer_state, learning_rate, eps,
+              stochastic_rounding):
+        """Gradient reduction + optimizer on the current stream, after the plan is ready."""
+        grad_output = _check_grad(grad_output, weights, self.T, self.B)
+        grad_indice_weights = None
+        if indice_weights is not None:
+            grad_indice_weights = torch.empty(self.n, dtype=grad_output.dtype, device=self.device)
+        stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
+        seed, offset = _rounding_stream(self.device) if stochastic else (0, 0)
+        torch.cuda.current_stream(self.device).wait_event(self.ready)
+        _workspaces[self.device] = self.workspace  # keep backward_workspace() pointing at the last plan
+        with torch.cuda.device(self.device):
+            _native.check(_native.load().tbe_backward_planned(
+                optimizer, _ptr(grad_output), _ptr(weights), self.code, self.total_rows, self.D, self.T, self.B,
+                self.n, _ptr(indice_weights), _ptr(optimizer_state), float(learning_rate), float(eps or 0.0),
+                _ptr(grad_indice_weights), int(stochastic), seed, offset, _ptr(self.workspace),
+                self.workspace.numel(), _stream(self.device)))
+        return grad_indice_weights
+
+
+def plan_backward(weights, table_offsets, indices, offsets):
+    """Starts the index-only half of the backward on a side stream (no counterpart in the
+    reference, which sorts inside its backward call, table_batched_embeddings_cuda.cu:1629-1655)."""
+    return BackwardPlan(weights, table_offsets, indices, offsets)
+
+
 def forward(weights, table_offsets, indices, offsets, indice_weights, L_max, BT_block_size, shmem):
     """batched_embedding_forward_cuda (table_batched_embeddings_cuda.cu:253-316).
 

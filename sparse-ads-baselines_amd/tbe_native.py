@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -84,6 +84,9 @@ SIGNATURES = {
                                         _i32, _f32, _vp, _u64, _vp]),
     "tbe_backward_exact_adagrad": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
                                                   _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _vp, _u64, _vp]),
+    "tbe_plan_batch": (ctypes.c_int, [_c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _i64, _i32, _i32, _vp, _u64, _vp]),
+    "tbe_backward_planned": (ctypes.c_int, [_i32, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _f32, _f32,
+                                            _vp, _i32, _u64, _u64, _vp, _u64, _vp]),
     "tbe_linearize": (ctypes.c_int, [_c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _c_i32p, _c_i32p, _vp]),
     "tbe_interleaved_rows": (ctypes.c_int, [_c_i32p, _i64, _c_i32p, _i32, _i32, _c_i32p, _vp]),
     "tbe_sort_workspace_bytes": (_u64, [_i64]),

@@ -334,3 +334,38 @@ def test_full_size_backward_properties():
     tbe_oracle.backward("sgd", go[:, :1, :].contiguous().cpu().numpy(), w_ref, np.zeros(1, np.int32), idx_np[:B * L],
                         offsets[:B + 1].cpu().numpy(), 0.01)
     assert_close(W[:E].cpu().numpy(), w_ref, 1e-5)
+
+
+@pytest.mark.parametrize("mode", ["sgd", "adagrad_weighted"])
+def test_plan_ahead_equals_single_call_backward(mode):
+    """tbe_plan_batch on a side stream + tbe_backward_planned give bit-identical results to the
+    one-call backward, directly and through the module with LookupFunction.plan_ahead."""
+    p = make_problem(60, T=3, E=500, D=64, B=200, L=12, dtype=np.float32, weighted=mode.endswith("weighted"),
+                     zipf=1.15)
+    optimizer = "sgd" if mode == "sgd" else "adagrad"
+    want = gpu_backward(p, optimizer, 0.05, 0.1)
+    w, go = dev(p["weights"]), dev(p["grad_output"])
+    to, idx, off = dev(p["table_offsets"]), dev(p["indices"]), dev(p["offsets"])
+    psw = dev(p["per_sample_weights"])
+    st = torch.zeros(w.shape[0], device=DEV)
+    plan = ext.plan_backward(w, to, idx, off)
+    out = ext.forward(w, to, idx, off, psw, 200, 1, False)  # the forward the plan is meant to overlap
+    code = tbe_native.OPT_SGD if optimizer == "sgd" else tbe_native.OPT_ROWWISE_ADAGRAD
+    gpsw = plan.apply(code, go, w, psw, st if optimizer != "sgd" else None, 0.05, 0.1, False)
+    torch.cuda.synchronize()
+    assert out.shape == (200, 3, 64)
+    assert w.cpu().numpy().tobytes() == want["weights"].tobytes()
+    if optimizer == "adagrad":
+        assert st.cpu().numpy().tobytes() == want["state"].tobytes()
+        assert gpsw.cpu().numpy().tobytes() == want["grad_psw"].tobytes()
+
+    ops.LookupFunction.plan_ahead = True
+    try:
+        cc = ops.TableBatchedEmbeddingBags(3, 500, 64, optimizer=ops.Optimizer.SGD if optimizer == "sgd" else
+                                           ops.Optimizer.EXACT_ROWWISE_ADAGRAD, learning_rate=0.05, eps=0.1).cuda()
+        cc.embedding_weights.data.copy_(dev(p["weights"]))
+        cc(idx, off, psw).backward(go)
+        torch.cuda.synchronize()
+        assert cc.embedding_weights.detach().cpu().numpy().tobytes() == want["weights"].tobytes()
+    finally:
+        ops.LookupFunction.plan_ahead = False
