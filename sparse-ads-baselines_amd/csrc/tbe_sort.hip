@@ -5,11 +5,12 @@
 //
 // The sort is the contract of cub::DeviceRadixSort::SortPairs as the reference
 // calls it (table_batched_embeddings_cuda.cu:1639-1655): ascending, stable,
-// key bits [0, end_bit).  Each pass is three kernels:
+// key bits [0, end_bit).  A pass handles a digit of 8 to 10 bits (the fewest passes that cover
+// end_bit).  Each pass is three kernels:
 //   histogram  per-tile digit counts (LDS atomics) -> counts[digit][tile]
 //   scan       one workgroup per digit: exclusive prefix over tiles, and the digit's total
 //   scatter    ranks each key inside its tile with wavefront ballots (all lanes
-//              holding the same digit are found with 8 ballots; the lowest lane
+//              holding the same digit are found with one ballot per digit bit; the lowest lane
 //              reserves the run in a per-wavefront LDS counter), reorders the
 //              tile in LDS so every digit's keys are contiguous, and writes
 //              them out in runs.
@@ -21,12 +22,11 @@
 namespace tbe {
 namespace {
 
-constexpr int kRadixBits = 8;
-constexpr int kBins = 1 << kRadixBits;            // 256 == kBlockThreads
+constexpr int kMaxRadixBits = 10;                 // widest digit of a pass
+constexpr int kMaxBins = 1 << kMaxRadixBits;
 constexpr int kItems = 16;                        // pairs per thread per tile
 constexpr int kTile = kBlockThreads * kItems;     // 4096
 constexpr int kWaveTile = kWave * kItems;         // 1024 pairs per wavefront
-static_assert(kBins == kBlockThreads, "one thread per digit");
 
 constexpr int kSegItems = 8;
 constexpr int kSegTile = kBlockThreads * kSegItems;  // 2048
@@ -100,12 +100,17 @@ __global__ __launch_bounds__(kBlockThreads) void interleaved_rows_kernel(
 }
 
 // ------------------------------------------------------------------ radix sort
+// BITS = digit width of the pass (8, 9 or 10): 2^BITS bins, each thread owns 2^BITS / 256
+// consecutive digits in the per-digit steps.
+template <int BITS>
 __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     const uint32_t *__restrict__ keys, int64_t n, int shift, uint32_t mask, int num_tiles,
     uint32_t *__restrict__ counts) {
-  __shared__ uint32_t s_hist[kBins];
+  constexpr int kBinsT = 1 << BITS;
+  __shared__ uint32_t s_hist[kBinsT];
   const int tid = threadIdx.x;
-  s_hist[tid] = 0;
+#pragma unroll
+  for (int d = tid; d < kBinsT; d += kBlockThreads) s_hist[d] = 0;
   __syncthreads();
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kTile;
 #pragma unroll
@@ -114,12 +119,14 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & mask], 1u);
   }
   __syncthreads();
-  counts[static_cast<int64_t>(tid) * num_tiles + blockIdx.x] = s_hist[tid];
+#pragma unroll
+  for (int d = tid; d < kBinsT; d += kBlockThreads)
+    counts[static_cast<int64_t>(d) * num_tiles + blockIdx.x] = s_hist[d];
 }
 
 // Workgroup `d` turns counts[d][0..num_tiles) into an exclusive prefix over tiles (keys with
 // digit d in earlier tiles) and publishes the row total; the scatter kernel adds the number
-// of keys with a smaller digit, which it gets from a scan of the 256 totals.
+// of keys with a smaller digit, which it gets from a scan of the digit totals.
 __global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
     uint32_t *__restrict__ counts, uint32_t *__restrict__ totals, int num_tiles) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
@@ -139,16 +146,19 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
   if (tid == 0) totals[d] = carry;
 }
 
+template <int BITS>
 __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ values_in,
     uint32_t *__restrict__ keys_out, uint32_t *__restrict__ values_out, int64_t n, int shift,
     uint32_t mask, int num_tiles, const uint32_t *__restrict__ bases,
     const uint32_t *__restrict__ totals) {
+  constexpr int kBinsT = 1 << BITS;
+  constexpr int kOwned = kBinsT / kBlockThreads;  // consecutive digits per thread
   __shared__ uint32_t s_keys[kTile];
   __shared__ uint32_t s_vals[kTile];
-  __shared__ uint32_t s_wave_count[kWavesPerBlock][kBins];
-  __shared__ uint32_t s_bin_start[kBins];
-  __shared__ uint32_t s_dest[kBins];
+  __shared__ uint32_t s_wave_count[kWavesPerBlock][kBinsT];
+  __shared__ uint32_t s_bin_start[kBinsT];
+  __shared__ uint32_t s_dest[kBinsT];
   __shared__ uint32_t s_scan[kWavesPerBlock];
 
   const int tid = threadIdx.x;
@@ -158,7 +168,9 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   const int tile_count = static_cast<int>(min(static_cast<int64_t>(kTile), n - tile_base));
 
 #pragma unroll
-  for (int w = 0; w < kWavesPerBlock; ++w) s_wave_count[w][tid] = 0;
+  for (int w = 0; w < kWavesPerBlock; ++w)
+#pragma unroll
+    for (int d = tid; d < kBinsT; d += kBlockThreads) s_wave_count[w][d] = 0;
 
   uint32_t key[kItems], val[kItems];
   const int64_t wave_base = tile_base + wave * kWaveTile;
@@ -179,7 +191,7 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t digit = (key[k] >> shift) & mask;
     unsigned long long peers = __ballot(valid);
 #pragma unroll
-    for (int bit = 0; bit < kRadixBits; ++bit) {
+    for (int bit = 0; bit < BITS; ++bit) {
       const bool set = (digit >> bit) & 1u;
       const unsigned long long vote = __ballot(set);
       peers &= set ? vote : ~vote;
@@ -195,23 +207,43 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   }
   __syncthreads();
 
-  // Thread `tid` owns digit `tid`: prefix over wavefronts, then over digits.
+  // Thread `tid` owns digits [tid * kOwned, (tid + 1) * kOwned): prefix over wavefronts, then
+  // over digits (thread-local, then across the workgroup).
   {
-    uint32_t running = 0;
+    uint32_t digit_count[kOwned];
+    uint32_t mine = 0;
 #pragma unroll
-    for (int w = 0; w < kWavesPerBlock; ++w) {
-      const uint32_t c = s_wave_count[w][tid];
-      s_wave_count[w][tid] = running;
-      running += c;
+    for (int q = 0; q < kOwned; ++q) {
+      const int d = tid * kOwned + q;
+      uint32_t running = 0;
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        const uint32_t c = s_wave_count[w][d];
+        s_wave_count[w][d] = running;
+        running += c;
+      }
+      digit_count[q] = running;
+      mine += running;
     }
     uint32_t total;
-    const uint32_t incl = block_inclusive_scan(running, s_scan, total);
-    const uint32_t bin_start = incl - running;
-    s_bin_start[tid] = bin_start;
+    uint32_t bin_start = block_inclusive_scan(mine, s_scan, total) - mine;
     __syncthreads();
-    const uint32_t digit_total = totals[tid];
-    const uint32_t smaller = block_inclusive_scan(digit_total, s_scan, total) - digit_total;
-    s_dest[tid] = smaller + bases[static_cast<int64_t>(tid) * num_tiles + blockIdx.x] - bin_start;
+    uint32_t totals_mine = 0;
+    uint32_t digit_total[kOwned];
+#pragma unroll
+    for (int q = 0; q < kOwned; ++q) {
+      digit_total[q] = totals[tid * kOwned + q];
+      totals_mine += digit_total[q];
+    }
+    uint32_t smaller = block_inclusive_scan(totals_mine, s_scan, total) - totals_mine;
+#pragma unroll
+    for (int q = 0; q < kOwned; ++q) {
+      const int d = tid * kOwned + q;
+      s_bin_start[d] = bin_start;
+      s_dest[d] = smaller + bases[static_cast<int64_t>(d) * num_tiles + blockIdx.x] - bin_start;
+      bin_start += digit_count[q];
+      smaller += digit_total[q];
+    }
   }
   __syncthreads();
 
@@ -316,20 +348,36 @@ inline int num_seg_tiles(int64_t n) { return static_cast<int>(ceil_div(n, kSegTi
 
 }  // namespace
 
-// Sort workspace: [tmp keys n][tmp values n][counts 256*tiles][totals 256*passes]
+// Sort workspace: [tmp keys n][tmp values n][counts 1024*tiles][totals 1024*passes]
 constexpr int kMaxPasses = 4;
 
 uint64_t sort_workspace_bytes(int64_t n) {
   const uint64_t tiles = num_sort_tiles(n > 0 ? n : 1);
   return align_up(static_cast<uint64_t>(n > 0 ? n : 1) * 4, 256) * 2 +
-         align_up(tiles * kBins * 4, 256) + align_up(kMaxPasses * kBins * 4, 256);
+         align_up(tiles * kMaxBins * 4, 256) + align_up(kMaxPasses * kMaxBins * 4, 256);
 }
+
+namespace {
+template <int BITS>
+void launch_radix_pass(const uint32_t *src_k, const uint32_t *src_v, uint32_t *dst_k, uint32_t *dst_v,
+                       int64_t n, int shift, uint32_t mask, int tiles, uint32_t *counts, uint32_t *totals,
+                       hipStream_t stream) {
+  const dim3 block(kBlockThreads);
+  TBE_LAUNCH("radix_histogram", stream, radix_histogram_kernel<BITS>, dim3(tiles), block, src_k, n, shift,
+             mask, tiles, counts);
+  TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, dim3(1 << BITS), block, counts, totals, tiles);
+  TBE_LAUNCH("radix_scatter", stream, radix_scatter_kernel<BITS>, dim3(tiles), block, src_k, src_v, dst_k,
+             dst_v, n, shift, mask, tiles, counts, totals);
+}
+}  // namespace
 
 int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
                int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
                hipStream_t stream) {
   if (n == 0) return TBE_OK;
-  const int passes = end_bit <= 0 ? 1 : static_cast<int>(ceil_div(end_bit, kRadixBits));
+  // Fewest passes with digits of at most 10 bits, the bits spread evenly over the passes
+  // (23 bits -> 8+8+7, 25 -> 9+8+8, 27 -> 9+9+9, 17 -> 9+8).
+  const int passes = end_bit <= 0 ? 1 : static_cast<int>(ceil_div(end_bit, kMaxRadixBits));
   const int tiles = num_sort_tiles(n);
   char *ws = static_cast<char *>(workspace);
   uint32_t *tmp_keys = reinterpret_cast<uint32_t *>(ws);
@@ -337,28 +385,29 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   uint32_t *tmp_vals = reinterpret_cast<uint32_t *>(ws);
   ws += align_up(static_cast<uint64_t>(n) * 4, 256);
   uint32_t *counts = reinterpret_cast<uint32_t *>(ws);
-  ws += align_up(static_cast<uint64_t>(tiles) * kBins * 4, 256);
+  ws += align_up(static_cast<uint64_t>(tiles) * kMaxBins * 4, 256);
   uint32_t *totals = reinterpret_cast<uint32_t *>(ws);
 
-  const dim3 block(kBlockThreads);
   const uint32_t *src_k = reinterpret_cast<const uint32_t *>(keys_in);
   const uint32_t *src_v = reinterpret_cast<const uint32_t *>(values_in);
+  int shift = 0;
   for (int pass = 0; pass < passes; ++pass) {
-    const int shift = pass * kRadixBits;
-    const int bits = end_bit <= 0 ? 0 : min(kRadixBits, end_bit - shift);
+    const int remaining = end_bit <= 0 ? 0 : end_bit - shift;
+    const int bits = static_cast<int>(ceil_div(remaining, passes - pass));
     const uint32_t mask = (1u << bits) - 1u;
     const bool to_out = ((passes - 1 - pass) % 2) == 0;
     uint32_t *dst_k = to_out ? reinterpret_cast<uint32_t *>(keys_out) : tmp_keys;
     uint32_t *dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
-    uint32_t *pass_totals = totals + pass * kBins;
-    TBE_LAUNCH("radix_histogram", stream, radix_histogram_kernel, dim3(tiles), block, src_k, n,
-               shift, mask, tiles, counts);
-    TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, dim3(kBins), block, counts, pass_totals,
-               tiles);
-    TBE_LAUNCH("radix_scatter", stream, radix_scatter_kernel, dim3(tiles), block, src_k, src_v,
-               dst_k, dst_v, n, shift, mask, tiles, counts, pass_totals);
+    uint32_t *pass_totals = totals + pass * kMaxBins;
+    if (bits <= 8)
+      launch_radix_pass<8>(src_k, src_v, dst_k, dst_v, n, shift, mask, tiles, counts, pass_totals, stream);
+    else if (bits == 9)
+      launch_radix_pass<9>(src_k, src_v, dst_k, dst_v, n, shift, mask, tiles, counts, pass_totals, stream);
+    else
+      launch_radix_pass<10>(src_k, src_v, dst_k, dst_v, n, shift, mask, tiles, counts, pass_totals, stream);
     src_k = dst_k;
     src_v = dst_v;
+    shift += bits;
   }
   return check_launch("tbe_sort_pairs");
 }

@@ -36,7 +36,9 @@ def _vp(t):
 # ------------------------------------------------------- stages, bit-exact
 @pytest.mark.parametrize("n,hi,end_bit", [(0, 10, 4), (1, 10, 4), (63, 2, 1), (64, 300, 9), (4095, 1 << 8, 8),
                                           (4096, 1 << 16, 16), (4097, 1 << 23, 23), (100000, 7, 3),
-                                          (250001, 1 << 25, 25), (70000, 1 << 30, 31), (5000, 1000, 0)])
+                                          (250001, 1 << 25, 25), (70000, 1 << 30, 31), (5000, 1000, 0),
+                                          (33333, 1 << 17, 17), (50001, 1 << 19, 19), (81920, 1 << 20, 20),
+                                          (120000, 1 << 27, 27), (60000, 1 << 29, 29), (9000, 1 << 10, 10)])
 def test_sort_pairs_is_stable_and_bit_exact(oracle, n, hi, end_bit):
     rs = np.random.RandomState(n % 97)
     keys = rs.randint(0, hi, size=n).astype(np.int32)
