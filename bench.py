@@ -323,7 +323,7 @@ def main():
     U = 0
     if w["optimizer"]:
         lay = tbe_native.backward_workspace_layout(w["n"], D, tbe_native.DTYPE_F16 if w["fp16"] else
-                                                   tbe_native.DTYPE_F32)
+                                                   tbe_native.DTYPE_F32, T)
         ws = ext.backward_workspace(dev)
         U = int(ws[lay.num_unique:lay.num_unique + 4].view(torch.int32)[0])
     a_fwd, a_bwd, a_update = algorithmic_bytes(w, U)

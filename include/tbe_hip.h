@@ -87,7 +87,9 @@ TBE_API int tbe_forward(const void *weights, int32_t dtype, int32_t D,
  * Byte offsets of the regions of the backward workspace.  After a backward call
  * the first five regions hold the intermediate results that the parity gates
  * inspect (all int32):
- *   keys              [N]   table_offsets[t] + indices[p]             (tbe.cu:1495)
+ *   keys              [N]   table_offsets[t] + indices[p]             (tbe.cu:1495); written by
+ *                           tbe_backward_mixed only -- the uniform-D entry points sort the
+ *                           indices table by table and leave this region untouched
  *   keys_sorted       [N]   stable ascending sort of keys             (tbe.cu:1639-1655)
  *   positions_sorted  [N]   position p of each sorted key (IndexInfo.indices_idx, tbe.cu:1217)
  *   segment_starts    [U+1] first sorted position of each unique key, then N (tbe.cu:1523-1539)
@@ -112,7 +114,8 @@ typedef struct tbe_workspace_layout {
   int64_t max_partial_rows;
 } tbe_workspace_layout_t;
 
-TBE_API int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int32_t dtype,
+/* T (number of tables) sizes the sort scratch: no sort tile straddles two tables. */
+TBE_API int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int32_t dtype, int32_t T,
                                   tbe_workspace_layout_t *layout);
 
 /* Exact SGD:  weights[r][:] -= lr * sum_{p: key[p]==r} grad_output[b(p)][t(p)][:]
@@ -121,11 +124,15 @@ TBE_API int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int32_
  * (table_batched_embeddings_cuda.cu:383-435, "backward_sgd" in
  * table_batched_embeddings.cpp:59), whose per-lookup read-modify-write is only
  * correct when no row repeats (test_table_batched_embeddings.py:177-193).
- * `total_rows` is the row count of `weights`; it fixes the number of key bits
- * sorted, as optimizer_state.numel() does at tbe.cu:1643.
+ * `total_rows` is the row count of `weights`.  `max_table_rows` is an upper bound of the row
+ * count of the largest table, or 0 when unknown (total_rows is then used): it fixes the number
+ * of key bits sorted, as optimizer_state.numel() does at tbe.cu:1643 -- the lookups of a table
+ * are consecutive, so each table's indices are sorted on their own and the bits of a row
+ * inside its table suffice.  The sorted order is that of the (table, row) keys either way; an
+ * index >= 2^ceil(log2(bound + 1)) is an error of the caller, like any out-of-range index.
  */
 TBE_API int tbe_backward_sgd(const void *grad_output, void *weights, int32_t dtype,
-                     int64_t total_rows, int32_t D,
+                     int64_t total_rows, int64_t max_table_rows, int32_t D,
                      const int32_t *table_offsets, int32_t T,
                      const int32_t *indices, int64_t num_indices,
                      const int32_t *offsets, int32_t B,
@@ -143,7 +150,7 @@ TBE_API int tbe_backward_sgd(const void *grad_output, void *weights, int32_t dty
  * the reference leaves the weighted exact case unimplemented (tbe.cu:1552, 1678).
  */
 TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, int32_t dtype,
-                               int64_t total_rows, int32_t D,
+                               int64_t total_rows, int64_t max_table_rows, int32_t D,
                                const int32_t *table_offsets, int32_t T,
                                const int32_t *indices, int64_t num_indices,
                                const int32_t *offsets, int32_t B,
@@ -154,7 +161,7 @@ TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, i
                                void *workspace, uint64_t workspace_bytes, void *stream);
 
 /* The backward in two calls, so that the integer half can overlap other work.
- * tbe_plan_batch runs the stages that depend on the indices only -- linearize, sort, run
+ * tbe_plan_batch runs the stages that depend on the indices only -- gradient rows, sort, run
  * boundaries (table_batched_embeddings_cuda.cu:1618-1655 and the head test :1523-1539) -- and
  * leaves the result in `workspace`; it may run on another stream than the forward, while the
  * forward gathers.  tbe_backward_planned runs the gradient reduction and the optimizer
@@ -165,7 +172,7 @@ TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, i
 TBE_API int tbe_plan_batch(const int32_t *table_offsets, int32_t T,
                            const int32_t *indices, int64_t num_indices,
                            const int32_t *offsets, int32_t B, int64_t total_rows,
-                           int32_t D, int32_t dtype,
+                           int64_t max_table_rows, int32_t D, int32_t dtype,
                            void *workspace, uint64_t workspace_bytes, void *stream);
 
 TBE_API int tbe_backward_planned(int32_t optimizer, const void *grad_output, void *weights, int32_t dtype,
@@ -186,10 +193,11 @@ TBE_API int tbe_backward_planned(int32_t optimizer, const void *grad_output, voi
  * F16 the call equals tbe_backward_exact_adagrad.
  */
 TBE_API int tbe_backward_exact_adagrad_stochastic(
-    const void *grad_output, void *weights, int32_t dtype, int64_t total_rows, int32_t D,
-    const int32_t *table_offsets, int32_t T, const int32_t *indices, int64_t num_indices,
-    const int32_t *offsets, int32_t B, const void *per_sample_weights, void *optimizer_state,
-    float learning_rate, float eps, void *grad_per_sample_weights, uint64_t seed, uint64_t offset,
+    const void *grad_output, void *weights, int32_t dtype, int64_t total_rows,
+    int64_t max_table_rows, int32_t D, const int32_t *table_offsets, int32_t T,
+    const int32_t *indices, int64_t num_indices, const int32_t *offsets, int32_t B,
+    const void *per_sample_weights, void *optimizer_state, float learning_rate, float eps,
+    void *grad_per_sample_weights, uint64_t seed, uint64_t offset,
     void *workspace, uint64_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------- stages, individually callable
@@ -216,7 +224,8 @@ TBE_API int tbe_sort_pairs(const int32_t *keys_in, const int32_t *values_in,
 
 /* Run boundaries of a sorted key array: segment_starts[u] = first i with the
  * u-th distinct key, segment_starts[U] = n, *num_unique = U (device memory).
- * Same rule as the segment-head test at table_batched_embeddings_cuda.cu:1523-1539. */
+ * Same rule as the segment-head test at table_batched_embeddings_cuda.cu:1523-1539.
+ * keys_sorted must be 16-byte aligned (it is read in 16-byte vectors). */
 TBE_API uint64_t tbe_segments_workspace_bytes(int64_t n);
 TBE_API int tbe_find_segments(const int32_t *keys_sorted, int64_t n,
                       int32_t *segment_starts, int32_t *num_unique,
@@ -245,7 +254,7 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
  * (:1350-1469, "backward_exact_adagrad_mixed_D", .cpp:64), serves the approximate variant
  * (.cpp:63) and adds exact SGD; per-sample weights as in tbe_backward_exact_adagrad;
  * stochastic_rounding / seed / offset as in tbe_backward_exact_adagrad_stochastic.  The
- * workspace is a backward workspace sized with tbe_backward_workspace_layout(N, 4, dtype).
+ * workspace is a backward workspace sized with tbe_backward_workspace_layout(N, 4, dtype, T).
  */
 TBE_API int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp16_vector_width,
                               const int64_t *table_offsets, const int32_t *dim_offsets,
@@ -331,7 +340,8 @@ TBE_API int tbe_cache_init(const tbe_cache_t *cache, void *stream);
 /* Steps 1-5 above.  `workspace` is a backward workspace (tbe_backward_workspace_layout)
  * and keeps the batch's plan for tbe_backward_cached; `cache_workspace` follows
  * tbe_cache_workspace_layout.  `side_stream` must differ from `stream`. */
-TBE_API int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_t total_rows, int32_t D,
+TBE_API int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_t total_rows,
+                              int64_t max_table_rows, int32_t D,
                               const int32_t *table_offsets, int32_t T,
                               const int32_t *indices, int64_t num_indices,
                               const int32_t *offsets, int32_t B, int32_t step,

@@ -21,7 +21,7 @@ int key_bits(int64_t total_rows) {
   return bits;
 }
 
-void compute_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t *l) {
+void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *l) {
   const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
   const uint64_t ints = align_up(nn * 4, 256);
   // a segment enters the chunk queue when it has more than kShortSegment occurrences and owns
@@ -36,7 +36,7 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t 
   l->positions_sorted = off; off += ints;
   l->segment_starts = off; off += align_up((nn + 1) * 4, 256);
   l->num_unique = off; off += 256;
-  l->sort_scratch = off; off += align_up(sort_workspace_bytes(n), 256);
+  l->sort_scratch = off; off += align_up(sort_workspace_bytes(n, T), 256);
   l->segment_scratch = off; off += align_up(segments_workspace_bytes(n), 256);
   l->segment_ids = off; off += ints;
   l->long_segments = off; off += align_up(static_cast<uint64_t>(l->max_long_segments) * 16, 256);
@@ -50,23 +50,27 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t 
 
 int key_bits_for(int64_t total_rows) { return key_bits(total_rows); }
 
-void backward_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t *l) {
-  compute_layout(n, D, dtype, l);
+void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *l) {
+  compute_layout(n, D, dtype, T, l);
 }
 
-// linearize -> sort -> run boundaries (and the segment of every sorted position) into the
-// workspace regions of `l`.
+// gradient rows -> sort -> run boundaries (and the segment of every sorted position) into the
+// workspace regions of `l`.  The lookups of a table are consecutive, so the (table, row) order
+// of the reference's sort (tbe.cu:1639-1655) is reached by sorting every table's indices on
+// their own; the last pass adds the table's first row, and keys_sorted / positions_sorted come
+// out as the sort of the linearized keys would leave them.  The `keys` region stays unwritten.
 int build_plan(const tbe_workspace_layout_t &l, void *workspace, const int32_t *table_offsets,
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
-               int64_t total_rows, hipStream_t stream) {
+               int64_t total_rows, int64_t max_table_rows, hipStream_t stream) {
   char *ws = static_cast<char *>(workspace);
-  int32_t *keys = reinterpret_cast<int32_t *>(ws + l.keys);
   int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
-  int rc = linearize(table_offsets, T, indices, offsets, B, keys,
+  int rc = linearize(table_offsets, T, indices, offsets, B, nullptr,
                      reinterpret_cast<int32_t *>(ws + l.grad_rows), stream);
   if (rc) return rc;
-  rc = sort_pairs(keys, nullptr, keys_sorted, reinterpret_cast<int32_t *>(ws + l.positions_sorted),
-                  n, key_bits(total_rows), ws + l.sort_scratch, stream);
+  const int64_t largest = (max_table_rows > 0 && max_table_rows < total_rows) ? max_table_rows : total_rows;
+  const SortTables tables{offsets, B, T, table_offsets};
+  rc = sort_pairs(indices, nullptr, keys_sorted, reinterpret_cast<int32_t *>(ws + l.positions_sorted),
+                  n, key_bits(largest), ws + l.sort_scratch, stream, &tables);
   if (rc) return rc;
   return find_segments(keys_sorted, n, reinterpret_cast<int32_t *>(ws + l.segment_starts),
                        reinterpret_cast<int32_t *>(ws + l.num_unique),
@@ -81,6 +85,7 @@ struct BackwardCall {
   void *weights;
   int32_t dtype;
   int64_t total_rows;
+  int64_t max_table_rows;
   int32_t D;
   const int32_t *table_offsets;
   int32_t T;
@@ -111,6 +116,7 @@ int run_backward(const char *name, const BackwardCall &c) {
   TBE_REQUIRE(c.D % 4 == 0, "%s: D must be a multiple of 4 (got %d)", name, c.D);
   TBE_REQUIRE(c.dtype >= TBE_DTYPE_F32 && c.dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, c.dtype);
   TBE_REQUIRE(c.total_rows > 0 && c.total_rows < INT32_MAX, "%s: total_rows out of range", name);
+  TBE_REQUIRE(c.max_table_rows >= 0, "%s: max_table_rows must not be negative", name);
   TBE_REQUIRE(c.num_indices >= 0 && c.num_indices < INT32_MAX, "%s: num_indices out of range", name);
   TBE_REQUIRE(static_cast<int64_t>(c.T) * c.B < INT32_MAX, "%s: T*B out of range", name);
   TBE_REQUIRE(c.grad_output && c.weights, "%s: null pointer argument", name);
@@ -122,7 +128,7 @@ int run_backward(const char *name, const BackwardCall &c) {
   if (c.num_indices == 0) return TBE_OK;
 
   tbe_workspace_layout_t l;
-  compute_layout(c.num_indices, c.D, c.dtype, &l);
+  compute_layout(c.num_indices, c.D, c.dtype, c.T, &l);
   if (!c.workspace || c.workspace_bytes < l.total_bytes)
     return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
                 (unsigned long long)l.total_bytes, (unsigned long long)c.workspace_bytes);
@@ -135,7 +141,7 @@ int run_backward(const char *name, const BackwardCall &c) {
 
   if (!c.planned) {
     const int rc = build_plan(l, c.workspace, c.table_offsets, c.T, c.indices, c.num_indices,
-                              c.offsets, c.B, c.total_rows, c.stream);
+                              c.offsets, c.B, c.total_rows, c.max_table_rows, c.stream);
     if (rc) return rc;
   }
 
@@ -172,7 +178,7 @@ int run_backward(const char *name, const BackwardCall &c) {
 }  // namespace tbe
 
 extern "C" int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int32_t dtype,
-                                             tbe_workspace_layout_t *layout) {
+                                             int32_t T, tbe_workspace_layout_t *layout) {
   using namespace tbe;
   TBE_REQUIRE(layout, "tbe_backward_workspace_layout: null layout");
   TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX,
@@ -180,16 +186,17 @@ extern "C" int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int
   TBE_REQUIRE(D > 0 && D % 4 == 0, "tbe_backward_workspace_layout: D must be a positive multiple of 4 (got %d)", D);
   TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64,
               "tbe_backward_workspace_layout: bad dtype %d", dtype);
-  compute_layout(num_indices, D, dtype, layout);
+  TBE_REQUIRE(T > 0, "tbe_backward_workspace_layout: T must be positive (got %d)", T);
+  compute_layout(num_indices, D, dtype, T, layout);
   return TBE_OK;
 }
 
 extern "C" int tbe_backward_sgd(const void *grad_output, void *weights, int32_t dtype,
-                                int64_t total_rows, int32_t D, const int32_t *table_offsets,
+                                int64_t total_rows, int64_t max_table_rows, int32_t D, const int32_t *table_offsets,
                                 int32_t T, const int32_t *indices, int64_t num_indices,
                                 const int32_t *offsets, int32_t B, float learning_rate,
                                 void *workspace, uint64_t workspace_bytes, void *stream) {
-  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
+  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, max_table_rows, D, table_offsets, T, indices,
                       num_indices, offsets, B, nullptr, nullptr, learning_rate, 0.0f, nullptr,
                       workspace, workspace_bytes, static_cast<hipStream_t>(stream), tbe::kOptSgd,
                       false, nullptr, nullptr, tbe::StochasticRounding{0, 0, 0}};
@@ -197,7 +204,7 @@ extern "C" int tbe_backward_sgd(const void *grad_output, void *weights, int32_t 
 }
 
 extern "C" int tbe_backward_exact_adagrad(const void *grad_output, void *weights, int32_t dtype,
-                                          int64_t total_rows, int32_t D,
+                                          int64_t total_rows, int64_t max_table_rows, int32_t D,
                                           const int32_t *table_offsets, int32_t T,
                                           const int32_t *indices, int64_t num_indices,
                                           const int32_t *offsets, int32_t B,
@@ -205,7 +212,7 @@ extern "C" int tbe_backward_exact_adagrad(const void *grad_output, void *weights
                                           float learning_rate, float eps,
                                           void *grad_per_sample_weights, void *workspace,
                                           uint64_t workspace_bytes, void *stream) {
-  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
+  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, max_table_rows, D, table_offsets, T, indices,
                       num_indices, offsets, B, per_sample_weights, optimizer_state, learning_rate,
                       eps, grad_per_sample_weights, workspace, workspace_bytes,
                       static_cast<hipStream_t>(stream), tbe::kOptAdagrad, false, nullptr, nullptr,
@@ -214,12 +221,13 @@ extern "C" int tbe_backward_exact_adagrad(const void *grad_output, void *weights
 }
 
 extern "C" int tbe_backward_exact_adagrad_stochastic(
-    const void *grad_output, void *weights, int32_t dtype, int64_t total_rows, int32_t D,
-    const int32_t *table_offsets, int32_t T, const int32_t *indices, int64_t num_indices,
-    const int32_t *offsets, int32_t B, const void *per_sample_weights, void *optimizer_state,
-    float learning_rate, float eps, void *grad_per_sample_weights, uint64_t seed, uint64_t offset,
+    const void *grad_output, void *weights, int32_t dtype, int64_t total_rows,
+    int64_t max_table_rows, int32_t D, const int32_t *table_offsets, int32_t T,
+    const int32_t *indices, int64_t num_indices, const int32_t *offsets, int32_t B,
+    const void *per_sample_weights, void *optimizer_state, float learning_rate, float eps,
+    void *grad_per_sample_weights, uint64_t seed, uint64_t offset,
     void *workspace, uint64_t workspace_bytes, void *stream) {
-  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, D, table_offsets, T, indices,
+  tbe::BackwardCall c{grad_output, weights, dtype, total_rows, max_table_rows, D, table_offsets, T, indices,
                       num_indices, offsets, B, per_sample_weights, optimizer_state, learning_rate,
                       eps, grad_per_sample_weights, workspace, workspace_bytes,
                       static_cast<hipStream_t>(stream), tbe::kOptAdagrad, false, nullptr, nullptr,
@@ -241,7 +249,7 @@ extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
   TBE_REQUIRE(unique_slots || num_indices == 0, "tbe_backward_cached: null unique_slots");
   TBE_REQUIRE(optimizer != TBE_OPT_SGD || !per_sample_weights,
               "tbe_backward_cached: SGD takes no per-sample weights");
-  BackwardCall c{grad_output, cache->backing_rows, dtype, total_rows, D, nullptr, T, nullptr,
+  BackwardCall c{grad_output, cache->backing_rows, dtype, total_rows, 0, D, nullptr, T, nullptr,
                  num_indices, nullptr, B, per_sample_weights, optimizer_state, learning_rate, eps,
                  grad_per_sample_weights, workspace, workspace_bytes,
                  static_cast<hipStream_t>(stream),
@@ -252,25 +260,27 @@ extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
 
 extern "C" int tbe_plan_batch(const int32_t *table_offsets, int32_t T, const int32_t *indices,
                               int64_t num_indices, const int32_t *offsets, int32_t B,
-                              int64_t total_rows, int32_t D, int32_t dtype, void *workspace,
-                              uint64_t workspace_bytes, void *stream) {
+                              int64_t total_rows, int64_t max_table_rows, int32_t D,
+                              int32_t dtype, void *workspace, uint64_t workspace_bytes,
+                              void *stream) {
   using namespace tbe;
   const char *name = "tbe_plan_batch";
   TBE_REQUIRE(T > 0 && B > 0, "%s: T and B must be positive (got %d, %d)", name, T, B);
   TBE_REQUIRE(D > 0 && D % 4 == 0, "%s: D must be a positive multiple of 4 (got %d)", name, D);
   TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
   TBE_REQUIRE(total_rows > 0 && total_rows < INT32_MAX, "%s: total_rows out of range", name);
+  TBE_REQUIRE(max_table_rows >= 0, "%s: max_table_rows must not be negative", name);
   TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
   TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "%s: T*B out of range", name);
   TBE_REQUIRE(table_offsets && offsets && (indices || num_indices == 0), "%s: null pointer argument", name);
   if (num_indices == 0) return TBE_OK;
   tbe_workspace_layout_t l;
-  compute_layout(num_indices, D, dtype, &l);
+  compute_layout(num_indices, D, dtype, T, &l);
   if (!workspace || workspace_bytes < l.total_bytes)
     return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
                 (unsigned long long)l.total_bytes, (unsigned long long)workspace_bytes);
   return build_plan(l, workspace, table_offsets, T, indices, num_indices, offsets, B, total_rows,
-                    static_cast<hipStream_t>(stream));
+                    max_table_rows, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tbe_backward_planned(int32_t optimizer, const void *grad_output, void *weights,
@@ -285,7 +295,7 @@ extern "C" int tbe_backward_planned(int32_t optimizer, const void *grad_output, 
               "tbe_backward_planned: bad optimizer %d", optimizer);
   TBE_REQUIRE(optimizer != TBE_OPT_SGD || !per_sample_weights,
               "tbe_backward_planned: SGD takes no per-sample weights");
-  BackwardCall c{grad_output, weights, dtype, total_rows, D, nullptr, T, nullptr, num_indices,
+  BackwardCall c{grad_output, weights, dtype, total_rows, 0, D, nullptr, T, nullptr, num_indices,
                  nullptr, B, per_sample_weights, optimizer_state, learning_rate, eps,
                  grad_per_sample_weights, workspace, workspace_bytes,
                  static_cast<hipStream_t>(stream),

@@ -323,7 +323,7 @@ extern "C" int tbe_cache_init(const tbe_cache_t *cache, void *stream) {
 }
 
 extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_t total_rows,
-                                 int32_t D, const int32_t *table_offsets, int32_t T,
+                                 int64_t max_table_rows, int32_t D, const int32_t *table_offsets, int32_t T,
                                  const int32_t *indices, int64_t num_indices,
                                  const int32_t *offsets, int32_t B, int32_t step, void *workspace,
                                  uint64_t workspace_bytes, void *cache_workspace,
@@ -335,13 +335,14 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
   TBE_REQUIRE(D > 0 && D % 4 == 0, "%s: D must be a positive multiple of 4 (got %d)", name, D);
   TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
   TBE_REQUIRE(total_rows > 0 && total_rows < INT32_MAX, "%s: total_rows out of range", name);
+  TBE_REQUIRE(max_table_rows >= 0, "%s: max_table_rows must not be negative", name);
   TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
   TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "%s: T*B out of range", name);
   TBE_REQUIRE(step > 0, "%s: steps are numbered from 1 (got %d)", name, step);
   TBE_REQUIRE(table_offsets && offsets && (indices || num_indices == 0), "%s: null pointer argument", name);
   TBE_REQUIRE(stream != side_stream, "%s: side_stream must differ from stream", name);
   tbe_workspace_layout_t l;
-  backward_layout(num_indices, D, dtype, &l);
+  backward_layout(num_indices, D, dtype, T, &l);
   tbe_cache_workspace_layout_t cl;
   cache_layout(num_indices, cache->num_sets, &cl);
   if (!workspace || workspace_bytes < l.total_bytes)
@@ -360,7 +361,7 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
   TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(1), block, stats, static_cast<int64_t>(8), 0);
   if (num_indices == 0) return check_launch(name);
 
-  int rc = build_plan(l, workspace, table_offsets, T, indices, num_indices, offsets, B, total_rows, s);
+  int rc = build_plan(l, workspace, table_offsets, T, indices, num_indices, offsets, B, total_rows, max_table_rows, s);
   if (rc) return rc;
   const int32_t *keys_sorted = i32(ws, l.keys_sorted);
   const int32_t *segment_starts = i32(ws, l.segment_starts);

@@ -377,7 +377,7 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
               "%s: per_sample_weights and grad_per_sample_weights must both be given or both be null", name);
   if (num_indices == 0) return TBE_OK;
   tbe_workspace_layout_t l;
-  backward_layout(num_indices, 4, dtype, &l);  // no partial rows are used: size them for D = 4
+  backward_layout(num_indices, 4, dtype, T, &l);  // no partial rows are used: size them for D = 4
   if (!workspace || workspace_bytes < l.total_bytes)
     return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
                 (unsigned long long)l.total_bytes, (unsigned long long)workspace_bytes);
@@ -389,7 +389,7 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
              dim3(static_cast<unsigned>(ceil_div(num_bags * 16, kBlockThreads))), dim3(kBlockThreads),
              table_dim_offsets, indices, offsets, B, T, static_cast<int>(num_bags), i32(l.keys), i32(l.grad_rows));
   int rc = sort_pairs(i32(l.keys), nullptr, i32(l.keys_sorted), i32(l.positions_sorted), num_indices,
-                      key_bits_for(total_rows), ws + l.sort_scratch, s);
+                      key_bits_for(total_rows), ws + l.sort_scratch, s, nullptr);
   if (rc) return rc;
   rc = find_segments(i32(l.keys_sorted), num_indices, i32(l.segment_starts), i32(l.num_unique), nullptr,
                      ws + l.segment_scratch, s);

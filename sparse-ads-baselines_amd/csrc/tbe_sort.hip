@@ -6,9 +6,9 @@
 // The sort is the contract of cub::DeviceRadixSort::SortPairs as the reference
 // calls it (table_batched_embeddings_cuda.cu:1639-1655): ascending, stable,
 // key bits [0, end_bit).  A pass handles a digit of 8 to 10 bits (the fewest passes that cover
-// end_bit).  Each pass is three kernels:
-//   histogram  per-tile digit counts (LDS atomics) -> counts[digit][tile]
-//   scan       one workgroup per digit: exclusive prefix over tiles, and the digit's total
+// end_bit).  Each pass is four kernels:
+//   histogram  per-tile digit counts (LDS atomics) -> counts[table][digit][tile]
+//   scan       exclusive prefix sum over counts[] (workgroup sums, then the chunks)
 //   scatter    ranks each key inside its tile with wavefront ballots (all lanes
 //              holding the same digit are found with one ballot per digit bit; the lowest lane
 //              reserves the run in a per-wavefront LDS counter), reorders the
@@ -17,7 +17,7 @@
 // A tile is 4096 pairs; position order inside a tile is (wavefront, item, lane),
 // which the ranking preserves, so the sort is stable.
 
-#include "tbe_common.h"
+#include "tbe_stages.h"
 
 namespace tbe {
 namespace {
@@ -60,7 +60,8 @@ __device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t x, uint32_t *s
 // 16 lanes per bag.  Mirrors linear_index_weight_offsets_kernel
 // (table_batched_embeddings_cuda.cu:1471-1497); instead of the 8-byte
 // IndexInfo{b_t, indices_idx} payload it records the gradient row b*T + t of
-// each position, and the sort carries the position itself.
+// each position, and the sort carries the position itself.  `keys` may be null (the fused
+// backward sorts the indices themselves, table by table).
 constexpr int kLinLanes = 16;
 __global__ __launch_bounds__(kBlockThreads) void linearize_kernel(
     const int32_t *__restrict__ table_offsets, const int32_t *__restrict__ indices,
@@ -73,13 +74,17 @@ __global__ __launch_bounds__(kBlockThreads) void linearize_kernel(
   const int sub = static_cast<int>(gid % kLinLanes);
   const int t = bag / B;
   const int b = bag - t * B;
-  const int32_t row0 = table_offsets[t];
+  const int32_t row0 = keys ? table_offsets[t] : 0;
   const int32_t grow = b * num_tables + t;
   const int start = offsets[bag];
   const int end = offsets[bag + 1];
-  for (int p = start + sub; p < end; p += kLinLanes) {
-    keys[p] = row0 + indices[p];
-    grad_rows[p] = grow;
+  if (keys) {
+    for (int p = start + sub; p < end; p += kLinLanes) {
+      keys[p] = row0 + indices[p];
+      grad_rows[p] = grow;
+    }
+  } else {
+    for (int p = start + sub; p < end; p += kLinLanes) grad_rows[p] = grow;
   }
 }
 
@@ -100,58 +105,183 @@ __global__ __launch_bounds__(kBlockThreads) void interleaved_rows_kernel(
 }
 
 // ------------------------------------------------------------------ radix sort
+// The pairs may come in consecutive *tables* (table t owns positions [offsets[t*B], offsets[(t+1)*B]),
+// as in the bag layout): every table is then sorted on its own, so only the bits of a row number
+// inside its table are sorted, and the result is the sort by (table, row).  Tiles never straddle
+// tables: table t owns ceil(n_t / 4096) tiles, tile_prefix[] is the running tile count.  Without
+// tables the whole input is one table.
+//
+// counts[] holds, for table t with tiles_t tiles, a [bins][tiles_t] block at bins * tile_prefix[t]:
+// in that order (table, digit, tile) one exclusive prefix sum over the whole array is the output
+// position of the first key of every (table, digit, tile) run.
+
+constexpr int kScanItems = 8;
+constexpr int kScanChunk = kBlockThreads * kScanItems;  // 2048 count entries per workgroup
+
+__global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
+    const int32_t *__restrict__ offsets, int B, int num_tables, uint32_t n,
+    uint32_t *__restrict__ table_starts, uint32_t *__restrict__ tile_prefix) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int tid = threadIdx.x;
+  uint32_t carry = 0;
+  for (int c0 = 0; c0 < num_tables; c0 += kBlockThreads) {
+    const int t = c0 + tid;
+    uint32_t tiles = 0;
+    if (t < num_tables) {
+      uint32_t start = 0, end = n;
+      if (offsets) {
+        start = min(static_cast<uint32_t>(max(offsets[static_cast<int64_t>(t) * B], 0)), n);
+        if (t + 1 < num_tables)
+          end = min(static_cast<uint32_t>(max(offsets[static_cast<int64_t>(t + 1) * B], 0)), n);
+      }
+      end = max(end, start);
+      tiles = (end - start + kTile - 1) / kTile;
+      table_starts[t] = start;
+    }
+    uint32_t total;
+    const uint32_t incl = block_inclusive_scan(tiles, s_wave, total);
+    if (t < num_tables) tile_prefix[t] = carry + incl - tiles;
+    carry += total;
+    __syncthreads();
+  }
+  if (tid == 0) {
+    table_starts[num_tables] = n;
+    tile_prefix[num_tables] = carry;
+  }
+}
+
+// What a workgroup needs to know about its tile.
+struct TileInfo {
+  int table;
+  int64_t begin;       // first position of the tile
+  int count;           // pairs in the tile (0: nothing to do)
+  int64_t count_base;  // index of counts[table][digit 0][this tile]
+  int table_tiles;     // stride between digits in counts[]
+};
+
+template <int BITS>
+__device__ __forceinline__ TileInfo locate_tile(const uint32_t *__restrict__ table_starts,
+                                                const uint32_t *__restrict__ tile_prefix,
+                                                int num_tables, int max_tiles) {
+  TileInfo info{0, 0, 0, 0, 0};
+  const uint32_t tile = blockIdx.x;
+  if (tile >= tile_prefix[num_tables]) return info;
+  int lo = 0, hi = num_tables;  // tile_prefix[lo] <= tile < tile_prefix[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (tile_prefix[mid] <= tile) lo = mid; else hi = mid;
+  }
+  const uint32_t first_tile = tile_prefix[lo];
+  const uint32_t tiles = tile_prefix[lo + 1] - first_tile;
+  if (first_tile + tiles > static_cast<uint32_t>(max_tiles)) return info;  // inconsistent offsets
+  const uint32_t j = tile - first_tile;
+  info.table = lo;
+  info.begin = static_cast<int64_t>(table_starts[lo]) + static_cast<int64_t>(j) * kTile;
+  const int64_t left = static_cast<int64_t>(table_starts[lo + 1]) - info.begin;
+  info.count = static_cast<int>(max(int64_t{0}, min(left, static_cast<int64_t>(kTile))));
+  info.count_base = (static_cast<int64_t>(first_tile) << BITS) + j;
+  info.table_tiles = static_cast<int>(tiles);
+  return info;
+}
+
 // BITS = digit width of the pass (8, 9 or 10): 2^BITS bins, each thread owns 2^BITS / 256
 // consecutive digits in the per-digit steps.
 template <int BITS>
 __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
-    const uint32_t *__restrict__ keys, int64_t n, int shift, uint32_t mask, int num_tiles,
-    uint32_t *__restrict__ counts) {
+    const uint32_t *__restrict__ keys, const uint32_t *__restrict__ table_starts,
+    const uint32_t *__restrict__ tile_prefix, int num_tables, int max_tiles, int shift,
+    uint32_t mask, uint32_t *__restrict__ counts) {
   constexpr int kBinsT = 1 << BITS;
   __shared__ uint32_t s_hist[kBinsT];
+  const TileInfo tile = locate_tile<BITS>(table_starts, tile_prefix, num_tables, max_tiles);
+  if (tile.table_tiles == 0) return;
   const int tid = threadIdx.x;
 #pragma unroll
   for (int d = tid; d < kBinsT; d += kBlockThreads) s_hist[d] = 0;
   __syncthreads();
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * kTile;
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
-    const int64_t i = base + k * kBlockThreads + tid;
-    if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & mask], 1u);
+    const int i = k * kBlockThreads + tid;
+    if (i < tile.count) atomicAdd(&s_hist[(keys[tile.begin + i] >> shift) & mask], 1u);
   }
   __syncthreads();
 #pragma unroll
   for (int d = tid; d < kBinsT; d += kBlockThreads)
-    counts[static_cast<int64_t>(d) * num_tiles + blockIdx.x] = s_hist[d];
+    counts[tile.count_base + static_cast<int64_t>(d) * tile.table_tiles] = s_hist[d];
 }
 
-// Workgroup `d` turns counts[d][0..num_tiles) into an exclusive prefix over tiles (keys with
-// digit d in earlier tiles) and publishes the row total; the scatter kernel adds the number
-// of keys with a smaller digit, which it gets from a scan of the digit totals.
-__global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
-    uint32_t *__restrict__ counts, uint32_t *__restrict__ totals, int num_tiles) {
-  __shared__ uint32_t s_wave[kWavesPerBlock];
-  const int tid = threadIdx.x;
-  const int d = blockIdx.x;
-  uint32_t carry = 0;
-  uint32_t *row = counts + static_cast<int64_t>(d) * num_tiles;
-  for (int c0 = 0; c0 < num_tiles; c0 += kBlockThreads) {
-    const int i = c0 + tid;
-    const uint32_t x = i < num_tiles ? row[i] : 0u;
-    uint32_t total;
-    const uint32_t incl = block_inclusive_scan(x, s_wave, total);
-    if (i < num_tiles) row[i] = carry + incl - x;
-    carry += total;
-    __syncthreads();
+// Exclusive prefix sum over counts[0, bins * tiles): workgroup sums first, then every workgroup
+// adds up the sums before it and scans its own chunk.
+__device__ __forceinline__ void load_scan_items(const uint32_t *__restrict__ counts, int64_t first,
+                                                int64_t entries, uint32_t (&x)[kScanItems]) {
+  if (first < entries) {  // `entries` is a multiple of 256, so all eight are inside
+    const uint4 a = *reinterpret_cast<const uint4 *>(counts + first);
+    const uint4 b = *reinterpret_cast<const uint4 *>(counts + first + 4);
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+    x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+  } else {
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) x[k] = 0;
   }
-  if (tid == 0) totals[d] = carry;
 }
 
+__global__ __launch_bounds__(kBlockThreads) void radix_scan_reduce_kernel(
+    const uint32_t *__restrict__ counts, const uint32_t *__restrict__ tile_prefix, int num_tables,
+    int bits, uint32_t *__restrict__ block_sums) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int64_t entries = static_cast<int64_t>(tile_prefix[num_tables]) << bits;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kScanChunk + threadIdx.x * kScanItems;
+  uint32_t x[kScanItems];
+  load_scan_items(counts, first, entries, x);
+  uint32_t mine = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) mine += x[k];
+  uint32_t total;
+  (void)block_inclusive_scan(mine, s_wave, total);
+  if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
+    uint32_t *__restrict__ counts, const uint32_t *__restrict__ tile_prefix, int num_tables,
+    int bits, const uint32_t *__restrict__ block_sums) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int64_t entries = static_cast<int64_t>(tile_prefix[num_tables]) << bits;
+  const int64_t chunk_first = static_cast<int64_t>(blockIdx.x) * kScanChunk;
+  if (chunk_first >= entries) return;
+  uint32_t before = 0;
+  for (int i = threadIdx.x; i < static_cast<int>(blockIdx.x); i += kBlockThreads) before += block_sums[i];
+  uint32_t prior;
+  (void)block_inclusive_scan(before, s_wave, prior);
+  __syncthreads();
+  const int64_t first = chunk_first + threadIdx.x * kScanItems;
+  uint32_t x[kScanItems];
+  load_scan_items(counts, first, entries, x);
+  uint32_t mine = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) mine += x[k];
+  uint32_t total;
+  uint32_t running = prior + block_inclusive_scan(mine, s_wave, total) - mine;
+  if (first < entries) {
+    uint32_t y[kScanItems];
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+      y[k] = running;
+      running += x[k];
+    }
+    *reinterpret_cast<uint4 *>(counts + first) = make_uint4(y[0], y[1], y[2], y[3]);
+    *reinterpret_cast<uint4 *>(counts + first + 4) = make_uint4(y[4], y[5], y[6], y[7]);
+  }
+}
+
+// key_bias (nullable): added to the keys of table t as they are written (the last pass turns
+// rows inside a table into rows of the concatenated tables).
 template <int BITS>
 __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ values_in,
-    uint32_t *__restrict__ keys_out, uint32_t *__restrict__ values_out, int64_t n, int shift,
-    uint32_t mask, int num_tiles, const uint32_t *__restrict__ bases,
-    const uint32_t *__restrict__ totals) {
+    uint32_t *__restrict__ keys_out, uint32_t *__restrict__ values_out,
+    const uint32_t *__restrict__ table_starts, const uint32_t *__restrict__ tile_prefix,
+    int num_tables, int max_tiles, int shift, uint32_t mask, const uint32_t *__restrict__ bases,
+    const int32_t *__restrict__ key_bias) {
   constexpr int kBinsT = 1 << BITS;
   constexpr int kOwned = kBinsT / kBlockThreads;  // consecutive digits per thread
   __shared__ uint32_t s_keys[kTile];
@@ -161,11 +291,11 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   __shared__ uint32_t s_dest[kBinsT];
   __shared__ uint32_t s_scan[kWavesPerBlock];
 
+  const TileInfo tile = locate_tile<BITS>(table_starts, tile_prefix, num_tables, max_tiles);
+  if (tile.table_tiles == 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
-  const int64_t tile_base = static_cast<int64_t>(blockIdx.x) * kTile;
-  const int tile_count = static_cast<int>(min(static_cast<int64_t>(kTile), n - tile_base));
 
 #pragma unroll
   for (int w = 0; w < kWavesPerBlock; ++w)
@@ -173,11 +303,12 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     for (int d = tid; d < kBinsT; d += kBlockThreads) s_wave_count[w][d] = 0;
 
   uint32_t key[kItems], val[kItems];
-  const int64_t wave_base = tile_base + wave * kWaveTile;
+  const int wave_first = wave * kWaveTile;
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
-    const int64_t i = wave_base + k * kWave + lane;
-    const bool valid = i < n;
+    const int local = wave_first + k * kWave + lane;
+    const bool valid = local < tile.count;
+    const int64_t i = tile.begin + local;
     key[k] = valid ? keys_in[i] : 0xffffffffu;
     val[k] = valid ? (values_in ? values_in[i] : static_cast<uint32_t>(i)) : 0u;
   }
@@ -187,7 +318,7 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   uint32_t rank[kItems];
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
-    const bool valid = (wave_base + k * kWave + lane) < n;
+    const bool valid = (wave_first + k * kWave + lane) < tile.count;
     const uint32_t digit = (key[k] >> shift) & mask;
     unsigned long long peers = __ballot(valid);
 #pragma unroll
@@ -227,29 +358,19 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     }
     uint32_t total;
     uint32_t bin_start = block_inclusive_scan(mine, s_scan, total) - mine;
-    __syncthreads();
-    uint32_t totals_mine = 0;
-    uint32_t digit_total[kOwned];
-#pragma unroll
-    for (int q = 0; q < kOwned; ++q) {
-      digit_total[q] = totals[tid * kOwned + q];
-      totals_mine += digit_total[q];
-    }
-    uint32_t smaller = block_inclusive_scan(totals_mine, s_scan, total) - totals_mine;
 #pragma unroll
     for (int q = 0; q < kOwned; ++q) {
       const int d = tid * kOwned + q;
       s_bin_start[d] = bin_start;
-      s_dest[d] = smaller + bases[static_cast<int64_t>(d) * num_tiles + blockIdx.x] - bin_start;
+      s_dest[d] = bases[tile.count_base + static_cast<int64_t>(d) * tile.table_tiles] - bin_start;
       bin_start += digit_count[q];
-      smaller += digit_total[q];
     }
   }
   __syncthreads();
 
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
-    const bool valid = (wave_base + k * kWave + lane) < n;
+    const bool valid = (wave_first + k * kWave + lane) < tile.count;
     if (valid) {
       const uint32_t digit = (key[k] >> shift) & mask;
       const uint32_t local = s_bin_start[digit] + s_wave_count[wave][digit] + rank[k];
@@ -259,34 +380,44 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   }
   __syncthreads();
 
+  const uint32_t bias = key_bias ? static_cast<uint32_t>(key_bias[tile.table]) : 0u;
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
     const int local = k * kBlockThreads + tid;
-    if (local < tile_count) {
+    if (local < tile.count) {
       const uint32_t kk = s_keys[local];
       const uint32_t dst = s_dest[(kk >> shift) & mask] + static_cast<uint32_t>(local);
-      keys_out[dst] = kk;
+      keys_out[dst] = kk + bias;
       values_out[dst] = s_vals[local];
     }
   }
 }
 
 // -------------------------------------------------------------- find segments
-// Thread owns kSegItems consecutive sorted positions.  head(i) = i == 0 || key[i] != key[i-1]
-// (table_batched_embeddings_cuda.cu:1523-1525).
+// Thread owns kSegItems = 8 consecutive sorted positions (two 16-byte loads).
+// head(i) = i == 0 || key[i] != key[i-1]   (table_batched_embeddings_cuda.cu:1523-1525).
 __device__ __forceinline__ uint32_t segment_head_flags(const uint32_t *__restrict__ keys, int64_t n,
                                                        int64_t first) {
-  uint32_t flags = 0;
   if (first >= n) return 0;
-  uint32_t prev = first > 0 ? keys[first - 1] : 0u;
+  uint32_t cur[kSegItems];
+  if (first + kSegItems <= n) {
+    const uint4 a = *reinterpret_cast<const uint4 *>(keys + first);
+    const uint4 b = *reinterpret_cast<const uint4 *>(keys + first + 4);
+    cur[0] = a.x; cur[1] = a.y; cur[2] = a.z; cur[3] = a.w;
+    cur[4] = b.x; cur[5] = b.y; cur[6] = b.z; cur[7] = b.w;
+  } else {
+#pragma unroll
+    for (int k = 0; k < kSegItems; ++k) cur[k] = first + k < n ? keys[first + k] : 0u;
+  }
+  // the key before this thread's first one: the neighbouring lane holds it, except in lane 0
+  uint32_t prev = __shfl_up(cur[kSegItems - 1], 1, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0 && first > 0) prev = keys[first - 1];
+  uint32_t flags = 0;
 #pragma unroll
   for (int k = 0; k < kSegItems; ++k) {
     const int64_t i = first + k;
-    if (i < n) {
-      const uint32_t cur = keys[i];
-      if (i == 0 || cur != prev) flags |= 1u << k;
-      prev = cur;
-    }
+    if (i < n && (i == 0 || cur[k] != prev)) flags |= 1u << k;
+    prev = cur[k];
   }
   return flags;
 }
@@ -325,89 +456,146 @@ __global__ __launch_bounds__(kBlockThreads) void segment_scan_kernel(
   if (clear_queue_counters && tid >= 1 && tid <= 3) num_unique[tid] = 0;
 }
 
+// The heads of a tile are compacted in LDS and leave as one contiguous run; the segment of
+// every position leaves in 16-byte stores.
 __global__ __launch_bounds__(kBlockThreads) void segment_write_kernel(
     const uint32_t *__restrict__ keys, int64_t n, const uint32_t *__restrict__ tile_base,
     int32_t *__restrict__ segment_starts, int32_t *__restrict__ segment_ids) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
-  const int64_t first = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x) * kSegItems;
+  __shared__ int32_t s_heads[kSegTile];
+  const int64_t tile_first = static_cast<int64_t>(blockIdx.x) * kSegTile;
+  const int64_t first = tile_first + threadIdx.x * kSegItems;
   const uint32_t flags = segment_head_flags(keys, n, first);
   const uint32_t mine = __popc(flags);
   uint32_t total;
   const uint32_t incl = block_inclusive_scan(mine, s_wave, total);
-  uint32_t u = tile_base[blockIdx.x] + incl - mine;
+  const uint32_t base = tile_base[blockIdx.x];
+  uint32_t local = incl - mine;
+  int32_t ids[kSegItems];
 #pragma unroll
   for (int k = 0; k < kSegItems; ++k) {
-    if (flags & (1u << k)) segment_starts[u++] = static_cast<int32_t>(first + k);
-    // u now counts the heads at or before this position: its segment is u - 1
-    if (segment_ids && first + k < n) segment_ids[first + k] = static_cast<int32_t>(u) - 1;
+    if (flags & (1u << k)) s_heads[local++] = static_cast<int32_t>(first + k);
+    // `local` now counts the tile's heads at or before this position: its segment is base + local - 1
+    ids[k] = static_cast<int32_t>(base + local) - 1;
   }
+  if (segment_ids) {
+    if (first + kSegItems <= n) {
+      *reinterpret_cast<int4 *>(segment_ids + first) = make_int4(ids[0], ids[1], ids[2], ids[3]);
+      *reinterpret_cast<int4 *>(segment_ids + first + 4) = make_int4(ids[4], ids[5], ids[6], ids[7]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < kSegItems; ++k)
+        if (first + k < n) segment_ids[first + k] = ids[k];
+    }
+  }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < total; i += kBlockThreads) segment_starts[base + i] = s_heads[i];
 }
 
-inline int num_sort_tiles(int64_t n) { return static_cast<int>(ceil_div(n, kTile)); }
 inline int num_seg_tiles(int64_t n) { return static_cast<int>(ceil_div(n, kSegTile)); }
 
 }  // namespace
 
-// Sort workspace: [tmp keys n][tmp values n][counts 1024*tiles][totals 1024*passes]
-constexpr int kMaxPasses = 4;
+// Sort workspace: [tmp keys n][tmp values n][counts 1024 * max_tiles][workgroup sums of the count
+// scan][table_starts T+1][tile_prefix T+1]; max_tiles = ceil(n / 4096) + T.
+namespace {
+struct SortScratch {
+  uint64_t tmp_keys, tmp_vals, counts, block_sums, table_starts, tile_prefix, total;
+  int max_tiles;
+  int scan_blocks;  // for the widest digit
+};
 
-uint64_t sort_workspace_bytes(int64_t n) {
-  const uint64_t tiles = num_sort_tiles(n > 0 ? n : 1);
-  return align_up(static_cast<uint64_t>(n > 0 ? n : 1) * 4, 256) * 2 +
-         align_up(tiles * kMaxBins * 4, 256) + align_up(kMaxPasses * kMaxBins * 4, 256);
+SortScratch sort_scratch(int64_t n, int32_t num_tables) {
+  SortScratch s;
+  const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
+  const uint64_t tables = static_cast<uint64_t>(num_tables > 0 ? num_tables : 1);
+  s.max_tiles = static_cast<int>(ceil_div(nn, kTile) + tables);
+  s.scan_blocks = static_cast<int>(ceil_div(static_cast<uint64_t>(s.max_tiles) * kMaxBins, kScanChunk));
+  uint64_t off = 0;
+  s.tmp_keys = off; off += align_up(nn * 4, 256);
+  s.tmp_vals = off; off += align_up(nn * 4, 256);
+  s.counts = off; off += align_up(static_cast<uint64_t>(s.max_tiles) * kMaxBins * 4, 256);
+  s.block_sums = off; off += align_up(static_cast<uint64_t>(s.scan_blocks) * 4, 256);
+  s.table_starts = off; off += align_up((tables + 1) * 4, 256);
+  s.tile_prefix = off; off += align_up((tables + 1) * 4, 256);
+  s.total = off;
+  return s;
 }
 
-namespace {
+struct RadixPass {
+  const uint32_t *src_k, *src_v;
+  uint32_t *dst_k, *dst_v;
+  const uint32_t *table_starts, *tile_prefix;
+  int num_tables, max_tiles, shift;
+  uint32_t mask;
+  uint32_t *counts, *block_sums;
+  const int32_t *key_bias;
+};
+
 template <int BITS>
-void launch_radix_pass(const uint32_t *src_k, const uint32_t *src_v, uint32_t *dst_k, uint32_t *dst_v,
-                       int64_t n, int shift, uint32_t mask, int tiles, uint32_t *counts, uint32_t *totals,
-                       hipStream_t stream) {
+void launch_radix_pass(const RadixPass &p, hipStream_t stream) {
   const dim3 block(kBlockThreads);
-  TBE_LAUNCH("radix_histogram", stream, radix_histogram_kernel<BITS>, dim3(tiles), block, src_k, n, shift,
-             mask, tiles, counts);
-  TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, dim3(1 << BITS), block, counts, totals, tiles);
-  TBE_LAUNCH("radix_scatter", stream, radix_scatter_kernel<BITS>, dim3(tiles), block, src_k, src_v, dst_k,
-             dst_v, n, shift, mask, tiles, counts, totals);
+  const dim3 tiles(p.max_tiles);
+  const dim3 scan_blocks(static_cast<unsigned>(ceil_div(static_cast<int64_t>(p.max_tiles) << BITS, kScanChunk)));
+  TBE_LAUNCH("radix_histogram", stream, radix_histogram_kernel<BITS>, tiles, block, p.src_k, p.table_starts,
+             p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts);
+  TBE_LAUNCH("radix_scan_reduce", stream, radix_scan_reduce_kernel, scan_blocks, block, p.counts,
+             p.tile_prefix, p.num_tables, BITS, p.block_sums);
+  TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, scan_blocks, block, p.counts, p.tile_prefix,
+             p.num_tables, BITS, p.block_sums);
+  TBE_LAUNCH("radix_scatter", stream, radix_scatter_kernel<BITS>, tiles, block, p.src_k, p.src_v, p.dst_k,
+             p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts,
+             p.key_bias);
 }
 }  // namespace
 
+uint64_t sort_workspace_bytes(int64_t n, int32_t num_tables) { return sort_scratch(n, num_tables).total; }
+
 int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
                int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
-               hipStream_t stream) {
+               hipStream_t stream, const SortTables *tables) {
   if (n == 0) return TBE_OK;
   // Fewest passes with digits of at most 10 bits, the bits spread evenly over the passes
   // (23 bits -> 8+8+7, 25 -> 9+8+8, 27 -> 9+9+9, 17 -> 9+8).
   const int passes = end_bit <= 0 ? 1 : static_cast<int>(ceil_div(end_bit, kMaxRadixBits));
-  const int tiles = num_sort_tiles(n);
+  const int num_tables = tables ? tables->num_tables : 1;
+  const SortScratch scratch = sort_scratch(n, num_tables);
   char *ws = static_cast<char *>(workspace);
-  uint32_t *tmp_keys = reinterpret_cast<uint32_t *>(ws);
-  ws += align_up(static_cast<uint64_t>(n) * 4, 256);
-  uint32_t *tmp_vals = reinterpret_cast<uint32_t *>(ws);
-  ws += align_up(static_cast<uint64_t>(n) * 4, 256);
-  uint32_t *counts = reinterpret_cast<uint32_t *>(ws);
-  ws += align_up(static_cast<uint64_t>(tiles) * kMaxBins * 4, 256);
-  uint32_t *totals = reinterpret_cast<uint32_t *>(ws);
+  uint32_t *tmp_keys = reinterpret_cast<uint32_t *>(ws + scratch.tmp_keys);
+  uint32_t *tmp_vals = reinterpret_cast<uint32_t *>(ws + scratch.tmp_vals);
 
-  const uint32_t *src_k = reinterpret_cast<const uint32_t *>(keys_in);
-  const uint32_t *src_v = reinterpret_cast<const uint32_t *>(values_in);
-  int shift = 0;
+  RadixPass p;
+  p.table_starts = reinterpret_cast<uint32_t *>(ws + scratch.table_starts);
+  p.tile_prefix = reinterpret_cast<uint32_t *>(ws + scratch.tile_prefix);
+  p.num_tables = num_tables;
+  p.max_tiles = scratch.max_tiles;
+  p.counts = reinterpret_cast<uint32_t *>(ws + scratch.counts);
+  p.block_sums = reinterpret_cast<uint32_t *>(ws + scratch.block_sums);
+  TBE_LAUNCH("sort_setup", stream, sort_setup_kernel, dim3(1), dim3(kBlockThreads),
+             tables ? tables->offsets : nullptr, tables ? tables->bags_per_table : 0, num_tables,
+             static_cast<uint32_t>(n), const_cast<uint32_t *>(p.table_starts),
+             const_cast<uint32_t *>(p.tile_prefix));
+
+  p.src_k = reinterpret_cast<const uint32_t *>(keys_in);
+  p.src_v = reinterpret_cast<const uint32_t *>(values_in);
+  p.shift = 0;
   for (int pass = 0; pass < passes; ++pass) {
-    const int remaining = end_bit <= 0 ? 0 : end_bit - shift;
+    const int remaining = end_bit <= 0 ? 0 : end_bit - p.shift;
     const int bits = static_cast<int>(ceil_div(remaining, passes - pass));
-    const uint32_t mask = (1u << bits) - 1u;
+    p.mask = (1u << bits) - 1u;
     const bool to_out = ((passes - 1 - pass) % 2) == 0;
-    uint32_t *dst_k = to_out ? reinterpret_cast<uint32_t *>(keys_out) : tmp_keys;
-    uint32_t *dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
-    uint32_t *pass_totals = totals + pass * kMaxBins;
+    p.dst_k = to_out ? reinterpret_cast<uint32_t *>(keys_out) : tmp_keys;
+    p.dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
+    p.key_bias = (tables && pass == passes - 1) ? tables->key_bias : nullptr;
     if (bits <= 8)
-      launch_radix_pass<8>(src_k, src_v, dst_k, dst_v, n, shift, mask, tiles, counts, pass_totals, stream);
+      launch_radix_pass<8>(p, stream);
     else if (bits == 9)
-      launch_radix_pass<9>(src_k, src_v, dst_k, dst_v, n, shift, mask, tiles, counts, pass_totals, stream);
+      launch_radix_pass<9>(p, stream);
     else
-      launch_radix_pass<10>(src_k, src_v, dst_k, dst_v, n, shift, mask, tiles, counts, pass_totals, stream);
-    src_k = dst_k;
-    src_v = dst_v;
-    shift += bits;
+      launch_radix_pass<10>(p, stream);
+    p.src_k = p.dst_k;
+    p.src_v = p.dst_v;
+    p.shift += bits;
   }
   return check_launch("tbe_sort_pairs");
 }
@@ -478,7 +666,7 @@ extern "C" int tbe_interleaved_rows(const int32_t *indices, int64_t num_indices,
   return check_launch("tbe_interleaved_rows");
 }
 
-extern "C" uint64_t tbe_sort_workspace_bytes(int64_t n) { return tbe::sort_workspace_bytes(n); }
+extern "C" uint64_t tbe_sort_workspace_bytes(int64_t n) { return tbe::sort_workspace_bytes(n, 1); }
 
 extern "C" int tbe_sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
                               int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
@@ -488,11 +676,11 @@ extern "C" int tbe_sort_pairs(const int32_t *keys_in, const int32_t *values_in, 
   TBE_REQUIRE(end_bit >= 0 && end_bit <= 32, "tbe_sort_pairs: end_bit must be in [0, 32] (got %d)", end_bit);
   if (n == 0) return TBE_OK;
   TBE_REQUIRE(keys_in && keys_out && values_out, "tbe_sort_pairs: null pointer argument");
-  if (!workspace || workspace_bytes < sort_workspace_bytes(n))
+  if (!workspace || workspace_bytes < sort_workspace_bytes(n, 1))
     return fail(TBE_ERR_WORKSPACE, "tbe_sort_pairs: workspace of %llu bytes needed, %llu given",
-                (unsigned long long)sort_workspace_bytes(n), (unsigned long long)workspace_bytes);
+                (unsigned long long)sort_workspace_bytes(n, 1), (unsigned long long)workspace_bytes);
   return sort_pairs(keys_in, values_in, keys_out, values_out, n, end_bit, workspace,
-                    static_cast<hipStream_t>(stream));
+                    static_cast<hipStream_t>(stream), nullptr);
 }
 
 extern "C" uint64_t tbe_segments_workspace_bytes(int64_t n) { return tbe::segments_workspace_bytes(n); }
@@ -504,6 +692,7 @@ extern "C" int tbe_find_segments(const int32_t *keys_sorted, int64_t n, int32_t 
   TBE_REQUIRE(n >= 0 && n < INT32_MAX, "tbe_find_segments: n out of range");
   TBE_REQUIRE(segment_starts && num_unique, "tbe_find_segments: null pointer argument");
   TBE_REQUIRE(keys_sorted || n == 0, "tbe_find_segments: null keys");
+  TBE_REQUIRE(reinterpret_cast<uintptr_t>(keys_sorted) % 16 == 0, "tbe_find_segments: keys_sorted must be 16-byte aligned");
   if (!workspace || workspace_bytes < segments_workspace_bytes(n))
     return fail(TBE_ERR_WORKSPACE, "tbe_find_segments: workspace of %llu bytes needed, %llu given",
                 (unsigned long long)segments_workspace_bytes(n), (unsigned long long)workspace_bytes);

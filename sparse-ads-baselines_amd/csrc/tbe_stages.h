@@ -10,10 +10,20 @@ int linearize(const int32_t *table_offsets, int32_t T, const int32_t *indices,
               const int32_t *offsets, int32_t B, int32_t *keys, int32_t *grad_rows,
               hipStream_t stream);
 
-uint64_t sort_workspace_bytes(int64_t n);
+// Pairs that come table by table (positions [offsets[t*B], offsets[(t+1)*B]) belong to table t)
+// can be sorted per table: keys are then rows inside a table, end_bit covers the largest table,
+// and key_bias[t] (nullable) is added to the keys of table t in the output.
+struct SortTables {
+  const int32_t *offsets;   // [T*B+1] bag offsets
+  int32_t bags_per_table;   // B
+  int32_t num_tables;       // T
+  const int32_t *key_bias;  // [T] first row of every table
+};
+
+uint64_t sort_workspace_bytes(int64_t n, int32_t num_tables);
 int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
                int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
-               hipStream_t stream);
+               hipStream_t stream, const SortTables *tables);
 
 uint64_t segments_workspace_bytes(int64_t n);
 // segment_ids (nullable): receives, for every sorted position, the index of its segment.
@@ -61,9 +71,11 @@ struct UpdateArgs {
 int segment_update(const UpdateArgs &args, hipStream_t stream);
 
 int key_bits_for(int64_t total_rows);
-void backward_layout(int64_t n, int32_t D, int32_t dtype, tbe_workspace_layout_t *layout);
+void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *layout);
+// max_table_rows: an upper bound of the rows of the largest table (0 = unknown, total_rows is
+// used); it sets how many key bits are sorted.
 int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int32_t *table_offsets,
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
-               int64_t total_rows, hipStream_t stream);
+               int64_t total_rows, int64_t max_table_rows, hipStream_t stream);
 
 }  // namespace tbe

@@ -7,6 +7,7 @@ C-ABI library (include/tbe_hip.h).  torch is used for device memory and streams
 only -- no arithmetic happens here.
 """
 import ctypes
+import weakref
 
 import torch
 
@@ -52,6 +53,25 @@ def _check_common(weights, table_offsets, indices, offsets):
     return T, B
 
 
+_table_rows = {}  # id(table_offsets) -> (weak reference, tensor version, total_rows, largest table)
+
+
+def max_table_rows(table_offsets, total_rows):
+    """Rows of the largest table, read back from `table_offsets` once per tensor (one device to
+    host copy, then cached for as long as the tensor lives and is not written).  The backward
+    sorts that many key bits per table instead of the bits of `total_rows`."""
+    ident = id(table_offsets)
+    hit = _table_rows.get(ident)
+    if hit is not None and hit[0]() is table_offsets and hit[1:3] == (table_offsets._version, total_rows):
+        return hit[3]
+    starts = table_offsets.cpu().tolist() + [total_rows]
+    sizes = [b - a for a, b in zip(starts, starts[1:])]
+    largest = max(sizes) if min(sizes) >= 0 and starts[0] >= 0 else 0  # 0: unknown, sort all the bits
+    ref = weakref.ref(table_offsets, lambda _, ident=ident: _table_rows.pop(ident, None))
+    _table_rows[ident] = (ref, table_offsets._version, total_rows, largest)
+    return largest
+
+
 def _rounding_stream(device):
     """(seed, offset) for one stochastically rounded backward call, taken from PyTorch's
     generator of `device` the way the reference reserves Philox offsets
@@ -88,7 +108,7 @@ class BackwardPlan:
         self.code = _DTYPE_CODES[weights.dtype]
         self.total_rows = weights.size(0)
         self.device = weights.device
-        layout = _native.backward_workspace_layout(self.n, self.D, self.code)
+        layout = _native.backward_workspace_layout(self.n, self.D, self.code, T)
         # one buffer per call: it lives from the forward to the backward of the same step
         self.workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=self.device)
         side = BackwardPlan._side_streams.get(self.device)
@@ -103,8 +123,8 @@ class BackwardPlan:
         side.wait_stream(main)  # indices / offsets may still be in flight on the caller's stream
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_plan_batch(
-                _ptr(table_offsets), T, _ptr(indices), self.n, _ptr(offsets), B, self.total_rows, self.D, self.code,
-                _ptr(self.workspace), self.workspace.numel(), ctypes.c_void_p(side.cuda_stream)))
+                _ptr(table_offsets), T, _ptr(indices), self.n, _ptr(offsets), B, self.total_rows,
+                max_table_rows(table_offsets, self.total_rows), self.D, self.code, _ptr(self.workspace), self.workspace.numel(), ctypes.c_void_p(side.cuda_stream)))
         self.ready = torch.cuda.Event()
         self.ready.record(side)
 
@@ -171,11 +191,12 @@ def backward_sgd(grad_output, weights, table_offsets, indices, offsets, learning
     grad_output = _check_grad(grad_output, weights, T, B)
     D = weights.size(1)
     code = _DTYPE_CODES[weights.dtype]
-    layout = _native.backward_workspace_layout(indices.numel(), D, code)
+    layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
     ws = _workspace(weights.device, layout.total_bytes)
     with torch.cuda.device(weights.device):
         _native.check(_native.load().tbe_backward_sgd(
-            _ptr(grad_output), _ptr(weights), code, weights.size(0), D, _ptr(table_offsets), T,
+            _ptr(grad_output), _ptr(weights), code, weights.size(0),
+            max_table_rows(table_offsets, weights.size(0)), D, _ptr(table_offsets), T,
             _ptr(indices), indices.numel(), _ptr(offsets), B, float(learning_rate), _ptr(ws), ws.numel(),
             _stream(weights.device)))
     return None
@@ -203,19 +224,21 @@ def backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets
         _require(indice_weights.is_contiguous() and indice_weights.numel() == indices.numel(),
                  "indice_weights must be contiguous with one entry per index")
         grad_indice_weights = torch.empty(indices.shape, dtype=grad_output.dtype, device=weights.device)
-    layout = _native.backward_workspace_layout(indices.numel(), D, code)
+    layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
     ws = _workspace(weights.device, layout.total_bytes)
     with torch.cuda.device(weights.device):
         if stochastic_rounding and weights.dtype == torch.float16:
             seed, offset = _rounding_stream(weights.device)
             _native.check(_native.load().tbe_backward_exact_adagrad_stochastic(
-                _ptr(grad_output), _ptr(weights), code, weights.size(0), D, _ptr(table_offsets), T,
+                _ptr(grad_output), _ptr(weights), code, weights.size(0),
+                max_table_rows(table_offsets, weights.size(0)), D, _ptr(table_offsets), T,
                 _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state),
                 float(learning_rate), float(eps), _ptr(grad_indice_weights), seed, offset, _ptr(ws), ws.numel(),
                 _stream(weights.device)))
         else:  # rounding to nearest; stochastic rounding only exists for fp16 (tbe.cu:557-578)
             _native.check(_native.load().tbe_backward_exact_adagrad(
-                _ptr(grad_output), _ptr(weights), code, weights.size(0), D, _ptr(table_offsets), T,
+                _ptr(grad_output), _ptr(weights), code, weights.size(0),
+                max_table_rows(table_offsets, weights.size(0)), D, _ptr(table_offsets), T,
                 _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state),
                 float(learning_rate), float(eps), _ptr(grad_indice_weights), _ptr(ws), ws.numel(),
                 _stream(weights.device)))
@@ -305,7 +328,7 @@ def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_of
     state_dtype = torch.float64 if weights.dtype == torch.float64 else torch.float32
     _require(optimizer_state.dtype == state_dtype and optimizer_state.is_contiguous(),
              "optimizer_state must be contiguous %s" % state_dtype)
-    layout = _native.backward_workspace_layout(indices.numel(), 4, code)
+    layout = _native.backward_workspace_layout(indices.numel(), 4, code, T)
     ws = _workspace(weights.device, layout.total_bytes)
     stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
     seed, offset = _rounding_stream(weights.device) if stochastic else (0, 0)

@@ -10,6 +10,7 @@ import ctypes
 import torch
 
 import tbe_native as _native
+from table_batched_embeddings import max_table_rows as _max_table_rows
 
 _DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F16,
                 torch.float64: _native.DTYPE_F64}
@@ -73,13 +74,14 @@ class RowCache:
         n = indices.numel()
         self.step += 1
         self._n, self._T, self._B = n, T, B
-        self._plan_layout = _native.backward_workspace_layout(n, self.D, self.dtype_code)
+        self._plan_layout = _native.backward_workspace_layout(n, self.D, self.dtype_code, T)
         self._layout = _native.cache_workspace_layout(n, self.num_sets)
         self._plan_ws = self._grow(self._plan_ws, self._plan_layout.total_bytes)
         self._cache_ws = self._grow(self._cache_ws, self._layout.total_bytes)
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_cache_prepare(
-                ctypes.byref(self.handle), self.dtype_code, self.backing.size(0), self.D, _ptr(table_offsets), T,
+                ctypes.byref(self.handle), self.dtype_code, self.backing.size(0),
+                _max_table_rows(table_offsets, self.backing.size(0)), self.D, _ptr(table_offsets), T,
                 _ptr(indices), n, _ptr(offsets), B, self.step, _ptr(self._plan_ws), self._plan_ws.numel(),
                 _ptr(self._cache_ws), self._cache_ws.numel(), self._stream(),
                 ctypes.c_void_p(self.side_stream.cuda_stream)))

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -79,12 +79,12 @@ SIGNATURES = {
     "tbe_profile_count": (_i32, []),
     "tbe_profile_get": (ctypes.c_int, [_i32, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_f32)]),
     "tbe_forward": (ctypes.c_int, [_vp, _i32, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp, _vp, _vp]),
-    "tbe_backward_workspace_layout": (ctypes.c_int, [_i64, _i32, _i32, ctypes.POINTER(WorkspaceLayout)]),
-    "tbe_backward_sgd": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p,
+    "tbe_backward_workspace_layout": (ctypes.c_int, [_i64, _i32, _i32, _i32, ctypes.POINTER(WorkspaceLayout)]),
+    "tbe_backward_sgd": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p,
                                         _i32, _f32, _vp, _u64, _vp]),
-    "tbe_backward_exact_adagrad": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
+    "tbe_backward_exact_adagrad": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
                                                   _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _vp, _u64, _vp]),
-    "tbe_plan_batch": (ctypes.c_int, [_c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _i64, _i32, _i32, _vp, _u64, _vp]),
+    "tbe_plan_batch": (ctypes.c_int, [_c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _i64, _i64, _i32, _i32, _vp, _u64, _vp]),
     "tbe_backward_planned": (ctypes.c_int, [_i32, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _f32, _f32,
                                             _vp, _i32, _u64, _u64, _vp, _u64, _vp]),
     "tbe_linearize": (ctypes.c_int, [_c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _c_i32p, _c_i32p, _vp]),
@@ -99,12 +99,12 @@ SIGNATURES = {
     "tbe_backward_mixed": (ctypes.c_int, [_i32, _vp, _vp, _i32, _i32, _i64, _vp, _c_i32p, _c_i32p, _i32, _i32,
                                           _c_i32p, _i64, _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _i32, _u64, _u64,
                                           _vp, _u64, _vp]),
-    "tbe_backward_exact_adagrad_stochastic": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p,
+    "tbe_backward_exact_adagrad_stochastic": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p,
                                                              _i64, _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _u64,
                                                              _u64, _vp, _u64, _vp]),
     "tbe_cache_workspace_layout": (ctypes.c_int, [_i64, _i64, ctypes.POINTER(CacheWorkspaceLayout)]),
     "tbe_cache_init": (ctypes.c_int, [_cache_p, _vp]),
-    "tbe_cache_prepare": (ctypes.c_int, [_cache_p, _i32, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32,
+    "tbe_cache_prepare": (ctypes.c_int, [_cache_p, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32,
                                          _i32, _vp, _u64, _vp, _u64, _vp, _vp]),
     "tbe_forward_cached": (ctypes.c_int, [_cache_p, _i32, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp,
                                           _c_i32p, _vp, _vp]),
@@ -153,9 +153,9 @@ def check(code):
         raise RuntimeError(msg.decode("utf-8", "replace") if msg else "tbe error %d" % code)
 
 
-def backward_workspace_layout(num_indices, D, dtype_code):
+def backward_workspace_layout(num_indices, D, dtype_code, T):
     layout = WorkspaceLayout()
-    check(load().tbe_backward_workspace_layout(num_indices, D, dtype_code, ctypes.byref(layout)))
+    check(load().tbe_backward_workspace_layout(num_indices, D, dtype_code, T, ctypes.byref(layout)))
     return layout
 
 

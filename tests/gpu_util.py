@@ -24,16 +24,16 @@ def gpu_forward(p, weighted=None):
     return out.cpu().numpy()
 
 
-def workspace_views(n, D, dtype):
+def workspace_views(n, D, dtype, T):
     """Sorted keys, sorted positions and segment starts left in the workspace by the last backward."""
-    lay = tbe_native.backward_workspace_layout(n, D, CODES[np.dtype(dtype)])
+    lay = tbe_native.backward_workspace_layout(n, D, CODES[np.dtype(dtype)], T)
     ws = ext.backward_workspace(DEV if isinstance(DEV, torch.device) else torch.device(DEV))
 
     def view(off, count):
         return ws[off:off + 4 * count].view(torch.int32).cpu().numpy()
 
     U = int(view(lay.num_unique, 1)[0])
-    return dict(keys=view(lay.keys, n), keys_sorted=view(lay.keys_sorted, n),
+    return dict(keys_sorted=view(lay.keys_sorted, n),
                 positions_sorted=view(lay.positions_sorted, n), segment_starts=view(lay.segment_starts, U + 1),
                 num_unique=U, counters=view(lay.num_unique, 3))
 
@@ -54,7 +54,7 @@ def gpu_backward(p, optimizer, lr, eps=0.0, state=None):
         st = torch.zeros(w.shape[0], dtype=st_dtype, device=DEV) if state is None else dev(state)
         gpsw = ext.backward_exact_adagrad(go, w, *args, psw, st, lr, eps, False, 1)
     torch.cuda.synchronize()
-    views = workspace_views(p["n"], p["D"], p["weights"].dtype) if p["n"] else None
+    views = workspace_views(p["n"], p["D"], p["weights"].dtype, p["T"]) if p["n"] else None
     return dict(weights=w.cpu().numpy(), state=None if st is None else st.cpu().numpy(),
                 grad_psw=None if gpsw is None else gpsw.cpu().numpy(), views=views)
 

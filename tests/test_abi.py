@@ -41,7 +41,7 @@ def test_abi_version_matches_binding():
 
 
 def test_workspace_layout_is_ordered_and_sized():
-    lay = tbe_native.backward_workspace_layout(5242880, 128, tbe_native.DTYPE_F32)
+    lay = tbe_native.backward_workspace_layout(5242880, 128, tbe_native.DTYPE_F32, 64)
     offs = [lay.keys, lay.grad_rows, lay.keys_sorted, lay.positions_sorted, lay.segment_starts, lay.num_unique,
             lay.sort_scratch, lay.segment_scratch, lay.segment_ids, lay.long_segments, lay.chunk_segments,
             lay.partial_sums]
@@ -51,8 +51,8 @@ def test_workspace_layout_is_ordered_and_sized():
     assert lay.total_bytes >= lay.partial_sums + lay.max_partial_rows * 128 * 4
     assert lay.partial_sums - lay.chunk_segments >= lay.max_chunks * 32
     assert lay.total_bytes < 512 << 20
-    half = tbe_native.backward_workspace_layout(1000, 64, tbe_native.DTYPE_F16)
-    dbl = tbe_native.backward_workspace_layout(1000, 64, tbe_native.DTYPE_F64)
+    half = tbe_native.backward_workspace_layout(1000, 64, tbe_native.DTYPE_F16, 3)
+    dbl = tbe_native.backward_workspace_layout(1000, 64, tbe_native.DTYPE_F64, 3)
     assert dbl.total_bytes > half.total_bytes  # fp64 partial sums are 8 bytes wide
 
 
@@ -85,13 +85,13 @@ def test_null_pointers_and_bad_dtype_are_rejected():
 
 def test_backward_rejects_small_workspace_and_mismatched_weighting():
     lib = tbe_native.load()
-    rc = lib.tbe_backward_sgd(_fake(), _fake(), 0, 100, 4, _fake(), 1, _fake(), 10, _fake(), 1, 0.1, _fake(), 16,
+    rc = lib.tbe_backward_sgd(_fake(), _fake(), 0, 100, 0, 4, _fake(), 1, _fake(), 10, _fake(), 1, 0.1, _fake(), 16,
                               _null())
     assert rc == 2 and "workspace" in lib.tbe_last_error().decode()
-    rc = lib.tbe_backward_exact_adagrad(_fake(), _fake(), 0, 100, 4, _fake(), 1, _fake(), 10, _fake(), 1, _fake(),
+    rc = lib.tbe_backward_exact_adagrad(_fake(), _fake(), 0, 100, 0, 4, _fake(), 1, _fake(), 10, _fake(), 1, _fake(),
                                         _fake(), 0.1, 0.1, _null(), _fake(), 1 << 30, _null())
     assert rc == 1 and "per_sample_weights" in lib.tbe_last_error().decode()
-    rc = lib.tbe_backward_exact_adagrad(_fake(), _fake(), 0, 100, 4, _fake(), 1, _fake(), 10, _fake(), 1, _null(),
+    rc = lib.tbe_backward_exact_adagrad(_fake(), _fake(), 0, 100, 0, 4, _fake(), 1, _fake(), 10, _fake(), 1, _null(),
                                         _null(), 0.1, 0.1, _null(), _fake(), 1 << 30, _null())
     assert rc == 1 and "optimizer_state" in lib.tbe_last_error().decode()
 

@@ -24,14 +24,14 @@ pytestmark = pytest.mark.gpu
 def _run(p, seed, offset, weighted=False):
     w = dev(p["weights"])
     st = torch.zeros(w.shape[0], device=DEV)
-    lay = tbe_native.backward_workspace_layout(p["n"], p["D"], tbe_native.DTYPE_F16)
+    lay = tbe_native.backward_workspace_layout(p["n"], p["D"], tbe_native.DTYPE_F16, p["T"])
     ws = torch.empty(lay.total_bytes, dtype=torch.uint8, device=DEV)
     go, to, idx, off = dev(p["grad_output"]), dev(p["table_offsets"]), dev(p["indices"]), dev(p["offsets"])
     psw = dev(p["per_sample_weights"]) if weighted else None
     gpsw = torch.empty(p["n"], dtype=torch.float16, device=DEV) if weighted else None
     vp = lambda t: ctypes.c_void_p(t.data_ptr() if t is not None else 0)
     tbe_native.check(tbe_native.load().tbe_backward_exact_adagrad_stochastic(
-        vp(go), vp(w), tbe_native.DTYPE_F16, w.shape[0], p["D"], vp(to), p["T"], vp(idx), p["n"], vp(off), p["B"],
+        vp(go), vp(w), tbe_native.DTYPE_F16, w.shape[0], 0, p["D"], vp(to), p["T"], vp(idx), p["n"], vp(off), p["B"],
         vp(psw), vp(st), 0.05, 0.1, vp(gpsw), seed, offset, vp(ws), ws.numel(),
         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
     torch.cuda.synchronize()
