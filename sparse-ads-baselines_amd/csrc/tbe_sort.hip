@@ -284,18 +284,32 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const int32_t *__restrict__ key_bias) {
   constexpr int kBinsT = 1 << BITS;
   constexpr int kOwned = kBinsT / kBlockThreads;  // consecutive digits per thread
+  // The per-wavefront digit counters are only needed until every key knows its slot in the
+  // reordered tile.  For 10-bit digits (16 KB of counters) they share LDS with the reordered
+  // keys, which keeps four workgroups on a compute unit at the price of one more barrier.
+  constexpr bool kShareCounters = BITS >= 10;
   __shared__ uint32_t s_keys[kTile];
   __shared__ uint32_t s_vals[kTile];
-  __shared__ uint32_t s_wave_count[kWavesPerBlock][kBinsT];
+  __shared__ uint32_t s_own_count[kShareCounters ? 1 : kWavesPerBlock][kShareCounters ? 1 : kBinsT];
   __shared__ uint32_t s_bin_start[kBinsT];
   __shared__ uint32_t s_dest[kBinsT];
   __shared__ uint32_t s_scan[kWavesPerBlock];
+  static_assert(kWavesPerBlock * kBinsT <= kTile, "digit counters must fit the key buffer");
+  uint32_t(*s_wave_count)[kBinsT] =
+      kShareCounters ? reinterpret_cast<uint32_t(*)[kBinsT]>(s_keys) : reinterpret_cast<uint32_t(*)[kBinsT]>(s_own_count);
 
   const TileInfo tile = locate_tile<BITS>(table_starts, tile_prefix, num_tables, max_tiles);
   if (tile.table_tiles == 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
+
+  // output position of the tile's first key of every digit this thread owns (needed late;
+  // fetched first so the latency hides behind the ranking)
+  uint32_t digit_base[kOwned];
+#pragma unroll
+  for (int q = 0; q < kOwned; ++q)
+    digit_base[q] = bases[tile.count_base + static_cast<int64_t>(tid * kOwned + q) * tile.table_tiles];
 
 #pragma unroll
   for (int w = 0; w < kWavesPerBlock; ++w)
@@ -362,20 +376,26 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     for (int q = 0; q < kOwned; ++q) {
       const int d = tid * kOwned + q;
       s_bin_start[d] = bin_start;
-      s_dest[d] = bases[tile.count_base + static_cast<int64_t>(d) * tile.table_tiles] - bin_start;
+      s_dest[d] = digit_base[q] - bin_start;
       bin_start += digit_count[q];
     }
   }
   __syncthreads();
 
+  // slot of every key in the reordered tile; the counters are dead after this
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const uint32_t digit = (key[k] >> shift) & mask;
+    const bool valid = (wave_first + k * kWave + lane) < tile.count;
+    rank[k] += valid ? s_bin_start[digit] + s_wave_count[wave][digit] : 0u;
+  }
+  if constexpr (kShareCounters) __syncthreads();
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
     const bool valid = (wave_first + k * kWave + lane) < tile.count;
     if (valid) {
-      const uint32_t digit = (key[k] >> shift) & mask;
-      const uint32_t local = s_bin_start[digit] + s_wave_count[wave][digit] + rank[k];
-      s_keys[local] = key[k];
-      s_vals[local] = val[k];
+      s_keys[rank[k]] = key[k];
+      s_vals[rank[k]] = val[k];
     }
   }
   __syncthreads();

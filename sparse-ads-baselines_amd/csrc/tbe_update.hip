@@ -52,11 +52,13 @@ __device__ __forceinline__ T *resolve_row(T *weights, T *cache_rows,
 }
 
 // Applies the optimizer to one row held by a lane group.  `w_old` and `G` are
-// this lane's vector of the row.
+// this lane's vector of the row; `state_old` is *state_row, read by the caller ahead of the
+// gradient sum so that its latency is off the row's critical path (unused for SGD).
 template <typename T, int VEC, int CHUNKS, int OPT, bool STREAMING = false>
 __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_old,
                                              const RowVec<T, VEC> &G,
-                                             typename AccOf<T>::type *state_row, float lr,
+                                             typename AccOf<T>::type *state_row,
+                                             typename AccOf<T>::type state_old, float lr,
                                              float eps, int chunks, int group_base, int c,
                                              const StochasticRounding &sr, int64_t element) {
   using A = typename AccOf<T>::type;
@@ -69,7 +71,7 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 #pragma unroll
     for (int i = 0; i < VEC; ++i) local += G.v[i] * G.v[i];
     const A gss = group_sum<CHUNKS, A>(local, chunks, group_base);
-    const A s_new = *state_row + gss;
+    const A s_new = state_old + gss;
     if (c == 0) *state_row = s_new;
     const A mult = adagrad_multiplier<A>(s_new, lr, eps);
 #pragma unroll
@@ -89,8 +91,11 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 // to a queue that update_chunks_kernel drains with one wavefront per chunk.
 // Tile size in sorted positions: 32 per lane group, so narrow rows (many groups per wavefront)
 // get larger tiles and the per-tile bookkeeping is amortised over the same number of rows.
+#ifndef TBE_TPG
+#define TBE_TPG 32
+#endif
 constexpr int tile_positions(int chunks_template) {
-  return chunks_template == 0 ? 64 : (32 * (kWave / chunks_template) > 256 ? 256 : 32 * (kWave / chunks_template));
+  return chunks_template == 0 ? 64 : (chunks_template >= 32 ? 32 * (kWave / chunks_template) : (TBE_TPG * (kWave / chunks_template) > 256 ? 256 : TBE_TPG * (kWave / chunks_template)));
 }
 
 struct ChunkRecord {   // 32 bytes
@@ -120,7 +125,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
   using R = typename V::R;
 
   constexpr int kTilePositions = tile_positions(CHUNKS);
-  constexpr int kStageCap = kTilePositions + 64;  // occurrences staged in LDS per wavefront
+  constexpr int kStageCap = kTilePositions + kShortSegment;  // occurrences staged in LDS per wavefront
   __shared__ int32_t s_bounds[kWavesPerBlock][kTilePositions + 1];
   __shared__ int32_t s_keys[kWavesPerBlock][kTilePositions];
   __shared__ int32_t s_grow[kWavesPerBlock][kStageCap];
@@ -141,30 +146,63 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
   // p0 is its head.
   const int64_t p0 = tile * kTilePositions;
   const int64_t p1 = min(n, p0 + kTilePositions);
-  int u_first = segment_ids[p0];
-  if (segment_starts[u_first] != p0) ++u_first;
-  int u_limit;
-  if (p1 < n) {
-    u_limit = segment_ids[p1];
-    if (segment_starts[u_limit] != p1) ++u_limit;
-  } else {
-    u_limit = counters[0];
-  }
+  const bool last_tile = p1 >= n;
+  const int id0 = segment_ids[p0];
+  const int id1 = last_tile ? 0 : segment_ids[p1];
+  const int start0 = segment_starts[id0];
+  const int start1 = last_tile ? 0 : segment_starts[id1];
+  const int u_first = id0 + (start0 != p0 ? 1 : 0);
+  const int u_limit = last_tile ? counters[0] : id1 + (start1 != p1 ? 1 : 0);
   const int nseg = u_limit - u_first;  // <= kTilePositions
   if (nseg <= 0) return;
 
-  for (int k = lane; k <= nseg; k += kWave) {
-    const int sb = segment_starts[u_first + k];
-    s_bounds[wave][k] = sb;
-    if (k < nseg) s_keys[wave][k] = keys_sorted[sb];
+  // Bookkeeping into LDS.  All loads of one level are issued before the first dependent load,
+  // so a tile pays two memory round trips here however many positions it holds.
+  {
+    constexpr int kBoundIters = (kTilePositions + 1 + kWave - 1) / kWave;
+    int sb[kBoundIters];
+#pragma unroll
+    for (int q = 0; q < kBoundIters; ++q) {
+      const int k = q * kWave + lane;
+      sb[q] = segment_starts[u_first + min(k, nseg)];  // clamped, not predicated: no branch per load
+    }
+    int kv[kBoundIters];
+#pragma unroll
+    for (int q = 0; q < kBoundIters; ++q) {
+      const int k = q * kWave + lane;
+      kv[q] = keys_sorted[min(static_cast<int64_t>(sb[q]), n - 1)];
+    }
+#pragma unroll
+    for (int q = 0; q < kBoundIters; ++q) {
+      const int k = q * kWave + lane;
+      if (k <= nseg) s_bounds[wave][k] = sb[q];
+      if (k < nseg) s_keys[wave][k] = kv[q];
+    }
   }
   __builtin_amdgcn_wave_barrier();
   const int tile_begin = s_bounds[wave][0];
   const int staged = min(s_bounds[wave][nseg] - tile_begin, kStageCap);
-  for (int i = lane; i < staged; i += kWave) {
-    const int pos = positions_sorted[tile_begin + i];
-    s_grow[wave][i] = grad_rows[pos];
-    if constexpr (WEIGHTED) s_pos[wave][i] = pos;
+  {
+    constexpr int kStageIters = (kStageCap + kWave - 1) / kWave;
+    int pos[kStageIters], grow[kStageIters];
+#pragma unroll
+    for (int q = 0; q < kStageIters; ++q) {
+      const int i = q * kWave + lane;
+      pos[q] = positions_sorted[tile_begin + min(i, staged - 1)];
+    }
+#pragma unroll
+    for (int q = 0; q < kStageIters; ++q) {
+      const int i = q * kWave + lane;
+      grow[q] = grad_rows[pos[q]];
+    }
+#pragma unroll
+    for (int q = 0; q < kStageIters; ++q) {
+      const int i = q * kWave + lane;
+      if (i < staged) {
+        s_grow[wave][i] = grow[q];
+        if constexpr (WEIGHTED) s_pos[wave][i] = pos[q];
+      }
+    }
   }
   __builtin_amdgcn_wave_barrier();
 
@@ -200,45 +238,50 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
       continue;
     }
     T *wrow = resolve_row(weights, cache_rows, unique_slots, u, static_cast<int64_t>(key), D) + col;
+    // each row is touched once per step: streaming accesses keep L2 for gradient rows.  The
+    // row is requested right after the first gradient rows and stays packed until it is used,
+    // so that converting it (fp16) does not put its latency in front of theirs.
+    R w_raw;
+    A state_old = A(0);
     V w_old;
-    w_old.load_streaming(wrow);  // each row is touched once per step: keep L2 for gradient rows
     V G;
     G.zero();
     for (int i0 = seg_begin; i0 < seg_end; i0 += UNROLL) {
       R raw[UNROLL];
       int pos[UNROLL];
-      A pw[UNROLL];
+      T pw_raw[UNROLL];
 #pragma unroll
       for (int q = 0; q < UNROLL; ++q) {
         const int i = i0 + q;
         if (i < seg_end) {
+          // a short segment starts inside the tile and has at most kShortSegment occurrences,
+          // so all of them are among the staged ones
           const int rel = i - tile_begin;
-          int64_t grow;
-          if (rel < kStageCap) {
-            grow = s_grow[wave][rel];
-            if constexpr (WEIGHTED) pos[q] = s_pos[wave][rel];
-          } else {
-            const int p = positions_sorted[i];
-            grow = grad_rows[p];
-            if constexpr (WEIGHTED) pos[q] = p;
-          }
+          const int64_t grow = s_grow[wave][rel];
+          if constexpr (WEIGHTED) pos[q] = s_pos[wave][rel];
           raw[q] = V::load_raw(grad_output + grow * D + col);
-          if constexpr (WEIGHTED) pw[q] = to_acc(psw[pos[q]]);
+          if constexpr (WEIGHTED) pw_raw[q] = psw[pos[q]];
         }
       }
+      if (i0 == seg_begin) {  // requested after the first gradient rows, see above
+        w_raw = V::load_raw_streaming(wrow);
+        if constexpr (OPT == kOptAdagrad) state_old = state[key];
+      }
+      if constexpr (WEIGHTED) w_old.unpack(w_raw);
 #pragma unroll
       for (int q = 0; q < UNROLL; ++q) {
         if (i0 + q < seg_end) {
           V x;
           x.unpack(raw[q]);
           if constexpr (WEIGHTED) {
+            const A pw = to_acc(pw_raw[q]);
             A dot = A(0);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
             dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
             if (c == 0) grad_psw[pos[q]] = from_acc<T, A>(dot);
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * pw[q];
+            for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * pw;
           } else {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i];
@@ -246,8 +289,10 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
         }
       }
     }
-    apply_update<T, VEC, CHUNKS, OPT, true>(wrow, w_old, G, state ? state + key : nullptr, lr, eps,
-                                            chunks, group_base, c, sr, static_cast<int64_t>(key) * D + col);
+    w_old.unpack(w_raw);
+    apply_update<T, VEC, CHUNKS, OPT, true>(wrow, w_old, G, state ? state + key : nullptr, state_old, lr,
+                                            eps, chunks, group_base, c, sr,
+                                            static_cast<int64_t>(key) * D + col);
   }
 }
 
@@ -287,6 +332,10 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     V w_old;
     w_old.zero();
     if (active && (WEIGHTED || rec.partial < 0)) w_old.load(wrow);
+    A state_old = A(0);
+    if constexpr (OPT == kOptAdagrad) {
+      if (rec.partial < 0) state_old = state[rec.key];
+    }
     V G;
     G.zero();
     for (int base = rec.begin; base < rec.end; base += kWave) {
@@ -363,8 +412,9 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
 #pragma unroll
         for (int i = 0; i < VEC; ++i) dst[i] = G.v[i];
       } else {
-        apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, lr,
-                                          eps, chunks, 0, c, sr, static_cast<int64_t>(rec.key) * D + col);
+        apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, state_old,
+                                          lr, eps, chunks, 0, c, sr,
+                                          static_cast<int64_t>(rec.key) * D + col);
       }
     }
   }
@@ -400,6 +450,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     V w_old;
     w_old.zero();
     if (r == 0) w_old.load(wrow);
+    A state_old = A(0);
+    if constexpr (OPT == kOptAdagrad) state_old = state[rec.key];
     V G;
     G.zero();
     if (active) {
@@ -430,8 +482,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
       }
     }
     if (r == 0) {
-      apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, lr, eps,
-                                        chunks, 0, c, sr, static_cast<int64_t>(rec.key) * D + col);
+      apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, state_old, lr,
+                                        eps, chunks, 0, c, sr, static_cast<int64_t>(rec.key) * D + col);
     }
   }
 }

@@ -7,7 +7,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtbe_hip.so")
+# TBE_HIP_LIBRARY names another build of the library (same ABI version, checked on load).
+LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
 ABI_VERSION = 9
