@@ -35,6 +35,26 @@ def test_forward_matches_oracle(oracle, shape, weighted, dtype):
     assert_close(got, want, TOL[np.dtype(dtype)])
 
 
+@pytest.mark.parametrize("dtype,D", [(np.float32, 128), (np.float16, 64), (np.float32, 12), (np.float64, 16)])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_forward_thousands_of_ragged_bags(oracle, dtype, D, weighted):
+    """Nine thousand ragged bags: empty ones, bags of more than 64 lookups (several index slices
+    per bag), a bag count that is not a multiple of the wavefronts per workgroup."""
+    p = make_problem(77, T=3, E=400, D=D, B=3001, L=9, dtype=dtype, ragged=True, weighted=weighted, zipf=1.2)
+    lengths = np.diff(p["offsets"]).copy()
+    rs = np.random.RandomState(5)
+    lengths[rs.randint(0, lengths.size, size=40)] = rs.randint(65, 200, size=40)  # a few long bags
+    p["offsets"] = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    p["n"] = int(p["offsets"][-1])
+    p["indices"] = rs.randint(0, 400, size=p["n"]).astype(np.int32)
+    if weighted:
+        p["per_sample_weights"] = rs.uniform(0, 1, size=p["n"]).astype(dtype)
+    want = oracle.forward(p["weights"], p["table_offsets"], p["indices"], p["offsets"], p["per_sample_weights"])
+    got = gpu_forward(p)
+    assert_close(got, want, TOL[np.dtype(dtype)])
+    assert not got[(lengths == 0).reshape(3, 3001).T].any()  # empty bags give zeros
+
+
 @pytest.mark.parametrize("name", GOLDEN_CASES)
 def test_forward_matches_embeddingbag_fixture(name):
     g = load_golden(name)
