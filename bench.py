@@ -70,9 +70,9 @@ def make_workload(config, seed=0):
         T, D, B = 26, 128, 65536
         rows = np.floor(np.exp(rs.uniform(np.log(1e3), np.log(2e7), size=T))).astype(np.int64)
         w = dict(T=T, E=[int(r) for r in rows], D=D, B=B, fp16=False, weighted=False, optimizer="sgd", lr=0.01,
-                 eps=0.0, cache_slots=1 << 22, n=0, seed=seed, indices=None, offsets=None,
+                 eps=0.0, cache_slots=1 << 22, stage_slots=1 << 23, n=0, seed=seed, indices=None, offsets=None,
                  name="cfg5 DLRM-style + row cache: T=26 rows log-uniform [1e3,2e7] (sum %d) D=128 fp32 in pinned host "
-                      "memory, 2^22-slot LRU cache, B=65536 L=clip(Poisson(30),1,100) Zipf(1.1) per-table hot set, "
+                      "memory, 2^22-slot LRU cache + 2^23 staging rows, B=65536 L=clip(Poisson(30),1,100) Zipf(1.1) per-table hot set, "
                       "fwd + exact SGD lr=0.01, indices re-drawn every step" % int(rows.sum()))
         return w
     else:
@@ -182,7 +182,8 @@ def run_cached(args, w):
     t0 = time.perf_counter()
     module = ops.TableBatchedEmbeddingBags(T, w["E"], D, optimizer=ops.Optimizer.SGD, learning_rate=w["lr"],
                                            managed=ops.EmbeddingLocation.HOST_CACHED,
-                                           cache_slots=w["cache_slots"]).cuda()
+                                           cache_slots=w["cache_slots"],
+                                           cache_stage_slots=w["stage_slots"]).cuda()
     module.embedding_weights.data.mul_(0.01)
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t0
@@ -225,7 +226,10 @@ def run_cached(args, w):
     kernels = {k: {"launches_per_step": len(v) / len(extra), "avg_us": 1e3 * sum(v) / len(v)}
                for k, v in per_kernel.items()}
     row_bytes = D * 4
-    link_bytes = [(st["inserted"] + st["written_back"] + 3 * st["uncached"]) * row_bytes for st in stats]
+    # inserted and staged rows are fetched once, evicted and staged rows written once; an uncached row is
+    # read per lookup in the forward (counted once here) and read + written in the backward
+    link_bytes = [(st["inserted"] + st["written_back"] + 2 * st["staged"] + 3 * st["uncached"]) * row_bytes
+                  for st in stats]
     mean_lookups = sum(b[0].numel() for b in batches[args.warmup:]) / args.steps
     sec = elapsed / args.steps
     dominant = max(kernels, key=lambda k: kernels[k]["avg_us"] * kernels[k]["launches_per_step"])
@@ -234,7 +238,7 @@ def run_cached(args, w):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": w["name"], "T": T, "D": D, "B": B, "mean_lookups_per_step": mean_lookups,
-                   "cache_slots": w["cache_slots"], "seed": w["seed"], "host_table_GB": sum(w["E"]) * row_bytes / 1e9,
+                   "cache_slots": w["cache_slots"], "stage_slots": w["stage_slots"], "seed": w["seed"], "host_table_GB": sum(w["E"]) * row_bytes / 1e9,
                    "setup_seconds": setup_s},
         "effective_GBps": (bytes_alg / len(extra)) / sec / 1e9,
         "effective_frac_of_hbm_peak": (bytes_alg / len(extra)) / sec / HBM_PEAK,

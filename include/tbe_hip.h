@@ -292,17 +292,26 @@ TBE_API int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void 
  *   3. the missing rows of a set are inserted in ascending key order; the victim
  *      is the slot with the smallest (priority, way) among slots not used in this
  *      step, priority = last_used (LRU) or use_count (LFU); empty slots (priority 0)
- *      go first; if every slot of the set was used in this step the row stays
- *      uncached for the step and is read / updated in the backing table directly;
+ *      go first; if every slot of the set was used in this step the row is *staged*:
+ *      it gets a row of the staging area that follows the slots in `rows` (index
+ *      num_sets * 64 + s, s < stage_slots) for this step only, without a tag; when the
+ *      staging area is exhausted (or stage_slots is 0) the row stays uncached for the
+ *      step and is read / updated in the backing table directly;
  *   4. on the side stream, evicted rows are written back to the backing table and
- *      the inserted rows are fetched into their slots (every resident row counts
+ *      the inserted and the staged rows are fetched into their slots (every resident row counts
  *      as dirty: the optimizer updates each row it looks up); the side stream is
  *      joined to `stream` by an event before the call returns control of `stream`
  *      to the caller's next kernel;
  *   5. unique_slots[u] / lookup_slots[p] tell the forward and backward kernels
- *      where each row lives (slot >= 0, or -1 = backing table).
+ *      where each row lives (slot >= 0, or -1 = backing table);
+ *   6. tbe_backward_cached, after the update, copies the staged rows back to the
+ *      backing table.  A staged row thus crosses the host link once in each
+ *      direction per step, however many lookups hit it (an uncached row is read
+ *      once per lookup in the forward and read and written once in the backward).
  * The resulting tags / slots are a pure function of the key sequence, so a CPU
- * model can reproduce them bit for bit.
+ * model can reproduce them bit for bit (a staged row is an uncached row of the
+ * model; its staging index is the rank of the miss inside its set plus the number
+ * of misses of the sets before it, so it is reproducible too).
  */
 #define TBE_CACHE_WAYS 64
 enum { TBE_CACHE_LRU = 0, TBE_CACHE_LFU = 1 };
@@ -311,24 +320,25 @@ typedef struct tbe_cache {
   int32_t *tags;        /* [num_sets * 64] key of the row held by each slot, -1 = empty  */
   int32_t *last_used;   /* [num_sets * 64] step of the slot's last use, 0 = never        */
   int32_t *use_count;   /* [num_sets * 64] steps that used the row since it was inserted */
-  void *rows;           /* [num_sets * 64][D] cached rows                                */
+  void *rows;           /* [num_sets * 64 + stage_slots][D] cached rows, then the staging area */
   void *backing_rows;   /* device-visible address of the backing table [total_rows][D]   */
   int64_t num_sets;
   int32_t policy;       /* TBE_CACHE_LRU or TBE_CACHE_LFU                                */
+  int64_t stage_slots;  /* rows of the staging area (0 = none); num_sets * 64 + stage_slots < 2^31 */
 } tbe_cache_t;
 
 /* Byte offsets into the cache workspace (separate from the backward workspace). */
 typedef struct tbe_cache_workspace_layout {
   uint64_t total_bytes;
-  uint64_t unique_slots;   /* int32 [U]  slot of each unique row, -1 = backing table          */
+  uint64_t unique_slots;   /* int32 [U]  slot of each unique row (>= num_sets * 64: staged), -1 = backing table */
   uint64_t lookup_slots;   /* int32 [N]  the same, per lookup position                         */
-  uint64_t evicted_keys;   /* int32 [U]  -2 untouched, -1 filled an empty slot, >= 0 key written back */
+  uint64_t evicted_keys;   /* int32 [U]  -2 untouched, -1 filled an empty or staging slot, >= 0 key written back */
   uint64_t miss_sets;      /* int32 [U]  set of each missing row                               */
   uint64_t miss_list;      /* int32 [U]  missing rows grouped by set                           */
   uint64_t set_counts;     /* int32 [num_sets] misses per set                                  */
   uint64_t set_fill;       /* int32 [num_sets]                                                 */
   uint64_t set_starts;     /* int32 [num_sets + 1]                                             */
-  uint64_t stats;          /* int32 [8]: unique rows, hits, misses, inserted, written back, uncached */
+  uint64_t stats;          /* int32 [8]: unique rows, hits, misses, inserted, written back, uncached, staged */
 } tbe_cache_workspace_layout_t;
 
 TBE_API int tbe_cache_workspace_layout(int64_t num_indices, int64_t num_sets,
@@ -358,7 +368,8 @@ TBE_API int tbe_forward_cached(const tbe_cache_t *cache, int32_t dtype, int32_t 
                                void *output, void *stream);
 
 /* The fused update of tbe_backward_sgd / tbe_backward_exact_adagrad on the plan that
- * tbe_cache_prepare left in `workspace`, updating each row where it lives. */
+ * tbe_cache_prepare left in `workspace`, updating each row where it lives; staged rows are
+ * then copied back to the backing table. */
 TBE_API int tbe_backward_cached(int32_t optimizer, const void *grad_output, const tbe_cache_t *cache,
                                 int32_t dtype, int64_t total_rows, int32_t D, int32_t T, int32_t B,
                                 int64_t num_indices, const void *per_sample_weights,

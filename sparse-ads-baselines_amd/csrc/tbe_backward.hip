@@ -255,7 +255,15 @@ extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
                  static_cast<hipStream_t>(stream),
                  optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad, true, unique_slots, cache->rows,
                  StochasticRounding{0, 0, 0}};
-  return run_backward("tbe_backward_cached", c);
+  if (int rc = run_backward("tbe_backward_cached", c)) return rc;
+  if (cache->stage_slots <= 0 || num_indices == 0) return TBE_OK;
+  tbe_workspace_layout_t l;
+  backward_layout(num_indices, D, dtype, T, &l);
+  const char *ws = static_cast<const char *>(workspace);
+  return cache_unstage(cache, dtype, D, reinterpret_cast<const int32_t *>(ws + l.keys_sorted),
+                       reinterpret_cast<const int32_t *>(ws + l.segment_starts),
+                       reinterpret_cast<const int32_t *>(ws + l.num_unique), unique_slots, num_indices,
+                       static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tbe_plan_batch(const int32_t *table_offsets, int32_t T, const int32_t *indices,

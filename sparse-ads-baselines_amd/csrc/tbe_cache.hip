@@ -35,7 +35,7 @@ __device__ __forceinline__ uint32_t cache_set_of(uint32_t key, uint32_t num_sets
   return static_cast<uint32_t>((static_cast<uint64_t>(h) * num_sets) >> 32);
 }
 
-enum { kStatUnique = 0, kStatHits, kStatMisses, kStatInserted, kStatWrittenBack, kStatUncached };
+enum { kStatUnique = 0, kStatHits, kStatMisses, kStatInserted, kStatWrittenBack, kStatUncached, kStatStaged };
 
 __global__ __launch_bounds__(kBlockThreads) void cache_fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
@@ -150,11 +150,11 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
     int64_t num_sets, int32_t policy, int32_t step, const int32_t *__restrict__ keys_sorted,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ set_starts,
     const int32_t *__restrict__ miss_list, int32_t *__restrict__ unique_slots,
-    int32_t *__restrict__ evicted_keys, int32_t *__restrict__ stats) {
+    int32_t *__restrict__ evicted_keys, int32_t *__restrict__ stats, int64_t stage_slots) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
-  int inserted = 0, written_back = 0, uncached = 0;
+  int inserted = 0, written_back = 0, uncached = 0, staged = 0;
   for (int64_t set = wave_id; set < num_sets; set += stride) {
     const int begin = set_starts[set];
     const int end = set_starts[set + 1];
@@ -163,6 +163,7 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
     int32_t tag = tags[slot];
     int32_t used = last_used[slot];
     int32_t count = use_count[slot];
+    int staged_in_set = 0;
     int32_t previous = -1;  // missing rows are taken in ascending order of their index u
     for (int it = begin; it < end; ++it) {
       int32_t candidate = INT32_MAX;
@@ -182,7 +183,20 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
 #pragma unroll
       for (int m = kWave / 2; m > 0; m >>= 1) best = min(best, static_cast<uint32_t>(__shfl_xor(static_cast<int>(best), m, kWave)));
       if (best == 0xffffffffu) {
-        ++uncached;  // every way already serves this step: the row stays in the backing table
+        // Every way already serves this step.  The row gets a staging row for the step (index:
+        // misses of the sets before this one + rows staged by this set so far), or, when the
+        // staging area is exhausted, stays in the backing table.
+        const int64_t stage = static_cast<int64_t>(begin) + staged_in_set;
+        if (stage < stage_slots) {
+          if (lane == 0) {
+            unique_slots[u] = static_cast<int32_t>(num_sets * kWays + stage);
+            evicted_keys[u] = -1;
+          }
+          ++staged_in_set;
+          ++staged;
+        } else {
+          ++uncached;
+        }
         continue;
       }
       const int way = __ffsll(static_cast<long long>(__ballot(priority == best))) - 1;
@@ -207,6 +221,7 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
     if (inserted) atomicAdd(&stats[kStatInserted], inserted);
     if (written_back) atomicAdd(&stats[kStatWrittenBack], written_back);
     if (uncached) atomicAdd(&stats[kStatUncached], uncached);
+    if (staged) atomicAdd(&stats[kStatStaged], staged);
   }
 }
 
@@ -231,6 +246,26 @@ __global__ __launch_bounds__(kBlockThreads) void cache_fill_kernel(
       for (int i = lane; i < row_units; i += kWave) old_row[i] = slot_row[i];
     }
     for (int i = lane; i < row_units; i += kWave) slot_row[i] = new_row[i];
+  }
+}
+
+// After the update: staged rows (slot >= first_stage_slot) go back to the backing table.
+__global__ __launch_bounds__(kBlockThreads) void cache_unstage_kernel(
+    const uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
+    const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
+    int64_t first_stage_slot) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int U = counters[0];
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  for (int64_t u = wave_id; u < U; u += stride) {
+    const int64_t slot = unique_slots[u];
+    if (slot < first_stage_slot) continue;
+    const int64_t key = keys_sorted[segment_starts[u]];
+    const uint64_t *src = cache_rows + slot * row_units;
+    uint64_t *dst = backing_rows + key * row_units;
+    for (int i = lane; i < row_units; i += kWave) dst[i] = src[i];
   }
 }
 
@@ -283,6 +318,8 @@ int validate_cache(const char *name, const tbe_cache_t *cache) {
   TBE_REQUIRE(cache->tags && cache->last_used && cache->use_count && cache->rows && cache->backing_rows,
               "%s: cache has a null array", name);
   TBE_REQUIRE(cache->num_sets > 0 && cache->num_sets * kWays < INT32_MAX, "%s: num_sets out of range", name);
+  TBE_REQUIRE(cache->stage_slots >= 0 && cache->num_sets * kWays + cache->stage_slots < INT32_MAX,
+              "%s: stage_slots out of range", name);
   TBE_REQUIRE(cache->policy == TBE_CACHE_LRU || cache->policy == TBE_CACHE_LFU, "%s: bad policy %d", name,
               cache->policy);
   return TBE_OK;
@@ -298,6 +335,20 @@ hipEvent_t join_event(int which) {
 }
 
 }  // namespace
+
+int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int32_t *keys_sorted,
+                  const int32_t *segment_starts, const int32_t *counters,
+                  const int32_t *unique_slots, int64_t num_indices, hipStream_t stream) {
+  if (cache->stage_slots <= 0 || num_indices == 0) return TBE_OK;
+  const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
+  TBE_LAUNCH("cache_unstage", stream, cache_unstage_kernel,
+             dim3(grid_for(num_indices, kWavesPerBlock, 256 * 16)), dim3(kBlockThreads),
+             static_cast<const uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows),
+             row_units, keys_sorted, segment_starts, counters, unique_slots,
+             cache->num_sets * static_cast<int64_t>(kWays));
+  return check_launch("tbe_backward_cached");
+}
+
 }  // namespace tbe
 
 extern "C" int tbe_cache_workspace_layout(int64_t num_indices, int64_t num_sets,
@@ -382,7 +433,7 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
   TBE_LAUNCH("cache_insert", s, cache_insert_kernel, dim3(grid_for(num_sets, kWavesPerBlock, 256 * 16)), block,
              cache->tags, cache->last_used, cache->use_count, num_sets, cache->policy, step, keys_sorted,
              segment_starts, i32(cw, cl.set_starts), i32(cw, cl.miss_list), i32(cw, cl.unique_slots),
-             i32(cw, cl.evicted_keys), stats);
+             i32(cw, cl.evicted_keys), stats, cache->stage_slots);
 
   // Row traffic over the host link goes to the side stream while this stream builds the
   // per-lookup slot table; the side stream is joined before anything reads the cached rows.

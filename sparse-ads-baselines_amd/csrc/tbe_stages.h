@@ -78,4 +78,9 @@ int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int3
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
                int64_t total_rows, int64_t max_table_rows, hipStream_t stream);
 
+// Copies the rows that tbe_cache_prepare staged for this step back to the backing table.
+int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int32_t *keys_sorted,
+                  const int32_t *segment_starts, const int32_t *counters,
+                  const int32_t *unique_slots, int64_t num_indices, hipStream_t stream);
+
 }  // namespace tbe

@@ -15,7 +15,7 @@ from table_batched_embeddings import max_table_rows as _max_table_rows
 _DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F16,
                 torch.float64: _native.DTYPE_F64}
 _POLICIES = {"lru": _native.CACHE_LRU, "lfu": _native.CACHE_LFU}
-STAT_NAMES = ("unique_rows", "hits", "misses", "inserted", "written_back", "uncached")
+STAT_NAMES = ("unique_rows", "hits", "misses", "inserted", "written_back", "uncached", "staged")
 
 
 def _ptr(t):
@@ -23,10 +23,13 @@ def _ptr(t):
 
 
 class RowCache:
-    def __init__(self, backing_weights, cache_slots, policy="lru"):
+    def __init__(self, backing_weights, cache_slots, policy="lru", stage_slots=0):
         """backing_weights: [rows, D] tensor whose storage is device-visible host memory
         (table_batched_embeddings.new_host_mapped_tensor) -- or plain device memory, which is
-        useful for tests.  cache_slots is rounded down to a multiple of 64 (one set)."""
+        useful for tests.  cache_slots is rounded down to a multiple of 64 (one set).
+        stage_slots: rows of HBM that hold, for one step, the rows no slot could take (every way
+        of their set already serves the step): they then cross the host link once per step and
+        direction instead of once per lookup.  Sized for the misses of a step it stages them all."""
         if policy not in _POLICIES:
             raise ValueError("cache policy must be 'lru' or 'lfu'")
         if not backing_weights.is_cuda or backing_weights.dim() != 2 or not backing_weights.is_contiguous():
@@ -42,9 +45,12 @@ class RowCache:
         self.tags = torch.empty(slots, dtype=torch.int32, device=self.device)
         self.last_used = torch.empty(slots, dtype=torch.int32, device=self.device)
         self.use_count = torch.empty(slots, dtype=torch.int32, device=self.device)
-        self.rows = torch.empty(slots, self.D, dtype=backing_weights.dtype, device=self.device)
+        self.stage_slots = int(stage_slots)
+        if self.stage_slots < 0:
+            raise ValueError("stage_slots must not be negative")
+        self.rows = torch.empty(slots + self.stage_slots, self.D, dtype=backing_weights.dtype, device=self.device)
         self.handle = _native.Cache(_ptr(self.tags), _ptr(self.last_used), _ptr(self.use_count), _ptr(self.rows),
-                                    _ptr(self.backing), self.num_sets, _POLICIES[policy])
+                                    _ptr(self.backing), self.num_sets, _POLICIES[policy], self.stage_slots)
         self.side_stream = torch.cuda.Stream(device=self.device)  # default priority
         self.step = 0
         self._plan_ws = None

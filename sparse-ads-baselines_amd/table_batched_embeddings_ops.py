@@ -136,7 +136,8 @@ class TableBatchedEmbeddingBags(nn.Module):
 
     def __init__(self, num_tables, num_embeddings, embedding_dim, optimizer=Optimizer.SGD,
                  learning_rate=0.01, eps=None, stochastic_rounding=False, fp16=False,
-                 managed=EmbeddingLocation.DEVICE, cache_slots=None, cache_policy="lru"):
+                 managed=EmbeddingLocation.DEVICE, cache_slots=None, cache_policy="lru",
+                 cache_stage_slots=0):
         super(TableBatchedEmbeddingBags, self).__init__()
         assert managed in (EmbeddingLocation.DEVICE, EmbeddingLocation.HOST_MAPPED,
                            EmbeddingLocation.HOST_CACHED)
@@ -166,7 +167,7 @@ class TableBatchedEmbeddingBags(nn.Module):
         if managed == EmbeddingLocation.HOST_CACHED:
             assert cache_slots is not None, "HOST_CACHED needs cache_slots"
             self.row_cache = table_batched_embeddings_cache.RowCache(self.embedding_weights.data, cache_slots,
-                                                                     cache_policy)
+                                                                     cache_policy, cache_stage_slots)
             # checkpoints must see the rows the cache holds
             self.register_state_dict_pre_hook(lambda module, prefix, keep_vars: module.flush_cache())
         self.register_buffer("table_offsets",

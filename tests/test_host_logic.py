@@ -45,7 +45,8 @@ def test_module_constructor_signature_matches_reference():
     params = inspect.signature(ops.TableBatchedEmbeddingBags.__init__).parameters
     # the reference's nine arguments in order, then the cache extension
     assert list(params)[1:] == ["num_tables", "num_embeddings", "embedding_dim", "optimizer", "learning_rate", "eps",
-                                "stochastic_rounding", "fp16", "managed", "cache_slots", "cache_policy"]
+                                "stochastic_rounding", "fp16", "managed", "cache_slots", "cache_policy",
+                                "cache_stage_slots"]
     assert params["optimizer"].default is ops.Optimizer.SGD
     assert params["learning_rate"].default == 0.01
     assert params["managed"].default is ops.EmbeddingLocation.DEVICE
