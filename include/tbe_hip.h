@@ -367,14 +367,17 @@ TBE_API int tbe_forward_cached(const tbe_cache_t *cache, int32_t dtype, int32_t 
                                const void *per_sample_weights, const int32_t *lookup_slots,
                                void *output, void *stream);
 
-/* The fused update of tbe_backward_sgd / tbe_backward_exact_adagrad on the plan that
- * tbe_cache_prepare left in `workspace`, updating each row where it lives; staged rows are
- * then copied back to the backing table. */
+/* The fused update of tbe_backward_sgd / tbe_backward_exact_adagrad(_stochastic) on the plan
+ * that tbe_cache_prepare left in `workspace`, updating each row where it lives; staged rows are
+ * then copied back to the backing table.  stochastic_rounding / seed / offset as in
+ * tbe_backward_exact_adagrad_stochastic: the random word of a weight depends on its place in the
+ * table, not on where the row currently lives, so a cached run equals an uncached one. */
 TBE_API int tbe_backward_cached(int32_t optimizer, const void *grad_output, const tbe_cache_t *cache,
                                 int32_t dtype, int64_t total_rows, int32_t D, int32_t T, int32_t B,
                                 int64_t num_indices, const void *per_sample_weights,
                                 void *optimizer_state, float learning_rate, float eps,
                                 void *grad_per_sample_weights,
+                                int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
                                 void *workspace, uint64_t workspace_bytes,
                                 const int32_t *unique_slots, void *stream);
 

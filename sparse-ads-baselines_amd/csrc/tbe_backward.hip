@@ -240,6 +240,7 @@ extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
                                    int32_t D, int32_t T, int32_t B, int64_t num_indices,
                                    const void *per_sample_weights, void *optimizer_state,
                                    float learning_rate, float eps, void *grad_per_sample_weights,
+                                   int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
                                    void *workspace, uint64_t workspace_bytes,
                                    const int32_t *unique_slots, void *stream) {
   using namespace tbe;
@@ -254,7 +255,7 @@ extern "C" int tbe_backward_cached(int32_t optimizer, const void *grad_output,
                  grad_per_sample_weights, workspace, workspace_bytes,
                  static_cast<hipStream_t>(stream),
                  optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad, true, unique_slots, cache->rows,
-                 StochasticRounding{0, 0, 0}};
+                 StochasticRounding{seed, offset, (stochastic_rounding && dtype == TBE_DTYPE_F16) ? 1 : 0}};
   if (int rc = run_backward("tbe_backward_cached", c)) return rc;
   if (cache->stage_slots <= 0 || num_indices == 0) return TBE_OK;
   tbe_workspace_layout_t l;

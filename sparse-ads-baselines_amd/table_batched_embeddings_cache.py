@@ -124,9 +124,11 @@ class RowCache:
                 _ptr(offsets), B, _ptr(per_sample_weights), _ptr(slots), _ptr(output), self._stream()))
         return output
 
-    def backward(self, optimizer, grad_output, per_sample_weights, optimizer_state, learning_rate, eps):
+    def backward(self, optimizer, grad_output, per_sample_weights, optimizer_state, learning_rate, eps,
+                 stochastic_rounding=None):
         """optimizer: 'sgd' or 'adagrad'.  Updates rows where they live; returns the gradient
-        w.r.t. per_sample_weights or None."""
+        w.r.t. per_sample_weights or None.  stochastic_rounding: None, or the (seed, offset) of
+        the random stream that rounds updated fp16 weights (Adagrad only)."""
         grad_output = grad_output.contiguous()
         grad_psw = None
         if per_sample_weights is not None:
@@ -138,8 +140,10 @@ class RowCache:
                 code, _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.backing.size(0), self.D,
                 self._T, self._B, self._n, _ptr(per_sample_weights),
                 _ptr(optimizer_state) if optimizer != "sgd" else ctypes.c_void_p(0), float(learning_rate),
-                float(eps or 0.0), _ptr(grad_psw), _ptr(self._plan_ws), self._plan_ws.numel(), _ptr(unique),
-                self._stream()))
+                float(eps or 0.0), _ptr(grad_psw), int(stochastic_rounding is not None),
+                stochastic_rounding[0] if stochastic_rounding else 0,
+                stochastic_rounding[1] if stochastic_rounding else 0, _ptr(self._plan_ws), self._plan_ws.numel(),
+                _ptr(unique), self._stream()))
         return grad_psw
 
     def flush(self):

@@ -121,8 +121,12 @@ class CachedLookupFunction(torch.autograd.Function):
             kind = "sgd"
         else:
             kind = "adagrad"
+        rounding = None
+        if module.stochastic_rounding and kind == "adagrad" and weights.dtype == torch.float16:
+            rounding = table_batched_embeddings._rounding_stream(weights.device)
         grad_per_sample_weight = module.row_cache.backward(
-            kind, grad_output, per_sample_weights, module.optimizer_state, module.learning_rate, module.eps)
+            kind, grad_output, per_sample_weights, module.optimizer_state, module.learning_rate, module.eps,
+            rounding)
         empty_grad = None
         if ctx.needs_input_grad[0]:
             empty_grad = torch.sparse_coo_tensor(

@@ -147,6 +147,45 @@ def test_staging_leaves_cache_state_as_the_model_says(oracle, stage_slots):
     assert saw_uncached == (stage_slots == 9)
 
 
+def test_cached_stochastic_rounding_equals_uncached_bit_exact():
+    """fp16 weights with stochastic rounding: the random word of a weight is keyed by its place
+    in the table, so the rows come out bit-identical whether they are updated in a cache slot, a
+    staging row or the backing table."""
+    import ctypes
+    import tbe_native
+    rs = np.random.RandomState(8)
+    T, rows, B, L, D = 2, [900, 150], 40, 8, 64
+    table_offsets = dev(np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
+    total = sum(rows)
+    start = (torch.rand(total, D, device=DEV) * 0.02 - 0.01).half()
+    plain_w, cached_w = start.clone(), start.clone()
+    plain_state, cached_state = torch.zeros(total, device=DEV), torch.zeros(total, device=DEV)
+    cache = tc.RowCache(cached_w, 2 * 64, "lru", stage_slots=50)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    for step in range(4):
+        indices, offsets = _draw_batch(rs, T, rows, B, L, 1.2)
+        idx, off = dev(indices), dev(offsets)
+        go = torch.randn(B, T, D, device=DEV).half()
+        lay = tbe_native.backward_workspace_layout(indices.size, D, tbe_native.DTYPE_F16, T)
+        ws = torch.empty(lay.total_bytes, dtype=torch.uint8, device=DEV)
+        tbe_native.check(tbe_native.load().tbe_backward_exact_adagrad_stochastic(
+            vp(go), vp(plain_w), tbe_native.DTYPE_F16, total, 0, D, vp(table_offsets), T, vp(idx), indices.size,
+            vp(off), B, None, vp(plain_state), 0.05, 0.1, None, 99, 4 * step, vp(ws), ws.numel(),
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        cache.prepare(table_offsets, idx, off)
+        cache.backward("adagrad", go, None, cached_state, 0.05, 0.1, stochastic_rounding=(99, 4 * step))
+        st = cache.stats()
+        assert st["staged"] > 0 and st["uncached"] > 0 and st["hits"] + st["inserted"] > 0
+    cache.flush()
+    torch.cuda.synchronize()
+    assert torch.equal(cached_w, plain_w) and torch.equal(cached_state, plain_state)
+    # and the rounding is really stochastic: round-to-nearest gives other bits
+    rn_w = start.clone()
+    ext.backward_exact_adagrad(go, rn_w, table_offsets, idx, off, None, torch.zeros(total, device=DEV), 0.05, 0.1,
+                               False, 1)
+    assert not torch.equal(rn_w, start)
+
+
 def test_flush_before_any_step_and_empty_batch():
     backing = torch.randn(100, 16, device=DEV)
     before = backing.clone()
