@@ -226,6 +226,9 @@ template <> __device__ __forceinline__ double from_acc<double, double>(double x)
 __device__ __forceinline__ float shfl_idx(float v, int src) { return __shfl(v, src, kWave); }
 __device__ __forceinline__ int shfl_idx(int v, int src) { return __shfl(v, src, kWave); }
 __device__ __forceinline__ double shfl_idx(double v, int src) { return __shfl(v, src, kWave); }
+__device__ __forceinline__ int64_t shfl_idx(int64_t v, int src) {
+  return static_cast<int64_t>(__shfl(static_cast<long long>(v), src, kWave));
+}
 __device__ __forceinline__ float shfl_x(float v, int m) { return __shfl_xor(v, m, kWave); }
 __device__ __forceinline__ double shfl_x(double v, int m) { return __shfl_xor(v, m, kWave); }
 

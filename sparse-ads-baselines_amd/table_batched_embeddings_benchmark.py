@@ -22,9 +22,22 @@ import table_batched_embeddings_ops as ops
 HBM_PEAK_GBPS = 8000.0
 
 
+KERNEL_TIMES = False  # --kernels: also log the average duration of every library kernel of an op
+
+
 def time_calls(iters, fn):
     fn()
     torch.cuda.synchronize()
+    if KERNEL_TIMES:
+        import tbe_native
+        with tbe_native.profile() as prof:
+            for _ in range(3):
+                fn()
+        per_kernel = {}
+        for name, ms in prof.launches:
+            per_kernel.setdefault(name, []).append(ms)
+        logging.info("  kernels (us x launches per call): %s", ", ".join(
+            "%s %.1f x%d" % (k, 1e3 * sum(v) / len(v), len(v) // 3) for k, v in per_kernel.items()))
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
     start.record()
@@ -116,10 +129,13 @@ def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
 @click.option("--fp16", is_flag=True, default=False)
 @click.option("--managed", is_flag=True, default=False)
 @click.option("--mixed", is_flag=True, default=False)
+@click.option("--kernels", is_flag=True, default=False, help="Log per-kernel times of every op")
 @click.option("--alpha", default=0.0, help="Zipf exponent of the indices (0 = uniform)")
 @click.option("--seed", default=42)
-def cli(num_tables, num_embeddings, embedding_dim, batch_size, bag_size, iters, remote, fp16, managed, mixed, alpha,
-        seed):
+def cli(num_tables, num_embeddings, embedding_dim, batch_size, bag_size, iters, remote, fp16, managed, mixed, kernels,
+        alpha, seed):
+    global KERNEL_TIMES
+    KERNEL_TIMES = kernels
     logging.basicConfig(level=logging.INFO, stream=sys.stderr)
     if remote:
         raise click.UsageError("--remote (cluster submission) is not available; run the benchmark locally")
