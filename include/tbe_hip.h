@@ -88,8 +88,8 @@ TBE_API int tbe_forward(const void *weights, int32_t dtype, int32_t D,
  * the first five regions hold the intermediate results that the parity gates
  * inspect (all int32):
  *   keys              [N]   table_offsets[t] + indices[p]             (tbe.cu:1495); written by
- *                           tbe_backward_mixed only -- the uniform-D entry points sort the
- *                           indices table by table and leave this region untouched
+ *                           the stage entry point tbe_linearize only -- the backward entry points
+ *                           sort the indices table by table and leave this region untouched
  *   keys_sorted       [N]   stable ascending sort of keys             (tbe.cu:1639-1655)
  *   positions_sorted  [N]   position p of each sorted key (IndexInfo.indices_idx, tbe.cu:1217)
  *   segment_starts    [U+1] first sorted position of each unique key, then N (tbe.cu:1523-1539)
@@ -253,7 +253,8 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
  * tbe_backward_mixed replaces batched_embedding_backward_adagrad_exact_mixed_D_cuda
  * (:1350-1469, "backward_exact_adagrad_mixed_D", .cpp:64), serves the approximate variant
  * (.cpp:63) and adds exact SGD; per-sample weights as in tbe_backward_exact_adagrad;
- * stochastic_rounding / seed / offset as in tbe_backward_exact_adagrad_stochastic.  The
+ * stochastic_rounding / seed / offset as in tbe_backward_exact_adagrad_stochastic;
+ * max_table_rows as in tbe_backward_sgd (0 = unknown).  The
  * workspace is a backward workspace sized with tbe_backward_workspace_layout(N, 4, dtype, T).
  */
 TBE_API int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp16_vector_width,
@@ -264,7 +265,7 @@ TBE_API int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp16_v
                               const void *per_sample_weights, void *output, void *stream);
 
 TBE_API int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void *weights, int32_t dtype,
-                               int32_t fp16_vector_width, int64_t total_rows,
+                               int32_t fp16_vector_width, int64_t total_rows, int64_t max_table_rows,
                                const int64_t *table_offsets, const int32_t *table_dim_offsets,
                                const int32_t *dim_offsets, int32_t total_D, int32_t T,
                                const int32_t *indices, int64_t num_indices,

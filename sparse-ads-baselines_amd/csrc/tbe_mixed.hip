@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
   }
 }
 
-// keys[p] = table_dim_offsets[t] + indices[p]; grad_rows[p] = b * T + t.
+// keys[p] = table_dim_offsets[t] + indices[p] (skipped when `keys` is null); grad_rows[p] = b * T + t.
 __global__ __launch_bounds__(kBlockThreads) void linearize_mixed_kernel(
     const int32_t *__restrict__ table_dim_offsets, const int32_t *__restrict__ indices,
     const int32_t *__restrict__ offsets, int B, int num_tables, int num_bags,
@@ -108,12 +108,16 @@ __global__ __launch_bounds__(kBlockThreads) void linearize_mixed_kernel(
   const int bag = static_cast<int>(bag64);
   const int t = bag / B;
   const int b = bag - t * B;
-  const int32_t row0 = table_dim_offsets[t];
   const int32_t grow = b * num_tables + t;
   const int end = offsets[bag + 1];
-  for (int p = offsets[bag] + static_cast<int>(gid % kLanes); p < end; p += kLanes) {
-    keys[p] = row0 + indices[p];
-    grad_rows[p] = grow;
+  if (keys) {
+    const int32_t row0 = table_dim_offsets[t];
+    for (int p = offsets[bag] + static_cast<int>(gid % kLanes); p < end; p += kLanes) {
+      keys[p] = row0 + indices[p];
+      grad_rows[p] = grow;
+    }
+  } else {
+    for (int p = offsets[bag] + static_cast<int>(gid % kLanes); p < end; p += kLanes) grad_rows[p] = grow;
   }
 }
 
@@ -704,7 +708,7 @@ extern "C" int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp1
 
 extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void *weights,
                                   int32_t dtype, int32_t fp16_vector_width, int64_t total_rows,
-                                  const int64_t *table_offsets, const int32_t *table_dim_offsets,
+                                  int64_t max_table_rows, const int64_t *table_offsets, const int32_t *table_dim_offsets,
                                   const int32_t *dim_offsets, int32_t total_D, int32_t T,
                                   const int32_t *indices, int64_t num_indices,
                                   const int32_t *offsets, int32_t B,
@@ -740,6 +744,7 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   if (int rc = validate_mixed(name, a)) return rc;
   TBE_REQUIRE(grad_output && table_dim_offsets, "%s: null pointer argument", name);
   TBE_REQUIRE(total_rows > 0 && total_rows < INT32_MAX, "%s: total_rows out of range", name);
+  TBE_REQUIRE(max_table_rows >= 0, "%s: max_table_rows must not be negative", name);
   TBE_REQUIRE(a.optimizer == kOptSgd || optimizer_state, "%s: optimizer_state is null", name);
   TBE_REQUIRE((per_sample_weights == nullptr) == (grad_per_sample_weights == nullptr),
               "%s: per_sample_weights and grad_per_sample_weights must both be given or both be null", name);
@@ -755,9 +760,12 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   const int64_t num_bags = static_cast<int64_t>(T) * B;
   TBE_LAUNCH("linearize_mixed", s, linearize_mixed_kernel,
              dim3(static_cast<unsigned>(ceil_div(num_bags * 16, kBlockThreads))), dim3(kBlockThreads),
-             table_dim_offsets, indices, offsets, B, T, static_cast<int>(num_bags), i32(l.keys), i32(l.grad_rows));
-  int rc = sort_pairs(i32(l.keys), nullptr, i32(l.keys_sorted), i32(l.positions_sorted), num_indices,
-                      key_bits_for(total_rows), ws + l.sort_scratch, s, nullptr);
+             table_dim_offsets, indices, offsets, B, T, static_cast<int>(num_bags), nullptr, i32(l.grad_rows));
+  // every table's indices are sorted on their own; the last pass adds the table's first row id
+  const int64_t largest = (max_table_rows > 0 && max_table_rows < total_rows) ? max_table_rows : total_rows;
+  const SortTables tables{offsets, B, T, table_dim_offsets};
+  int rc = sort_pairs(indices, nullptr, i32(l.keys_sorted), i32(l.positions_sorted), num_indices,
+                      key_bits_for(largest), ws + l.sort_scratch, s, &tables);
   if (rc) return rc;
   rc = find_segments(i32(l.keys_sorted), num_indices, i32(l.segment_starts), i32(l.num_unique), nullptr,
                      ws + l.segment_scratch, s, /*clear_queue_counters=*/true);

@@ -59,12 +59,13 @@ _table_rows = {}  # id(table_offsets) -> (weak reference, tensor version, total_
 def max_table_rows(table_offsets, total_rows):
     """Rows of the largest table, read back from `table_offsets` once per tensor (one device to
     host copy, then cached for as long as the tensor lives and is not written).  The backward
-    sorts that many key bits per table instead of the bits of `total_rows`."""
+    sorts that many key bits per table instead of the bits of `total_rows`.  total_rows=None:
+    `table_offsets` has T+1 entries and ends with the total."""
     ident = id(table_offsets)
     hit = _table_rows.get(ident)
     if hit is not None and hit[0]() is table_offsets and hit[1:3] == (table_offsets._version, total_rows):
         return hit[3]
-    starts = table_offsets.cpu().tolist() + [total_rows]
+    starts = table_offsets.cpu().tolist() + ([total_rows] if total_rows is not None else [])
     sizes = [b - a for a, b in zip(starts, starts[1:])]
     largest = max(sizes) if min(sizes) >= 0 and starts[0] >= 0 else 0  # 0: unknown, sort all the bits
     ref = weakref.ref(table_offsets, lambda _, ident=ident: _table_rows.pop(ident, None))
@@ -335,7 +336,7 @@ def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_of
     with torch.cuda.device(weights.device):
         _native.check(_native.load().tbe_backward_mixed(
             optimizer, _ptr(grad_output), _ptr(weights), code, _fp16_vector_width(dim_offsets), total_rows,
-            _ptr(table_offsets), _ptr(table_dim_offsets), _ptr(dim_offsets), int(total_D), T, _ptr(indices),
+            max_table_rows(table_dim_offsets, None), _ptr(table_offsets), _ptr(table_dim_offsets), _ptr(dim_offsets), int(total_D), T, _ptr(indices),
             indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state), float(learning_rate),
             float(eps or 0.0), _ptr(grad_indice_weights), int(stochastic), seed, offset, _ptr(ws), ws.numel(),
             _stream(weights.device)))
