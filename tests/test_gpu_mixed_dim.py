@@ -44,8 +44,22 @@ def test_forward_mixed_matches_oracle(oracle, tables, weighted, dtype):
 @pytest.mark.parametrize("mode", ["sgd", "adagrad", "adagrad_weighted"])
 @pytest.mark.parametrize("tables", TABLE_SETS)
 def test_backward_mixed_matches_oracle(oracle, tables, mode, dtype):
+    _check_backward_mixed(oracle, tables, mode, dtype, B=23, L=8)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("mode", ["sgd", "adagrad", "adagrad_weighted"])
+def test_backward_mixed_hot_rows(oracle, mode, dtype):
+    """Thousands of lookups per table: rows with one occurrence (strip fast path), a few (strip
+    batches), 17..256 (one wavefront per row) and more than 256 (16 wavefronts per row), also in
+    a table whose rows are wider than 64 vectors, and more than 64 unique rows per table."""
+    tables = [(3, 520), (2000, 36), (5, 64), (4000, 128), (1, 8), (700, 200)]
+    _check_backward_mixed(oracle, tables, mode, dtype, B=300, L=24)
+
+
+def _check_backward_mixed(oracle, tables, mode, dtype, B, L):
     weighted = mode.endswith("weighted")
-    p = make_mixed_problem(len(tables) + 7, tables, B=23, L=8, dtype=dtype, weighted=weighted)
+    p = make_mixed_problem(len(tables) + 7, tables, B=B, L=L, dtype=dtype, weighted=weighted)
     optimizer = "sgd" if mode == "sgd" else "adagrad"
     w_ref = p["weights"].copy()
     st_dtype = np.float64 if dtype == np.float64 else np.float32
