@@ -142,3 +142,19 @@ def test_mixed_bad_arguments():
     with pytest.raises(RuntimeError, match="multiple of 4"):
         ext.forward_mixed_D(w, torch.tensor([0, 6], device=DEV), torch.tensor([0, 6], dtype=torch.int32, device=DEV),
                             6, i32[:1], i32[:2], None, 200, 1, False)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_backward_mixed_random_sweep(oracle, seed):
+    """Seeded random table sets: 1..12 tables, rows from 1 to thousands, widths from 4 to wider
+    than a wavefront pass (power-of-two and odd vector counts), bags from a handful to hundreds,
+    so that single-occurrence rows, batches, wavefront-per-row and workgroup-per-row all occur."""
+    rs = np.random.RandomState(500 + seed)
+    T = int(rs.choice([1, 2, 3, 6, 12]))
+    tables = [(int(rs.choice([1, 3, 40, 600, 5000])), int(rs.choice([4, 8, 12, 20, 32, 64, 100, 128, 256, 264, 520])))
+              for _ in range(T)]
+    dtype = [np.float32, np.float16, np.float64][seed % 3]
+    mode = ["sgd", "adagrad", "adagrad_weighted"][(seed // 3) % 3]
+    B = int(rs.choice([1, 9, 70, 400]))
+    L = int(rs.choice([1, 5, 20]))
+    _check_backward_mixed(oracle, tables, mode, dtype, B=B, L=L)
