@@ -1,4 +1,5 @@
-// Pooled forward gather-sum for gfx950: one 64-lane wavefront per bag.
+// Pooled forward gather-sum for gfx950: one 64-lane wavefront per bag (forward_kernel), or one
+// lane group per bag for short bags of narrow rows (forward_grouped_kernel).
 //
 // A row of D elements is `chunks` 16-byte vectors.  `chunks` consecutive lanes
 // own one row at a time, so one wavefront-wide load instruction fetches
@@ -125,6 +126,102 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
   }
 }
 
+// Narrow rows (4, 8 or 16 vectors) and short bags: one lane *group* per bag, 64 / CHUNKS bags
+// per wavefront.  A bag of 20 rows keeps a wavefront-per-bag kernel busy for one partly filled
+// batch and pays a cross-group reduction; here every group walks its own bag (32 indices fetched
+// per step, up to 8 independent row loads in flight per lane), nothing is reduced across lanes
+// and the instruction stream is shared by all the wavefront's bags.  Same sums as
+// forward_kernel in a different order (each lane adds its bag's rows in bag order).
+template <typename T, int VEC, int CHUNKS, bool WEIGHTED, bool CACHED>
+__global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
+    const T *__restrict__ weights, const int32_t *__restrict__ table_offsets,
+    const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
+    const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D, int num_bags,
+    int64_t blocks_per_xcd, const int32_t *__restrict__ lookup_slots,
+    const T *__restrict__ cache_rows) {
+  using V = RowVec<T, VEC>;
+  using A = typename V::A;
+  using R = typename V::R;
+  constexpr int kGroups = kWave / CHUNKS;
+  constexpr int kPerLane = 32 / CHUNKS;        // indices held per lane: a step covers 32 lookups of every bag
+  constexpr int kStep = kPerLane * CHUNKS;
+  constexpr int kUnroll = CHUNKS < 8 ? CHUNKS : 8;
+  static_assert(CHUNKS == 4 || CHUNKS == 8 || CHUNKS == 16, "lane groups of 4, 8 or 16 vectors");
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int r = lane / CHUNKS;
+  const int c = lane - r * CHUNKS;
+  const int group_base = r * CHUNKS;
+  const int64_t wave_index = xcd_contiguous(blockIdx.x, blocks_per_xcd) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t bag64 = wave_index * kGroups + r;
+  const bool valid = bag64 < num_bags;
+  const int bag = static_cast<int>(valid ? bag64 : num_bags - 1);
+  const int t = bag / B;
+  const int b = bag - t * B;
+  const int start = offsets[bag];
+  const int end = valid ? offsets[bag + 1] : start;
+  const int64_t table_row0 = table_offsets[t];
+  const T *col = weights + static_cast<int64_t>(c) * VEC;
+
+  V acc;
+  acc.zero();
+  for (int base = start; __ballot(base < end) != 0ull; base += kStep) {
+    int idx[kPerLane], slot[kPerLane];
+    A w[kPerLane];
+#pragma unroll
+    for (int q = 0; q < kPerLane; ++q) {
+      const int p = base + q * CHUNKS + c;
+      idx[q] = 0;
+      slot[q] = -1;
+      w[q] = A(0);
+      if (p < end) {
+        idx[q] = __builtin_nontemporal_load(indices + p);
+        if constexpr (WEIGHTED) w[q] = to_acc(psw[p]);
+        if constexpr (CACHED) slot[q] = __builtin_nontemporal_load(lookup_slots + p);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < kPerLane; ++q) {
+      const int left = end - (base + q * CHUNKS);  // rows of this group's bag in this slice
+      if (__ballot(left > 0) == 0ull) break;
+#pragma unroll
+      for (int j0 = 0; j0 < CHUNKS; j0 += kUnroll) {
+        if (__ballot(j0 < left) == 0ull) break;
+        R raw[kUnroll];
+        A ww[kUnroll];
+        bool ok[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const int j = j0 + u;
+          ok[u] = j < left;
+          const int src = group_base + j;
+          const int i = shfl_idx(idx[q], src);
+          if constexpr (WEIGHTED) ww[u] = shfl_idx(w[q], src);
+          const T *row = col + (table_row0 + i) * D;
+          if constexpr (CACHED) {
+            const int s = shfl_idx(slot[q], src);
+            if (s >= 0) row = cache_rows + static_cast<int64_t>(s) * D + static_cast<int64_t>(c) * VEC;
+          }
+          if (ok[u]) raw[u] = V::load_raw(row);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          if (ok[u]) {
+            V x;
+            x.unpack(raw[u]);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+              if constexpr (WEIGHTED) acc.v[k] += x.v[k] * ww[u];
+              else acc.v[k] += x.v[k];
+            }
+          }
+        }
+      }
+    }
+  }
+  if (valid) acc.store(output + (static_cast<int64_t>(b) * num_tables + t) * D + static_cast<int64_t>(c) * VEC);
+}
+
 // Rows wider than 64 vectors: the wavefront walks the row in blocks of 64
 // vectors and sums the bag serially per block.
 template <typename T, int VEC, bool WEIGHTED, bool CACHED, int UNROLL>
@@ -212,6 +309,7 @@ struct ForwardArgs {
   void *output;
   const int32_t *lookup_slots;  // null unless the rows are fronted by the HBM row cache
   const void *cache_rows;
+  int64_t num_indices;
 };
 
 template <typename T, int VEC, bool WEIGHTED, bool CACHED>
@@ -230,7 +328,23 @@ void launch_forward(const ForwardArgs &a, const RowGeometry &g, hipStream_t stre
   TBE_LAUNCH("forward", stream, (forward_kernel<T, VEC, CH, WEIGHTED, CACHED, kUnroll>), grid, \
              block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, g.chunks,   \
              num_bags, per_xcd, a.lookup_slots, cr)
-  if (g.wide) {
+  // short bags of narrow rows: a lane group per bag instead of a wavefront per bag
+  const bool grouped = !g.wide && (g.tmpl == 4 || g.tmpl == 8 || g.tmpl == 16) &&
+                       a.num_indices <= static_cast<int64_t>(num_bags) * 48;
+  if (grouped) {
+    const int groups = kWave / g.tmpl;
+    const int64_t gblocks = ceil_div(ceil_div(num_bags, groups), kWavesPerBlock);
+    const int64_t gper_xcd = ceil_div(gblocks, kNumXcd);
+    const dim3 ggrid(static_cast<unsigned>(gper_xcd * kNumXcd));
+#define TBE_FWD_GROUPED(CH)                                                                       \
+  TBE_LAUNCH("forward", stream, (forward_grouped_kernel<T, VEC, CH, WEIGHTED, CACHED>), ggrid,    \
+             block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, num_bags,      \
+             gper_xcd, a.lookup_slots, cr)
+    if (g.tmpl == 4) TBE_FWD_GROUPED(4);
+    else if (g.tmpl == 8) TBE_FWD_GROUPED(8);
+    else TBE_FWD_GROUPED(16);
+#undef TBE_FWD_GROUPED
+  } else if (g.wide) {
     TBE_LAUNCH("forward_wide", stream, (forward_wide_kernel<T, VEC, WEIGHTED, CACHED, 4>), grid,
                block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, g.chunks,
                num_bags, per_xcd, a.lookup_slots, cr);
@@ -296,7 +410,7 @@ extern "C" int tbe_forward(const void *weights, int32_t dtype, int32_t D,
                            const void *per_sample_weights, void *output, void *stream) {
   using namespace tbe;
   const ForwardArgs a{weights, dtype, D, table_offsets, T, indices, offsets, B,
-                      per_sample_weights, output, nullptr, nullptr};
+                      per_sample_weights, output, nullptr, nullptr, num_indices};
   if (int rc = validate_forward("tbe_forward", a, num_indices)) return rc;
   return run_forward(a, static_cast<hipStream_t>(stream));
 }
@@ -311,11 +425,11 @@ extern "C" int tbe_forward_cached(const tbe_cache_t *cache, int32_t dtype, int32
   TBE_REQUIRE(cache && cache->rows && cache->backing_rows, "tbe_forward_cached: null cache");
   TBE_REQUIRE(lookup_slots || num_indices == 0, "tbe_forward_cached: null lookup_slots");
   const ForwardArgs a{cache->backing_rows, dtype, D, table_offsets, T, indices, offsets, B,
-                      per_sample_weights, output, lookup_slots, cache->rows};
+                      per_sample_weights, output, lookup_slots, cache->rows, num_indices};
   if (int rc = validate_forward("tbe_forward_cached", a, num_indices)) return rc;
   if (num_indices == 0) {
     const ForwardArgs plain{cache->backing_rows, dtype, D, table_offsets, T, indices, offsets, B,
-                            per_sample_weights, output, nullptr, nullptr};
+                            per_sample_weights, output, nullptr, nullptr, num_indices};
     return run_forward(plain, static_cast<hipStream_t>(stream));
   }
   return run_forward(a, static_cast<hipStream_t>(stream));
