@@ -135,18 +135,13 @@ struct MixedRow {
 // gradient rows per group are in flight).  A wavefront takes the batches first_batch,
 // first_batch + batch_stride, ...; its groups are combined into group 0 in a fixed tree.
 // Returns with G (valid in group 0) and w_old (valid in every group when WEIGHTED, else in
-// group 0).  pre_w / pre_g (have_pre): the packed row and the packed gradient row of the first
-// occurrence, requested by the caller ahead of time; first_* (have_first): position, bag and
-// weight of the first occurrence.
+// group 0).
 template <typename T, int VEC, bool WEIGHTED, int UNROLL>
 __device__ __forceinline__ void mixed_accumulate_narrow(
     const T *__restrict__ grad_output, const T *__restrict__ weights, const T *__restrict__ psw,
     T *__restrict__ grad_psw, int num_tables, int total_D,
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows, int lane,
-    const MixedRow &row, int first_batch, int batch_stride, bool have_first, int first_pos,
-    int first_bag, typename AccOf<T>::type first_w, bool have_pre,
-    const typename RowVec<T, VEC>::R &pre_w, const typename RowVec<T, VEC>::R &pre_g,
-    RowVec<T, VEC> &w_old, RowVec<T, VEC> &G) {
+    const MixedRow &row, int first_batch, int batch_stride, RowVec<T, VEC> &w_old, RowVec<T, VEC> &G) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -163,23 +158,16 @@ __device__ __forceinline__ void mixed_accumulate_narrow(
   const T *wrow = weights + row.row_element;
   const T *gcol = grad_output + row.dim_start;
   w_old.zero();
-  if (have_pre) {
-    if (active && (WEIGHTED || r == 0)) w_old.unpack(pre_w);
-  } else if (active && (WEIGHTED || r == 0)) {
-    w_old.load(wrow + col);
-  }
+  if (active && (WEIGHTED || r == 0)) w_old.load(wrow + col);
   G.zero();
   for (int base = row.seg_begin + first_batch * kWave; base < row.seg_end; base += batch_stride * kWave) {
     const int n = min(kWave, row.seg_end - base);
-    const bool first_batch_of_row = base == row.seg_begin;
-    int my_pos = first_pos, my_bag = first_bag;
-    A my_w = first_w;
-    if (!have_first || n > 1 || !first_batch_of_row) {
-      if (lane < n) {
-        my_pos = positions_sorted[base + lane];
-        my_bag = grad_rows[my_pos] / num_tables;
-        if constexpr (WEIGHTED) my_w = to_acc(psw[my_pos]);
-      }
+    int my_pos = 0, my_bag = 0;
+    A my_w = A(1);
+    if (lane < n) {
+      my_pos = positions_sorted[base + lane];
+      my_bag = grad_rows[my_pos] / num_tables;
+      if constexpr (WEIGHTED) my_w = to_acc(psw[my_pos]);
     }
     for (int j0 = 0; j0 < n; j0 += groups * UNROLL) {
       R raw[UNROLL];
@@ -191,10 +179,7 @@ __device__ __forceinline__ void mixed_accumulate_narrow(
         ok[k] = active && j < n;
         src[k] = ok[k] ? j : 0;
         const int64_t bag = shfl_idx(my_bag, src[k]);
-        if (ok[k]) {
-          if (k == 0 && have_pre && first_batch_of_row && j == 0) raw[k] = pre_g;
-          else raw[k] = V::load_raw(gcol + bag * total_D + col);
-        }
+        if (ok[k]) raw[k] = V::load_raw(gcol + bag * total_D + col);
       }
 #pragma unroll
       for (int k = 0; k < UNROLL; ++k) {
@@ -341,35 +326,68 @@ __device__ __forceinline__ void mixed_update_wide(
   }
 }
 
-// Short rows.  A wavefront takes strips of 64 consecutive unique rows.  What a row needs before
-// its first gradient row can be requested -- segment bounds, key, first position, table (from
-// the gradient row id b*T+t of the first occurrence), the table's width and offsets, optimizer
-// state -- is fetched for the 64 rows at once, one row per lane, so the dependent loads are paid
-// per strip; the rows and first gradient rows of four rows are requested before the first of them
-// is reduced, so a row with one occurrence (the common case) waits for no load of its own.
-// Rows of more than kShortSegment occurrences (the hot rows, which are neighbours in key order)
-// are not reduced here: their indices go to two queues that update_mixed_long_kernel drains --
-// one wavefront per row of at most kChunkLen occurrences, one workgroup of 16 wavefronts per
-// longer row -- so that they spread over the machine.
-template <typename T, int VEC, int OPT, bool WEIGHTED, int UNROLL>
-__global__ __launch_bounds__(kBlockThreads) void update_mixed_kernel(
+// Short rows.  A wavefront takes strips of 64 consecutive unique rows.
+//
+// First, one row per lane: what a row needs before its gradient rows can be requested -- segment
+// bounds, key, positions, bag and table of each occurrence (from the gradient row ids b*T+t),
+// the table's width and offsets, optimizer state -- is fetched for the 64 rows at once, so the
+// dependent loads are paid per strip.  Rows of more than kMixedShort occurrences (the hot rows,
+// which are neighbours in key order) and rows wider than 64 vectors are not reduced here: their
+// indices go to two queues that update_mixed_long_kernel drains -- one wavefront per row of at
+// most kChunkLen occurrences, one workgroup of 16 wavefronts per longer row -- so that they
+// spread over the machine.  The other rows leave a 32-byte record in LDS (in row order), and
+// every occurrence of theirs leaves the element offset of its gradient row (and its position,
+// for per-sample weights).
+//
+// Then, one row per lane *group*, 64 / group_lanes rows at a time, so the instruction stream is
+// shared by several rows.  The group size fits the widest row of the strip (a strip spans a table
+// boundary now and then).  Each group adds its row's occurrences in order.  The packed row and
+// the first kMixedAhead packed gradient rows of an iteration are requested one iteration ahead.
+//
+// bag_magic / bag_shift: b = (grow * bag_magic) >> bag_shift for every gradient row id
+// grow = b*T+t < 2^31 (division by the invariant T).
+// Empty statement that reads and "rewrites" the registers of x: what was loaded into x has
+// arrived when it is passed.
+template <typename X> __device__ __forceinline__ void register_fence(X &x) {
+  static_assert(sizeof(X) % 4 == 0, "whole registers");
+  uint32_t words[sizeof(X) / 4];
+  __builtin_memcpy(words, &x, sizeof(X));
+#pragma unroll
+  for (size_t i = 0; i < sizeof(X) / 4; ++i) asm volatile("" : "+v"(words[i]));
+  __builtin_memcpy(&x, words, sizeof(X));
+}
+
+constexpr int kMixedShort = 8;
+constexpr int kMixedAhead = 4;
+template <typename T, int VEC, int OPT, bool WEIGHTED>
+__global__ __launch_bounds__(kBlockThreads, (WEIGHTED || VEC == 8) ? 4 : 5) void update_mixed_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
     T *__restrict__ grad_psw, const int64_t *__restrict__ table_offsets,
     const int32_t *__restrict__ table_dim_offsets, const int32_t *__restrict__ dim_offsets,
-    int num_tables, int total_D, const int32_t *__restrict__ keys_sorted,
-    const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
-    const int32_t *__restrict__ segment_starts, int32_t *__restrict__ counters,
-    int32_t *__restrict__ long_rows, int32_t *__restrict__ huge_rows, float lr, float eps,
-    StochasticRounding sr) {
+    int num_tables, uint32_t bag_magic, int bag_shift, int total_D,
+    const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ positions_sorted,
+    const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ segment_starts,
+    int32_t *__restrict__ counters, int32_t *__restrict__ long_rows,
+    int32_t *__restrict__ huge_rows, float lr, float eps, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
+  static_assert(sizeof(A) == 4 || sizeof(A) == 8, "optimizer state is float or double");
+  // a row's record: {occurrences, first slot, key, D}, {first element of the row (64 bits), state}
+  __shared__ int4 s_row[kWavesPerBlock][kWave][2];
+  // occurrences of a strip's short rows: at most 64 rows of kMixedShort occurrences
+  __shared__ int s_goff[kWavesPerBlock][kWave * kMixedShort];
+  __shared__ int s_pos[kWavesPerBlock][WEIGHTED ? kWave * kMixedShort : 1];
   const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
   const int U = counters[0];
-  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + wave;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
   const int64_t num_strips = (static_cast<int64_t>(U) + kWave - 1) / kWave;
+  auto bag_of = [&](int grow) {
+    return static_cast<int>((static_cast<uint64_t>(static_cast<uint32_t>(grow)) * bag_magic) >> bag_shift);
+  };
 
   for (int64_t strip = wave_id; strip < num_strips; strip += stride) {
     const int64_t u0 = strip * kWave;
@@ -379,22 +397,28 @@ __global__ __launch_bounds__(kBlockThreads) void update_mixed_kernel(
     const int l_begin = segment_starts[my_u];
     const int l_end = segment_starts[my_u + 1];
     const int32_t l_key = keys_sorted[l_begin];
-    const int l_pos0 = positions_sorted[l_begin];
-    const int l_grow0 = grad_rows[l_pos0];
-    const int l_bag0 = l_grow0 / num_tables;
-    const int l_table = l_grow0 - l_bag0 * num_tables;
+    // the first kMixedShort occurrences (the last one again, past the row's end)
+    int l_pos[kMixedShort], l_bag[kMixedShort];
+#pragma unroll
+    for (int i = 0; i < kMixedShort; ++i) l_pos[i] = positions_sorted[min(l_begin + i, l_end - 1)];
+#pragma unroll
+    for (int i = 0; i < kMixedShort; ++i) l_bag[i] = grad_rows[l_pos[i]];
+    const int bag0 = bag_of(l_bag[0]);
+    const int l_table = l_bag[0] - bag0 * num_tables;
+#pragma unroll
+    for (int i = 1; i < kMixedShort; ++i) l_bag[i] = bag_of(l_bag[i]);
+    l_bag[0] = bag0;
     const int l_dim_start = dim_offsets[l_table];
     const int l_D = dim_offsets[l_table + 1] - l_dim_start;
     const int64_t l_row_element =
         table_offsets[l_table] + static_cast<int64_t>(l_key - table_dim_offsets[l_table]) * l_D;
     A l_state = A(0);
     if constexpr (OPT == kOptAdagrad) l_state = state[l_key];
-    A l_w0 = A(1);
-    if constexpr (WEIGHTED) l_w0 = to_acc(psw[l_pos0]);
 
-    // hand the longer rows of the strip to their queues (one atomic per strip and queue)
-    const bool is_long = lane < rows_here && l_end - l_begin > kShortSegment;
-    const bool is_huge = is_long && l_end - l_begin > kChunkLen;
+    // hand the longer rows of the strip to their queues (one atomic per strip and queue);
+    // rows wider than 64 vectors count as longer rows whatever their length
+    const bool is_huge = lane < rows_here && l_end - l_begin > kChunkLen;
+    const bool is_long = lane < rows_here && (l_end - l_begin > kMixedShort || l_D / VEC > kWave);
     const unsigned long long long_mask = __ballot(is_long);
     const unsigned long long huge_mask = __ballot(is_huge);
     const unsigned long long medium_mask = long_mask & ~huge_mask;
@@ -411,92 +435,175 @@ __global__ __launch_bounds__(kBlockThreads) void update_mixed_kernel(
       first_slot = shfl_idx(first_slot, 0);
       if (is_huge) huge_rows[first_slot + __popcll(huge_mask & ((1ull << lane) - 1ull))] = static_cast<int32_t>(my_u);
     }
+    const unsigned long long todo = ~long_mask & (rows_here == kWave ? ~0ull : ((1ull << rows_here) - 1ull));
+    if (todo == 0ull) continue;
 
-    // The bookkeeping of row j, read from lane j into scalar registers (j is the same in every lane).
-    auto lane_i32 = [](int v, int j) { return __builtin_amdgcn_readlane(v, j); };
-    auto lane_i64 = [&](int64_t v, int j) {
-      const unsigned int lo = static_cast<unsigned int>(__builtin_amdgcn_readlane(static_cast<int>(v), j));
-      const int hi = __builtin_amdgcn_readlane(static_cast<int>(v >> 32), j);
-      return (static_cast<int64_t>(hi) << 32) | lo;
-    };
-    auto row_of = [&](int j) {
-      return MixedRow{lane_i32(l_begin, j), lane_i32(l_end, j), lane_i32(l_key, j), lane_i32(l_dim_start, j),
-                      lane_i32(l_D, j), lane_i64(l_row_element, j)};
-    };
-    // requests the packed row and the packed first gradient row of row j (narrow rows only)
-    auto request = [&](int j, const MixedRow &row, R &w, R &g) {
-      const int chunks = row.D / VEC;
-      if (chunks > kWave) return false;
-      const int group_shift = chunks > 1 ? 32 - __builtin_clz(chunks - 1) : 0;
-      const int r = lane >> group_shift;
-      const int c = lane & ((1 << group_shift) - 1);
-      const int64_t col = static_cast<int64_t>(c) * VEC;
-      const int64_t bag = lane_i32(l_bag0, j);
-      if (c < chunks && (WEIGHTED || r == 0)) w = V::load_raw(weights + row.row_element + col);
-      if (c < chunks && r == 0) g = V::load_raw(grad_output + row.dim_start + bag * total_D + col);
-      return true;
-    };
-
-    // Short rows in blocks of kAhead: the loads of the whole block are requested before its first
-    // row is reduced, so kAhead rows' worth of memory traffic is in flight per wavefront.
-    constexpr int kAhead = 4;
-    unsigned long long todo = ~long_mask & (rows_here == kWave ? ~0ull : ((1ull << rows_here) - 1ull));
-    while (todo) {
-      int index[kAhead];
-      MixedRow rows[kAhead];
-      R pre_w[kAhead], pre_g[kAhead];
-      bool have_pre[kAhead];
+    // records and occurrences to LDS; the k-th short row of the strip gets record k, the lanes
+    // without a short row fill the records behind them with empty rows
+    const bool is_short = (todo >> lane) & 1ull;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const int num_short = __popcll(todo);
+    const int my_rank = is_short ? __popcll(todo & below) : num_short + __popcll(~todo & below);
+    const int my_len = is_short ? l_end - l_begin : 0;
+    int my_offset = my_len;
 #pragma unroll
-      for (int p = 0; p < kAhead; ++p) {
-        index[p] = -1;
-        have_pre[p] = false;
-        if (todo) {
-          index[p] = __ffsll(static_cast<long long>(todo)) - 1;
-          todo &= todo - 1;
-          rows[p] = row_of(index[p]);
-          have_pre[p] = request(index[p], rows[p], pre_w[p], pre_g[p]);
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int y = __shfl_up(my_offset, d, kWave);
+      if (lane >= d) my_offset += y;
+    }
+    my_offset -= my_len;  // exclusive prefix: first occurrence slot of the row
+    int st_lo = 0, st_hi = 0;
+    if constexpr (sizeof(A) == 4) {
+      st_lo = __builtin_bit_cast(int, l_state);
+    } else {
+      const long long bits = __builtin_bit_cast(long long, l_state);
+      st_lo = static_cast<int>(bits);
+      st_hi = static_cast<int>(bits >> 32);
+    }
+    s_row[wave][my_rank][0] = make_int4(my_len, my_offset, l_key, is_short ? l_D : 0);
+    s_row[wave][my_rank][1] =
+        make_int4(static_cast<int>(l_row_element), static_cast<int>(l_row_element >> 32), st_lo, st_hi);
+#pragma unroll
+    for (int i = 0; i < kMixedShort; ++i) {
+      if (i < my_len) {
+        s_goff[wave][my_offset + i] = l_bag[i] * total_D + l_dim_start;
+        if constexpr (WEIGHTED) s_pos[wave][my_offset + i] = l_pos[i];
+      }
+    }
+    int strip_D = is_short ? l_D : 0;
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) strip_D = max(strip_D, __shfl_xor(strip_D, m, kWave));
+    __builtin_amdgcn_wave_barrier();
+
+    const int max_chunks = strip_D / VEC;
+    const int group_shift = max_chunks > 1 ? 32 - __builtin_clz(max_chunks - 1) : 0;
+    const int group_lanes = 1 << group_shift;
+    const int groups = kWave >> group_shift;
+    const int r = lane >> group_shift;
+    const int c = lane & (group_lanes - 1);
+    const int col = c * VEC;
+
+    // Two sets of requested data take turns, so that nothing is copied from one to the other.
+    struct Fetched {
+      R w;
+      R raw[kMixedAhead];
+      A pw[kMixedAhead];
+    };
+    auto request = [&](int k0, Fetched &f) {
+      const int4 d0 = s_row[wave][k0 + r][0];
+      const int4 d1 = s_row[wave][k0 + r][1];
+      const int len = d0.x, slot0 = d0.y;
+      const bool active = col < d0.w;
+      const int64_t row_element =
+          (static_cast<int64_t>(d1.y) << 32) | static_cast<int64_t>(static_cast<uint32_t>(d1.x));
+      if (active) f.w = V::load_raw_streaming(weights + row_element + col);
+#pragma unroll
+      for (int u = 0; u < kMixedAhead; ++u) {
+        if (__ballot(u < len) == 0ull) break;
+        if (u < len && active) {
+          f.raw[u] = V::load_raw(grad_output + static_cast<int64_t>(s_goff[wave][slot0 + u]) + col);
+          if constexpr (WEIGHTED) f.pw[u] = to_acc(psw[s_pos[wave][slot0 + u]]);
         }
       }
+    };
+    // The compiler has to finish the loads of f here: placed before the next request, it keeps the
+    // wait for f from also waiting for that request.
+    auto landed = [&](Fetched &f) {
+      register_fence(f.w);
 #pragma unroll
-      for (int p = 0; p < kAhead; ++p) {
-        if (index[p] < 0) continue;
-        const int j = index[p];
-        const A state_old = __builtin_bit_cast(A, [&] {
-          if constexpr (sizeof(A) == 4) return lane_i32(__builtin_bit_cast(int, l_state), j);
-          else return lane_i64(__builtin_bit_cast(int64_t, l_state), j);
-        }());
-        if (have_pre[p] && rows[p].seg_end - rows[p].seg_begin == 1) {
-          // one occurrence, already requested: no batch to fetch, nothing to combine
-          const int chunks = rows[p].D / VEC;
-          V w_old, G;
-          w_old.zero();
-          G.zero();
-          if (lane < chunks) {
-            w_old.unpack(pre_w[p]);
-            G.unpack(pre_g[p]);
-          }
-          if constexpr (WEIGHTED) {
-            A dot = A(0);
+      for (int u = 0; u < kMixedAhead; ++u) {
+        register_fence(f.raw[u]);
+        if constexpr (WEIGHTED) register_fence(f.pw[u]);
+      }
+    };
+    auto consume = [&](int k0, Fetched &f) {
+      const int4 d0 = s_row[wave][k0 + r][0];
+      const int4 d1 = s_row[wave][k0 + r][1];
+      const int len = d0.x, slot0 = d0.y;
+      const int32_t key = d0.z;
+      const bool active = col < d0.w;
+      const int64_t row_element =
+          (static_cast<int64_t>(d1.y) << 32) | static_cast<int64_t>(static_cast<uint32_t>(d1.x));
+      A state_old;
+      if constexpr (sizeof(A) == 4) {
+        state_old = __builtin_bit_cast(A, d1.z);
+      } else {
+        state_old = __builtin_bit_cast(
+            A, (static_cast<long long>(d1.w) << 32) | static_cast<long long>(static_cast<uint32_t>(d1.z)));
+      }
+      V w_old, G, x;
+      w_old.unpack(f.w);
+      if constexpr (WEIGHTED) {  // lanes beside the row must not bring stale values into the dot products
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * G.v[i];
-            dot = group_sum<kWave, A>(dot, kWave, 0);  // lanes outside the row add 0
-            if (lane == 0) grad_psw[lane_i32(l_pos0, j)] = from_acc<T, A>(dot);
-            const A pw = shfl_idx(l_w0, j);
+        for (int i = 0; i < VEC; ++i) w_old.v[i] = active ? w_old.v[i] : A(0);
+      }
+      G.zero();
+      auto add = [&](int u, const R &packed, A weight) {
+        x.unpack(packed);
+        const bool ok = u < len && active;
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) G.v[i] *= pw;
-          }
-          mixed_apply_narrow<T, VEC, OPT>(weights, state, lr, eps, sr, lane, rows[p], state_old, w_old, G);
-        } else if (rows[p].D / VEC <= kWave) {
-          V w_old, G;
-          mixed_accumulate_narrow<T, VEC, WEIGHTED, UNROLL>(
-              grad_output, weights, psw, grad_psw, num_tables, total_D, positions_sorted, grad_rows, lane, rows[p], 0,
-              1, true, lane_i32(l_pos0, j), lane_i32(l_bag0, j), shfl_idx(l_w0, j), have_pre[p], pre_w[p], pre_g[p],
-              w_old, G);
-          mixed_apply_narrow<T, VEC, OPT>(weights, state, lr, eps, sr, lane, rows[p], state_old, w_old, G);
+        for (int i = 0; i < VEC; ++i) x.v[i] = ok ? x.v[i] : A(0);
+        if constexpr (WEIGHTED) {
+          weight = ok ? weight : A(1);
+          A dot = A(0);
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
+          for (int m = group_lanes >> 1; m > 0; m >>= 1) dot += shfl_x(dot, m);
+          if (u < len && c == 0) grad_psw[s_pos[wave][slot0 + u]] = from_acc<T, A>(dot);
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * weight;
         } else {
-          mixed_update_wide<T, VEC, OPT, WEIGHTED>(grad_output, weights, state, psw, grad_psw, num_tables, total_D,
-                                                   positions_sorted, grad_rows, lr, eps, sr, lane, rows[p], state_old);
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i];
         }
+      };
+#pragma unroll
+      for (int u = 0; u < kMixedAhead; ++u) {
+        if (__ballot(u < len) == 0ull) break;
+        add(u, f.raw[u], f.pw[u]);
+      }
+      // occurrences kMixedAhead.. of the longer rows are fetched here
+      for (int i0 = kMixedAhead; __ballot(i0 < len) != 0ull; i0 += kMixedAhead) {
+        R raw[kMixedAhead];
+        A pw[kMixedAhead];
+#pragma unroll
+        for (int u = 0; u < kMixedAhead; ++u) {
+          pw[u] = A(1);
+          if (i0 + u < len && active) {
+            raw[u] = V::load_raw(grad_output + static_cast<int64_t>(s_goff[wave][slot0 + i0 + u]) + col);
+            if constexpr (WEIGHTED) pw[u] = to_acc(psw[s_pos[wave][slot0 + i0 + u]]);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kMixedAhead; ++u) add(i0 + u, raw[u], pw[u]);
+      }
+      A mult = static_cast<A>(lr);
+      if constexpr (OPT == kOptAdagrad) {
+        A gss = A(0);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) gss += G.v[i] * G.v[i];
+        for (int m = group_lanes >> 1; m > 0; m >>= 1) gss += shfl_x(gss, m);
+        const A s_new = state_old + gss;
+        if (len > 0 && c == 0) state[key] = s_new;
+        mult = mixed_multiplier<A>(s_new, lr, eps);
+      }
+      if (active) {
+        V w;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) w.v[i] = w_old.v[i] - G.v[i] * mult;
+        store_row<T, VEC, true>(weights + row_element + col, w, sr, row_element + col);
+      }
+    };
+    Fetched fa{}, fb{};
+    request(0, fa);
+    for (int k0 = 0; k0 < num_short; k0 += 2 * groups) {
+      landed(fa);
+      if (k0 + groups < num_short) request(k0 + groups, fb);
+      consume(k0, fa);
+      if (k0 + groups < num_short) {
+        landed(fb);
+        if (k0 + 2 * groups < num_short) request(k0 + 2 * groups, fa);
+        consume(k0 + groups, fb);
       }
     }
   }
@@ -520,7 +627,6 @@ __global__ __launch_bounds__((WAVES > 1 ? WAVES : kWavesPerBlock) * kWave) void 
     int queue_counter, const int32_t *__restrict__ queue, float lr, float eps, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
-  using R = typename V::R;
   constexpr int kRowsPerBlock = WAVES > 1 ? 1 : kWavesPerBlock;
   __shared__ A s_partial[WAVES > 1 ? WAVES : 1][WAVES > 1 ? kWave * VEC : 1];
   const int lane = threadIdx.x & (kWave - 1);
@@ -548,10 +654,9 @@ __global__ __launch_bounds__((WAVES > 1 ? WAVES : kWavesPerBlock) * kWave) void 
       continue;
     }
     V w_old, G;
-    const R none{};
     mixed_accumulate_narrow<T, VEC, WEIGHTED, UNROLL>(grad_output, weights, psw, grad_psw, num_tables, total_D,
                                                       positions_sorted, grad_rows, lane, row, wave_in_row, WAVES,
-                                                      false, 0, 0, A(1), false, none, none, w_old, G);
+                                                      w_old, G);
     if constexpr (WAVES > 1) {
       __syncthreads();  // the previous row's partial sums have been read
       if (lane < chunks) {
@@ -619,16 +724,24 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
   A *st = static_cast<A *>(a.state);
   const T *psw = static_cast<const T *>(a.psw);
   T *gpsw = static_cast<T *>(a.grad_psw);
-  // queues of row indices: rows of 17..256 occurrences (at most n / 17 of them) and longer rows (n / 257)
-  int32_t *long_rows = i32(l.chunk_segments);
+  // queues of row indices: rows of 9..256 occurrences or wider than 64 vectors (at most one per
+  // lookup) and rows of more occurrences (n / 257)
+  int32_t *long_rows = i32(l.segment_ids);
   int32_t *huge_rows = i32(l.long_segments);
   const int64_t want = ceil_div(ceil_div(a.n, kWave), kWavesPerBlock);
   const dim3 grid(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want, 256 * 32))));
-  TBE_LAUNCH("update_mixed", stream, (update_mixed_kernel<T, VEC, OPT, WEIGHTED, 4>), grid, dim3(kBlockThreads),
-             go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, a.total_D,
-             i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
+  // b = grow / T for grow < 2^31 as a multiplication and a shift: magic = ceil(2^(31 + s) / T) with
+  // s = ceil(log2 T) fits 32 bits and gives the exact quotient
+  int log2_T = 0;
+  while ((int64_t{1} << log2_T) < a.T) ++log2_T;
+  const int bag_shift = 31 + log2_T;
+  const uint32_t bag_magic =
+      static_cast<uint32_t>(((uint64_t{1} << bag_shift) + static_cast<uint64_t>(a.T) - 1) / static_cast<uint64_t>(a.T));
+  TBE_LAUNCH("update_mixed", stream, (update_mixed_kernel<T, VEC, OPT, WEIGHTED>), grid, dim3(kBlockThreads),
+             go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, bag_magic, bag_shift,
+             a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
              i32(l.num_unique), long_rows, huge_rows, a.lr, a.eps, a.sr);
-  const int64_t want_long = ceil_div(a.n / (kShortSegment + 1) + 1, kWavesPerBlock);
+  const int64_t want_long = ceil_div(a.n, kWavesPerBlock);
   const dim3 grid_long(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 8))));
   TBE_LAUNCH("update_mixed_long", stream, (update_mixed_long_kernel<T, VEC, OPT, WEIGHTED, 4, 1>), grid_long,
              dim3(kBlockThreads), go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T,
@@ -745,6 +858,8 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   TBE_REQUIRE(grad_output && table_dim_offsets, "%s: null pointer argument", name);
   TBE_REQUIRE(total_rows > 0 && total_rows < INT32_MAX, "%s: total_rows out of range", name);
   TBE_REQUIRE(max_table_rows >= 0, "%s: max_table_rows must not be negative", name);
+  TBE_REQUIRE(static_cast<int64_t>(B) * total_D < INT32_MAX, "%s: grad_output of B*total_D = %lld elements is too large",
+              name, static_cast<long long>(B) * total_D);
   TBE_REQUIRE(a.optimizer == kOptSgd || optimizer_state, "%s: optimizer_state is null", name);
   TBE_REQUIRE((per_sample_weights == nullptr) == (grad_per_sample_weights == nullptr),
               "%s: per_sample_weights and grad_per_sample_weights must both be given or both be null", name);

@@ -51,10 +51,21 @@ def test_backward_mixed_matches_oracle(oracle, tables, mode, dtype):
 @pytest.mark.parametrize("mode", ["sgd", "adagrad", "adagrad_weighted"])
 def test_backward_mixed_hot_rows(oracle, mode, dtype):
     """Thousands of lookups per table: rows with one occurrence (strip fast path), a few (strip
-    batches), 17..256 (one wavefront per row) and more than 256 (16 wavefronts per row), also in
+    batches), 9..256 (one wavefront per row) and more than 256 (16 wavefronts per row), also in
     a table whose rows are wider than 64 vectors, and more than 64 unique rows per table."""
     tables = [(3, 520), (2000, 36), (5, 64), (4000, 128), (1, 8), (700, 200)]
     _check_backward_mixed(oracle, tables, mode, dtype, B=300, L=24)
+
+
+@pytest.mark.parametrize("T", [37, 100])
+@pytest.mark.parametrize("mode", ["sgd", "adagrad_weighted"])
+def test_backward_mixed_many_small_tables(oracle, mode, T):
+    """Dozens of tables of a few rows each: a strip of 64 unique rows spans many tables of
+    different widths (narrow, odd vector counts, wider than 64 vectors side by side), and the
+    bag of a gradient row id b*T+t is found for table counts that are not small powers of two."""
+    widths = [4, 8, 12, 260, 64, 20, 36, 128, 4, 100]
+    tables = [(1 + (3 * t) % 9, widths[t % len(widths)]) for t in range(T)]
+    _check_backward_mixed(oracle, tables, mode, np.float32, B=50, L=3)
 
 
 def _check_backward_mixed(oracle, tables, mode, dtype, B, L):
