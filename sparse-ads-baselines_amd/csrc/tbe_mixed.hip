@@ -131,11 +131,12 @@ struct MixedRow {
 
 // Narrow rows (at most 64 vectors): `chunks` = D / VEC consecutive lanes form a lane group, the
 // 64 / chunks groups split the occurrences of a 64-position batch (the batch's positions,
-// gradient rows and weights are fetched with one load per lane, then UNROLL independent
+// gradient rows and weights are fetched with one load per lane, then up to UNROLL independent
 // gradient rows per group are in flight).  A wavefront takes the batches first_batch,
-// first_batch + batch_stride, ...; its groups are combined into group 0 in a fixed tree.
-// Returns with G (valid in group 0) and w_old (valid in every group when WEIGHTED, else in
-// group 0).
+// first_batch + batch_stride, ...; the positions of a batch are requested two batches ahead and
+// its gradient row ids and weights one batch ahead, so a batch waits for gradient rows only.
+// The groups are combined into group 0 in a fixed tree.  Returns with G (valid in group 0) and
+// w_old (valid in every group when WEIGHTED, else in group 0).
 template <typename T, int VEC, bool WEIGHTED, int UNROLL>
 __device__ __forceinline__ void mixed_accumulate_narrow(
     const T *__restrict__ grad_output, const T *__restrict__ weights, const T *__restrict__ psw,
@@ -155,20 +156,33 @@ __device__ __forceinline__ void mixed_accumulate_narrow(
   const int c = lane & (group_lanes - 1);
   const bool active = c < chunks;
   const int64_t col = static_cast<int64_t>(c) * VEC;
+  const int64_t safe_col = active ? col : 0;
   const T *wrow = weights + row.row_element;
   const T *gcol = grad_output + row.dim_start;
   w_old.zero();
   if (active && (WEIGHTED || r == 0)) w_old.load(wrow + col);
   G.zero();
-  for (int base = row.seg_begin + first_batch * kWave; base < row.seg_end; base += batch_stride * kWave) {
+  const int step = batch_stride * kWave;
+  // lanes past the row's end ask for its first position: any valid index will do
+  auto position_at = [&](int64_t i) { return positions_sorted[i < row.seg_end ? i : row.seg_begin]; };
+  int base = row.seg_begin + first_batch * kWave;
+  int pos_now = position_at(base + lane);
+  int pos_next = position_at(static_cast<int64_t>(base) + step + lane);
+  int grow_now = grad_rows[pos_now];
+  A w_now = A(1);
+  if constexpr (WEIGHTED) w_now = to_acc(psw[pos_now]);
+  for (; base < row.seg_end; base += min(step, row.seg_end - base)) {
     const int n = min(kWave, row.seg_end - base);
-    int my_pos = 0, my_bag = 0;
-    A my_w = A(1);
-    if (lane < n) {
-      my_pos = positions_sorted[base + lane];
-      my_bag = grad_rows[my_pos] / num_tables;
-      if constexpr (WEIGHTED) my_w = to_acc(psw[my_pos]);
-    }
+    const int my_pos = pos_now;
+    const int my_bag = grow_now / num_tables;
+    const A my_w = w_now;
+    pos_now = pos_next;
+    pos_next = position_at(static_cast<int64_t>(base) + 2 * step + lane);
+    grow_now = grad_rows[pos_now];
+    if constexpr (WEIGHTED) w_now = to_acc(psw[pos_now]);
+    // Straight-line code: every lane loads (a lane without an occurrence or beside the row's
+    // columns loads what occurrence 0 / column 0 loads and drops it), so that the UNROLL loads
+    // of a step are issued back to back.
     for (int j0 = 0; j0 < n; j0 += groups * UNROLL) {
       R raw[UNROLL];
       bool ok[UNROLL];
@@ -177,9 +191,12 @@ __device__ __forceinline__ void mixed_accumulate_narrow(
       for (int k = 0; k < UNROLL; ++k) {
         const int j = j0 + k * groups + r;
         ok[k] = active && j < n;
-        src[k] = ok[k] ? j : 0;
+        src[k] = j < n ? j : 0;
+      }
+#pragma unroll
+      for (int k = 0; k < UNROLL; ++k) {
         const int64_t bag = shfl_idx(my_bag, src[k]);
-        if (ok[k]) raw[k] = V::load_raw(gcol + bag * total_D + col);
+        raw[k] = V::load_raw(gcol + bag * total_D + safe_col);
       }
 #pragma unroll
       for (int k = 0; k < UNROLL; ++k) {
@@ -190,8 +207,9 @@ __device__ __forceinline__ void mixed_accumulate_narrow(
           pos = shfl_idx(my_pos, src[k]);
         }
         V x;
-        x.zero();
-        if (ok[k]) x.unpack(raw[k]);
+        x.unpack(raw[k]);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = ok[k] ? x.v[i] : A(0);
         if constexpr (WEIGHTED) {
           A dot = A(0);
 #pragma unroll
@@ -743,13 +761,13 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
              i32(l.num_unique), long_rows, huge_rows, a.lr, a.eps, a.sr);
   const int64_t want_long = ceil_div(a.n, kWavesPerBlock);
   const dim3 grid_long(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 8))));
-  TBE_LAUNCH("update_mixed_long", stream, (update_mixed_long_kernel<T, VEC, OPT, WEIGHTED, 4, 1>), grid_long,
+  TBE_LAUNCH("update_mixed_long", stream, (update_mixed_long_kernel<T, VEC, OPT, WEIGHTED, 8, 1>), grid_long,
              dim3(kBlockThreads), go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T,
              a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
              i32(l.num_unique), 2, long_rows, a.lr, a.eps, a.sr);
   const int64_t want_huge = a.n / (kChunkLen + 1) + 1;
   const dim3 grid_huge(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_huge, 256 * 2))));
-  TBE_LAUNCH("update_mixed_huge", stream, (update_mixed_long_kernel<T, VEC, OPT, WEIGHTED, 4, kHugeWaves>),
+  TBE_LAUNCH("update_mixed_huge", stream, (update_mixed_long_kernel<T, VEC, OPT, WEIGHTED, 8, kHugeWaves>),
              grid_huge, dim3(kHugeWaves * kWave), go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets,
              a.dim_offsets, a.T, a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows),
              i32(l.segment_starts), i32(l.num_unique), 1, huge_rows, a.lr, a.eps, a.sr);
