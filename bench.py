@@ -33,13 +33,13 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 # this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
 # reads for a plain 1 GiB device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Keyed by (kernel, config).
 MEASURED_TRAFFIC = {
-    ("update_short", 3): int((1274957.2 * 2.0 + 1278127.1) * 1024),
-    ("update_chunks", 3): int((391374.6 * 2.0 + 8339.5) * 1024),
-    ("forward", 3): int((836349.7 * 2.0 + 131072.0) * 1024),
-    ("forward", 2): int((1227827.0 * 2.0 + 131072.0) * 1024),
-    ("update_short", 4): int((188435.5 * 2.0 + 188389.5) * 1024),
-    ("update_chunks", 4): int((426814.3 * 2.0 + 100117.9) * 1024),
-    ("forward", 4): int((74906.6 * 2.0 + 32768.0) * 1024),
+    ("update_short", 3): int((1275006.0 * 2.0 + 1278126.8) * 1024),
+    ("update_chunks", 3): int((390355.5 * 2.0 + 8370.4) * 1024),
+    ("forward", 3): int((836325.8 * 2.0 + 131072.0) * 1024),
+    ("forward", 2): int((1227789.3 * 2.0 + 131072.0) * 1024),
+    ("update_short", 4): int((188331.6 * 2.0 + 188408.0) * 1024),
+    ("update_chunks", 4): int((424157.1 * 2.0 + 98875.2) * 1024),
+    ("forward", 4): int((84016.5 * 2.0 + 32768.0) * 1024),
 }
 
 

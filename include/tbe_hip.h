@@ -256,6 +256,8 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
  * stochastic_rounding / seed / offset as in tbe_backward_exact_adagrad_stochastic;
  * max_table_rows as in tbe_backward_sgd (0 = unknown).  The
  * workspace is a backward workspace sized with tbe_backward_workspace_layout(N, 4, dtype, T).
+ * grad_output may hold at most 2^31 - 1 elements (B * total_D), so that the element offset of a
+ * gradient row fits 32 bits.
  */
 TBE_API int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp16_vector_width,
                               const int64_t *table_offsets, const int32_t *dim_offsets,

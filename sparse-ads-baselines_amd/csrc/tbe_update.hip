@@ -338,15 +338,25 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     }
     V G;
     G.zero();
+    // The positions of a 64-position batch are requested two batches ahead, its gradient row ids
+    // and weights one batch ahead (lanes past the chunk's end ask for its first position: any
+    // valid index will do), so a batch waits for gradient rows only.
+    auto position_at = [&](int64_t i) { return positions_sorted[i < rec.end ? i : rec.begin]; };
+    int pos_now = position_at(static_cast<int64_t>(rec.begin) + lane);
+    int pos_next = position_at(static_cast<int64_t>(rec.begin) + kWave + lane);
+    int grow_now = grad_rows[pos_now];
+    A w_now = A(0);
+    if constexpr (WEIGHTED) w_now = to_acc(psw[pos_now]);
     for (int base = rec.begin; base < rec.end; base += kWave) {
       const int n = min(kWave, rec.end - base);
-      int my_pos = 0, my_grow = 0;
-      A my_w = A(0);
-      if (lane < n) {
-        my_pos = positions_sorted[base + lane];
-        my_grow = grad_rows[my_pos];
-        if constexpr (WEIGHTED) my_w = to_acc(psw[my_pos]);
-      }
+      const int my_pos = pos_now, my_grow = grow_now;
+      const A my_w = w_now;
+      pos_now = pos_next;
+      pos_next = position_at(static_cast<int64_t>(base) + 2 * kWave + lane);
+      grow_now = grad_rows[pos_now];
+      if constexpr (WEIGHTED) w_now = to_acc(psw[pos_now]);
+      // Straight-line code: every lane loads (a lane without an occurrence loads what occurrence
+      // 0 loads and drops it), so that the UNROLL loads of a step are issued back to back.
       for (int j0 = 0; j0 < n; j0 += groups * UNROLL) {
         R raw[UNROLL];
         bool ok[UNROLL];
@@ -355,9 +365,12 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
         for (int k = 0; k < UNROLL; ++k) {
           const int j = j0 + k * groups + r;
           ok[k] = active && j < n;
-          src[k] = ok[k] ? j : 0;
+          src[k] = j < n ? j : 0;
+        }
+#pragma unroll
+        for (int k = 0; k < UNROLL; ++k) {
           const int64_t grow = shfl_idx(my_grow, src[k]);
-          if (ok[k]) raw[k] = V::load_raw(grad_output + grow * D + col);
+          raw[k] = V::load_raw(grad_output + grow * D + col);
         }
 #pragma unroll
         for (int k = 0; k < UNROLL; ++k) {
@@ -367,21 +380,21 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
             pw = shfl_idx(my_w, src[k]);
             pos = shfl_idx(my_pos, src[k]);
           }
-          if (ok[k]) {
-            V x;
-            x.unpack(raw[k]);
-            if constexpr (WEIGHTED) {
-              A dot = A(0);
+          V x;
+          x.unpack(raw[k]);
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
-              dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
-              if (c == 0) grad_psw[pos] = from_acc<T, A>(dot);
+          for (int i = 0; i < VEC; ++i) x.v[i] = ok[k] ? x.v[i] : A(0);
+          if constexpr (WEIGHTED) {
+            A dot = A(0);
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * pw;
-            } else {
+            for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
+            dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
+            if (ok[k] && c == 0) grad_psw[pos] = from_acc<T, A>(dot);
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i];
-            }
+            for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * pw;
+          } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i];
           }
         }
       }
@@ -579,7 +592,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_wide_kernel(
 }
 
 constexpr int kShortUnroll = 4;
-constexpr int kLongUnroll = 4;
+constexpr int kLongUnroll = 8;
 
 template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED>
 void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream) {
