@@ -107,7 +107,8 @@ typedef struct tbe_workspace_layout {
   uint64_t segment_scratch;
   uint64_t segment_ids;      /* int32 [N]: index of the unique row of each sorted position */
   uint64_t long_segments;    /* 16-byte records [max_long_segments]: rows reduced in several chunks */
-  uint64_t chunk_segments;   /* 32-byte records [max_chunks]: queue of occurrence chunks        */
+  uint64_t chunk_segments;   /* 32-byte records [8][max_chunks / 8]: queues of occurrence chunks,
+                              * one per eighth of the sorted positions                          */
   uint64_t partial_sums;     /* accumulator-typed [max_partial_rows][D]                         */
   int64_t max_long_segments;
   int64_t max_chunks;

@@ -27,7 +27,7 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspac
   // a segment enters the chunk queue when it has more than kShortSegment occurrences and owns
   // partial rows when it has more than kChunkLen
   l->max_long_segments = static_cast<int64_t>(nn / (kChunkLen + 1) + 1);
-  l->max_chunks = static_cast<int64_t>(nn / kChunkLen + nn / (kShortSegment + 1) + 2);
+  l->max_chunks = static_cast<int64_t>(kNumXcd * chunk_queue_capacity(static_cast<int64_t>(nn)));
   l->max_partial_rows = static_cast<int64_t>(nn / kChunkLen + nn / (kChunkLen + 1) + 2);
   uint64_t off = 0;
   l->keys = off; off += ints;

@@ -472,8 +472,8 @@ __global__ __launch_bounds__(kBlockThreads) void segment_scan_kernel(
     num_unique[0] = static_cast<int32_t>(carry);
     segment_starts[carry] = static_cast<int32_t>(n);
   }
-  // the update stage keeps three queue counters next to U; starting them at zero here saves a launch
-  if (clear_queue_counters && tid >= 1 && tid <= 3) num_unique[tid] = 0;
+  // the update stage keeps its queue counters next to U; starting them at zero here saves a launch
+  if (clear_queue_counters && tid >= 1 && tid < kNumCounters) num_unique[tid] = 0;
 }
 
 // The heads of a tile are compacted in LDS and leave as one contiguous run; the segment of

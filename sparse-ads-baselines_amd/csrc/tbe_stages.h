@@ -37,6 +37,19 @@ int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts
 // whole wavefronts in chunks of at most kChunkLen occurrences.
 constexpr int kShortSegment = 16;
 constexpr int kChunkLen = 256;
+// Integers kept next to the number of unique rows (all zeroed when the segments are found):
+// [1] long rows, [3] partial rows, [8..15] chunk records queued by each XCD.
+constexpr int kNumCounters = 16;
+constexpr int kChunkQueueCount = 8;
+// The short-row kernel's workgroups of XCD x own the segments that start in the x-th eighth of
+// the sorted positions (rounded up to whole workgroups: at most 1024 positions more) and queue
+// their chunk records in a region of their own.  Segments are consecutive, so only the last
+// segment that starts in an eighth can reach beyond it: the records of one XCD are bounded by
+// those of its eighth plus those of one segment of any length.
+inline int64_t chunk_queue_capacity(int64_t n) {
+  const int64_t eighth = (n + 7) / 8 + 1024;
+  return eighth / (kShortSegment + 1) + eighth / kChunkLen + n / kChunkLen + 8;
+}
 
 enum { kOptSgd = 0, kOptAdagrad = 1 };
 
@@ -53,7 +66,7 @@ struct UpdateArgs {
   int32_t *counters;            // [0] = U (input), [1] = #long records, [2] = #chunk records, [3] = #partial rows
   const int32_t *segment_ids;   // [N] segment of every sorted position
   void *long_segments;          // 16-byte records [max_long]: segments cut into several chunks
-  void *chunk_segments;         // 32-byte records [max_chunks]: the chunk queue
+  void *chunk_segments;         // 32-byte records [8][max_chunks / 8]: one chunk queue per XCD
   void *partial_sums;           // acc [max_partial][D]
   const int32_t *unique_slots;  // cache-fronted tables: slot of each unique row (-1 = not resident)
   void *cache_rows;             // cache-fronted tables: [slots][D] rows in HBM

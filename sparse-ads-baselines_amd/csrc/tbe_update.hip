@@ -117,9 +117,9 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ segment_ids,
     int32_t *__restrict__ counters, LongRecord *__restrict__ long_records,
-    ChunkRecord *__restrict__ chunk_records, int64_t n, int64_t num_tiles, int64_t tiles_per_xcd,
-    int D, int chunks_rt, float lr, float eps, const int32_t *__restrict__ unique_slots,
-    T *__restrict__ cache_rows, StochasticRounding sr) {
+    ChunkRecord *__restrict__ chunk_records, int64_t max_chunks, int64_t n, int64_t num_tiles,
+    int64_t tiles_per_xcd, int D, int chunks_rt, float lr, float eps,
+    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -135,6 +135,12 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
   const int wave = threadIdx.x >> 6;
   const int64_t tile = xcd_contiguous(blockIdx.x, tiles_per_xcd) * kWavesPerBlock + wave;
   if (tile >= num_tiles) return;
+  // The workgroups of an XCD walk one eighth of the sorted positions in order, so the chunk
+  // records they queue are in (table, row) order: each XCD keeps its own queue, which
+  // update_chunks_kernel drains on the same XCD in that order (the gradient rows of a table then
+  // stay in that XCD's L2 while its hot rows are reduced).
+  const int xcd = blockIdx.x % kNumXcd;
+  ChunkRecord *chunk_queue = chunk_records + xcd * (max_chunks / kNumXcd);
   const int chunks = CHUNKS > 0 ? CHUNKS : chunks_rt;
   const int groups = kWave / chunks;
   const int r = lane / chunks;
@@ -217,7 +223,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
       const int nch = (len + kChunkLen - 1) / kChunkLen;
       int first_chunk = 0, first_partial = -1;
       if (c == 0) {
-        first_chunk = atomicAdd(&counters[2], nch);
+        first_chunk = atomicAdd(&counters[kChunkQueueCount + xcd], nch);
         if (nch > 1) {
           first_partial = atomicAdd(&counters[3], nch);
           long_records[atomicAdd(&counters[1], 1)] = LongRecord{u, key, first_partial, nch};
@@ -233,7 +239,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
         rec.u = u;
         rec.partial = nch > 1 ? first_partial + k : -1;
         rec.pad[0] = rec.pad[1] = rec.pad[2] = 0;
-        chunk_records[first_chunk + k] = rec;
+        chunk_queue[first_chunk + k] = rec;
       }
       continue;
     }
@@ -297,8 +303,9 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
 }
 
 // ------------------------------------------------ medium / long segments: chunks
-// One wavefront per chunk record (grid-stride over the queue).  Lane group r adds
-// occurrences r, r + groups, ... of the chunk; the groups are combined in a fixed tree.
+// One wavefront per chunk record.  The wavefronts of an XCD take the records of that XCD's
+// queue, consecutive records at the same time.  Lane group r adds occurrences r, r + groups,
+// ... of the chunk; the groups are combined in a fixed tree.
 // A chunk that is a whole segment is applied to its row at once; a chunk of a longer
 // segment stores its sum as a partial row for update_long_finish_kernel.
 template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL>
@@ -307,7 +314,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
     T *__restrict__ grad_psw, const int32_t *__restrict__ positions_sorted,
     const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ counters,
-    const ChunkRecord *__restrict__ chunk_records,
+    const ChunkRecord *__restrict__ chunk_records, int64_t max_chunks,
     typename AccOf<T>::type *__restrict__ partial_sums, int D, int chunks_rt, float lr, float eps,
     const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
@@ -321,13 +328,15 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
   const int c = lane - r * chunks;
   const int group_base = r * chunks;
   const bool active = r < groups;
-  const int num_chunks = counters[2];
   const int64_t col = static_cast<int64_t>(c) * VEC;
-  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  const int xcd = blockIdx.x % kNumXcd;
+  const ChunkRecord *chunk_queue = chunk_records + xcd * (max_chunks / kNumXcd);
+  const int num_chunks = counters[kChunkQueueCount + xcd];
+  const int64_t wave_in_xcd = static_cast<int64_t>(blockIdx.x / kNumXcd) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = static_cast<int64_t>(gridDim.x / kNumXcd) * kWavesPerBlock;
 
-  for (int64_t q = wave_id; q < num_chunks; q += stride) {
-    const ChunkRecord rec = chunk_records[q];
+  for (int64_t q = wave_in_xcd; q < num_chunks; q += stride) {
+    const ChunkRecord rec = chunk_queue[q];
     T *wrow = resolve_row(weights, cache_rows, unique_slots, rec.u, static_cast<int64_t>(rec.key), D) + col;
     V w_old;
     w_old.zero();
@@ -615,16 +624,18 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   TBE_LAUNCH("update_short", stream,
              (update_short_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kShortUnroll>), grid_short, block,
              go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
-             a.segment_starts, a.segment_ids, a.counters, long_records, chunk_records,
+             a.segment_starts, a.segment_ids, a.counters, long_records, chunk_records, a.max_chunks,
              a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,
              a.unique_slots, cr, a.stochastic_rounding);
 
   const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
-  const dim3 grid_chunks(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_chunks, 256 * 8))));
+  // a multiple of the XCD count, so that every XCD gets as many workgroups
+  const dim3 grid_chunks(static_cast<unsigned>(
+      kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), 1024))));
   TBE_LAUNCH("update_chunks", stream,
              (update_chunks_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kLongUnroll>), grid_chunks, block,
              go, w, st, psw, gpsw, a.positions_sorted, a.grad_rows, a.counters, chunk_records,
-             partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr,
+             a.max_chunks, partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr,
              a.stochastic_rounding);
 
   const int64_t want_long = ceil_div(a.max_long, kWavesPerBlock);
@@ -676,7 +687,7 @@ void launch_variant(const UpdateArgs &a, const RowGeometry &g, hipStream_t strea
 int segment_update(const UpdateArgs &a, hipStream_t stream) {
   if (a.num_indices == 0) return TBE_OK;
   const RowGeometry g = row_geometry(a.dtype, a.D);
-  // counters[1..3] were zeroed when the plan's segments were found
+  // the queue counters were zeroed when the plan's segments were found
   switch (a.dtype) {
     case TBE_DTYPE_F32: launch_variant<float, 4>(a, g, stream); break;
     case TBE_DTYPE_F16:
