@@ -304,7 +304,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
 
 // ------------------------------------------------ medium / long segments: chunks
 // One wavefront per chunk record.  The wavefronts of an XCD take the records of that XCD's
-// queue, consecutive records at the same time.  Lane group r adds occurrences r, r + groups,
+// queue, consecutive records at the same time (see below for queues of unequal length).  Lane group r adds occurrences r, r + groups,
 // ... of the chunk; the groups are combined in a fixed tree.
 // A chunk that is a whole segment is applied to its row at once; a chunk of a longer
 // segment stores its sum as a partial row for update_long_finish_kernel.
@@ -329,14 +329,47 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
   const int group_base = r * chunks;
   const bool active = r < groups;
   const int64_t col = static_cast<int64_t>(c) * VEC;
+  // An XCD drains its own queue up to one and a half times the average queue length; what the
+  // longer queues hold beyond that is dealt to the wavefronts of all XCDs, so that a batch whose
+  // hot rows sit in one table still uses the whole machine.  All of it is index arithmetic on
+  // the eight queue lengths: no wavefront waits for another.
   const int xcd = blockIdx.x % kNumXcd;
-  const ChunkRecord *chunk_queue = chunk_records + xcd * (max_chunks / kNumXcd);
-  const int num_chunks = counters[kChunkQueueCount + xcd];
-  const int64_t wave_in_xcd = static_cast<int64_t>(blockIdx.x / kNumXcd) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t queue_capacity = max_chunks / kNumXcd;
+  int queue_len[kNumXcd];
+  int64_t total = 0;
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) {
+    queue_len[x] = counters[kChunkQueueCount + x];
+    total += queue_len[x];
+  }
+  const int fair = static_cast<int>(total / kNumXcd + total / 16 + 1);
+  int64_t shared_total = 0;
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) shared_total += max(0, queue_len[x] - fair);
+  const int own = min(queue_len[xcd], fair);
+  int64_t q = static_cast<int64_t>(blockIdx.x / kNumXcd) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x / kNumXcd) * kWavesPerBlock;
+  int64_t g = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t shared_stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
 
-  for (int64_t q = wave_in_xcd; q < num_chunks; q += stride) {
-    const ChunkRecord rec = chunk_queue[q];
+  while (true) {
+    const ChunkRecord *next;
+    if (q < own) {
+      next = chunk_records + xcd * queue_capacity + q;
+      q += stride;
+    } else if (g < shared_total) {
+      int64_t before = 0;
+      int x = 0;
+      while (g >= before + max(0, queue_len[x] - fair)) {
+        before += max(0, queue_len[x] - fair);
+        ++x;
+      }
+      next = chunk_records + x * queue_capacity + fair + (g - before);
+      g += shared_stride;
+    } else {
+      break;
+    }
+    const ChunkRecord rec = *next;
     T *wrow = resolve_row(weights, cache_rows, unique_slots, rec.u, static_cast<int64_t>(rec.key), D) + col;
     V w_old;
     w_old.zero();
@@ -477,10 +510,23 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     V G;
     G.zero();
     if (active) {
-      for (int k = r; k < rec.num_chunks; k += groups) {
-        const A *src = partial_sums + static_cast<int64_t>(rec.first_partial + k) * D + col;
+      // eight partial rows are requested before the first is added (same order of additions)
+      constexpr int kAhead = 8;
+      for (int k0 = r; k0 < rec.num_chunks; k0 += groups * kAhead) {
+        A part[kAhead][VEC];
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) G.v[i] += src[i];
+        for (int a = 0; a < kAhead; ++a) {
+          const int k = min(k0 + a * groups, rec.num_chunks - 1);  // clamped: no branch per load
+          const A *src = partial_sums + static_cast<int64_t>(rec.first_partial + k) * D + col;
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) part[a][i] = src[i];
+        }
+#pragma unroll
+        for (int a = 0; a < kAhead; ++a) {
+          const bool real = k0 + a * groups < rec.num_chunks;
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) G.v[i] += real ? part[a][i] : A(0);
+        }
       }
     }
     if constexpr (CHUNKS > 0) {
