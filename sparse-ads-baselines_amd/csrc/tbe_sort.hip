@@ -199,12 +199,20 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
 #pragma unroll
   for (int d = tid; d < kBinsT; d += kBlockThreads) s_hist[d] = 0;
   __syncthreads();
+  // every thread loads all its keys first (an index past the tile's end is clamped, the key
+  // dropped): straight-line loads are issued back to back, predicated ones one at a time
+  if (tile.count > 0) {
+    uint32_t key[kItems];
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
-    const int i = k * kBlockThreads + tid;
-    if (i < tile.count) atomicAdd(&s_hist[(keys[tile.begin + i] >> shift) & mask], 1u);
+    for (int k = 0; k < kItems; ++k)
+      key[k] = keys[tile.begin + min(k * kBlockThreads + tid, tile.count - 1)];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+      if (k * kBlockThreads + tid < tile.count) atomicAdd(&s_hist[(key[k] >> shift) & mask], 1u);
+    }
   }
   __syncthreads();
+  // (one 4-byte store per digit, a tile apart: these scattered stores are most of this kernel's time)
 #pragma unroll
   for (int d = tid; d < kBinsT; d += kBlockThreads)
     counts[tile.count_base + static_cast<int64_t>(d) * tile.table_tiles] = s_hist[d];
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
       kShareCounters ? reinterpret_cast<uint32_t(*)[kBinsT]>(s_keys) : reinterpret_cast<uint32_t(*)[kBinsT]>(s_own_count);
 
   const TileInfo tile = locate_tile<BITS>(table_starts, tile_prefix, num_tables, max_tiles);
-  if (tile.table_tiles == 0) return;
+  if (tile.table_tiles == 0 || tile.count == 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
@@ -318,13 +326,23 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
 
   uint32_t key[kItems], val[kItems];
   const int wave_first = wave * kWaveTile;
+  // straight-line loads (an index past the tile's end is clamped, what it loads replaced)
+#pragma unroll
+  for (int k = 0; k < kItems; ++k)
+    key[k] = keys_in[tile.begin + min(wave_first + k * kWave + lane, tile.count - 1)];
+  if (values_in) {
+#pragma unroll
+    for (int k = 0; k < kItems; ++k)
+      val[k] = values_in[tile.begin + min(wave_first + k * kWave + lane, tile.count - 1)];
+  } else {
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) val[k] = static_cast<uint32_t>(tile.begin + wave_first + k * kWave + lane);
+  }
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
-    const int local = wave_first + k * kWave + lane;
-    const bool valid = local < tile.count;
-    const int64_t i = tile.begin + local;
-    key[k] = valid ? keys_in[i] : 0xffffffffu;
-    val[k] = valid ? (values_in ? values_in[i] : static_cast<uint32_t>(i)) : 0u;
+    const bool valid = wave_first + k * kWave + lane < tile.count;
+    key[k] = valid ? key[k] : 0xffffffffu;
+    val[k] = valid ? val[k] : 0u;
   }
   __syncthreads();
 
