@@ -33,13 +33,13 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 # this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
 # reads for a plain 1 GiB device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Keyed by (kernel, config).
 MEASURED_TRAFFIC = {
-    ("update_short", 3): int((1275006.0 * 2.0 + 1278126.8) * 1024),
-    ("update_chunks", 3): int((390355.5 * 2.0 + 8370.4) * 1024),
-    ("forward", 3): int((836325.8 * 2.0 + 131072.0) * 1024),
-    ("forward", 2): int((1227789.3 * 2.0 + 131072.0) * 1024),
-    ("update_short", 4): int((188331.6 * 2.0 + 188408.0) * 1024),
-    ("update_chunks", 4): int((424157.1 * 2.0 + 98875.2) * 1024),
-    ("forward", 4): int((84016.5 * 2.0 + 32768.0) * 1024),
+    ("update_short", 3): int((1275360.5 * 2.0 + 1278141.7) * 1024),
+    ("update_chunks", 3): int((242600.2 * 2.0 + 8309.4) * 1024),
+    ("forward", 3): int((836333.5 * 2.0 + 131072.0) * 1024),
+    ("forward", 2): int((1227809.0 * 2.0 + 131072.0) * 1024),
+    ("update_short", 4): int((188417.4 * 2.0 + 188415.7) * 1024),
+    ("update_chunks", 4): int((70822.0 * 2.0 + 52396.2) * 1024),
+    ("forward", 4): int((84001.3 * 2.0 + 32768.0) * 1024),
 }
 
 
