@@ -42,12 +42,12 @@ constexpr int kChunkLen = 256;
 constexpr int kNumCounters = 16;
 constexpr int kChunkQueueCount = 8;
 // The short-row kernel's workgroups of XCD x own the segments that start in the x-th eighth of
-// the sorted positions (rounded up to whole workgroups: at most 1024 positions more) and queue
+// the sorted positions (rounded up to whole workgroups: fewer than 1200 positions more) and queue
 // their chunk records in a region of their own.  Segments are consecutive, so only the last
 // segment that starts in an eighth can reach beyond it: the records of one XCD are bounded by
 // those of its eighth plus those of one segment of any length.
 inline int64_t chunk_queue_capacity(int64_t n) {
-  const int64_t eighth = (n + 7) / 8 + 1024;
+  const int64_t eighth = (n + 7) / 8 + 2048;
   return eighth / (kShortSegment + 1) + eighth / kChunkLen + n / kChunkLen + 8;
 }
 

@@ -222,6 +222,30 @@ def test_backward_matches_embeddingbag_fixture(name):
         assert_close(got["grad_psw"], g["expected_grad_psw"], tol)
 
 
+@pytest.mark.parametrize("dtype,D,occurrences", [(np.float32, 128, 17), (np.float16, 64, 17), (np.float32, 16, 257)])
+def test_queues_hold_the_most_chunk_records_a_batch_can_produce(oracle, dtype, D, occurrences):
+    """Every row occurs 17 times (the most segments that leave the short-row kernel: one chunk
+    record per 17 lookups) or 257 times (two chunks and a partial-row record each): the eight
+    queues together receive exactly the number of records the arithmetic predicts, and nothing
+    around them is overwritten (the update still matches the oracle)."""
+    rs = np.random.RandomState(11)
+    T, B, L = 3, 1700, 12
+    n = T * B * L
+    per_table = B * L
+    rows = per_table // occurrences + 1
+    p = make_problem(12, T, rows, D, B, L, dtype, ragged=False, weighted=False)
+    for t in range(T):
+        ids = np.repeat(np.arange(rows, dtype=np.int32), occurrences)[:per_table]
+        p["indices"][t * per_table:(t + 1) * per_table] = rs.permutation(ids)
+    w, st, ref, got = _run_both(oracle, p, "sgd", 0.01, 0.1)
+    lengths = np.diff(ref["segment_starts"])
+    assert (lengths == occurrences).sum() >= T * (rows - 1)
+    counters = got["views"]["counters"]
+    assert counters[8:16].sum() == np.ceil(lengths[lengths > 16] / 256).sum()
+    assert counters[1] == (lengths > 256).sum()
+    _check(p, w, st, ref, got, "sgd")
+
+
 @pytest.mark.parametrize("dtype,D", [(np.float32, 128), (np.float16, 64), (np.float32, 12), (np.float64, 8)])
 @pytest.mark.parametrize("mode", ["sgd", "adagrad_weighted"])
 def test_hot_rows_take_the_chunked_path(oracle, dtype, D, mode):
