@@ -647,7 +647,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_wide_kernel(
 }
 
 constexpr int kShortUnroll = 4;
-constexpr int kLongUnroll = 8;
+constexpr int kLongUnroll = 8;  // 4 for weighted 8-element fp16 vectors: registers, hence occupancy
 
 template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED>
 void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream) {
@@ -679,7 +679,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   const dim3 grid_chunks(static_cast<unsigned>(
       kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), 1024))));
   TBE_LAUNCH("update_chunks", stream,
-             (update_chunks_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kLongUnroll>), grid_chunks, block,
+             (update_chunks_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, (WEIGHTED && VEC == 8) ? 4 : kLongUnroll>), grid_chunks, block,
              go, w, st, psw, gpsw, a.positions_sorted, a.grad_rows, a.counters, chunk_records,
              a.max_chunks, partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr,
              a.stochastic_rounding);
