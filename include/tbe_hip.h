@@ -169,6 +169,8 @@ TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, i
  * (kernel :1499-1587) on that workspace once `grad_output` exists; `stream` must be ordered
  * after the plan (e.g. by an event).  Together they equal tbe_backward_sgd /
  * tbe_backward_exact_adagrad(_stochastic); optimizer is TBE_OPT_SGD or TBE_OPT_ROWWISE_ADAGRAD.
+ * A plan serves ONE tbe_backward_planned call (the update fills the queue counters that the plan
+ * left at zero); plan again for the next batch or the next update.
  */
 TBE_API int tbe_plan_batch(const int32_t *table_offsets, int32_t T,
                            const int32_t *indices, int64_t num_indices,
