@@ -495,19 +495,41 @@ __global__ __launch_bounds__(kBlockThreads) void segment_scan_kernel(
 }
 
 // The heads of a tile are compacted in LDS and leave as one contiguous run; the segment of
-// every position leaves in 16-byte stores.
+// every position leaves in 16-byte stores.  SUM_TILES: `tile_base` holds the head count of
+// every tile, not yet scanned: the workgroup adds up the counts of the tiles before its own (a
+// few thousand tiles at most: see find_segments), and the last workgroup does what
+// segment_scan_kernel does at its end -- one launch less on the path of every backward.
+template <bool SUM_TILES>
 __global__ __launch_bounds__(kBlockThreads) void segment_write_kernel(
     const uint32_t *__restrict__ keys, int64_t n, const uint32_t *__restrict__ tile_base,
-    int32_t *__restrict__ segment_starts, int32_t *__restrict__ segment_ids) {
+    int32_t *__restrict__ segment_starts, int32_t *__restrict__ segment_ids,
+    int32_t *__restrict__ num_unique, int clear_queue_counters) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
+  __shared__ uint32_t s_wave_tiles[kWavesPerBlock];
   __shared__ int32_t s_heads[kSegTile];
   const int64_t tile_first = static_cast<int64_t>(blockIdx.x) * kSegTile;
   const int64_t first = tile_first + threadIdx.x * kSegItems;
+  uint32_t tiles_before = 0;
+  if constexpr (SUM_TILES) {
+    for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kBlockThreads) tiles_before += tile_base[i];
+  }
   const uint32_t flags = segment_head_flags(keys, n, first);
   const uint32_t mine = __popc(flags);
   uint32_t total;
   const uint32_t incl = block_inclusive_scan(mine, s_wave, total);
-  const uint32_t base = tile_base[blockIdx.x];
+  uint32_t base;
+  if constexpr (SUM_TILES) {
+    (void)block_inclusive_scan(tiles_before, s_wave_tiles, base);
+    if (blockIdx.x == gridDim.x - 1) {
+      if (threadIdx.x == 0) {
+        num_unique[0] = static_cast<int32_t>(base + total);
+        segment_starts[base + total] = static_cast<int32_t>(n);
+      }
+      if (clear_queue_counters && threadIdx.x >= 1 && threadIdx.x < kNumCounters) num_unique[threadIdx.x] = 0;
+    }
+  } else {
+    base = tile_base[blockIdx.x];
+  }
   uint32_t local = incl - mine;
   int32_t ids[kSegItems];
 #pragma unroll
@@ -652,11 +674,19 @@ int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts
   if (tiles > 0)
     TBE_LAUNCH("segment_count", stream, segment_count_kernel, dim3(tiles), block, keys, n,
                tile_heads);
+  // Up to a few thousand tiles, every workgroup of the last kernel sums the counts before its
+  // own (a few KB from L2 each); beyond that a kernel of one workgroup scans them first.
+  constexpr int kMaxSummedTiles = 4096;
+  if (tiles > 0 && tiles <= kMaxSummedTiles) {
+    TBE_LAUNCH("segment_write", stream, segment_write_kernel<true>, dim3(tiles), block, keys, n,
+               tile_heads, segment_starts, segment_ids, num_unique, clear_queue_counters ? 1 : 0);
+    return check_launch("tbe_find_segments");
+  }
   TBE_LAUNCH("segment_scan", stream, segment_scan_kernel, dim3(1), block, tile_heads, tiles, n,
              segment_starts, num_unique, clear_queue_counters ? 1 : 0);
   if (tiles > 0)
-    TBE_LAUNCH("segment_write", stream, segment_write_kernel, dim3(tiles), block, keys, n,
-               tile_heads, segment_starts, segment_ids);
+    TBE_LAUNCH("segment_write", stream, segment_write_kernel<false>, dim3(tiles), block, keys, n,
+               tile_heads, segment_starts, segment_ids, num_unique, 0);
   return check_launch("tbe_find_segments");
 }
 

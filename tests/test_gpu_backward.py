@@ -77,7 +77,8 @@ def test_sort_pairs_carries_arbitrary_values(oracle):
     np.testing.assert_array_equal(v_out.cpu().numpy(), want_v)
 
 
-@pytest.mark.parametrize("n,hi", [(0, 5), (1, 5), (2047, 3), (2048, 100000), (2049, 1), (300000, 120000)])
+@pytest.mark.parametrize("n,hi", [(0, 5), (1, 5), (2047, 3), (2048, 100000), (2049, 1), (300000, 120000),
+                                  (8388608, 2000000), (8400000, 3000000)])  # 4096 tiles, and one tile count beyond
 def test_find_segments_bit_exact(oracle, n, hi):
     keys = np.sort(np.random.RandomState(n % 89).randint(0, hi, size=n)).astype(np.int32)
     lib = tbe_native.load()
