@@ -96,31 +96,6 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
   }
 }
 
-// keys[p] = table_dim_offsets[t] + indices[p] (skipped when `keys` is null); grad_rows[p] = b * T + t.
-__global__ __launch_bounds__(kBlockThreads) void linearize_mixed_kernel(
-    const int32_t *__restrict__ table_dim_offsets, const int32_t *__restrict__ indices,
-    const int32_t *__restrict__ offsets, int B, int num_tables, int num_bags,
-    int32_t *__restrict__ keys, int32_t *__restrict__ grad_rows) {
-  constexpr int kLanes = 16;
-  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int64_t bag64 = gid / kLanes;
-  if (bag64 >= num_bags) return;
-  const int bag = static_cast<int>(bag64);
-  const int t = bag / B;
-  const int b = bag - t * B;
-  const int32_t grow = b * num_tables + t;
-  const int end = offsets[bag + 1];
-  if (keys) {
-    const int32_t row0 = table_dim_offsets[t];
-    for (int p = offsets[bag] + static_cast<int>(gid % kLanes); p < end; p += kLanes) {
-      keys[p] = row0 + indices[p];
-      grad_rows[p] = grow;
-    }
-  } else {
-    for (int p = offsets[bag] + static_cast<int>(gid % kLanes); p < end; p += kLanes) grad_rows[p] = grow;
-  }
-}
-
 // Everything a wavefront needs to know about one unique row.
 struct MixedRow {
   int seg_begin, seg_end;  // sorted positions of its occurrences
@@ -890,15 +865,14 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   hipStream_t s = static_cast<hipStream_t>(stream);
   char *ws = static_cast<char *>(workspace);
   auto i32 = [&](uint64_t off) { return reinterpret_cast<int32_t *>(ws + off); };
-  const int64_t num_bags = static_cast<int64_t>(T) * B;
-  TBE_LAUNCH("linearize_mixed", s, linearize_mixed_kernel,
-             dim3(static_cast<unsigned>(ceil_div(num_bags * 16, kBlockThreads))), dim3(kBlockThreads),
-             table_dim_offsets, indices, offsets, B, T, static_cast<int>(num_bags), nullptr, i32(l.grad_rows));
+  // gradient row b*T + t of every position (the keys themselves are not needed: see below)
+  int rc = linearize(table_dim_offsets, T, indices, offsets, B, nullptr, i32(l.grad_rows), s);
+  if (rc) return rc;
   // every table's indices are sorted on their own; the last pass adds the table's first row id
   const int64_t largest = (max_table_rows > 0 && max_table_rows < total_rows) ? max_table_rows : total_rows;
   const SortTables tables{offsets, B, T, table_dim_offsets};
-  int rc = sort_pairs(indices, nullptr, i32(l.keys_sorted), i32(l.positions_sorted), num_indices,
-                      key_bits_for(largest), ws + l.sort_scratch, s, &tables);
+  rc = sort_pairs(indices, nullptr, i32(l.keys_sorted), i32(l.positions_sorted), num_indices,
+                  key_bits_for(largest), ws + l.sort_scratch, s, &tables);
   if (rc) return rc;
   rc = find_segments(i32(l.keys_sorted), num_indices, i32(l.segment_starts), i32(l.num_unique), nullptr,
                      ws + l.segment_scratch, s, /*clear_queue_counters=*/true);
