@@ -411,6 +411,62 @@ def test_full_size_backward_properties():
     assert_close(W[:E].cpu().numpy(), w_ref, 1e-5)
 
 
+def test_full_size_weighted_adagrad_fp16_properties():
+    """BASELINE config 4 shape (T=32, E=1e6, D=64 fp16 weights, fp32 state from 0, B=8192, bag
+    lengths uniform in [0, 40] with empty bags, per-sample weights ~U(0,1), Zipf(1.2) indices,
+    exact row-wise Adagrad lr=0.01 eps=1e-8): sort / segment properties, untouched rows and state
+    bit-identical, and the first table (weights, state, per-sample-weight gradients) against the
+    oracle."""
+    from oracle import tbe_oracle
+    T, E, D, B = 32, 1000000, 64, 8192
+    rs = np.random.RandomState(4)
+    lengths = rs.randint(0, 41, size=T * B)
+    off_np = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    n = int(off_np[-1])
+    idx_np = (rs.zipf(1.2, size=n) % E).astype(np.int32)
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    W = torch.empty(T * E, D, device=DEV).uniform_(-0.01, 0.01, generator=gen).half()
+    W0 = W.clone()
+    state = torch.zeros(T * E, device=DEV)
+    go = torch.randn(B, T, D, device=DEV, generator=gen).half()
+    psw = torch.rand(n, device=DEV, generator=gen).half()
+    idx, offsets = torch.from_numpy(idx_np).to(DEV), torch.from_numpy(off_np).to(DEV)
+    table_offsets = torch.arange(T, dtype=torch.int32, device=DEV) * E
+    grad_psw = ext.backward_exact_adagrad(go, W, table_offsets, idx, offsets, psw, state, 0.01, 1e-8, False, 1)
+    _sync()
+    lay = tbe_native.backward_workspace_layout(n, D, tbe_native.DTYPE_F16, T)
+    ws = ext.backward_workspace(torch.device(DEV))
+    view = lambda off, cnt: ws[off:off + 4 * cnt].view(torch.int32)
+    ks, ps = view(lay.keys_sorted, n), view(lay.positions_sorted, n)
+    U = int(view(lay.num_unique, 1)[0])
+    ss = view(lay.segment_starts, U + 1).long()
+    table_of_position = torch.repeat_interleave(torch.arange(T, device=DEV),
+                                                torch.from_numpy(lengths.reshape(T, B).sum(1)).to(DEV))
+    want_keys = idx.long() + table_of_position * E
+    assert bool((ks[1:] >= ks[:-1]).all())
+    assert torch.equal(torch.sort(ps.long())[0], torch.arange(n, device=DEV))
+    assert torch.equal(want_keys[ps.long()], ks.long())
+    same = ks[1:] == ks[:-1]
+    assert bool((ps[1:][same] > ps[:-1][same]).all())
+    assert U == int(torch.unique(want_keys).numel())
+    assert int(ss[0]) == 0 and int(ss[-1]) == n and bool((ss[1:] > ss[:-1]).all())
+    seg_len = ss[1:] - ss[:-1]
+    assert int(seg_len.max()) > 20000            # the hot rows of Zipf(1.2): thousands of chunks
+    touched = torch.zeros(T * E, dtype=torch.bool, device=DEV)
+    touched[want_keys] = True
+    assert torch.equal(W[~touched], W0[~touched]) and not bool(state[~touched].any())
+    assert bool((state[touched] >= 0).all()) and bool(torch.isfinite(W.float()).all())
+    # first table against the oracle
+    n0 = int(off_np[B])
+    w_ref = W0[:E].cpu().numpy().copy()
+    st_ref = np.zeros(E, np.float32)
+    ref = tbe_oracle.backward("adagrad", go[:, :1, :].contiguous().cpu().numpy(), w_ref, np.zeros(1, np.int32),
+                              idx_np[:n0], off_np[:B + 1], 0.01, 1e-8, st_ref, psw[:n0].cpu().numpy())
+    assert_close(W[:E].cpu().numpy(), w_ref, 1e-2)
+    assert_close(state[:E].cpu().numpy(), st_ref, 1e-3)
+    assert_close(grad_psw[:n0].cpu().numpy(), ref["grad_psw"], 1e-2)
+
+
 @pytest.mark.parametrize("mode", ["sgd", "adagrad_weighted"])
 def test_plan_ahead_equals_single_call_backward(mode):
     """tbe_plan_batch on a side stream + tbe_backward_planned give bit-identical results to the
