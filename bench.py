@@ -254,6 +254,71 @@ def run_cached(args, w):
     print(json.dumps(result))
 
 
+def parity_gates(torch, ext, tbe_native, w, module, indices, offsets, psw, grad_output, step):
+    """Untimed checks after the timed region, torch only: the integer stages of the last backward
+    (sorted, a permutation, pairs intact, stable, strict run heads: bit-exact properties), one more
+    step against a snapshot (rows no lookup touches keep their bits; for SGD the column sums of
+    the update equal lr * the column sums of the gathered gradients, 1e-5), and the pooled output
+    of 512 bags against an fp64 gather-sum (1e-5 fp32, 1e-2 fp16).  A failed gate ends the run."""
+    dev = indices.device
+    T, E, D, B, n = w["T"], w["E"], w["D"], w["B"], w["n"]
+    out = {}
+    lengths = (offsets[1:] - offsets[:-1]).long()
+    table_of_position = torch.repeat_interleave(torch.arange(T, device=dev), lengths.view(T, B).sum(1))
+    keys = indices.long() + table_of_position * E
+    W = module.embedding_weights.data
+    tol = 1e-2 if w["fp16"] else 1e-5
+    if w["optimizer"]:
+        lay = tbe_native.backward_workspace_layout(n, D, tbe_native.DTYPE_F16 if w["fp16"] else tbe_native.DTYPE_F32, T)
+        ws = ext.backward_workspace(dev)
+        view = lambda off, cnt: ws[off:off + 4 * cnt].view(torch.int32)
+        ks, ps = view(lay.keys_sorted, n), view(lay.positions_sorted, n)
+        U = int(view(lay.num_unique, 1)[0])
+        ss = view(lay.segment_starts, U + 1).long()
+        same = ks[1:] == ks[:-1]
+        out["sort_is_sorted"] = bool((ks[1:] >= ks[:-1]).all())
+        out["sort_is_permutation"] = bool(torch.equal(torch.sort(ps.long())[0], torch.arange(n, device=dev)))
+        out["sort_keeps_pairs"] = bool(torch.equal(keys[ps.long()], ks.long()))
+        out["sort_is_stable"] = bool((ps[1:][same] > ps[:-1][same]).all())
+        out["unique_rows_match"] = U == int(torch.unique(keys).numel())
+        out["segments_are_runs"] = bool(int(ss[0]) == 0 and int(ss[-1]) == n and (ss[1:] > ss[:-1]).all()
+                                        and (ks[ss[1:-1]] != ks[ss[1:-1] - 1]).all())
+        before = W.clone()
+        step()
+        torch.cuda.synchronize()
+        touched = torch.zeros(W.shape[0], dtype=torch.bool, device=dev)
+        touched[keys] = True
+        out["untouched_rows_keep_bits"] = bool(torch.equal(W[~touched], before[~touched]))
+        if w["optimizer"] == "sgd":
+            bag_weight = lengths.view(T, B).t().contiguous().double()  # [B][T] lookups per bag
+            want = w["lr"] * (grad_output.double() * bag_weight.unsqueeze(-1)).sum((0, 1))
+            got = (before.double() - W.double()).sum(0)
+            err = float((got - want).abs().max() / want.abs().max())  # relative to the largest column sum
+            out["sgd_column_checksum_max_rel_err"] = err
+            out["sgd_column_checksum_ok"] = err <= 1e-5
+        del before
+    with torch.no_grad():
+        pooled = ext.forward(W, module.table_offsets, indices, offsets, psw, 200, 1, False)
+        bags = torch.randperm(T * B, device=dev, generator=torch.Generator(device=dev).manual_seed(1))[:512]
+        worst = 0.0
+        for bag in bags.tolist():
+            t, b = divmod(bag, B)
+            lo, hi = int(offsets[bag]), int(offsets[bag + 1])
+            rows = W[(t * E + indices[lo:hi].long())].double()
+            if psw is not None:
+                rows = rows * psw[lo:hi].double().unsqueeze(-1)
+            want = rows.sum(0)
+            got = pooled[b, t].double()
+            scale = float(want.abs().max().clamp_min(1e-6))
+            worst = max(worst, float((got - want).abs().max()) / scale)
+    out["forward_sample_max_rel_err"] = worst
+    out["forward_sample_ok"] = worst <= tol
+    failed = [k for k, v in out.items() if v is False]
+    if failed:
+        raise SystemExit("bench.py: parity gate failed: %s (%s)" % (", ".join(failed), json.dumps(out)))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -395,6 +460,7 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    result["parity"] = parity_gates(torch, ext, tbe_native, w, module, indices, offsets, psw, grad_output, step)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w, torch)
     else:
