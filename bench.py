@@ -33,13 +33,13 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 # this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
 # reads for a plain 1 GiB device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Keyed by (kernel, config).
 MEASURED_TRAFFIC = {
-    ("update_short", 3): int((1275360.5 * 2.0 + 1278141.7) * 1024),
-    ("update_chunks", 3): int((242600.2 * 2.0 + 8309.4) * 1024),
-    ("forward", 3): int((836333.5 * 2.0 + 131072.0) * 1024),
-    ("forward", 2): int((1227809.0 * 2.0 + 131072.0) * 1024),
-    ("update_short", 4): int((188417.4 * 2.0 + 188415.7) * 1024),
-    ("update_chunks", 4): int((70822.0 * 2.0 + 52396.2) * 1024),
-    ("forward", 4): int((84001.3 * 2.0 + 32768.0) * 1024),
+    ("update_short", 3): int((1274997.9 * 2.0 + 1278140.9) * 1024),
+    ("update_chunks", 3): int((242757.8 * 2.0 + 8308.9) * 1024),
+    ("forward", 3): int((836268.7 * 2.0 + 131072.0) * 1024),
+    ("forward", 2): int((1227766.6 * 2.0 + 131072.0) * 1024),
+    ("update_short", 4): int((188504.3 * 2.0 + 188517.1) * 1024),
+    ("update_chunks", 4): int((72265.6 * 2.0 + 53419.2) * 1024),
+    ("forward", 4): int((84006.1 * 2.0 + 32768.0) * 1024),
 }
 
 
