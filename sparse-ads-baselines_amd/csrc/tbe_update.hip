@@ -91,11 +91,11 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 // to a queue that update_chunks_kernel drains with one wavefront per chunk.
 // Tile size in sorted positions: 32 per lane group, so narrow rows (many groups per wavefront)
 // get larger tiles and the per-tile bookkeeping is amortised over the same number of rows.
-#ifndef TBE_TPG
-#define TBE_TPG 32
-#endif
+// (at most 256 positions; 64 for the variant whose row width is only known at run time)
 constexpr int tile_positions(int chunks_template) {
-  return chunks_template == 0 ? 64 : (chunks_template >= 32 ? 32 * (kWave / chunks_template) : (TBE_TPG * (kWave / chunks_template) > 256 ? 256 : TBE_TPG * (kWave / chunks_template)));
+  if (chunks_template == 0) return 64;
+  const int positions = 32 * (kWave / chunks_template);
+  return positions > 256 ? 256 : positions;
 }
 
 struct ChunkRecord {   // 32 bytes
@@ -304,8 +304,9 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
 
 // ------------------------------------------------ medium / long segments: chunks
 // One wavefront per chunk record.  The wavefronts of an XCD take the records of that XCD's
-// queue, consecutive records at the same time (see below for queues of unequal length).  Lane group r adds occurrences r, r + groups,
-// ... of the chunk; the groups are combined in a fixed tree.
+// queue, consecutive records at the same time (see below for queues of unequal length).  Lane
+// group r adds occurrences r, r + groups, ... of the chunk; the groups are combined in a fixed
+// tree.
 // A chunk that is a whole segment is applied to its row at once; a chunk of a longer
 // segment stores its sum as a partial row for update_long_finish_kernel.
 template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL>
@@ -679,7 +680,8 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   const dim3 grid_chunks(static_cast<unsigned>(
       kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), 1024))));
   TBE_LAUNCH("update_chunks", stream,
-             (update_chunks_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, (WEIGHTED && VEC == 8) ? 4 : kLongUnroll>), grid_chunks, block,
+             (update_chunks_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, (WEIGHTED && VEC == 8) ? 4 : kLongUnroll>),
+             grid_chunks, block,
              go, w, st, psw, gpsw, a.positions_sorted, a.grad_rows, a.counters, chunk_records,
              a.max_chunks, partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr,
              a.stochastic_rounding);
