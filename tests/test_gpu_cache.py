@@ -110,6 +110,60 @@ def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, sta
     ext.free_host_tensor(cached_w)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_cached_training_random_sweep(seed):
+    """Seeded random shapes of the cached-equals-uncached property: table counts and sizes, row
+    widths (narrow, odd vector counts, wider than 64 vectors), dtype, optimizer, policy, cache
+    and staging sizes from "nearly everything misses" to "everything fits", index skew."""
+    rs = np.random.RandomState(700 + seed)
+    T = int(rs.choice([1, 2, 5]))
+    rows = [int(rs.choice([3, 60, 900, 6000])) for _ in range(T)]
+    D = int(rs.choice([4, 12, 32, 64, 128, 260]))
+    dtype = [torch.float32, torch.float16, torch.float64][seed % 3]
+    mode = ["sgd", "adagrad", "adagrad_weighted"][(seed // 3) % 3]
+    policy = ["lru", "lfu"][seed % 2]
+    num_sets = int(rs.choice([1, 3, 17, 200]))
+    stage_slots = int(rs.choice([0, 5, 300, 100000]))
+    B, L, zipf = int(rs.choice([1, 30, 200])), int(rs.choice([1, 6, 25])), float(rs.choice([1.05, 1.3, 2.0]))
+    table_offsets = dev(np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
+    total = sum(rows)
+    start = (torch.rand(total, D, device=DEV, dtype=torch.float64) * 0.02 - 0.01).to(dtype)
+    plain_w = start.clone()
+    cached_w = ext.new_host_mapped_tensor(torch.empty(1, device=DEV, dtype=dtype), (total, D))
+    cached_w.copy_(start)
+    st_dtype = torch.float64 if dtype == torch.float64 else torch.float32
+    plain_state = torch.zeros(total, device=DEV, dtype=st_dtype)
+    cached_state = torch.zeros(total, device=DEV, dtype=st_dtype)
+    cache = tc.RowCache(cached_w, num_sets * 64, policy, stage_slots)
+    weighted = mode.endswith("weighted")
+    opt = "sgd" if mode == "sgd" else "adagrad"
+    for step in range(5):
+        indices, offsets = _draw_batch(rs, T, rows, B, L, zipf)
+        idx, off = dev(indices), dev(offsets)
+        go = torch.randn(B, T, D, device=DEV, dtype=torch.float64).to(dtype)
+        psw = torch.rand(indices.size, device=DEV, dtype=torch.float64).to(dtype) if weighted else None
+        want = ext.forward(plain_w, table_offsets, idx, off, psw, 200, 1, False)
+        if opt == "sgd":
+            ext.backward_sgd(go, plain_w, table_offsets, idx, off, 0.05, 200, 1, False)
+            want_g = None
+        else:
+            want_g = ext.backward_exact_adagrad(go, plain_w, table_offsets, idx, off, psw, plain_state, 0.05, 0.1,
+                                                False, 1)
+        cache.prepare(table_offsets, idx, off)
+        got = cache.forward(table_offsets, idx, off, psw)
+        got_g = cache.backward(opt, go, psw, cached_state, 0.05, 0.1)
+        assert torch.equal(got, want), "forward output differs at step %d" % step
+        if weighted and indices.size:
+            assert torch.equal(got_g, want_g)
+        resident = cache.resident_keys()
+        assert resident.numel() == torch.unique(resident).numel() <= num_sets * 64
+    cache.flush()
+    torch.cuda.synchronize()
+    assert torch.equal(cached_w, plain_w)
+    assert torch.equal(cached_state, plain_state)
+    ext.free_host_tensor(cached_w)
+
+
 @pytest.mark.parametrize("stage_slots", [100000, 9])
 def test_staging_leaves_cache_state_as_the_model_says(oracle, stage_slots):
     """A staged row is an uncached row of the model: tags, recency and frequency words are
