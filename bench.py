@@ -8,7 +8,7 @@ fused update) through autograd, as the reference's tests drive it
 (test_table_batched_embeddings.py:197-212).  Inputs are resident in HBM before the timed
 region.  Prints ONE JSON line.  Everything runs on one GPU.
 
-Default workload = BASELINE config 3 (the shape the target is quoted on):
+Default workload = configuration 3 (the shape the bandwidth target is quoted on):
 T=64 tables x 100k rows x D=128 fp32, B=4096 bags per table, L=20, Zipf(1.05) indices,
 exact SGD lr=0.01.  --config 2 times the forward alone on uniform indices; --config 4 the
 fp16 / weighted / exact row-wise Adagrad shape; --config 5 the DLRM-style shape whose tables
@@ -47,7 +47,7 @@ def make_workload(config, seed=0):
     rs = np.random.RandomState(seed)
     if config in (2, 3):
         T, E, D, B, L = 64, 100000, 128, 4096, 20
-        T = int(os.environ.get("TBE_BENCH_TABLES", T))  # experiments only; the default is the BASELINE shape
+        T = int(os.environ.get("TBE_BENCH_TABLES", T))  # experiments only; the default is the shape the target is quoted on
         lengths = np.full(T * B, L, dtype=np.int64)
         n = T * B * L
         if config == 2:

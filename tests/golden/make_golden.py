@@ -68,7 +68,7 @@ def torch_reference(T, E, D, B, lengths, offsets, indices, weights, grad_output,
 
 
 CASES = {
-    # BASELINE config 1: tiny TBE, T=2, E=1000, D=32 fp32, B=64, L=4, uniform indices, SGD lr=0.1, seed 0
+    # the smallest benchmark configuration: tiny TBE, T=2, E=1000, D=32 fp32, B=64, L=4, uniform indices, SGD lr=0.1, seed 0
     "cfg1_sgd_f32": dict(seed=0, T=2, E=1000, D=32, B=64, L=4, dtype=np.float32, optimizer="sgd", lr=0.1, eps=0.0),
     "ragged_adagrad_f32": dict(seed=1, T=3, E=50, D=16, B=40, L=9, dtype=np.float32, ragged=True, dup_heavy=True,
                                optimizer="adagrad", lr=0.5, eps=0.2),

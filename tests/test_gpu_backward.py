@@ -358,7 +358,7 @@ def test_gradcheck_on_per_sample_weights_in_double():
 
 
 def test_full_size_backward_properties():
-    """BASELINE config 3 shape (T=64, E=1e5, D=128 fp32, B=4096, L=20, Zipf(1.05) indices,
+    """The shape of bench.py --config 3 (T=64, E=1e5, D=128 fp32, B=4096, L=20, Zipf(1.05) indices,
     exact SGD lr=0.01).  Size-independent properties instead of the oracle:
     sortedness + permutation + stability of the sort, key/position consistency, strict
     segment boundaries, the column checksum of the update (linearity), untouched rows
@@ -412,7 +412,7 @@ def test_full_size_backward_properties():
 
 
 def test_full_size_weighted_adagrad_fp16_properties():
-    """BASELINE config 4 shape (T=32, E=1e6, D=64 fp16 weights, fp32 state from 0, B=8192, bag
+    """The shape of bench.py --config 4 (T=32, E=1e6, D=64 fp16 weights, fp32 state from 0, B=8192, bag
     lengths uniform in [0, 40] with empty bags, per-sample weights ~U(0,1), Zipf(1.2) indices,
     exact row-wise Adagrad lr=0.01 eps=1e-8): sort / segment properties, untouched rows and state
     bit-identical, and the first table (weights, state, per-sample-weight gradients) against the

@@ -1,5 +1,5 @@
 """GPU parity of the pooled forward (tbe_forward through the C ABI) against the CPU oracle,
-the EmbeddingBag fixtures, and size-independent properties at BASELINE's full shape.
+the EmbeddingBag fixtures, and size-independent properties at the benchmark's full shape.
 
 Tolerances (north star): fp32 1e-5 relative, fp16 1e-2; fp64 1e-12.  The kernel sums a
 bag in a different (fixed) order than the oracle's serial loop, so fp results are compared
@@ -139,7 +139,7 @@ def test_bad_arguments_raise_runtime_error():
 
 
 def test_full_size_forward_properties():
-    """BASELINE config 2 shape (T=64, E=1e5, D=128 fp32, B=4096, L=20, uniform indices).
+    """The shape of bench.py --config 2 (T=64, E=1e5, D=128 fp32, B=4096, L=20, uniform indices).
     The oracle is too slow for 5.2 M lookups, so: (a) the first two tables are compared with
     the oracle; (b) column checksum: sum_b,t out[b,t,:] == sum_p W[key_p,:] computed by an
     independent torch gather in fp64; (c) every output row of a table filled with a per-table
