@@ -167,19 +167,22 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
   acc.zero();
   for (int base = start; __ballot(base < end) != 0ull; base += kStep) {
     int idx[kPerLane], slot[kPerLane];
+    T w_raw[kPerLane];
     A w[kPerLane];
 #pragma unroll
     for (int q = 0; q < kPerLane; ++q) {
       const int p = base + q * CHUNKS + c;
-      idx[q] = 0;
+      idx[q] = 0;  // a lane without a lookup keeps row 0 of the table: loaded below, never added
       slot[q] = -1;
-      w[q] = A(0);
+      w_raw[q] = T(0);
       if (p < end) {
         idx[q] = __builtin_nontemporal_load(indices + p);
-        if constexpr (WEIGHTED) w[q] = to_acc(psw[p]);
+        if constexpr (WEIGHTED) w_raw[q] = psw[p];  // converted once all of the step's loads are issued
         if constexpr (CACHED) slot[q] = __builtin_nontemporal_load(lookup_slots + p);
       }
     }
+#pragma unroll
+    for (int q = 0; q < kPerLane; ++q) w[q] = WEIGHTED ? to_acc(w_raw[q]) : A(0);
 #pragma unroll
     for (int q = 0; q < kPerLane; ++q) {
       const int left = end - (base + q * CHUNKS);  // rows of this group's bag in this slice
@@ -202,18 +205,16 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
             const int s = shfl_idx(slot[q], src);
             if (s >= 0) row = cache_rows + static_cast<int64_t>(s) * D + static_cast<int64_t>(c) * VEC;
           }
-          if (ok[u]) raw[u] = V::load_raw(row);
+          raw[u] = V::load_raw(row);  // every lane loads (straight-line code keeps the loads back to back)
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-          if (ok[u]) {
-            V x;
-            x.unpack(raw[u]);
+          V x;
+          x.unpack(raw[u]);
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-              if constexpr (WEIGHTED) acc.v[k] += x.v[k] * ww[u];
-              else acc.v[k] += x.v[k];
-            }
+          for (int k = 0; k < VEC; ++k) {
+            const A term = WEIGHTED ? x.v[k] * ww[u] : x.v[k];
+            acc.v[k] += ok[u] ? term : A(0);
           }
         }
       }
