@@ -16,6 +16,7 @@
 // tuned per width like the uniform-D ones.  The integer stages (sort, segments) are shared.
 
 #include <algorithm>
+#include <type_traits>
 
 #include "tbe_stages.h"
 
@@ -30,6 +31,12 @@ template <> __device__ __forceinline__ double mixed_multiplier<double>(double s,
   return static_cast<double>(lr) * (1.0 / (sqrt(s) + static_cast<double>(eps)));
 }
 
+// One wavefront per bag.  A table's rows are `chunks` = D_t / VEC vectors; for rows of at most
+// 64 vectors the lanes form 64 / group_lanes lane groups (group_lanes = chunks rounded up to a
+// power of two: group and column of a lane are a shift and a mask whatever the width), the
+// groups split the bag's rows and are combined by a butterfly at the end -- a table of 32
+// columns keeps all 64 lanes busy with 8 rows per load instruction instead of 8 lanes with one.
+// Wider rows are walked in blocks of 64 vectors, one row per load.
 template <typename T, int VEC, bool WEIGHTED, int UNROLL>
 __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
     const T *__restrict__ weights, const int64_t *__restrict__ table_offsets,
@@ -54,6 +61,71 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
   const int end = offsets[bag + 1];
   T *out_row = output + static_cast<int64_t>(b) * total_D + dim_start;
 
+  if (chunks <= kWave) {
+    const int group_shift = chunks > 1 ? 32 - __builtin_clz(chunks - 1) : 0;
+    const int group_lanes = 1 << group_shift;
+    const int groups = kWave >> group_shift;
+    const int r = lane >> group_shift;
+    const int c = lane & (group_lanes - 1);
+    const bool active = c < chunks;
+    // a lane beside the row's columns loads the row's last vector and drops it
+    const T *col = table + static_cast<int64_t>(min(c, chunks - 1)) * VEC;
+    V acc;
+    acc.zero();
+    for (int base = start; base < end; base += kWave) {
+      const int n = min(kWave, end - base);
+      int my_idx = 0;
+      T my_w_raw = T(0);
+      if (lane < n) {
+        my_idx = __builtin_nontemporal_load(indices + base + lane);
+        if constexpr (WEIGHTED) my_w_raw = psw[base + lane];
+      }
+      const A my_w = WEIGHTED ? to_acc(my_w_raw) : A(0);
+      // `count` rows per lane group at a time; the loads of a step are straight-line code (every
+      // lane loads; a lane past the batch's end loads the batch's first row again and drops it)
+      // so they are issued back to back.  The step sizes 8, 4, 2, 1 follow the rows that are left,
+      // so that a bag of one row costs one load instruction, not eight.
+      int j0 = 0;
+      auto step = [&](auto count) {
+        constexpr int kCount = decltype(count)::value;
+        R raw[kCount];
+        A w[kCount];
+        bool ok[kCount];
+#pragma unroll
+        for (int u = 0; u < kCount; ++u) {
+          const int j = j0 + u * groups + r;
+          ok[u] = active && j < n;
+          const int src = j < n ? j : 0;
+          const int64_t idx = shfl_idx(my_idx, src);
+          if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, src);
+          raw[u] = V::load_raw(col + idx * D);
+        }
+#pragma unroll
+        for (int u = 0; u < kCount; ++u) {
+          V x;
+          x.unpack(raw[u]);
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) {
+            const A term = WEIGHTED ? x.v[i] * w[u] : x.v[i];
+            acc.v[i] += ok[u] ? term : A(0);
+          }
+        }
+        j0 += kCount * groups;
+      };
+      while (n - j0 >= groups * UNROLL) step(std::integral_constant<int, UNROLL>{});
+      if (n - j0 >= groups * 4) step(std::integral_constant<int, 4>{});
+      if (n - j0 >= groups * 2) step(std::integral_constant<int, 2>{});
+      while (j0 < n) step(std::integral_constant<int, 1>{});
+    }
+    // combine the groups (butterfly over the group index: every group ends with the sum)
+    for (int m = kWave >> 1; m >= group_lanes; m >>= 1) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc.v[i] += shfl_x(acc.v[i], m);
+    }
+    if (r == 0 && active) acc.store(out_row + static_cast<int64_t>(c) * VEC);
+    return;
+  }
+
   for (int cb = 0; cb < chunks; cb += kWave) {
     const int c = cb + lane;
     const bool ok_c = c < chunks;
@@ -68,18 +140,18 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
         my_idx = indices[base + lane];
         if constexpr (WEIGHTED) my_w = to_acc(psw[base + lane]);
       }
-      for (int j0 = 0; j0 < n; j0 += UNROLL) {
-        R raw[UNROLL];
-        A w[UNROLL];
+      for (int j0 = 0; j0 < n; j0 += 4) {
+        R raw[4];
+        A w[4];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
+        for (int u = 0; u < 4; ++u) {
           const int j = min(j0 + u, n - 1);
           const int64_t idx = shfl_idx(my_idx, j);
           if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, j);
           if (ok_c && j0 + u < n) raw[u] = V::load_raw(col + idx * D);
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
+        for (int u = 0; u < 4; ++u) {
           if (ok_c && j0 + u < n) {
             V x;
             x.unpack(raw[u]);
@@ -701,10 +773,10 @@ void launch_forward_mixed(const MixedArgs &a, hipStream_t stream) {
   const T *p = static_cast<const T *>(a.psw);
   T *o = static_cast<T *>(a.output);
   if (a.psw)
-    TBE_LAUNCH("forward_mixed", stream, (forward_mixed_kernel<T, VEC, true, 4>), grid, block, w,
+    TBE_LAUNCH("forward_mixed", stream, (forward_mixed_kernel<T, VEC, true, 8>), grid, block, w,
                a.table_offsets, a.dim_offsets, a.indices, a.offsets, p, o, a.B, a.total_D, num_bags, per_xcd);
   else
-    TBE_LAUNCH("forward_mixed", stream, (forward_mixed_kernel<T, VEC, false, 4>), grid, block, w,
+    TBE_LAUNCH("forward_mixed", stream, (forward_mixed_kernel<T, VEC, false, 8>), grid, block, w,
                a.table_offsets, a.dim_offsets, a.indices, a.offsets, p, o, a.B, a.total_D, num_bags, per_xcd);
 }
 
