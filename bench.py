@@ -33,13 +33,13 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 # this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
 # reads for a plain 1 GiB device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Keyed by (kernel, config).
 MEASURED_TRAFFIC = {
-    ("update_short", 3): int((1274997.9 * 2.0 + 1278140.9) * 1024),
-    ("update_chunks", 3): int((242757.8 * 2.0 + 8308.9) * 1024),
-    ("forward", 3): int((836268.7 * 2.0 + 131072.0) * 1024),
-    ("forward", 2): int((1227766.6 * 2.0 + 131072.0) * 1024),
-    ("update_short", 4): int((188504.3 * 2.0 + 188517.1) * 1024),
-    ("update_chunks", 4): int((72265.6 * 2.0 + 53419.2) * 1024),
-    ("forward", 4): int((84006.1 * 2.0 + 32768.0) * 1024),
+    ("update_short", 3): int((1274937.7 * 2.0 + 1278141.8) * 1024),
+    ("update_chunks", 3): int((242588.5 * 2.0 + 8309.0) * 1024),
+    ("forward", 3): int((836296.1 * 2.0 + 131072.0) * 1024),
+    ("forward", 2): int((1227738.4 * 2.0 + 131072.0) * 1024),
+    ("update_short", 4): int((188383.6 * 2.0 + 188470.0) * 1024),
+    ("update_chunks", 4): int((72411.1 * 2.0 + 53625.9) * 1024),
+    ("forward", 4): int((84678.9 * 2.0 + 32768.0) * 1024),
 }
 
 
