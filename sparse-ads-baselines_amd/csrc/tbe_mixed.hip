@@ -60,6 +60,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
   const int start = offsets[bag];
   const int end = offsets[bag + 1];
   T *out_row = output + static_cast<int64_t>(b) * total_D + dim_start;
+  if (chunks <= 0) return;  // a table without columns has no output
 
   if (chunks <= kWave) {
     const int group_shift = chunks > 1 ? 32 - __builtin_clz(chunks - 1) : 0;
