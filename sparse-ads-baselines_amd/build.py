@@ -49,7 +49,10 @@ def build(verbose=False):
     hipcc = _hipcc()
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
-    sources = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    sources = list(SOURCES)
+    missing = [s for s in sources if not os.path.exists(os.path.join(CSRC, s))]
+    if missing:  # a library linked without one of its files would only fail at symbol lookup
+        raise RuntimeError("missing HIP sources under %s: %s" % (CSRC, ", ".join(missing)))
     objects = [os.path.join(obj_dir, s.replace(".hip", ".o")) for s in sources]
 
     def compile_one(pair):

@@ -162,6 +162,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
   const int end = valid ? offsets[bag + 1] : start;
   const int64_t table_row0 = table_offsets[t];
   const T *col = weights + static_cast<int64_t>(c) * VEC;
+  const int idle_idx = -static_cast<int>(table_row0);
 
   V acc;
   acc.zero();
@@ -172,8 +173,11 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
 #pragma unroll
     for (int q = 0; q < kPerLane; ++q) {
       const int p = base + q * CHUNKS + c;
-      idx[q] = 0;  // a lane without a lookup keeps row 0 of the table: loaded below, never added
-      slot[q] = -1;
+      // A lane without a lookup still loads (never adds) a row: row 0 of `weights` -- the index
+      // cancels the table's first row, so the address exists even for a table without rows -- or,
+      // behind the row cache, slot 0, so that idle lanes never reach over the host link.
+      idx[q] = idle_idx;
+      slot[q] = CACHED ? 0 : -1;
       w_raw[q] = T(0);
       if (p < end) {
         idx[q] = __builtin_nontemporal_load(indices + p);

@@ -278,17 +278,23 @@ def _check_mixed(weights, table_offsets, dim_offsets, indices, offsets):
 
 
 # fp16 rows are moved 16 bytes at a time when every table's D allows it, else 8 bytes.  The choice
-# needs the per-table dims on the host; it is cached per dim_offsets tensor.
-_fp16_width = {}
+# (and the one-time check that every D_t is a positive multiple of 4) needs the per-table dims on
+# the host; it is cached per dim_offsets tensor, identified the way max_table_rows identifies its
+# tensor: a data pointer says nothing once the allocator has recycled the block.
+_fp16_width = {}  # id(dim_offsets) -> (weak reference, tensor version, vector width)
 
 
 def _fp16_vector_width(dim_offsets):
-    key = (dim_offsets.data_ptr(), dim_offsets.numel())
-    if key not in _fp16_width:
-        dims = torch.diff(dim_offsets).cpu()
-        _require(bool((dims % 4 == 0).all()) and bool((dims > 0).all()), "every D_t must be a positive multiple of 4")
-        _fp16_width[key] = 8 if bool((dims % 8 == 0).all()) else 4
-    return _fp16_width[key]
+    ident = id(dim_offsets)
+    hit = _fp16_width.get(ident)
+    if hit is not None and hit[0]() is dim_offsets and hit[1] == dim_offsets._version:
+        return hit[2]
+    dims = torch.diff(dim_offsets).cpu()
+    _require(bool((dims % 4 == 0).all()) and bool((dims > 0).all()), "every D_t must be a positive multiple of 4")
+    width = 8 if bool((dims % 8 == 0).all()) else 4
+    ref = weakref.ref(dim_offsets, lambda _, ident=ident: _fp16_width.pop(ident, None))
+    _fp16_width[ident] = (ref, dim_offsets._version, width)
+    return width
 
 
 def forward_mixed_D(weights, table_offsets, dim_offsets, total_D, indices, offsets, indice_weights, L_max,

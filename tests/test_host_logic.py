@@ -89,3 +89,43 @@ def test_bench_refuses_more_than_one_gpu():
     out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True,
                          text=True, timeout=120)
     assert out.returncode != 0 and "one GPU" in out.stderr and out.stdout.strip() == ""
+
+
+def test_fp16_vector_width_is_cached_per_tensor_not_per_address():
+    """Two dim_offsets tensors that the allocator places at one address (same T) keep their own
+    widths and their own D_t % 4 check; an in-place edit of the tensor invalidates its entry."""
+    first = torch.tensor([0, 8, 24, 40], dtype=torch.int32)          # widths 8, 16, 16
+    address = first.data_ptr()
+    assert ext._fp16_vector_width(first) == 8
+    # the same storage, reinterpreted as another tensor object with other dims (what a recycled
+    # allocator block looks like): same data pointer, same number of entries
+    second = torch.empty(0, dtype=torch.int32).set_(first.untyped_storage(), 0, (4,))
+    assert second.data_ptr() == address and second.numel() == first.numel()
+    second.copy_(torch.tensor([0, 12, 24, 40], dtype=torch.int32))   # widths 12, 12, 16
+    assert ext._fp16_vector_width(second) == 4
+    # an in-place edit of a tensor invalidates its own entry
+    third = torch.tensor([0, 8, 16], dtype=torch.int32)
+    assert ext._fp16_vector_width(third) == 8
+    third[2] = 20
+    assert ext._fp16_vector_width(third) == 4
+    bad = torch.tensor([0, 6, 12], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        ext._fp16_vector_width(bad)
+    # entries die with their tensors
+    ident = id(bad)
+    del bad
+    assert ident not in ext._fp16_width
+
+
+def test_build_refuses_a_missing_source(tmp_path, monkeypatch):
+    import importlib.util
+    import os
+    from conftest import ROOT
+    spec = importlib.util.spec_from_file_location(
+        "tbe_build_under_test", os.path.join(ROOT, "sparse-ads-baselines_amd", "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    monkeypatch.setattr(mod, "SOURCES", mod.SOURCES + ["not_there.hip"])
+    monkeypatch.setattr(mod, "LIB_PATH", str(tmp_path / "lib.so"))
+    with pytest.raises(RuntimeError, match="not_there.hip"):
+        mod.build()
