@@ -2,10 +2,14 @@
  * tbe_hip.h -- C ABI of the MI355X (gfx950) table-batched embedding-bag library.
  *
  * Every entry point takes plain device pointers, sizes and an opaque HIP stream
- * (a hipStream_t passed as void*; NULL = the default stream).  Nothing here
- * allocates device memory: scratch is a caller-owned workspace whose size is
- * reported by the *_workspace_* queries.  No entry point synchronises the host
- * with the device.
+ * (a hipStream_t passed as void*; NULL = the default stream).  No compute entry
+ * point allocates device memory: scratch is a caller-owned workspace whose size
+ * is reported by the *_workspace_* queries (tbe_backward_sgd_static uses an array
+ * the library holds instead).  The exceptions are the allocators at the end of
+ * this file (tbe_host_mapped_alloc, tbe_managed_alloc), the HIP events that the
+ * kernel-timing aid creates between tbe_profile_begin/end, and the two events
+ * tbe_cache_prepare creates once per calling thread to join its side stream.  No entry
+ * point other than tbe_profile_end synchronises the host with the device.
  *
  * Return value: 0 (TBE_OK) on success, a TBE_ERR_* code otherwise; the message
  * of the last failure on the calling thread is returned by tbe_last_error().
@@ -139,6 +143,29 @@ TBE_API int tbe_backward_sgd(const void *grad_output, void *weights, int32_t dty
                      const int32_t *offsets, int32_t B,
                      float learning_rate,
                      void *workspace, uint64_t workspace_bytes, void *stream);
+
+/* tbe_backward_sgd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference,
+ * which allocates its sort buffers inside every backward call
+ * (table_batched_embeddings_cuda.cu:1618-1647).  Same arguments, same kernels and bit-identical
+ * results, but the workspace is an array of TBE_STATIC_SCRATCH_BYTES that the library's code
+ * object holds on every device it runs on; the call makes no hipMalloc / hipFree and no other
+ * allocating call.  A batch whose workspace (tbe_backward_workspace_layout(...).total_bytes)
+ * exceeds TBE_STATIC_SCRATCH_BYTES is refused with TBE_ERR_WORKSPACE -- about 0.8 M lookups fit.
+ * The first call on a device resolves the array's address there (make it outside a capture).
+ * All calls on one device share the array, which keeps the previous call's contents: every
+ * counter the pipeline needs at zero is cleared by its own kernels at the start of each call,
+ * and two calls that overlap on one device (different streams or threads) race.  After the call
+ * the array holds the intermediate results in the layout of tbe_backward_workspace_layout, as a
+ * caller's workspace would.
+ */
+#define TBE_STATIC_SCRATCH_BYTES (32ull << 20)
+TBE_API int tbe_backward_sgd_static(const void *grad_output, void *weights, int32_t dtype,
+                                    int64_t total_rows, int64_t max_table_rows, int32_t D,
+                                    const int32_t *table_offsets, int32_t T,
+                                    const int32_t *indices, int64_t num_indices,
+                                    const int32_t *offsets, int32_t B,
+                                    float learning_rate, void *stream);
 
 /* Exact row-wise Adagrad (table_batched_embeddings_cuda.cu:1589-1706 with
  * AdaGradFunctor, :437-471; "backward_exact_adagrad" in table_batched_embeddings.cpp:61):

@@ -7,6 +7,8 @@
 
 #include <math.h>
 
+#include <mutex>
+
 #include "tbe_stages.h"
 
 namespace tbe {
@@ -201,6 +203,72 @@ extern "C" int tbe_backward_sgd(const void *grad_output, void *weights, int32_t 
                       workspace, workspace_bytes, static_cast<hipStream_t>(stream), tbe::kOptSgd,
                       false, nullptr, nullptr, tbe::StochasticRounding{0, 0, 0}};
   return tbe::run_backward("tbe_backward_sgd", c);
+}
+
+// ------------------------------------------------------------ library-held scratch
+// tbe_backward_sgd_static runs tbe_backward_sgd's pipeline on this array instead of a caller's
+// workspace, for callers that may not allocate.  The array belongs to the code object: every
+// device the library runs on holds its own copy, at its own address, until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; the address kernels
+// and layouts use is the one that call returns for the current device.
+static __device__ __align__(256) unsigned char scratch[TBE_STATIC_SCRATCH_BYTES];
+
+namespace tbe {
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_address[kMaxDevices] = {};  // per device, resolved on the first call there
+
+// Device address of `scratch` on the current device.
+int static_scratch(const char *name, void **address) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(TBE_ERR_HIP, "%s: hipGetDevice: %s", name, hipGetErrorString(e));
+  if (device < 0 || device >= kMaxDevices)
+    return fail(TBE_ERR_UNSUPPORTED, "%s: device %d is beyond the %d devices tracked", name, device, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_address[device]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(TBE_ERR_HIP, "%s: hipGetSymbolAddress(scratch) on device %d: %s", name, device,
+                  hipGetErrorString(e));
+    g_scratch_address[device] = p;
+  }
+  *address = g_scratch_address[device];
+  return TBE_OK;
+}
+}  // namespace
+}  // namespace tbe
+
+extern "C" int tbe_backward_sgd_static(const void *grad_output, void *weights, int32_t dtype,
+                                       int64_t total_rows, int64_t max_table_rows, int32_t D,
+                                       const int32_t *table_offsets, int32_t T,
+                                       const int32_t *indices, int64_t num_indices,
+                                       const int32_t *offsets, int32_t B, float learning_rate,
+                                       void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_backward_sgd_static";
+  // the layout query's own preconditions, so that a bad shape is reported as such and not as a size
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(D > 0 && D % 4 == 0, "%s: D must be a positive multiple of 4 (got %d)", name, D);
+  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
+  TBE_REQUIRE(T > 0, "%s: T must be positive (got %d)", name, T);
+  tbe_workspace_layout_t l;
+  compute_layout(num_indices, D, dtype, T, &l);
+  if (l.total_bytes > TBE_STATIC_SCRATCH_BYTES)
+    return fail(TBE_ERR_WORKSPACE,
+                "%s: %lld lookups of %d tables need %llu bytes of scratch, the library holds %llu; "
+                "use tbe_backward_sgd with a workspace of the caller's",
+                name, (long long)num_indices, T, (unsigned long long)l.total_bytes,
+                (unsigned long long)TBE_STATIC_SCRATCH_BYTES);
+  void *address = nullptr;
+  if (int rc = static_scratch(name, &address)) return rc;
+  BackwardCall c{grad_output, weights, dtype, total_rows, max_table_rows, D, table_offsets, T, indices,
+                 num_indices, offsets, B, nullptr, nullptr, learning_rate, 0.0f, nullptr,
+                 address, TBE_STATIC_SCRATCH_BYTES, static_cast<hipStream_t>(stream), kOptSgd,
+                 false, nullptr, nullptr, StochasticRounding{0, 0, 0}};
+  return run_backward(name, c);
 }
 
 extern "C" int tbe_backward_exact_adagrad(const void *grad_output, void *weights, int32_t dtype,

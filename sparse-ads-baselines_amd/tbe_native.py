@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -68,6 +68,7 @@ class CacheWorkspaceLayout(ctypes.Structure):
 
 
 CACHE_WAYS = 64
+STATIC_SCRATCH_BYTES = 32 << 20  # TBE_STATIC_SCRATCH_BYTES
 CACHE_LRU, CACHE_LFU = 0, 1
 OPT_SGD, OPT_ROWWISE_ADAGRAD = 0, 1
 _cache_p = ctypes.POINTER(Cache)
@@ -84,6 +85,8 @@ SIGNATURES = {
     "tbe_backward_workspace_layout": (ctypes.c_int, [_i64, _i32, _i32, _i32, ctypes.POINTER(WorkspaceLayout)]),
     "tbe_backward_sgd": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p,
                                         _i32, _f32, _vp, _u64, _vp]),
+    "tbe_backward_sgd_static": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
+                                               _c_i32p, _i32, _f32, _vp]),
     "tbe_backward_exact_adagrad": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
                                                   _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _vp, _u64, _vp]),
     "tbe_plan_batch": (ctypes.c_int, [_c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _i64, _i64, _i32, _i32, _vp, _u64, _vp]),
