@@ -67,14 +67,7 @@ def make_workload(config, seed=0):
                 "lr=0.01 eps=1e-8")
         w = dict(T=T, E=E, D=D, B=B, fp16=True, weighted=True, optimizer="adagrad", lr=0.01, eps=1e-8)
     elif config == 5:
-        T, D, B = 26, 128, 65536
-        rows = np.floor(np.exp(rs.uniform(np.log(1e3), np.log(2e7), size=T))).astype(np.int64)
-        w = dict(T=T, E=[int(r) for r in rows], D=D, B=B, fp16=False, weighted=False, optimizer="sgd", lr=0.01,
-                 eps=0.0, cache_slots=1 << 22, stage_slots=1 << 23, n=0, seed=seed, indices=None, offsets=None,
-                 name="cfg5 DLRM-style + row cache: T=26 rows log-uniform [1e3,2e7] (sum %d) D=128 fp32 in pinned host "
-                      "memory, 2^22-slot LRU cache + 2^23 staging rows, B=65536 L=clip(Poisson(30),1,100) Zipf(1.1) per-table hot set, "
-                      "fwd + exact SGD lr=0.01, indices re-drawn every step" % int(rows.sum()))
-        return w
+        return make_cfg5_workload(seed)
     else:
         raise SystemExit("bench.py: --config must be 2, 3, 4 or 5")
     w["name"] = name
@@ -83,6 +76,23 @@ def make_workload(config, seed=0):
     w["n"] = n
     w["seed"] = seed
     return w
+
+
+def make_cfg5_workload(seed=0, T=26, D=128, B=65536, row_range=(1e3, 2e7), cache_slots=1 << 22,
+                       stage_slots=1 << 23):
+    """Configuration 5: T tables whose row counts are log-uniform in `row_range` (fixed by the
+    seed), in pinned host memory behind an LRU row cache of `cache_slots` slots; the staging area
+    (rows that find no slot in a step) is twice the cache.  The other arguments scale the same
+    workload down for tests."""
+    rs = np.random.RandomState(seed)
+    rows = np.floor(np.exp(rs.uniform(np.log(row_range[0]), np.log(row_range[1]), size=T))).astype(np.int64)
+    return dict(T=T, E=[int(r) for r in rows], D=D, B=B, fp16=False, weighted=False, optimizer="sgd", lr=0.01,
+                eps=0.0, cache_slots=cache_slots, stage_slots=stage_slots, n=0, seed=seed, indices=None,
+                offsets=None,
+                name="cfg5 DLRM-style + row cache: T=%d rows log-uniform [%g,%g] (sum %d) D=%d fp32 in pinned host "
+                     "memory, %d-slot LRU cache + %d staging rows, B=%d L=clip(Poisson(30),1,100) Zipf(1.1) "
+                     "per-table hot set, fwd + exact SGD lr=0.01, indices re-drawn every step"
+                     % (T, row_range[0], row_range[1], int(rows.sum()), D, cache_slots, stage_slots, B))
 
 
 def zipf_on_device(torch, a, n, gen, dev):

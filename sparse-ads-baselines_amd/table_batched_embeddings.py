@@ -20,7 +20,7 @@ _DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F
 # buffers, segment lists).  The reference allocates these per call
 # (table_batched_embeddings_cuda.cu:1618-1647).
 _workspaces = {}
-# Storage of host-resident tensors handed out by new_*_tensor, keyed by data pointer.
+# Owners of the host-resident allocations handed out by new_*_tensor (weak), keyed by device address.
 _host_allocations = {}
 
 
@@ -398,13 +398,47 @@ def construct_offsets(batch_offsets_per_table, total_indices_per_table):
     return output
 
 
-class _DeviceArray:
-    """Exposes a raw device-visible address to torch through __cuda_array_interface__."""
+class _HostAllocation:
+    """Owner of one host-resident allocation, exposed to torch through __cuda_array_interface__.
 
-    def __init__(self, ptr, shape, typestr):
-        self.__cuda_array_interface__ = {"shape": tuple(shape), "typestr": typestr, "data": (ptr, False),
+    torch.as_tensor keeps a reference to the exporting object inside the tensor's storage and drops
+    it when the last tensor (or view, or Parameter) on that storage dies, so releasing the memory
+    here ties it to the storage's lifetime -- the role of the deleters that the reference attaches
+    to its DataPtrs (CUDAManagedDeleter / CUDAHostMappedDeleter,
+    table_batched_embeddings_cuda.cu:795-835).  free_host_tensor() releases it early."""
+
+    def __init__(self, device_ptr, numel, typestr, device, release):
+        self.__cuda_array_interface__ = {"shape": (int(numel),), "typestr": typestr, "data": (device_ptr, False),
                                          "version": 2, "strides": None}
+        self.device_ptr = device_ptr
+        self._device = device
+        self._release = release
 
+    def release(self):
+        """Frees the allocation once (kernels that still use it are waited for); returns the
+        library's return code, or None when it was released before."""
+        release, self._release = self._release, None
+        if release is None:
+            return None
+        _host_allocations.pop(self.device_ptr, None)
+        try:
+            torch.cuda.synchronize(self._device)
+        except Exception:  # interpreter shutdown: the runtime may be gone already
+            pass
+        code = release()
+        for callback in list(release_observers):
+            callback(self.device_ptr)
+        return code
+
+    def __del__(self):
+        try:
+            self.release()
+        except Exception:
+            pass
+
+
+# Called with the device address of every host allocation that is released (tests observe this).
+release_observers = []
 
 _TYPESTR = {torch.float32: "<f4", torch.float16: "<f2", torch.float64: "<f8"}
 
@@ -413,15 +447,17 @@ def _wrap_host_memory(self, sizes, device_ptr, release):
     numel = 1
     for s in sizes:
         numel *= int(s)
-    tensor = torch.as_tensor(_DeviceArray(device_ptr, (numel,), _TYPESTR[self.dtype]), device=self.device)
-    tensor = tensor.view(*[int(s) for s in sizes])
-    _host_allocations[tensor.data_ptr()] = release
+    owner = _HostAllocation(device_ptr, numel, _TYPESTR[self.dtype], self.device, release)
+    tensor = torch.as_tensor(owner, device=self.device).view(*[int(s) for s in sizes])
+    # weak: the storage holds the only strong reference, so dropping the tensor frees the memory
+    _host_allocations[device_ptr] = weakref.ref(owner)
     return tensor
 
 
 def new_managed_tensor(self, sizes):
     """new_managed_tensor (table_batched_embeddings_cuda.cu:864-871): a tensor tagged with
-    `self`'s device and dtype whose pages are managed memory preferring the host."""
+    `self`'s device and dtype whose pages are managed memory preferring the host.  The memory is
+    released when the tensor's storage dies, as the reference's CUDAManagedDeleter does (:795)."""
     _require(self.is_cuda and self.dtype in _TYPESTR, "prototype must be a floating GPU tensor")
     nbytes = self.element_size()
     for s in sizes:
@@ -436,7 +472,11 @@ def new_managed_tensor(self, sizes):
 
 def new_host_mapped_tensor(self, sizes):
     """new_host_mapped_tensor (table_batched_embeddings_cuda.cu:873-880): pinned host memory
-    mapped into the device's address space, tagged as a tensor on `self`'s device."""
+    mapped into the device's address space, tagged as a tensor on `self`'s device; released when
+    the tensor's storage dies (CUDAHostMappedDeleter, :812-818).  Unlike the reference (:823) the
+    pages are not write-combined: the host reads this table (checkpoints, state_dict, the CPU
+    side of tests), and reads of write-combined memory bypass the CPU caches; the GPU's accesses
+    over the link are the same either way."""
     _require(self.is_cuda and self.dtype in _TYPESTR, "prototype must be a floating GPU tensor")
     nbytes = self.element_size()
     for s in sizes:
@@ -451,9 +491,10 @@ def new_host_mapped_tensor(self, sizes):
 
 
 def free_host_tensor(tensor):
-    """Releases the storage behind a tensor made by new_managed_tensor / new_host_mapped_tensor.
-    The tensor (and every view of it) must not be used afterwards."""
-    release = _host_allocations.pop(tensor.data_ptr(), None)
-    _require(release is not None, "tensor was not allocated by this module")
-    torch.cuda.synchronize(tensor.device)
-    _native.check(release())
+    """Releases the storage behind a tensor made by new_managed_tensor / new_host_mapped_tensor
+    right away instead of when its storage dies.  The tensor (and every view of it) must not be
+    used afterwards."""
+    ref = _host_allocations.get(tensor.data_ptr())
+    owner = ref() if ref is not None else None
+    _require(owner is not None, "tensor was not allocated by this module")
+    _native.check(owner.release() or 0)

@@ -53,11 +53,15 @@ class RowCache:
                                     _ptr(self.backing), self.num_sets, _POLICIES[policy], self.stage_slots)
         self.side_stream = torch.cuda.Stream(device=self.device)  # default priority
         self.step = 0
+        # prepare() leaves ONE plan (sort, slots of this batch's rows) in the workspaces; plan_id
+        # names it, so that a backward can tell whether the plan is still the one of its forward
+        self.plan_id = 0
         self._plan_ws = None
         self._cache_ws = None
         self._layout = None
         self._plan_layout = None
         self._n = 0
+        self._planned_backward_done = True  # nothing is planned yet
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_cache_init(ctypes.byref(self.handle), self._stream()))
 
@@ -79,7 +83,9 @@ class RowCache:
         B = (offsets.numel() - 1) // T
         n = indices.numel()
         self.step += 1
+        self.plan_id += 1
         self._n, self._T, self._B = n, T, B
+        self._planned_backward_done = False
         self._plan_layout = _native.backward_workspace_layout(n, self.D, self.dtype_code, T)
         self._layout = _native.cache_workspace_layout(n, self.num_sets)
         self._plan_ws = self._grow(self._plan_ws, self._plan_layout.total_bytes)
@@ -125,10 +131,26 @@ class RowCache:
         return output
 
     def backward(self, optimizer, grad_output, per_sample_weights, optimizer_state, learning_rate, eps,
-                 stochastic_rounding=None):
+                 stochastic_rounding=None, plan_id=None):
         """optimizer: 'sgd' or 'adagrad'.  Updates rows where they live; returns the gradient
         w.r.t. per_sample_weights or None.  stochastic_rounding: None, or the (seed, offset) of
-        the random stream that rounds updated fp16 weights (Adagrad only)."""
+        the random stream that rounds updated fp16 weights (Adagrad only).  plan_id: the value of
+        self.plan_id after the prepare() of the batch this gradient belongs to; a later prepare()
+        has replaced that batch's plan and slots (and may have evicted its rows), so the call is
+        refused instead of applying the gradient to another batch's rows."""
+        if plan_id is not None and plan_id != self.plan_id:
+            raise RuntimeError(
+                "the row cache was prepared for another batch since this batch's forward (plan %d, now %d): "
+                "a cache-fronted module holds one planned batch at a time -- run each forward's backward "
+                "before the next forward" % (plan_id, self.plan_id))
+        if self._planned_backward_done:
+            raise RuntimeError("this batch's backward has already run; its plan serves one update")
+        if (grad_output.dtype != self.backing.dtype or grad_output.device != self.device
+                or tuple(grad_output.shape) != (self._B, self._T, self.D)):
+            raise RuntimeError("grad_output must be [B=%d, T=%d, D=%d] of %s on %s (got %s of %s)"
+                               % (self._B, self._T, self.D, self.backing.dtype, self.device,
+                                  tuple(grad_output.shape), grad_output.dtype))
+        self._planned_backward_done = True
         grad_output = grad_output.contiguous()
         grad_psw = None
         if per_sample_weights is not None:
@@ -151,6 +173,20 @@ class RowCache:
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_cache_flush(ctypes.byref(self.handle), self.dtype_code, self.D,
                                                          self._stream()))
+
+    def invalidate(self, write_back=True):
+        """Empties the cache (tags, recency and frequency words back to their initial values), after
+        writing the resident rows back to the backing table unless write_back is False.  Needed
+        whenever the backing table is written behind the cache's back (loading a checkpoint,
+        assigning to the weights): a resident row would otherwise keep serving, and later write
+        back, its old value.  Any planned batch is dropped."""
+        if write_back:
+            self.flush()
+        self.plan_id += 1
+        self._planned_backward_done = True
+        self._n = 0
+        with torch.cuda.device(self.device):
+            _native.check(_native.load().tbe_cache_init(ctypes.byref(self.handle), self._stream()))
 
     def resident_keys(self):
         """Sorted keys of the rows currently held (synchronises)."""

@@ -109,6 +109,7 @@ class CachedLookupFunction(torch.autograd.Function):
         cache = module.row_cache
         cache.prepare(module.table_offsets, indices, offsets)
         ctx.module = module
+        ctx.plan_id = cache.plan_id
         ctx.save_for_backward(weights, per_sample_weights)
         return cache.forward(module.table_offsets, indices, offsets, per_sample_weights)
 
@@ -126,7 +127,7 @@ class CachedLookupFunction(torch.autograd.Function):
             rounding = table_batched_embeddings._rounding_stream(weights.device)
         grad_per_sample_weight = module.row_cache.backward(
             kind, grad_output, per_sample_weights, module.optimizer_state, module.learning_rate, module.eps,
-            rounding)
+            rounding, plan_id=ctx.plan_id)
         empty_grad = None
         if ctx.needs_input_grad[0]:
             empty_grad = torch.sparse_coo_tensor(
@@ -172,8 +173,11 @@ class TableBatchedEmbeddingBags(nn.Module):
             assert cache_slots is not None, "HOST_CACHED needs cache_slots"
             self.row_cache = table_batched_embeddings_cache.RowCache(self.embedding_weights.data, cache_slots,
                                                                      cache_policy, cache_stage_slots)
-            # checkpoints must see the rows the cache holds
+            # checkpoints must see the rows the cache holds ...
             self.register_state_dict_pre_hook(lambda module, prefix, keep_vars: module.flush_cache())
+            # ... and a loaded checkpoint must not be shadowed (or later overwritten) by rows that
+            # were resident before it was loaded
+            self.register_load_state_dict_pre_hook(lambda module, *args: module.invalidate_cache())
         self.register_buffer("table_offsets",
                              torch.tensor([0] + np.cumsum(rows[:-1]).tolist()).int())
         # unused by SGD, kept so state dicts interchange (table_batched_embeddings_ops.py:177-180)
@@ -187,6 +191,12 @@ class TableBatchedEmbeddingBags(nn.Module):
         """Writes the rows held by the HBM cache back to embedding_weights (no-op without a cache)."""
         if self.row_cache is not None:
             self.row_cache.flush()
+
+    def invalidate_cache(self):
+        """Writes the resident rows back, then empties the cache.  Call it after writing to
+        embedding_weights directly (load_state_dict does so itself); no-op without a cache."""
+        if self.row_cache is not None:
+            self.row_cache.invalidate()
 
     def forward(self, sharded_sparse_features, sharded_offsets, per_sample_weights=None):
         if self.row_cache is not None:

@@ -268,15 +268,48 @@ def test_hot_rows_take_the_chunked_path(oracle, dtype, D, mode):
     # each of the eight XCDs]
     assert got["views"]["counters"][1] == (lengths > 256).sum()
     assert got["views"]["counters"][8:16].sum() == np.ceil(lengths[lengths > 16] / 256).sum()
-    # long serial fp32 sums: the oracle itself is ~1e-4 from the fp64 truth here, so compare
-    # both against each other at the accumulated-rounding level
-    tol = {np.dtype(np.float32): 2e-4, np.dtype(np.float16): 1e-2, np.dtype(np.float64): 1e-7}[np.dtype(dtype)]
     np.testing.assert_array_equal(got["views"]["positions_sorted"], ref["positions_sorted"])
     np.testing.assert_array_equal(got["views"]["segment_starts"], ref["segment_starts"])
-    assert_close(got["weights"], w, tol)
+    # The truth is the update computed in fp64 from the same inputs.  The HIP path has to be within
+    # the stated tolerance of IT (fp32: 1e-5 relative), and no further from it than the oracle's
+    # serial fp32 sum is (the oracle adds ~42 k terms one by one, the kernels in trees of chunks).
+    tol = TOL[np.dtype(dtype)]
+    w64, st64 = _fp64_update(p, optimizer, 0.001, 0.1)
+    assert_close(got["weights"], w64, tol, "HIP weights vs fp64")
+    err_gpu = np.abs(got["weights"].astype(np.float64) - w64).max()
+    err_oracle = np.abs(w.astype(np.float64) - w64).max()
+    floor = np.abs(w64).max() * np.finfo(np.dtype(dtype)).eps  # one rounding of the stored weight
+    if dtype != np.float64:  # for fp64 inputs the fp64 sum is the oracle's own arithmetic, not the truth
+        assert err_gpu <= 2 * err_oracle + floor, (err_gpu, err_oracle)
+    # oracle vs HIP: the looser secondary check (both carry their own fp32 rounding)
+    loose = {np.dtype(np.float32): 2e-4, np.dtype(np.float16): 1e-2, np.dtype(np.float64): 1e-7}[np.dtype(dtype)]
+    assert_close(got["weights"], w, loose)
     if optimizer == "adagrad":
+        assert_close(got["state"], st64, 1e-5 if dtype != np.float64 else 1e-12, "HIP state vs fp64")
         assert_close(got["state"], st, 1e-3)
         assert_close(got["grad_psw"], ref["grad_psw"], TOL[np.dtype(dtype)])
+
+
+def _fp64_update(p, optimizer, lr, eps):
+    """The exact update in fp64 numpy (test_table_batched_embeddings.py:190-193, 296-318):
+    G[r] = sum over the occurrences of row r of (psw *) grad_output[b, t]; SGD w -= lr * G;
+    row-wise Adagrad state = sum_d G^2 (from zero), w -= lr / (sqrt(state) + eps) * G."""
+    T, B = p["T"], p["B"]
+    bag = np.repeat(np.arange(T * B), np.diff(p["offsets"]))
+    t, b = bag // B, bag % B
+    rows = p["table_offsets"][t].astype(np.int64) + p["indices"]
+    g = p["grad_output"].astype(np.float64)[b, t, :]
+    if p.get("per_sample_weights") is not None:
+        g = g * p["per_sample_weights"].astype(np.float64)[:, None]
+    G = np.zeros(p["weights"].shape, np.float64)
+    np.add.at(G, rows, g)
+    w = p["weights"].astype(np.float64)
+    lr = float(np.float32(lr))
+    if optimizer == "sgd":
+        return w - lr * G, None
+    state = (G * G).sum(axis=1)
+    mult = np.where(state > 0, lr / (np.sqrt(state) + float(np.float32(eps))), 0.0)
+    return w - mult[:, None] * G, state
 
 
 def test_two_backward_runs_are_bit_identical():
