@@ -1,6 +1,6 @@
 """Headline benchmark: table-batched embedding bags, forward + fused exact-SGD backward.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5] [--no-cpu] [--only]
 
 One step = one pass of the hot path over one batch of seeded synthetic input: the
 module's forward (pooled gather-sum) and its backward (linearize, radix sort, segments,
@@ -10,9 +10,11 @@ region.  Prints ONE JSON line.  Everything runs on one GPU.
 
 Default workload = configuration 3 (the shape the bandwidth target is quoted on):
 T=64 tables x 100k rows x D=128 fp32, B=4096 bags per table, L=20, Zipf(1.05) indices,
-exact SGD lr=0.01.  --config 2 times the forward alone on uniform indices; --config 4 the
-fp16 / weighted / exact row-wise Adagrad shape; --config 5 the DLRM-style shape whose tables
-live in pinned host memory behind the HBM row cache (indices re-drawn every step).
+exact SGD lr=0.01.  The default run then times configurations 2 (the forward alone on uniform
+indices) and 4 (the fp16 / weighted / exact row-wise Adagrad shape) the same way and adds them
+to the line as compact records under "other_configs" (--only leaves them out; --config 2 / 4
+run one of them as the main record).  --config 5 is the DLRM-style shape whose tables live in
+pinned host memory behind the HBM row cache (indices re-drawn every step).
 """
 import argparse
 import json
@@ -29,18 +31,43 @@ for _p in (ROOT, os.path.join(ROOT, "sparse-ads-baselines_amd")):
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
 
-# Bytes that crossed the L2 <-> memory-fabric boundary per launch, from two rocprofv3 --pmc runs of
-# this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
-# reads for a plain 1 GiB device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Keyed by (kernel, config).
-MEASURED_TRAFFIC = {
-    ("update_short", 3): int((1274937.7 * 2.0 + 1278141.8) * 1024),
-    ("update_chunks", 3): int((242588.5 * 2.0 + 8309.0) * 1024),
-    ("forward", 3): int((836296.1 * 2.0 + 131072.0) * 1024),
-    ("forward", 2): int((1227738.4 * 2.0 + 131072.0) * 1024),
-    ("update_short", 4): int((188383.6 * 2.0 + 188470.0) * 1024),
-    ("update_chunks", 4): int((72411.1 * 2.0 + 53625.9) * 1024),
-    ("forward", 4): int((84678.9 * 2.0 + 32768.0) * 1024),
-}
+HOST_LINK_PEAK = 63.0e9  # bytes/s per direction: PCIe 5.0 x16 (32 GT/s x 16 lanes x 128b/130b)
+
+PROFILE_STEMS = {2: "cfg2_forward", 3: "cfg3_fwd_bwd_sgd", 4: "cfg4_fwd_bwd_weighted_adagrad"}
+
+
+def measured_traffic(config, kernel):
+    """Bytes that crossed the L2 <-> memory-fabric boundary per launch of `kernel`, read from the
+    committed counter summary of this configuration (profiles/cfg<N>_*_pmc_traffic.txt: two
+    rocprofv3 --pmc runs of this script, FETCH_SIZE then WRITE_SIZE, KiB per dispatch).  Each
+    counter is scaled by what it reads for a plain device copy of known size in the same run
+    (the factors are parsed from the summary's calibration line).  Returns None when there is no
+    summary or no row for the kernel.  The figures describe the kernels as they were when the
+    summary was taken; `source` names the file so that a reader can check its date."""
+    import re
+
+    stem = PROFILE_STEMS.get(config)
+    path = os.path.join(ROOT, "profiles", "%s_pmc_traffic.txt" % stem) if stem else None
+    if not path or not os.path.exists(path):
+        return None
+    text = open(path).read()
+    factors = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
+    for counter in factors:
+        m = re.search(r"%s reads [0-9.]+ KiB \(factor ([0-9.]+)\)" % counter, text)
+        if m:
+            factors[counter] = float(m.group(1))
+    kib = {}
+    for line in text.splitlines():
+        if line.startswith("#") or "tbe::%s" % kernel not in line:
+            continue
+        m = re.search(r"(FETCH_SIZE|WRITE_SIZE)\s+(\d+)\s+([0-9.]+)", line)
+        if m and m.group(1) not in kib:
+            kib[m.group(1)] = float(m.group(3))
+    if set(kib) != set(factors):
+        return None
+    return {"bytes": int((kib["FETCH_SIZE"] * factors["FETCH_SIZE"] + kib["WRITE_SIZE"] * factors["WRITE_SIZE"]) * 1024),
+            "fetch_KiB": kib["FETCH_SIZE"], "write_KiB": kib["WRITE_SIZE"], "fetch_factor": factors["FETCH_SIZE"],
+            "write_factor": factors["WRITE_SIZE"], "source": os.path.relpath(path, ROOT)}
 
 
 def make_workload(config, seed=0):
@@ -172,11 +199,59 @@ def cpu_baseline(w, torch, tables=8, iters=3):
     opt = w["optimizer"] or "sgd"
     sec = torch_cpu_path.time_steps(cpu, (w["indices"][:hi], w["offsets"][:T * B + 1], B, go, opt, w["lr"],
                                           w["eps"], psw), warmup=1, iters=iters)
+    # the same algorithmic bytes as the GPU figure, for the sample's lookups, bags and distinct rows
+    keys = w["indices"][:hi].astype(np.int64) + np.repeat(np.arange(T, dtype=np.int64) * E,
+                                                          np.diff(w["offsets"][:T * B + 1:B]))
+    sample = dict(w, T=T, n=hi)
+    a_fwd, a_bwd, _ = algorithmic_bytes(sample, int(np.unique(keys).size))
     return {"value": T * B / sec, "unit": "bags/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": "first %d of %d tables of the same workload (%d bags/step), 1 warm-up + %d timed steps, "
                       "per-table torch.nn.EmbeddingBag(sparse=True) forward+backward + Python %s update, fp32"
                       % (T, w["T"], T * B, iters, opt),
-            "ms_per_step": sec * 1e3}
+            "ms_per_step": sec * 1e3, "GBps": (a_fwd + a_bwd) / sec / 1e9,
+            "algorithmic_bytes_per_step": a_fwd + a_bwd}
+
+
+def cpu_baseline_cached(w, torch, dev, bags_per_table=4096, iters=3):
+    """Configuration 5 on the reference's CPU path: the full-size tables (per-table
+    torch.nn.EmbeddingBag) on a bounded sample of the batch -- `bags_per_table` of the 65 536 bags of
+    every table, drawn by the same generator.  Two optimizers are timed: the test-suite's dense
+    `weight - weight.grad * lr`, which touches every row of every table each step, and a
+    coalesced index_add_ of the touched rows only."""
+    from oracle import torch_cpu_path
+
+    T, D = w["T"], w["D"]
+    sample = dict(w, B=bags_per_table)
+    indices, offsets = draw_cfg5_batch(torch, sample, 10 ** 6, dev)
+    indices, offsets = indices.cpu().numpy(), offsets.cpu().numpy()
+    go = np.random.RandomState(w["seed"] + 1).randn(bags_per_table, T, D).astype(np.float32)
+    torch.set_num_threads(os.cpu_count() or 1)
+    t0 = time.perf_counter()
+    cpu = torch_cpu_path.CpuTables(None, w["E"], D, fill=0.001)
+    setup_s = time.perf_counter() - t0
+    table_of = np.repeat(np.arange(T), np.diff(offsets[::bags_per_table]))
+    starts = np.concatenate([[0], np.cumsum(w["E"][:-1])]).astype(np.int64)
+    U = int(np.unique(starts[table_of] + indices).size)
+    sample["n"] = int(indices.size)
+    a_fwd, a_bwd, _ = algorithmic_bytes(sample, U)
+    args = (indices, offsets, bags_per_table, go, "sgd", w["lr"], 0.0, None)
+    out = {}
+    for update in ("dense", "index_add"):
+        sec = torch_cpu_path.time_steps(cpu, args, warmup=1, iters=iters, update=update)
+        out[update] = {"value": T * bags_per_table / sec, "ms_per_step": sec * 1e3,
+                       "GBps": (a_fwd + a_bwd) / sec / 1e9}
+    what = ("all %d full-size tables (%.1f GB), %d of the %d bags per table drawn by the same generator "
+            "(%d lookups, %d distinct rows per step), 1 warm-up + %d timed steps per optimizer variant, "
+            "per-table torch.nn.EmbeddingBag(sparse=True) forward+backward, fp32"
+            % (T, sum(w["E"]) * D * 4 / 1e9, bags_per_table, w["B"], indices.size, U, iters))
+    return {"value": out["dense"]["value"], "unit": "bags/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": what + "; value = the test-suite's dense SGD update (weight - weight.grad * lr over whole "
+                             "tables, test_table_batched_embeddings.py:193)",
+            "ms_per_step": out["dense"]["ms_per_step"], "GBps": out["dense"]["GBps"],
+            "algorithmic_bytes_per_step": a_fwd + a_bwd, "setup_seconds": setup_s,
+            "index_add_variant": dict(out["index_add"], unit="bags/s",
+                                      note="same sample; SGD applied to the rows of the coalesced sparse "
+                                           "gradient only (weight.index_add_)")}
 
 
 def run_cached(args, w):
@@ -202,7 +277,6 @@ def run_cached(args, w):
     gen = torch.Generator(device=dev).manual_seed(w["seed"])
     grad_output = torch.randn(B, T, D, device=dev, generator=gen)
     torch.cuda.synchronize()
-    stats = []
 
     def step(i):
         indices, offsets = batches[i]
@@ -216,52 +290,106 @@ def run_cached(args, w):
         step(i)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    sec = elapsed / args.steps
 
-    # a second, untimed pass over fresh batches collects per-step cache counters and kernel times
-    per_kernel = {}
-    lookups = 0
+    # Untimed replay of the same batches on an emptied cache: the cache's decisions depend on the
+    # keys only, so every step repeats the decisions of its timed twin.  It collects, per step, the
+    # cache counters (one host synchronisation each, which is why they are not read in the timed
+    # loop), the hit rate by lookup, and the kernel durations.
+    cache = module.row_cache
+    cache.invalidate()
+    slots = w["cache_slots"]
+    per_step, per_kernel = [], {}
     bytes_alg = 0
-    extra = [draw_cfg5_batch(torch, w, total + s, dev) for s in range(min(3, args.steps))]
     with tbe_native.profile() as prof:
-        for indices, offsets in extra:
-            module(indices, offsets).backward(grad_output)
-            st = module.row_cache.stats()
-            stats.append(st)
-            w["n"] = indices.numel()
-            a_fwd, a_bwd, _ = algorithmic_bytes(w, st["unique_rows"])
-            bytes_alg += a_fwd + a_bwd
-            lookups += indices.numel()
+        for i in range(total):
+            indices, offsets = batches[i]
+            out = module(indices, offsets)
+            st = cache.stats()
+            U = st["unique_rows"]
+            lay, ws = cache._plan_layout, cache._plan_ws
+            starts = ws[lay.segment_starts:lay.segment_starts + 4 * (U + 1)].view(torch.int32).long()
+            occurrences = starts[1:] - starts[:-1]
+            unique_slots = cache.unique_slots()
+            hit = (cache.evicted_keys() == -2) & (unique_slots >= 0) & (unique_slots < slots)
+            st["lookups"] = int(indices.numel())
+            st["lookups_hit"] = int(occurrences[hit].sum())
+            st["hit_rate_unique_rows"] = st["hits"] / max(U, 1)
+            st["hit_rate_lookups"] = st["lookups_hit"] / max(st["lookups"], 1)
+            out.backward(grad_output)
+            if i >= args.warmup:
+                per_step.append(st)
+                a_fwd, a_bwd, _ = algorithmic_bytes(dict(w, n=st["lookups"]), U)
+                bytes_alg += a_fwd + a_bwd
+    torch.cuda.synchronize()
+    replay_steps = total
     for name, ms in prof.launches:
         per_kernel.setdefault(name, []).append(ms)
-    kernels = {k: {"launches_per_step": len(v) / len(extra), "avg_us": 1e3 * sum(v) / len(v)}
+    kernels = {k: {"launches_per_step": len(v) / replay_steps, "avg_us": 1e3 * sum(v) / len(v)}
                for k, v in per_kernel.items()}
     row_bytes = D * 4
-    # inserted and staged rows are fetched once, evicted and staged rows written once; an uncached row is
-    # read per lookup in the forward (counted once here) and read + written in the backward
-    link_bytes = [(st["inserted"] + st["written_back"] + 2 * st["staged"] + 3 * st["uncached"]) * row_bytes
-                  for st in stats]
-    mean_lookups = sum(b[0].numel() for b in batches[args.warmup:]) / args.steps
-    sec = elapsed / args.steps
-    dominant = max(kernels, key=lambda k: kernels[k]["avg_us"] * kernels[k]["launches_per_step"])
+    # Rows over the host link per step.  In: inserted and staged rows are fetched once, an uncached row
+    # is read by the forward (once per lookup; counted once) and by the update.  Out: evicted and staged
+    # rows are written once, an uncached row is written by the update.
+    link_in = [(st["inserted"] + st["staged"] + 2 * st["uncached"]) * row_bytes for st in per_step]
+    link_out = [(st["written_back"] + st["staged"] + st["uncached"]) * row_bytes for st in per_step]
+    mean = lambda xs: sum(xs) / max(len(xs), 1)
+    steady = per_step[len(per_step) // 2:]
+    fill_us = kernels.get("cache_fill", {}).get("avg_us")
+    unstage_us = kernels.get("cache_unstage", {}).get("avg_us")
+    fill_in = mean([(st["inserted"] + st["staged"]) * row_bytes for st in per_step])
+    link_achieved = (mean(link_in) + mean(link_out)) / sec / 1e9
+    roofline = {
+        "bound": "host-link", "kernel": "cache_fill",
+        "achieved": fill_in / (fill_us * 1e-6) / 1e9 if fill_us else None,
+        "peak": HOST_LINK_PEAK / 1e9, "unit": "GB/s",
+        "frac": fill_in / (fill_us * 1e-6) / HOST_LINK_PEAK if fill_us else None,
+        "traffic": None,
+        "peak_is": "one direction of the host link (PCIe 5.0 x16, 32 GT/s x 16 lanes x 128b/130b = 63.0 GB/s); "
+                   "achieved = bytes the kernel fetches from the host table (inserted + staged rows x %d B) over "
+                   "its average duration, measured with HIP events on its stream in the replay" % row_bytes,
+        "avg_launch_us": fill_us,
+        "host_to_device_bytes_per_launch": fill_in,
+        "device_to_host_bytes_per_launch": mean([st["written_back"] * row_bytes for st in per_step]),
+        "whole_step": {"host_link_bytes_in": mean(link_in), "host_link_bytes_out": mean(link_out),
+                       "achieved_GBps_both_directions": link_achieved,
+                       "frac_of_one_direction_peak": link_achieved * 1e9 / HOST_LINK_PEAK,
+                       "note": "fill (in) and unstage (out) run one after the other around the update, so "
+                               "one direction is busy at a time: the step is bounded by in/peak + out/peak"},
+        "cache_unstage": {"avg_launch_us": unstage_us,
+                          "device_to_host_bytes_per_launch": mean([st["staged"] * row_bytes for st in per_step]),
+                          "achieved": (mean([st["staged"] * row_bytes for st in per_step]) / (unstage_us * 1e-6) / 1e9
+                                       if unstage_us else None)},
+    }
+    mean_lookups = mean([st["lookups"] for st in per_step])
     result = {
         "metric": "tbe_fwd_bwd_bags_per_sec", "value": T * B / sec, "unit": "bags/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": w["name"], "T": T, "D": D, "B": B, "mean_lookups_per_step": mean_lookups,
-                   "cache_slots": w["cache_slots"], "stage_slots": w["stage_slots"], "seed": w["seed"], "host_table_GB": sum(w["E"]) * row_bytes / 1e9,
-                   "setup_seconds": setup_s},
-        "effective_GBps": (bytes_alg / len(extra)) / sec / 1e9,
-        "effective_frac_of_hbm_peak": (bytes_alg / len(extra)) / sec / HBM_PEAK,
-        "cache": {"per_step": stats,
-                  "hit_rate_unique_rows": [st["hits"] / max(st["unique_rows"], 1) for st in stats],
-                  "host_link_bytes_per_step": link_bytes},
-        "roofline": {"bound": "host-link", "kernel": dominant, "achieved": None, "peak": None, "unit": "GB/s",
-                     "frac": None, "traffic": None,
-                     "note": "misses and uncached rows cross the host link; see cache.host_link_bytes_per_step"},
+                   "cache_slots": w["cache_slots"], "stage_slots": w["stage_slots"], "seed": w["seed"],
+                   "host_table_GB": sum(w["E"]) * row_bytes / 1e9, "setup_seconds": setup_s},
+        "effective_GBps": (bytes_alg / len(per_step)) / sec / 1e9,
+        "effective_frac_of_hbm_peak": (bytes_alg / len(per_step)) / sec / HBM_PEAK,
+        "cache": {
+            "hit_rate_unique_rows": {"mean": mean([st["hit_rate_unique_rows"] for st in per_step]),
+                                     "second_half_mean": mean([st["hit_rate_unique_rows"] for st in steady]),
+                                     "per_step": [round(st["hit_rate_unique_rows"], 4) for st in per_step]},
+            "hit_rate_lookups": {"mean": mean([st["hit_rate_lookups"] for st in per_step]),
+                                 "second_half_mean": mean([st["hit_rate_lookups"] for st in steady]),
+                                 "per_step": [round(st["hit_rate_lookups"], 4) for st in per_step]},
+            "first_timed_step": per_step[0], "last_step": per_step[-1],
+            "note": "counters of the timed steps, collected in an untimed replay of the same batches on an "
+                    "emptied cache (the cache's decisions are a function of the keys alone)"},
+        "roofline": roofline,
         "kernels": kernels,
-        "cpu_baseline": None,
     }
-    print(json.dumps(result))
+    # the pinned table goes before the CPU baseline builds its own copy of the tables
+    del module, cache, batches, out
+    import gc
+    gc.collect()
+    result["cpu_baseline"] = None if args.no_cpu else cpu_baseline_cached(w, torch, dev)
+    return result
 
 
 def parity_gates(torch, ext, tbe_native, w, module, indices, offsets, psw, grad_output, step):
@@ -329,35 +457,17 @@ def parity_gates(torch, ext, tbe_native, w, module, indices, offsets, psw, grad_
     return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=3)
-    ap.add_argument("--profile-steps", type=int, default=10)
-    ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a plain 1 GiB device-to-device copy 5 times, as the known-size "
-                         "reference for rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this path runs on one GPU; --gpus %d is not supported (run with --gpus 1)" % args.gpus,
-              file=sys.stderr)
-        sys.exit(2)
-
+def run_resident(args, config, steps, warmup, profile_steps, with_cpu):
+    """Configurations 2-4 (tables resident in HBM): the timed steps, per-kernel durations from HIP
+    events on the launch stream, the roofline of the dominant kernel and the parity gates."""
     import torch
 
     import table_batched_embeddings as ext
     import table_batched_embeddings_ops as ops
     import tbe_native
 
-    if not torch.cuda.is_available():
-        raise SystemExit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
-    w = make_workload(args.config)
-    if args.config == 5:
-        return run_cached(args, w)
+    w = make_workload(config)
     T, E, D, B = w["T"], w["E"], w["D"], w["B"]
     optimizer = {"sgd": ops.Optimizer.SGD, "adagrad": ops.Optimizer.EXACT_ROWWISE_ADAGRAD,
                  None: ops.Optimizer.SGD}[w["optimizer"]]
@@ -390,15 +500,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
+    ms_per_step = elapsed / steps * 1e3
     bags = T * B
 
     # unique rows of the batch, for the byte count (read back from the backward workspace)
@@ -427,33 +537,37 @@ def main():
 
     # per-kernel durations from HIP events recorded by the library on the launch stream
     per_kernel = {}
-    if args.profile_steps > 0:
+    if profile_steps > 0:
         with tbe_native.profile() as prof:
-            for _ in range(args.profile_steps):
+            for _ in range(profile_steps):
                 step()
         for name, ms in prof.launches:
             per_kernel.setdefault(name, []).append(ms)
-    kernels = {k: {"launches_per_step": len(v) / max(args.profile_steps, 1), "avg_us": 1e3 * sum(v) / len(v)}
+    kernels = {k: {"launches_per_step": len(v) / max(profile_steps, 1), "avg_us": 1e3 * sum(v) / len(v)}
                for k, v in per_kernel.items()}
     kernel_bytes = {"forward": a_fwd, "update_short": a_update_short, "update_chunks": a_update_chunks}
     roofline = None
     if kernels:
         dominant = max((k for k in kernels if k in kernel_bytes and kernel_bytes[k]),
                        key=lambda k: kernels[k]["avg_us"] * kernels[k]["launches_per_step"])
-        achieved = kernel_bytes[dominant] / (kernels[dominant]["avg_us"] * 1e-6) / 1e9
+        seconds = kernels[dominant]["avg_us"] * 1e-6
+        achieved = kernel_bytes[dominant] / seconds / 1e9
+        traffic = measured_traffic(config, dominant)
         roofline = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK / 1e9,
                     "unit": "GB/s", "frac": achieved / (HBM_PEAK / 1e9),
-                    "traffic": MEASURED_TRAFFIC.get((dominant, args.config)),
+                    "traffic": traffic["bytes"] if traffic else None,
+                    "traffic_source": traffic,
+                    "counter_frac_of_peak": traffic["bytes"] / seconds / HBM_PEAK if traffic else None,
                     "algorithmic_bytes_per_launch": kernel_bytes[dominant],
                     "avg_launch_us": kernels[dominant]["avg_us"]}
 
     result = {
         "metric": "tbe_fwd_bwd_bags_per_sec" if w["optimizer"] else "tbe_fwd_bags_per_sec",
-        "value": bags / (elapsed / args.steps),
+        "value": bags / (elapsed / steps),
         "unit": "bags/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -462,8 +576,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": w["name"], "T": T, "rows_per_table": E, "D": D, "B": B, "lookups": w["n"],
                    "unique_rows": U, "seed": w["seed"]},
-        "effective_GBps": (a_fwd + a_bwd) / (elapsed / args.steps) / 1e9,
-        "effective_frac_of_hbm_peak": (a_fwd + a_bwd) / (elapsed / args.steps) / HBM_PEAK,
+        "effective_GBps": (a_fwd + a_bwd) / (elapsed / steps) / 1e9,
+        "effective_frac_of_hbm_peak": (a_fwd + a_bwd) / (elapsed / steps) / HBM_PEAK,
         "algorithmic_bytes": {"forward": a_fwd, "backward": a_bwd, "update_short": a_update_short,
                               "update_chunks": a_update_chunks,
                               "short_segments": short_share},
@@ -471,10 +585,62 @@ def main():
         "kernels": kernels,
     }
     result["parity"] = parity_gates(torch, ext, tbe_native, w, module, indices, offsets, psw, grad_output, step)
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(w, torch)
-    else:
-        result["cpu_baseline"] = None
+    result["cpu_baseline"] = cpu_baseline(w, torch) if with_cpu else None
+    return result
+
+
+def compact(result):
+    """The driver-timed essentials of a secondary configuration."""
+    r = result["roofline"] or {}
+    return {"workload": result["config"]["workload"], "metric": result["metric"], "value": result["value"],
+            "unit": result["unit"], "steps": result["steps"], "warmup": result["warmup"],
+            "ms_per_step": result["ms_per_step"], "dtype": result["dtype"],
+            "effective_GBps": result["effective_GBps"],
+            "effective_frac_of_hbm_peak": result["effective_frac_of_hbm_peak"],
+            "roofline": {k: r.get(k) for k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "traffic",
+                                               "counter_frac_of_peak", "avg_launch_us")},
+            "kernel_us_per_step": {k: round(v["avg_us"] * v["launches_per_step"], 2)
+                                   for k, v in result["kernels"].items()},
+            "parity": result["parity"]}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=3)
+    ap.add_argument("--profile-steps", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only", action="store_true",
+                    help="with the default configuration: leave out the compact records of configurations 2 and 4")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device-to-device copy 5 times, as the known-size "
+                         "reference for rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on one GPU; --gpus %d is not supported (run with --gpus 1)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    if args.config == 5:
+        print(json.dumps(run_cached(args, make_workload(5))))
+        return
+    result = run_resident(args, args.config, args.steps, args.warmup, args.profile_steps, not args.no_cpu)
+    if args.config == 3 and not args.only and not args.calibrate_copy:
+        # the other HBM-resident configurations, timed the same way in the same run (no CPU leg)
+        import gc
+        others = {}
+        for other in (2, 4):
+            gc.collect()
+            torch.cuda.empty_cache()
+            others["cfg%d" % other] = compact(run_resident(args, other, args.steps, args.warmup,
+                                                           min(args.profile_steps, 5), False))
+        result["other_configs"] = others
     print(json.dumps(result))
 
 

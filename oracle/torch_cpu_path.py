@@ -14,20 +14,29 @@ import torch
 
 
 class CpuTables:
-    def __init__(self, weights, rows, D):
-        """weights: float32 numpy [sum(rows), D]."""
+    def __init__(self, weights, rows, D, fill=None):
+        """weights: float32 numpy [sum(rows), D]; or None, then every table is filled with the
+        constant `fill` (timing runs on tables too large to draw and copy: values do not change
+        the work)."""
         self.bags = []
         self.states = []
         r0 = 0
         for E in rows:
-            bag = torch.nn.EmbeddingBag(E, D, mode="sum", sparse=True)
-            bag.weight.data.copy_(torch.from_numpy(np.ascontiguousarray(weights[r0:r0 + E])).float())
+            if weights is None:
+                init = torch.full((E, D), float(fill))
+            else:
+                init = torch.from_numpy(np.ascontiguousarray(weights[r0:r0 + E])).float()
+            bag = torch.nn.EmbeddingBag(E, D, mode="sum", sparse=True, _weight=init)
             self.bags.append(bag)
             self.states.append(torch.zeros(E))
             r0 += E
 
-    def step(self, indices, offsets, B, grad_output, optimizer, lr, eps=0.0, per_sample_weights=None):
-        """One forward + backward + optimizer pass over all tables; returns output [B, T, D]."""
+    def step(self, indices, offsets, B, grad_output, optimizer, lr, eps=0.0, per_sample_weights=None,
+             update="dense"):
+        """One forward + backward + optimizer pass over all tables; returns output [B, T, D].
+        update="dense" is the optimizer as the reference's test writes it (it touches every row of
+        every table); update="index_add" applies the same SGD step to the rows of the coalesced
+        sparse gradient only."""
         outs = []
         for t, bag in enumerate(self.bags):
             lo, hi = int(offsets[t * B]), int(offsets[(t + 1) * B])
@@ -41,9 +50,13 @@ class CpuTables:
             out.backward(torch.from_numpy(np.ascontiguousarray(grad_output[:, t, :])).float())
             grad = bag.weight.grad
             with torch.no_grad():
-                if optimizer == "sgd":
+                if optimizer == "sgd" and update == "index_add":
+                    g = grad.coalesce()
+                    bag.weight.data.index_add_(0, g.indices()[0], g.values(), alpha=-lr)
+                elif optimizer == "sgd":
                     bag.weight.data = bag.weight - grad * lr
                 else:
+                    assert update == "dense"
                     dense = grad.to_dense()
                     self.states[t] += dense.pow(2).sum(dim=1)
                     bag.weight.data = torch.addcdiv(bag.weight, dense, (self.states[t].sqrt() + eps).view(-1, 1),
@@ -52,10 +65,10 @@ class CpuTables:
         return torch.stack(outs, dim=1)
 
 
-def time_steps(tables, step_args, warmup=1, iters=3):
+def time_steps(tables, step_args, warmup=1, iters=3, update="dense"):
     for _ in range(warmup):
-        tables.step(*step_args)
+        tables.step(*step_args, update=update)
     t0 = time.perf_counter()
     for _ in range(iters):
-        tables.step(*step_args)
+        tables.step(*step_args, update=update)
     return (time.perf_counter() - t0) / iters
