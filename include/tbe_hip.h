@@ -42,7 +42,11 @@ extern "C" {
 enum { TBE_DTYPE_F32 = 0, TBE_DTYPE_F16 = 1, TBE_DTYPE_F64 = 2 };
 
 /* optimizer selector of the entry points that serve several optimizers */
-enum { TBE_OPT_SGD = 0, TBE_OPT_ROWWISE_ADAGRAD = 1 };
+enum {
+  TBE_OPT_SGD = 0,
+  TBE_OPT_ROWWISE_ADAGRAD = 1,        /* exact: one update per distinct row with its summed gradient */
+  TBE_OPT_APPROX_ROWWISE_ADAGRAD = 2  /* per lookup, see tbe_backward_approx_adagrad (tbe_backward_mixed only) */
+};
 
 enum {
   TBE_OK = 0,
@@ -188,6 +192,35 @@ TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, i
                                void *grad_per_sample_weights,
                                void *workspace, uint64_t workspace_bytes, void *stream);
 
+/* Approximate row-wise Adagrad: the per-lookup update of
+ * batched_embedding_backward_adagrad_approx_cuda (table_batched_embeddings_cuda.cu:706-793, kernel
+ * :648-704, functors :437-553; "backward_approx_adagrad" in table_batched_embeddings.cpp:60).
+ * For every lookup p of bag (t, b), with g = grad_output[b][t][:] and r = its row:
+ *   wss = sum_d g_d^2 (* psw[p]^2);  state[r] += wss
+ *   mult = (psw[p] *) lr / (sqrt(state[r]) + eps)           (the state AFTER this lookup's addition)
+ *   grad_per_sample_weights[p] = <weights[r], g>            (the row as it is at that moment)
+ *   weights[r] -= mult * g                                  (stored in the weights' type each time)
+ * The reference runs all bags at once with plain loads and stores, so its result is only defined
+ * when no row occurs twice in the batch (all its test draws, test_table_batched_embeddings.py:244).
+ * Here the lookups of a row are applied one at a time in ascending position (table-major bag
+ * order, then the order inside the bag): the reference's arithmetic executed serially.  The two
+ * agree whenever the reference's result is defined; when rows repeat this library returns the
+ * serial result, deterministically.  With stochastic_rounding (fp16 only) the k-th update of a
+ * row within the call draws its bits with the Philox key seed ^ (k * 0x9E3779B97F4A7C15): k = 0
+ * is the stream of tbe_backward_exact_adagrad_stochastic.  Arguments as in
+ * tbe_backward_exact_adagrad_stochastic.
+ */
+TBE_API int tbe_backward_approx_adagrad(const void *grad_output, void *weights, int32_t dtype,
+                                        int64_t total_rows, int64_t max_table_rows, int32_t D,
+                                        const int32_t *table_offsets, int32_t T,
+                                        const int32_t *indices, int64_t num_indices,
+                                        const int32_t *offsets, int32_t B,
+                                        const void *per_sample_weights, void *optimizer_state,
+                                        float learning_rate, float eps,
+                                        void *grad_per_sample_weights,
+                                        int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
+                                        void *workspace, uint64_t workspace_bytes, void *stream);
+
 /* The backward in two calls, so that the integer half can overlap other work.
  * tbe_plan_batch runs the stages that depend on the indices only -- gradient rows, sort, run
  * boundaries (table_batched_embeddings_cuda.cu:1618-1655 and the head test :1523-1539) -- and
@@ -281,8 +314,9 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
  * tbe_forward_mixed replaces batched_embedding_forward_mixed_D_cuda
  * (table_batched_embeddings_cuda.cu:945-1004, "forward_mixed_D" in table_batched_embeddings.cpp:66);
  * tbe_backward_mixed replaces batched_embedding_backward_adagrad_exact_mixed_D_cuda
- * (:1350-1469, "backward_exact_adagrad_mixed_D", .cpp:64), serves the approximate variant
- * (.cpp:63) and adds exact SGD; per-sample weights as in tbe_backward_exact_adagrad;
+ * (:1350-1469, "backward_exact_adagrad_mixed_D", .cpp:64), with TBE_OPT_APPROX_ROWWISE_ADAGRAD
+ * batched_embedding_backward_adagrad_approx_mixed_D_cuda (:1076-1163, .cpp:63; semantics of
+ * tbe_backward_approx_adagrad), and adds exact SGD; per-sample weights as in tbe_backward_exact_adagrad;
  * stochastic_rounding / seed / offset as in tbe_backward_exact_adagrad_stochastic;
  * max_table_rows as in tbe_backward_sgd (0 = unknown).  The
  * workspace is a backward workspace sized with tbe_backward_workspace_layout(N, 4, dtype, T).

@@ -391,6 +391,104 @@ int oracle_backward(int optimizer, const void *grad_output, void *weights, int d
   return 0;
 }
 
+/* ---------------------------------------------- approximate row-wise Adagrad
+ * batched_embedding_backward_adagrad_approx_kernel_1 (tbe.cu:648-704) and its mixed-D twin
+ * (tbe.cu:1006-1074) with AdaGradFunctor / WeightedAdaGradFunctor (tbe.cu:437-471, 483-553).
+ * Per bag (t, b): gss = sum_d grad_output[b][t][d]^2; then per lookup p of the bag
+ *   wss    = gss (* psw[p] * psw[p])
+ *   old    = state[row]; state[row] = old + wss                       (update_momentum)
+ *   mult   = (psw[p] *) lr * (1.0 / (sqrt(old + wss) + eps))
+ *   grad_psw[p] = <weights[row], grad_output[b][t]>                   (weighted: the row as it is now)
+ *   weights[row] -= grad_output[b][t] * mult, stored in the weights' type  (update_weight)
+ * The reference runs the bags concurrently with plain loads and stores, so its result is only
+ * defined when no row occurs twice in a batch (the only case its test draws,
+ * test_table_batched_embeddings.py:244).  This restatement is the same kernel run ONE LOOKUP AT A
+ * TIME in position order (table-major bags, then the bag's lookups): the outcome every
+ * interleaving of the reference agrees with when rows do not repeat, and the serial one when
+ * they do.  fp16 weights are rounded after every lookup, as update_weight's store does; with
+ * stochastic rounding the k-th update of a row in a call draws its bits with the Philox key
+ * seed ^ (k * 0x9E3779B97F4A7C15) (k = 0 is the exact update's stream).
+ * Uniform tables: D > 0, table_offsets = first ROW of each table [T], mixed_* NULL.
+ * Mixed-D tables: D = 0, mixed_table_offsets = first ELEMENT [T+1], table_dim_offsets = first row id
+ * [T+1], dim_offsets = first output column [T+1], grad_output [B][total_D].
+ */
+int oracle_backward_approx(const void *grad_output, void *weights, int dtype, int64_t total_rows,
+                           int32_t D, const int32_t *table_offsets,
+                           const int64_t *mixed_table_offsets, const int32_t *table_dim_offsets,
+                           const int32_t *dim_offsets, int32_t total_D, int32_t T,
+                           const int32_t *indices, const int32_t *offsets, int32_t B, const void *psw,
+                           void *optimizer_state, float lr, float eps, void *grad_psw,
+                           int32_t stochastic_rounding, uint64_t sr_seed, uint64_t sr_offset) {
+  const int mixed = D == 0;
+  int32_t *times = (int32_t *)calloc((size_t)(total_rows > 0 ? total_rows : 1), 4);
+  int32_t max_D = D;
+  if (mixed)
+    for (int32_t t = 0; t < T; ++t)
+      if (dim_offsets[t + 1] - dim_offsets[t] > max_D) max_D = dim_offsets[t + 1] - dim_offsets[t];
+  float *tmp = (float *)malloc((size_t)(max_D > 0 ? max_D : 1) * 4);
+  for (int32_t t = 0; t < T; ++t) {
+    const int32_t Dt = mixed ? dim_offsets[t + 1] - dim_offsets[t] : D;
+    for (int32_t b = 0; b < B; ++b) {
+      const int64_t g0 = mixed ? (int64_t)b * total_D + dim_offsets[t] : ((int64_t)b * T + t) * D;
+      double gss_d = 0;
+      float gss_f = 0;
+      for (int32_t d = 0; d < Dt; ++d) {
+        if (dtype == F64) { const double g = ((const double *)grad_output)[g0 + d]; gss_d += g * g; }
+        else { const float g = load_f(grad_output, dtype, g0 + d); gss_f += g * g; }
+      }
+      for (int32_t p = offsets[t * B + b]; p < offsets[t * B + b + 1]; ++p) {
+        const int64_t row = mixed ? (int64_t)table_dim_offsets[t] + indices[p] : (int64_t)table_offsets[t] + indices[p];
+        const int64_t w0 = mixed ? mixed_table_offsets[t] + (int64_t)indices[p] * Dt : row * D;
+        const int32_t k = times[row]++;
+        if (dtype == F64) {
+          const double pw = psw ? ((const double *)psw)[p] : 1.0;
+          const double wss = psw ? gss_d * pw * pw : gss_d;
+          double *st = (double *)optimizer_state + row;
+          const double old = *st;
+          *st = old + wss;
+          const double mult = psw ? pw * lr * (1.0 / (sqrt(old + wss) + eps)) : lr * (1.0 / (sqrt(old + wss) + eps));
+          double *w = (double *)weights + w0;
+          const double *g = (const double *)grad_output + g0;
+          if (psw) {
+            double dot = 0;
+            for (int32_t d = 0; d < Dt; ++d) dot += w[d] * g[d];
+            ((double *)grad_psw)[p] = dot;
+          }
+          for (int32_t d = 0; d < Dt; ++d) w[d] -= g[d] * mult;
+        } else {
+          const float pw = psw ? load_f(psw, dtype, p) : 1.0f;
+          const float wss = psw ? gss_f * pw * pw : gss_f;
+          float *st = (float *)optimizer_state + row;
+          const float old = *st;
+          *st = old + wss;
+          const float mult = psw ? (float)(pw * lr * (1.0 / (sqrtf(old + wss) + eps)))
+                                 : (float)(lr * (1.0 / (sqrtf(old + wss) + eps)));
+          if (psw) {
+            float dot = 0;
+            for (int32_t d = 0; d < Dt; ++d) dot += load_f(weights, dtype, w0 + d) * load_f(grad_output, dtype, g0 + d);
+            store_f(grad_psw, dtype, p, dot);
+          }
+          if (stochastic_rounding && dtype == F16) {
+            for (int32_t d = 0; d < Dt; ++d)
+              tmp[d] = load_f(weights, dtype, w0 + d) - load_f(grad_output, dtype, g0 + d) * mult;
+            store_row_stochastic((uint16_t *)weights + w0, tmp, Dt, w0,
+                                 sr_seed ^ ((uint64_t)k * 0x9E3779B97F4A7C15ull), sr_offset);
+          } else {
+            for (int32_t d = 0; d < Dt; ++d) {
+              float w = load_f(weights, dtype, w0 + d);
+              w -= load_f(grad_output, dtype, g0 + d) * mult;
+              store_f(weights, dtype, w0 + d, w);
+            }
+          }
+        }
+      }
+    }
+  }
+  free(times);
+  free(tmp);
+  return 0;
+}
+
 /* --------------------------------------------------------- construct_offsets
  * construct_offsets_kernel (tbe.cu:1165-1188): out[0] = 0 (at::zeros, :1201),
  * out[1 + t*B + b] = next start (or table total for the last bag) - start.

@@ -123,6 +123,62 @@ def backward(optimizer, grad_output, weights, table_offsets, indices, offsets, l
     return {"keys_sorted": ks, "positions_sorted": ps, "segment_starts": ss[: U.value + 1].copy(), "grad_psw": gpsw}
 
 
+def backward_approx(grad_output, weights, table_offsets, indices, offsets, lr, eps, optimizer_state,
+                    per_sample_weights=None, stochastic_rounding=None):
+    """Approximate row-wise Adagrad, one lookup at a time in position order (oracle_backward_approx):
+    in place on `weights` [rows, D] and `optimizer_state`; returns grad_psw or None."""
+    assert weights.flags["C_CONTIGUOUS"] and weights.ndim == 2 and weights.dtype in _CODES
+    code = _CODES[weights.dtype]
+    grad_output = np.ascontiguousarray(grad_output, dtype=weights.dtype)
+    table_offsets, indices, offsets = _i32(table_offsets), _i32(indices), _i32(offsets)
+    T = table_offsets.size
+    B = (offsets.size - 1) // T
+    D = weights.shape[1]
+    assert grad_output.shape == (B, T, D)
+    want = np.float64 if weights.dtype == np.float64 else np.float32
+    assert optimizer_state.dtype == want and optimizer_state.flags["C_CONTIGUOUS"]
+    psw = gpsw = None
+    if per_sample_weights is not None:
+        psw = np.ascontiguousarray(per_sample_weights, dtype=weights.dtype)
+        gpsw = np.zeros(indices.size, dtype=weights.dtype)
+    sr = stochastic_rounding
+    lib().oracle_backward_approx(_p(grad_output), _p(weights), ctypes.c_int(code), ctypes.c_int64(weights.shape[0]),
+                                 ctypes.c_int32(D), _p(table_offsets), None, None, None, ctypes.c_int32(0),
+                                 ctypes.c_int32(T), _p(indices), _p(offsets), ctypes.c_int32(B), _p(psw),
+                                 _p(optimizer_state), ctypes.c_float(lr), ctypes.c_float(eps), _p(gpsw),
+                                 ctypes.c_int32(0 if sr is None else 1), ctypes.c_uint64(0 if sr is None else sr[0]),
+                                 ctypes.c_uint64(0 if sr is None else sr[1]))
+    return gpsw
+
+
+def backward_approx_mixed(grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, indices, offsets, lr,
+                          eps, optimizer_state, per_sample_weights=None, stochastic_rounding=None):
+    """The same for tables with per-table dimension (flat 1-D weights, grad_output [B, total_D])."""
+    assert weights.flags["C_CONTIGUOUS"] and weights.ndim == 1
+    code = _CODES[weights.dtype]
+    grad_output = np.ascontiguousarray(grad_output, dtype=weights.dtype)
+    table_offsets = np.ascontiguousarray(table_offsets, dtype=np.int64)
+    table_dim_offsets, dim_offsets = _i32(table_dim_offsets), _i32(dim_offsets)
+    indices, offsets = _i32(indices), _i32(offsets)
+    T = table_offsets.size - 1
+    B = (offsets.size - 1) // T
+    total_D = int(dim_offsets[-1])
+    assert grad_output.shape == (B, total_D)
+    psw = gpsw = None
+    if per_sample_weights is not None:
+        psw = np.ascontiguousarray(per_sample_weights, dtype=weights.dtype)
+        gpsw = np.zeros(indices.size, dtype=weights.dtype)
+    sr = stochastic_rounding
+    lib().oracle_backward_approx(_p(grad_output), _p(weights), ctypes.c_int(code),
+                                 ctypes.c_int64(int(table_dim_offsets[-1])), ctypes.c_int32(0), None,
+                                 _p(table_offsets), _p(table_dim_offsets), _p(dim_offsets), ctypes.c_int32(total_D),
+                                 ctypes.c_int32(T), _p(indices), _p(offsets), ctypes.c_int32(B), _p(psw),
+                                 _p(optimizer_state), ctypes.c_float(lr), ctypes.c_float(eps), _p(gpsw),
+                                 ctypes.c_int32(0 if sr is None else 1), ctypes.c_uint64(0 if sr is None else sr[0]),
+                                 ctypes.c_uint64(0 if sr is None else sr[1]))
+    return gpsw
+
+
 def construct_offsets(batch_offsets_per_table, total_indices_per_table):
     per_table = _i32(batch_offsets_per_table)
     totals = _i32(total_indices_per_table)

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libtbe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = ["tbe_api.hip", "tbe_forward.hip", "tbe_sort.hip", "tbe_update.hip", "tbe_backward.hip",
-           "tbe_cache.hip", "tbe_mixed.hip"]
+           "tbe_cache.hip", "tbe_mixed.hip", "tbe_approx.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -185,13 +185,14 @@ __device__ __forceinline__ uint32_t floats_to_half2_stochastic(float lo, float h
   return static_cast<uint32_t>(__half_as_ushort(a)) | (static_cast<uint32_t>(__half_as_ushort(b)) << 16);
 }
 
-// Stores VEC accumulator values at p.  For fp16 with stochastic rounding enabled, element e of
-// the table (e = row * D + column, a multiple of 4) takes word (e % 4) of
-// Philox(counter = {e / 4, offset}, key = seed), so the bits depend on the element and the
-// call, not on the launch geometry.
-template <typename T, int VEC, bool STREAMING>
-__device__ __forceinline__ void store_row(T *p, const RowVec<T, VEC> &v, const StochasticRounding &sr,
-                                          int64_t element) {
+// VEC accumulator values packed into the stored type: round to nearest even, or, for fp16 with
+// stochastic rounding enabled, element e of the table (e = row * D + column, a multiple of 4)
+// takes word (e % 4) of Philox(counter = {e / 4, offset}, key = seed), so the bits depend on the
+// element and the call, not on the launch geometry.
+template <typename T, int VEC>
+__device__ __forceinline__ typename RowVec<T, VEC>::R pack_rounded(const RowVec<T, VEC> &v,
+                                                                   const StochasticRounding &sr,
+                                                                   int64_t element) {
   if constexpr (sizeof(T) == 2) {
     if (sr.enabled) {
       uint32_t words[VEC / 2];
@@ -207,7 +208,19 @@ __device__ __forceinline__ void store_row(T *p, const RowVec<T, VEC> &v, const S
       }
       typename RowVec<T, VEC>::R raw;
       __builtin_memcpy(&raw, words, sizeof(raw));
-      *reinterpret_cast<typename RowVec<T, VEC>::R *>(p) = raw;
+      return raw;
+    }
+  }
+  return v.pack();
+}
+
+// Stores VEC accumulator values at p, rounded as pack_rounded does.
+template <typename T, int VEC, bool STREAMING>
+__device__ __forceinline__ void store_row(T *p, const RowVec<T, VEC> &v, const StochasticRounding &sr,
+                                          int64_t element) {
+  if constexpr (sizeof(T) == 2) {
+    if (sr.enabled) {
+      *reinterpret_cast<typename RowVec<T, VEC>::R *>(p) = pack_rounded<T, VEC>(v, sr, element);
       return;
     }
   }

@@ -917,8 +917,9 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   a.lr = learning_rate;
   a.eps = eps;
   a.sr = StochasticRounding{seed, offset, (stochastic_rounding && dtype == TBE_DTYPE_F16) ? 1 : 0};
-  TBE_REQUIRE(optimizer == TBE_OPT_SGD || optimizer == TBE_OPT_ROWWISE_ADAGRAD, "%s: bad optimizer %d", name,
-              optimizer);
+  TBE_REQUIRE(optimizer == TBE_OPT_SGD || optimizer == TBE_OPT_ROWWISE_ADAGRAD ||
+                  optimizer == TBE_OPT_APPROX_ROWWISE_ADAGRAD,
+              "%s: bad optimizer %d", name, optimizer);
   a.optimizer = optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad;
   if (int rc = validate_mixed(name, a)) return rc;
   TBE_REQUIRE(grad_output && table_dim_offsets, "%s: null pointer argument", name);
@@ -950,6 +951,11 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   rc = find_segments(i32(l.keys_sorted), num_indices, i32(l.segment_starts), i32(l.num_unique), nullptr,
                      ws + l.segment_scratch, s, /*clear_queue_counters=*/true);
   if (rc) return rc;
+  if (optimizer == TBE_OPT_APPROX_ROWWISE_ADAGRAD)
+    return approx_update(grad_output, weights, optimizer_state, per_sample_weights, grad_per_sample_weights,
+                         dtype, dtype == TBE_DTYPE_F16 ? a.vec : (dtype == TBE_DTYPE_F32 ? 4 : 2), 0, num_indices,
+                         learning_rate, eps, table_offsets, table_dim_offsets, dim_offsets, total_D, T, a.sr, l,
+                         workspace, s);
   switch (dtype) {
     case TBE_DTYPE_F32: launch_update_mixed_variant<float, 4>(a, l, ws, s); break;
     case TBE_DTYPE_F16:

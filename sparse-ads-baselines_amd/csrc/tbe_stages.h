@@ -91,6 +91,15 @@ int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int3
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
                int64_t total_rows, int64_t max_table_rows, hipStream_t stream);
 
+// The approximate row-wise Adagrad update (one lookup at a time per row, in position order) on a
+// workspace that holds the batch's plan.  Uniform tables: D > 0 and the mixed_* pointers null;
+// mixed-D tables: D = 0.
+int approx_update(const void *grad_output, void *weights, void *state, const void *psw, void *grad_psw,
+                  int32_t dtype, int32_t fp16_vector_width, int32_t D, int64_t n, float lr, float eps,
+                  const int64_t *mixed_table_offsets, const int32_t *table_dim_offsets,
+                  const int32_t *dim_offsets, int32_t total_D, int32_t T, StochasticRounding sr,
+                  const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream);
+
 // Copies the rows that tbe_cache_prepare staged for this step back to the backing table.
 int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int32_t *keys_sorted,
                   const int32_t *segment_starts, const int32_t *counters,

@@ -246,15 +246,49 @@ def backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets
     return grad_indice_weights
 
 
+def _check_adagrad_args(grad_output, weights, table_offsets, indices, offsets, indice_weights, optimizer_state,
+                        BT_block_size):
+    T, B = _check_common(weights, table_offsets, indices, offsets)
+    _require(BT_block_size > 0, "BT_block_size must be positive")
+    grad_output = _check_grad(grad_output, weights, T, B)
+    state_dtype = torch.float64 if weights.dtype == torch.float64 else torch.float32
+    _require(optimizer_state.dtype == state_dtype, "optimizer_state must be %s" % state_dtype)
+    _require(optimizer_state.is_contiguous() and optimizer_state.numel() == weights.size(0),
+             "optimizer_state must be contiguous with one entry per row")
+    _require(optimizer_state.device == weights.device, "optimizer_state must live on the weights' device")
+    grad_indice_weights = None
+    if indice_weights is not None:
+        _require(indice_weights.dtype == weights.dtype, "indice_weights must have the weights' dtype")
+        _require(indice_weights.is_contiguous() and indice_weights.numel() == indices.numel(),
+                 "indice_weights must be contiguous with one entry per index")
+        grad_indice_weights = torch.empty(indices.shape, dtype=grad_output.dtype, device=weights.device)
+    return T, B, grad_output, grad_indice_weights
+
+
 def backward_approx_adagrad(grad_output, weights, table_offsets, indices, offsets, indice_weights,
                             optimizer_state, learning_rate, eps, L_max, stochastic_rounding,
                             BT_block_size):
-    """Signature of batched_embedding_backward_adagrad_approx_cuda
-    (table_batched_embeddings.cpp:17-21).  Served by the exact row-wise update, which coincides
-    with the approximate one whenever no row repeats across bags -- the only case the
-    reference tests (test_table_batched_embeddings.py:244)."""
-    return backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets, indice_weights,
-                                  optimizer_state, learning_rate, eps, stochastic_rounding, BT_block_size)
+    """batched_embedding_backward_adagrad_approx_cuda (table_batched_embeddings_cuda.cu:706-793):
+    every lookup adds its bag's ||grad||^2 (times its squared weight) to the row's state and
+    moves the row by its own multiplier.  The lookups of a row are applied one at a time in
+    position order, so the result equals the reference's wherever that is defined (no row twice
+    in the batch) and is the serial, reproducible one where the reference races.  L_max (the
+    reference's shared-memory bound on the bag length, :738) does not exist here."""
+    T, B, grad_output, grad_indice_weights = _check_adagrad_args(
+        grad_output, weights, table_offsets, indices, offsets, indice_weights, optimizer_state, BT_block_size)
+    D = weights.size(1)
+    code = _DTYPE_CODES[weights.dtype]
+    layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
+    ws = _workspace(weights.device, layout.total_bytes)
+    stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
+    seed, offset = _rounding_stream(weights.device) if stochastic else (0, 0)
+    with torch.cuda.device(weights.device):
+        _native.check(_native.load().tbe_backward_approx_adagrad(
+            _ptr(grad_output), _ptr(weights), code, weights.size(0), max_table_rows(table_offsets, weights.size(0)),
+            D, _ptr(table_offsets), T, _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights),
+            _ptr(optimizer_state), float(learning_rate), float(eps), _ptr(grad_indice_weights), int(stochastic),
+            seed, offset, _ptr(ws), ws.numel(), _stream(weights.device)))
+    return grad_indice_weights
 
 
 def _check_mixed(weights, table_offsets, dim_offsets, indices, offsets):
@@ -362,10 +396,11 @@ def backward_exact_adagrad_mixed_D(grad_output, weights, table_offsets, table_di
 def backward_approx_adagrad_mixed_D(grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, total_D,
                                     indices, offsets, indice_weights, optimizer_state, learning_rate, eps, L_max,
                                     stochastic_rounding, BT_block_size):
-    """Signature of batched_embedding_backward_adagrad_approx_mixed_D_cuda
-    (table_batched_embeddings.cpp:38-43), served by the exact row-wise update."""
+    """batched_embedding_backward_adagrad_approx_mixed_D_cuda (table_batched_embeddings_cuda.cu:1076-1163,
+    table_batched_embeddings.cpp:38-43): the per-lookup update of backward_approx_adagrad for
+    tables with per-table dimension."""
     _require(BT_block_size > 0, "BT_block_size must be positive")
-    return _backward_mixed(_native.OPT_ROWWISE_ADAGRAD, grad_output, weights, table_offsets, table_dim_offsets,
+    return _backward_mixed(_native.OPT_APPROX_ROWWISE_ADAGRAD, grad_output, weights, table_offsets, table_dim_offsets,
                            dim_offsets, total_D, indices, offsets, indice_weights, optimizer_state, learning_rate,
                            eps, stochastic_rounding)
 

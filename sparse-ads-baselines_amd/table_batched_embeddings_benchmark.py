@@ -106,16 +106,34 @@ def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
         sgd = lambda: table_batched_embeddings.backward_sgd_mixed_D(
             go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets,
             cc.optimizer_state, lr)
-        ada = lambda: table_batched_embeddings.backward_exact_adagrad_mixed_D(
-            go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets, None,
-            cc.optimizer_state, lr, eps, False, 1)
     else:
         sgd = lambda: table_batched_embeddings.backward_sgd(go, w, cc.table_offsets, indices, offsets, lr, L, 1,
                                                             False)
-        ada = lambda: table_batched_embeddings.backward_exact_adagrad(
-            go, w, cc.table_offsets, indices, offsets, None, cc.optimizer_state, lr, eps, False, 1)
     report("Backward-SGD-EXACT", time_calls(iters, sgd), 2 * fwd_bytes, shape)
-    report("Backward-ADAGRAD-nonstochastic-EXACT", time_calls(iters, ada), 2 * fwd_bytes, shape)
+
+    # the reference's rows (table_batched_embeddings_benchmark.py:266-357): approximate and exact
+    # row-wise Adagrad, with stochastic rounding as well when the weights are fp16; the launch knob
+    # it sweeps (BT_block_size) does not exist here, so each row is printed once
+    def adagrad(exact, stochastic):
+        if mixed:
+            if exact:
+                return lambda: table_batched_embeddings.backward_exact_adagrad_mixed_D(
+                    go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets,
+                    None, cc.optimizer_state, lr, eps, stochastic, 1)
+            return lambda: table_batched_embeddings.backward_approx_adagrad_mixed_D(
+                go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets, None,
+                cc.optimizer_state, lr, eps, L, stochastic, 1)
+        if exact:
+            return lambda: table_batched_embeddings.backward_exact_adagrad(
+                go, w, cc.table_offsets, indices, offsets, None, cc.optimizer_state, lr, eps, stochastic, 1)
+        return lambda: table_batched_embeddings.backward_approx_adagrad(
+            go, w, cc.table_offsets, indices, offsets, None, cc.optimizer_state, lr, eps, L, stochastic, 1)
+
+    for exact in (0, 1):
+        for stochastic in ((0, 1) if fp16 else (0,)):
+            name = "Backward-ADAGRAD-%s-%s-NR" % ("stochastic" if stochastic else "nonstochastic",
+                                                  "EXACT" if exact else "APPROX")
+            report(name, time_calls(iters, adagrad(exact, bool(stochastic))), 2 * fwd_bytes, shape)
 
 
 @click.command()

@@ -6,7 +6,9 @@ weight layout and `forward(indices, offsets, per_sample_weights)` signature; the
 optimizer is applied inside backward.  Differences, all extensions:
   * `num_embeddings` may be a list of per-table row counts;
   * SGD backward is exact (each distinct row updated once with its summed gradient);
-  * EXACT_ROWWISE_ADAGRAD accepts per-sample weights.
+  * EXACT_ROWWISE_ADAGRAD accepts per-sample weights;
+  * APPROX_ROWWISE_ADAGRAD applies the lookups of a row one at a time in position order, so a
+    batch in which rows repeat has a defined, reproducible result.
 """
 import enum
 import logging
@@ -56,7 +58,8 @@ class LookupFunction(torch.autograd.Function):
         # pay: the forward gather occupies every CU and a default-priority side stream only gets
         # the slots it leaves, so the step time is unchanged.  Off unless a caller opts in.
         ctx.plan = None
-        if LookupFunction.plan_ahead and any(ctx.needs_input_grad):
+        if (LookupFunction.plan_ahead and any(ctx.needs_input_grad)
+                and optimizer != Optimizer.APPROX_ROWWISE_ADAGRAD):
             ctx.plan = table_batched_embeddings.plan_backward(weights, table_offsets, indices, offsets)
         return table_batched_embeddings.forward(
             weights, table_offsets, indices, offsets, per_sample_weights, L_max,
@@ -171,6 +174,8 @@ class TableBatchedEmbeddingBags(nn.Module):
         self.row_cache = None
         if managed == EmbeddingLocation.HOST_CACHED:
             assert cache_slots is not None, "HOST_CACHED needs cache_slots"
+            if optimizer == Optimizer.APPROX_ROWWISE_ADAGRAD:
+                raise NotImplementedError("cache-fronted tables serve SGD and EXACT_ROWWISE_ADAGRAD")
             self.row_cache = table_batched_embeddings_cache.RowCache(self.embedding_weights.data, cache_slots,
                                                                      cache_policy, cache_stage_slots)
             # checkpoints must see the rows the cache holds ...

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -70,7 +70,7 @@ class CacheWorkspaceLayout(ctypes.Structure):
 CACHE_WAYS = 64
 STATIC_SCRATCH_BYTES = 32 << 20  # TBE_STATIC_SCRATCH_BYTES
 CACHE_LRU, CACHE_LFU = 0, 1
-OPT_SGD, OPT_ROWWISE_ADAGRAD = 0, 1
+OPT_SGD, OPT_ROWWISE_ADAGRAD, OPT_APPROX_ROWWISE_ADAGRAD = 0, 1, 2
 _cache_p = ctypes.POINTER(Cache)
 
 # name -> (restype, argtypes); exactly the declarations of include/tbe_hip.h
@@ -107,6 +107,9 @@ SIGNATURES = {
     "tbe_backward_exact_adagrad_stochastic": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p,
                                                              _i64, _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _u64,
                                                              _u64, _vp, _u64, _vp]),
+    "tbe_backward_approx_adagrad": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
+                                                   _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _i32, _u64, _u64, _vp,
+                                                   _u64, _vp]),
     "tbe_cache_workspace_layout": (ctypes.c_int, [_i64, _i64, ctypes.POINTER(CacheWorkspaceLayout)]),
     "tbe_cache_init": (ctypes.c_int, [_cache_p, _vp]),
     "tbe_cache_prepare": (ctypes.c_int, [_cache_p, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32,

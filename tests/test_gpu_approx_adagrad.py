@@ -1,0 +1,150 @@
+"""GPU parity of the approximate row-wise Adagrad (tbe_backward_approx_adagrad and
+tbe_backward_mixed with TBE_OPT_APPROX_ROWWISE_ADAGRAD, through the extension-module mirror)
+against the oracle's one-lookup-at-a-time restatement of the reference kernel
+(table_batched_embeddings_cuda.cu:648-704).  Rows repeat inside bags and across bags in every
+case here; tolerances: fp32 1e-5, fp16 1e-2 (weights are rounded after every lookup on both
+sides), fp64 1e-7."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_mixed_problem, make_problem
+from gpu_util import DEV, assert_close, dev
+
+import table_batched_embeddings as ext
+import table_batched_embeddings_ops as ops
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float16): 1e-2, np.dtype(np.float64): 1e-7}
+
+
+def _run_gpu(p, lr, eps, state0=None, stochastic=False):
+    w = dev(p["weights"])
+    st_dtype = torch.float64 if w.dtype == torch.float64 else torch.float32
+    st = torch.zeros(w.shape[0], dtype=st_dtype, device=DEV) if state0 is None else dev(state0)
+    g = ext.backward_approx_adagrad(dev(p["grad_output"]), w, dev(p["table_offsets"]), dev(p["indices"]),
+                                    dev(p["offsets"]), dev(p["per_sample_weights"]), st, lr, eps, 200, stochastic, 1)
+    torch.cuda.synchronize()
+    return w.cpu().numpy(), st.cpu().numpy(), None if g is None else g.cpu().numpy()
+
+
+def _run_oracle(oracle, p, lr, eps, state0=None, stochastic_rounding=None):
+    w = p["weights"].copy()
+    st = np.zeros(w.shape[0], np.float64 if w.dtype == np.float64 else np.float32) if state0 is None else state0.copy()
+    g = oracle.backward_approx(p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], lr, eps, st,
+                               p["per_sample_weights"], stochastic_rounding)
+    return w, st, g
+
+
+@pytest.mark.parametrize("dtype,D", [(np.float32, 128), (np.float32, 4), (np.float32, 12), (np.float16, 64),
+                                     (np.float16, 36), (np.float64, 8), (np.float32, 520), (np.float16, 1032)])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_approx_adagrad_matches_oracle_with_repeated_rows(oracle, dtype, D, weighted):
+    p = make_problem(31, T=3, E=60, D=D, B=90, L=7, dtype=dtype, weighted=weighted, zipf=1.3)
+    assert np.unique(p["indices"]).size < p["n"] // 4  # rows repeat, inside bags and across them
+    state0 = np.random.RandomState(1).uniform(0, 2, size=p["weights"].shape[0]).astype(
+        np.float64 if dtype == np.float64 else np.float32)
+    w, st, g = _run_gpu(p, 0.05, 0.1, state0)
+    w_ref, st_ref, g_ref = _run_oracle(oracle, p, 0.05, 0.1, state0)
+    tol = TOL[np.dtype(dtype)]
+    assert_close(st, st_ref, 1e-5 if dtype != np.float64 else 1e-10, "state")
+    assert_close(w, w_ref, tol, "weights")
+    if weighted:
+        assert_close(g, g_ref, tol if dtype != np.float16 else 2e-2, "grad of per-sample weights")
+    # rows no lookup touches keep their bits
+    touched = np.zeros(p["weights"].shape[0], bool)
+    bag_table = np.repeat(np.arange(p["T"] * p["B"]), np.diff(p["offsets"])) // p["B"]
+    touched[p["table_offsets"][bag_table] + p["indices"]] = True
+    assert w[~touched].tobytes() == p["weights"][~touched].tobytes()
+    assert st[~touched].tobytes() == state0[~touched].tobytes()
+
+
+def test_approx_differs_from_exact_where_it_should_and_reruns_are_bit_identical(oracle):
+    p = make_problem(32, T=2, E=30, D=32, B=200, L=5, dtype=np.float32, zipf=1.2)
+    a = _run_gpu(p, 0.05, 0.1)
+    b = _run_gpu(p, 0.05, 0.1)
+    assert a[0].tobytes() == b[0].tobytes() and a[1].tobytes() == b[1].tobytes()
+    w_exact, st_exact = p["weights"].copy(), np.zeros(60, np.float32)
+    oracle.backward("adagrad", p["grad_output"], w_exact, p["table_offsets"], p["indices"], p["offsets"], 0.05, 0.1,
+                    st_exact)
+    # per-lookup sums of squares exceed the square of the summed gradient whenever gradients cancel
+    assert np.abs(a[1] - st_exact).max() > 1.0
+
+
+def test_approx_adagrad_hot_row_and_long_bags(oracle):
+    """One row takes 70 % of 24 k lookups (a serial chain of ~17 k updates in one lane group),
+    bags of up to 300 lookups (the reference caps a bag at L_max = 200 shared-memory slots,
+    table_batched_embeddings_cuda.cu:738; there is no cap here)."""
+    rs = np.random.RandomState(33)
+    p = make_problem(33, T=2, E=40, D=64, B=80, L=300, dtype=np.float32, weighted=True)
+    hot = rs.rand(p["n"]) < 0.7
+    p["indices"][hot] = 5
+    w, st, g = _run_gpu(p, 0.001, 0.1)
+    w_ref, st_ref, g_ref = _run_oracle(oracle, p, 0.001, 0.1)
+    assert_close(st, st_ref, 1e-5)
+    assert_close(w, w_ref, 1e-5)
+    assert_close(g, g_ref, 1e-4)  # dot products of rows that 17 k fp32 updates have moved
+
+
+def test_approx_adagrad_stochastic_rounding_matches_oracle_stream(oracle):
+    p = make_problem(34, T=2, E=25, D=32, B=60, L=6, dtype=np.float16, weighted=False, zipf=1.2)
+    torch.manual_seed(1234)
+    gen = torch.cuda.default_generators[0]
+    seed, offset = gen.initial_seed() & 0xFFFFFFFFFFFFFFFF, gen.get_offset()
+    w, st, _ = _run_gpu(p, 0.05, 0.1, stochastic=True)
+    assert gen.get_offset() == offset + 4
+    w_ref, st_ref, _ = _run_oracle(oracle, p, 0.05, 0.1, stochastic_rounding=(seed, offset))
+    assert_close(st, st_ref, 1e-5)
+    # same random words for the k-th update of every element: the rounded rows agree except where
+    # the fp32 value differs in its last bits (different summation order of ||g||^2)
+    differing = (w.view(np.uint16) != w_ref.view(np.uint16)).mean()
+    assert differing < 0.02, differing
+    assert_close(w, w_ref, 1e-2)
+    w_rn, _, _ = _run_gpu(p, 0.05, 0.1, stochastic=False)
+    assert (w.view(np.uint16) != w_rn.view(np.uint16)).mean() > 0.2  # and it is not round-to-nearest
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.float64])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_approx_adagrad_mixed_D_matches_oracle(oracle, dtype, weighted):
+    tables = [(30, 8), (7, 32), (100, 4), (16, 12), (3, 520), (40, 128)]
+    p = make_mixed_problem(35, tables, B=40, L=9, dtype=dtype, weighted=weighted)
+    w = dev(p["weights"])
+    st_np = np.zeros(sum(r for r, _ in tables), np.float64 if dtype == np.float64 else np.float32)
+    st = dev(st_np)
+    g = ext.backward_approx_adagrad_mixed_D(
+        dev(p["grad_output"]), w, dev(p["table_offsets"]), dev(p["table_dim_offsets"]), dev(p["dim_offsets"]),
+        int(p["dim_offsets"][-1]), dev(p["indices"]), dev(p["offsets"]), dev(p["per_sample_weights"]), st, 0.05, 0.1,
+        200, False, 1)
+    w_ref = p["weights"].copy()
+    g_ref = oracle.backward_approx_mixed(p["grad_output"], w_ref, p["table_offsets"], p["table_dim_offsets"],
+                                         p["dim_offsets"], p["indices"], p["offsets"], 0.05, 0.1, st_np,
+                                         p["per_sample_weights"])
+    tol = TOL[np.dtype(dtype)]
+    assert_close(st.cpu().numpy(), st_np, 1e-5 if dtype != np.float64 else 1e-10)
+    assert_close(w.cpu().numpy(), w_ref, tol)
+    if weighted:
+        assert_close(g.cpu().numpy(), g_ref, tol if dtype != np.float16 else 2e-2)
+
+
+def test_module_with_the_approximate_optimizer_and_repeated_rows(oracle):
+    """Optimizer.APPROX_ROWWISE_ADAGRAD through the module, with replacement (the reference's test
+    has to draw without, test_table_batched_embeddings.py:244): two steps against the oracle."""
+    T, E, D, B, L = 3, 50, 32, 40, 6
+    p = make_problem(36, T, E, D, B, L, np.float32, ragged=True, weighted=True, zipf=1.2)
+    cc = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.APPROX_ROWWISE_ADAGRAD, learning_rate=0.5,
+                                       eps=0.2).cuda()
+    cc.embedding_weights.data.copy_(dev(p["weights"]))
+    w_ref, st_ref = p["weights"].copy(), np.zeros(T * E, np.float32)
+    for _ in range(2):
+        psw = dev(p["per_sample_weights"]).requires_grad_(True)
+        cc(dev(p["indices"]), dev(p["offsets"]), psw).backward(dev(p["grad_output"]))
+        g_ref = oracle.backward_approx(p["grad_output"], w_ref, p["table_offsets"], p["indices"], p["offsets"], 0.5,
+                                       0.2, st_ref, p["per_sample_weights"])
+        assert_close(psw.grad.cpu().numpy(), g_ref, 1e-5)
+    assert_close(cc.optimizer_state.cpu().numpy(), st_ref, 1e-5)
+    assert_close(cc.embedding_weights.detach().cpu().numpy(), w_ref, 1e-5)
+    with pytest.raises(NotImplementedError):
+        ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.APPROX_ROWWISE_ADAGRAD,
+                                      managed=ops.EmbeddingLocation.HOST_CACHED, cache_slots=64)

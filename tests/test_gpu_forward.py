@@ -185,5 +185,15 @@ def test_benchmark_cli_runs_with_reference_flags():
     out = subprocess.run(cmd, capture_output=True, text=True, timeout=280)
     assert out.returncode == 0, out.stderr[-2000:]
     records = [json.loads(line) for line in out.stdout.splitlines() if line.startswith("{")]
-    assert [r["op"] for r in records] == ["Forward", "Backward-SGD-EXACT", "Backward-ADAGRAD-nonstochastic-EXACT"]
+    # the reference's rows (:240, :266-357) for fp16 weights, plus exact SGD
+    assert [r["op"] for r in records] == [
+        "Forward", "Backward-SGD-EXACT", "Backward-ADAGRAD-nonstochastic-APPROX-NR",
+        "Backward-ADAGRAD-stochastic-APPROX-NR", "Backward-ADAGRAD-nonstochastic-EXACT-NR",
+        "Backward-ADAGRAD-stochastic-EXACT-NR"]
     assert all(r["BW_GBps"] > 0 for r in records)
+    for extra in (["--managed"], ["--mixed"]):  # host-resident tables / per-table dimensions
+        out = subprocess.run(cmd[:-1] + extra, capture_output=True, text=True, timeout=280)
+        assert out.returncode == 0, out.stderr[-2000:]
+        ops_run = [json.loads(line)["op"] for line in out.stdout.splitlines() if line.startswith("{")]
+        assert ops_run == ["Forward", "Backward-SGD-EXACT", "Backward-ADAGRAD-nonstochastic-APPROX-NR",
+                           "Backward-ADAGRAD-nonstochastic-EXACT-NR"]

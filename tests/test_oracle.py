@@ -455,3 +455,130 @@ def test_interleaved_layout_matches_embeddingbag(oracle):
         y.backward(torch.from_numpy(go[:, t, :].copy()))
         want = bag.weight.detach() - bag.weight.grad.to_dense() * 0.05
         np.testing.assert_allclose(w[:, t, :], want.numpy(), rtol=1e-5, atol=1e-6)
+
+
+# ------------------------------------------------- approximate row-wise Adagrad
+# oracle_backward_approx restates batched_embedding_backward_adagrad_approx_kernel_1
+# (tbe.cu:648-704) one lookup at a time.  Pinned by: hand-computed cases that tell the state used
+# by the multiplier (after the lookup's own addition), the per-lookup weighting and the row a
+# weighted lookup sees (already moved by earlier lookups) apart from their plausible mistakes; the
+# reference test-suite's own oracle (torch.nn.EmbeddingBag + Python Adagrad,
+# test_table_batched_embeddings.py:296-318) on indices drawn without replacement, the only case
+# that test covers; a closed form for k identical hits; equality with the exact update when no
+# row repeats; the mixed-D addressing against the uniform one.
+def _one_row_problem(grads, lengths, D=4):
+    """One table with one row; bag b has lengths[b] lookups of it and output gradient grads[b]."""
+    B = len(grads)
+    offsets = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    indices = np.zeros(int(offsets[-1]), np.int32)
+    go = np.asarray(grads, np.float32).reshape(B, 1, D)
+    return indices, offsets, go
+
+
+def test_approx_adagrad_two_bags_by_hand(oracle):
+    indices, offsets, go = _one_row_problem([[1, 2, 2, 0], [0, 3, 4, 0]], [1, 1])
+    w = np.ones((1, 4), np.float32)
+    state = np.array([7.0], np.float32)
+    oracle.backward_approx(go, w, np.zeros(1, np.int32), indices, offsets, 0.5, 0.0, state)
+    # lookup 0: state 7 + 9 = 16, multiplier 0.5 / 4; lookup 1: state 16 + 25 = 41, multiplier 0.5 / sqrt(41)
+    w1 = 1.0 - 0.125 * np.array([1, 2, 2, 0])
+    w2 = w1 - 0.5 / np.sqrt(41.0) * np.array([0, 3, 4, 0])
+    assert state[0] == 41.0
+    np.testing.assert_allclose(w[0], w2, rtol=1e-6)
+    # the exact update would have summed the gradients first: G = [1, 5, 6, 0], state 7 + 62
+    assert abs(state[0] - 69.0) > 1
+
+
+def test_approx_adagrad_weighted_by_hand(oracle):
+    indices, offsets, go = _one_row_problem([[1, 2, 2, 0], [0, 3, 4, 0]], [1, 1])
+    w = np.ones((1, 4), np.float32)
+    state = np.array([7.0], np.float32)
+    psw = np.array([2.0, 0.5], np.float32)
+    gpsw = oracle.backward_approx(go, w, np.zeros(1, np.int32), indices, offsets, 0.5, 0.0, state, psw)
+    s1 = 7.0 + 9.0 * 4.0
+    m1 = 2.0 * 0.5 / np.sqrt(s1)
+    w1 = 1.0 - m1 * np.array([1, 2, 2, 0])
+    s2 = s1 + 25.0 * 0.25
+    m2 = 0.5 * 0.5 / np.sqrt(s2)
+    w2 = w1 - m2 * np.array([0, 3, 4, 0])
+    np.testing.assert_allclose(state[0], s2, rtol=1e-6)
+    np.testing.assert_allclose(w[0], w2, rtol=1e-6)
+    # the first lookup sees the untouched row, the second the row the first one left behind
+    np.testing.assert_allclose(gpsw, [5.0, 3 * w1[1] + 4 * w1[2]], rtol=1e-6)
+    assert abs(gpsw[1] - 7.0) > 0.1  # ... not the row as it was before the call
+
+
+def test_approx_adagrad_repeat_inside_a_bag_and_k_identical_hits(oracle):
+    # one bag, the same row twice: state 7 -> 16 -> 25, multipliers lr/4 and lr/5
+    indices, offsets, go = _one_row_problem([[1, 2, 2, 0]], [2])
+    w = np.ones((1, 4), np.float32)
+    state = np.array([7.0], np.float32)
+    oracle.backward_approx(go, w, np.zeros(1, np.int32), indices, offsets, 0.5, 0.0, state)
+    assert state[0] == 25.0
+    np.testing.assert_allclose(w[0], 1.0 - 0.5 * (1 / 4 + 1 / 5) * np.array([1, 2, 2, 0]), rtol=1e-6)
+    # k bags with the same gradient g, state from 0, eps 0: state = k |g|^2 and
+    # w = w0 - lr * g / |g| * sum_{j=1..k} 1 / sqrt(j)
+    k, g = 37, np.array([0.5, -1.0, 2.0, 0.25])
+    indices, offsets, go = _one_row_problem([g] * k, [1] * k)
+    w = np.full((1, 4), 0.3, np.float64)
+    state = np.zeros(1, np.float64)
+    oracle.backward_approx(go.astype(np.float64), w, np.zeros(1, np.int32), indices, offsets, 0.1, 0.0, state)
+    norm = np.sqrt((g * g).sum())
+    np.testing.assert_allclose(state[0], k * norm ** 2, rtol=1e-12)
+    lr = float(np.float32(0.1))  # the learning rate is a float on the interface
+    np.testing.assert_allclose(w[0], 0.3 - lr * g / norm * (1.0 / np.sqrt(np.arange(1, k + 1))).sum(), rtol=1e-12)
+
+
+@pytest.mark.parametrize("weighted", [False, True])
+def test_approx_adagrad_matches_embedding_bag_without_replacement(oracle, weighted):
+    """The reference's own check of its approximate kernel (test_table_batched_embeddings.py:
+    244-318): indices drawn without replacement, per-table torch.nn.EmbeddingBag gradient,
+    state = grad^2 summed per row, weights = addcdiv(w, -lr, grad, sqrt(state) + eps)."""
+    import torch
+    rs = np.random.RandomState(21)
+    T, E, D, B, L, lr, eps = 3, 400, 16, 12, 5, 0.5, 0.2
+    weights = rs.uniform(-1, 1, size=(T * E, D)).astype(np.float32)
+    indices = np.concatenate([rs.choice(E, size=B * L, replace=False) for _ in range(T)]).astype(np.int32)
+    offsets = np.arange(0, T * B * L + 1, L, dtype=np.int32)
+    go = rs.randn(B, T, D).astype(np.float32)
+    psw = rs.uniform(0.2, 1.5, size=T * B * L).astype(np.float32) if weighted else None
+    table_offsets = (np.arange(T) * E).astype(np.int32)
+    want_w, want_s = weights.copy(), np.zeros(T * E, np.float32)
+    for t in range(T):
+        bag = torch.nn.EmbeddingBag(E, D, mode="sum", sparse=True)
+        bag.weight.data.copy_(torch.from_numpy(weights[t * E:(t + 1) * E]))
+        idx = torch.from_numpy(indices[t * B * L:(t + 1) * B * L].astype(np.int64))
+        off = torch.arange(0, B * L, L)
+        kw = {"per_sample_weights": torch.from_numpy(psw[t * B * L:(t + 1) * B * L])} if weighted else {}
+        bag(idx, off, **kw).backward(torch.from_numpy(go[:, t, :].copy()))
+        dense = bag.weight.grad.to_dense()
+        st = dense.pow(2).sum(1)
+        want_s[t * E:(t + 1) * E] = st.numpy()
+        want_w[t * E:(t + 1) * E] = torch.addcdiv(bag.weight.data, dense, (st.sqrt() + eps).view(-1, 1),
+                                                  value=-lr).numpy()
+    w, s = weights.copy(), np.zeros(T * E, np.float32)
+    oracle.backward_approx(go, w, table_offsets, indices, offsets, lr, eps, s, psw)
+    np.testing.assert_allclose(s, want_s, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(w, want_w, rtol=1e-5, atol=1e-6)
+    # and the exact update agrees when no row repeats (bit for bit when unweighted)
+    w2, s2 = weights.copy(), np.zeros(T * E, np.float32)
+    oracle.backward("adagrad", go, w2, table_offsets, indices, offsets, lr, eps, s2, psw)
+    if weighted:
+        np.testing.assert_allclose(w, w2, rtol=1e-5, atol=1e-6)
+    else:
+        assert w.tobytes() == w2.tobytes() and s.tobytes() == s2.tobytes()
+
+
+def test_approx_adagrad_mixed_addressing_equals_uniform(oracle):
+    rs = np.random.RandomState(22)
+    T, E, D, B, L = 3, 50, 8, 20, 4
+    p = make_problem(23, T, E, D, B, L, np.float32, weighted=True, zipf=1.2)
+    w, s = p["weights"].copy(), np.zeros(T * E, np.float32)
+    g1 = oracle.backward_approx(p["grad_output"], w, p["table_offsets"], p["indices"], p["offsets"], 0.1, 0.01, s,
+                                p["per_sample_weights"])
+    wm, sm = p["weights"].reshape(-1).copy(), np.zeros(T * E, np.float32)
+    g2 = oracle.backward_approx_mixed(
+        p["grad_output"].reshape(B, T * D), wm, np.arange(T + 1) * E * D, np.arange(T + 1) * E, np.arange(T + 1) * D,
+        p["indices"], p["offsets"], 0.1, 0.01, sm, p["per_sample_weights"])
+    assert wm.tobytes() == w.tobytes() and sm.tobytes() == s.tobytes() and g1.tobytes() == g2.tobytes()
+    assert (np.diff(p["offsets"]) > 1).any() and np.unique(p["indices"]).size < p["n"]  # rows do repeat here
