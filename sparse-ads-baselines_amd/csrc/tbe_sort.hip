@@ -6,9 +6,14 @@
 // The sort is the contract of cub::DeviceRadixSort::SortPairs as the reference
 // calls it (table_batched_embeddings_cuda.cu:1639-1655): ascending, stable,
 // key bits [0, end_bit).  A pass handles a digit of 8 to 10 bits (the fewest passes that cover
-// end_bit).  Each pass is four kernels:
-//   histogram  per-tile digit counts (LDS atomics) -> counts[table][digit][tile]
-//   scan       exclusive prefix sum over counts[] (workgroup sums, then the chunks)
+// end_bit).  Each pass is three or four kernels:
+//   histogram  per-tile digit counts (LDS atomics)
+//   scan       turns the counts into the output position of every (table, digit, tile) run.
+//              Many tables of few tiles each (the backward's case: every table is sorted on its
+//              own): counts[tile][digit], the histogram also adds its counts to per-table digit
+//              totals, and ONE kernel with a workgroup per table scans the totals over the
+//              digits and walks the table's tiles.  Otherwise: counts[table][digit][tile] and a
+//              linear exclusive prefix sum over the whole array (workgroup sums, then the chunks)
 //   scatter    ranks each key inside its tile with wavefront ballots (all lanes
 //              holding the same digit are found with one ballot per digit bit; the lowest lane
 //              reserves the run in a per-wavefront LDS counter), reorders the
@@ -16,6 +21,8 @@
 //              them out in runs.
 // A tile is 4096 pairs; position order inside a tile is (wavefront, item, lane),
 // which the ranking preserves, so the sort is stable.
+
+#include <algorithm>
 
 #include "tbe_stages.h"
 
@@ -27,6 +34,11 @@ constexpr int kMaxBins = 1 << kMaxRadixBits;
 constexpr int kItems = 16;                        // pairs per thread per tile
 constexpr int kTile = kBlockThreads * kItems;     // 4096
 constexpr int kWaveTile = kWave * kItems;         // 1024 pairs per wavefront
+
+// Per-table scan: tables of at most this many tiles are scanned inside the scatter kernel (every
+// workgroup adds up the counts of the earlier tiles of its table itself); a batch with a larger
+// table runs radix_table_scan_kernel first.  tile_prefix[T + 1] holds the choice (1 = inside).
+constexpr int kInlineScanTiles = 48;
 
 constexpr int kSegItems = 8;
 constexpr int kSegTile = kBlockThreads * kSegItems;  // 2048
@@ -118,12 +130,20 @@ __global__ __launch_bounds__(kBlockThreads) void interleaved_rows_kernel(
 constexpr int kScanItems = 8;
 constexpr int kScanChunk = kBlockThreads * kScanItems;  // 2048 count entries per workgroup
 
+// Workgroup 0 derives the tables' position ranges and tile counts; all workgroups clear the
+// per-table digit totals of every pass (`totals_words` words; none with the linear scan).
 __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
     const int32_t *__restrict__ offsets, int B, int num_tables, uint32_t n,
-    uint32_t *__restrict__ table_starts, uint32_t *__restrict__ tile_prefix) {
+    uint32_t *__restrict__ table_starts, uint32_t *__restrict__ tile_prefix,
+    uint32_t *__restrict__ totals, int64_t totals_words) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   const int tid = threadIdx.x;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + tid) * 4; i < totals_words;
+       i += static_cast<int64_t>(gridDim.x) * kBlockThreads * 4)
+    *reinterpret_cast<uint4 *>(totals + i) = make_uint4(0, 0, 0, 0);
+  if (blockIdx.x != 0) return;
   uint32_t carry = 0;
+  uint32_t most = 0;
   for (int c0 = 0; c0 < num_tables; c0 += kBlockThreads) {
     const int t = c0 + tid;
     uint32_t tiles = 0;
@@ -142,11 +162,18 @@ __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
     const uint32_t incl = block_inclusive_scan(tiles, s_wave, total);
     if (t < num_tables) tile_prefix[t] = carry + incl - tiles;
     carry += total;
+    most = max(most, tiles);
     __syncthreads();
   }
+  // the table with the most tiles decides how the per-table scan is done (see radix_scatter_kernel)
+  for (int d = 1; d < kWave; d <<= 1) most = max(most, static_cast<uint32_t>(__shfl_xor(static_cast<int>(most), d, kWave)));
+  if ((tid & (kWave - 1)) == 0) s_wave[tid >> 6] = most;
+  __syncthreads();
   if (tid == 0) {
+    for (int w = 1; w < kWavesPerBlock; ++w) most = max(most, s_wave[w]);
     table_starts[num_tables] = n;
     tile_prefix[num_tables] = carry;
+    tile_prefix[num_tables + 1] = most <= kInlineScanTiles ? 1u : 0u;
   }
 }
 
@@ -157,13 +184,14 @@ struct TileInfo {
   int count;           // pairs in the tile (0: nothing to do)
   int64_t count_base;  // index of counts[table][digit 0][this tile]
   int table_tiles;     // stride between digits in counts[]
+  int64_t tile_index;  // number of the tile among all tiles
 };
 
 template <int BITS>
 __device__ __forceinline__ TileInfo locate_tile(const uint32_t *__restrict__ table_starts,
                                                 const uint32_t *__restrict__ tile_prefix,
                                                 int num_tables, int max_tiles) {
-  TileInfo info{0, 0, 0, 0, 0};
+  TileInfo info{0, 0, 0, 0, 0, 0};
   const uint32_t tile = blockIdx.x;
   if (tile >= tile_prefix[num_tables]) return info;
   int lo = 0, hi = num_tables;  // tile_prefix[lo] <= tile < tile_prefix[hi]
@@ -181,16 +209,26 @@ __device__ __forceinline__ TileInfo locate_tile(const uint32_t *__restrict__ tab
   info.count = static_cast<int>(max(int64_t{0}, min(left, static_cast<int64_t>(kTile))));
   info.count_base = (static_cast<int64_t>(first_tile) << BITS) + j;
   info.table_tiles = static_cast<int>(tiles);
+  info.tile_index = static_cast<int64_t>(tile);
   return info;
+}
+
+// Where the count of digit d of a tile lives.  LOCAL: counts[tile][digit] (a tile's counts are
+// contiguous: coalesced stores and loads); else counts[table][digit][tile] (the order of the
+// linear scan).
+template <int BITS, bool LOCAL>
+__device__ __forceinline__ int64_t count_index(const TileInfo &tile, int d) {
+  if constexpr (LOCAL) return (tile.tile_index << BITS) + d;
+  else return tile.count_base + static_cast<int64_t>(d) * tile.table_tiles;
 }
 
 // BITS = digit width of the pass (8, 9 or 10): 2^BITS bins, each thread owns 2^BITS / 256
 // consecutive digits in the per-digit steps.
-template <int BITS>
+template <int BITS, bool LOCAL>
 __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     const uint32_t *__restrict__ keys, const uint32_t *__restrict__ table_starts,
     const uint32_t *__restrict__ tile_prefix, int num_tables, int max_tiles, int shift,
-    uint32_t mask, uint32_t *__restrict__ counts) {
+    uint32_t mask, uint32_t *__restrict__ counts, uint32_t *__restrict__ totals) {
   constexpr int kBinsT = 1 << BITS;
   __shared__ uint32_t s_hist[kBinsT];
   const TileInfo tile = locate_tile<BITS>(table_starts, tile_prefix, num_tables, max_tiles);
@@ -212,10 +250,73 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     }
   }
   __syncthreads();
-  // (one 4-byte store per digit, a tile apart: these scattered stores are most of this kernel's time)
+  // (linear-scan layout: one 4-byte store per digit, a tile apart -- these scattered stores are
+  // most of the kernel's time there; per-table layout: coalesced stores, and the table's digit
+  // totals collect the counts with integer atomics, whose order does not matter)
 #pragma unroll
-  for (int d = tid; d < kBinsT; d += kBlockThreads)
-    counts[tile.count_base + static_cast<int64_t>(d) * tile.table_tiles] = s_hist[d];
+  for (int d = tid; d < kBinsT; d += kBlockThreads) {
+    const uint32_t c = s_hist[d];
+    counts[count_index<BITS, LOCAL>(tile, d)] = c;
+    if constexpr (LOCAL) {
+      if (c) atomicAdd(&totals[(static_cast<int64_t>(tile.table) << BITS) + d], c);
+    }
+  }
+}
+
+// Per-table scan (LOCAL layout): workgroup t turns table t's counts[tile][digit] into output
+// positions.  Thread `tid` owns 2^BITS / 256 consecutive digits: exclusive scan of the table's
+// digit totals (thread-local, then across the workgroup) gives the first output position of every
+// digit, then the thread walks the table's tiles, replacing each count by the running position.
+template <int BITS>
+__global__ __launch_bounds__(kBlockThreads) void radix_table_scan_kernel(
+    uint32_t *__restrict__ counts, const uint32_t *__restrict__ totals,
+    const uint32_t *__restrict__ table_starts, const uint32_t *__restrict__ tile_prefix,
+    int max_tiles) {
+  constexpr int kBinsT = 1 << BITS;
+  constexpr int kOwned = kBinsT / kBlockThreads;
+  constexpr int kAhead = 4;  // tiles whose counts are requested together
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int t = blockIdx.x;
+  if (tile_prefix[gridDim.x + 1] != 0u) return;  // every table is small: the scatter kernel scans
+  const uint32_t first_tile = tile_prefix[t];
+  const uint32_t tiles = tile_prefix[t + 1] - first_tile;
+  if (tiles == 0 || first_tile + tiles > static_cast<uint32_t>(max_tiles)) return;
+  const int d0 = threadIdx.x * kOwned;
+  uint32_t running[kOwned];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int q = 0; q < kOwned; ++q) {
+    running[q] = totals[(static_cast<int64_t>(t) << BITS) + d0 + q];
+    mine += running[q];
+  }
+  uint32_t total;
+  uint32_t start = table_starts[t] + block_inclusive_scan(mine, s_wave, total) - mine;
+#pragma unroll
+  for (int q = 0; q < kOwned; ++q) {
+    const uint32_t c = running[q];
+    running[q] = start;
+    start += c;
+  }
+  uint32_t *mine_counts = counts + (static_cast<int64_t>(first_tile) << BITS) + d0;
+  for (uint32_t j0 = 0; j0 < tiles; j0 += kAhead) {
+    uint32_t c[kAhead][kOwned];
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) {
+      const uint32_t j = min(j0 + a, tiles - 1);  // clamped: straight-line loads
+#pragma unroll
+      for (int q = 0; q < kOwned; ++q) c[a][q] = mine_counts[(static_cast<int64_t>(j) << BITS) + q];
+    }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) {
+      if (j0 + a < tiles) {
+#pragma unroll
+        for (int q = 0; q < kOwned; ++q) {
+          mine_counts[(static_cast<int64_t>(j0 + a) << BITS) + q] = running[q];
+          running[q] += c[a][q];
+        }
+      }
+    }
+  }
 }
 
 // Exclusive prefix sum over counts[0, bins * tiles): workgroup sums first, then every workgroup
@@ -283,13 +384,13 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
 
 // key_bias (nullable): added to the keys of table t as they are written (the last pass turns
 // rows inside a table into rows of the concatenated tables).
-template <int BITS>
+template <int BITS, bool LOCAL>
 __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ values_in,
     uint32_t *__restrict__ keys_out, uint32_t *__restrict__ values_out,
     const uint32_t *__restrict__ table_starts, const uint32_t *__restrict__ tile_prefix,
     int num_tables, int max_tiles, int shift, uint32_t mask, const uint32_t *__restrict__ bases,
-    const int32_t *__restrict__ key_bias) {
+    const uint32_t *__restrict__ totals, const int32_t *__restrict__ key_bias) {
   constexpr int kBinsT = 1 << BITS;
   constexpr int kOwned = kBinsT / kBlockThreads;  // consecutive digits per thread
   // The per-wavefront digit counters are only needed until every key knows its slot in the
@@ -315,9 +416,37 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   // output position of the tile's first key of every digit this thread owns (needed late;
   // fetched first so the latency hides behind the ranking)
   uint32_t digit_base[kOwned];
+  uint32_t digit_total[kOwned];  // per-table layout, scan done here: keys of the table with each digit
+  bool inline_scan = false;
+  if constexpr (LOCAL) inline_scan = tile_prefix[num_tables + 1] != 0u;
+  if (inline_scan) {
+    // bases[] still holds counts[tile][digit]: this tile's keys of digit d go behind the table's
+    // keys of smaller digits (added up further down, once the totals are here) and behind the keys
+    // of digit d in the earlier tiles of the table
+    const int j = static_cast<int>(tile.tile_index - (tile.count_base >> BITS));  // tile inside its table
+    const uint32_t *first = bases + ((tile.count_base >> BITS) << BITS) + tid * kOwned;
 #pragma unroll
-  for (int q = 0; q < kOwned; ++q)
-    digit_base[q] = bases[tile.count_base + static_cast<int64_t>(tid * kOwned + q) * tile.table_tiles];
+    for (int q = 0; q < kOwned; ++q) {
+      digit_total[q] = totals[(static_cast<int64_t>(tile.table) << BITS) + tid * kOwned + q];
+      digit_base[q] = 0;
+    }
+    constexpr int kAhead = 8;
+    for (int j0 = 0; j0 < j; j0 += kAhead) {
+      uint32_t c[kAhead][kOwned];
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+        for (int q = 0; q < kOwned; ++q)
+          c[a][q] = first[(static_cast<int64_t>(min(j0 + a, j - 1)) << BITS) + q];
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+        for (int q = 0; q < kOwned; ++q) digit_base[q] += (j0 + a < j) ? c[a][q] : 0u;
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < kOwned; ++q) digit_base[q] = bases[count_index<BITS, LOCAL>(tile, tid * kOwned + q)];
+  }
 
 #pragma unroll
   for (int w = 0; w < kWavesPerBlock; ++w)
@@ -390,6 +519,20 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     }
     uint32_t total;
     uint32_t bin_start = block_inclusive_scan(mine, s_scan, total) - mine;
+    if (inline_scan) {
+      // first output position of every digit inside the table: exclusive scan of the table's totals
+      uint32_t table_sum = 0;
+#pragma unroll
+      for (int q = 0; q < kOwned; ++q) table_sum += digit_total[q];
+      __syncthreads();  // s_scan is read by every wavefront above
+      uint32_t all;
+      uint32_t digit_start = table_starts[tile.table] + block_inclusive_scan(table_sum, s_scan, all) - table_sum;
+#pragma unroll
+      for (int q = 0; q < kOwned; ++q) {
+        digit_base[q] += digit_start;
+        digit_start += digit_total[q];
+      }
+    }
 #pragma unroll
     for (int q = 0; q < kOwned; ++q) {
       const int d = tid * kOwned + q;
@@ -557,13 +700,22 @@ inline int num_seg_tiles(int64_t n) { return static_cast<int>(ceil_div(n, kSegTi
 }  // namespace
 
 // Sort workspace: [tmp keys n][tmp values n][counts 1024 * max_tiles][workgroup sums of the count
-// scan][table_starts T+1][tile_prefix T+1]; max_tiles = ceil(n / 4096) + T.
+// scan][table_starts T+1][tile_prefix T+2][digit totals 4 * 1024 * T]; max_tiles = ceil(n / 4096) + T.
 namespace {
 struct SortScratch {
-  uint64_t tmp_keys, tmp_vals, counts, block_sums, table_starts, tile_prefix, total;
+  uint64_t tmp_keys, tmp_vals, counts, block_sums, table_starts, tile_prefix, totals, total;
   int max_tiles;
   int scan_blocks;  // for the widest digit
+  int64_t totals_words;  // per-table digit totals of all passes (0: linear scan)
 };
+
+constexpr int kMaxPasses = 4;  // 32 key bits in digits of at least 8
+
+// The per-table scan walks a table's tiles one after the other in one workgroup: it is used when
+// the tables have few tiles each on average (the batch's lookups are spread over many tables).
+inline bool use_table_scan(int64_t n, int32_t num_tables, bool have_tables) {
+  return have_tables && num_tables >= 8 && ceil_div(n, kTile) <= static_cast<int64_t>(num_tables) * 128;
+}
 
 SortScratch sort_scratch(int64_t n, int32_t num_tables) {
   SortScratch s;
@@ -577,7 +729,10 @@ SortScratch sort_scratch(int64_t n, int32_t num_tables) {
   s.counts = off; off += align_up(static_cast<uint64_t>(s.max_tiles) * kMaxBins * 4, 256);
   s.block_sums = off; off += align_up(static_cast<uint64_t>(s.scan_blocks) * 4, 256);
   s.table_starts = off; off += align_up((tables + 1) * 4, 256);
-  s.tile_prefix = off; off += align_up((tables + 1) * 4, 256);
+  s.tile_prefix = off; off += align_up((tables + 2) * 4, 256);
+  // (sized for every table count, so that the layout does not depend on the path taken)
+  s.totals_words = static_cast<int64_t>(tables) * kMaxBins * kMaxPasses;
+  s.totals = off; off += align_up(static_cast<uint64_t>(s.totals_words) * 4, 256);
   s.total = off;
   return s;
 }
@@ -589,6 +744,7 @@ struct RadixPass {
   int num_tables, max_tiles, shift;
   uint32_t mask;
   uint32_t *counts, *block_sums;
+  uint32_t *totals;  // this pass's per-table digit totals, zeroed; null: linear scan
   const int32_t *key_bias;
 };
 
@@ -596,16 +752,26 @@ template <int BITS>
 void launch_radix_pass(const RadixPass &p, hipStream_t stream) {
   const dim3 block(kBlockThreads);
   const dim3 tiles(p.max_tiles);
+  if (p.totals) {
+    TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, true>), tiles, block, p.src_k,
+               p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, p.totals);
+    TBE_LAUNCH("radix_table_scan", stream, radix_table_scan_kernel<BITS>, dim3(p.num_tables), block, p.counts,
+               p.totals, p.table_starts, p.tile_prefix, p.max_tiles);
+    TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, true>), tiles, block, p.src_k, p.src_v,
+               p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
+               p.counts, p.totals, p.key_bias);
+    return;
+  }
   const dim3 scan_blocks(static_cast<unsigned>(ceil_div(static_cast<int64_t>(p.max_tiles) << BITS, kScanChunk)));
-  TBE_LAUNCH("radix_histogram", stream, radix_histogram_kernel<BITS>, tiles, block, p.src_k, p.table_starts,
-             p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts);
+  TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, false>), tiles, block, p.src_k,
+             p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, nullptr);
   TBE_LAUNCH("radix_scan_reduce", stream, radix_scan_reduce_kernel, scan_blocks, block, p.counts,
              p.tile_prefix, p.num_tables, BITS, p.block_sums);
   TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, scan_blocks, block, p.counts, p.tile_prefix,
              p.num_tables, BITS, p.block_sums);
-  TBE_LAUNCH("radix_scatter", stream, radix_scatter_kernel<BITS>, tiles, block, p.src_k, p.src_v, p.dst_k,
-             p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts,
-             p.key_bias);
+  TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, false>), tiles, block, p.src_k, p.src_v,
+             p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
+             p.counts, nullptr, p.key_bias);
 }
 }  // namespace
 
@@ -631,10 +797,14 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   p.max_tiles = scratch.max_tiles;
   p.counts = reinterpret_cast<uint32_t *>(ws + scratch.counts);
   p.block_sums = reinterpret_cast<uint32_t *>(ws + scratch.block_sums);
-  TBE_LAUNCH("sort_setup", stream, sort_setup_kernel, dim3(1), dim3(kBlockThreads),
+  const bool table_scan = use_table_scan(n, num_tables, tables != nullptr) && passes <= kMaxPasses;
+  uint32_t *totals = reinterpret_cast<uint32_t *>(ws + scratch.totals);
+  const int64_t totals_words = table_scan ? static_cast<int64_t>(num_tables) * kMaxBins * passes : 0;
+  const unsigned setup_blocks = static_cast<unsigned>(1 + std::min<int64_t>(ceil_div(totals_words, kBlockThreads * 4), 255));
+  TBE_LAUNCH("sort_setup", stream, sort_setup_kernel, dim3(setup_blocks), dim3(kBlockThreads),
              tables ? tables->offsets : nullptr, tables ? tables->bags_per_table : 0, num_tables,
              static_cast<uint32_t>(n), const_cast<uint32_t *>(p.table_starts),
-             const_cast<uint32_t *>(p.tile_prefix));
+             const_cast<uint32_t *>(p.tile_prefix), totals, totals_words);
 
   p.src_k = reinterpret_cast<const uint32_t *>(keys_in);
   p.src_v = reinterpret_cast<const uint32_t *>(values_in);
@@ -647,6 +817,7 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
     p.dst_k = to_out ? reinterpret_cast<uint32_t *>(keys_out) : tmp_keys;
     p.dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
     p.key_bias = (tables && pass == passes - 1) ? tables->key_bias : nullptr;
+    p.totals = table_scan ? totals + static_cast<int64_t>(pass) * num_tables * kMaxBins : nullptr;
     if (bits <= 8)
       launch_radix_pass<8>(p, stream);
     else if (bits == 9)
