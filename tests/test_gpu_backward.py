@@ -131,7 +131,9 @@ def _plan_views(p, max_table_rows):
     return view(lay.keys_sorted, n), view(lay.positions_sorted, n), view(lay.segment_starts, U + 1)
 
 
-@pytest.mark.parametrize("case", ["ragged_rows", "empty_tables", "many_small_tables", "multi_tile_tables", "one_table"])
+@pytest.mark.parametrize("case", ["ragged_rows", "empty_tables", "many_small_tables", "multi_tile_tables", "one_table",
+                                  "eight_tables_of_thirty_tiles", "one_large_table_among_nine",
+                                  "ten_bit_digits"])
 def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
     """The plan sorts every table's indices on their own (fewer key bits); keys_sorted,
     positions_sorted and segment_starts must equal the stable sort of table_offsets[t] + index
@@ -149,6 +151,25 @@ def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
         p["n"] = int(p["offsets"][-1])
     elif case == "many_small_tables":
         p = make_problem(13, T=700, E=37, D=4, B=3, L=4, dtype=np.float32)
+    elif case == "eight_tables_of_thirty_tiles":
+        # many tables, every one of at most 48 sort tiles: the per-table count scan runs inside the
+        # scatter kernel
+        p = make_problem(16, T=8, E=0, D=4, B=3000, L=40, dtype=np.float32, ragged=False, zipf=1.1,
+                         rows=[70000, 300, 1 << 17, 5, 90000, 1000, 131071, 2])
+    elif case == "one_large_table_among_nine":
+        # one table of 63 tiles among small ones: the scan kernel with a workgroup per table runs
+        rs = np.random.RandomState(17)
+        T, B = 9, 3200
+        rows = [4000, 100, 50000, 1 << 17, 7, 900, 30000, 12, 65536]
+        lengths = np.full((T, B), 2)
+        lengths[3] = 80
+        offsets = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
+        indices = np.concatenate([rs.zipf(1.2, size=int(lengths[t].sum())) % rows[t] for t in range(T)])
+        p = dict(T=T, B=B, rows=rows, n=int(offsets[-1]), offsets=offsets, indices=indices.astype(np.int32),
+                 table_offsets=np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
+    elif case == "ten_bit_digits":
+        p = make_problem(18, T=8, E=0, D=4, B=2000, L=30, dtype=np.float32, zipf=1.05,
+                         rows=[1 << 20, 1000000, 999999, 1 << 19, 3, 1 << 20, 70, 524289])
     elif case == "multi_tile_tables":
         p = make_problem(14, T=3, E=0, D=4, B=1500, L=12, dtype=np.float32, zipf=1.1, rows=[1 << 17, 100, 300000])
     else:
