@@ -604,6 +604,36 @@ def compact(result):
             "parity": result["parity"]}
 
 
+def probe_bandwidth(torch):
+    """Context for the roofline fractions: what plain streaming kernels of the framework reach on
+    this GPU over a 3.2 GB fp32 array (the size of the configuration-3 table) -- copy (read +
+    write), fill (write), in-place add (read + write of the same lines), sum (read)."""
+    dev = torch.device("cuda:0")
+    n = 800_000_000
+    x = torch.empty(n, device=dev).normal_()
+    y = torch.empty_like(x)
+
+    def seconds(fn, iters=10):
+        fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / iters * 1e-3
+
+    b = n * 4
+    out = {"bytes": b,
+           "copy_GBps": 2 * b / seconds(lambda: y.copy_(x)) / 1e9,
+           "fill_GBps": b / seconds(lambda: y.fill_(1.0)) / 1e9,
+           "add_inplace_GBps": 2 * b / seconds(lambda: x.add_(1.0)) / 1e9,
+           "sum_GBps": b / seconds(lambda: x.sum()) / 1e9,
+           "hbm_peak_GBps": HBM_PEAK / 1e9}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -614,6 +644,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", action="store_true",
                     help="with the default configuration: leave out the compact records of configurations 2 and 4")
+    ap.add_argument("--probe-bandwidth", action="store_true",
+                    help="instead of a workload: bandwidth of plain copy / fill / add / sum kernels on 3.2 GB")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy 5 times, as the known-size "
                          "reference for rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
@@ -627,6 +659,8 @@ def main():
 
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
+    if args.probe_bandwidth:
+        return probe_bandwidth(torch)
     if args.config == 5:
         print(json.dumps(run_cached(args, make_workload(5))))
         return

@@ -82,6 +82,11 @@ struct UpdateArgs {
 };
 
 int segment_update(const UpdateArgs &args, hipStream_t stream);
+// The approximate row-wise Adagrad for rows of at most kShortSegment occurrences, with the
+// position-balanced tiles of the exact update (rows no wider than 64 vectors: approx_short_serves);
+// longer rows are appended to `queue` as unique-row numbers, their count in args.counters[1].
+bool approx_short_serves(int32_t dtype, int32_t D);
+int segment_update_approx_short(const UpdateArgs &args, int32_t *queue, hipStream_t stream);
 
 int key_bits_for(int64_t total_rows);
 void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *layout);

@@ -23,20 +23,11 @@
 
 #include <algorithm>
 
+#include "tbe_rowwise.h"
 #include "tbe_stages.h"
 
 namespace tbe {
 namespace {
-
-template <typename A> __device__ __forceinline__ A adagrad_multiplier(A state_new, float lr, float eps);
-// lr * (1.0 / (sqrt(s) + eps)) with the reference's types: float sqrt and add,
-// double reciprocal and product, rounded to float (tbe.cu:453-454).
-template <> __device__ __forceinline__ float adagrad_multiplier<float>(float s, float lr, float eps) {
-  return static_cast<float>(static_cast<double>(lr) * (1.0 / static_cast<double>(sqrtf(s) + eps)));
-}
-template <> __device__ __forceinline__ double adagrad_multiplier<double>(double s, float lr, float eps) {
-  return static_cast<double>(lr) * (1.0 / (sqrt(s) + static_cast<double>(eps)));
-}
 
 // Address of the row behind the u-th unique key: its slot in the HBM row cache when the
 // tables are cache-fronted and the row is resident, else its row in `weights`.
@@ -109,7 +100,12 @@ struct LongRecord {    // 16 bytes: a segment cut into several chunks
   int32_t u, key, first_partial, num_chunks;
 };
 
-template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL>
+// APPROX (row-wise Adagrad only): the approximate optimizer's per-lookup update
+// (batched_embedding_backward_adagrad_approx_kernel_1, tbe.cu:648-704) instead of one update with the
+// summed gradient -- every occurrence, in position order, adds its bag's ||grad||^2 (times its
+// squared weight) to the state and moves the row by its own multiplier.  Segments longer than
+// kShortSegment are then queued as unique-row numbers for tbe_approx.hip's wavefront-per-row kernel.
+template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL, bool APPROX = false>
 __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
@@ -119,10 +115,12 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     int32_t *__restrict__ counters, LongRecord *__restrict__ long_records,
     ChunkRecord *__restrict__ chunk_records, int64_t max_chunks, int64_t n, int64_t num_tiles,
     int64_t tiles_per_xcd, int D, int chunks_rt, float lr, float eps,
-    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr) {
+    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr,
+    int32_t *__restrict__ approx_long_queue) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
+  static_assert(!APPROX || OPT == kOptAdagrad, "the approximate update is a row-wise Adagrad");
 
   constexpr int kTilePositions = tile_positions(CHUNKS);
   constexpr int kStageCap = kTilePositions + kShortSegment;  // occurrences staged in LDS per wavefront
@@ -218,6 +216,12 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const int seg_end = s_bounds[wave][j + 1];
     const int len = seg_end - seg_begin;
     const int32_t key = s_keys[wave][j];
+    if constexpr (APPROX) {
+      if (len > kShortSegment) {
+        if (c == 0) approx_long_queue[atomicAdd(&counters[1], 1)] = u;
+        continue;
+      }
+    }
     if (len > kShortSegment) {
       // Hand the segment to the chunk queue.
       const int nch = (len + kChunkLen - 1) / kChunkLen;
@@ -273,6 +277,36 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
         w_raw = V::load_raw_streaming(wrow);
         if constexpr (OPT == kOptAdagrad) state_old = state[key];
       }
+      if constexpr (APPROX) {
+        // w_old is the row as the occurrences so far have left it, state_old the running state
+        if (i0 == seg_begin) w_old.unpack(w_raw);
+#pragma unroll
+        for (int q = 0; q < UNROLL; ++q) {
+          if (i0 + q < seg_end) {
+            V x;
+            x.unpack(raw[q]);
+            A local = A(0);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) local += x.v[i] * x.v[i];
+            const A gss = group_sum<CHUNKS, A>(local, chunks, group_base);
+            A pw = A(1);
+            if constexpr (WEIGHTED) pw = to_acc(pw_raw[q]);
+            state_old = state_old + (WEIGHTED ? gss * pw * pw : gss);
+            const A mult = approx_multiplier<A>(state_old, pw, WEIGHTED, lr, eps);
+            if constexpr (WEIGHTED) {
+              A dot = A(0);
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
+              dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
+              if (c == 0) grad_psw[pos[q]] = from_acc<T, A>(dot);
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) w_old.v[i] = w_old.v[i] - x.v[i] * mult;
+            round_trip<T, VEC>(w_old, rounding_of_update(sr, i0 + q - seg_begin), static_cast<int64_t>(key) * D + col);
+          }
+        }
+        continue;
+      }
       if constexpr (WEIGHTED) w_old.unpack(w_raw);
 #pragma unroll
       for (int q = 0; q < UNROLL; ++q) {
@@ -294,6 +328,12 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
           }
         }
       }
+    }
+    if constexpr (APPROX) {
+      // (fp16: the last update already rounded the row to the stored type, this conversion is exact)
+      if (c == 0) state[key] = state_old;
+      w_old.store_streaming(wrow);
+      continue;
     }
     w_old.unpack(w_raw);
     apply_update<T, VEC, CHUNKS, OPT, true>(wrow, w_old, G, state ? state + key : nullptr, state_old, lr,
@@ -673,7 +713,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
              go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
              a.segment_starts, a.segment_ids, a.counters, long_records, chunk_records, a.max_chunks,
              a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,
-             a.unique_slots, cr, a.stochastic_rounding);
+             a.unique_slots, cr, a.stochastic_rounding, static_cast<int32_t *>(nullptr));
 
   const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
   // a multiple of the XCD count, so that every XCD gets as many workgroups
@@ -691,6 +731,37 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, OPT>),
              grid_finish, block, w, st, a.counters, long_records, partial, a.D, g.chunks,
              a.learning_rate, a.eps, a.unique_slots, cr, a.stochastic_rounding);
+}
+
+// The short-row kernel alone, in its per-lookup (approximate Adagrad) form; rows of more than
+// kShortSegment occurrences are left in `queue` (their count in counters[1]).
+template <typename T, int VEC, int CHUNKS, bool WEIGHTED>
+void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *queue, hipStream_t stream) {
+  using A = typename AccOf<T>::type;
+  const int64_t num_tiles = ceil_div(a.num_indices, tile_positions(CHUNKS));
+  const int64_t tiles_per_xcd = ceil_div(ceil_div(num_tiles, kWavesPerBlock), kNumXcd);
+  const dim3 grid_short(static_cast<unsigned>(tiles_per_xcd * kNumXcd));
+  TBE_LAUNCH("update_approx_short", stream,
+             (update_short_kernel<T, VEC, CHUNKS, kOptAdagrad, WEIGHTED, kShortUnroll, true>), grid_short,
+             dim3(kBlockThreads), static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),
+             static_cast<A *>(a.optimizer_state), static_cast<const T *>(a.per_sample_weights),
+             static_cast<T *>(a.grad_per_sample_weights), a.keys_sorted, a.positions_sorted, a.grad_rows,
+             a.segment_starts, a.segment_ids, a.counters, static_cast<LongRecord *>(nullptr),
+             static_cast<ChunkRecord *>(nullptr), int64_t{0}, a.num_indices, num_tiles, tiles_per_xcd, a.D,
+             g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr), static_cast<T *>(nullptr),
+             a.stochastic_rounding, queue);
+}
+
+template <typename T, int VEC, bool WEIGHTED>
+void launch_approx_short_geometry(const UpdateArgs &a, const RowGeometry &g, int32_t *queue, hipStream_t stream) {
+  switch (g.tmpl) {
+    case 64: launch_approx_short<T, VEC, 64, WEIGHTED>(a, g, queue, stream); break;
+    case 32: launch_approx_short<T, VEC, 32, WEIGHTED>(a, g, queue, stream); break;
+    case 16: launch_approx_short<T, VEC, 16, WEIGHTED>(a, g, queue, stream); break;
+    case 8: launch_approx_short<T, VEC, 8, WEIGHTED>(a, g, queue, stream); break;
+    case 4: launch_approx_short<T, VEC, 4, WEIGHTED>(a, g, queue, stream); break;
+    default: launch_approx_short<T, VEC, 0, WEIGHTED>(a, g, queue, stream); break;
+  }
 }
 
 template <typename T, int VEC, int OPT, bool WEIGHTED>
@@ -731,6 +802,29 @@ void launch_variant(const UpdateArgs &a, const RowGeometry &g, hipStream_t strea
 }
 
 }  // namespace
+
+bool approx_short_serves(int32_t dtype, int32_t D) { return !row_geometry(dtype, D).wide; }
+
+int segment_update_approx_short(const UpdateArgs &a, int32_t *queue, hipStream_t stream) {
+  if (a.num_indices == 0) return TBE_OK;
+  const RowGeometry g = row_geometry(a.dtype, a.D);
+  const bool weighted = a.per_sample_weights != nullptr;
+#define TBE_APPROX_SHORT(TYPE, VECTOR)                                                        \
+  do {                                                                                       \
+    if (weighted) launch_approx_short_geometry<TYPE, VECTOR, true>(a, g, queue, stream);     \
+    else launch_approx_short_geometry<TYPE, VECTOR, false>(a, g, queue, stream);             \
+  } while (0)
+  switch (a.dtype) {
+    case TBE_DTYPE_F32: TBE_APPROX_SHORT(float, 4); break;
+    case TBE_DTYPE_F16:
+      if (g.vec == 8) TBE_APPROX_SHORT(__half, 8);
+      else TBE_APPROX_SHORT(__half, 4);
+      break;
+    default: TBE_APPROX_SHORT(double, 2); break;
+  }
+#undef TBE_APPROX_SHORT
+  return check_launch("tbe approximate Adagrad update (short rows)");
+}
 
 int segment_update(const UpdateArgs &a, hipStream_t stream) {
   if (a.num_indices == 0) return TBE_OK;
