@@ -17,7 +17,10 @@
  * tests/test_oracle.py; in short: forward / SGD / Adagrad against
  * torch.nn.EmbeddingBag + the Python optimizer of
  * test_table_batched_embeddings.py:184-193, 296-318 (golden fixture and live),
- * sort against numpy's stable argsort, segments against numpy.unique,
+ * approximate Adagrad against the same EmbeddingBag + Python optimizer with
+ * indices drawn without replacement (test_table_batched_embeddings.py:244),
+ * hand-computed repeated-row cases and a closed form for one row looked up
+ * n times, sort against numpy's stable argsort, segments against numpy.unique,
  * construct_offsets against its closed form, fp16 conversion against numpy's
  * float16 over all 65536 bit patterns.  The cache model restates this
  * repository's own specification (the reference has no cache): its parity is
