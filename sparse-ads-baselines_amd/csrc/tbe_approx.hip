@@ -32,6 +32,7 @@
 // only `row -= mult * grad` (and its rounding) remains a serial chain, fed by prefetched rows.
 
 #include <algorithm>
+#include <type_traits>
 
 #include "tbe_rowwise.h"
 #include "tbe_stages.h"
@@ -52,6 +53,41 @@ __device__ __forceinline__ int64_t broadcast_lane(int64_t v, int src) {
 }
 __device__ __forceinline__ double broadcast_lane(double v, int src) {
   return __longlong_as_double(broadcast_lane(static_cast<int64_t>(__double_as_longlong(v)), src));
+}
+
+// A value that is the same in every lane, moved to scalar registers.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int64_t uniform(int64_t v) {
+  const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
+  const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v >> 32)));
+  return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// v of the lane a data-parallel-primitive pattern selects, 0 where the pattern has no source lane
+// or the row mask leaves the lane out.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_or_zero(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
+}
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ double dpp_or_zero(double v) {
+  const int64_t bits = __double_as_longlong(v);
+  const uint32_t lo = static_cast<uint32_t>(
+      __builtin_amdgcn_update_dpp(0, static_cast<int>(bits), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
+  const uint32_t hi = static_cast<uint32_t>(
+      __builtin_amdgcn_update_dpp(0, static_cast<int>(bits >> 32), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
+  return __longlong_as_double(static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo));
+}
+
+// Inclusive prefix sum over the 64 lanes without a trip through LDS: shifts inside the rows of 16
+// lanes, then the last lane of row 0 / 2 added to row 1 / 3 and the last lane of row 1 to rows 2
+// and 3 (row_shr:n = 0x110 + n, row_bcast:15 = 0x142, row_bcast:31 = 0x143).
+template <typename A> __device__ __forceinline__ A wave_inclusive_sum(A x) {
+  x += dpp_or_zero<0x111, 0xf>(x);
+  x += dpp_or_zero<0x112, 0xf>(x);
+  x += dpp_or_zero<0x114, 0xf>(x);
+  x += dpp_or_zero<0x118, 0xf>(x);
+  x += dpp_or_zero<0x142, 0xa>(x);
+  x += dpp_or_zero<0x143, 0xc>(x);
+  return x;
 }
 
 // Sum over the `group` lanes (a power of two) around the caller; every lane gets the result.
@@ -266,144 +302,350 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
   }
 }
 
-// One wavefront per queued row.  Same arithmetic as approx_adagrad_kernel, except that the
-// running state of the 64 occurrences of a batch comes from a wavefront prefix sum instead of
-// dependent additions.  Per batch: bookkeeping one occurrence per lane, requested a batch ahead;
-// ||grad||^2 of the 64 gradient rows by all lane groups side by side; the 64 multipliers side by
-// side; then the serial `row -= mult * grad` walk by lane group 0, which requests the rows
-// (cache-resident by then) eight at a time.
+// ||grad||^2 (times the squared per-sample weight) of every lookup, by position: the addend of the
+// row state that the lookup's update starts with.  One lane group per bag reads the bag's gradient
+// row once and writes the value to the bag's positions, so the kernel below neither gathers a
+// gradient row twice nor forms a norm inside its serial walk.  Nothing reads the values when no
+// row was queued, and the kernel returns at once.
 template <typename T, int VEC, bool WEIGHTED, bool MIXED>
-__global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
-    const T *__restrict__ grad_output, T *__restrict__ weights,
-    typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw, T *__restrict__ grad_psw,
-    const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ positions_sorted,
-    const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ segment_starts,
-    const int32_t *__restrict__ counters, const int32_t *__restrict__ long_queue, int D, int group,
-    float lr, float eps, MixedTables mt, StochasticRounding sr) {
+__global__ __launch_bounds__(kBlockThreads) void approx_lookup_norms_kernel(
+    const T *__restrict__ grad_output, const T *__restrict__ psw, const int32_t *__restrict__ offsets,
+    const int32_t *__restrict__ counters, typename AccOf<T>::type *__restrict__ lookup_wss, int B,
+    int T_tables, int D, int group, MixedTables mt) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
-  using R = typename V::R;
-  constexpr int kRows = 8;  // gradient rows a lane group has in flight while the norms are formed
-  constexpr int batch_rows = kWave;
-  __shared__ A s_gss_all[kWavesPerBlock][kWave];
-
+  if (counters[1] == 0) return;
   const int lane = threadIdx.x & (kWave - 1);
-  A *s_gss = s_gss_all[threadIdx.x >> 6];
   const int r = lane / group;
   const int c = lane - r * group;
   const int groups = kWave / group;
-  const int num_long = counters[1];
-  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
-  const int64_t wave_stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
-
-  for (int64_t q = wave_id; q < num_long; q += wave_stride) {
-    const int u = long_queue[q];
-    const int seg_begin = segment_starts[u];
-    const int seg_end = segment_starts[u + 1];
-    const int64_t key = keys_sorted[seg_begin];
-    const RowPlace place = place_row<MIXED>(key, grad_rows[positions_sorted[seg_begin]], D, mt);
-    const int row_chunks = place.row_D / VEC;
-    const bool mine = c < row_chunks;
-    const bool owner = r == 0 && mine;  // lane group 0 holds the row
-    T *wrow = weights + place.row_element;
-    const int64_t col = static_cast<int64_t>(c) * VEC;
-    V w;
-    w.zero();
-    if (owner) w.load(wrow + col);
-    A s = state[key];
-
-    // bookkeeping of the first batch: one occurrence per lane
-    int cur_pos = positions_sorted[min(seg_begin + lane, seg_end - 1)];
-    int64_t cur_goff = grad_row_offset<MIXED>(grad_rows[cur_pos], place, mt);
-    A cur_pw = A(1);
-    if constexpr (WEIGHTED) cur_pw = to_acc(psw[cur_pos]);
-
-    for (int k0 = seg_begin; k0 < seg_end; k0 += batch_rows) {
-      const int nb = min(batch_rows, seg_end - k0);
-      // the next batch's bookkeeping is requested now and used one iteration later
-      const int nxt_pos = positions_sorted[min(k0 + batch_rows + lane, seg_end - 1)];
-      const int nxt_grow = grad_rows[nxt_pos];
-      A nxt_pw = A(1);
-      if constexpr (WEIGHTED) nxt_pw = to_acc(psw[nxt_pos]);
-
-      // gradient rows -> LDS, and ||grad||^2 of every occurrence: lane group r takes occurrences
-      // r, r + groups, ...
-      for (int j0 = 0; j0 < nb; j0 += groups * kRows) {
-        R raw[kRows];
+  const int64_t bags = static_cast<int64_t>(B) * T_tables;
+  const int64_t bag = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * groups + r;
+  const bool valid = bag < bags;
+  const int t = valid ? static_cast<int>(bag / B) : 0;
+  const int b = valid ? static_cast<int>(bag - static_cast<int64_t>(t) * B) : 0;
+  const int begin = valid ? offsets[bag] : 0;
+  const int end = valid ? offsets[bag + 1] : 0;
+  int row_D = D;
+  int64_t goff = (static_cast<int64_t>(b) * T_tables + t) * D;
+  if constexpr (MIXED) {
+    const int column0 = mt.dim_offsets[t];
+    row_D = mt.dim_offsets[t + 1] - column0;
+    goff = static_cast<int64_t>(b) * mt.total_D + column0;
+  }
+  const int row_chunks = end > begin ? row_D / VEC : 0;  // a bag without lookups needs no norm
+  A local = A(0);
+  for (int cb = c; cb < row_chunks; cb += group) {
+    V x;
+    x.load(grad_output + goff + static_cast<int64_t>(cb) * VEC);
 #pragma unroll
-        for (int x = 0; x < kRows; ++x) {
-          const int j = min(j0 + x * groups + r, nb - 1);
-          const int64_t goff = shfl_idx(cur_goff, j);
-          if (mine) raw[x] = V::load_raw(grad_output + goff + col);
-        }
-#pragma unroll
-        for (int x = 0; x < kRows; ++x) {
-          const int j = j0 + x * groups + r;
-          A local = A(0);
-          if (mine) {
-            V g;
-            g.unpack(raw[x]);
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) local += g.v[i] * g.v[i];
-          }
-          const A gss = group_sum_pow2<A>(local, group);
-          if (c == 0 && j < nb) s_gss[j] = gss;
-        }
-      }
-      __builtin_amdgcn_wave_barrier();
-      // running state and multiplier of every occurrence, one per lane
-      A wss = A(0);
-      if (lane < nb) {
-        const A gss = s_gss[lane];
-        wss = WEIGHTED ? gss * cur_pw * cur_pw : gss;
-      }
-      A incl = wss;
-#pragma unroll
-      for (int d = 1; d < kWave; d <<= 1) {
-        const A y = __shfl_up(incl, d, kWave);
-        if (lane >= d) incl += y;
-      }
-      const A my_mult = lane < nb ? approx_multiplier<A>(s + incl, cur_pw, WEIGHTED, lr, eps) : A(0);
-      s = s + broadcast_lane(incl, nb - 1);
-
-      // the row itself: one update after the other
-      for (int j0 = 0; j0 < nb; j0 += kBatch) {
-        R raw[kBatch];
-#pragma unroll
-        for (int b = 0; b < kBatch; ++b) {
-          const int64_t goff = broadcast_lane(cur_goff, min(j0 + b, nb - 1));
-          if (owner) raw[b] = V::load_raw(grad_output + goff + col);
-        }
-#pragma unroll
-        for (int b = 0; b < kBatch; ++b) {
-          const int j = j0 + b;
-          if (j >= nb) break;
-          const A mult = broadcast_lane(my_mult, j);
-          A dot = A(0);
-          if (owner) {
-            V g;
-            g.unpack(raw[b]);
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-              if constexpr (WEIGHTED) dot += w.v[i] * g.v[i];
-              w.v[i] = w.v[i] - g.v[i] * mult;
-            }
-            round_trip<T, VEC>(w, rounding_of_update(sr, k0 + j - seg_begin), place.row_element + col);
-          }
-          if constexpr (WEIGHTED) {
-            dot = group_sum_pow2<A>(dot, group);
-            const int pos = broadcast_lane(cur_pos, j);
-            if (lane == 0) grad_psw[pos] = from_acc<T, A>(dot);
-          }
-        }
-      }
-      __builtin_amdgcn_wave_barrier();  // the next batch overwrites the norms in LDS
-      cur_pos = nxt_pos;
-      cur_goff = grad_row_offset<MIXED>(nxt_grow, place, mt);
-      cur_pw = nxt_pw;
+    for (int i = 0; i < VEC; ++i) local += x.v[i] * x.v[i];
+  }
+  const A gss = group_sum_pow2<A>(local, group);
+  for (int p = begin + c; p < end; p += group) {
+    A wss = gss;
+    if constexpr (WEIGHTED) {
+      const A pw = to_acc(psw[p]);
+      wss = gss * pw * pw;
     }
-    if (lane == 0) state[key] = s;
-    if (owner) w.store(wrow + col);
+    lookup_wss[p] = wss;
+  }
+}
+
+// E consecutive elements of a row, loaded with one instruction of E * sizeof(T) bytes.
+template <typename T, int E> struct alignas(E * sizeof(T)) LanePack { T x[E]; };
+
+// The E values of a lane after they were stored in the weights' type and read again: nothing for
+// fp32 / fp64; fp16: round to nearest even, or, with stochastic rounding, element e takes word
+// e % 4 of the Philox block of elements 4 * (e / 4) ... (the rule of pack_rounded).
+template <typename T, int E, bool STOCHASTIC, typename A>
+__device__ __forceinline__ void round_lane_elements(A (&v)[E], const StochasticRounding &sr, int64_t element) {
+  if constexpr (sizeof(T) == 2) {
+    if constexpr (STOCHASTIC) {
+      constexpr int kBlocks = E >= 4 ? E / 4 : 1;
+#pragma unroll
+      for (int q = 0; q < kBlocks; ++q) {
+        const uint64_t block = static_cast<uint64_t>(element) / 4 + q;
+        const uint4 rnd = philox4x32_10(
+            make_uint4(static_cast<uint32_t>(block), static_cast<uint32_t>(block >> 32),
+                       static_cast<uint32_t>(sr.offset), static_cast<uint32_t>(sr.offset >> 32)),
+            make_uint2(static_cast<uint32_t>(sr.seed), static_cast<uint32_t>(sr.seed >> 32)));
+        const uint32_t word[4] = {rnd.x, rnd.y, rnd.z, rnd.w};
+        constexpr int kHere = E >= 4 ? 4 : E;
+        const int first = E >= 4 ? 0 : static_cast<int>(element & 3);  // (a multiple of E)
+#pragma unroll
+        for (int i = 0; i < kHere; ++i) {
+          uint32_t bits = word[0];
+#pragma unroll
+          for (int x = 1; x < 4; ++x) bits = (first + i == x) ? word[x] : bits;
+          A &value = v[4 * q + i];
+          value = __half2float(__float2half_rz(__uint_as_float(__float_as_uint(value) + (bits >> 19))));
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < E; ++i) v[i] = __half2float(__float2half_rn(v[i]));
+    }
+  }
+}
+
+template <typename T> struct LongRowArgs {
+  using A = typename AccOf<T>::type;
+  const T *grad_output;
+  T *weights;
+  A *state;
+  const T *psw;
+  T *grad_psw;
+  const int32_t *positions_sorted;
+  const int32_t *grad_rows;
+  const A *lookup_wss;
+  float lr, eps;
+  MixedTables mt;  // (T == 0: uniform tables)
+  StochasticRounding sr;
+  uint64_t grad_bytes;  // size of grad_output
+};
+
+// First element of gradient row `grad_row` for a row at `p` (mixed-D tables: mt.T > 0).
+__device__ __forceinline__ int64_t long_row_grad_offset(int grad_row, const RowPlace &p, const MixedTables &mt) {
+  if (mt.T > 0) return static_cast<int64_t>(grad_row / mt.T) * p.grad_stride + p.grad_column;
+  return static_cast<int64_t>(grad_row) * p.grad_stride;
+}
+
+// A LanePack read through a buffer descriptor: scalar byte offset of the row plus the lane's
+// byte offset, so that a row request is two instructions (a lane read and the load).
+template <typename P>
+__device__ __forceinline__ P buffer_load_pack(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_bytes, uint32_t row_bytes) {
+  P out;
+  if constexpr (sizeof(P) == 2) {
+    const uint16_t v = __builtin_amdgcn_raw_buffer_load_b16(rsrc, lane_bytes, row_bytes, 0);
+    __builtin_memcpy(&out, &v, 2);
+  } else if constexpr (sizeof(P) == 4) {
+    const uint32_t v = __builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_bytes, row_bytes, 0);
+    __builtin_memcpy(&out, &v, 4);
+  } else if constexpr (sizeof(P) == 8) {
+    const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_bytes, row_bytes, 0);
+    __builtin_memcpy(&out, &v, 8);
+  } else {
+    const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes, row_bytes, 0);
+    __builtin_memcpy(&out, &v, 16);
+  }
+  return out;
+}
+
+// The walk over one queued row by a whole wavefront: lane l owns elements [l * E, l * E + E) of
+// the row from the first to the last occurrence.  Occurrences are taken 64 at a time: their
+// bookkeeping (position, gradient row, per-sample weight, state addend) sits one per lane and is
+// requested two batches (positions: three) ahead; the running state of the 64 comes from a
+// wavefront prefix sum and their multipliers (a double-precision division each) are formed side
+// by side.  What remains serial is `row -= mult * grad` (and its rounding) per occurrence.  Its
+// gradient rows are requested well ahead, across batch boundaries, so that the chain does not
+// wait for memory: into a ring of 64 registers (64, 32 or 16 rows, by the bytes of a row that a
+// lane holds), each slot refilled as soon as it has been applied; with stochastic rounding, where the random bits
+// are most of the work per occurrence, 16 ahead into one of two sets of 16.
+template <typename T, int E, bool WEIGHTED, bool STOCHASTIC, bool BIG>
+__device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_begin, int seg_end, int64_t key,
+                                              const RowPlace &place, int lane) {
+  using A = typename AccOf<T>::type;
+  using P = LanePack<T, E>;
+  constexpr int kAhead = 16;
+  constexpr int kRing = STOCHASTIC ? 2 * kAhead : (E * sizeof(T) <= 4 ? kWave : E * sizeof(T) <= 8 ? kWave / 2 : kWave / 4);
+  const bool active = lane * E < place.row_D;
+  const int lane_off = active ? lane * E : 0;  // (idle lanes shadow lane 0 and store nothing)
+  T *wrow = a.weights + place.row_element + lane_off;
+  A w[E];
+  {
+    const P p = *reinterpret_cast<const P *>(wrow);
+#pragma unroll
+    for (int i = 0; i < E; ++i) w[i] = to_acc(p.x[i]);
+  }
+  A s = a.state[key];
+
+  // Bookkeeping, one occurrence per lane: this batch's and the next one's complete, the positions
+  // of the batch after that on their way.  Everything a batch needs was requested at least a
+  // whole batch earlier, so waiting for it never waits for the row requests behind it.
+  const int last = seg_end - 1;
+  int cur_pos = a.positions_sorted[min(seg_begin + lane, last)];
+  int nxt_pos = a.positions_sorted[min(seg_begin + kWave + lane, last)];
+  int aft_pos = a.positions_sorted[min(seg_begin + 2 * kWave + lane, last)];
+  // where a gradient row starts: its first element, or (grad_output below 4 GiB) its first byte
+  using Off = typename std::conditional<BIG, int64_t, int>::type;
+  auto offset_of = [&](int grad_row) {
+    const int64_t element = long_row_grad_offset(grad_row, place, a.mt);
+    if constexpr (BIG) return element;
+    else return static_cast<int>(static_cast<uint32_t>(element) * static_cast<uint32_t>(sizeof(T)));
+  };
+  Off cur_goff = offset_of(a.grad_rows[cur_pos]);
+  Off nxt_goff = offset_of(a.grad_rows[nxt_pos]);
+  A cur_pw = A(1), nxt_pw = A(1);
+  if constexpr (WEIGHTED) {
+    cur_pw = to_acc(a.psw[cur_pos]);
+    nxt_pw = to_acc(a.psw[nxt_pos]);
+  }
+  A cur_wss = a.lookup_wss[cur_pos];
+  A nxt_wss = a.lookup_wss[nxt_pos];
+  // (waited for here, before the first row requests)
+  asm volatile("" : "+v"(aft_pos), "+v"(nxt_goff), "+v"(nxt_pw), "+v"(nxt_wss) : : "memory");
+
+  const uint32_t lane_bytes = static_cast<uint32_t>(lane_off) * static_cast<uint32_t>(sizeof(T));
+  const __amdgpu_buffer_rsrc_t grad_buffer = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(a.grad_output), 0, static_cast<int>(static_cast<uint32_t>(BIG ? 0 : a.grad_bytes)), 0x00020000);
+  auto row_of = [&](Off goffs, int src_lane) {
+    if constexpr (BIG) return *reinterpret_cast<const P *>(a.grad_output + lane_off + broadcast_lane(goffs, src_lane));
+    else return buffer_load_pack<P>(grad_buffer, lane_bytes, static_cast<uint32_t>(broadcast_lane(goffs, src_lane)));
+  };
+  P ring[kRing];
+  {
+    const int nb = min(kWave, seg_end - seg_begin);
+    constexpr int kFirst = STOCHASTIC ? kAhead : kRing;
+#pragma unroll
+    for (int c = 0; c < kFirst; c += kAhead) {
+      if (c < nb) {
+#pragma unroll
+        for (int b = 0; b < kAhead; ++b) ring[c + b] = row_of(cur_goff, min(c + b, nb - 1));
+      }
+    }
+  }
+
+  for (int k0 = seg_begin; k0 < seg_end; k0 += kWave) {
+    const int nb = min(kWave, seg_end - k0);
+    const int nb_next = min(kWave, seg_end - k0 - kWave);  // <= 0: this is the last batch
+    // requested now, used from the next iteration on
+    const int aft_grow = a.grad_rows[aft_pos];
+    A aft_pw = A(1);
+    if constexpr (WEIGHTED) aft_pw = to_acc(a.psw[aft_pos]);
+    const A aft_wss = a.lookup_wss[aft_pos];
+    const int fut_pos = a.positions_sorted[min(k0 + 3 * kWave + lane, last)];
+
+    // running state and multiplier of every occurrence, one per lane
+    const A incl = wave_inclusive_sum<A>(lane < nb ? cur_wss : A(0));
+    const A my_mult = lane < nb ? approx_multiplier<A>(s + incl, cur_pw, WEIGHTED, a.lr, a.eps) : A(0);
+    s = s + broadcast_lane(incl, nb - 1);
+
+    // occurrence j of the batch, its gradient row in `grad`
+    auto apply = [&](const P &grad, int j) {
+      const A mult = broadcast_lane(my_mult, j);
+      A dot = A(0);
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const A g = to_acc(grad.x[i]);
+        if constexpr (WEIGHTED) dot += w[i] * g;
+        w[i] = w[i] - g * mult;
+      }
+      if constexpr (STOCHASTIC)
+        round_lane_elements<T, E, true, A>(w, rounding_of_update(a.sr, k0 + j - seg_begin),
+                                           place.row_element + lane_off);
+      else round_lane_elements<T, E, false, A>(w, a.sr, place.row_element + lane_off);
+      if constexpr (WEIGHTED) {
+        dot = active ? dot : A(0);
+#pragma unroll
+        for (int m = kWave / 2; m > 0; m >>= 1) dot += shfl_x(dot, m);
+        const int pos = broadcast_lane(cur_pos, j);
+        if (lane == 0) a.grad_psw[pos] = from_acc<T, A>(dot);
+      }
+    };
+
+    if constexpr (STOCHASTIC) {
+      // one block of 16 occurrences: request the block after it into `fill`, then apply `use`
+      auto block = [&](P *use, P *fill, int j0) {
+        Off src = cur_goff;
+        int first = 0, limit = 0;
+        if (j0 + kAhead < nb) {
+          first = j0 + kAhead;
+          limit = nb - 1;
+        } else if (nb_next > 0) {
+          src = nxt_goff;
+          limit = nb_next - 1;
+        }
+#pragma unroll
+        for (int b = 0; b < kAhead; ++b) fill[b] = row_of(src, min(first + b, limit));
+#pragma unroll
+        for (int b = 0; b < kAhead; ++b) {
+          if (j0 + b < nb) apply(use[b], j0 + b);
+        }
+      };
+      // blocks are taken in pairs so that the two register sets swap roles in place; the second
+      // block of a pair may find nothing left to apply and then only renews the request for the
+      // next batch's first rows
+      int j0 = 0;
+      do {  // (nb > 0)
+        block(ring, ring + kAhead, j0);
+        block(ring + kAhead, ring, j0 + kAhead);
+        j0 += 2 * kAhead;
+      } while (j0 < nb);
+    } else if (nb == kWave && nb_next == kWave) {
+      // a full batch followed by a full batch: straight-line code
+#pragma unroll
+      for (int j = 0; j < kWave; ++j) {
+        apply(ring[j % kRing], j);
+        if (j + kRing < kWave) ring[j % kRing] = row_of(cur_goff, j + kRing);
+        else ring[j % kRing] = row_of(nxt_goff, j + kRing - kWave);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kWave; ++j) {
+        if (j < nb) {
+          apply(ring[j % kRing], j);
+          const int target = (j + kRing) % kWave;  // occurrence j + kRing of the row ...
+          if (j + kRing < kWave) {                 // ... is in this batch
+            if (target < nb) ring[j % kRing] = row_of(cur_goff, target);
+          } else if (nb_next > 0) {                // ... or in the next one
+            ring[j % kRing] = row_of(nxt_goff, min(target, nb_next - 1));
+          }
+        }
+      }
+    }
+    cur_pos = nxt_pos;
+    cur_goff = nxt_goff;
+    cur_pw = nxt_pw;
+    cur_wss = nxt_wss;
+    nxt_pos = aft_pos;
+    nxt_goff = offset_of(aft_grow);
+    nxt_pw = aft_pw;
+    nxt_wss = aft_wss;
+    aft_pos = fut_pos;
+  }
+  if (lane == 0) a.state[key] = s;
+  if (active) {
+    P p;
+#pragma unroll
+    for (int i = 0; i < E; ++i) p.x[i] = from_acc<T, A>(w[i]);  // (fp16: already rounded, exact)
+    *reinterpret_cast<P *>(wrow) = p;
+  }
+}
+
+// One wavefront per queued row (a row of at most 64 vectors with more occurrences than the kernel
+// that queued it handles itself).  BIG: grad_output has 4 GiB or more, its rows are addressed
+// with 64-bit offsets instead of through a buffer descriptor.
+template <typename T, bool WEIGHTED, bool STOCHASTIC, bool BIG>
+__global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
+    LongRowArgs<T> a, const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
+    const int32_t *__restrict__ counters, const int32_t *__restrict__ long_queue, int D) {
+  // (what is the same in every lane of the wavefront is told to the compiler, so that the walk's
+  // control flow and addressing stay scalar)
+  const int lane = threadIdx.x & (kWave - 1);
+  const int num_long = uniform(counters[1]);
+  const int wave_id = uniform(static_cast<int>(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
+  const int wave_stride = static_cast<int>(gridDim.x) * kWavesPerBlock;
+  for (int q = wave_id; q < num_long; q += wave_stride) {
+    const int u = uniform(long_queue[q]);
+    const int seg_begin = uniform(segment_starts[u]);
+    const int seg_end = uniform(segment_starts[u + 1]);
+    const int64_t key = uniform(keys_sorted[seg_begin]);
+    const int first_grad_row = uniform(a.grad_rows[a.positions_sorted[seg_begin]]);
+    RowPlace place = a.mt.T > 0 ? place_row<true>(key, first_grad_row, D, a.mt)
+                                : place_row<false>(key, first_grad_row, D, a.mt);
+    place.row_D = uniform(place.row_D);
+    place.row_element = uniform(place.row_element);
+    place.grad_stride = uniform(place.grad_stride);
+    place.grad_column = uniform(place.grad_column);
+    // elements per lane: the row spread over the 64 lanes, in loads of at most 16 bytes
+    const int per_lane = (place.row_D + kWave - 1) / kWave;
+    if (per_lane <= 1) walk_long_row<T, 1, WEIGHTED, STOCHASTIC, BIG>(a, seg_begin, seg_end, key, place, lane);
+    else if (per_lane <= 2) walk_long_row<T, 2, WEIGHTED, STOCHASTIC, BIG>(a, seg_begin, seg_end, key, place, lane);
+    else if constexpr (sizeof(T) <= 4) {
+      if (per_lane <= 4) walk_long_row<T, 4, WEIGHTED, STOCHASTIC, BIG>(a, seg_begin, seg_end, key, place, lane);
+      else if constexpr (sizeof(T) == 2) walk_long_row<T, 8, WEIGHTED, STOCHASTIC, BIG>(a, seg_begin, seg_end, key, place, lane);
+    }
   }
 }
 
@@ -420,6 +662,8 @@ struct ApproxArgs {
   float lr, eps;
   MixedTables mt;
   StochasticRounding sr;
+  const int32_t *offsets;  // [T * B + 1] first position of every bag
+  int32_t B, T;
 };
 
 template <typename T, int VEC>
@@ -446,23 +690,41 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
   const dim3 grid_long(static_cast<unsigned>(
       std::max<int64_t>(1, std::min<int64_t>(ceil_div(most_long, kWavesPerBlock), 256 * 8))));
   const dim3 block_long(kBlockThreads);
+  // the queued rows' kernel reads the state addend of every lookup from the sort's ping-pong
+  // buffers (8 bytes per lookup, free once the batch is sorted)
+  A *lookup_wss = reinterpret_cast<A *>(ws + l.sort_scratch);
+  const int64_t bags = static_cast<int64_t>(a.B) * a.T;
+  const dim3 grid_norms(static_cast<unsigned>(ceil_div(ceil_div(bags, groups), kWavesPerBlock)));
+  const uint64_t grad_bytes = static_cast<uint64_t>(a.B) * (mixed ? a.mt.total_D : static_cast<int64_t>(a.T) * a.D) * sizeof(T);
+  MixedTables long_tables = a.mt;
+  if (!mixed) long_tables.T = 0;
+  LongRowArgs<T> la{static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights), static_cast<A *>(a.state),
+                    static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw), i32(l.positions_sorted),
+                    i32(l.grad_rows), lookup_wss, a.lr, a.eps, long_tables, a.sr, grad_bytes};
+  const bool big = grad_bytes >= (1ull << 32);
+  const bool stochastic = sizeof(T) == 2 && a.sr.enabled;
+#define TBE_APPROX_LONG_KERNEL(WEIGHTED, STOCHASTIC, BIG)                                              \
+  TBE_LAUNCH("update_approx_long", stream, (approx_adagrad_long_kernel<T, WEIGHTED, STOCHASTIC, BIG>), \
+             grid_long, block_long, la, i32(l.keys_sorted), i32(l.segment_starts), counters,           \
+             long_queue, a.D)
+#define TBE_APPROX_LONG(WEIGHTED, MIXED)                                                               \
+  TBE_LAUNCH("update_approx_norms", stream, (approx_lookup_norms_kernel<T, VEC, WEIGHTED, MIXED>),     \
+             grid_norms, block, static_cast<const T *>(a.grad_output), static_cast<const T *>(a.psw),  \
+             a.offsets, counters, lookup_wss, a.B, a.T, a.D, group, a.mt);                             \
+  if (stochastic) {                                                                                    \
+    if (big) { TBE_APPROX_LONG_KERNEL(WEIGHTED, sizeof(T) == 2, true); }                               \
+    else { TBE_APPROX_LONG_KERNEL(WEIGHTED, sizeof(T) == 2, false); }                                  \
+  } else {                                                                                             \
+    if (big) { TBE_APPROX_LONG_KERNEL(WEIGHTED, false, true); }                                        \
+    else { TBE_APPROX_LONG_KERNEL(WEIGHTED, false, false); }                                           \
+  }
 #define TBE_APPROX(WEIGHTED, MIXED)                                                                    \
   TBE_LAUNCH("update_approx", stream, (approx_adagrad_kernel<T, VEC, WEIGHTED, MIXED>), grid, block,   \
              static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),                       \
              static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),   \
              i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),     \
              counters, long_queue, a.D, group, a.lr, a.eps, a.mt, a.sr);                               \
-  TBE_LAUNCH("update_approx_long", stream, (approx_adagrad_long_kernel<T, VEC, WEIGHTED, MIXED>),      \
-             grid_long, block_long, static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights), \
-             static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),   \
-             i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),     \
-             counters, long_queue, a.D, group, a.lr, a.eps, a.mt, a.sr)
-#define TBE_APPROX_LONG(WEIGHTED)                                                                      \
-  TBE_LAUNCH("update_approx_long", stream, (approx_adagrad_long_kernel<T, VEC, WEIGHTED, false>),      \
-             grid_long, block_long, static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights), \
-             static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),   \
-             i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),     \
-             counters, long_queue, a.D, group, a.lr, a.eps, a.mt, a.sr)
+  TBE_APPROX_LONG(WEIGHTED, MIXED)
   if (mixed) {
     if (a.psw) { TBE_APPROX(true, true); }
     else { TBE_APPROX(false, true); }
@@ -490,13 +752,14 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
     ua.eps = a.eps;
     ua.stochastic_rounding = a.sr;
     (void)segment_update_approx_short(ua, long_queue, stream);
-    if (a.psw) { TBE_APPROX_LONG(true); }
-    else { TBE_APPROX_LONG(false); }
+    if (a.psw) { TBE_APPROX_LONG(true, false); }
+    else { TBE_APPROX_LONG(false, false); }
   } else {
     if (a.psw) { TBE_APPROX(true, false); }
     else { TBE_APPROX(false, false); }
   }
 #undef TBE_APPROX_LONG
+#undef TBE_APPROX_LONG_KERNEL
 #undef TBE_APPROX
 }
 
@@ -507,10 +770,10 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
 int approx_update(const void *grad_output, void *weights, void *state, const void *psw, void *grad_psw,
                   int32_t dtype, int32_t fp16_vector_width, int32_t D, int64_t n, float lr, float eps,
                   const int64_t *mixed_table_offsets, const int32_t *table_dim_offsets,
-                  const int32_t *dim_offsets, int32_t total_D, int32_t T, StochasticRounding sr,
-                  const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream) {
+                  const int32_t *dim_offsets, int32_t total_D, int32_t T, const int32_t *offsets, int32_t B,
+                  StochasticRounding sr, const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream) {
   ApproxArgs a{grad_output, weights, state, psw, grad_psw, dtype, fp16_vector_width, D, n, lr, eps,
-               MixedTables{mixed_table_offsets, table_dim_offsets, dim_offsets, total_D, T}, sr};
+               MixedTables{mixed_table_offsets, table_dim_offsets, dim_offsets, total_D, T}, sr, offsets, B, T};
   char *ws = static_cast<char *>(workspace);
   switch (dtype) {
     case TBE_DTYPE_F32: launch_approx<float, 4>(a, l, ws, stream); break;
@@ -561,7 +824,7 @@ extern "C" int tbe_backward_approx_adagrad(const void *grad_output, void *weight
     return rc;
   const RowGeometry g = row_geometry(dtype, D);
   return approx_update(grad_output, weights, optimizer_state, per_sample_weights, grad_per_sample_weights,
-                       dtype, g.vec, D, num_indices, learning_rate, eps, nullptr, nullptr, nullptr, 0, T,
+                       dtype, g.vec, D, num_indices, learning_rate, eps, nullptr, nullptr, nullptr, 0, T, offsets, B,
                        StochasticRounding{seed, offset, (stochastic_rounding && dtype == TBE_DTYPE_F16) ? 1 : 0},
                        l, workspace, s);
 }

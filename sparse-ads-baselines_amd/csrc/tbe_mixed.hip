@@ -954,7 +954,7 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   if (optimizer == TBE_OPT_APPROX_ROWWISE_ADAGRAD)
     return approx_update(grad_output, weights, optimizer_state, per_sample_weights, grad_per_sample_weights,
                          dtype, dtype == TBE_DTYPE_F16 ? a.vec : (dtype == TBE_DTYPE_F32 ? 4 : 2), 0, num_indices,
-                         learning_rate, eps, table_offsets, table_dim_offsets, dim_offsets, total_D, T, a.sr, l,
+                         learning_rate, eps, table_offsets, table_dim_offsets, dim_offsets, total_D, T, offsets, B, a.sr, l,
                          workspace, s);
   switch (dtype) {
     case TBE_DTYPE_F32: launch_update_mixed_variant<float, 4>(a, l, ws, s); break;

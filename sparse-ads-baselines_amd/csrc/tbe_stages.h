@@ -102,8 +102,8 @@ int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int3
 int approx_update(const void *grad_output, void *weights, void *state, const void *psw, void *grad_psw,
                   int32_t dtype, int32_t fp16_vector_width, int32_t D, int64_t n, float lr, float eps,
                   const int64_t *mixed_table_offsets, const int32_t *table_dim_offsets,
-                  const int32_t *dim_offsets, int32_t total_D, int32_t T, StochasticRounding sr,
-                  const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream);
+                  const int32_t *dim_offsets, int32_t total_D, int32_t T, const int32_t *offsets, int32_t B,
+                  StochasticRounding sr, const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream);
 
 // Copies the rows that tbe_cache_prepare staged for this step back to the backing table.
 int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int32_t *keys_sorted,

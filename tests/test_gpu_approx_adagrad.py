@@ -87,6 +87,88 @@ def test_approx_adagrad_hot_row_and_long_bags(oracle):
     assert_close(g, g_ref, 1e-4)  # dot products of rows that 17 k fp32 updates have moved
 
 
+@pytest.mark.parametrize("dtype,D", [(np.float32, 8), (np.float32, 64), (np.float32, 128), (np.float32, 200),
+                                     (np.float32, 256), (np.float16, 64), (np.float16, 100), (np.float16, 256),
+                                     (np.float16, 512), (np.float64, 64), (np.float64, 128)])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_approx_adagrad_rows_of_many_occurrences_in_every_lane_layout(oracle, dtype, D, weighted):
+    """Rows with more than 16 occurrences get a wavefront each, whose lanes hold 1, 2, 4 or 8 elements of
+    the row and which takes the occurrences 64 at a time.  The run lengths drawn here end inside the first
+    batch, on a batch boundary, one past it and several batches on, in blocks of every parity."""
+    rs = np.random.RandomState(36)
+    lengths = [17, 31, 32, 33, 48, 49, 63, 64, 65, 80, 96, 127, 128, 129, 200, 333]
+    T, E, L = 2, 40, 8
+    B = (sum(lengths) + 120 + L - 1) // L
+    p = make_problem(36, T=T, E=E, D=D, B=B, L=L, dtype=dtype, ragged=False, weighted=weighted)
+    for t in range(T):
+        rows = np.concatenate([np.full(n, r, np.int32) for r, n in enumerate(lengths)])
+        rest = rs.randint(len(lengths), E, size=B * L - rows.size).astype(np.int32)
+        p["indices"][t * B * L:(t + 1) * B * L] = rs.permutation(np.concatenate([rows, rest]))
+    state0 = rs.uniform(0, 2, size=p["weights"].shape[0]).astype(np.float64 if dtype == np.float64 else np.float32)
+    w, st, g = _run_gpu(p, 0.01, 0.1, state0)
+    w_ref, st_ref, g_ref = _run_oracle(oracle, p, 0.01, 0.1, state0)
+    tol = TOL[np.dtype(dtype)]
+    assert_close(st, st_ref, 1e-5 if dtype != np.float64 else 1e-10, "state")
+    assert_close(w, w_ref, tol, "weights")
+    if weighted:
+        assert_close(g, g_ref, tol if dtype != np.float16 else 2e-2, "grad of per-sample weights")
+
+
+@pytest.mark.timeout(300)
+def test_approx_adagrad_with_a_gradient_tensor_beyond_4GiB():
+    """Below 4 GiB the wavefront-per-row kernel addresses gradient rows through a buffer descriptor with
+    32-bit offsets, from 4 GiB on with 64-bit addresses.  A batch whose few non-empty bags are spread over a
+    4.3 GB grad_output must come out bit for bit like the same bags packed into a small one."""
+    B, T, D, E, L = 1 << 16, 64, 256, 50, 8
+    t_used, bags = 37, 300
+    rs = np.random.RandomState(38)
+    gen = torch.Generator(device=DEV).manual_seed(38)
+    grad_big = torch.randn(B, T, D, device=DEV, generator=gen)
+    assert grad_big.numel() * 4 >= 1 << 32
+    chosen = np.sort(np.concatenate([rs.choice(B - 2, bags - 2, replace=False), [B - 2, B - 1]])).astype(np.int64)
+    idx = rs.randint(0, E, size=(bags, L)).astype(np.int32)
+    idx[rs.rand(bags, L) < 0.7] = 3
+    lengths = np.zeros((T, B), np.int64)
+    lengths[t_used, chosen] = L
+    offsets_big = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
+    weights = rs.uniform(-0.01, 0.01, size=(T * E, D)).astype(np.float32)
+    table_offsets = (np.arange(T) * E).astype(np.int32)
+
+    def run(grad, table_offsets, offsets, w):
+        st = torch.zeros(w.shape[0], dtype=torch.float32, device=DEV)
+        ext.backward_approx_adagrad(grad, w, dev(table_offsets), dev(idx.reshape(-1)), dev(offsets), None, st, 0.01,
+                                    0.1, 200, False, 1)
+        torch.cuda.synchronize()
+        return w.cpu().numpy(), st.cpu().numpy()
+
+    w_big, st_big = run(grad_big, table_offsets, offsets_big, dev(weights))
+    grad_small = grad_big[torch.from_numpy(chosen).to(DEV), t_used].reshape(bags, 1, D).contiguous()
+    del grad_big
+    rows = slice(t_used * E, (t_used + 1) * E)
+    w_small, st_small = run(grad_small, np.zeros(1, np.int32), (np.arange(bags + 1) * L).astype(np.int32),
+                            dev(weights[rows]))
+    assert st_big[rows].tobytes() == st_small.tobytes()
+    assert w_big[rows].tobytes() == w_small.tobytes()
+    assert st_big[3 + t_used * E] > 0 and np.bincount(idx.reshape(-1)).max() > 1500
+    untouched = np.ones(T * E, bool)
+    untouched[rows] = False
+    assert w_big[untouched].tobytes() == weights[untouched].tobytes()
+
+
+def test_approx_adagrad_stochastic_rounding_of_rows_of_many_occurrences(oracle):
+    """The k-th update of a hot row draws the oracle's random words in the wavefront-per-row kernel too."""
+    p = make_problem(37, T=2, E=12, D=64, B=64, L=10, dtype=np.float16, ragged=False, weighted=False, zipf=1.5)
+    assert np.bincount(p["indices"][:640]).max() > 130
+    torch.manual_seed(99)
+    gen = torch.cuda.default_generators[0]
+    seed, offset = gen.initial_seed() & 0xFFFFFFFFFFFFFFFF, gen.get_offset()
+    w, st, _ = _run_gpu(p, 0.05, 0.1, stochastic=True)
+    w_ref, st_ref, _ = _run_oracle(oracle, p, 0.05, 0.1, stochastic_rounding=(seed, offset))
+    assert_close(st, st_ref, 1e-5)
+    assert (w.view(np.uint16) != w_ref.view(np.uint16)).mean() < 0.05
+    assert_close(w, w_ref, 1e-2)
+
+
 def test_approx_adagrad_stochastic_rounding_matches_oracle_stream(oracle):
     p = make_problem(34, T=2, E=25, D=32, B=60, L=6, dtype=np.float16, weighted=False, zipf=1.2)
     torch.manual_seed(1234)
