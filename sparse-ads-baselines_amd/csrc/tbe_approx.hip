@@ -142,7 +142,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ positions_sorted,
     const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ segment_starts,
     int32_t *__restrict__ counters, int32_t *__restrict__ long_queue, int D, int group, float lr,
-    float eps, MixedTables mt, StochasticRounding sr) {
+    float eps, MixedTables mt, StochasticRounding sr, const int32_t *__restrict__ only_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -152,7 +152,8 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
   const int c = lane - r * group;
   const int group_base = r * group;
   const int groups = kWave / group;
-  const int U = counters[0];
+  // every unique row, or (only_rows) the rows another kernel has left in a queue of counters[2] entries
+  const int U = only_rows ? counters[2] : counters[0];
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t wave_stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
   const int batch = group < kBatch ? group : kBatch;  // one lane of the group fetches one occurrence's bookkeeping
@@ -165,9 +166,11 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
     const int rows_here = static_cast<int>(min(static_cast<int64_t>(kWave), U - strip));
     int lane_begin = 0, lane_end = 0, lane_key = 0, lane_pos0 = 0, lane_grow0 = 0;
     A lane_state = A(0), lane_pw0 = A(1);
+    int lane_u = static_cast<int>(strip) + lane;
     if (lane < rows_here) {
-      lane_begin = segment_starts[strip + lane];
-      lane_end = segment_starts[strip + lane + 1];
+      if (only_rows) lane_u = only_rows[strip + lane];
+      lane_begin = segment_starts[lane_u];
+      lane_end = segment_starts[lane_u + 1];
       lane_key = keys_sorted[lane_begin];
       lane_pos0 = positions_sorted[lane_begin];
       lane_state = state[lane_key];
@@ -177,7 +180,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
   for (int i0 = 0; i0 < rows_here; i0 += groups) {
     const bool valid = i0 + r < rows_here;
     const int src = valid ? i0 + r : 0;
-    const int64_t u = strip + src;
+    const int64_t u = shfl_idx(lane_u, src);
     const int seg_begin = shfl_idx(lane_begin, src);
     int seg_end = shfl_idx(lane_end, src);
     if (!valid) seg_end = seg_begin;
@@ -664,6 +667,9 @@ struct ApproxArgs {
   StochasticRounding sr;
   const int32_t *offsets;  // [T * B + 1] first position of every bag
   int32_t B, T;
+  // mixed-D tables: the rows of at most 64 vectors and kMixedShort occurrences are done and the
+  // longer ones queued (update_mixed_approx_short); this queue holds the rows wider than 64 vectors
+  const int32_t *wide_rows;
 };
 
 template <typename T, int VEC>
@@ -723,7 +729,7 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
              static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),                       \
              static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),   \
              i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),     \
-             counters, long_queue, a.D, group, a.lr, a.eps, a.mt, a.sr);                               \
+             counters, long_queue, a.D, group, a.lr, a.eps, a.mt, a.sr, a.wide_rows);                  \
   TBE_APPROX_LONG(WEIGHTED, MIXED)
   if (mixed) {
     if (a.psw) { TBE_APPROX(true, true); }
@@ -773,7 +779,8 @@ int approx_update(const void *grad_output, void *weights, void *state, const voi
                   const int32_t *dim_offsets, int32_t total_D, int32_t T, const int32_t *offsets, int32_t B,
                   StochasticRounding sr, const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream) {
   ApproxArgs a{grad_output, weights, state, psw, grad_psw, dtype, fp16_vector_width, D, n, lr, eps,
-               MixedTables{mixed_table_offsets, table_dim_offsets, dim_offsets, total_D, T}, sr, offsets, B, T};
+               MixedTables{mixed_table_offsets, table_dim_offsets, dim_offsets, total_D, T}, sr, offsets, B, T,
+               D == 0 ? approx_mixed_wide_queue(l, workspace) : nullptr};
   char *ws = static_cast<char *>(workspace);
   switch (dtype) {
     case TBE_DTYPE_F32: launch_approx<float, 4>(a, l, ws, stream); break;

@@ -18,6 +18,7 @@
 #include <algorithm>
 #include <type_traits>
 
+#include "tbe_rowwise.h"
 #include "tbe_stages.h"
 
 namespace tbe {
@@ -425,7 +426,13 @@ template <typename X> __device__ __forceinline__ void register_fence(X &x) {
 
 constexpr int kMixedShort = 8;
 constexpr int kMixedAhead = 4;
-template <typename T, int VEC, int OPT, bool WEIGHTED>
+// APPROX (row-wise Adagrad only): the approximate update's per-lookup form -- every occurrence adds
+// its bag's ||grad||^2 (times its squared weight) to the row's state and moves the row by its own
+// multiplier, one occurrence after the other in position order, the row rounded to the weights'
+// type every time (the arithmetic of approx_adagrad_kernel).  Rows of more than kMixedShort
+// occurrences then go to ONE queue (`huge_rows`, counters[1]) whatever their length, and rows wider
+// than 64 vectors to the other (`long_rows`, counters[2]).
+template <typename T, int VEC, int OPT, bool WEIGHTED, bool APPROX = false>
 __global__ __launch_bounds__(kBlockThreads, (WEIGHTED || VEC == 8) ? 4 : 5) void update_mixed_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
@@ -483,8 +490,10 @@ __global__ __launch_bounds__(kBlockThreads, (WEIGHTED || VEC == 8) ? 4 : 5) void
 
     // hand the longer rows of the strip to their queues (one atomic per strip and queue);
     // rows wider than 64 vectors count as longer rows whatever their length
-    const bool is_huge = lane < rows_here && l_end - l_begin > kChunkLen;
-    const bool is_long = lane < rows_here && (l_end - l_begin > kMixedShort || l_D / VEC > kWave);
+    const bool is_wide = l_D / VEC > kWave;
+    const bool is_huge = lane < rows_here && (APPROX ? (l_end - l_begin > kMixedShort && !is_wide)
+                                                     : l_end - l_begin > kChunkLen);
+    const bool is_long = lane < rows_here && (l_end - l_begin > kMixedShort || is_wide);
     const unsigned long long long_mask = __ballot(is_long);
     const unsigned long long huge_mask = __ballot(is_huge);
     const unsigned long long medium_mask = long_mask & ~huge_mask;
@@ -604,12 +613,35 @@ __global__ __launch_bounds__(kBlockThreads, (WEIGHTED || VEC == 8) ? 4 : 5) void
         for (int i = 0; i < VEC; ++i) w_old.v[i] = active ? w_old.v[i] : A(0);
       }
       G.zero();
+      A running = state_old;  // APPROX: the row's state after the occurrences applied so far
       auto add = [&](int u, const R &packed, A weight) {
         x.unpack(packed);
         const bool ok = u < len && active;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) x.v[i] = ok ? x.v[i] : A(0);
-        if constexpr (WEIGHTED) {
+        if constexpr (APPROX) {
+          // w_old is the row as the earlier occurrences left it
+          A gss = A(0);
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) gss += x.v[i] * x.v[i];
+          for (int m = group_lanes >> 1; m > 0; m >>= 1) gss += shfl_x(gss, m);
+          A mult = A(0);
+          if (u < len) {
+            if constexpr (!WEIGHTED) weight = A(1);
+            running = running + (WEIGHTED ? gss * weight * weight : gss);
+            mult = approx_multiplier<A>(running, weight, WEIGHTED, lr, eps);
+          }
+          if constexpr (WEIGHTED) {
+            A dot = A(0);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
+            for (int m = group_lanes >> 1; m > 0; m >>= 1) dot += shfl_x(dot, m);
+            if (u < len && c == 0) grad_psw[s_pos[wave][slot0 + u]] = from_acc<T, A>(dot);
+          }
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) w_old.v[i] = w_old.v[i] - x.v[i] * mult;
+          round_trip<T, VEC>(w_old, rounding_of_update(sr, u), row_element + col);
+        } else if constexpr (WEIGHTED) {
           weight = ok ? weight : A(1);
           A dot = A(0);
 #pragma unroll
@@ -642,6 +674,12 @@ __global__ __launch_bounds__(kBlockThreads, (WEIGHTED || VEC == 8) ? 4 : 5) void
         }
 #pragma unroll
         for (int u = 0; u < kMixedAhead; ++u) add(i0 + u, raw[u], pw[u]);
+      }
+      if constexpr (APPROX) {
+        if (len > 0 && c == 0) state[key] = running;
+        // (fp16: the last occurrence already rounded the row to the stored type)
+        if (len > 0 && active) w_old.store_streaming(weights + row_element + col);
+        return;
       }
       A mult = static_cast<A>(lr);
       if constexpr (OPT == kOptAdagrad) {
@@ -821,6 +859,34 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
              i32(l.segment_starts), i32(l.num_unique), 1, huge_rows, a.lr, a.eps, a.sr);
 }
 
+// The approximate update's strip kernel: rows of at most 64 vectors and kMixedShort occurrences
+// are applied, the others queued for approx_update.
+template <typename T, int VEC, bool WEIGHTED>
+void launch_update_mixed_approx(const MixedArgs &a, const tbe_workspace_layout_t &l, char *ws, hipStream_t stream) {
+  using A = typename AccOf<T>::type;
+  auto i32 = [&](uint64_t off) { return reinterpret_cast<int32_t *>(ws + off); };
+  const int64_t want = ceil_div(ceil_div(a.n, kWave), kWavesPerBlock);
+  const dim3 grid(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want, 256 * 32))));
+  int log2_T = 0;
+  while ((int64_t{1} << log2_T) < a.T) ++log2_T;
+  const int bag_shift = 31 + log2_T;
+  const uint32_t bag_magic =
+      static_cast<uint32_t>(((uint64_t{1} << bag_shift) + static_cast<uint64_t>(a.T) - 1) / static_cast<uint64_t>(a.T));
+  TBE_LAUNCH("update_mixed_approx", stream, (update_mixed_kernel<T, VEC, kOptAdagrad, WEIGHTED, true>), grid,
+             dim3(kBlockThreads), static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),
+             static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),
+             a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, bag_magic, bag_shift, a.total_D,
+             i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
+             i32(l.num_unique), approx_mixed_wide_queue(l, ws), approx_mixed_long_queue(l, ws), a.lr, a.eps, a.sr);
+}
+
+template <typename T, int VEC>
+void launch_update_mixed_approx_variant(const MixedArgs &a, const tbe_workspace_layout_t &l, char *ws,
+                                        hipStream_t stream) {
+  if (a.psw) launch_update_mixed_approx<T, VEC, true>(a, l, ws, stream);
+  else launch_update_mixed_approx<T, VEC, false>(a, l, ws, stream);
+}
+
 template <typename T, int VEC>
 void launch_update_mixed_variant(const MixedArgs &a, const tbe_workspace_layout_t &l, char *ws,
                                  hipStream_t stream) {
@@ -951,11 +1017,20 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   rc = find_segments(i32(l.keys_sorted), num_indices, i32(l.segment_starts), i32(l.num_unique), nullptr,
                      ws + l.segment_scratch, s, /*clear_queue_counters=*/true);
   if (rc) return rc;
-  if (optimizer == TBE_OPT_APPROX_ROWWISE_ADAGRAD)
+  if (optimizer == TBE_OPT_APPROX_ROWWISE_ADAGRAD) {
+    switch (dtype) {
+      case TBE_DTYPE_F32: launch_update_mixed_approx_variant<float, 4>(a, l, ws, s); break;
+      case TBE_DTYPE_F16:
+        if (a.vec == 8) launch_update_mixed_approx_variant<__half, 8>(a, l, ws, s);
+        else launch_update_mixed_approx_variant<__half, 4>(a, l, ws, s);
+        break;
+      default: launch_update_mixed_approx_variant<double, 2>(a, l, ws, s); break;
+    }
     return approx_update(grad_output, weights, optimizer_state, per_sample_weights, grad_per_sample_weights,
                          dtype, dtype == TBE_DTYPE_F16 ? a.vec : (dtype == TBE_DTYPE_F32 ? 4 : 2), 0, num_indices,
                          learning_rate, eps, table_offsets, table_dim_offsets, dim_offsets, total_D, T, offsets, B, a.sr, l,
                          workspace, s);
+  }
   switch (dtype) {
     case TBE_DTYPE_F32: launch_update_mixed_variant<float, 4>(a, l, ws, s); break;
     case TBE_DTYPE_F16:

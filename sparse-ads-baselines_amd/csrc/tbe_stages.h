@@ -98,12 +98,24 @@ int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int3
 
 // The approximate row-wise Adagrad update (one lookup at a time per row, in position order) on a
 // workspace that holds the batch's plan.  Uniform tables: D > 0 and the mixed_* pointers null;
-// mixed-D tables: D = 0.
+// mixed-D tables: D = 0, and the strip kernel of tbe_backward_mixed has already applied the rows
+// of few occurrences and filled the two queues above.
 int approx_update(const void *grad_output, void *weights, void *state, const void *psw, void *grad_psw,
                   int32_t dtype, int32_t fp16_vector_width, int32_t D, int64_t n, float lr, float eps,
                   const int64_t *mixed_table_offsets, const int32_t *table_dim_offsets,
                   const int32_t *dim_offsets, int32_t total_D, int32_t T, const int32_t *offsets, int32_t B,
                   StochasticRounding sr, const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream);
+
+// Where the approximate update of mixed-D tables keeps its two queues of unique-row indices inside
+// the backward workspace: rows of at most 64 vectors with more occurrences than the strip kernel
+// applies itself (counted in counters[1]; the queue approx_update's wavefront-per-row kernel
+// drains), and rows wider than 64 vectors (counters[2]).
+inline int32_t *approx_mixed_long_queue(const tbe_workspace_layout_t &l, void *workspace) {
+  return reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + l.chunk_segments);
+}
+inline int32_t *approx_mixed_wide_queue(const tbe_workspace_layout_t &l, void *workspace) {
+  return reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + l.segment_ids);
+}
 
 // Copies the rows that tbe_cache_prepare staged for this step back to the backing table.
 int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int32_t *keys_sorted,
