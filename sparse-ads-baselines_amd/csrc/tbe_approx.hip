@@ -317,7 +317,10 @@ __global__ __launch_bounds__(kBlockThreads) void approx_lookup_norms_kernel(
     int T_tables, int D, int group, MixedTables mt) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
-  if (counters[1] == 0) return;
+  int queued = counters[1];  // (one queue, or one per XCD)
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) queued += counters[kChunkQueueCount + x];
+  if (queued == 0) return;
   const int lane = threadIdx.x & (kWave - 1);
   const int r = lane / group;
   const int c = lane - r * group;
@@ -622,15 +625,53 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
 template <typename T, bool WEIGHTED, bool STOCHASTIC, bool BIG>
 __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     LongRowArgs<T> a, const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
-    const int32_t *__restrict__ counters, const int32_t *__restrict__ long_queue, int D) {
+    const int32_t *__restrict__ counters, const int32_t *__restrict__ long_queue, int queue_capacity, int D) {
   // (what is the same in every lane of the wavefront is told to the compiler, so that the walk's
   // control flow and addressing stay scalar)
   const int lane = threadIdx.x & (kWave - 1);
-  const int num_long = uniform(counters[1]);
-  const int wave_id = uniform(static_cast<int>(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
-  const int wave_stride = static_cast<int>(gridDim.x) * kWavesPerBlock;
-  for (int q = wave_id; q < num_long; q += wave_stride) {
-    const int u = uniform(long_queue[q]);
+  const int wave_in_block = uniform(static_cast<int>(threadIdx.x >> 6));
+  // One queue (queue_capacity == 0, its length in counters[1]), or one per XCD as the short-row
+  // kernel fills them: the workgroups of an XCD take their own queue in order -- it is in (table,
+  // row) order, so the gradient rows of a table stay in that XCD's L2 while its rows are walked --
+  // up to 1.5 times the average length; what the longer queues hold beyond that is dealt to the
+  // wavefronts of all XCDs.
+  const int xcd = static_cast<int>(blockIdx.x % kNumXcd);
+  int queue_len[kNumXcd];
+  int total = 0;
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) {
+    queue_len[x] = queue_capacity > 0 ? uniform(counters[kChunkQueueCount + x]) : 0;
+    total += queue_len[x];
+  }
+  const int fair = total / kNumXcd + total / 16 + 1;
+  int shared_total = queue_capacity > 0 ? 0 : uniform(counters[1]);
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) shared_total += max(0, queue_len[x] - fair);
+  const int own = min(queue_len[xcd], fair);
+  int q = static_cast<int>(blockIdx.x / kNumXcd) * kWavesPerBlock + wave_in_block;
+  const int stride = static_cast<int>(gridDim.x / kNumXcd) * kWavesPerBlock;
+  int g = static_cast<int>(blockIdx.x) * kWavesPerBlock + wave_in_block;
+  const int shared_stride = static_cast<int>(gridDim.x) * kWavesPerBlock;
+  while (true) {
+    int slot;
+    if (q < own) {
+      slot = xcd * queue_capacity + q;
+      q += stride;
+    } else if (g < shared_total) {
+      slot = g;
+      if (queue_capacity > 0) {
+        int before = 0, x = 0;
+        while (g >= before + max(0, queue_len[x] - fair)) {
+          before += max(0, queue_len[x] - fair);
+          ++x;
+        }
+        slot = x * queue_capacity + fair + (g - before);
+      }
+      g += shared_stride;
+    } else {
+      break;
+    }
+    const int u = uniform(long_queue[slot]);
     const int seg_begin = uniform(segment_starts[u]);
     const int seg_end = uniform(segment_starts[u + 1]);
     const int64_t key = uniform(keys_sorted[seg_begin]);
@@ -693,8 +734,12 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
   int32_t *counters = reinterpret_cast<int32_t *>(ws + l.num_unique);
   int32_t *long_queue = reinterpret_cast<int32_t *>(ws + l.chunk_segments);
   const int64_t most_long = a.n / (kShortSegment + 1) + 1;  // (the short-row kernel queues rows of 17 and more)
+  // (a multiple of the XCD count, so that every XCD has the same number of workgroups)
   const dim3 grid_long(static_cast<unsigned>(
-      std::max<int64_t>(1, std::min<int64_t>(ceil_div(most_long, kWavesPerBlock), 256 * 8))));
+      kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(most_long, kWavesPerBlock * kNumXcd), 256))));
+  // uniform tables whose rows fit a wavefront: the short-row kernel fills one queue per XCD
+  const int queue_capacity =
+      (!mixed && approx_short_serves(a.dtype, a.D)) ? static_cast<int>(approx_long_queue_capacity(a.n)) : 0;
   const dim3 block_long(kBlockThreads);
   // the queued rows' kernel reads the state addend of every lookup from the sort's ping-pong
   // buffers (8 bytes per lookup, free once the batch is sorted)
@@ -712,7 +757,7 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
 #define TBE_APPROX_LONG_KERNEL(WEIGHTED, STOCHASTIC, BIG)                                              \
   TBE_LAUNCH("update_approx_long", stream, (approx_adagrad_long_kernel<T, WEIGHTED, STOCHASTIC, BIG>), \
              grid_long, block_long, la, i32(l.keys_sorted), i32(l.segment_starts), counters,           \
-             long_queue, a.D)
+             long_queue, queue_capacity, a.D)
 #define TBE_APPROX_LONG(WEIGHTED, MIXED)                                                               \
   TBE_LAUNCH("update_approx_norms", stream, (approx_lookup_norms_kernel<T, VEC, WEIGHTED, MIXED>),     \
              grid_norms, block, static_cast<const T *>(a.grad_output), static_cast<const T *>(a.psw),  \

@@ -51,6 +51,11 @@ inline int64_t chunk_queue_capacity(int64_t n) {
   return eighth / (kShortSegment + 1) + eighth / kChunkLen + n / kChunkLen + 8;
 }
 
+// Room of one XCD's queue of rows that the approximate update's short-row kernel leaves to the
+// wavefront-per-row kernel: the rows of more than kShortSegment occurrences that start in the
+// XCD's eighth of the sorted positions (an eighth is rounded up to whole workgroups of tiles).
+inline int64_t approx_long_queue_capacity(int64_t n) { return (n / 8 + 8192) / (kShortSegment + 1) + 2; }
+
 enum { kOptSgd = 0, kOptAdagrad = 1 };
 
 struct UpdateArgs {

@@ -218,7 +218,9 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const int32_t key = s_keys[wave][j];
     if constexpr (APPROX) {
       if (len > kShortSegment) {
-        if (c == 0) approx_long_queue[atomicAdd(&counters[1], 1)] = u;
+        // (one queue per XCD, like the chunk records: `max_chunks` is the room of all eight)
+        if (c == 0)
+          approx_long_queue[xcd * (max_chunks / kNumXcd) + atomicAdd(&counters[kChunkQueueCount + xcd], 1)] = u;
         continue;
       }
     }
@@ -734,7 +736,8 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
 }
 
 // The short-row kernel alone, in its per-lookup (approximate Adagrad) form; rows of more than
-// kShortSegment occurrences are left in `queue` (their count in counters[1]).
+// kShortSegment occurrences are left in `queue`: eight queues of approx_long_queue_capacity() row
+// numbers, one per XCD, their lengths in counters[kChunkQueueCount ...].
 template <typename T, int VEC, int CHUNKS, bool WEIGHTED>
 void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *queue, hipStream_t stream) {
   using A = typename AccOf<T>::type;
@@ -747,7 +750,8 @@ void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *que
              static_cast<A *>(a.optimizer_state), static_cast<const T *>(a.per_sample_weights),
              static_cast<T *>(a.grad_per_sample_weights), a.keys_sorted, a.positions_sorted, a.grad_rows,
              a.segment_starts, a.segment_ids, a.counters, static_cast<LongRecord *>(nullptr),
-             static_cast<ChunkRecord *>(nullptr), int64_t{0}, a.num_indices, num_tiles, tiles_per_xcd, a.D,
+             static_cast<ChunkRecord *>(nullptr), kNumXcd * approx_long_queue_capacity(a.num_indices),
+             a.num_indices, num_tiles, tiles_per_xcd, a.D,
              g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr), static_cast<T *>(nullptr),
              a.stochastic_rounding, queue);
 }
