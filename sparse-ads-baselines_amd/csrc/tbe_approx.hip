@@ -630,11 +630,14 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
   // control flow and addressing stay scalar)
   const int lane = threadIdx.x & (kWave - 1);
   const int wave_in_block = uniform(static_cast<int>(threadIdx.x >> 6));
-  // One queue (queue_capacity == 0, its length in counters[1]), or one per XCD as the short-row
-  // kernel fills them: the workgroups of an XCD take their own queue in order -- it is in (table,
-  // row) order, so the gradient rows of a table stay in that XCD's L2 while its rows are walked --
-  // up to 1.5 times the average length; what the longer queues hold beyond that is dealt to the
-  // wavefronts of all XCDs.
+  // queue_capacity == 0: one queue, its length in counters[1].  Otherwise, as the short-row kernel
+  // leaves them: one queue per XCD (lengths in counters[kChunkQueueCount ...]) and behind them the
+  // queue of the rows of more than kApproxHuge occurrences (counters[1]).  Those come first, one
+  // per wavefront, so that the longest walks start when the kernel does.  Then the workgroups of
+  // an XCD take their own queue in order -- it is in (table, row) order, so the gradient rows of a
+  // table stay in that XCD's L2 while its rows are walked -- up to 1.5 times the average length;
+  // what the longer queues hold beyond that is dealt to the wavefronts of all XCDs.  All of it is
+  // index arithmetic on the queue lengths: no wavefront waits for another.
   const int xcd = static_cast<int>(blockIdx.x % kNumXcd);
   int queue_len[kNumXcd];
   int total = 0;
@@ -644,30 +647,32 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     total += queue_len[x];
   }
   const int fair = total / kNumXcd + total / 16 + 1;
-  int shared_total = queue_capacity > 0 ? 0 : uniform(counters[1]);
+  const int first_total = uniform(counters[1]);  // the rows every wavefront helps with first
+  int shared_total = 0;
 #pragma unroll
   for (int x = 0; x < kNumXcd; ++x) shared_total += max(0, queue_len[x] - fair);
   const int own = min(queue_len[xcd], fair);
   int q = static_cast<int>(blockIdx.x / kNumXcd) * kWavesPerBlock + wave_in_block;
   const int stride = static_cast<int>(gridDim.x / kNumXcd) * kWavesPerBlock;
-  int g = static_cast<int>(blockIdx.x) * kWavesPerBlock + wave_in_block;
-  const int shared_stride = static_cast<int>(gridDim.x) * kWavesPerBlock;
+  const int all_stride = static_cast<int>(gridDim.x) * kWavesPerBlock;
+  int first = static_cast<int>(blockIdx.x) * kWavesPerBlock + wave_in_block;
+  int g = first;
   while (true) {
     int slot;
-    if (q < own) {
+    if (first < first_total) {
+      slot = kNumXcd * queue_capacity + first;
+      first += all_stride;
+    } else if (q < own) {
       slot = xcd * queue_capacity + q;
       q += stride;
     } else if (g < shared_total) {
-      slot = g;
-      if (queue_capacity > 0) {
-        int before = 0, x = 0;
-        while (g >= before + max(0, queue_len[x] - fair)) {
-          before += max(0, queue_len[x] - fair);
-          ++x;
-        }
-        slot = x * queue_capacity + fair + (g - before);
+      int before = 0, x = 0;
+      while (g >= before + max(0, queue_len[x] - fair)) {
+        before += max(0, queue_len[x] - fair);
+        ++x;
       }
-      g += shared_stride;
+      slot = x * queue_capacity + fair + (g - before);
+      g += all_stride;
     } else {
       break;
     }
@@ -740,6 +745,7 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
   // uniform tables whose rows fit a wavefront: the short-row kernel fills one queue per XCD
   const int queue_capacity =
       (!mixed && approx_short_serves(a.dtype, a.D)) ? static_cast<int>(approx_long_queue_capacity(a.n)) : 0;
+
   const dim3 block_long(kBlockThreads);
   // the queued rows' kernel reads the state addend of every lookup from the sort's ping-pong
   // buffers (8 bytes per lookup, free once the batch is sorted)
@@ -827,6 +833,13 @@ int approx_update(const void *grad_output, void *weights, void *state, const voi
                MixedTables{mixed_table_offsets, table_dim_offsets, dim_offsets, total_D, T}, sr, offsets, B, T,
                D == 0 ? approx_mixed_wide_queue(l, workspace) : nullptr};
   char *ws = static_cast<char *>(workspace);
+  // the queues of long rows borrow the chunk records' region: eight of approx_long_queue_capacity()
+  // rows and one of the rows of more than kApproxHuge occurrences, or one queue of at most n / 9 rows
+  const uint64_t queue_words = static_cast<uint64_t>(kNumXcd) * approx_long_queue_capacity(n) +
+                               static_cast<uint64_t>(n) / (kApproxHuge + 1) + 1 + static_cast<uint64_t>(n) / 9;
+  if (queue_words * 4 > static_cast<uint64_t>(l.max_chunks) * 32)
+    return fail(TBE_ERR_WORKSPACE, "tbe approximate Adagrad update: queues of %llu rows do not fit the workspace",
+                (unsigned long long)queue_words);
   switch (dtype) {
     case TBE_DTYPE_F32: launch_approx<float, 4>(a, l, ws, stream); break;
     case TBE_DTYPE_F16:

@@ -41,6 +41,7 @@ constexpr int kChunkLen = 256;
 // [1] long rows, [3] partial rows, [8..15] chunk records queued by each XCD.
 constexpr int kNumCounters = 16;
 constexpr int kChunkQueueCount = 8;
+constexpr int kApproxHuge = 256;   // occurrences from which on the approximate update walks a row before the others
 // The short-row kernel's workgroups of XCD x own the segments that start in the x-th eighth of
 // the sorted positions (rounded up to whole workgroups: fewer than 1200 positions more) and queue
 // their chunk records in a region of their own.  Segments are consecutive, so only the last
@@ -55,6 +56,7 @@ inline int64_t chunk_queue_capacity(int64_t n) {
 // wavefront-per-row kernel: the rows of more than kShortSegment occurrences that start in the
 // XCD's eighth of the sorted positions (an eighth is rounded up to whole workgroups of tiles).
 inline int64_t approx_long_queue_capacity(int64_t n) { return (n / 8 + 8192) / (kShortSegment + 1) + 2; }
+// (behind the eight queues: the rows of more than kApproxHuge occurrences, at most n / 257 + 1)
 
 enum { kOptSgd = 0, kOptAdagrad = 1 };
 

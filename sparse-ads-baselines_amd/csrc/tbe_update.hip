@@ -219,8 +219,11 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     if constexpr (APPROX) {
       if (len > kShortSegment) {
         // (one queue per XCD, like the chunk records: `max_chunks` is the room of all eight)
-        if (c == 0)
-          approx_long_queue[xcd * (max_chunks / kNumXcd) + atomicAdd(&counters[kChunkQueueCount + xcd], 1)] = u;
+        // and one behind them for the rows of very many occurrences
+        if (c == 0) {
+          if (len > kApproxHuge) approx_long_queue[max_chunks + atomicAdd(&counters[1], 1)] = u;
+          else approx_long_queue[xcd * (max_chunks / kNumXcd) + atomicAdd(&counters[kChunkQueueCount + xcd], 1)] = u;
+        }
         continue;
       }
     }
