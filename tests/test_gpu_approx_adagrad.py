@@ -155,6 +155,132 @@ def test_approx_adagrad_with_a_gradient_tensor_beyond_4GiB():
     assert w_big[untouched].tobytes() == weights[untouched].tobytes()
 
 
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("weighted", [False, True])
+def test_full_size_approx_adagrad_against_the_fp64_closed_form(oracle, weighted):
+    """The benchmark's headline shape (T=64, E=1e5, D=128 fp32, B=4096, L=20, Zipf(1.05): 5.2 M lookups,
+    the hottest row of a table some 4000 times).  The serial per-lookup update has a closed form that
+    torch evaluates in fp64 on the device: with the lookups of a row in position order,
+        state_k = state_0 + sum_{j<=k} wss_j,   mult_k = (psw_k *) lr / (sqrt(state_k) + eps),
+        row_final = row_0 - sum_k mult_k * g_k,   grad_psw_k = <row_0 - sum_{j<k} mult_j g_j, g_k>.
+    State and weights of every row are compared with it; the per-sample-weight gradients, whose closed
+    form is quadratic in a row's occurrences, and the first table's rows are compared with the oracle."""
+    T, E, D, B, L = 64, 100000, 128, 4096, 20
+    lr, eps = 0.05, 0.1
+    n = T * B * L
+    rs = np.random.RandomState(40)
+    idx_np = (rs.zipf(1.05, size=n) % E).astype(np.int32)
+    gen = torch.Generator(device=DEV).manual_seed(40)
+    W = torch.empty(T * E, D, device=DEV).uniform_(-0.01, 0.01, generator=gen)
+    W0 = W.clone()
+    go = torch.randn(B, T, D, device=DEV, generator=gen) * 0.1
+    state = torch.empty(T * E, device=DEV).uniform_(0.0, 2.0, generator=gen)
+    state0 = state.clone()
+    psw = torch.empty(n, device=DEV).uniform_(0.0, 1.0, generator=gen) if weighted else None
+    idx = torch.from_numpy(idx_np).to(DEV)
+    offsets = torch.arange(0, n + 1, L, dtype=torch.int32, device=DEV)
+    table_offsets = torch.arange(T, dtype=torch.int32, device=DEV) * E
+    g_psw = ext.backward_approx_adagrad(go, W, table_offsets, idx, offsets, psw, state, lr, eps, 200, False, 1)
+    torch.cuda.synchronize()
+
+    pos = torch.arange(n, device=DEV)
+    t_of = pos // (B * L)
+    b_of = (pos % (B * L)) // L
+    key = idx.long() + t_of * E
+    wss = (go.double() ** 2).sum(-1)[b_of, t_of]
+    if weighted:
+        wss = wss * psw.double() ** 2
+    order = torch.sort(key, stable=True)[1]          # (row, position) order
+    key_s, wss_s = key[order], wss[order]
+    csum = torch.cumsum(wss_s, 0)
+    head = torch.ones(n, dtype=torch.bool, device=DEV)
+    head[1:] = key_s[1:] != key_s[:-1]
+    seg_of = torch.cumsum(head.long(), 0) - 1
+    before = (csum - wss_s)[head][seg_of]             # sum of the earlier rows' addends
+    state_k = state0.double()[key_s] + (csum - before)
+    mult = lr / (torch.sqrt(state_k) + eps)
+    if weighted:
+        mult = mult * psw.double()[order]
+    want_state = state0.double().index_add(0, key, wss)
+    assert_close(state.cpu().numpy(), want_state.cpu().numpy(), 1e-5, "state")
+    delta = torch.zeros(T * E, D, dtype=torch.float64, device=DEV)
+    chunk = 1 << 20
+    for lo in range(0, n, chunk):                     # (pieces: the products of all lookups would take 5 GB)
+        sel = order[lo:lo + chunk]
+        delta.index_add_(0, key_s[lo:lo + chunk], mult[lo:lo + chunk, None] * go[b_of[sel], t_of[sel]].double())
+    want_W = W0.double() - delta
+    err = (W.double() - want_W).abs().max().item()
+    scale = want_W.abs().max().item()
+    assert err <= 1e-5 * scale, (err, scale)
+    touched = torch.zeros(T * E, dtype=torch.bool, device=DEV)
+    touched[key] = True
+    assert torch.equal(W[~touched], W0[~touched]) and torch.equal(state[~touched], state0[~touched])
+    # the first table (81 920 lookups) against the oracle, gradients of the per-sample weights included
+    w_ref = W0[:E].cpu().numpy().copy()
+    st_ref = state0[:E].cpu().numpy().copy()
+    g_ref = oracle.backward_approx(go[:, :1, :].contiguous().cpu().numpy(), w_ref, np.zeros(1, np.int32),
+                                   idx_np[:B * L], offsets[:B + 1].cpu().numpy(), lr, eps, st_ref,
+                                   psw[:B * L].cpu().numpy() if weighted else None, None)
+    assert_close(W[:E].cpu().numpy(), w_ref, 1e-5, "first table")
+    assert_close(state[:E].cpu().numpy(), st_ref, 1e-5, "first table's state")
+    if weighted:
+        assert_close(g_psw[:B * L].cpu().numpy(), g_ref, 1e-4, "first table's per-sample-weight gradients")
+
+
+@pytest.mark.timeout(600)
+def test_full_size_mixed_D_approx_adagrad_against_the_fp64_closed_form():
+    """The mixed-D benchmark's shape (64 tables of 1e5 rows, widths 64 ... 192 in steps of 4, fp32, B=4096,
+    L=20, Zipf(1.05)) against the same closed form, table by table."""
+    T, E, B, L = 64, 100000, 4096, 20
+    lr, eps = 0.05, 0.1
+    n = T * B * L
+    rs = np.random.RandomState(41)
+    dims = [int((rs.randint(64, 193) + 3) // 4 * 4) for _ in range(T)]
+    dim_offsets = np.concatenate([[0], np.cumsum(dims)]).astype(np.int32)
+    total_D = int(dim_offsets[-1])
+    table_offsets = np.concatenate([[0], np.cumsum([E * d for d in dims])]).astype(np.int64)
+    table_dim_offsets = (np.arange(T + 1) * E).astype(np.int32)
+    idx_np = (rs.zipf(1.05, size=n) % E).astype(np.int32)
+    gen = torch.Generator(device=DEV).manual_seed(41)
+    W = torch.empty(int(table_offsets[-1]), device=DEV).uniform_(-0.01, 0.01, generator=gen)
+    W0 = W.clone()
+    go = torch.randn(B, total_D, device=DEV, generator=gen) * 0.1
+    state = torch.empty(T * E, device=DEV).uniform_(0.0, 2.0, generator=gen)
+    state0 = state.clone()
+    idx = torch.from_numpy(idx_np).to(DEV)
+    offsets = torch.arange(0, n + 1, L, dtype=torch.int32, device=DEV)
+    ext.backward_approx_adagrad_mixed_D(go, W, dev(table_offsets), dev(table_dim_offsets), dev(dim_offsets), total_D,
+                                        idx, offsets, None, state, lr, eps, 200, False, 1)
+    torch.cuda.synchronize()
+    pos = torch.arange(B * L, device=DEV)
+    b_of = pos // L
+    worst = 0.0
+    for t in range(T):
+        g = go[:, int(dim_offsets[t]):int(dim_offsets[t + 1])].double()
+        key = idx[t * B * L:(t + 1) * B * L].long()
+        wss = (g ** 2).sum(-1)[b_of]
+        order = torch.sort(key, stable=True)[1]
+        key_s, wss_s = key[order], wss[order]
+        csum = torch.cumsum(wss_s, 0)
+        head = torch.ones(B * L, dtype=torch.bool, device=DEV)
+        head[1:] = key_s[1:] != key_s[:-1]
+        before = (csum - wss_s)[head][torch.cumsum(head.long(), 0) - 1]
+        st0 = state0[t * E:(t + 1) * E].double()
+        mult = lr / (torch.sqrt(st0[key_s] + (csum - before)) + eps)
+        want_state = st0.index_add(0, key, wss)
+        assert_close(state[t * E:(t + 1) * E].cpu().numpy(), want_state.cpu().numpy(), 1e-5, "state of table %d" % t)
+        rows = slice(int(table_offsets[t]), int(table_offsets[t + 1]))
+        delta = torch.zeros(E, dims[t], dtype=torch.float64, device=DEV)
+        delta.index_add_(0, key_s, mult[:, None] * g[b_of[order]])
+        want = W0[rows].view(E, dims[t]).double() - delta
+        got = W[rows].view(E, dims[t]).double()
+        worst = max(worst, ((got - want).abs().max() / want.abs().max()).item())
+        untouched = torch.ones(E, dtype=torch.bool, device=DEV)
+        untouched[key] = False
+        assert torch.equal(W[rows].view(E, dims[t])[untouched], W0[rows].view(E, dims[t])[untouched])
+    assert worst <= 1e-5, worst
+
+
 def test_approx_adagrad_stochastic_rounding_of_rows_of_many_occurrences(oracle):
     """The k-th update of a hot row draws the oracle's random words in the wavefront-per-row kernel too."""
     p = make_problem(37, T=2, E=12, D=64, B=64, L=10, dtype=np.float16, ragged=False, weighted=False, zipf=1.5)
