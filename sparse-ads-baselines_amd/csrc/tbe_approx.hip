@@ -63,33 +63,6 @@ __device__ __forceinline__ int64_t uniform(int64_t v) {
   return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
-// v of the lane a data-parallel-primitive pattern selects, 0 where the pattern has no source lane
-// or the row mask leaves the lane out.
-template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_or_zero(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
-}
-template <int CTRL, int ROW_MASK> __device__ __forceinline__ double dpp_or_zero(double v) {
-  const int64_t bits = __double_as_longlong(v);
-  const uint32_t lo = static_cast<uint32_t>(
-      __builtin_amdgcn_update_dpp(0, static_cast<int>(bits), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
-  const uint32_t hi = static_cast<uint32_t>(
-      __builtin_amdgcn_update_dpp(0, static_cast<int>(bits >> 32), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
-  return __longlong_as_double(static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo));
-}
-
-// Inclusive prefix sum over the 64 lanes without a trip through LDS: shifts inside the rows of 16
-// lanes, then the last lane of row 0 / 2 added to row 1 / 3 and the last lane of row 1 to rows 2
-// and 3 (row_shr:n = 0x110 + n, row_bcast:15 = 0x142, row_bcast:31 = 0x143).
-template <typename A> __device__ __forceinline__ A wave_inclusive_sum(A x) {
-  x += dpp_or_zero<0x111, 0xf>(x);
-  x += dpp_or_zero<0x112, 0xf>(x);
-  x += dpp_or_zero<0x114, 0xf>(x);
-  x += dpp_or_zero<0x118, 0xf>(x);
-  x += dpp_or_zero<0x142, 0xa>(x);
-  x += dpp_or_zero<0x143, 0xc>(x);
-  return x;
-}
-
 // Sum over the `group` lanes (a power of two) around the caller; every lane gets the result.
 template <typename A> __device__ __forceinline__ A group_sum_pow2(A v, int group) {
   for (int m = group >> 1; m > 0; m >>= 1) v += shfl_x(v, m);
@@ -808,9 +781,24 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
     ua.learning_rate = a.lr;
     ua.eps = a.eps;
     ua.stochastic_rounding = a.sr;
-    (void)segment_update_approx_short(ua, long_queue, stream);
-    if (a.psw) { TBE_APPROX_LONG(true, false); }
-    else { TBE_APPROX_LONG(false, false); }
+    if (approx_sums_long_rows(a.dtype, a.D, a.psw != nullptr)) {
+      // fp32 / fp64 rows without per-sample weights: the update of a row is a weighted sum of its
+      // gradient rows, so the longer rows are summed in chunks like the exact update's
+      ua.long_segments = ws + l.long_segments;
+      ua.chunk_segments = ws + l.chunk_segments;
+      ua.partial_sums = ws + l.partial_sums;
+      ua.max_long = l.max_long_segments;
+      ua.max_chunks = l.max_chunks;
+      (void)segment_update_approx_short(ua, nullptr, stream);
+      TBE_LAUNCH("update_approx_norms", stream, (approx_lookup_norms_kernel<T, VEC, false, false>), grid_norms,
+                 block, static_cast<const T *>(a.grad_output), static_cast<const T *>(nullptr), a.offsets, counters,
+                 lookup_wss, a.B, a.T, a.D, group, a.mt);
+      (void)segment_update_approx_sum_long(ua, lookup_wss, stream);
+    } else {
+      (void)segment_update_approx_short(ua, long_queue, stream);
+      if (a.psw) { TBE_APPROX_LONG(true, false); }
+      else { TBE_APPROX_LONG(false, false); }
+    }
   } else {
     if (a.psw) { TBE_APPROX(true, false); }
     else { TBE_APPROX(false, false); }

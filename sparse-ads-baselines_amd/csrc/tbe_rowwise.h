@@ -28,6 +28,33 @@ template <> __device__ __forceinline__ double approx_multiplier<double>(double s
   return weighted ? pw * static_cast<double>(lr) * inv : static_cast<double>(lr) * inv;
 }
 
+// v of the lane a data-parallel-primitive pattern selects, 0 where the pattern has no source lane
+// or the row mask leaves the lane out.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_or_zero(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
+}
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ double dpp_or_zero(double v) {
+  const int64_t bits = __double_as_longlong(v);
+  const uint32_t lo = static_cast<uint32_t>(
+      __builtin_amdgcn_update_dpp(0, static_cast<int>(bits), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
+  const uint32_t hi = static_cast<uint32_t>(
+      __builtin_amdgcn_update_dpp(0, static_cast<int>(bits >> 32), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
+  return __longlong_as_double(static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo));
+}
+
+// Inclusive prefix sum over the 64 lanes without a trip through LDS: shifts inside the rows of 16
+// lanes, then the last lane of row 0 / 2 added to row 1 / 3 and the last lane of row 1 to rows 2
+// and 3 (row_shr:n = 0x110 + n, row_bcast:15 = 0x142, row_bcast:31 = 0x143).
+template <typename A> __device__ __forceinline__ A wave_inclusive_sum(A x) {
+  x += dpp_or_zero<0x111, 0xf>(x);
+  x += dpp_or_zero<0x112, 0xf>(x);
+  x += dpp_or_zero<0x114, 0xf>(x);
+  x += dpp_or_zero<0x118, 0xf>(x);
+  x += dpp_or_zero<0x142, 0xa>(x);
+  x += dpp_or_zero<0x143, 0xc>(x);
+  return x;
+}
+
 // The value a row vector has after it was stored in the weights' type and read again.
 template <typename T, int VEC>
 __device__ __forceinline__ void round_trip(RowVec<T, VEC> &w, const StochasticRounding &sr, int64_t element) {

@@ -94,6 +94,12 @@ int segment_update(const UpdateArgs &args, hipStream_t stream);
 // longer rows are appended to `queue` as unique-row numbers, their count in args.counters[1].
 bool approx_short_serves(int32_t dtype, int32_t D);
 int segment_update_approx_short(const UpdateArgs &args, int32_t *queue, hipStream_t stream);
+// fp32 / fp64 rows without per-sample weights: the approximate update of a row is a weighted sum
+// of its gradient rows, so its long rows are summed in chunks like the exact update's.  Then
+// segment_update_approx_short() is called with a null queue (the rows go to the chunk queues of
+// its UpdateArgs) and, once the lookups' state addends are known, segment_update_approx_sum_long().
+bool approx_sums_long_rows(int32_t dtype, int32_t D, bool weighted);
+int segment_update_approx_sum_long(const UpdateArgs &args, const void *lookup_wss, hipStream_t stream);
 
 int key_bits_for(int64_t total_rows);
 void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *layout);

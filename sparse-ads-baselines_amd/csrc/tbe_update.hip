@@ -105,7 +105,10 @@ struct LongRecord {    // 16 bytes: a segment cut into several chunks
 // summed gradient -- every occurrence, in position order, adds its bag's ||grad||^2 (times its
 // squared weight) to the state and moves the row by its own multiplier.  Segments longer than
 // kShortSegment are then queued as unique-row numbers for tbe_approx.hip's wavefront-per-row kernel.
-template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL, bool APPROX = false>
+// APPROX_SUM (with APPROX, rows without per-sample weights in fp32 / fp64): longer segments take the
+// chunk queue like the exact update's, for update_chunks_kernel's per-lookup form.
+template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL, bool APPROX = false,
+          bool APPROX_SUM = false>
 __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
@@ -216,7 +219,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const int seg_end = s_bounds[wave][j + 1];
     const int len = seg_end - seg_begin;
     const int32_t key = s_keys[wave][j];
-    if constexpr (APPROX) {
+    if constexpr (APPROX && !APPROX_SUM) {
       if (len > kShortSegment) {
         // (one queue per XCD, like the chunk records: `max_chunks` is the room of all eight)
         // and one behind them for the rows of very many occurrences
@@ -354,7 +357,15 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
 // tree.
 // A chunk that is a whole segment is applied to its row at once; a chunk of a longer
 // segment stores its sum as a partial row for update_long_finish_kernel.
-template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL>
+// APPROX (instantiated as SGD without per-sample weights, fp32 / fp64 rows): the approximate
+// Adagrad of a row without per-sample weights is row_0 - sum_k mult_k * g_k with
+// mult_k = lr / (sqrt(state_0 + sum_{j<=k} wss_j) + eps), so its long rows are summed in chunks like
+// the exact update's.  `psw` then holds wss of every lookup by position (approx_lookup_norms_kernel);
+// a chunk adds up the addends of the row's earlier occurrences, forms the multipliers of its own
+// 64 at a time (a wavefront prefix sum) and adds mult * g.  A chunk that is a whole segment writes
+// the row and its state; the state of a row of several chunks is left to approx_long_state_kernel
+// (every chunk of the row reads the old one).
+template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL, bool APPROX = false>
 __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
@@ -362,10 +373,13 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ counters,
     const ChunkRecord *__restrict__ chunk_records, int64_t max_chunks,
     typename AccOf<T>::type *__restrict__ partial_sums, int D, int chunks_rt, float lr, float eps,
-    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr) {
+    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr,
+    const int32_t *__restrict__ segment_starts) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
+  static_assert(!APPROX || (OPT == kOptSgd && !WEIGHTED && sizeof(T) == sizeof(A)),
+                "the per-lookup form sums fp32 / fp64 rows without per-sample weights");
 
   const int lane = threadIdx.x & (kWave - 1);
   const int chunks = CHUNKS > 0 ? CHUNKS : chunks_rt;
@@ -426,6 +440,26 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     }
     V G;
     G.zero();
+    // APPROX: the row's state before the chunk's first occurrence
+    A running = A(0);
+    if constexpr (APPROX) {
+      constexpr int kAhead = 16;
+      const int seg_begin = segment_starts[rec.u];
+      A earlier = A(0);
+      for (int i0 = seg_begin; i0 < rec.begin; i0 += kAhead * kWave) {
+        int p[kAhead];
+        A x[kAhead];
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) p[k] = positions_sorted[min(i0 + k * kWave + lane, rec.begin - 1)];
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) x[k] = to_acc(psw[p[k]]);
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) earlier += (i0 + k * kWave + lane < rec.begin) ? x[k] : A(0);
+      }
+#pragma unroll
+      for (int m = kWave / 2; m > 0; m >>= 1) earlier += shfl_x(earlier, m);
+      running = state[rec.key] + earlier;
+    }
     // The positions of a 64-position batch are requested two batches ahead, its gradient row ids
     // and weights one batch ahead (lanes past the chunk's end ask for its first position: any
     // valid index will do), so a batch waits for gradient rows only.
@@ -434,15 +468,21 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     int pos_next = position_at(static_cast<int64_t>(rec.begin) + kWave + lane);
     int grow_now = grad_rows[pos_now];
     A w_now = A(0);
-    if constexpr (WEIGHTED) w_now = to_acc(psw[pos_now]);
+    if constexpr (WEIGHTED || APPROX) w_now = to_acc(psw[pos_now]);
     for (int base = rec.begin; base < rec.end; base += kWave) {
       const int n = min(kWave, rec.end - base);
       const int my_pos = pos_now, my_grow = grow_now;
-      const A my_w = w_now;
+      A my_w = w_now;
       pos_now = pos_next;
       pos_next = position_at(static_cast<int64_t>(base) + 2 * kWave + lane);
       grow_now = grad_rows[pos_now];
-      if constexpr (WEIGHTED) w_now = to_acc(psw[pos_now]);
+      if constexpr (WEIGHTED || APPROX) w_now = to_acc(psw[pos_now]);
+      if constexpr (APPROX) {
+        // lane j holds occurrence base + j: its state is the running one plus the addends up to it
+        const A incl = wave_inclusive_sum<A>(lane < n ? my_w : A(0));
+        my_w = lane < n ? approx_multiplier<A>(running + incl, A(1), false, lr, eps) : A(0);
+        running = running + shfl_idx(incl, n - 1);
+      }
       // Straight-line code: every lane loads (a lane without an occurrence loads what occurrence
       // 0 loads and drops it), so that the UNROLL loads of a step are issued back to back.
       for (int j0 = 0; j0 < n; j0 += groups * UNROLL) {
@@ -468,11 +508,15 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
             pw = shfl_idx(my_w, src[k]);
             pos = shfl_idx(my_pos, src[k]);
           }
+          if constexpr (APPROX) pw = shfl_idx(my_w, src[k]);
           V x;
           x.unpack(raw[k]);
 #pragma unroll
           for (int i = 0; i < VEC; ++i) x.v[i] = ok[k] ? x.v[i] : A(0);
-          if constexpr (WEIGHTED) {
+          if constexpr (APPROX) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * pw;
+          } else if constexpr (WEIGHTED) {
             A dot = A(0);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
@@ -512,12 +556,51 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
         A *dst = partial_sums + static_cast<int64_t>(rec.partial) * D + col;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) dst[i] = G.v[i];
+      } else if constexpr (APPROX) {
+        V w_new;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) w_new.v[i] = w_old.v[i] - G.v[i];
+        w_new.store(wrow);
+        if (c == 0) state[rec.key] = running;
       } else {
         apply_update<T, VEC, CHUNKS, OPT>(wrow, w_old, G, state ? state + rec.key : nullptr, state_old,
                                           lr, eps, chunks, 0, c, sr,
                                           static_cast<int64_t>(rec.key) * D + col);
       }
     }
+  }
+}
+
+// The approximate Adagrad's rows that were summed in several chunks: their state takes the addends
+// of all their lookups (one wavefront per row; update_long_finish_kernel writes the row itself).
+template <typename A>
+__global__ __launch_bounds__(kBlockThreads) void approx_long_state_kernel(
+    A *__restrict__ state, const A *__restrict__ lookup_wss, const int32_t *__restrict__ positions_sorted,
+    const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
+    const LongRecord *__restrict__ long_records) {
+  constexpr int kAhead = 16;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int num_long = counters[1];
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  for (int64_t slot = wave_id; slot < num_long; slot += stride) {
+    const LongRecord rec = long_records[slot];
+    const int seg_begin = segment_starts[rec.u];
+    const int seg_end = segment_starts[rec.u + 1];
+    A sum = A(0);
+    for (int i0 = seg_begin; i0 < seg_end; i0 += kAhead * kWave) {
+      int p[kAhead];
+      A x[kAhead];
+#pragma unroll
+      for (int k = 0; k < kAhead; ++k) p[k] = positions_sorted[min(i0 + k * kWave + lane, seg_end - 1)];
+#pragma unroll
+      for (int k = 0; k < kAhead; ++k) x[k] = lookup_wss[p[k]];
+#pragma unroll
+      for (int k = 0; k < kAhead; ++k) sum += (i0 + k * kWave + lane < seg_end) ? x[k] : A(0);
+    }
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) sum += shfl_x(sum, m);
+    if (lane == 0) state[rec.key] += sum;
   }
 }
 
@@ -729,7 +812,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
              grid_chunks, block,
              go, w, st, psw, gpsw, a.positions_sorted, a.grad_rows, a.counters, chunk_records,
              a.max_chunks, partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, cr,
-             a.stochastic_rounding);
+             a.stochastic_rounding, static_cast<const int32_t *>(nullptr));
 
   const int64_t want_long = ceil_div(a.max_long, kWavesPerBlock);
   const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
@@ -747,6 +830,21 @@ void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *que
   const int64_t num_tiles = ceil_div(a.num_indices, tile_positions(CHUNKS));
   const int64_t tiles_per_xcd = ceil_div(ceil_div(num_tiles, kWavesPerBlock), kNumXcd);
   const dim3 grid_short(static_cast<unsigned>(tiles_per_xcd * kNumXcd));
+  if constexpr (!WEIGHTED && sizeof(T) == sizeof(A)) {
+    if (queue == nullptr) {
+      // fp32 / fp64 rows without per-sample weights: longer rows go to the chunk queues
+      TBE_LAUNCH("update_approx_short", stream,
+                 (update_short_kernel<T, VEC, CHUNKS, kOptAdagrad, false, kShortUnroll, true, true>), grid_short,
+                 dim3(kBlockThreads), static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),
+                 static_cast<A *>(a.optimizer_state), static_cast<const T *>(nullptr), static_cast<T *>(nullptr),
+                 a.keys_sorted, a.positions_sorted, a.grad_rows, a.segment_starts, a.segment_ids, a.counters,
+                 reinterpret_cast<LongRecord *>(a.long_segments), reinterpret_cast<ChunkRecord *>(a.chunk_segments),
+                 a.max_chunks, a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,
+                 static_cast<const int32_t *>(nullptr), static_cast<T *>(nullptr), a.stochastic_rounding,
+                 static_cast<int32_t *>(nullptr));
+      return;
+    }
+  }
   TBE_LAUNCH("update_approx_short", stream,
              (update_short_kernel<T, VEC, CHUNKS, kOptAdagrad, WEIGHTED, kShortUnroll, true>), grid_short,
              dim3(kBlockThreads), static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),
@@ -831,6 +929,65 @@ int segment_update_approx_short(const UpdateArgs &a, int32_t *queue, hipStream_t
   }
 #undef TBE_APPROX_SHORT
   return check_launch("tbe approximate Adagrad update (short rows)");
+}
+
+namespace {
+template <typename T, int VEC, int CHUNKS>
+void launch_approx_sum_long(const UpdateArgs &a, const RowGeometry &g, const void *lookup_wss, hipStream_t stream) {
+  using A = typename AccOf<T>::type;
+  if constexpr (sizeof(T) == sizeof(A)) {
+    T *w = static_cast<T *>(a.weights);
+    A *st = static_cast<A *>(a.optimizer_state);
+    A *partial = static_cast<A *>(a.partial_sums);
+    LongRecord *long_records = reinterpret_cast<LongRecord *>(a.long_segments);
+    ChunkRecord *chunk_records = reinterpret_cast<ChunkRecord *>(a.chunk_segments);
+    const dim3 block(kBlockThreads);
+    const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
+    const dim3 grid_chunks(static_cast<unsigned>(
+        kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), 1024))));
+    TBE_LAUNCH("update_approx_chunks", stream,
+               (update_chunks_kernel<T, VEC, CHUNKS, kOptSgd, false, kLongUnroll, true>), grid_chunks, block,
+               static_cast<const T *>(a.grad_output), w, st, static_cast<const T *>(lookup_wss),
+               static_cast<T *>(nullptr), a.positions_sorted, a.grad_rows, a.counters, chunk_records, a.max_chunks,
+               partial, a.D, g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr),
+               static_cast<T *>(nullptr), a.stochastic_rounding, a.segment_starts);
+    const int64_t want_long = ceil_div(a.max_long, kWavesPerBlock);
+    const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
+    // (the partial rows already carry the multipliers: the row takes their sum as it is)
+    TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, kOptSgd>), grid_finish,
+               block, w, st, a.counters, long_records, partial, a.D, g.chunks, 1.0f, a.eps,
+               static_cast<const int32_t *>(nullptr), static_cast<T *>(nullptr), a.stochastic_rounding);
+    TBE_LAUNCH("update_approx_state", stream, (approx_long_state_kernel<A>), grid_finish, block, st,
+               static_cast<const A *>(lookup_wss), a.positions_sorted, a.segment_starts, a.counters, long_records);
+  }
+}
+
+template <typename T, int VEC>
+void launch_approx_sum_long_geometry(const UpdateArgs &a, const RowGeometry &g, const void *wss, hipStream_t stream) {
+  switch (g.tmpl) {
+    case 64: launch_approx_sum_long<T, VEC, 64>(a, g, wss, stream); break;
+    case 32: launch_approx_sum_long<T, VEC, 32>(a, g, wss, stream); break;
+    case 16: launch_approx_sum_long<T, VEC, 16>(a, g, wss, stream); break;
+    case 8: launch_approx_sum_long<T, VEC, 8>(a, g, wss, stream); break;
+    case 4: launch_approx_sum_long<T, VEC, 4>(a, g, wss, stream); break;
+    default: launch_approx_sum_long<T, VEC, 0>(a, g, wss, stream); break;
+  }
+}
+}  // namespace
+
+bool approx_sums_long_rows(int32_t dtype, int32_t D, bool weighted) {
+  return !weighted && dtype != TBE_DTYPE_F16 && approx_short_serves(dtype, D);
+}
+
+// The long rows of the approximate update in its chunked form (approx_sums_long_rows()): the short-row
+// kernel, called with a null queue, has left them in the chunk queues of `a`; `lookup_wss` holds
+// ||grad||^2 of every lookup by position.
+int segment_update_approx_sum_long(const UpdateArgs &a, const void *lookup_wss, hipStream_t stream) {
+  if (a.num_indices == 0) return TBE_OK;
+  const RowGeometry g = row_geometry(a.dtype, a.D);
+  if (a.dtype == TBE_DTYPE_F32) launch_approx_sum_long_geometry<float, 4>(a, g, lookup_wss, stream);
+  else launch_approx_sum_long_geometry<double, 2>(a, g, lookup_wss, stream);
+  return check_launch("tbe approximate Adagrad update (summed rows)");
 }
 
 int segment_update(const UpdateArgs &a, hipStream_t stream) {
