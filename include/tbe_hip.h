@@ -205,7 +205,10 @@ TBE_API int tbe_backward_exact_adagrad(const void *grad_output, void *weights, i
  * Here the lookups of a row are applied one at a time in ascending position (table-major bag
  * order, then the order inside the bag): the reference's arithmetic executed serially.  The two
  * agree whenever the reference's result is defined; when rows repeat this library returns the
- * serial result, deterministically.  With stochastic_rounding (fp16 only) the k-th update of a
+ * serial result, deterministically.  (fp32 / fp64 rows without per-sample weights: nothing
+ * rounds the row between its lookups and nothing reads it, so a row of many lookups is written
+ * once, as row - sum_k mult_k * g_k with the sum taken in a fixed tree order -- the serial result
+ * up to the rounding of the additions.)  With stochastic_rounding (fp16 only) the k-th update of a
  * row within the call draws its bits with the Philox key seed ^ (k * 0x9E3779B97F4A7C15): k = 0
  * is the stream of tbe_backward_exact_adagrad_stochastic.  Arguments as in
  * tbe_backward_exact_adagrad_stochastic.
