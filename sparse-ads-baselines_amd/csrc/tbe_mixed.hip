@@ -425,6 +425,12 @@ template <typename X> __device__ __forceinline__ void register_fence(X &x) {
 }
 
 constexpr int kMixedShort = 8;
+// Workgroups per compute unit the strip kernel is compiled for: as many as its registers allow
+// without spilling (per-sample weights, 8-element vectors, fp64 and the per-lookup form each need more).
+constexpr int mixed_strip_blocks(bool weighted, bool wide_vectors, bool approx, bool fp64) {
+  const int heavy = (weighted ? 1 : 0) + (wide_vectors ? 1 : 0) + (approx ? 1 : 0) + (fp64 && (weighted || approx) ? 1 : 0);
+  return heavy == 0 ? 5 : heavy == 1 ? 4 : 3;
+}
 constexpr int kMixedAhead = 4;
 // APPROX (row-wise Adagrad only): the approximate update's per-lookup form -- every occurrence adds
 // its bag's ||grad||^2 (times its squared weight) to the row's state and moves the row by its own
@@ -433,7 +439,7 @@ constexpr int kMixedAhead = 4;
 // occurrences then go to ONE queue (`huge_rows`, counters[1]) whatever their length, and rows wider
 // than 64 vectors to the other (`long_rows`, counters[2]).
 template <typename T, int VEC, int OPT, bool WEIGHTED, bool APPROX = false>
-__global__ __launch_bounds__(kBlockThreads, (WEIGHTED || VEC == 8) ? 4 : 5) void update_mixed_kernel(
+__global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 8, APPROX, sizeof(T) == 8)) void update_mixed_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
     T *__restrict__ grad_psw, const int64_t *__restrict__ table_offsets,
