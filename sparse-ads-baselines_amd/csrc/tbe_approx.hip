@@ -368,6 +368,38 @@ __device__ __forceinline__ void round_lane_elements(A (&v)[E], const StochasticR
   }
 }
 
+// Stochastic rounding of a lane's E < 4 elements with Philox blocks shared inside a quad of lanes.
+// The 4 / E lanes whose elements fall into one block of four would each draw the same block for
+// an occurrence; instead they draw it for 4 / E consecutive occurrences, one each (`rnd`, drawn
+// with the occurrence's key), and for occurrence number SLOT of those a lane reads its words from
+// the quad's lane that drew them.  The words and the rounding are those of round_lane_elements.
+template <int E, int SLOT> __device__ __forceinline__ uint32_t quad_word(uint32_t v) {
+  // lanes of a quad read from lane SLOT (E == 1), or lanes 0, 1 from lane SLOT and lanes 2, 3 from lane 2 + SLOT
+  constexpr int kPattern = E == 1 ? (SLOT | SLOT << 2 | SLOT << 4 | SLOT << 6)
+                                  : (SLOT | SLOT << 2 | (2 + SLOT) << 4 | (2 + SLOT) << 6);
+  return static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), kPattern, 0xf, 0xf, true));
+}
+template <int E, int SLOT, typename A>
+__device__ __forceinline__ void round_with_shared_draw(A (&v)[E], const uint4 &rnd, int lane) {
+  static_assert(E == 1 || E == 2, "lanes that hold less than a block of four elements");
+  const uint32_t word[4] = {quad_word<E, SLOT>(rnd.x), quad_word<E, SLOT>(rnd.y), quad_word<E, SLOT>(rnd.z),
+                            quad_word<E, SLOT>(rnd.w)};
+  const int first = (lane * E) & 3;  // the lane's first element inside its block (rows start on a block)
+#pragma unroll
+  for (int i = 0; i < E; ++i) {
+    uint32_t bits = word[0];
+#pragma unroll
+    for (int x = 1; x < 4; ++x) bits = (first + i == x) ? word[x] : bits;
+    v[i] = __half2float(__float2half_rz(__uint_as_float(__float_as_uint(v[i]) + (bits >> 19))));
+  }
+}
+__device__ __forceinline__ uint4 draw_block(const StochasticRounding &sr, int64_t element) {
+  const uint64_t block = static_cast<uint64_t>(element) / 4;
+  return philox4x32_10(make_uint4(static_cast<uint32_t>(block), static_cast<uint32_t>(block >> 32),
+                                  static_cast<uint32_t>(sr.offset), static_cast<uint32_t>(sr.offset >> 32)),
+                       make_uint2(static_cast<uint32_t>(sr.seed), static_cast<uint32_t>(sr.seed >> 32)));
+}
+
 template <typename T> struct LongRowArgs {
   using A = typename AccOf<T>::type;
   const T *grad_output;
@@ -500,8 +532,11 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
     const A my_mult = lane < nb ? approx_multiplier<A>(s + incl, cur_pw, WEIGHTED, a.lr, a.eps) : A(0);
     s = s + broadcast_lane(incl, nb - 1);
 
-    // occurrence j of the batch, its gradient row in `grad`
-    auto apply = [&](const P &grad, int j) {
+    // occurrence j of the batch, its gradient row in `grad`; with stochastic rounding and fewer
+    // than four elements per lane, `shared_draw` holds the random words that this lane drew for
+    // one of the kShare occurrences around j and `slot` tells which of them j is
+    constexpr int kShare = (STOCHASTIC && E < 4) ? 4 / E : 1;
+    auto apply = [&](const P &grad, int j, const uint4 &shared_draw, int slot) {
       const A mult = broadcast_lane(my_mult, j);
       A dot = A(0);
 #pragma unroll
@@ -510,10 +545,19 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
         if constexpr (WEIGHTED) dot += w[i] * g;
         w[i] = w[i] - g * mult;
       }
-      if constexpr (STOCHASTIC)
+      if constexpr (STOCHASTIC && E < 4) {
+        if (slot == 0) round_with_shared_draw<E, 0, A>(w, shared_draw, lane);
+        else if (slot == 1) round_with_shared_draw<E, 1, A>(w, shared_draw, lane);
+        else if constexpr (E == 1) {
+          if (slot == 2) round_with_shared_draw<E, 2, A>(w, shared_draw, lane);
+          else round_with_shared_draw<E, 3, A>(w, shared_draw, lane);
+        }
+      } else if constexpr (STOCHASTIC) {
         round_lane_elements<T, E, true, A>(w, rounding_of_update(a.sr, k0 + j - seg_begin),
                                            place.row_element + lane_off);
-      else round_lane_elements<T, E, false, A>(w, a.sr, place.row_element + lane_off);
+      } else {
+        round_lane_elements<T, E, false, A>(w, a.sr, place.row_element + lane_off);
+      }
       if constexpr (WEIGHTED) {
         dot = active ? dot : A(0);
 #pragma unroll
@@ -537,9 +581,18 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
         }
 #pragma unroll
         for (int b = 0; b < kAhead; ++b) fill[b] = row_of(src, min(first + b, limit));
+        uint4 draw = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
         for (int b = 0; b < kAhead; ++b) {
-          if (j0 + b < nb) apply(use[b], j0 + b);
+          if (j0 + b < nb) {
+            if constexpr (kShare > 1) {
+              // one draw per lane serves kShare occurrences: this lane's is for occurrence b + lane % kShare
+              if (b % kShare == 0)
+                draw = draw_block(rounding_of_update(a.sr, k0 + j0 + b + (lane % kShare) - seg_begin),
+                                  place.row_element + lane_off);
+            }
+            apply(use[b], j0 + b, draw, b % kShare);
+          }
         }
       };
       // blocks are taken in pairs so that the two register sets swap roles in place; the second
@@ -555,7 +608,7 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
       // a full batch followed by a full batch: straight-line code
 #pragma unroll
       for (int j = 0; j < kWave; ++j) {
-        apply(ring[j % kRing], j);
+        apply(ring[j % kRing], j, make_uint4(0u, 0u, 0u, 0u), 0);
         if (j + kRing < kWave) ring[j % kRing] = row_of(cur_goff, j + kRing);
         else ring[j % kRing] = row_of(nxt_goff, j + kRing - kWave);
       }
@@ -563,7 +616,7 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
 #pragma unroll
       for (int j = 0; j < kWave; ++j) {
         if (j < nb) {
-          apply(ring[j % kRing], j);
+          apply(ring[j % kRing], j, make_uint4(0u, 0u, 0u, 0u), 0);
           const int target = (j + kRing) % kWave;  // occurrence j + kRing of the row ...
           if (j + kRing < kWave) {                 // ... is in this batch
             if (target < nb) ring[j % kRing] = row_of(cur_goff, target);

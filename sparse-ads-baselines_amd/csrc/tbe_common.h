@@ -161,8 +161,11 @@ template <> __device__ __forceinline__ uint2 RowVec<__half, 4>::pack() const {
 __device__ __forceinline__ uint4 philox4x32_10(uint4 ctr, uint2 key) {
 #pragma unroll
   for (int round = 0; round < 10; ++round) {
-    const uint32_t hi0 = __umulhi(0xD2511F53u, ctr.x), lo0 = 0xD2511F53u * ctr.x;
-    const uint32_t hi1 = __umulhi(0xCD9E8D57u, ctr.z), lo1 = 0xCD9E8D57u * ctr.z;
+    // (one 32 x 32 -> 64-bit multiplication per product instead of a high and a low one)
+    const uint64_t p0 = static_cast<uint64_t>(0xD2511F53u) * ctr.x;
+    const uint64_t p1 = static_cast<uint64_t>(0xCD9E8D57u) * ctr.z;
+    const uint32_t hi0 = static_cast<uint32_t>(p0 >> 32), lo0 = static_cast<uint32_t>(p0);
+    const uint32_t hi1 = static_cast<uint32_t>(p1 >> 32), lo1 = static_cast<uint32_t>(p1);
     ctr = make_uint4(hi1 ^ ctr.y ^ key.x, lo1, hi0 ^ ctr.w ^ key.y, lo0);
     key.x += 0x9E3779B9u;
     key.y += 0xBB67AE85u;
