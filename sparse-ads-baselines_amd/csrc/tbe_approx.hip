@@ -358,7 +358,7 @@ __device__ __forceinline__ void round_lane_elements(A (&v)[E], const StochasticR
 #pragma unroll
           for (int x = 1; x < 4; ++x) bits = (first + i == x) ? word[x] : bits;
           A &value = v[4 * q + i];
-          value = __half2float(__float2half_rz(__uint_as_float(__float_as_uint(value) + (bits >> 19))));
+          value = round_trip_stochastic(value, bits);
         }
       }
     } else {
@@ -390,7 +390,7 @@ __device__ __forceinline__ void round_with_shared_draw(A (&v)[E], const uint4 &r
     uint32_t bits = word[0];
 #pragma unroll
     for (int x = 1; x < 4; ++x) bits = (first + i == x) ? word[x] : bits;
-    v[i] = __half2float(__float2half_rz(__uint_as_float(__float_as_uint(v[i]) + (bits >> 19))));
+    v[i] = round_trip_stochastic(v[i], bits);
   }
 }
 __device__ __forceinline__ uint4 draw_block(const StochasticRounding &sr, int64_t element) {

@@ -182,10 +182,29 @@ struct StochasticRounding {
 // fp32 -> fp16 with stochastic rounding as in stochastic_rounding_vector
 // (table_batched_embeddings_cuda.cu:564-578): 13 random bits are added to the fp32 pattern,
 // then the value is truncated toward zero.
+// fp32 -> fp16 toward zero, bit for bit what __float2half_rz returns for every fp32 pattern (NaN
+// payloads aside) in a third of its instructions: in fp16's normal range the 13 mantissa bits it
+// has no room for are dropped, after which the conversion is exact (finite magnitudes beyond the
+// largest fp16 value stay at it); below the smallest normal value the result counts whole
+// multiples of 2^-24; infinities and NaNs convert as they are.
+__device__ __forceinline__ uint16_t float_to_half_rz_bits(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const float ax = fabsf(x);
+  const float cut = __builtin_amdgcn_fmed3f(__uint_as_float(u & 0xFFFFE000u), -65504.0f, 65504.0f);
+  const __half normal = __float2half_rn(!(ax <= 3.4028234664e38f) ? x : cut);
+  const uint32_t steps = static_cast<uint32_t>(ax * 16777216.0f);
+  const uint16_t tiny = static_cast<uint16_t>(((u >> 16) & 0x8000u) | steps);
+  return ax < 6.103515625e-05f ? tiny : __half_as_ushort(normal);
+}
+// one value rounded stochastically to fp16 and back: `word` is the element's random word
+__device__ __forceinline__ float round_trip_stochastic(float v, uint32_t word) {
+  return __half2float(__ushort_as_half(float_to_half_rz_bits(__uint_as_float(__float_as_uint(v) + (word >> 19)))));
+}
+
 __device__ __forceinline__ uint32_t floats_to_half2_stochastic(float lo, float hi, uint32_t r0, uint32_t r1) {
-  const __half a = __float2half_rz(__uint_as_float(__float_as_uint(lo) + (r0 >> 19)));
-  const __half b = __float2half_rz(__uint_as_float(__float_as_uint(hi) + (r1 >> 19)));
-  return static_cast<uint32_t>(__half_as_ushort(a)) | (static_cast<uint32_t>(__half_as_ushort(b)) << 16);
+  const uint16_t a = float_to_half_rz_bits(__uint_as_float(__float_as_uint(lo) + (r0 >> 19)));
+  const uint16_t b = float_to_half_rz_bits(__uint_as_float(__float_as_uint(hi) + (r1 >> 19)));
+  return static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 16);
 }
 
 // VEC accumulator values packed into the stored type: round to nearest even, or, for fp16 with
