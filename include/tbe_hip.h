@@ -305,6 +305,13 @@ TBE_API int tbe_construct_offsets(const int32_t *batch_offsets_per_table,
                           const int32_t *total_indices_per_table,
                           int32_t T, int32_t B, int32_t *output, void *stream);
 
+/* Stage entry point for tests: out[i] = fp16 bit pattern of values[i] rounded stochastically with
+ * the random word random_words[i], the element rule of stochastic_rounding_vector
+ * (table_batched_embeddings_cuda.cu:564-578: the word's top 13 bits are added to the fp32 pattern,
+ * the sum is converted toward zero) as every kernel here that rounds stochastically applies it. */
+TBE_API int tbe_stochastic_round(const float *values, const uint32_t *random_words, uint16_t *out,
+                                 int64_t n, void *stream);
+
 /* ---------------------------------------------- per-table embedding dimension
  * The reference's MixedDim path (table_batched_embeddings_ops.py:204-435):
  *   weights            1-D; table t occupies elements [table_offsets[t], table_offsets[t+1]),

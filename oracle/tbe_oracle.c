@@ -152,6 +152,10 @@ uint16_t oracle_stochastic_round(float value, uint32_t random_bits) {
   return float_to_half_rz(f);
 }
 
+void oracle_stochastic_round_many(const float *values, const uint32_t *random_bits, uint16_t *out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) out[i] = oracle_stochastic_round(values[i], random_bits[i]);
+}
+
 /* Stores `count` (a multiple of 4) fp16 values starting at table element `element` (a multiple
  * of 4): element e takes word e % 4 of Philox(counter = {e / 4, offset}, key = seed). */
 static void store_row_stochastic(uint16_t *dst, const float *values, int32_t count, int64_t element,

@@ -292,6 +292,16 @@ def stochastic_round(value, random_bits):
     return fn(float(value), int(random_bits))
 
 
+def stochastic_round_many(values, random_bits):
+    """oracle_stochastic_round over arrays: float32 values, uint32 words -> uint16 fp16 patterns."""
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    random_bits = np.ascontiguousarray(random_bits, dtype=np.uint32)
+    out = np.empty(values.shape, np.uint16)
+    lib().oracle_stochastic_round_many(values.ctypes.data_as(ctypes.c_void_p), random_bits.ctypes.data_as(ctypes.c_void_p),
+                                       out.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(values.size))
+    return out
+
+
 # ------------------------------------------------------ interleaved [E][T][D] tables
 def forward_etd(weights, indices, offsets):
     """weights float32 [E, T, D]; offsets flattened [B*T+1] -> output [B, T, D]."""

@@ -3,6 +3,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <algorithm>
 #include <mutex>
 #include <vector>
 
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(kBlockThreads) void construct_offsets_kernel(
 
 extern "C" const char *tbe_last_error(void) { return tbe::g_last_error; }
 
-extern "C" int32_t tbe_abi_version(void) { return 14; }
+extern "C" int32_t tbe_abi_version(void) { return 15; }
 
 extern "C" int tbe_profile_begin(void) {
   using namespace tbe;
@@ -130,6 +131,30 @@ extern "C" int tbe_profile_get(int32_t i, const char **name, float *milliseconds
   *name = g_profile[i].name;
   *milliseconds = g_profile[i].ms;
   return TBE_OK;
+}
+
+namespace tbe {
+namespace {
+__global__ __launch_bounds__(kBlockThreads) void stochastic_round_kernel(const float *__restrict__ values,
+                                                                        const uint32_t *__restrict__ words,
+                                                                        uint16_t *__restrict__ out, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < n; i += stride)
+    out[i] = static_cast<uint16_t>(floats_to_half2_stochastic(values[i], 0.0f, words[i], 0u) & 0xffffu);
+}
+}  // namespace
+}  // namespace tbe
+
+extern "C" int tbe_stochastic_round(const float *values, const uint32_t *random_words, uint16_t *out,
+                                    int64_t n, void *stream) {
+  using namespace tbe;
+  TBE_REQUIRE(n >= 0, "tbe_stochastic_round: n must not be negative");
+  if (n == 0) return TBE_OK;
+  TBE_REQUIRE(values && random_words && out, "tbe_stochastic_round: null pointer argument");
+  const dim3 grid(static_cast<unsigned>(std::min<int64_t>(ceil_div(n, kBlockThreads), 256 * 16)));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  TBE_LAUNCH("stochastic_round", s, stochastic_round_kernel, grid, dim3(kBlockThreads), values, random_words, out, n);
+  return check_launch("tbe_stochastic_round");
 }
 
 extern "C" int tbe_construct_offsets(const int32_t *batch_offsets_per_table,

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -99,6 +99,7 @@ SIGNATURES = {
     "tbe_segments_workspace_bytes": (_u64, [_i64]),
     "tbe_find_segments": (ctypes.c_int, [_c_i32p, _i64, _c_i32p, _c_i32p, _vp, _u64, _vp]),
     "tbe_construct_offsets": (ctypes.c_int, [_c_i32p, _c_i32p, _i32, _i32, _c_i32p, _vp]),
+    "tbe_stochastic_round": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp]),
     "tbe_forward_mixed": (ctypes.c_int, [_vp, _i32, _i32, _vp, _c_i32p, _i32, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp,
                                          _vp, _vp]),
     "tbe_backward_mixed": (ctypes.c_int, [_i32, _vp, _vp, _i32, _i32, _i64, _i64, _vp, _c_i32p, _c_i32p, _i32, _i32,

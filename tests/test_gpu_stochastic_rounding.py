@@ -85,6 +85,35 @@ def test_reproducible_per_stream_and_unbiased():
     assert bias_sr.mean() < 0.08 and bias_sr.mean() < 0.5 * bias_rn.mean()
 
 
+def test_rounding_rule_matches_the_oracle_bit_for_bit(oracle):
+    """tbe_stochastic_round applies the kernels' element rule (random bits added to the fp32 pattern, then
+    a conversion toward zero done on bit patterns) to arrays: four million patterns over all exponents with
+    random words, the fp16 subnormal range, the largest finite values and the first that overflow."""
+    rs = np.random.RandomState(6)
+    bits = np.concatenate([
+        rs.randint(0, 2 ** 32, size=4_000_000, dtype=np.uint64).astype(np.uint32),
+        np.arange(0x33000000, 0x38900000, 211, dtype=np.uint32),
+        np.arange(0xb3000000, 0xb8900000, 211, dtype=np.uint32),
+        np.arange(0x477fc000, 0x47802000, dtype=np.uint32),
+        np.array([0, 0x80000000, 0x7f7fffff, 0xff7fffff, 0x7f800000, 0xff800000, 1, 0x80000001], np.uint32)])
+    words = rs.randint(0, 2 ** 32, size=bits.size, dtype=np.uint64).astype(np.uint32)
+    words[::7] = 0
+    words[3::7] = 0xffffffff
+    values = bits.view(np.float32)
+    out = torch.empty(bits.size, dtype=torch.int16, device=DEV)
+    v, w = dev(values), torch.from_numpy(words.view(np.int32)).to(DEV)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    tbe_native.check(tbe_native.load().tbe_stochastic_round(vp(v), vp(w), vp(out), bits.size,
+                                                            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.uint16)
+    want = oracle.stochastic_round_many(values, words)
+    summed = (bits.astype(np.uint64) + (words >> 19)).astype(np.uint32).view(np.float32)   # what gets converted
+    nan = np.isnan(summed)
+    assert got[~nan].tobytes() == want[~nan].tobytes()
+    assert bool(np.isnan(got[nan].view(np.float16)).all())
+
+
 def test_module_with_stochastic_rounding_like_the_reference_test(oracle):
     """test_backward_adagrad with stochastic_rounding=True, fp16 (test_table_batched_embeddings.py:
     219-318): state and weights within the reference's own 1e-3 tolerances of the exact update."""

@@ -411,6 +411,28 @@ def test_stochastic_round_rule(oracle):
     assert half(oracle.stochastic_round(-x, 0)) == -lo and half(oracle.stochastic_round(-x, 0xffffffff)) == -hi
 
 
+def test_conversion_toward_zero_against_numpy(oracle):
+    """With a zero random word the rule is the plain fp32 -> fp16 conversion toward zero.  numpy
+    converts to nearest; where that landed beyond the value, the neighbour toward zero is the
+    answer.  Two million bit patterns over all exponents, plus the fp16 subnormal range, the
+    largest finite values and the first values that overflow."""
+    rs = np.random.RandomState(5)
+    bits = np.concatenate([
+        rs.randint(0, 2 ** 32, size=2_000_000, dtype=np.uint64).astype(np.uint32),
+        np.arange(0x33000000, 0x38900000, 977, dtype=np.uint32),          # 2^-25 ... 2^-14 and a bit beyond
+        np.arange(0x477fd000, 0x47801000, dtype=np.uint32),               # around 65504 ... 65536
+        np.array([0, 0x80000000, 0x7f7fffff, 0xff7fffff, 0x7f800000, 0xff800000, 1, 0x80000001], np.uint32)])
+    x = bits.view(np.float32)
+    keep = ~np.isnan(x)
+    x = x[keep]
+    got = oracle.stochastic_round_many(x, np.zeros(x.size, np.uint32)).view(np.float16)
+    with np.errstate(over="ignore"):
+        near = x.astype(np.float16)
+    beyond = np.abs(near.astype(np.float64)) > np.abs(x.astype(np.float64))
+    want = np.where(beyond, np.nextafter(near, np.float16(0)), near)
+    assert want.view(np.uint16).tobytes() == got.view(np.uint16).tobytes()
+
+
 def test_stochastic_backward_is_within_one_ulp_and_reproducible(oracle):
     p = make_problem(31, T=2, E=40, D=16, B=30, L=6, dtype=np.float16, zipf=1.3)
     runs = []
