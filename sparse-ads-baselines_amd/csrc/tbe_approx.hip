@@ -498,6 +498,8 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
   asm volatile("" : "+v"(aft_pos), "+v"(nxt_goff), "+v"(nxt_pw), "+v"(nxt_wss) : : "memory");
 
   const uint32_t lane_bytes = static_cast<uint32_t>(lane_off) * static_cast<uint32_t>(sizeof(T));
+  // (a raw buffer over grad_output: no stride, its size in bytes, 32-bit data format -- reads past
+  // the end return zero)
   const __amdgpu_buffer_rsrc_t grad_buffer = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T *>(a.grad_output), 0, static_cast<int>(static_cast<uint32_t>(BIG ? 0 : a.grad_bytes)), 0x00020000);
   auto row_of = [&](Off goffs, int src_lane) {
