@@ -228,6 +228,59 @@ def test_full_size_approx_adagrad_against_the_fp64_closed_form(oracle, weighted)
 
 
 @pytest.mark.timeout(600)
+def test_full_size_weighted_fp16_approx_adagrad_properties(oracle):
+    """The shape of bench.py --config 4 (T=32, E=1e6, D=64 fp16, B=8192, bag lengths uniform in [0, 40] with
+    empty bags, per-sample weights, Zipf(1.2): 5.2 M lookups, the hottest row of a table some 29 000 times)
+    with the approximate optimizer.  fp16 rows are rounded after every lookup, so the weights have no closed
+    form; size-independent properties instead: the state of every row grows by the sum of its lookups'
+    ||g||^2 * psw^2 (fp64 sum at 1e-5), rows without a lookup keep their bits, reruns are bit-identical, and the
+    first table's rows, state and per-sample-weight gradients equal the oracle's serial walk."""
+    T, E, D, B = 32, 1000000, 64, 8192
+    lr, eps = 0.01, 0.1
+    rs = np.random.RandomState(42)
+    lengths = rs.randint(0, 41, size=(T, B))
+    offsets_np = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
+    n = int(offsets_np[-1])
+    idx_np = (rs.zipf(1.2, size=n) % E).astype(np.int32)
+    gen = torch.Generator(device=DEV).manual_seed(42)
+    W0 = torch.empty(T * E, D, device=DEV).uniform_(-0.01, 0.01, generator=gen).half()
+    go = (torch.randn(B, T, D, device=DEV, generator=gen) * 0.1).half()
+    state0 = torch.empty(T * E, device=DEV).uniform_(0.0, 2.0, generator=gen)
+    psw = torch.empty(n, device=DEV).uniform_(0.0, 1.0, generator=gen).half()
+    idx, offsets = torch.from_numpy(idx_np).to(DEV), torch.from_numpy(offsets_np).to(DEV)
+    table_offsets = torch.arange(T, dtype=torch.int32, device=DEV) * E
+
+    def run():
+        W, state = W0.clone(), state0.clone()
+        g = ext.backward_approx_adagrad(go, W, table_offsets, idx, offsets, psw, state, lr, eps, 200, False, 1)
+        torch.cuda.synchronize()
+        return W, state, g
+
+    W, state, g_psw = run()
+    W2, state2, g2 = run()
+    assert torch.equal(W, W2) and torch.equal(state, state2) and torch.equal(g_psw, g2)
+    bag_of = torch.repeat_interleave(torch.arange(T * B, device=DEV), torch.from_numpy(lengths.reshape(-1)).to(DEV))
+    t_of, b_of = bag_of // B, bag_of % B
+    key = idx.long() + t_of * E
+    wss = (go.double() ** 2).sum(-1)[b_of, t_of] * psw.double() ** 2
+    want_state = state0.double().index_add(0, key, wss)
+    assert_close(state.cpu().numpy(), want_state.cpu().numpy(), 1e-5, "state")
+    touched = torch.zeros(T * E, dtype=torch.bool, device=DEV)
+    touched[key] = True
+    assert torch.equal(W[~touched], W0[~touched]) and torch.equal(state[~touched], state0[~touched])
+    assert int(torch.bincount(idx[:int(offsets_np[B])].long()).max()) > 20000
+    # the first table against the oracle
+    n0 = int(offsets_np[B])
+    w_ref = W0[:E].cpu().numpy().copy()
+    st_ref = state0[:E].cpu().numpy().copy()
+    g_ref = oracle.backward_approx(go[:, :1, :].contiguous().cpu().numpy(), w_ref, np.zeros(1, np.int32), idx_np[:n0],
+                                   offsets_np[:B + 1], lr, eps, st_ref, psw[:n0].cpu().numpy(), None)
+    assert_close(state[:E].cpu().numpy(), st_ref, 1e-5, "first table's state")
+    assert_close(W[:E].float().cpu().numpy(), w_ref.astype(np.float32), 1e-2, "first table")
+    assert_close(g_psw[:n0].float().cpu().numpy(), g_ref.astype(np.float32), 2e-2, "first table's per-sample-weight gradients")
+
+
+@pytest.mark.timeout(600)
 def test_full_size_mixed_D_approx_adagrad_against_the_fp64_closed_form():
     """The mixed-D benchmark's shape (64 tables of 1e5 rows, widths 64 ... 192 in steps of 4, fp32, B=4096,
     L=20, Zipf(1.05)) against the same closed form, table by table."""
