@@ -385,6 +385,15 @@ TBE_API int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void 
  *      backing table.  A staged row thus crosses the host link once in each
  *      direction per step, however many lookups hit it (an uncached row is read
  *      once per lookup in the forward and read and written once in the backward).
+ * Deferred write-back (stage_of_row given): step 6 is put off to the next tbe_cache_prepare, and
+ * `rows` holds TWO staging areas that take turns (a step with an odd number stages into rows
+ * [num_sets * 64 + stage_slots, num_sets * 64 + 2 * stage_slots), an even one into the area before
+ * it).  In step 4 of the next call a row that is fetched again is read from the staging row that
+ * still holds it instead of from the backing table, and is not written back at all (its slot or new
+ * staging row holds the newer copy); the staged rows that are not fetched again are written back in
+ * the same launch as the fetches, so both directions of the host link are busy at once.
+ * tbe_cache_flush writes back whatever is still pending.  Until then the backing table's copy of a
+ * staged row is stale, like that of a cached row.
  * The resulting tags / slots are a pure function of the key sequence, so a CPU
  * model can reproduce them bit for bit (a staged row is an uncached row of the
  * model; its staging index is the rank of the miss inside its set plus the number
@@ -402,6 +411,11 @@ typedef struct tbe_cache {
   int64_t num_sets;
   int32_t policy;       /* TBE_CACHE_LRU or TBE_CACHE_LFU                                */
   int64_t stage_slots;  /* rows of the staging area (0 = none); num_sets * 64 + stage_slots < 2^31 */
+  /* deferred write-back of staged rows (all null / 0: staged rows go back right after the update) */
+  int32_t *stage_of_row;  /* [total_rows] row of `rows` that has held the row since the last step, -1 = none;
+                           * then `rows` is [num_sets * 64 + 2 * stage_slots][D]                       */
+  int32_t *stage_keys;    /* [2 * stage_slots] key held by each staging row, -1 = none                 */
+  int64_t total_rows;     /* rows of the backing table                                                 */
 } tbe_cache_t;
 
 /* Byte offsets into the cache workspace (separate from the backward workspace). */
@@ -415,13 +429,15 @@ typedef struct tbe_cache_workspace_layout {
   uint64_t set_counts;     /* int32 [num_sets] misses per set                                  */
   uint64_t set_fill;       /* int32 [num_sets]                                                 */
   uint64_t set_starts;     /* int32 [num_sets + 1]                                             */
-  uint64_t stats;          /* int32 [8]: unique rows, hits, misses, inserted, written back, uncached, staged */
+  uint64_t stats;          /* int32 [8]: unique rows, hits, misses, inserted, written back, uncached, staged,
+                            * fetched from a staging row (deferred write-back)                  */
+  uint64_t fetch_source;   /* int32 [U]  deferred write-back: row of `rows` a fetched row comes from, -1 = backing table */
 } tbe_cache_workspace_layout_t;
 
 TBE_API int tbe_cache_workspace_layout(int64_t num_indices, int64_t num_sets,
                                        tbe_cache_workspace_layout_t *layout);
 
-/* Empties the cache: tags = -1, last_used = use_count = 0. */
+/* Empties the cache: tags = -1, last_used = use_count = 0 (and stage_of_row = stage_keys = -1). */
 TBE_API int tbe_cache_init(const tbe_cache_t *cache, void *stream);
 
 /* Steps 1-5 above.  `workspace` is a backward workspace (tbe_backward_workspace_layout)

@@ -10,6 +10,9 @@
 //   insert   one wavefront per set: for each missing row in ascending order, victim = lowest
 //            (priority, way) among slots not used in this step (wavefront min + ballot)
 //   fill     (side stream) write back the evicted row, fetch the new row over the host link
+//            (deferred write-back, cache->stage_of_row: or from the staging row that has held it
+//            since the step before; beside it, in the same launch, the rows staged by the step
+//            before that this step does not fetch go back to the backing table)
 //   locate   slot of every lookup position, for the forward gather
 // Every decision is a function of integers only, so the tags after a step are reproducible.
 
@@ -35,7 +38,8 @@ __device__ __forceinline__ uint32_t cache_set_of(uint32_t key, uint32_t num_sets
   return static_cast<uint32_t>((static_cast<uint64_t>(h) * num_sets) >> 32);
 }
 
-enum { kStatUnique = 0, kStatHits, kStatMisses, kStatInserted, kStatWrittenBack, kStatUncached, kStatStaged };
+enum { kStatUnique = 0, kStatHits, kStatMisses, kStatInserted, kStatWrittenBack, kStatUncached, kStatStaged,
+       kStatFromStaging };
 
 __global__ __launch_bounds__(kBlockThreads) void cache_fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
@@ -150,7 +154,8 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
     int64_t num_sets, int32_t policy, int32_t step, const int32_t *__restrict__ keys_sorted,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ set_starts,
     const int32_t *__restrict__ miss_list, int32_t *__restrict__ unique_slots,
-    int32_t *__restrict__ evicted_keys, int32_t *__restrict__ stats, int64_t stage_slots) {
+    int32_t *__restrict__ evicted_keys, int32_t *__restrict__ stats, int64_t stage_slots,
+    int64_t stage_base) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
@@ -189,7 +194,7 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
         const int64_t stage = static_cast<int64_t>(begin) + staged_in_set;
         if (stage < stage_slots) {
           if (lane == 0) {
-            unique_slots[u] = static_cast<int32_t>(num_sets * kWays + stage);
+            unique_slots[u] = static_cast<int32_t>(stage_base + stage);
             evicted_keys[u] = -1;
           }
           ++staged_in_set;
@@ -225,27 +230,121 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
   }
 }
 
+// Deferred write-back, after the step's slots are decided: where each row that this step fetches
+// comes from, and where the rows that it stages are.  A fetched row that the step before staged
+// is still in that step's staging row: fetch_source[u] = that row of `rows` (else -1: the backing
+// table), and the entry of the staging row is marked consumed (-(key + 2)) so that it is not
+// written back.  A row staged now is entered into stage_of_row / stage_keys.
+__global__ __launch_bounds__(kBlockThreads) void cache_resolve_kernel(
+    const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
+    const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
+    const int32_t *__restrict__ evicted_keys, int32_t *__restrict__ stage_of_row,
+    int32_t *__restrict__ stage_keys, int32_t *__restrict__ fetch_source, int64_t num_slots,
+    int32_t *__restrict__ stats) {
+  const int U = counters[0];
+  int from_staging = 0;
+  for (int64_t u = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; u < U;
+       u += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    if (evicted_keys[u] == -2) continue;  // a hit, or a row left in the backing table
+    const int32_t key = keys_sorted[segment_starts[u]];
+    const int32_t slot = unique_slots[u];
+    const int32_t held = stage_of_row[key];
+    fetch_source[u] = held;
+    if (held >= 0) {
+      stage_keys[held - num_slots] = -(key + 2);
+      ++from_staging;
+    }
+    if (slot >= num_slots) {
+      stage_of_row[key] = slot;
+      stage_keys[slot - num_slots] = key;
+    } else if (held >= 0) {
+      stage_of_row[key] = -1;  // the row lives in a slot of the cache now
+    }
+  }
+  for (int m = kWave / 2; m > 0; m >>= 1) from_staging += __shfl_xor(from_staging, m, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0 && from_staging) atomicAdd(&stats[kStatFromStaging], from_staging);
+}
+
 // One wavefront per row; rows move as 8-byte units (row_units = D * element size / 8).
+// fetch_source (deferred write-back): per unique row, the row of `rows` to fetch it from, or -1.
+// old_stage_keys (deferred write-back): the launch also carries the write-back of the step
+// before -- workgroups with an odd index copy the rows of that step's staging area whose entry
+// holds a key (not consumed, not empty) to the backing table, so that both directions of the
+// host link are busy at once; the workgroups with an even index fetch.
 __global__ __launch_bounds__(kBlockThreads) void cache_fill_kernel(
     uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
     const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
-    const int32_t *__restrict__ evicted_keys) {
+    const int32_t *__restrict__ evicted_keys, const int32_t *__restrict__ fetch_source,
+    const int32_t *__restrict__ old_stage_keys, int64_t old_stage_base, int64_t stage_slots) {
   const int lane = threadIdx.x & (kWave - 1);
+  int64_t block = blockIdx.x, blocks = gridDim.x;
+  if (old_stage_keys) {
+    const bool writes_back = block & 1;
+    block >>= 1;
+    blocks >>= 1;  // (the grid has an even number of workgroups)
+    if (writes_back) {
+      const int64_t wave_id = block * kWavesPerBlock + (threadIdx.x >> 6);
+      const int64_t stride = blocks * kWavesPerBlock;
+      for (int64_t i = wave_id; i < stage_slots; i += stride) {
+        const int64_t key = old_stage_keys[i];
+        if (key < 0) continue;
+        const uint64_t *src = cache_rows + (old_stage_base + i) * row_units;
+        uint64_t *dst = backing_rows + key * row_units;
+        for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
+      }
+      return;
+    }
+  }
   const int U = counters[0];
-  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  const int64_t wave_id = block * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = blocks * kWavesPerBlock;
   for (int64_t u = wave_id; u < U; u += stride) {
     const int32_t evicted = evicted_keys[u];
     if (evicted == -2) continue;
     const int64_t key = keys_sorted[segment_starts[u]];
     uint64_t *slot_row = cache_rows + static_cast<int64_t>(unique_slots[u]) * row_units;
     const uint64_t *new_row = backing_rows + key * row_units;
+    if (fetch_source) {
+      const int64_t held = fetch_source[u];
+      if (held >= 0) new_row = cache_rows + held * row_units;
+    }
     if (evicted >= 0) {
       uint64_t *old_row = backing_rows + static_cast<int64_t>(evicted) * row_units;
       for (int i = lane; i < row_units; i += kWave) old_row[i] = slot_row[i];
     }
     for (int i = lane; i < row_units; i += kWave) slot_row[i] = new_row[i];
+  }
+}
+
+// Deferred write-back, outside a step (flush): the rows of a staging area that hold a key.
+__global__ __launch_bounds__(kBlockThreads) void cache_unstage_area_kernel(
+    const uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    const int32_t *__restrict__ stage_keys, int64_t stage_base, int64_t stage_slots) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  for (int64_t i = wave_id; i < stage_slots; i += stride) {
+    const int64_t key = stage_keys[i];
+    if (key < 0) continue;
+    const uint64_t *src = cache_rows + (stage_base + i) * row_units;
+    uint64_t *dst = backing_rows + key * row_units;
+    for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
+  }
+}
+
+// Deferred write-back: the staging area of the step before is released -- its entries are
+// emptied, and stage_of_row forgets the rows it held unless they have been staged again since.
+__global__ __launch_bounds__(kBlockThreads) void cache_retire_stage_kernel(
+    int32_t *__restrict__ stage_of_row, int32_t *__restrict__ old_stage_keys, int64_t old_stage_base,
+    int64_t stage_slots) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < stage_slots;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int32_t entry = old_stage_keys[i];
+    if (entry == -1) continue;
+    const int32_t key = entry >= 0 ? entry : -(entry + 2);
+    if (stage_of_row[key] == old_stage_base + i) stage_of_row[key] = -1;
+    old_stage_keys[i] = -1;
   }
 }
 
@@ -306,6 +405,7 @@ void cache_layout(int64_t n, int64_t num_sets, tbe_cache_workspace_layout_t *l) 
   l->set_fill = off; off += sets;
   l->set_starts = off; off += sets;
   l->stats = off; off += 256;
+  l->fetch_source = off; off += ints;
   l->total_bytes = off;
 }
 
@@ -322,7 +422,27 @@ int validate_cache(const char *name, const tbe_cache_t *cache) {
               "%s: stage_slots out of range", name);
   TBE_REQUIRE(cache->policy == TBE_CACHE_LRU || cache->policy == TBE_CACHE_LFU, "%s: bad policy %d", name,
               cache->policy);
+  if (cache->stage_of_row) {
+    TBE_REQUIRE(cache->stage_keys && cache->total_rows > 0 && cache->total_rows < INT32_MAX,
+                "%s: deferred write-back needs stage_keys and total_rows", name);
+    TBE_REQUIRE(cache->num_sets * kWays + 2 * cache->stage_slots < INT32_MAX, "%s: stage_slots out of range", name);
+  }
   return TBE_OK;
+}
+
+// Deferred write-back: the rows of the staging area at `stage_base` that still wait for their
+// write-back go to the backing table, and the area is released.
+void write_back_stage(const tbe_cache_t *cache, int row_units, int64_t half, hipStream_t stream) {
+  const int64_t base = cache->num_sets * kWays + half * cache->stage_slots;
+  int32_t *keys = cache->stage_keys + half * cache->stage_slots;
+  // (the fetching half of the launch finds no rows: a null counter block is not read with U = 0)
+  TBE_LAUNCH("cache_unstage", stream, cache_unstage_area_kernel,
+             dim3(grid_for(cache->stage_slots, kWavesPerBlock, 256 * 16)), dim3(kBlockThreads),
+             static_cast<const uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units, keys,
+             base, cache->stage_slots);
+  TBE_LAUNCH("cache_retire_stage", stream, cache_retire_stage_kernel,
+             dim3(grid_for(cache->stage_slots, kBlockThreads, 1024)), dim3(kBlockThreads), cache->stage_of_row, keys,
+             base, cache->stage_slots);
 }
 
 // One event per calling thread, used to order the two streams.
@@ -340,6 +460,7 @@ int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int3
                   const int32_t *segment_starts, const int32_t *counters,
                   const int32_t *unique_slots, int64_t num_indices, hipStream_t stream) {
   if (cache->stage_slots <= 0 || num_indices == 0) return TBE_OK;
+  if (cache->stage_of_row) return TBE_OK;  // deferred: the next tbe_cache_prepare (or a flush) writes them back
   const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
   TBE_LAUNCH("cache_unstage", stream, cache_unstage_kernel,
              dim3(grid_for(num_indices, kWavesPerBlock, 256 * 16)), dim3(kBlockThreads),
@@ -370,6 +491,13 @@ extern "C" int tbe_cache_init(const tbe_cache_t *cache, void *stream) {
   TBE_LAUNCH("cache_init", s, cache_fill_i32_kernel, grid, block, cache->tags, slots, -1);
   TBE_LAUNCH("cache_init", s, cache_fill_i32_kernel, grid, block, cache->last_used, slots, 0);
   TBE_LAUNCH("cache_init", s, cache_fill_i32_kernel, grid, block, cache->use_count, slots, 0);
+  if (cache->stage_of_row) {
+    TBE_LAUNCH("cache_init", s, cache_fill_i32_kernel, dim3(grid_for(cache->total_rows, kBlockThreads, 4096)), block,
+               cache->stage_of_row, cache->total_rows, -1);
+    TBE_LAUNCH("cache_init", s, cache_fill_i32_kernel,
+               dim3(grid_for(2 * cache->stage_slots + 1, kBlockThreads, 4096)), block, cache->stage_keys,
+               2 * cache->stage_slots, -1);
+  }
   return check_launch("tbe_cache_init");
 }
 
@@ -410,6 +538,13 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
   int32_t *stats = i32(cw, cl.stats);
   const dim3 block(kBlockThreads);
   TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(1), block, stats, static_cast<int64_t>(8), 0);
+  const int unit_count = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
+  if (cache->stage_of_row && cache->stage_slots > 0) {
+    // deferred write-back: the area this step stages into must be empty.  It is, when steps are
+    // numbered consecutively (the step before the last released it); otherwise its rows go back now.
+    write_back_stage(cache, unit_count, step & 1, s);
+    if (num_indices == 0) write_back_stage(cache, unit_count, 1 - (step & 1), s);
+  }
   if (num_indices == 0) return check_launch(name);
 
   int rc = build_plan(l, workspace, table_offsets, T, indices, num_indices, offsets, B, total_rows, max_table_rows, s);
@@ -418,6 +553,13 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
   const int32_t *segment_starts = i32(ws, l.segment_starts);
   const int32_t *counters = i32(ws, l.num_unique);
   const int64_t num_sets = cache->num_sets;
+  const int64_t num_slots = num_sets * kWays;
+  // deferred write-back: two staging areas take turns; this step stages into one while the rows
+  // the step before left in the other are fetched from there or written back
+  const bool deferred = cache->stage_of_row != nullptr && cache->stage_slots > 0;
+  const int64_t half = deferred ? (step & 1) : 0;
+  const int64_t stage_base = num_slots + half * cache->stage_slots;
+  const int64_t old_stage_base = num_slots + (1 - half) * cache->stage_slots;
 
   TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(grid_for(2 * (num_sets + 1), kBlockThreads, 1024)),
              block, i32(cw, cl.set_counts), static_cast<int64_t>((cl.set_starts - cl.set_counts) / 4), 0);
@@ -433,7 +575,11 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
   TBE_LAUNCH("cache_insert", s, cache_insert_kernel, dim3(grid_for(num_sets, kWavesPerBlock, 256 * 16)), block,
              cache->tags, cache->last_used, cache->use_count, num_sets, cache->policy, step, keys_sorted,
              segment_starts, i32(cw, cl.set_starts), i32(cw, cl.miss_list), i32(cw, cl.unique_slots),
-             i32(cw, cl.evicted_keys), stats, cache->stage_slots);
+             i32(cw, cl.evicted_keys), stats, cache->stage_slots, stage_base);
+  if (deferred)
+    TBE_LAUNCH("cache_resolve", s, cache_resolve_kernel, dim3(grid_for(num_indices, kBlockThreads, 256 * 16)), block,
+               keys_sorted, segment_starts, counters, i32(cw, cl.unique_slots), i32(cw, cl.evicted_keys),
+               cache->stage_of_row, cache->stage_keys, i32(cw, cl.fetch_source), num_slots, stats);
 
   // Row traffic over the host link goes to the side stream while this stream builds the
   // per-lookup slot table; the side stream is joined before anything reads the cached rows.
@@ -443,10 +589,17 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
   if (e == hipSuccess) e = hipStreamWaitEvent(side, ready, 0);
   if (e != hipSuccess) return fail(TBE_ERR_HIP, "%s: %s", name, hipGetErrorString(e));
   const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
-  TBE_LAUNCH("cache_fill", side, cache_fill_kernel, dim3(grid_for(num_indices, kWavesPerBlock, 256 * 16)),
-             block, static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows),
-             row_units, keys_sorted, segment_starts, counters, i32(cw, cl.unique_slots),
-             i32(cw, cl.evicted_keys));
+  int32_t *old_stage_keys = deferred ? cache->stage_keys + (1 - half) * cache->stage_slots : nullptr;
+  TBE_LAUNCH("cache_fill", side, cache_fill_kernel,
+             dim3((deferred ? 2 : 1) * grid_for(num_indices, kWavesPerBlock, 256 * 16)), block,
+             static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units,
+             keys_sorted, segment_starts, counters, i32(cw, cl.unique_slots), i32(cw, cl.evicted_keys),
+             deferred ? i32(cw, cl.fetch_source) : static_cast<int32_t *>(nullptr), old_stage_keys, old_stage_base,
+             cache->stage_slots);
+  if (deferred)
+    TBE_LAUNCH("cache_retire_stage", side, cache_retire_stage_kernel,
+               dim3(grid_for(cache->stage_slots, kBlockThreads, 1024)), block, cache->stage_of_row, old_stage_keys,
+               old_stage_base, cache->stage_slots);
   TBE_LAUNCH("cache_locate", s, cache_locate_kernel, dim3(grid_for(num_indices, kBlockThreads, 256 * 16)), block,
              i32(ws, l.positions_sorted), i32(ws, l.segment_ids), i32(cw, cl.unique_slots), num_indices,
              i32(cw, cl.lookup_slots));
@@ -464,6 +617,11 @@ extern "C" int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t slots = cache->num_sets * kWays;
   const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
+  if (cache->stage_of_row && cache->stage_slots > 0) {
+    // the rows the last step staged (one of the two areas; the other is empty)
+    write_back_stage(cache, row_units, 0, s);
+    write_back_stage(cache, row_units, 1, s);
+  }
   TBE_LAUNCH("cache_flush", s, cache_flush_kernel, dim3(grid_for(slots, kWavesPerBlock, 256 * 16)),
              dim3(kBlockThreads), cache->tags, static_cast<const uint64_t *>(cache->rows),
              static_cast<uint64_t *>(cache->backing_rows), row_units, slots);

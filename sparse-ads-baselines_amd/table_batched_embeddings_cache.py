@@ -15,7 +15,7 @@ from table_batched_embeddings import max_table_rows as _max_table_rows
 _DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F16,
                 torch.float64: _native.DTYPE_F64}
 _POLICIES = {"lru": _native.CACHE_LRU, "lfu": _native.CACHE_LFU}
-STAT_NAMES = ("unique_rows", "hits", "misses", "inserted", "written_back", "uncached", "staged")
+STAT_NAMES = ("unique_rows", "hits", "misses", "inserted", "written_back", "uncached", "staged", "from_staging")
 
 
 def _ptr(t):
@@ -23,13 +23,17 @@ def _ptr(t):
 
 
 class RowCache:
-    def __init__(self, backing_weights, cache_slots, policy="lru", stage_slots=0):
+    def __init__(self, backing_weights, cache_slots, policy="lru", stage_slots=0, deferred_write_back=True):
         """backing_weights: [rows, D] tensor whose storage is device-visible host memory
         (table_batched_embeddings.new_host_mapped_tensor) -- or plain device memory, which is
         useful for tests.  cache_slots is rounded down to a multiple of 64 (one set).
         stage_slots: rows of HBM that hold, for one step, the rows no slot could take (every way
         of their set already serves the step): they then cross the host link once per step and
-        direction instead of once per lookup.  Sized for the misses of a step it stages them all."""
+        direction instead of once per lookup.  Sized for the misses of a step it stages them all.
+        deferred_write_back (with a staging area): staged rows go back to the table during the NEXT
+        prepare(), beside its fetches, so that both directions of the host link work at once; a row
+        that the next batch needs again is taken from its staging row and not written back at all.
+        This takes a second staging area and four bytes per row of the table in HBM."""
         if policy not in _POLICIES:
             raise ValueError("cache policy must be 'lru' or 'lfu'")
         if not backing_weights.is_cuda or backing_weights.dim() != 2 or not backing_weights.is_contiguous():
@@ -48,9 +52,17 @@ class RowCache:
         self.stage_slots = int(stage_slots)
         if self.stage_slots < 0:
             raise ValueError("stage_slots must not be negative")
-        self.rows = torch.empty(slots + self.stage_slots, self.D, dtype=backing_weights.dtype, device=self.device)
+        self.deferred_write_back = bool(deferred_write_back) and self.stage_slots > 0
+        areas = 2 if self.deferred_write_back else 1
+        self.rows = torch.empty(slots + areas * self.stage_slots, self.D, dtype=backing_weights.dtype,
+                                device=self.device)
+        self.stage_of_row = self.stage_keys = None
+        if self.deferred_write_back:
+            self.stage_of_row = torch.empty(backing_weights.size(0), dtype=torch.int32, device=self.device)
+            self.stage_keys = torch.empty(2 * self.stage_slots, dtype=torch.int32, device=self.device)
         self.handle = _native.Cache(_ptr(self.tags), _ptr(self.last_used), _ptr(self.use_count), _ptr(self.rows),
-                                    _ptr(self.backing), self.num_sets, _POLICIES[policy], self.stage_slots)
+                                    _ptr(self.backing), self.num_sets, _POLICIES[policy], self.stage_slots,
+                                    _ptr(self.stage_of_row), _ptr(self.stage_keys), backing_weights.size(0))
         self.side_stream = torch.cuda.Stream(device=self.device)  # default priority
         self.step = 0
         # prepare() leaves ONE plan (sort, slots of this batch's rows) in the workspaces; plan_id
@@ -169,7 +181,8 @@ class RowCache:
         return grad_psw
 
     def flush(self):
-        """Writes every resident row back to the backing table."""
+        """Writes every resident row (and every staged row whose write-back is still pending) back to
+        the backing table."""
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_cache_flush(ctypes.byref(self.handle), self.dtype_code, self.D,
                                                          self._stream()))

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -56,6 +56,9 @@ class Cache(ctypes.Structure):
         ("num_sets", _i64),
         ("policy", _i32),
         ("stage_slots", _i64),
+        ("stage_of_row", _vp),
+        ("stage_keys", _vp),
+        ("total_rows", _i64),
     ]
 
 
@@ -64,7 +67,7 @@ class CacheWorkspaceLayout(ctypes.Structure):
 
     _fields_ = [(name, _u64) for name in (
         "total_bytes", "unique_slots", "lookup_slots", "evicted_keys", "miss_sets", "miss_list",
-        "set_counts", "set_fill", "set_starts", "stats")]
+        "set_counts", "set_fill", "set_starts", "stats", "fetch_source")]
 
 
 CACHE_WAYS = 64

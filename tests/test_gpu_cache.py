@@ -49,7 +49,7 @@ def test_cache_state_matches_model_bit_exact(oracle, policy, num_sets):
         np.testing.assert_array_equal(cache.last_used.cpu().numpy(), model.last_used)
         np.testing.assert_array_equal(cache.use_count.cpu().numpy(), model.use_count)
         np.testing.assert_array_equal(cache.resident_keys().cpu().numpy(), model.resident())
-        assert list(cache.stats().values()) == stats.tolist() + [0]  # nothing is staged without a staging area
+        assert list(cache.stats().values()) == stats.tolist() + [0, 0]  # nothing is staged without a staging area
         # per-lookup slots agree with per-unique slots
         all_keys = table_offsets[np.repeat(np.arange(T * B), np.diff(offsets)) // B] + indices
         np.testing.assert_array_equal(cache.lookup_slots.cpu().numpy(), slots[np.searchsorted(keys, all_keys)])
@@ -58,14 +58,17 @@ def test_cache_state_matches_model_bit_exact(oracle, policy, num_sets):
 @pytest.mark.parametrize("mode,dtype,D", [("sgd", torch.float32, 128), ("adagrad", torch.float32, 64),
                                           ("adagrad_weighted", torch.float16, 64), ("sgd", torch.float32, 520),
                                           ("sgd", torch.float64, 12)])
-@pytest.mark.parametrize("num_sets,stage_slots", [(2, 0), (40, 0), (2, 4096), (2, 7)])
-def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, stage_slots):
+@pytest.mark.parametrize("num_sets,stage_slots,deferred", [(2, 0, False), (40, 0, False), (2, 4096, False),
+                                                          (2, 7, False), (2, 4096, True), (2, 7, True),
+                                                          (5, 300, True)])
+def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, stage_slots, deferred):
     """Several forward + backward steps through the cache, then a flush: outputs of every step,
     the final table, optimizer state and per-sample-weight gradients are bit-identical to the
     same steps on a table that lives entirely in device memory.  With 2 sets most rows are
     served straight from the backing table; with 40 most are cached.  With a staging area the rows
     that find no slot are staged in HBM for the step and copied back after the update (all of
-    them with 4096 staging rows, some with 7)."""
+    them with 4096 staging rows, some with 7) -- or, with deferred write-back, kept until the next
+    step, which fetches the rows it needs again from there and writes the others back."""
     rs = np.random.RandomState(3)
     T, rows, B, L = 3, [700, 90, 3000], 48, 9
     table_offsets = dev(np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
@@ -77,7 +80,7 @@ def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, sta
     st_dtype = torch.float64 if dtype == torch.float64 else torch.float32
     plain_state = torch.zeros(total, device=DEV, dtype=st_dtype)
     cached_state = torch.zeros(total, device=DEV, dtype=st_dtype)
-    cache = tc.RowCache(cached_w, num_sets * 64, "lru", stage_slots)
+    cache = tc.RowCache(cached_w, num_sets * 64, "lru", stage_slots, deferred_write_back=deferred)
     weighted = mode.endswith("weighted")
     opt = "sgd" if mode == "sgd" else "adagrad"
     served_uncached = served_staged = 0
@@ -105,7 +108,8 @@ def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, sta
     torch.cuda.synchronize()
     assert torch.equal(cached_w, plain_w)
     assert torch.equal(cached_state, plain_state)
-    assert (served_uncached > 0) == (num_sets == 2 and stage_slots < 4096)
+    if num_sets != 5:
+        assert (served_uncached > 0) == (num_sets == 2 and stage_slots < 4096)
     assert (served_staged > 0) == (stage_slots > 0)
     ext.free_host_tensor(cached_w)
 
@@ -164,19 +168,22 @@ def test_cached_training_random_sweep(seed):
     ext.free_host_tensor(cached_w)
 
 
+@pytest.mark.parametrize("deferred", [False, True])
 @pytest.mark.parametrize("stage_slots", [100000, 9])
-def test_staging_leaves_cache_state_as_the_model_says(oracle, stage_slots):
+def test_staging_leaves_cache_state_as_the_model_says(oracle, stage_slots, deferred):
     """A staged row is an uncached row of the model: tags, recency and frequency words are
     unchanged by staging; rows the model leaves uncached get distinct staging rows behind the
     slots (index = misses of the earlier sets + rank among the set's staged rows) until the
-    staging area is full, the rest stay uncached."""
+    staging area is full, the rest stay uncached.  With deferred write-back the steps stage into
+    two areas in turn, and a row staged again is fetched from the staging row it had."""
     rs = np.random.RandomState(11)
     T, rows, B, L, D, num_sets = 3, [300, 5000, 40], 64, 12, 32, 2
     table_offsets = np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32)
     backing = torch.randn(sum(rows), D, device=DEV)
-    cache = tc.RowCache(backing, num_sets * 64, "lru", stage_slots)
+    cache = tc.RowCache(backing, num_sets * 64, "lru", stage_slots, deferred_write_back=deferred)
     model = oracle.CacheModel(num_sets, "lru")
     saw_uncached = False
+    from_staging = 0
     for step in range(5):
         indices, offsets = _draw_batch(rs, T, rows, B, L, 1.15)
         cache.prepare(dev(table_offsets), dev(indices), dev(offsets))
@@ -185,7 +192,9 @@ def test_staging_leaves_cache_state_as_the_model_says(oracle, stage_slots):
         got = cache.unique_slots().cpu().numpy()
         staged = got >= num_sets * 64
         np.testing.assert_array_equal(np.where(staged, -1, got), slots)
-        assert np.unique(got[staged]).size == staged.sum() and (got[staged] < num_sets * 64 + stage_slots).all()
+        area = num_sets * 64 + (stage_slots if deferred and cache.step % 2 else 0)   # first row of this step's area
+        assert np.unique(got[staged]).size == staged.sum()
+        assert (got[staged] >= area).all() and (got[staged] < area + stage_slots).all()
         got_evicted = cache.evicted_keys().cpu().numpy()
         np.testing.assert_array_equal(got_evicted[~staged], evicted[~staged])
         assert (got_evicted[staged] == -1).all()
@@ -198,7 +207,11 @@ def test_staging_leaves_cache_state_as_the_model_says(oracle, stage_slots):
         rows_now = cache.rows[torch.from_numpy(got[staged]).to(DEV).long()]
         assert torch.equal(rows_now, backing[torch.from_numpy(keys[staged]).to(DEV).long()])
         saw_uncached |= st["uncached"] > 0
+        from_staging += st["from_staging"]
     assert saw_uncached == (stage_slots == 9)
+    assert (from_staging > 0) == deferred
+    cache.flush()
+    torch.cuda.synchronize()
 
 
 def test_cached_stochastic_rounding_equals_uncached_bit_exact():
