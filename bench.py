@@ -301,6 +301,7 @@ def run_cached(args, w):
     slots = w["cache_slots"]
     per_step, per_kernel = [], {}
     bytes_alg = 0
+    staged_before = 0
     with tbe_native.profile() as prof:
         for i in range(total):
             indices, offsets = batches[i]
@@ -316,6 +317,9 @@ def run_cached(args, w):
             st["lookups_hit"] = int(occurrences[hit].sum())
             st["hit_rate_unique_rows"] = st["hits"] / max(U, 1)
             st["hit_rate_lookups"] = st["lookups_hit"] / max(st["lookups"], 1)
+            # staged rows of the step before that this step did not take over go back to the host now
+            st["staged_written_back"] = staged_before - st["from_staging"]
+            staged_before = st["staged"]
             out.backward(grad_output)
             if i >= args.warmup:
                 per_step.append(st)
@@ -328,16 +332,19 @@ def run_cached(args, w):
     kernels = {k: {"launches_per_step": len(v) / replay_steps, "avg_us": 1e3 * sum(v) / len(v)}
                for k, v in per_kernel.items()}
     row_bytes = D * 4
-    # Rows over the host link per step.  In: inserted and staged rows are fetched once, an uncached row
-    # is read by the forward (once per lookup; counted once) and by the update.  Out: evicted and staged
-    # rows are written once, an uncached row is written by the update.
-    link_in = [(st["inserted"] + st["staged"] + 2 * st["uncached"]) * row_bytes for st in per_step]
-    link_out = [(st["written_back"] + st["staged"] + st["uncached"]) * row_bytes for st in per_step]
+    # Rows over the host link per step.  In: inserted and staged rows are fetched once, from the host
+    # table unless the step before left them in its staging area; an uncached row is read by the forward
+    # (once per lookup; counted once) and by the update.  Out: evicted rows and the rows that the step
+    # before staged and this step did not take over are written once, an uncached row is written by the
+    # update.  One launch (cache_fill) carries the fetches and both kinds of write-back.
+    fetched = [(st["inserted"] + st["staged"] - st["from_staging"]) * row_bytes for st in per_step]
+    written = [(st["written_back"] + st["staged_written_back"]) * row_bytes for st in per_step]
+    link_in = [f + 2 * st["uncached"] * row_bytes for f, st in zip(fetched, per_step)]
+    link_out = [o + st["uncached"] * row_bytes for o, st in zip(written, per_step)]
     mean = lambda xs: sum(xs) / max(len(xs), 1)
     steady = per_step[len(per_step) // 2:]
     fill_us = kernels.get("cache_fill", {}).get("avg_us")
-    unstage_us = kernels.get("cache_unstage", {}).get("avg_us")
-    fill_in = mean([(st["inserted"] + st["staged"]) * row_bytes for st in per_step])
+    fill_in, fill_out = mean(fetched), mean(written)
     link_achieved = (mean(link_in) + mean(link_out)) / sec / 1e9
     roofline = {
         "bound": "host-link", "kernel": "cache_fill",
@@ -346,20 +353,21 @@ def run_cached(args, w):
         "frac": fill_in / (fill_us * 1e-6) / HOST_LINK_PEAK if fill_us else None,
         "traffic": None,
         "peak_is": "one direction of the host link (PCIe 5.0 x16, 32 GT/s x 16 lanes x 128b/130b = 63.0 GB/s); "
-                   "achieved = bytes the kernel fetches from the host table (inserted + staged rows x %d B) over "
-                   "its average duration, measured with HIP events on its stream in the replay" % row_bytes,
+                   "achieved = bytes the kernel fetches from the host table (inserted + staged rows that the "
+                   "step before did not leave on the device, x %d B) over its average duration, measured with "
+                   "HIP events on its stream in the replay; the same launch writes device_to_host_bytes_per_launch "
+                   "the other way" % row_bytes,
         "avg_launch_us": fill_us,
         "host_to_device_bytes_per_launch": fill_in,
-        "device_to_host_bytes_per_launch": mean([st["written_back"] * row_bytes for st in per_step]),
+        "device_to_host_bytes_per_launch": fill_out,
+        "device_to_host_achieved": fill_out / (fill_us * 1e-6) / 1e9 if fill_us else None,
+        "rows_taken_from_the_staging_area_per_step": mean([st["from_staging"] for st in per_step]),
         "whole_step": {"host_link_bytes_in": mean(link_in), "host_link_bytes_out": mean(link_out),
                        "achieved_GBps_both_directions": link_achieved,
                        "frac_of_one_direction_peak": link_achieved * 1e9 / HOST_LINK_PEAK,
-                       "note": "fill (in) and unstage (out) run one after the other around the update, so "
-                               "one direction is busy at a time: the step is bounded by in/peak + out/peak"},
-        "cache_unstage": {"avg_launch_us": unstage_us,
-                          "device_to_host_bytes_per_launch": mean([st["staged"] * row_bytes for st in per_step]),
-                          "achieved": (mean([st["staged"] * row_bytes for st in per_step]) / (unstage_us * 1e-6) / 1e9
-                                       if unstage_us else None)},
+                       "note": "fetches and write-backs share one launch, so both directions of the link are "
+                               "busy together: the step is bounded by max(in, out)/peak plus the kernels that "
+                               "work on device memory"},
     }
     mean_lookups = mean([st["lookups"] for st in per_step])
     result = {

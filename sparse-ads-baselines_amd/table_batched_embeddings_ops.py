@@ -145,7 +145,7 @@ class TableBatchedEmbeddingBags(nn.Module):
     def __init__(self, num_tables, num_embeddings, embedding_dim, optimizer=Optimizer.SGD,
                  learning_rate=0.01, eps=None, stochastic_rounding=False, fp16=False,
                  managed=EmbeddingLocation.DEVICE, cache_slots=None, cache_policy="lru",
-                 cache_stage_slots=0):
+                 cache_stage_slots=0, cache_deferred_write_back=True):
         super(TableBatchedEmbeddingBags, self).__init__()
         assert managed in (EmbeddingLocation.DEVICE, EmbeddingLocation.HOST_MAPPED,
                            EmbeddingLocation.HOST_CACHED)
@@ -177,7 +177,8 @@ class TableBatchedEmbeddingBags(nn.Module):
             if optimizer == Optimizer.APPROX_ROWWISE_ADAGRAD:
                 raise NotImplementedError("cache-fronted tables serve SGD and EXACT_ROWWISE_ADAGRAD")
             self.row_cache = table_batched_embeddings_cache.RowCache(self.embedding_weights.data, cache_slots,
-                                                                     cache_policy, cache_stage_slots)
+                                                                     cache_policy, cache_stage_slots,
+                                                                     cache_deferred_write_back)
             # checkpoints must see the rows the cache holds ...
             self.register_state_dict_pre_hook(lambda module, prefix, keep_vars: module.flush_cache())
             # ... and a loaded checkpoint must not be shadowed (or later overwritten) by rows that

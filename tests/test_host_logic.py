@@ -46,7 +46,7 @@ def test_module_constructor_signature_matches_reference():
     # the reference's nine arguments in order, then the cache extension
     assert list(params)[1:] == ["num_tables", "num_embeddings", "embedding_dim", "optimizer", "learning_rate", "eps",
                                 "stochastic_rounding", "fp16", "managed", "cache_slots", "cache_policy",
-                                "cache_stage_slots"]
+                                "cache_stage_slots", "cache_deferred_write_back"]
     assert params["optimizer"].default is ops.Optimizer.SGD
     assert params["learning_rate"].default == 0.01
     assert params["managed"].default is ops.EmbeddingLocation.DEVICE
