@@ -431,7 +431,6 @@ int validate_cache(const char *name, const tbe_cache_t *cache) {
 void write_back_stage(const tbe_cache_t *cache, int row_units, int64_t half, hipStream_t stream) {
   const int64_t base = cache->num_sets * kWays + half * cache->stage_slots;
   int32_t *keys = cache->stage_keys + half * cache->stage_slots;
-  // (the fetching half of the launch finds no rows: a null counter block is not read with U = 0)
   TBE_LAUNCH("cache_unstage", stream, cache_unstage_area_kernel,
              dim3(grid_for(cache->stage_slots, kWavesPerBlock, 256 * 16)), dim3(kBlockThreads),
              static_cast<const uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units, keys,

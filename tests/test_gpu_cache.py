@@ -114,6 +114,55 @@ def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, sta
     ext.free_host_tensor(cached_w)
 
 
+@pytest.mark.parametrize("stage_slots", [4096, 7])
+def test_deferred_write_back_with_irregular_steps(stage_slots):
+    """Deferred write-back picks its staging area by the parity of the step number.  Step numbers
+    that skip (two steps of the same parity in a row), an empty batch and a flush in the middle
+    of the run must leave nothing behind: outputs, flushed table and state stay bit-identical to
+    the run on device memory, and after every flush the host table itself is complete."""
+    rs = np.random.RandomState(11)
+    T, rows, B, L, D = 3, [700, 90, 3000], 48, 9, 64
+    table_offsets = dev(np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
+    total = sum(rows)
+    start = torch.rand(total, D, device=DEV) * 0.02 - 0.01
+    plain_w = start.clone()
+    cached_w = ext.new_host_mapped_tensor(torch.empty(1, device=DEV), (total, D))
+    cached_w.copy_(start)
+    plain_state = torch.zeros(total, device=DEV)
+    cached_state = torch.zeros(total, device=DEV)
+    cache = tc.RowCache(cached_w, 2 * 64, "lru", stage_slots, deferred_write_back=True)
+    empty = (np.zeros(0, dtype=np.int32), np.zeros(T * B + 1, dtype=np.int32))
+    staged = 0
+    for step, skip in enumerate([0, 1, 0, 2, 1, 0, 3, 0]):
+        cache.step += skip  # the next prepare uses step + 1
+        if step == 5:
+            indices, offsets = empty
+        else:
+            indices, offsets = _draw_batch(rs, T, rows, B, L, 1.2)
+        idx, off = dev(indices), dev(offsets)
+        cache.prepare(table_offsets, idx, off)
+        got = cache.forward(table_offsets, idx, off, None)
+        if indices.size == 0:
+            assert not got.any()
+        else:
+            go = torch.randn(B, T, D, device=DEV)
+            want = ext.forward(plain_w, table_offsets, idx, off, None, 200, 1, False)
+            ext.backward_exact_adagrad(go, plain_w, table_offsets, idx, off, None, plain_state, 0.05, 0.1, False, 1)
+            cache.backward("adagrad", go, None, cached_state, 0.05, 0.1)
+            assert torch.equal(got, want), "forward output differs at step %d" % step
+            staged += cache.stats()["staged"]
+        if step in (3, 5):
+            cache.flush()
+            torch.cuda.synchronize()
+            assert torch.equal(cached_w, plain_w), "host table incomplete after the flush at step %d" % step
+    cache.flush()
+    torch.cuda.synchronize()
+    assert staged > 0
+    assert torch.equal(cached_w, plain_w)
+    assert torch.equal(cached_state, plain_state)
+    ext.free_host_tensor(cached_w)
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_cached_training_random_sweep(seed):
     """Seeded random shapes of the cached-equals-uncached property: table counts and sizes, row
