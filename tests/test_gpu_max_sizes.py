@@ -1,0 +1,135 @@
+"""Maximum sizes: tables whose concatenated row count is the largest the int32 key type allows
+(2^31 - 2 rows, 17 to 34 GB of weights).  Keys, sort digits and row addresses are exercised up to
+their last bit: lookups hit the last rows of the last table and the rows on either side of every
+power-of-two boundary of the byte and element offsets.
+
+The expected values come from the same lookups on a compacted problem that keeps only the rows
+touched, in the same order (an order-preserving renumbering leaves the sorted order, the runs
+and every sum unchanged): the HIP path on the compacted tables must agree bit for bit, and the
+oracle on the compacted tables within the usual tolerance."""
+import numpy as np
+import pytest
+import torch
+
+import table_batched_embeddings as ext
+from gpu_util import DEV, assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+ROWS = [1000, 2 ** 31 - 2 - 1000]
+FILL = 0.25
+
+
+def _lookups(seed, B, L):
+    """Ragged bags over both tables; table 1 draws from a pool of boundary rows, the last rows
+    and random rows, with one row repeated often enough to take the long-run path."""
+    rs = np.random.RandomState(seed)
+    E1 = ROWS[1]
+    pool = [E1 - 1 - k for k in range(48)]
+    for bit in range(20, 31):
+        pool += [(1 << bit) - 1000 + d for d in (-1, 0, 1)]   # key = row + 1000 sits on 2^bit - 1, 2^bit, 2^bit + 1
+    pool += list(rs.randint(0, E1, size=200))
+    pool = np.array(pool, dtype=np.int64)
+    hot = E1 - 7
+    lengths = rs.randint(0, L + 1, size=(2, B))
+    offsets = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
+    n0, n1 = int(lengths[0].sum()), int(lengths[1].sum())
+    idx0 = rs.randint(0, ROWS[0], size=n0)
+    idx1 = pool[rs.randint(0, pool.size, size=n1)]
+    idx1[rs.rand(n1) < 0.15] = hot
+    indices = np.concatenate([idx0, idx1]).astype(np.int32)
+    assert (idx1 == hot).sum() > 32
+    return indices, offsets
+
+
+def _compact(indices, offsets, B):
+    """Order-preserving renumbering of the touched rows: (keys of the touched rows, ascending;
+    compact table_offsets; compact indices)."""
+    table_offsets = np.array([0, ROWS[0]], dtype=np.int64)
+    n0 = int(offsets[B])
+    keys = np.concatenate([indices[:n0].astype(np.int64), indices[n0:].astype(np.int64) + table_offsets[1]])
+    touched = np.unique(keys)
+    rank = np.searchsorted(touched, keys)
+    first_of_table1 = int(np.searchsorted(touched, table_offsets[1]))
+    compact_offsets = np.array([0, first_of_table1], dtype=np.int32)
+    compact_indices = rank.copy()
+    compact_indices[n0:] -= first_of_table1
+    return touched, compact_offsets, compact_indices.astype(np.int32)
+
+
+@pytest.mark.parametrize("mode,dtype,D", [("sgd", torch.float32, 4), ("adagrad_weighted", torch.float16, 8),
+                                          ("approx", torch.float32, 4)])
+def test_rows_up_to_the_int32_limit(oracle, mode, dtype, D):
+    B, L = 48, 12
+    total = sum(ROWS)
+    assert total == 2 ** 31 - 2
+    indices, offsets = _lookups(5, B, L)
+    touched, compact_offsets, compact_indices = _compact(indices, offsets, B)
+    n = indices.size
+    gen = torch.Generator(device=DEV).manual_seed(17)
+    rows0 = (torch.rand(touched.size, D, device=DEV, generator=gen, dtype=torch.float32) * 0.2 - 0.1).to(dtype)
+    touched_d = torch.from_numpy(touched).to(DEV)
+
+    big = torch.full((total, D), FILL, dtype=dtype, device=DEV)
+    big[touched_d] = rows0
+    small = rows0.clone()
+    go = torch.randn(B, 2, D, device=DEV, generator=gen, dtype=torch.float32).to(dtype)
+    weighted = mode.endswith("weighted")
+    psw = torch.rand(n, device=DEV, generator=gen, dtype=torch.float32).to(dtype) if weighted else None
+    big_to = dev(np.array([0, ROWS[0]], dtype=np.int32))
+    small_to = dev(compact_offsets)
+    idx_big, idx_small, off = dev(indices), dev(compact_indices), dev(offsets)
+
+    # forward
+    out_big = ext.forward(big, big_to, idx_big, off, psw, 200, 1, False)
+    out_small = ext.forward(small, small_to, idx_small, off, psw, 200, 1, False)
+    assert torch.equal(out_big, out_small)
+    np_dtype = {torch.float32: np.float32, torch.float16: np.float16}[dtype]
+    w_np = rows0.cpu().numpy()
+    want_out = oracle.forward(w_np, compact_offsets, compact_indices, offsets,
+                              None if psw is None else psw.cpu().numpy())
+    assert_close(out_big.cpu().numpy(), want_out, 1e-5 if dtype == torch.float32 else 2e-3, "forward")
+
+    # update
+    lr, eps = 0.05, 0.1
+    state_big = state_small = None
+    if mode != "sgd":
+        state_big = torch.zeros(total, device=DEV)
+        state_small = torch.zeros(touched.size, device=DEV)
+    if mode == "sgd":
+        ext.backward_sgd(go, big, big_to, idx_big, off, lr, 200, 1, False)
+        ext.backward_sgd(go, small, small_to, idx_small, off, lr, 200, 1, False)
+        g_big = g_small = None
+        want = oracle.backward("sgd", go.cpu().numpy(), w_np, compact_offsets, compact_indices, offsets, lr)
+        want_g, want_state = None, None
+    elif mode == "approx":
+        g_big = ext.backward_approx_adagrad(go, big, big_to, idx_big, off, psw, state_big, lr, eps, 200, False, 1)
+        g_small = ext.backward_approx_adagrad(go, small, small_to, idx_small, off, psw, state_small, lr, eps, 200,
+                                              False, 1)
+        want_state = np.zeros(touched.size, np.float32)
+        want_g = oracle.backward_approx(go.cpu().numpy(), w_np, compact_offsets, compact_indices, offsets, lr, eps,
+                                        want_state)
+    else:
+        g_big = ext.backward_exact_adagrad(go, big, big_to, idx_big, off, psw, state_big, lr, eps, False, 1)
+        g_small = ext.backward_exact_adagrad(go, small, small_to, idx_small, off, psw, state_small, lr, eps, False, 1)
+        want_state = np.zeros(touched.size, np.float32)
+        want_g = oracle.backward("adagrad", go.cpu().numpy(), w_np, compact_offsets, compact_indices, offsets, lr,
+                                 eps, want_state, psw.cpu().numpy())["grad_psw"]
+    torch.cuda.synchronize()
+    got_rows = big[touched_d]
+    assert torch.equal(got_rows, small), "rows of the full-size tables differ from the compacted run"
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert_close(got_rows.cpu().numpy(), w_np, tol, "weights")   # w_np was updated in place by the oracle
+    if state_big is not None:
+        assert torch.equal(state_big[touched_d], state_small)
+        assert_close(state_small.cpu().numpy(), want_state, 1e-5, "state")
+        state_big[touched_d] = 0
+        assert not bool(state_big.any()), "optimizer state written outside the touched rows"
+    if g_big is not None:
+        assert torch.equal(g_big, g_small)
+        assert_close(g_big.cpu().numpy(), want_g, 2e-3, "grad_psw")
+    # no other row of the 2^31 - 2 was written
+    big[touched_d] = FILL
+    assert bool((big == FILL).all()), "weights written outside the touched rows"
+    del big, state_big
+    torch.cuda.empty_cache()
