@@ -84,7 +84,6 @@ def test_rows_up_to_the_int32_limit(oracle, mode, dtype, D):
     out_big = ext.forward(big, big_to, idx_big, off, psw, 200, 1, False)
     out_small = ext.forward(small, small_to, idx_small, off, psw, 200, 1, False)
     assert torch.equal(out_big, out_small)
-    np_dtype = {torch.float32: np.float32, torch.float16: np.float16}[dtype]
     w_np = rows0.cpu().numpy()
     want_out = oracle.forward(w_np, compact_offsets, compact_indices, offsets,
                               None if psw is None else psw.cpu().numpy())
@@ -100,7 +99,7 @@ def test_rows_up_to_the_int32_limit(oracle, mode, dtype, D):
         ext.backward_sgd(go, big, big_to, idx_big, off, lr, 200, 1, False)
         ext.backward_sgd(go, small, small_to, idx_small, off, lr, 200, 1, False)
         g_big = g_small = None
-        want = oracle.backward("sgd", go.cpu().numpy(), w_np, compact_offsets, compact_indices, offsets, lr)
+        oracle.backward("sgd", go.cpu().numpy(), w_np, compact_offsets, compact_indices, offsets, lr)
         want_g, want_state = None, None
     elif mode == "approx":
         g_big = ext.backward_approx_adagrad(go, big, big_to, idx_big, off, psw, state_big, lr, eps, 200, False, 1)
@@ -130,6 +129,87 @@ def test_rows_up_to_the_int32_limit(oracle, mode, dtype, D):
         assert_close(g_big.cpu().numpy(), want_g, 2e-3, "grad_psw")
     # no other row of the 2^31 - 2 was written
     big[touched_d] = FILL
+    assert bool((big == FILL).all()), "weights written outside the touched rows"
+    del big, state_big
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("mode", ["adagrad_weighted", "approx"])
+def test_mixed_dim_rows_up_to_the_int32_limit(oracle, mode):
+    """The same for tables of different widths (a narrow table of 2^31 - 1002 rows after a wider
+    one of 1000): flat weights of 8.6 G elements, int64 element offsets, the row-number keys up
+    to their last bit."""
+    B, L = 48, 12
+    dims = [8, 4]
+    indices, offsets = _lookups(9, B, L)
+    touched, compact_row_offsets, compact_indices = _compact(indices, offsets, B)
+    n = indices.size
+    first1 = int(compact_row_offsets[1])
+    rows_small = [first1, touched.size - first1]
+    gen = torch.Generator(device=DEV).manual_seed(23)
+    small = torch.rand(rows_small[0] * dims[0] + rows_small[1] * dims[1], device=DEV, generator=gen) * 0.2 - 0.1
+    elements = [ROWS[0] * dims[0], ROWS[1] * dims[1]]
+    big = torch.full((sum(elements),), FILL, device=DEV)
+    # touched rows of the full-size tables take the compacted tables' values
+    keys0 = torch.from_numpy(touched[:first1]).to(DEV)
+    keys1 = torch.from_numpy(touched[first1:] - ROWS[0]).to(DEV)
+    big[:elements[0]].view(ROWS[0], dims[0])[keys0] = small[:rows_small[0] * dims[0]].view(-1, dims[0])
+    big[elements[0]:].view(ROWS[1], dims[1])[keys1] = small[rows_small[0] * dims[0]:].view(-1, dims[1])
+    go = torch.randn(B, sum(dims), device=DEV, generator=gen)
+    weighted = mode.endswith("weighted")
+    psw = torch.rand(n, device=DEV, generator=gen) if weighted else None
+    dim_offsets = dev(np.array([0, dims[0], sum(dims)], dtype=np.int32))
+
+    def arguments(rows):
+        return (dev(np.array([0, rows[0] * dims[0], rows[0] * dims[0] + rows[1] * dims[1]], dtype=np.int64)),
+                dev(np.array([0, rows[0], rows[0] + rows[1]], dtype=np.int32)))
+    big_to, big_rows = arguments(ROWS)
+    small_to, small_rows = arguments(rows_small)
+    idx_big, idx_small, off = dev(indices), dev(compact_indices), dev(offsets)
+
+    out_big = ext.forward_mixed_D(big, big_to, dim_offsets, sum(dims), idx_big, off, psw, 200, 1, False)
+    out_small = ext.forward_mixed_D(small, small_to, dim_offsets, sum(dims), idx_small, off, psw, 200, 1, False)
+    assert torch.equal(out_big, out_small)
+    w_np = small.cpu().numpy()
+    psw_np = None if psw is None else psw.cpu().numpy()
+    want_out = oracle.forward_mixed(w_np, small_to.cpu().numpy(), dim_offsets.cpu().numpy(), compact_indices, offsets,
+                                    psw_np)
+    assert_close(out_big.cpu().numpy(), want_out, 1e-5, "forward")
+
+    lr, eps = 0.05, 0.1
+    state_big = torch.zeros(sum(ROWS), device=DEV)
+    state_small = torch.zeros(touched.size, device=DEV)
+    want_state = np.zeros(touched.size, np.float32)
+    if mode == "approx":
+        run = lambda w, to, rows, idx, st: ext.backward_approx_adagrad_mixed_D(
+            go, w, to, rows, dim_offsets, sum(dims), idx, off, psw, st, lr, eps, 200, False, 1)
+        want_g = oracle.backward_approx_mixed(go.cpu().numpy(), w_np, small_to.cpu().numpy(),
+                                              small_rows.cpu().numpy(), dim_offsets.cpu().numpy(), compact_indices,
+                                              offsets, lr, eps, want_state, psw_np)
+    else:
+        run = lambda w, to, rows, idx, st: ext.backward_exact_adagrad_mixed_D(
+            go, w, to, rows, dim_offsets, sum(dims), idx, off, psw, st, lr, eps, False, 1)
+        want_g = oracle.backward_mixed("adagrad", go.cpu().numpy(), w_np, small_to.cpu().numpy(),
+                                       small_rows.cpu().numpy(), dim_offsets.cpu().numpy(), compact_indices, offsets,
+                                       lr, eps, want_state, psw_np)
+    g_big = run(big, big_to, big_rows, idx_big, state_big)
+    g_small = run(small, small_to, small_rows, idx_small, state_small)
+    torch.cuda.synchronize()
+    got0 = big[:elements[0]].view(ROWS[0], dims[0])[keys0].reshape(-1)
+    got1 = big[elements[0]:].view(ROWS[1], dims[1])[keys1].reshape(-1)
+    got = torch.cat([got0, got1])
+    assert torch.equal(got, small), "rows of the full-size tables differ from the compacted run"
+    assert_close(got.cpu().numpy(), w_np, 1e-5, "weights")
+    touched_d = torch.from_numpy(touched).to(DEV)
+    assert torch.equal(state_big[touched_d], state_small)
+    assert_close(state_small.cpu().numpy(), want_state, 1e-5, "state")
+    if weighted:
+        assert torch.equal(g_big, g_small)
+        assert_close(g_big.cpu().numpy(), want_g, 1e-5, "grad_psw")
+    state_big[touched_d] = 0
+    assert not bool(state_big.any()), "optimizer state written outside the touched rows"
+    big[:elements[0]].view(ROWS[0], dims[0])[keys0] = FILL
+    big[elements[0]:].view(ROWS[1], dims[1])[keys1] = FILL
     assert bool((big == FILL).all()), "weights written outside the touched rows"
     del big, state_big
     torch.cuda.empty_cache()
