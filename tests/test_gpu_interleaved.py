@@ -61,3 +61,32 @@ def test_ragged_offsets_and_function_level_calls(oracle):
     assert_close(w.cpu().numpy(), w_ref, 1e-5)
     with pytest.raises(NotImplementedError):
         se.forward_all2all(w, w)
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float16, 1e-2), (np.float64, 1e-12), (np.float32, 1e-5)])
+def test_half_and_double_tables(oracle, dtype, tol):
+    """The reference dispatches these kernels over half, float and double
+    (sparse_embedding_cuda_kernel.cu:599-882).  An interleaved table set is one table of E*T rows
+    whose row ind*T + t is row `ind` of table t, with the bags numbered b*T + t: the expected
+    values come from the table-batched oracle on that single table."""
+    rs = np.random.RandomState(6)
+    E, T, D, B = 150, 4, 24, 13
+    weights = (rs.randn(E, T, D) * 0.1).astype(dtype)
+    lengths = rs.randint(0, 7, size=B * T)
+    flat = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    indices = (rs.zipf(1.3, size=int(flat[-1])) % E).astype(np.int32)
+    merged = np.stack([flat[b * T:b * T + T + 1] for b in range(B)]).astype(np.int32)
+    go = rs.randn(B, T, D).astype(dtype)
+    table_of_lookup = np.repeat(np.arange(B * T) % T, lengths)
+    one_table_rows = (indices * T + table_of_lookup).astype(np.int32)
+    one_table = weights.reshape(E * T, D).copy()
+    zero = np.zeros(1, np.int32)
+    want = oracle.forward(one_table, zero, one_table_rows, flat).reshape(B, T, D)
+    w = dev(weights)
+    got = se.forward_offsets(w, dev(indices), dev(merged))
+    assert got.dtype == w.dtype
+    assert_close(got.cpu().numpy(), want, tol)
+    se.backward_update_offsets(dev(go), w, dev(indices), dev(merged), 0.1)
+    oracle.backward("sgd", go.reshape(B * T, 1, D), one_table, zero, one_table_rows, flat, 0.1)
+    torch.cuda.synchronize()
+    assert_close(w.cpu().numpy().reshape(E * T, D), one_table, tol)
