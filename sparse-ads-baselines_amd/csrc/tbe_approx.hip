@@ -400,6 +400,48 @@ __device__ __forceinline__ uint4 draw_block(const StochasticRounding &sr, int64_
                        make_uint2(static_cast<uint32_t>(sr.seed), static_cast<uint32_t>(sr.seed >> 32)));
 }
 
+// Cooperative walk of a very long fp16 row with stochastic rounding: the random bits are most of
+// the work per occurrence, and they do not depend on the values, so three wavefronts of the
+// workgroup draw them for the next 32 occurrences into LDS while the first wavefront walks the
+// current 32.  words[2][kCoopStep][kCoopD]: the 13 random bits of every element of the row for
+// every occurrence of a step, two steps deep.
+constexpr int kCoopD = 128;    // widest row walked this way (two elements per lane)
+constexpr int kCoopStep = 32;  // occurrences per step
+// The barrier between the steps of the cooperative walk: LDS traffic of the wavefront is complete
+// (the bits written, or the bits of the finished step read), but the walking wavefront's gradient
+// rows stay in flight -- __syncthreads() would wait for them too and drain the ring at every step.
+__device__ __forceinline__ void step_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+__device__ __forceinline__ void draw_step_bits(const StochasticRounding &sr, int64_t row_element, int row_D,
+                                               int first_occurrence, int count, uint16_t *words, int thread,
+                                               int threads) {
+  // A thread keeps one block of four elements and takes every (threads >> shift)-th occurrence,
+  // 2^shift being the blocks of a row rounded up to a power of two (threads is a multiple of
+  // 32): no division, and the occurrence's key advances by an addition.  The words are those of
+  // draw_block(rounding_of_update(sr, occurrence), row_element + 4 * block).
+  const int blocks_per_row = row_D / 4;
+  int shift = 0;
+  while ((1 << shift) < blocks_per_row) ++shift;
+  const int block = thread & ((1 << shift) - 1);
+  if (block >= blocks_per_row) return;
+  const int per_round = threads >> shift;
+  const uint64_t kKeyStep = 0x9E3779B97F4A7C15ull;  // (rounding_of_update)
+  int o = thread >> shift;
+  uint64_t key_term = static_cast<uint64_t>(first_occurrence + o) * kKeyStep;
+  const uint64_t round_term = static_cast<uint64_t>(per_round) * kKeyStep;
+  const uint64_t counter = static_cast<uint64_t>(row_element) / 4 + static_cast<uint64_t>(block);
+  for (; o < count; o += per_round, key_term += round_term) {
+    const uint64_t seed = sr.seed ^ key_term;
+    const uint4 r = philox4x32_10(
+        make_uint4(static_cast<uint32_t>(counter), static_cast<uint32_t>(counter >> 32),
+                   static_cast<uint32_t>(sr.offset), static_cast<uint32_t>(sr.offset >> 32)),
+        make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)));
+    uint2 packed;
+    packed.x = (r.x >> 19) | ((r.y >> 19) << 16);
+    packed.y = (r.z >> 19) | ((r.w >> 19) << 16);
+    *reinterpret_cast<uint2 *>(words + o * kCoopD + 4 * block) = packed;
+  }
+}
+
 template <typename T> struct LongRowArgs {
   using A = typename AccOf<T>::type;
   const T *grad_output;
@@ -453,13 +495,22 @@ __device__ __forceinline__ P buffer_load_pack(__amdgpu_buffer_rsrc_t rsrc, uint3
 // wait for memory: into a ring of 64 registers (64, 32 or 16 rows, by the bytes of a row that a
 // lane holds), each slot refilled as soon as it has been applied; with stochastic rounding, where the random bits
 // are most of the work per occurrence, 16 ahead into one of two sets of 16.
-template <typename T, int E, bool WEIGHTED, bool STOCHASTIC, bool BIG>
+// COOP (with STOCHASTIC, E <= 2): the wavefront is the first of a workgroup whose other wavefronts
+// draw the random bits (draw_step_bits) into `words`; it meets them at a barrier after every
+// kCoopStep occurrences.
+template <typename T, int E, bool WEIGHTED, bool STOCHASTIC, bool BIG, bool COOP = false>
 __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_begin, int seg_end, int64_t key,
-                                              const RowPlace &place, int lane) {
+                                              const RowPlace &place, int lane, const uint16_t *words = nullptr) {
   using A = typename AccOf<T>::type;
   using P = LanePack<T, E>;
+  static_assert(!COOP || (STOCHASTIC && E <= 2), "the cooperative walk is for stochastic rounding of narrow rows");
   constexpr int kAhead = 16;
-  constexpr int kRing = STOCHASTIC ? 2 * kAhead : (E * sizeof(T) <= 4 ? kWave : E * sizeof(T) <= 8 ? kWave / 2 : kWave / 4);
+  static_assert(kWave % kCoopStep == 0, "a batch is a whole number of steps");
+  int step = 0;  // (COOP) steps walked so far
+  // (the cooperative walk does not draw random words itself: it is as light per occurrence as the
+  // walk without stochastic rounding and needs as many rows in flight)
+  constexpr bool kInBlocks = STOCHASTIC && !COOP;
+  constexpr int kRing = kInBlocks ? 2 * kAhead : (E * sizeof(T) <= 4 ? kWave : E * sizeof(T) <= 8 ? kWave / 2 : kWave / 4);
   const bool active = lane * E < place.row_D;
   const int lane_off = active ? lane * E : 0;  // (idle lanes shadow lane 0 and store nothing)
   T *wrow = a.weights + place.row_element + lane_off;
@@ -509,7 +560,7 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
   P ring[kRing];
   {
     const int nb = min(kWave, seg_end - seg_begin);
-    constexpr int kFirst = STOCHASTIC ? kAhead : kRing;
+    constexpr int kFirst = kInBlocks ? kAhead : kRing;
 #pragma unroll
     for (int c = 0; c < kFirst; c += kAhead) {
       if (c < nb) {
@@ -538,6 +589,20 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
     // than four elements per lane, `shared_draw` holds the random words that this lane drew for
     // one of the kShare occurrences around j and `slot` tells which of them j is
     constexpr int kShare = (STOCHASTIC && E < 4) ? 4 / E : 1;
+    // (COOP) the 13 random bits of this lane's elements for occurrence j of the batch, from the
+    // buffer of the current step
+    auto bits_of = [&](int j) {
+      if constexpr (COOP) {
+        const uint16_t *mine = words + (step & 1) * (kCoopStep * kCoopD) + (j & (kCoopStep - 1)) * kCoopD + lane_off;
+        if constexpr (E == 1) return make_uint4(mine[0], 0u, 0u, 0u);
+        else {
+          const uint32_t two = *reinterpret_cast<const uint32_t *>(mine);
+          return make_uint4(two & 0xffffu, two >> 16, 0u, 0u);
+        }
+      } else {
+        return make_uint4(0u, 0u, 0u, 0u);
+      }
+    };
     auto apply = [&](const P &grad, int j, const uint4 &shared_draw, int slot) {
       const A mult = broadcast_lane(my_mult, j);
       A dot = A(0);
@@ -547,7 +612,11 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
         if constexpr (WEIGHTED) dot += w[i] * g;
         w[i] = w[i] - g * mult;
       }
-      if constexpr (STOCHASTIC && E < 4) {
+      if constexpr (COOP) {
+        // (shared_draw.x, .y: the 13 bits of the lane's elements)
+        w[0] = round_trip_with_bits(w[0], shared_draw.x);
+        if constexpr (E == 2) w[1] = round_trip_with_bits(w[1], shared_draw.y);
+      } else if constexpr (STOCHASTIC && E < 4) {
         if (slot == 0) round_with_shared_draw<E, 0, A>(w, shared_draw, lane);
         else if (slot == 1) round_with_shared_draw<E, 1, A>(w, shared_draw, lane);
         else if constexpr (E == 1) {
@@ -569,7 +638,7 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
       }
     };
 
-    if constexpr (STOCHASTIC) {
+    if constexpr (kInBlocks) {
       // one block of 16 occurrences: request the block after it into `fill`, then apply `use`
       auto block = [&](P *use, P *fill, int j0) {
         Off src = cur_goff;
@@ -608,22 +677,42 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
       } while (j0 < nb);
     } else if (nb == kWave && nb_next == kWave) {
       // a full batch followed by a full batch: straight-line code
+      uint4 bits = bits_of(0);
 #pragma unroll
       for (int j = 0; j < kWave; ++j) {
-        apply(ring[j % kRing], j, make_uint4(0u, 0u, 0u, 0u), 0);
+        const uint4 now = bits;
+        if ((j + 1) % kCoopStep != 0) bits = bits_of(j + 1);
+        apply(ring[j % kRing], j, now, 0);
         if (j + kRing < kWave) ring[j % kRing] = row_of(cur_goff, j + kRing);
         else ring[j % kRing] = row_of(nxt_goff, j + kRing - kWave);
+        if constexpr (COOP) {
+          if ((j + 1) % kCoopStep == 0) {
+            step_barrier();  // the next step's bits are there, this step's buffer may be refilled
+            ++step;
+            if (j + 1 < kWave) bits = bits_of(j + 1);
+          }
+        }
       }
     } else {
+      uint4 bits = bits_of(0);
 #pragma unroll
       for (int j = 0; j < kWave; ++j) {
         if (j < nb) {
-          apply(ring[j % kRing], j, make_uint4(0u, 0u, 0u, 0u), 0);
+          const uint4 now = bits;
+          if ((j + 1) % kCoopStep != 0) bits = bits_of(j + 1);
+          apply(ring[j % kRing], j, now, 0);
           const int target = (j + kRing) % kWave;  // occurrence j + kRing of the row ...
           if (j + kRing < kWave) {                 // ... is in this batch
             if (target < nb) ring[j % kRing] = row_of(cur_goff, target);
           } else if (nb_next > 0) {                // ... or in the next one
             ring[j % kRing] = row_of(nxt_goff, min(target, nb_next - 1));
+          }
+          if constexpr (COOP) {
+            if ((j + 1) % kCoopStep == 0 || j == nb - 1) {
+              step_barrier();
+              ++step;
+              if (j + 1 < kWave) bits = bits_of(j + 1);
+            }
           }
         }
       }
@@ -665,8 +754,81 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
   // an XCD take their own queue in order -- it is in (table, row) order, so the gradient rows of a
   // table stay in that XCD's L2 while its rows are walked -- up to 1.5 times the average length;
   // what the longer queues hold beyond that is dealt to the wavefronts of all XCDs.  All of it is
-  // index arithmetic on the queue lengths: no wavefront waits for another.
-  const int xcd = static_cast<int>(blockIdx.x % kNumXcd);
+  // index arithmetic on the queue lengths: no wavefront waits for another (outside the
+  // cooperative walk below, whose wavefronts meet at workgroup barriers).
+  // where a queued row is and what it looks like
+  struct QueuedRow {
+    int seg_begin, seg_end;
+    int64_t key;
+    RowPlace place;
+  };
+  auto row_at = [&](int slot) {
+    const int u = uniform(long_queue[slot]);
+    QueuedRow r;
+    r.seg_begin = uniform(segment_starts[u]);
+    r.seg_end = uniform(segment_starts[u + 1]);
+    r.key = uniform(keys_sorted[r.seg_begin]);
+    const int first_grad_row = uniform(a.grad_rows[a.positions_sorted[r.seg_begin]]);
+    r.place = a.mt.T > 0 ? place_row<true>(r.key, first_grad_row, D, a.mt)
+                         : place_row<false>(r.key, first_grad_row, D, a.mt);
+    r.place.row_D = uniform(r.place.row_D);
+    r.place.row_element = uniform(r.place.row_element);
+    r.place.grad_stride = uniform(r.place.grad_stride);
+    r.place.grad_column = uniform(r.place.grad_column);
+    return r;
+  };
+  int first_total = uniform(counters[1]);  // the rows every wavefront helps with first
+  int block_index = static_cast<int>(blockIdx.x);
+  int grid_blocks = static_cast<int>(gridDim.x);
+
+  if constexpr (STOCHASTIC) {
+    // Rows of more than kApproxHuge occurrences, at most kCoopD wide: a whole workgroup per row
+    // (see draw_step_bits).  When the grid is large enough, the first workgroups do nothing else
+    // -- as many as there are such rows, rounded up to a multiple of the XCD count, at most half
+    // the grid -- and the others share the remaining rows as if they were the whole grid.
+    __shared__ __align__(16) uint16_t s_words[2 * kCoopStep * kCoopD];
+    if (queue_capacity > 0 && a.mt.T == 0 && D <= kCoopD && first_total > 0) {
+      const bool dedicated = grid_blocks >= 2 * kNumXcd;
+      const int coop_blocks =
+          dedicated ? min((first_total + kNumXcd - 1) / kNumXcd * kNumXcd, grid_blocks / (2 * kNumXcd) * kNumXcd) : 0;
+      if (!dedicated || block_index < coop_blocks) {
+        // these walks are the longest chains of the launch and share their SIMDs with the
+        // wavefronts of other workgroups: they go first when both have an instruction ready
+        __builtin_amdgcn_s_setprio(3);
+        for (int h = block_index; h < first_total; h += dedicated ? coop_blocks : grid_blocks) {
+          const QueuedRow r = row_at(kNumXcd * queue_capacity + h);
+          const int len = r.seg_end - r.seg_begin;
+          const int steps = (len + kCoopStep - 1) / kCoopStep;
+          draw_step_bits(a.sr, r.place.row_element, r.place.row_D, 0, min(kCoopStep, len), s_words,
+                         static_cast<int>(threadIdx.x), kBlockThreads);
+          __syncthreads();
+          if (wave_in_block == 0) {
+            // (one barrier per step inside the walk)
+            if (r.place.row_D <= kWave)
+              walk_long_row<T, 1, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, lane, s_words);
+            else
+              walk_long_row<T, 2, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, lane, s_words);
+          } else {
+            for (int s = 1; s <= steps; ++s) {
+              if (s < steps)
+                draw_step_bits(a.sr, r.place.row_element, r.place.row_D, s * kCoopStep,
+                               min(kCoopStep, len - s * kCoopStep), s_words + (s & 1) * (kCoopStep * kCoopD),
+                               static_cast<int>(threadIdx.x) - kWave, kBlockThreads - kWave);
+              step_barrier();
+            }
+          }
+          __syncthreads();  // the buffers are free for the next row
+        }
+        if (dedicated) return;
+        __builtin_amdgcn_s_setprio(0);
+      }
+      block_index -= coop_blocks;
+      grid_blocks -= coop_blocks;
+      first_total = 0;
+    }
+  }
+
+  const int xcd = block_index % kNumXcd;
   int queue_len[kNumXcd];
   int total = 0;
 #pragma unroll
@@ -675,15 +837,14 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     total += queue_len[x];
   }
   const int fair = total / kNumXcd + total / 16 + 1;
-  const int first_total = uniform(counters[1]);  // the rows every wavefront helps with first
   int shared_total = 0;
 #pragma unroll
   for (int x = 0; x < kNumXcd; ++x) shared_total += max(0, queue_len[x] - fair);
   const int own = min(queue_len[xcd], fair);
-  int q = static_cast<int>(blockIdx.x / kNumXcd) * kWavesPerBlock + wave_in_block;
-  const int stride = static_cast<int>(gridDim.x / kNumXcd) * kWavesPerBlock;
-  const int all_stride = static_cast<int>(gridDim.x) * kWavesPerBlock;
-  int first = static_cast<int>(blockIdx.x) * kWavesPerBlock + wave_in_block;
+  int q = (block_index / kNumXcd) * kWavesPerBlock + wave_in_block;
+  const int stride = (grid_blocks / kNumXcd) * kWavesPerBlock;
+  const int all_stride = grid_blocks * kWavesPerBlock;
+  int first = block_index * kWavesPerBlock + wave_in_block;
   int g = first;
   while (true) {
     int slot;
@@ -704,24 +865,14 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     } else {
       break;
     }
-    const int u = uniform(long_queue[slot]);
-    const int seg_begin = uniform(segment_starts[u]);
-    const int seg_end = uniform(segment_starts[u + 1]);
-    const int64_t key = uniform(keys_sorted[seg_begin]);
-    const int first_grad_row = uniform(a.grad_rows[a.positions_sorted[seg_begin]]);
-    RowPlace place = a.mt.T > 0 ? place_row<true>(key, first_grad_row, D, a.mt)
-                                : place_row<false>(key, first_grad_row, D, a.mt);
-    place.row_D = uniform(place.row_D);
-    place.row_element = uniform(place.row_element);
-    place.grad_stride = uniform(place.grad_stride);
-    place.grad_column = uniform(place.grad_column);
+    const QueuedRow r = row_at(slot);
     // elements per lane: the row spread over the 64 lanes, in loads of at most 16 bytes
-    const int per_lane = (place.row_D + kWave - 1) / kWave;
-    if (per_lane <= 1) walk_long_row<T, 1, WEIGHTED, STOCHASTIC, BIG>(a, seg_begin, seg_end, key, place, lane);
-    else if (per_lane <= 2) walk_long_row<T, 2, WEIGHTED, STOCHASTIC, BIG>(a, seg_begin, seg_end, key, place, lane);
+    const int per_lane = (r.place.row_D + kWave - 1) / kWave;
+    if (per_lane <= 1) walk_long_row<T, 1, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, lane);
+    else if (per_lane <= 2) walk_long_row<T, 2, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, lane);
     else if constexpr (sizeof(T) <= 4) {
-      if (per_lane <= 4) walk_long_row<T, 4, WEIGHTED, STOCHASTIC, BIG>(a, seg_begin, seg_end, key, place, lane);
-      else if constexpr (sizeof(T) == 2) walk_long_row<T, 8, WEIGHTED, STOCHASTIC, BIG>(a, seg_begin, seg_end, key, place, lane);
+      if (per_lane <= 4) walk_long_row<T, 4, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, lane);
+      else if constexpr (sizeof(T) == 2) walk_long_row<T, 8, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, lane);
     }
   }
 }

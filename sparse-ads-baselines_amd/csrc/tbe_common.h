@@ -182,29 +182,31 @@ struct StochasticRounding {
 // fp32 -> fp16 with stochastic rounding as in stochastic_rounding_vector
 // (table_batched_embeddings_cuda.cu:564-578): 13 random bits are added to the fp32 pattern,
 // then the value is truncated toward zero.
-// fp32 -> fp16 toward zero, bit for bit what __float2half_rz returns for every fp32 pattern (NaN
-// payloads aside) in a third of its instructions: in fp16's normal range the 13 mantissa bits it
-// has no room for are dropped, after which the conversion is exact (finite magnitudes beyond the
-// largest fp16 value stay at it); below the smallest normal value the result counts whole
-// multiples of 2^-24; infinities and NaNs convert as they are.
-__device__ __forceinline__ uint16_t float_to_half_rz_bits(float x) {
-  const uint32_t u = __float_as_uint(x);
-  const float ax = fabsf(x);
-  const float cut = __builtin_amdgcn_fmed3f(__uint_as_float(u & 0xFFFFE000u), -65504.0f, 65504.0f);
-  const __half normal = __float2half_rn(!(ax <= 3.4028234664e38f) ? x : cut);
-  const uint32_t steps = static_cast<uint32_t>(ax * 16777216.0f);
-  const uint16_t tiny = static_cast<uint16_t>(((u >> 16) & 0x8000u) | steps);
-  return ax < 6.103515625e-05f ? tiny : __half_as_ushort(normal);
+// fp32 -> fp16 toward zero: the hardware's packed conversion (v_cvt_pkrtz_f16_f32), which rounds
+// toward zero whatever the rounding mode and returns, for every one of the 2^32 fp32 patterns,
+// the bits of __float2half_rz (checked exhaustively): finite magnitudes beyond the largest fp16
+// value stay at it, values below the smallest normal one become subnormals, infinities and NaNs
+// convert as they are.
+typedef __fp16 HalfPairRz __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t floats_to_half2_rz_bits(float lo, float hi) {
+  const HalfPairRz h = __builtin_amdgcn_cvt_pkrtz(lo, hi);
+  return __builtin_bit_cast(uint32_t, h);
 }
-// one value rounded stochastically to fp16 and back: `word` is the element's random word
+__device__ __forceinline__ uint16_t float_to_half_rz_bits(float x) {
+  return static_cast<uint16_t>(floats_to_half2_rz_bits(x, 0.0f) & 0xffffu);
+}
+// one value rounded stochastically to fp16 and back: `bits` are the 13 random bits of the element
+// (the top 13 of its random word), added below the fp16 mantissa before the cut toward zero
+__device__ __forceinline__ float round_trip_with_bits(float v, uint32_t bits) {
+  return __half2float(__ushort_as_half(float_to_half_rz_bits(__uint_as_float(__float_as_uint(v) + bits))));
+}
 __device__ __forceinline__ float round_trip_stochastic(float v, uint32_t word) {
-  return __half2float(__ushort_as_half(float_to_half_rz_bits(__uint_as_float(__float_as_uint(v) + (word >> 19)))));
+  return round_trip_with_bits(v, word >> 19);
 }
 
 __device__ __forceinline__ uint32_t floats_to_half2_stochastic(float lo, float hi, uint32_t r0, uint32_t r1) {
-  const uint16_t a = float_to_half_rz_bits(__uint_as_float(__float_as_uint(lo) + (r0 >> 19)));
-  const uint16_t b = float_to_half_rz_bits(__uint_as_float(__float_as_uint(hi) + (r1 >> 19)));
-  return static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 16);
+  return floats_to_half2_rz_bits(__uint_as_float(__float_as_uint(lo) + (r0 >> 19)),
+                                 __uint_as_float(__float_as_uint(hi) + (r1 >> 19)));
 }
 
 // VEC accumulator values packed into the stored type: round to nearest even, or, for fp16 with

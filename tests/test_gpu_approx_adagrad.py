@@ -348,6 +348,45 @@ def test_approx_adagrad_stochastic_rounding_of_rows_of_many_occurrences(oracle):
     assert_close(w, w_ref, 1e-2)
 
 
+@pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("D,B", [(8, 700), (64, 700), (100, 700), (128, 700), (256, 700), (64, 64)])
+def test_approx_adagrad_stochastic_rounding_bit_for_bit_with_dyadic_gradients(oracle, D, B, weighted):
+    """With gradient entries in {0, +-0.5, +-1} and per-sample weights in {0.5, 1, 2} every sum of
+    squares is exact in fp32 whatever its order and every product with the multiplier is exact, so
+    the kernels and the oracle compute the same fp32 values and, drawing the same random words,
+    must leave the same fp16 bits -- in the rows of a few occurrences, in the rows that get a
+    wavefront (17 to 256 occurrences) and in the rows of more than 256 occurrences, which up to
+    128 elements wide are walked by a workgroup whose other wavefronts draw the random bits
+    (D = 256: a single wavefront; B = 64: one table of 512 lookups, a grid too small to set
+    workgroups aside for them)."""
+    rs = np.random.RandomState(D + B)
+    T, E, L = (2 if B > 100 else 1), 60, 8
+    p = make_problem(40, T=T, E=E, D=D, B=B, L=L, dtype=np.float16, ragged=False, weighted=weighted)
+    n_t = B * L
+    hot = [257, 300, 1000, 2049] if B > 100 else [300]
+    mid = [17, 64, 65, 200, 256] if B > 100 else [40]
+    for t in range(T):
+        rows = np.concatenate([np.full(c, r, np.int32) for r, c in enumerate(hot + mid)])
+        rest = rs.randint(len(hot + mid), E, size=n_t - rows.size).astype(np.int32)
+        p["indices"][t * n_t:(t + 1) * n_t] = rs.permutation(np.concatenate([rows, rest]))
+    p["grad_output"] = rs.choice(np.array([0, 0.5, -0.5, 1, -1], np.float16), size=p["grad_output"].shape)
+    if weighted:
+        p["per_sample_weights"] = rs.choice(np.array([0.5, 1, 2], np.float16), size=p["n"])
+    torch.cuda.init()
+    torch.manual_seed(D)
+    gen = torch.cuda.default_generators[0]
+    seed, offset = gen.initial_seed() & 0xFFFFFFFFFFFFFFFF, gen.get_offset()
+    w, st, g = _run_gpu(p, 0.02, 0.1, stochastic=True)
+    w_ref, st_ref, g_ref = _run_oracle(oracle, p, 0.02, 0.1, stochastic_rounding=(seed, offset))
+    assert st.tobytes() == st_ref.tobytes()
+    differing = np.flatnonzero((w.view(np.uint16) != w_ref.view(np.uint16)).any(axis=1))
+    assert differing.size == 0, "rows with other bits than the oracle's: %s" % differing[:10]
+    if weighted:
+        assert_close(g, g_ref, 2e-2, "grad of per-sample weights")
+    w_rn, _, _ = _run_gpu(p, 0.02, 0.1, stochastic=False)
+    assert (w.view(np.uint16) != w_rn.view(np.uint16)).mean() > 0.05  # and it is not round-to-nearest
+
+
 def test_approx_adagrad_stochastic_rounding_matches_oracle_stream(oracle):
     p = make_problem(34, T=2, E=25, D=32, B=60, L=6, dtype=np.float16, weighted=False, zipf=1.2)
     torch.manual_seed(1234)
