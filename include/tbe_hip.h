@@ -424,10 +424,10 @@ typedef struct tbe_cache_workspace_layout {
   uint64_t unique_slots;   /* int32 [U]  slot of each unique row (>= num_sets * 64: staged), -1 = backing table */
   uint64_t lookup_slots;   /* int32 [N]  the same, per lookup position                         */
   uint64_t evicted_keys;   /* int32 [U]  -2 untouched, -1 filled an empty or staging slot, >= 0 key written back */
-  uint64_t miss_sets;      /* int32 [U]  set of each missing row                               */
-  uint64_t miss_list;      /* int32 [U]  missing rows grouped by set                           */
+  uint64_t miss_sets;      /* int32 [U]  set of each missing row (num_sets: the row is resident) */
+  uint64_t miss_list;      /* int32 [U]  missing rows grouped by set, ascending inside a set   */
   uint64_t set_counts;     /* int32 [num_sets] misses per set                                  */
-  uint64_t set_fill;       /* int32 [num_sets]                                                 */
+  uint64_t set_fill;       /* int32 [num_sets]  (not used)                                     */
   uint64_t set_starts;     /* int32 [num_sets + 1]                                             */
   uint64_t stats;          /* int32 [8]: unique rows, hits, misses, inserted, written back, uncached, staged,
                             * fetched from a staging row (deferred write-back)                  */

@@ -70,6 +70,7 @@ __global__ __launch_bounds__(kBlockThreads) void cache_lookup_kernel(
         const int64_t slot = slot0 + way;
         unique_slots[u] = static_cast<int32_t>(slot);
         evicted_keys[u] = -2;
+        miss_sets[u] = static_cast<int32_t>(num_sets);  // sorts behind every set
         last_used[slot] = step;
         const int32_t c = use_count[slot];
         use_count[slot] = c == INT32_MAX ? c : c + 1;
@@ -136,19 +137,6 @@ __global__ __launch_bounds__(kBlockThreads) void cache_scan_sets_kernel(
   if (tid == 0) set_starts[num_sets] = static_cast<int32_t>(carry);
 }
 
-__global__ __launch_bounds__(kBlockThreads) void cache_group_misses_kernel(
-    const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
-    const int32_t *__restrict__ miss_sets, const int32_t *__restrict__ set_starts,
-    int32_t *__restrict__ set_fill, int32_t *__restrict__ miss_list) {
-  const int U = counters[0];
-  for (int64_t u = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; u < U;
-       u += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    if (unique_slots[u] >= 0) continue;
-    const int set = miss_sets[u];
-    miss_list[set_starts[set] + atomicAdd(&set_fill[set], 1)] = static_cast<int32_t>(u);
-  }
-}
-
 __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
     int32_t *__restrict__ tags, int32_t *__restrict__ last_used, int32_t *__restrict__ use_count,
     int64_t num_sets, int32_t policy, int32_t step, const int32_t *__restrict__ keys_sorted,
@@ -168,55 +156,55 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
     int32_t tag = tags[slot];
     int32_t used = last_used[slot];
     int32_t count = use_count[slot];
-    int staged_in_set = 0;
-    int32_t previous = -1;  // missing rows are taken in ascending order of their index u
-    for (int it = begin; it < end; ++it) {
-      int32_t candidate = INT32_MAX;
-      for (int i = begin + lane; i < end; i += kWave) {
-        const int32_t u = miss_list[i];
-        if (u > previous && u < candidate) candidate = u;
-      }
+    // The set's missing rows, miss_list[begin, end), are in ascending order of their index u.  A
+    // way can take a row while it has not served this step; every insertion uses one up, so the
+    // first `takers` rows are inserted, one after the other (each picks its victim), and all the
+    // others are staged or left in the backing table, which needs no order: lanes do them side
+    // by side.  The work per set is bounded by 64 insertions plus a pass over its list.
+    const int takers = min(static_cast<int>(__popcll(__ballot(used < step))), end - begin);
+    for (int j0 = 0; j0 < takers; j0 += kWave) {
+      const int32_t my_u = miss_list[begin + min(j0 + lane, takers - 1)];
+      const int32_t my_key = keys_sorted[segment_starts[my_u]];
+      const int batch = min(kWave, takers - j0);
+      for (int j = 0; j < batch; ++j) {
+        const int32_t u = __shfl(my_u, j, kWave);
+        const int32_t key = __shfl(my_key, j, kWave);
+        // victim: lowest (priority, way) among slots not used in this step
+        const uint32_t priority = used < step ? static_cast<uint32_t>(policy == TBE_CACHE_LFU ? count : used)
+                                              : 0xffffffffu;
+        uint32_t best = priority;
 #pragma unroll
-      for (int m = kWave / 2; m > 0; m >>= 1) candidate = min(candidate, __shfl_xor(candidate, m, kWave));
-      const int32_t u = candidate;
-      previous = u;
-      const int32_t key = keys_sorted[segment_starts[u]];
-      // victim: lowest (priority, way) among slots not used in this step
-      const uint32_t priority = used < step ? static_cast<uint32_t>(policy == TBE_CACHE_LFU ? count : used)
-                                            : 0xffffffffu;
-      uint32_t best = priority;
-#pragma unroll
-      for (int m = kWave / 2; m > 0; m >>= 1) best = min(best, static_cast<uint32_t>(__shfl_xor(static_cast<int>(best), m, kWave)));
-      if (best == 0xffffffffu) {
-        // Every way already serves this step.  The row gets a staging row for the step (index:
-        // misses of the sets before this one + rows staged by this set so far), or, when the
-        // staging area is exhausted, stays in the backing table.
-        const int64_t stage = static_cast<int64_t>(begin) + staged_in_set;
-        if (stage < stage_slots) {
-          if (lane == 0) {
-            unique_slots[u] = static_cast<int32_t>(stage_base + stage);
-            evicted_keys[u] = -1;
-          }
-          ++staged_in_set;
-          ++staged;
-        } else {
-          ++uncached;
+        for (int m = kWave / 2; m > 0; m >>= 1) best = min(best, static_cast<uint32_t>(__shfl_xor(static_cast<int>(best), m, kWave)));
+        const int way = __ffsll(static_cast<long long>(__ballot(priority == best))) - 1;
+        const int32_t old_tag = __shfl(tag, way, kWave);
+        if (lane == way) {
+          tag = key;
+          used = step;
+          count = 1;
         }
-        continue;
+        if (lane == 0) {
+          unique_slots[u] = static_cast<int32_t>(set * kWays + way);
+          evicted_keys[u] = old_tag >= 0 ? old_tag : -1;
+        }
+        ++inserted;
+        if (old_tag >= 0) ++written_back;
       }
-      const int way = __ffsll(static_cast<long long>(__ballot(priority == best))) - 1;
-      const int32_t old_tag = __shfl(tag, way, kWave);
-      if (lane == way) {
-        tag = key;
-        used = step;
-        count = 1;
+    }
+    // Every way serves this step now.  The other rows get a staging row for the step (index:
+    // misses of the sets before this one + rank among the set's staged rows), or, when the
+    // staging area is exhausted, stay in the backing table.
+    for (int j0 = begin + takers; j0 < end; j0 += kWave) {
+      const int j = j0 + lane;
+      const int64_t stage = static_cast<int64_t>(j) - takers;
+      const bool here = j < end;
+      const bool fits = here && stage < stage_slots;
+      if (fits) {
+        const int32_t u = miss_list[j];
+        unique_slots[u] = static_cast<int32_t>(stage_base + stage);
+        evicted_keys[u] = -1;
       }
-      if (lane == 0) {
-        unique_slots[u] = static_cast<int32_t>(set * kWays + way);
-        evicted_keys[u] = old_tag >= 0 ? old_tag : -1;
-      }
-      ++inserted;
-      if (old_tag >= 0) ++written_back;
+      staged += static_cast<int>(__popcll(__ballot(fits)));
+      uncached += static_cast<int>(__popcll(__ballot(here && !fits)));
     }
     tags[slot] = tag;
     last_used[slot] = used;
@@ -564,9 +552,17 @@ extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_
              i32(cw, cl.miss_sets), i32(cw, cl.set_counts), stats);
   TBE_LAUNCH("cache_scan_sets", s, cache_scan_sets_kernel, dim3(1), block, i32(cw, cl.set_counts), num_sets,
              i32(cw, cl.set_starts));
-  TBE_LAUNCH("cache_group_misses", s, cache_group_misses_kernel,
-             dim3(grid_for(num_indices, kBlockThreads, 256 * 8)), block, counters, i32(cw, cl.unique_slots),
-             i32(cw, cl.miss_sets), i32(cw, cl.set_starts), i32(cw, cl.set_fill), i32(cw, cl.miss_list));
+  // the missing rows grouped by set, each set's in ascending order of u: a stable sort of (set, u)
+  // over the U unique rows (hits carry the key num_sets and end up behind every set).  The
+  // sorted keys go to the slot-per-lookup array, which is written later; the sort's scratch is
+  // the plan's, free since the plan was built.
+  {
+    int bits = 1;
+    while ((int64_t{1} << bits) <= num_sets) ++bits;
+    const int rc_sort = sort_pairs(i32(cw, cl.miss_sets), nullptr, i32(cw, cl.lookup_slots), i32(cw, cl.miss_list),
+                                   num_indices, bits, ws + l.sort_scratch, s, nullptr, counters);
+    if (rc_sort) return rc_sort;
+  }
   TBE_LAUNCH("cache_insert", s, cache_insert_kernel, dim3(grid_for(num_sets, kWavesPerBlock, 256 * 16)), block,
              cache->tags, cache->last_used, cache->use_count, num_sets, cache->policy, step, keys_sorted,
              segment_starts, i32(cw, cl.set_starts), i32(cw, cl.miss_list), i32(cw, cl.unique_slots),

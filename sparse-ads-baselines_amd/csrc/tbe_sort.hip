@@ -132,12 +132,15 @@ constexpr int kScanChunk = kBlockThreads * kScanItems;  // 2048 count entries pe
 
 // Workgroup 0 derives the tables' position ranges and tile counts; all workgroups clear the
 // per-table digit totals of every pass (`totals_words` words; none with the linear scan).
+// device_count (nullable): the number of pairs to sort when only the device knows it (at most n,
+// for which the launches are sized: tiles past the count find nothing to do).
 __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
     const int32_t *__restrict__ offsets, int B, int num_tables, uint32_t n,
     uint32_t *__restrict__ table_starts, uint32_t *__restrict__ tile_prefix,
-    uint32_t *__restrict__ totals, int64_t totals_words) {
+    uint32_t *__restrict__ totals, int64_t totals_words, const int32_t *__restrict__ device_count) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   const int tid = threadIdx.x;
+  if (device_count) n = min(n, static_cast<uint32_t>(max(*device_count, 0)));
   for (int64_t i = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + tid) * 4; i < totals_words;
        i += static_cast<int64_t>(gridDim.x) * kBlockThreads * 4)
     *reinterpret_cast<uint4 *>(totals + i) = make_uint4(0, 0, 0, 0);
@@ -779,7 +782,7 @@ uint64_t sort_workspace_bytes(int64_t n, int32_t num_tables) { return sort_scrat
 
 int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
                int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
-               hipStream_t stream, const SortTables *tables) {
+               hipStream_t stream, const SortTables *tables, const int32_t *device_count) {
   if (n == 0) return TBE_OK;
   // Fewest passes with digits of at most 10 bits, the bits spread evenly over the passes
   // (23 bits -> 8+8+7, 25 -> 9+8+8, 27 -> 9+9+9, 17 -> 9+8).
@@ -804,7 +807,7 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   TBE_LAUNCH("sort_setup", stream, sort_setup_kernel, dim3(setup_blocks), dim3(kBlockThreads),
              tables ? tables->offsets : nullptr, tables ? tables->bags_per_table : 0, num_tables,
              static_cast<uint32_t>(n), const_cast<uint32_t *>(p.table_starts),
-             const_cast<uint32_t *>(p.tile_prefix), totals, totals_words);
+             const_cast<uint32_t *>(p.tile_prefix), totals, totals_words, device_count);
 
   p.src_k = reinterpret_cast<const uint32_t *>(keys_in);
   p.src_v = reinterpret_cast<const uint32_t *>(values_in);

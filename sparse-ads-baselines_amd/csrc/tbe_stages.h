@@ -21,9 +21,10 @@ struct SortTables {
 };
 
 uint64_t sort_workspace_bytes(int64_t n, int32_t num_tables);
+// device_count (nullable): the number of pairs, read on the device (at most n; with tables == nullptr).
 int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_out,
                int32_t *values_out, int64_t n, int32_t end_bit, void *workspace,
-               hipStream_t stream, const SortTables *tables);
+               hipStream_t stream, const SortTables *tables, const int32_t *device_count = nullptr);
 
 uint64_t segments_workspace_bytes(int64_t n);
 // segment_ids (nullable): receives, for every sorted position, the index of its segment.

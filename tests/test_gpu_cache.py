@@ -55,6 +55,41 @@ def test_cache_state_matches_model_bit_exact(oracle, policy, num_sets):
         np.testing.assert_array_equal(cache.lookup_slots.cpu().numpy(), slots[np.searchsorted(keys, all_keys)])
 
 
+@pytest.mark.parametrize("num_sets,stage_slots", [(1, 0), (1, 50000), (3, 1000)])
+def test_many_misses_per_set(oracle, num_sets, stage_slots):
+    """Hundreds of thousands of missing rows on one to three sets (a cache far too small for the
+    batch): the work per set is one pass over its misses, and slots, evictions, tags and counters
+    still equal the model's; staged rows get consecutive staging rows in ascending key order."""
+    rs = np.random.RandomState(num_sets + stage_slots)
+    rows, B, L, D = 400000, 4096, 40, 4
+    table_offsets = np.zeros(1, np.int32)
+    backing = torch.zeros(rows, D, device=DEV)
+    cache = tc.RowCache(backing, num_sets * 64, "lru", stage_slots, deferred_write_back=stage_slots > 0)
+    model = oracle.CacheModel(num_sets, "lru")
+    for step in range(3):
+        indices = rs.randint(0, rows, size=B * L).astype(np.int32)
+        offsets = np.arange(0, B * L + 1, L, dtype=np.int32)
+        cache.prepare(dev(table_offsets), dev(indices), dev(offsets))
+        keys = np.unique(indices)
+        assert keys.size > 100000
+        slots, evicted, stats = model.step(keys)
+        got_slots = cache.unique_slots().cpu().numpy()
+        staged = got_slots >= num_sets * 64
+        np.testing.assert_array_equal(np.where(staged, -1, got_slots), slots)
+        np.testing.assert_array_equal(cache.tags.cpu().numpy(), model.tags)
+        np.testing.assert_array_equal(cache.last_used.cpu().numpy(), model.last_used)
+        st = cache.stats()
+        assert st["staged"] == min(stage_slots, int((slots < 0).sum())) == int(staged.sum())
+        assert st["uncached"] == int((slots < 0).sum()) - st["staged"]
+        assert [st[k] for k in ("unique_rows", "hits", "misses", "inserted", "written_back")] == stats.tolist()[:5]
+        if st["staged"]:
+            # one staging row each, all different, inside this step's area
+            rows_used = np.sort(got_slots[staged])
+            assert np.unique(rows_used).size == rows_used.size
+            area = num_sets * 64 + (cache.step % 2) * stage_slots
+            assert rows_used[0] >= area and rows_used[-1] < area + stage_slots
+
+
 @pytest.mark.parametrize("mode,dtype,D", [("sgd", torch.float32, 128), ("adagrad", torch.float32, 64),
                                           ("adagrad_weighted", torch.float16, 64), ("sgd", torch.float32, 520),
                                           ("sgd", torch.float64, 12)])
