@@ -59,32 +59,51 @@ __global__ __launch_bounds__(kBlockThreads) void cache_lookup_kernel(
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
   int hits = 0, misses = 0;
-  for (int64_t u = wave_id; u < U; u += stride) {
-    const int32_t key = keys_sorted[segment_starts[u]];
-    const uint32_t set = cache_set_of(static_cast<uint32_t>(key), num_sets);
-    const int64_t slot0 = static_cast<int64_t>(set) * kWays;
-    const unsigned long long match = __ballot(tags[slot0 + lane] == key);
-    if (match) {
-      const int way = __ffsll(static_cast<long long>(match)) - 1;
-      if (lane == 0) {
-        const int64_t slot = slot0 + way;
+  // A wavefront takes 64 unique rows at a time: every lane fetches the key of one of them, then
+  // the sets are probed eight at a time (the whole wavefront reads a set's 64 tags with one
+  // load), so that eight tag loads are in flight instead of one; lane j keeps the outcome of
+  // row j and writes it at the end.
+  constexpr int kProbe = 8;
+  for (int64_t u0 = wave_id * kWave; u0 < U; u0 += stride * kWave) {
+    const int rows = static_cast<int>(min(static_cast<int64_t>(kWave), U - u0));
+    const int64_t my_u = u0 + min(lane, rows - 1);
+    const int32_t my_key = keys_sorted[segment_starts[my_u]];
+    const uint32_t my_set = cache_set_of(static_cast<uint32_t>(my_key), num_sets);
+    int my_way = -1;
+    for (int j0 = 0; j0 < rows; j0 += kProbe) {
+      int32_t tag[kProbe];
+#pragma unroll
+      for (int q = 0; q < kProbe; ++q) {
+        const uint32_t set = static_cast<uint32_t>(__shfl(static_cast<int>(my_set), min(j0 + q, rows - 1), kWave));
+        tag[q] = tags[static_cast<int64_t>(set) * kWays + lane];
+      }
+#pragma unroll
+      for (int q = 0; q < kProbe; ++q) {
+        const int32_t key = __shfl(my_key, min(j0 + q, rows - 1), kWave);
+        const unsigned long long match = __ballot(tag[q] == key);
+        if (lane == j0 + q && match) my_way = __ffsll(static_cast<long long>(match)) - 1;
+      }
+    }
+    if (lane < rows) {
+      const int64_t u = u0 + lane;
+      if (my_way >= 0) {
+        const int64_t slot = static_cast<int64_t>(my_set) * kWays + my_way;
         unique_slots[u] = static_cast<int32_t>(slot);
         evicted_keys[u] = -2;
         miss_sets[u] = static_cast<int32_t>(num_sets);  // sorts behind every set
         last_used[slot] = step;
         const int32_t c = use_count[slot];
         use_count[slot] = c == INT32_MAX ? c : c + 1;
-      }
-      ++hits;
-    } else {
-      if (lane == 0) {
+      } else {
         unique_slots[u] = -1;
         evicted_keys[u] = -2;
-        miss_sets[u] = static_cast<int32_t>(set);
-        atomicAdd(&set_counts[set], 1);
+        miss_sets[u] = static_cast<int32_t>(my_set);
+        atomicAdd(&set_counts[my_set], 1);
       }
-      ++misses;
     }
+    const int hit_rows = static_cast<int>(__popcll(__ballot(lane < rows && my_way >= 0)));
+    hits += hit_rows;
+    misses += rows - hit_rows;
   }
   if (lane == 0) {
     if (hits) atomicAdd(&stats[kStatHits], hits);
@@ -301,19 +320,27 @@ __global__ __launch_bounds__(kBlockThreads) void cache_fill_kernel(
   }
 }
 
-// Deferred write-back, outside a step (flush): the rows of a staging area that hold a key.
+// Deferred write-back, outside a step (flush, or the check that the area a step stages into is
+// empty): the rows of a staging area that hold a key go to the backing table.  A wavefront reads
+// 64 entries at a time and copies the rows of those that hold one, so an empty area costs one
+// pass over its entries.
 __global__ __launch_bounds__(kBlockThreads) void cache_unstage_area_kernel(
     const uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
     const int32_t *__restrict__ stage_keys, int64_t stage_base, int64_t stage_slots) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
-  for (int64_t i = wave_id; i < stage_slots; i += stride) {
-    const int64_t key = stage_keys[i];
-    if (key < 0) continue;
-    const uint64_t *src = cache_rows + (stage_base + i) * row_units;
-    uint64_t *dst = backing_rows + key * row_units;
-    for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
+  for (int64_t i0 = wave_id * kWave; i0 < stage_slots; i0 += stride * kWave) {
+    const int32_t my_key = i0 + lane < stage_slots ? stage_keys[i0 + lane] : -1;
+    unsigned long long held = __ballot(my_key >= 0);
+    while (held) {
+      const int j = __ffsll(static_cast<long long>(held)) - 1;
+      held &= held - 1;
+      const int64_t key = __shfl(my_key, j, kWave);
+      const uint64_t *src = cache_rows + (stage_base + i0 + j) * row_units;
+      uint64_t *dst = backing_rows + key * row_units;
+      for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
+    }
   }
 }
 
