@@ -1,4 +1,6 @@
-"""Builds libtbe_hip.so (the C-ABI library declared in include/tbe_hip.h) for gfx950.
+"""Builds libtbe_hip.so (the C-ABI library declared in include/tbe_hip.h) for gfx950, and
+table_batched_embeddings_cpp.so, the pybind11 module over it (host code, compiled with g++
+against PyTorch's headers).
 
 Run as a script (`python build.py`) or call `build()`.  Each .hip file is
 compiled to an object in parallel and the objects are linked into one shared
@@ -14,6 +16,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libtbe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
+BINDING_NAME = "table_batched_embeddings_cpp"
+BINDING_PATH = os.path.join(HERE, BINDING_NAME + ".so")
+BINDING_SOURCE = "table_batched_embeddings_binding.cpp"
 SOURCES = ["tbe_api.hip", "tbe_forward.hip", "tbe_sort.hip", "tbe_update.hip", "tbe_backward.hip",
            "tbe_cache.hip", "tbe_mixed.hip", "tbe_approx.hip"]
 
@@ -69,7 +74,39 @@ def build(verbose=False):
     os.replace(tmp, LIB_PATH)
     if verbose and out.strip():
         print(out)
+    build_binding(verbose)
     return LIB_PATH
+
+
+def build_binding(verbose=False):
+    """Compiles the pybind11 module (BINDING_SOURCE) and links it against LIB_PATH and PyTorch.
+    It finds the library next to itself (rpath $ORIGIN)."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    source = os.path.join(CSRC, BINDING_SOURCE)
+    if not os.path.exists(source):
+        raise RuntimeError("missing source %s" % source)
+    gxx = shutil.which("g++")
+    if gxx is None:
+        raise RuntimeError("g++ not found; the pybind11 module needs a host C++ compiler")
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    includes = [os.path.join(os.path.dirname(HERE), "include")] + cpp_extension.include_paths() + \
+        ["/opt/rocm/include", sysconfig.get_paths()["include"]]
+    tmp = BINDING_PATH + ".tmp"
+    cmd = [gxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-DTORCH_EXTENSION_NAME=" + BINDING_NAME, "-DTORCH_API_INCLUDE_EXTENSION_H",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), "-w"]
+    cmd += ["-I" + d for d in includes]
+    cmd += [source, "-o", tmp, "-L" + torch_lib, "-L" + HERE, "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10",
+            "-lc10_hip", "-ltorch_hip", "-ltbe_hip", "-Wl,-rpath,$ORIGIN"]
+    out = _run(cmd)
+    os.replace(tmp, BINDING_PATH)
+    if verbose and out.strip():
+        print(out)
+    return BINDING_PATH
 
 
 if __name__ == "__main__":

@@ -1,0 +1,82 @@
+"""The pybind11 module (table_batched_embeddings_cpp, the C++ counterpart of the reference's
+table_batched_embeddings.cpp over the C ABI) against the Python module that binds the same
+entry points: same arguments, same results bit for bit, same errors."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_problem
+from gpu_util import DEV, assert_close, dev
+
+import table_batched_embeddings as ext
+import table_batched_embeddings_cpp as ext_cpp
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype,D,weighted", [(np.float32, 128, False), (np.float16, 64, True), (np.float64, 12, True)])
+def test_cpp_module_equals_python_module(oracle, dtype, D, weighted):
+    p = make_problem(51, T=4, E=300, D=D, B=40, L=9, dtype=dtype, weighted=weighted, zipf=1.2)
+    to, idx, off = dev(p["table_offsets"]), dev(p["indices"]), dev(p["offsets"])
+    psw = dev(p["per_sample_weights"])
+    go = dev(p["grad_output"])
+    st_dtype = torch.float64 if dtype == np.float64 else torch.float32
+
+    out_py = ext.forward(dev(p["weights"]), to, idx, off, psw, 200, 1, False)
+    out_cpp = ext_cpp.forward(dev(p["weights"]), to, idx, off, psw, 200, 1, False)
+    assert torch.equal(out_py, out_cpp)
+    assert_close(out_cpp.cpu().numpy(), oracle.forward(p["weights"], p["table_offsets"], p["indices"], p["offsets"],
+                                                       p["per_sample_weights"]),
+                 {np.float32: 1e-5, np.float16: 2e-3, np.float64: 1e-12}[dtype])
+
+    if not weighted:
+        w_py, w_cpp = dev(p["weights"]), dev(p["weights"])
+        assert ext_cpp.backward_sgd(go, w_cpp, to, idx, off, 0.05, 200, 1, False) is None
+        ext.backward_sgd(go, w_py, to, idx, off, 0.05, 200, 1, False)
+        assert torch.equal(w_py, w_cpp)
+
+    for fn in ("backward_exact_adagrad", "backward_approx_adagrad"):
+        w_py, w_cpp = dev(p["weights"]), dev(p["weights"])
+        s_py = torch.zeros(w_py.shape[0], device=DEV, dtype=st_dtype)
+        s_cpp = torch.zeros_like(s_py)
+        tail = (0.05, 0.1, False, 1) if fn == "backward_exact_adagrad" else (0.05, 0.1, 200, False, 1)
+        g_py = getattr(ext, fn)(go, w_py, to, idx, off, psw, s_py, *tail)
+        g_cpp = getattr(ext_cpp, fn)(go, w_cpp, to, idx, off, psw, s_cpp, *tail)
+        assert torch.equal(w_py, w_cpp) and torch.equal(s_py, s_cpp), fn
+        assert (g_py is None) == (g_cpp is None) == (not weighted)
+        if weighted:
+            assert torch.equal(g_py, g_cpp)
+
+
+def test_cpp_module_stochastic_rounding_uses_the_generator_like_the_python_module():
+    p = make_problem(52, T=2, E=50, D=32, B=30, L=6, dtype=np.float16, zipf=1.2)
+    to, idx, off, go = dev(p["table_offsets"]), dev(p["indices"]), dev(p["offsets"]), dev(p["grad_output"])
+    results = []
+    for module in (ext, ext_cpp):
+        torch.manual_seed(77)
+        gen = torch.cuda.default_generators[0]
+        before = gen.get_offset()
+        w = dev(p["weights"])
+        st = torch.zeros(w.shape[0], device=DEV)
+        module.backward_exact_adagrad(go, w, to, idx, off, None, st, 0.05, 0.1, True, 1)
+        module.backward_approx_adagrad(go, w, to, idx, off, None, st, 0.05, 0.1, 200, True, 1)
+        assert gen.get_offset() == before + 8
+        results.append((w, st))
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+
+
+def test_cpp_module_construct_offsets_and_errors():
+    rs = np.random.RandomState(5)
+    T, B = 3, 7
+    lengths = rs.randint(0, 5, size=(T, B)).astype(np.int32)
+    starts = np.concatenate([np.zeros((T, 1), np.int32), np.cumsum(lengths, axis=1)[:, :-1]], axis=1).astype(np.int32)
+    totals = lengths.sum(axis=1).astype(np.int32)
+    got = ext_cpp.construct_offsets(dev(starts), dev(totals))
+    assert torch.equal(got, ext.construct_offsets(dev(starts), dev(totals)))
+    w = torch.zeros(8, 6, device=DEV)  # D not a multiple of 4
+    i32 = torch.zeros(2, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        ext_cpp.forward(w, i32[:1], i32[:1], i32, None, 200, 1, False)
+    with pytest.raises(RuntimeError, match="BT_block_size"):
+        ext_cpp.backward_sgd(torch.zeros(1, 1, 8, device=DEV), torch.zeros(8, 8, device=DEV), i32[:1], i32[:1], i32,
+                             0.1, 200, 0, False)

@@ -25,6 +25,23 @@ def test_extension_module_exports_the_ten_reference_functions():
         assert callable(getattr(ext, name))
 
 
+def test_cpp_module_loads_and_rejects_cpu_tensors():
+    """The pybind11 module over the C ABI (the compiled counterpart of table_batched_embeddings.cpp:56-70)."""
+    import table_batched_embeddings_cpp as ext_cpp
+    import tbe_native
+    assert ext_cpp.abi_version() == tbe_native.ABI_VERSION
+    for name in ("forward", "backward_sgd", "backward_approx_adagrad", "backward_exact_adagrad", "construct_offsets"):
+        assert callable(getattr(ext_cpp, name))
+    # positional signatures of table_batched_embeddings.cpp:6-27 in the generated docstrings
+    assert ext_cpp.forward.__doc__.count("Tensor") >= 5 and "bool" in ext_cpp.forward.__doc__
+    w = torch.zeros(8, 4)
+    i32 = torch.zeros(2, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        ext_cpp.forward(w, i32[:1], i32, i32, None, 200, 1, False)
+    with pytest.raises(TypeError):
+        ext_cpp.forward(w, i32[:1], i32, i32, None, 200, 1)  # the reference's eight positional arguments
+
+
 def test_positional_signatures_match_the_pybind_declarations():
     # table_batched_embeddings.cpp:6-27
     assert list(inspect.signature(ext.forward).parameters) == [
