@@ -387,6 +387,25 @@ def test_approx_adagrad_stochastic_rounding_bit_for_bit_with_dyadic_gradients(or
     assert (w.view(np.uint16) != w_rn.view(np.uint16)).mean() > 0.05  # and it is not round-to-nearest
 
 
+def test_approx_adagrad_stochastic_rounding_more_long_rows_than_workgroups_set_aside(oracle):
+    """1100 rows of 300 occurrences each: more rows for the cooperative walk than the 1024
+    workgroups (half the largest grid) that are set aside for them, so those take a second
+    row each.  Dyadic gradients as above: bit for bit the oracle's result."""
+    rs = np.random.RandomState(8)
+    T, E, D, B, L = 1, 1100, 8, 41250, 8
+    p = make_problem(41, T=T, E=E, D=D, B=B, L=L, dtype=np.float16, ragged=False, weighted=False)
+    p["indices"][:] = rs.permutation(np.repeat(np.arange(E, dtype=np.int32), 300))
+    p["grad_output"] = rs.choice(np.array([0, 0.5, -0.5, 1, -1], np.float16), size=p["grad_output"].shape)
+    torch.cuda.init()
+    torch.manual_seed(3)
+    gen = torch.cuda.default_generators[0]
+    seed, offset = gen.initial_seed() & 0xFFFFFFFFFFFFFFFF, gen.get_offset()
+    w, st, _ = _run_gpu(p, 0.02, 0.1, stochastic=True)
+    w_ref, st_ref, _ = _run_oracle(oracle, p, 0.02, 0.1, stochastic_rounding=(seed, offset))
+    assert st.tobytes() == st_ref.tobytes()
+    assert w.tobytes() == w_ref.tobytes()
+
+
 def test_approx_adagrad_stochastic_rounding_matches_oracle_stream(oracle):
     p = make_problem(34, T=2, E=25, D=32, B=60, L=6, dtype=np.float16, weighted=False, zipf=1.2)
     torch.manual_seed(1234)
