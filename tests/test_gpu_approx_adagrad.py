@@ -115,29 +115,34 @@ def test_approx_adagrad_rows_of_many_occurrences_in_every_lane_layout(oracle, dt
 
 
 @pytest.mark.timeout(300)
-def test_approx_adagrad_with_a_gradient_tensor_beyond_4GiB():
+@pytest.mark.parametrize("dtype,T,D,stochastic", [(torch.float32, 64, 256, False), (torch.float16, 256, 128, False),
+                                                  (torch.float16, 256, 128, True)])
+def test_approx_adagrad_with_a_gradient_tensor_beyond_4GiB(dtype, T, D, stochastic):
     """Below 4 GiB the wavefront-per-row kernel addresses gradient rows through a buffer descriptor with
     32-bit offsets, from 4 GiB on with 64-bit addresses.  A batch whose few non-empty bags are spread over a
-    4.3 GB grad_output must come out bit for bit like the same bags packed into a small one."""
-    B, T, D, E, L = 1 << 16, 64, 256, 50, 8
+    4.3 GB grad_output must come out bit for bit like the same bags packed into a small one -- fp32 rows
+    (summed in chunks), fp16 rows (walked by a wavefront) and fp16 rows with stochastic rounding (the row of
+    1 700 occurrences is walked by a workgroup)."""
+    B, E, L = 1 << 16, 50, 8
     t_used, bags = 37, 300
     rs = np.random.RandomState(38)
     gen = torch.Generator(device=DEV).manual_seed(38)
-    grad_big = torch.randn(B, T, D, device=DEV, generator=gen)
-    assert grad_big.numel() * 4 >= 1 << 32
+    grad_big = torch.randn(B, T, D, device=DEV, generator=gen, dtype=dtype)
+    assert grad_big.numel() * grad_big.element_size() >= 1 << 32
     chosen = np.sort(np.concatenate([rs.choice(B - 2, bags - 2, replace=False), [B - 2, B - 1]])).astype(np.int64)
     idx = rs.randint(0, E, size=(bags, L)).astype(np.int32)
     idx[rs.rand(bags, L) < 0.7] = 3
     lengths = np.zeros((T, B), np.int64)
     lengths[t_used, chosen] = L
     offsets_big = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
-    weights = rs.uniform(-0.01, 0.01, size=(T * E, D)).astype(np.float32)
+    weights = rs.uniform(-0.01, 0.01, size=(T * E, D)).astype(np.float32 if dtype == torch.float32 else np.float16)
     table_offsets = (np.arange(T) * E).astype(np.int32)
 
     def run(grad, table_offsets, offsets, w):
         st = torch.zeros(w.shape[0], dtype=torch.float32, device=DEV)
+        torch.manual_seed(5)  # the same random stream for both runs
         ext.backward_approx_adagrad(grad, w, dev(table_offsets), dev(idx.reshape(-1)), dev(offsets), None, st, 0.01,
-                                    0.1, 200, False, 1)
+                                    0.1, 200, stochastic, 1)
         torch.cuda.synchronize()
         return w.cpu().numpy(), st.cpu().numpy()
 
@@ -145,10 +150,12 @@ def test_approx_adagrad_with_a_gradient_tensor_beyond_4GiB():
     grad_small = grad_big[torch.from_numpy(chosen).to(DEV), t_used].reshape(bags, 1, D).contiguous()
     del grad_big
     rows = slice(t_used * E, (t_used + 1) * E)
-    w_small, st_small = run(grad_small, np.zeros(1, np.int32), (np.arange(bags + 1) * L).astype(np.int32),
-                            dev(weights[rows]))
-    assert st_big[rows].tobytes() == st_small.tobytes()
-    assert w_big[rows].tobytes() == w_small.tobytes()
+    # (the whole table again, entered at the used table's first row: a row keeps its place in the
+    # table, on which the random words of the stochastic rounding depend)
+    w_small, st_small = run(grad_small, np.full(1, t_used * E, np.int32), (np.arange(bags + 1) * L).astype(np.int32),
+                            dev(weights))
+    assert st_big.tobytes() == st_small.tobytes()
+    assert w_big.tobytes() == w_small.tobytes()
     assert st_big[3 + t_used * E] > 0 and np.bincount(idx.reshape(-1)).max() > 1500
     untouched = np.ones(T * E, bool)
     untouched[rows] = False
