@@ -5,10 +5,10 @@
 // failures as RuntimeError, kernels launched on the current stream of the weights' device, nothing
 // synchronised.  Host code only: the kernels are in the library.
 //
-// The uniform-table functions of the hot path are bound here (forward, backward_sgd,
-// backward_exact_adagrad, backward_approx_adagrad, construct_offsets); the Python module
-// table_batched_embeddings.py binds the same entry points plus the mixed-dimension, host-memory and
-// plan-ahead ones.
+// All ten functions of the reference's module are bound (forward, backward_sgd,
+// backward_approx_adagrad, backward_exact_adagrad, their three mixed-dimension counterparts,
+// construct_offsets, new_managed_tensor, new_host_mapped_tensor); the Python module
+// table_batched_embeddings.py binds the same entry points plus the plan-ahead and cache ones.
 #include <torch/extension.h>
 
 // (PyTorch on ROCm presents the GPU under the device type "cuda": the guard and the stream are
@@ -20,6 +20,7 @@
 #include <map>
 #include <mutex>
 #include <iterator>
+#include <vector>
 
 #include "tbe_hip.h"
 
@@ -111,42 +112,59 @@ at::Tensor &workspace(const at::Tensor &like, uint64_t bytes) {
   return ws;
 }
 
-// The largest table's row count decides how many key bits the backward sorts.  It is derived
-// from table_offsets once per tensor (one device-to-host copy) and kept while that tensor lives
-// and is not written to: an entry holds a weak reference to the tensor, which also keeps its
-// address from being handed to another tensor, and the version counter it had.
-int64_t max_table_rows(const at::Tensor &table_offsets, int64_t total_rows) {
+// Small int32 tensors whose values the host needs (table_offsets for the largest table's row
+// count, which decides how many key bits the backward sorts; dim_offsets for the vector width of
+// fp16 rows) are copied to the host once per tensor and kept while that tensor lives and is not
+// written to: an entry holds a weak reference to the tensor, which also keeps its address from
+// being handed to another tensor, and the version counter it had.
+std::vector<int32_t> host_values(const at::Tensor &t) {
   struct Known {
     c10::weak_intrusive_ptr<c10::TensorImpl> tensor;
     uint32_t version;
-    int64_t total_rows;
-    int64_t largest;
+    std::vector<int32_t> values;
   };
   static std::mutex mutex;
   static std::map<const void *, Known> known;
-  const void *address = table_offsets.unsafeGetTensorImpl();
+  const void *address = t.unsafeGetTensorImpl();
   {
     std::lock_guard<std::mutex> lock(mutex);
     const auto it = known.find(address);
     if (it != known.end()) {
-      if (!it->second.tensor.expired() && it->second.version == table_offsets._version() &&
-          it->second.total_rows == total_rows)
-        return it->second.largest;
+      if (!it->second.tensor.expired() && it->second.version == t._version()) return it->second.values;
       known.erase(it);
     }
   }
-  const at::Tensor host = table_offsets.cpu();
-  const int32_t *starts = host.data_ptr<int32_t>();
-  int64_t largest = 0;
-  for (int64_t t = 0; t < host.numel(); ++t) {
-    const int64_t end = t + 1 < host.numel() ? starts[t + 1] : total_rows;
-    largest = std::max<int64_t>(largest, end - starts[t]);
-  }
+  const at::Tensor host = t.cpu().contiguous();
+  std::vector<int32_t> values(host.data_ptr<int32_t>(), host.data_ptr<int32_t>() + host.numel());
   std::lock_guard<std::mutex> lock(mutex);
   for (auto it = known.begin(); it != known.end();) it = it->second.tensor.expired() ? known.erase(it) : std::next(it);
-  known.emplace(address, Known{c10::weak_intrusive_ptr<c10::TensorImpl>(table_offsets.getIntrusivePtr()),
-                               table_offsets._version(), total_rows, largest});
+  known.emplace(address, Known{c10::weak_intrusive_ptr<c10::TensorImpl>(t.getIntrusivePtr()), t._version(), values});
+  return values;
+}
+
+// starts: first row of every table; uniform tables have T entries and end at total_rows, the
+// mixed-dimension modules pass T + 1 entries (total_rows < 0: the last entry is the end).
+int64_t max_table_rows(const at::Tensor &starts_tensor, int64_t total_rows) {
+  const std::vector<int32_t> starts = host_values(starts_tensor);
+  const int64_t tables = total_rows < 0 ? static_cast<int64_t>(starts.size()) - 1 : static_cast<int64_t>(starts.size());
+  int64_t largest = 0;
+  for (int64_t t = 0; t < tables; ++t) {
+    const int64_t end = t + 1 < static_cast<int64_t>(starts.size()) ? starts[t + 1] : total_rows;
+    largest = std::max<int64_t>(largest, end - starts[t]);
+  }
   return largest;
+}
+
+// fp16 rows move 16 bytes at a time when every table's D allows it, else 8 bytes.
+int32_t fp16_vector_width(const at::Tensor &dim_offsets) {
+  const std::vector<int32_t> offsets = host_values(dim_offsets);
+  int32_t width = 8;
+  for (size_t t = 0; t + 1 < offsets.size(); ++t) {
+    const int32_t d = offsets[t + 1] - offsets[t];
+    TORCH_CHECK(d > 0 && d % 4 == 0, "every D_t must be a positive multiple of 4");
+    if (d % 8 != 0) width = 4;
+  }
+  return width;
 }
 
 uint64_t workspace_bytes(const Shape &s, int32_t dtype) {
@@ -284,6 +302,153 @@ at::Tensor construct_offsets(at::Tensor batch_offsets_per_table, at::Tensor tota
   return output;
 }
 
+struct MixedShape {
+  int32_t T, B;
+  int64_t n;
+};
+
+// table_batched_embeddings_cuda.cu:945-962: weights is the flat 1-D buffer of all tables,
+// table_offsets int64 [T+1] element offsets, dim_offsets int32 [T+1] column offsets.
+MixedShape check_mixed(const at::Tensor &weights, const at::Tensor &table_offsets, const at::Tensor &dim_offsets,
+                       const at::Tensor &indices, const at::Tensor &offsets) {
+  TORCH_CHECK(weights.is_cuda(), "weights must be a GPU tensor");
+  TORCH_CHECK(weights.dim() == 1 && weights.is_contiguous(), "weights must be a contiguous 1-D tensor");
+  TORCH_CHECK(table_offsets.scalar_type() == at::kLong, "table_offsets must be int64");
+  for (const at::Tensor *t : {&dim_offsets, &indices, &offsets})
+    TORCH_CHECK(t->scalar_type() == at::kInt, "dim_offsets, indices and offsets must be int32");
+  for (const at::Tensor *t : {&table_offsets, &dim_offsets, &indices, &offsets}) {
+    TORCH_CHECK(t->device() == weights.device(), "all tensors must live on the weights' device");
+    TORCH_CHECK(t->dim() == 1 && t->is_contiguous(), "offsets and indices must be contiguous 1-D tensors");
+  }
+  MixedShape s;
+  s.T = static_cast<int32_t>(table_offsets.numel() - 1);
+  TORCH_CHECK(s.T > 0, "T must be positive");
+  TORCH_CHECK(dim_offsets.numel() == s.T + 1, "dim_offsets must hold T+1 entries");
+  s.B = static_cast<int32_t>((offsets.numel() - 1) / s.T);
+  TORCH_CHECK(s.B > 0 && offsets.numel() == static_cast<int64_t>(s.T) * s.B + 1, "offsets must hold T*B+1 entries");
+  s.n = indices.numel();
+  return s;
+}
+
+// batched_embedding_forward_mixed_D_cuda (table_batched_embeddings_cuda.cu:945-1004).
+at::Tensor forward_mixed_D(at::Tensor weights, at::Tensor table_offsets, at::Tensor dim_offsets, int64_t total_D,
+                           at::Tensor indices, at::Tensor offsets, c10::optional<at::Tensor> indice_weights,
+                           int64_t L_max, int64_t BT_block_size, bool shmem) {
+  (void)L_max;
+  (void)shmem;
+  const MixedShape s = check_mixed(weights, table_offsets, dim_offsets, indices, offsets);
+  TORCH_CHECK(BT_block_size != 0, "BT_block_size must be non-zero");
+  check_weights_of_lookups(indice_weights, weights, indices);
+  c10::DeviceGuard guard(weights.device());
+  at::Tensor output = at::empty({s.B, total_D}, weights.options());
+  check(tbe_forward_mixed(weights.data_ptr(), dtype_code(weights), fp16_vector_width(dim_offsets),
+                          table_offsets.data_ptr<int64_t>(), dim_offsets.data_ptr<int32_t>(),
+                          static_cast<int32_t>(total_D), s.T, indices.data_ptr<int32_t>(), s.n,
+                          offsets.data_ptr<int32_t>(), s.B, ptr(indice_weights), output.data_ptr(),
+                          stream_of(weights)));
+  return output;
+}
+
+c10::optional<at::Tensor> backward_mixed(int32_t optimizer, at::Tensor grad_output, const at::Tensor &weights,
+                                         const at::Tensor &table_offsets, const at::Tensor &table_dim_offsets,
+                                         const at::Tensor &dim_offsets, int64_t total_D, const at::Tensor &indices,
+                                         const at::Tensor &offsets, const c10::optional<at::Tensor> &indice_weights,
+                                         const at::Tensor &optimizer_state, double learning_rate, double eps,
+                                         bool stochastic_rounding, int64_t BT_block_size) {
+  const MixedShape s = check_mixed(weights, table_offsets, dim_offsets, indices, offsets);
+  TORCH_CHECK(BT_block_size > 0, "BT_block_size must be positive");
+  TORCH_CHECK(table_dim_offsets.scalar_type() == at::kInt && table_dim_offsets.numel() == s.T + 1 &&
+                  table_dim_offsets.is_contiguous() && table_dim_offsets.device() == weights.device(),
+              "table_dim_offsets must be a contiguous int32 tensor with T+1 entries on the weights' device");
+  TORCH_CHECK(grad_output.scalar_type() == weights.scalar_type() && grad_output.dim() == 2 &&
+                  grad_output.size(0) == s.B && grad_output.size(1) == total_D &&
+                  grad_output.device() == weights.device(),
+              "grad_output must be [B, total_D] of the weights' dtype");
+  grad_output = grad_output.contiguous();
+  const auto want = weights.scalar_type() == at::kDouble ? at::kDouble : at::kFloat;
+  TORCH_CHECK(optimizer_state.scalar_type() == want && optimizer_state.is_contiguous() &&
+                  optimizer_state.device() == weights.device(),
+              "optimizer_state must be contiguous float32 (float64 for float64 weights)");
+  check_weights_of_lookups(indice_weights, weights, indices);
+  const int32_t dtype = dtype_code(weights);
+  c10::DeviceGuard guard(weights.device());
+  c10::optional<at::Tensor> grad_indice_weights;
+  if (indice_weights.has_value()) grad_indice_weights = at::empty_like(*indice_weights);
+  tbe_workspace_layout_t layout;
+  check(tbe_backward_workspace_layout(s.n, 4, dtype, s.T, &layout));
+  at::Tensor &ws = workspace(weights, layout.total_bytes);
+  const bool rounds = stochastic_rounding && weights.scalar_type() == at::kHalf;
+  std::pair<uint64_t, uint64_t> stream{0, 0};
+  if (rounds) stream = rounding_stream(weights);
+  check(tbe_backward_mixed(optimizer, grad_output.data_ptr(), weights.data_ptr(), dtype, fp16_vector_width(dim_offsets),
+                           optimizer_state.numel(), max_table_rows(table_dim_offsets, -1),
+                           table_offsets.data_ptr<int64_t>(), table_dim_offsets.data_ptr<int32_t>(),
+                           dim_offsets.data_ptr<int32_t>(), static_cast<int32_t>(total_D), s.T,
+                           indices.data_ptr<int32_t>(), s.n, offsets.data_ptr<int32_t>(), s.B, ptr(indice_weights),
+                           optimizer_state.data_ptr(), static_cast<float>(learning_rate), static_cast<float>(eps),
+                           grad_indice_weights.has_value() ? grad_indice_weights->data_ptr() : nullptr, rounds ? 1 : 0,
+                           stream.first, stream.second, ws.data_ptr(), static_cast<uint64_t>(ws.numel()),
+                           stream_of(weights)));
+  return grad_indice_weights;
+}
+
+// batched_embedding_backward_adagrad_exact_mixed_D_cuda (table_batched_embeddings_cuda.cu:1350-1469).
+c10::optional<at::Tensor> backward_exact_adagrad_mixed_D(at::Tensor grad_output, at::Tensor weights,
+                                                         at::Tensor table_offsets, at::Tensor table_dim_offsets,
+                                                         at::Tensor dim_offsets, int64_t total_D, at::Tensor indices,
+                                                         at::Tensor offsets, c10::optional<at::Tensor> indice_weights,
+                                                         at::Tensor optimizer_state, double learning_rate, double eps,
+                                                         bool stochastic_rounding, int64_t BT_block_size) {
+  return backward_mixed(TBE_OPT_ROWWISE_ADAGRAD, grad_output, weights, table_offsets, table_dim_offsets, dim_offsets,
+                        total_D, indices, offsets, indice_weights, optimizer_state, learning_rate, eps,
+                        stochastic_rounding, BT_block_size);
+}
+
+// batched_embedding_backward_adagrad_approx_mixed_D_cuda (table_batched_embeddings_cuda.cu:1076-1163).
+c10::optional<at::Tensor> backward_approx_adagrad_mixed_D(at::Tensor grad_output, at::Tensor weights,
+                                                          at::Tensor table_offsets, at::Tensor table_dim_offsets,
+                                                          at::Tensor dim_offsets, int64_t total_D, at::Tensor indices,
+                                                          at::Tensor offsets, c10::optional<at::Tensor> indice_weights,
+                                                          at::Tensor optimizer_state, double learning_rate, double eps,
+                                                          int64_t L_max, bool stochastic_rounding,
+                                                          int64_t BT_block_size) {
+  (void)L_max;
+  return backward_mixed(TBE_OPT_APPROX_ROWWISE_ADAGRAD, grad_output, weights, table_offsets, table_dim_offsets,
+                        dim_offsets, total_D, indices, offsets, indice_weights, optimizer_state, learning_rate, eps,
+                        stochastic_rounding, BT_block_size);
+}
+
+int64_t bytes_of(const at::Tensor &self, const std::vector<int64_t> &sizes) {
+  TORCH_CHECK(self.is_cuda() && self.is_floating_point(), "the prototype must be a floating GPU tensor");
+  int64_t bytes = static_cast<int64_t>(self.element_size());
+  for (const int64_t size : sizes) {
+    TORCH_CHECK(size >= 0, "sizes must not be negative");
+    bytes *= size;
+  }
+  return bytes;
+}
+
+// new_managed_tensor (table_batched_embeddings_cuda.cu:864-871): managed memory preferring the
+// host, tagged with the prototype's device and dtype; released with the tensor's storage, as by
+// the reference's CUDAManagedDeleter (:795-812).
+at::Tensor new_managed_tensor(at::Tensor self, std::vector<int64_t> sizes) {
+  const int64_t bytes = bytes_of(self, sizes);
+  c10::DeviceGuard guard(self.device());
+  void *memory = nullptr;
+  check(tbe_managed_alloc(static_cast<uint64_t>(std::max<int64_t>(bytes, 1)), self.get_device(), &memory));
+  return at::from_blob(memory, sizes, [](void *p) { tbe_managed_free(p); }, self.options(), self.device());
+}
+
+// new_host_mapped_tensor (table_batched_embeddings_cuda.cu:873-880): pinned host memory mapped
+// into the device's address space; released with the tensor's storage (CUDAHostMappedDeleter, :820-835).
+at::Tensor new_host_mapped_tensor(at::Tensor self, std::vector<int64_t> sizes) {
+  const int64_t bytes = bytes_of(self, sizes);
+  c10::DeviceGuard guard(self.device());
+  void *host = nullptr, *device = nullptr;
+  check(tbe_host_mapped_alloc(static_cast<uint64_t>(std::max<int64_t>(bytes, 1)), &host, &device));
+  return at::from_blob(device, sizes, [host](void *) { tbe_host_mapped_free(host); }, self.options(), self.device());
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -292,5 +457,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("backward_exact_adagrad", &backward_exact_adagrad, "backward_exact_adagrad");
   m.def("backward_approx_adagrad", &backward_approx_adagrad, "backward_approx_adagrad");
   m.def("construct_offsets", &construct_offsets, "construct_offsets");
+  m.def("forward_mixed_D", &forward_mixed_D, "forward_mixed_D");
+  m.def("backward_exact_adagrad_mixed_D", &backward_exact_adagrad_mixed_D, "backward_exact_adagrad_mixed_D");
+  m.def("backward_approx_adagrad_mixed_D", &backward_approx_adagrad_mixed_D, "backward_approx_adagrad_mixed_D");
+  m.def("new_managed_tensor", &new_managed_tensor, "new_managed_tensor");
+  m.def("new_host_mapped_tensor", &new_host_mapped_tensor, "new_host_mapped_tensor");
   m.def("abi_version", []() { return tbe_abi_version(); }, "version of the C ABI the library exports");
 }

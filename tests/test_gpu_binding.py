@@ -80,3 +80,54 @@ def test_cpp_module_construct_offsets_and_errors():
     with pytest.raises(RuntimeError, match="BT_block_size"):
         ext_cpp.backward_sgd(torch.zeros(1, 1, 8, device=DEV), torch.zeros(8, 8, device=DEV), i32[:1], i32[:1], i32,
                              0.1, 200, 0, False)
+
+
+@pytest.mark.parametrize("dtype,weighted", [(np.float32, False), (np.float16, True)])
+def test_cpp_module_mixed_dimension_functions(dtype, weighted):
+    from conftest import make_mixed_problem
+    tables = [(30, 8), (7, 32), (100, 4), (900, 260), (16, 12)]
+    p = make_mixed_problem(9, tables, B=21, L=9, dtype=dtype, weighted=weighted)
+    to, tdo, do = dev(p["table_offsets"]), dev(p["table_dim_offsets"]), dev(p["dim_offsets"])
+    idx, off, psw, go = dev(p["indices"]), dev(p["offsets"]), dev(p["per_sample_weights"]), dev(p["grad_output"])
+    total_D = int(p["dim_offsets"][-1])
+    out_py = ext.forward_mixed_D(dev(p["weights"]), to, do, total_D, idx, off, psw, 200, 1, False)
+    out_cpp = ext_cpp.forward_mixed_D(dev(p["weights"]), to, do, total_D, idx, off, psw, 200, 1, False)
+    assert torch.equal(out_py, out_cpp)
+    for fn in ("backward_exact_adagrad_mixed_D", "backward_approx_adagrad_mixed_D"):
+        w_py, w_cpp = dev(p["weights"]), dev(p["weights"])
+        s_py = torch.zeros(sum(p["rows"]), device=DEV)
+        s_cpp = torch.zeros_like(s_py)
+        tail = (0.05, 0.1, False, 1) if "exact" in fn else (0.05, 0.1, 200, False, 1)
+        g_py = getattr(ext, fn)(go, w_py, to, tdo, do, total_D, idx, off, psw, s_py, *tail)
+        g_cpp = getattr(ext_cpp, fn)(go, w_cpp, to, tdo, do, total_D, idx, off, psw, s_cpp, *tail)
+        assert torch.equal(w_py, w_cpp) and torch.equal(s_py, s_cpp), fn
+        if weighted:
+            assert torch.equal(g_py, g_cpp)
+        else:
+            assert g_py is None and g_cpp is None
+
+
+@pytest.mark.parametrize("maker", ["new_host_mapped_tensor", "new_managed_tensor"])
+def test_cpp_module_host_tensors(maker):
+    """Tensors over host memory made by the compiled module behave like device tensors: torch ops
+    and the kernels read and update them; the memory goes with the storage (the reference's
+    deleters, table_batched_embeddings_cuda.cu:795-835)."""
+    p = make_problem(53, T=2, E=60, D=16, B=12, L=5, dtype=np.float32)
+    proto = torch.empty(1, device=DEV)
+    w_host = getattr(ext_cpp, maker)(proto, [2 * 60, 16])
+    assert w_host.is_cuda and w_host.dtype == torch.float32 and tuple(w_host.shape) == (120, 16)
+    w_host.copy_(dev(p["weights"]))
+    w_dev = dev(p["weights"])
+    to, idx, off, go = dev(p["table_offsets"]), dev(p["indices"]), dev(p["offsets"]), dev(p["grad_output"])
+    assert torch.equal(ext_cpp.forward(w_host, to, idx, off, None, 200, 1, False),
+                       ext_cpp.forward(w_dev, to, idx, off, None, 200, 1, False))
+    ext_cpp.backward_sgd(go, w_host, to, idx, off, 0.1, 200, 1, False)
+    ext_cpp.backward_sgd(go, w_dev, to, idx, off, 0.1, 200, 1, False)
+    torch.cuda.synchronize()
+    assert torch.equal(w_host, w_dev)
+    view = w_host[3:5]
+    del w_host          # the view keeps the storage, and with it the memory, alive
+    torch.cuda.synchronize()
+    assert torch.equal(view, w_dev[3:5])
+    del view
+    torch.cuda.synchronize()

@@ -30,7 +30,10 @@ def test_cpp_module_loads_and_rejects_cpu_tensors():
     import table_batched_embeddings_cpp as ext_cpp
     import tbe_native
     assert ext_cpp.abi_version() == tbe_native.ABI_VERSION
-    for name in ("forward", "backward_sgd", "backward_approx_adagrad", "backward_exact_adagrad", "construct_offsets"):
+    # the ten names of table_batched_embeddings.cpp:56-70
+    for name in ("forward", "backward_sgd", "backward_approx_adagrad", "backward_exact_adagrad",
+                 "backward_approx_adagrad_mixed_D", "backward_exact_adagrad_mixed_D", "forward_mixed_D",
+                 "construct_offsets", "new_managed_tensor", "new_host_mapped_tensor"):
         assert callable(getattr(ext_cpp, name))
     # positional signatures of table_batched_embeddings.cpp:6-27 in the generated docstrings
     assert ext_cpp.forward.__doc__.count("Tensor") >= 5 and "bool" in ext_cpp.forward.__doc__
