@@ -20,6 +20,21 @@ from torch import nn
 import table_batched_embeddings
 import table_batched_embeddings_cache
 
+# The module behind the ten functions that the reference imports as `table_batched_embeddings`
+# (table_batched_embeddings_ops.py:24, 53, 148): the Python binding of the C ABI by default, or the
+# compiled one (table_batched_embeddings_cpp, same names and positional arguments) after
+# use_extension().  What the reference's module does not have (plan-ahead, the row cache, exact SGD
+# for mixed-dimension tables) always comes from the Python binding.
+extension = table_batched_embeddings
+
+
+def use_extension(module):
+    """Routes the reference's ten extension functions through `module`
+    (table_batched_embeddings or table_batched_embeddings_cpp); returns the previous one."""
+    global extension
+    previous, extension = extension, module
+    return previous
+
 
 class Optimizer(enum.Enum):
     SGD = 1
@@ -61,7 +76,7 @@ class LookupFunction(torch.autograd.Function):
         if (LookupFunction.plan_ahead and any(ctx.needs_input_grad)
                 and optimizer != Optimizer.APPROX_ROWWISE_ADAGRAD):
             ctx.plan = table_batched_embeddings.plan_backward(weights, table_offsets, indices, offsets)
-        return table_batched_embeddings.forward(
+        return extension.forward(
             weights, table_offsets, indices, offsets, per_sample_weights, L_max,
             _launch_block(weights.shape[1]), False)
 
@@ -80,15 +95,15 @@ class LookupFunction(torch.autograd.Function):
                                                 ctx.learning_rate, ctx.eps, ctx.stochastic_rounding)
         elif ctx.optimizer == Optimizer.SGD:
             assert per_sample_weights is None
-            grad_per_sample_weight = table_batched_embeddings.backward_sgd(
+            grad_per_sample_weight = extension.backward_sgd(
                 grad_output, weights, table_offsets, indices, offsets, ctx.learning_rate, L_max,
                 _launch_block(weights.shape[1]), False)
         elif ctx.optimizer == Optimizer.APPROX_ROWWISE_ADAGRAD:
-            grad_per_sample_weight = table_batched_embeddings.backward_approx_adagrad(
+            grad_per_sample_weight = extension.backward_approx_adagrad(
                 grad_output, weights, table_offsets, indices, offsets, per_sample_weights,
                 optimizer_state, ctx.learning_rate, ctx.eps, L_max, ctx.stochastic_rounding, 1)
         else:
-            grad_per_sample_weight = table_batched_embeddings.backward_exact_adagrad(
+            grad_per_sample_weight = extension.backward_exact_adagrad(
                 grad_output, weights, table_offsets, indices, offsets, per_sample_weights,
                 optimizer_state, ctx.learning_rate, ctx.eps, ctx.stochastic_rounding, 1)
         # The update is already applied; autograd receives an empty sparse gradient of the
@@ -162,12 +177,12 @@ class TableBatchedEmbeddingBags(nn.Module):
             embedding_data = torch.randn(total_rows, embedding_dim, device=device, dtype=dtype)
         elif managed == EmbeddingLocation.HOST_MAPPED:
             logging.info("Allocating host-mapped embedding bag")
-            embedding_data = table_batched_embeddings.new_managed_tensor(
+            embedding_data = extension.new_managed_tensor(
                 torch.empty(1, device=device, dtype=dtype), (total_rows, embedding_dim))
             embedding_data.normal_()
         else:
             logging.info("Allocating pinned host embedding bag behind an HBM row cache")
-            embedding_data = table_batched_embeddings.new_host_mapped_tensor(
+            embedding_data = extension.new_host_mapped_tensor(
                 torch.empty(1, device=device, dtype=dtype), (total_rows, embedding_dim))
             embedding_data.normal_()
         self.embedding_weights = nn.Parameter(embedding_data)
@@ -227,7 +242,7 @@ class MixedDimLookupFunction(torch.autograd.Function):
         ctx.total_D = total_D
         ctx.save_for_backward(weights, table_offsets, table_dim_offsets, dim_offsets, indices, offsets,
                               per_sample_weights, optimizer_state)
-        return table_batched_embeddings.forward_mixed_D(
+        return extension.forward_mixed_D(
             weights, table_offsets, dim_offsets, total_D, indices, offsets, per_sample_weights, 200, 1, False)
 
     @staticmethod
@@ -241,11 +256,11 @@ class MixedDimLookupFunction(torch.autograd.Function):
                 grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, ctx.total_D, indices, offsets,
                 optimizer_state, ctx.learning_rate)
         elif ctx.optimizer == Optimizer.APPROX_ROWWISE_ADAGRAD:
-            grad_per_sample_weight = table_batched_embeddings.backward_approx_adagrad_mixed_D(
+            grad_per_sample_weight = extension.backward_approx_adagrad_mixed_D(
                 grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, ctx.total_D, indices, offsets,
                 per_sample_weights, optimizer_state, ctx.learning_rate, ctx.eps, L_max, ctx.stochastic_rounding, 1)
         else:
-            grad_per_sample_weight = table_batched_embeddings.backward_exact_adagrad_mixed_D(
+            grad_per_sample_weight = extension.backward_exact_adagrad_mixed_D(
                 grad_output, weights, table_offsets, table_dim_offsets, dim_offsets, ctx.total_D, indices, offsets,
                 per_sample_weights, optimizer_state, ctx.learning_rate, ctx.eps, ctx.stochastic_rounding, 1)
         empty_grad = None
@@ -275,7 +290,7 @@ class MixedDimTableBatchedEmbeddingBags(nn.Module):
             embedding_data = torch.randn(size=(numel,), device=device, dtype=dtype)
         else:
             logging.info("Allocating host-mapped embedding bag")
-            embedding_data = table_batched_embeddings.new_managed_tensor(
+            embedding_data = extension.new_managed_tensor(
                 torch.empty(1, device=device, dtype=dtype), (numel,))
             embedding_data.normal_()
         self.embedding_weights = nn.Parameter(embedding_data)

@@ -131,3 +131,40 @@ def test_cpp_module_host_tensors(maker):
     assert torch.equal(view, w_dev[3:5])
     del view
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("optimizer,fp16,weighted,managed", [("SGD", False, False, "DEVICE"),
+                                                             ("EXACT_ROWWISE_ADAGRAD", True, True, "DEVICE"),
+                                                             ("APPROX_ROWWISE_ADAGRAD", False, False, "HOST_MAPPED")])
+def test_module_over_the_compiled_extension(optimizer, fp16, weighted, managed):
+    """table_batched_embeddings_ops.py over the compiled module -- the reference's own layering
+    (Python module -> pybind11 extension -> kernels): the same training trajectory, bit for bit,
+    as over the Python binding."""
+    import table_batched_embeddings_ops as ops
+    T, E, D, B, L = 3, 200, 32, 24, 6
+    rs = np.random.RandomState(14)
+    results = []
+    for module in (ext, ext_cpp):
+        previous = ops.use_extension(module)
+        try:
+            torch.manual_seed(21)
+            cc = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=getattr(ops.Optimizer, optimizer), learning_rate=0.05,
+                                               eps=0.1, fp16=fp16, managed=getattr(ops.EmbeddingLocation, managed)).cuda()
+            steps = np.random.RandomState(15)
+            for _ in range(3):
+                indices = dev((steps.zipf(1.3, size=T * B * L) % E).astype(np.int32))
+                offsets = dev(np.arange(0, T * B * L + 1, L, dtype=np.int32))
+                psw = None
+                if weighted:
+                    psw = dev(steps.rand(T * B * L).astype(np.float16 if fp16 else np.float32)).requires_grad_()
+                out = cc(indices, offsets, psw)
+                out.backward(dev(steps.randn(B, T, D).astype(np.float16 if fp16 else np.float32)))
+            torch.cuda.synchronize()
+            results.append((cc.embedding_weights.detach().clone(), cc.optimizer_state.clone(),
+                            None if psw is None else psw.grad.clone()))
+        finally:
+            ops.use_extension(previous)
+    assert torch.equal(results[0][0], results[1][0])
+    assert torch.equal(results[0][1], results[1][1])
+    if weighted:
+        assert torch.equal(results[0][2], results[1][2])
