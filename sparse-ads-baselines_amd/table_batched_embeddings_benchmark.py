@@ -1,6 +1,7 @@
 """Micro-benchmark CLI with the flags of the reference's table_batched_embeddings_benchmark.py
 (:360-370): --num-tables 64 --num-embeddings 10000 --embedding-dim 32 --batch-size 128
---bag-size 32 --iters 100 [--fp16] [--managed] [--mixed] [--remote], plus --alpha / --seed.
+--bag-size 32 --iters 100 [--fp16] [--managed] [--mixed] [--remote], plus --alpha / --seed / --kernels /
+--compiled.
 
 Each operator is called directly on the extension-module mirror (not through autograd), after
 one warm-up call, `iters` times between two events on the current stream
@@ -18,6 +19,9 @@ import torch
 
 import table_batched_embeddings
 import table_batched_embeddings_ops as ops
+
+# the module whose functions are timed: the Python binding of the C ABI, or the compiled one (--compiled)
+EXT = table_batched_embeddings
 
 HBM_PEAK_GBPS = 8000.0
 
@@ -88,15 +92,15 @@ def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
     fwd_bytes = elem * B * T * L * D_eff
 
     if mixed:
-        fwd = lambda: table_batched_embeddings.forward_mixed_D(
+        fwd = lambda: EXT.forward_mixed_D(
             w, cc.table_offsets, cc.dim_offsets, cc.total_D, indices, offsets, None, L, 1, False)
     else:
-        fwd = lambda: table_batched_embeddings.forward(w, cc.table_offsets, indices, offsets, None, L, 1, False)
+        fwd = lambda: EXT.forward(w, cc.table_offsets, indices, offsets, None, L, 1, False)
     y0 = fwd()
     if not mixed:  # the launch knobs of the reference must not change results (:179-206)
         for bt in (1, 2, 4, 8, 16, 32, 64, 128):
             for shmem in (True, False):
-                assert torch.equal(table_batched_embeddings.forward(w, cc.table_offsets, indices, offsets, None, L,
+                assert torch.equal(EXT.forward(w, cc.table_offsets, indices, offsets, None, L,
                                                                     bt, shmem), y0)
     report("Forward", time_calls(iters, fwd), fwd_bytes, shape)
 
@@ -107,7 +111,7 @@ def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
             go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets,
             cc.optimizer_state, lr)
     else:
-        sgd = lambda: table_batched_embeddings.backward_sgd(go, w, cc.table_offsets, indices, offsets, lr, L, 1,
+        sgd = lambda: EXT.backward_sgd(go, w, cc.table_offsets, indices, offsets, lr, L, 1,
                                                             False)
     report("Backward-SGD-EXACT", time_calls(iters, sgd), 2 * fwd_bytes, shape)
 
@@ -117,16 +121,16 @@ def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
     def adagrad(exact, stochastic):
         if mixed:
             if exact:
-                return lambda: table_batched_embeddings.backward_exact_adagrad_mixed_D(
+                return lambda: EXT.backward_exact_adagrad_mixed_D(
                     go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets,
                     None, cc.optimizer_state, lr, eps, stochastic, 1)
-            return lambda: table_batched_embeddings.backward_approx_adagrad_mixed_D(
+            return lambda: EXT.backward_approx_adagrad_mixed_D(
                 go, w, cc.table_offsets, cc.table_dim_offsets, cc.dim_offsets, cc.total_D, indices, offsets, None,
                 cc.optimizer_state, lr, eps, L, stochastic, 1)
         if exact:
-            return lambda: table_batched_embeddings.backward_exact_adagrad(
+            return lambda: EXT.backward_exact_adagrad(
                 go, w, cc.table_offsets, indices, offsets, None, cc.optimizer_state, lr, eps, stochastic, 1)
-        return lambda: table_batched_embeddings.backward_approx_adagrad(
+        return lambda: EXT.backward_approx_adagrad(
             go, w, cc.table_offsets, indices, offsets, None, cc.optimizer_state, lr, eps, L, stochastic, 1)
 
     for exact in (0, 1):
@@ -150,10 +154,16 @@ def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
 @click.option("--kernels", is_flag=True, default=False, help="Log per-kernel times of every op")
 @click.option("--alpha", default=0.0, help="Zipf exponent of the indices (0 = uniform)")
 @click.option("--seed", default=42)
+@click.option("--compiled", is_flag=True, default=False,
+              help="Call the kernels through the pybind11 module (table_batched_embeddings_cpp)")
 def cli(num_tables, num_embeddings, embedding_dim, batch_size, bag_size, iters, remote, fp16, managed, mixed, kernels,
-        alpha, seed):
-    global KERNEL_TIMES
+        alpha, seed, compiled):
+    global KERNEL_TIMES, EXT
     KERNEL_TIMES = kernels
+    if compiled:
+        import table_batched_embeddings_cpp
+        EXT = table_batched_embeddings_cpp
+        ops.use_extension(EXT)
     logging.basicConfig(level=logging.INFO, stream=sys.stderr)
     if remote:
         raise click.UsageError("--remote (cluster submission) is not available; run the benchmark locally")
