@@ -83,9 +83,12 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 // Tile size in sorted positions: 32 per lane group, so narrow rows (many groups per wavefront)
 // get larger tiles and the per-tile bookkeeping is amortised over the same number of rows.
 // (at most 256 positions; 64 for the variant whose row width is only known at run time)
-constexpr int tile_positions(int chunks_template) {
-  if (chunks_template == 0) return 64;
-  const int positions = 32 * (kWave / chunks_template);
+// Small batches (fewer than kSmallBatchTiles such tiles: not enough wavefronts to fill the chip)
+// take tiles a quarter that size.
+constexpr int kSmallBatchTiles = 4096;
+constexpr int tile_positions(int chunks_template, bool small = false) {
+  if (chunks_template == 0) return small ? 16 : 64;
+  const int positions = (small ? 8 : 32) * (kWave / chunks_template);
   return positions > 256 ? 256 : positions;
 }
 
@@ -108,7 +111,7 @@ struct LongRecord {    // 16 bytes: a segment cut into several chunks
 // APPROX_SUM (with APPROX, rows without per-sample weights in fp32 / fp64): longer segments take the
 // chunk queue like the exact update's, for update_chunks_kernel's per-lookup form.
 template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL, bool APPROX = false,
-          bool APPROX_SUM = false>
+          bool APPROX_SUM = false, bool SMALL = false>
 __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
@@ -125,7 +128,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
   using R = typename V::R;
   static_assert(!APPROX || OPT == kOptAdagrad, "the approximate update is a row-wise Adagrad");
 
-  constexpr int kTilePositions = tile_positions(CHUNKS);
+  constexpr int kTilePositions = tile_positions(CHUNKS, SMALL);
   constexpr int kStageCap = kTilePositions + kShortSegment;  // occurrences staged in LDS per wavefront
   __shared__ int32_t s_bounds[kWavesPerBlock][kTilePositions + 1];
   __shared__ int32_t s_keys[kWavesPerBlock][kTilePositions];
@@ -793,15 +796,20 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   const int groups = kWave / g.chunks;
   const dim3 block(kBlockThreads);
 
-  const int64_t num_tiles = ceil_div(a.num_indices, tile_positions(CHUNKS));
+  const bool small = ceil_div(a.num_indices, tile_positions(CHUNKS)) < kSmallBatchTiles;
+  const int64_t num_tiles = ceil_div(a.num_indices, tile_positions(CHUNKS, small));
   const int64_t tiles_per_xcd = ceil_div(ceil_div(num_tiles, kWavesPerBlock), kNumXcd);
   const dim3 grid_short(static_cast<unsigned>(tiles_per_xcd * kNumXcd));
-  TBE_LAUNCH("update_short", stream,
-             (update_short_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kShortUnroll>), grid_short, block,
-             go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,
-             a.segment_starts, a.segment_ids, a.counters, long_records, chunk_records, a.max_chunks,
-             a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,
-             a.unique_slots, cr, a.stochastic_rounding, static_cast<int32_t *>(nullptr));
+#define TBE_UPDATE_SHORT(SMALL)                                                                             \
+  TBE_LAUNCH("update_short", stream,                                                                        \
+             (update_short_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kShortUnroll, false, false, SMALL>),       \
+             grid_short, block, go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,       \
+             a.segment_starts, a.segment_ids, a.counters, long_records, chunk_records, a.max_chunks,        \
+             a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,                \
+             a.unique_slots, cr, a.stochastic_rounding, static_cast<int32_t *>(nullptr))
+  if (small) { TBE_UPDATE_SHORT(true); }
+  else { TBE_UPDATE_SHORT(false); }
+#undef TBE_UPDATE_SHORT
 
   const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
   // a multiple of the XCD count, so that every XCD gets as many workgroups
