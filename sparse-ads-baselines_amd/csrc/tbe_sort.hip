@@ -38,7 +38,7 @@ constexpr int kWaveTile = kWave * kItems;         // 1024 pairs per wavefront
 // Per-table scan: tables of at most this many tiles are scanned inside the scatter kernel (every
 // workgroup adds up the counts of the earlier tiles of its table itself); a batch with a larger
 // table runs radix_table_scan_kernel first.  tile_prefix[T + 1] holds the choice (1 = inside).
-constexpr int kInlineScanTiles = 48;
+constexpr int kInlineScanTiles = 64;
 
 constexpr int kSegItems = 8;
 constexpr int kSegTile = kBlockThreads * kSegItems;  // 2048
@@ -741,6 +741,7 @@ SortScratch sort_scratch(int64_t n, int32_t num_tables) {
 }
 
 struct RadixPass {
+  bool tables_small;  // known on the host: no table can have more than kInlineScanTiles tiles
   const uint32_t *src_k, *src_v;
   uint32_t *dst_k, *dst_v;
   const uint32_t *table_starts, *tile_prefix;
@@ -758,8 +759,11 @@ void launch_radix_pass(const RadixPass &p, hipStream_t stream) {
   if (p.totals) {
     TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, true>), tiles, block, p.src_k,
                p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, p.totals);
-    TBE_LAUNCH("radix_table_scan", stream, radix_table_scan_kernel<BITS>, dim3(p.num_tables), block, p.counts,
-               p.totals, p.table_starts, p.tile_prefix, p.max_tiles);
+    // (the scatter kernel scans small tables itself, and this kernel returns at once when all
+    // are small; a batch of so few pairs that they must be does not launch it)
+    if (!p.tables_small)
+      TBE_LAUNCH("radix_table_scan", stream, radix_table_scan_kernel<BITS>, dim3(p.num_tables), block, p.counts,
+                 p.totals, p.table_starts, p.tile_prefix, p.max_tiles);
     TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, true>), tiles, block, p.src_k, p.src_v,
                p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
                p.counts, p.totals, p.key_bias);
@@ -794,6 +798,7 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   uint32_t *tmp_vals = reinterpret_cast<uint32_t *>(ws + scratch.tmp_vals);
 
   RadixPass p;
+  p.tables_small = ceil_div(n, kTile) <= kInlineScanTiles;
   p.table_starts = reinterpret_cast<uint32_t *>(ws + scratch.table_starts);
   p.tile_prefix = reinterpret_cast<uint32_t *>(ws + scratch.tile_prefix);
   p.num_tables = num_tables;
