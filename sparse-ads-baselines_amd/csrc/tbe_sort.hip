@@ -33,12 +33,20 @@ constexpr int kMaxRadixBits = 10;                 // widest digit of a pass
 constexpr int kMaxBins = 1 << kMaxRadixBits;
 constexpr int kItems = 16;                        // pairs per thread per tile
 constexpr int kTile = kBlockThreads * kItems;     // 4096
-constexpr int kWaveTile = kWave * kItems;         // 1024 pairs per wavefront
+// Small inputs are sorted in tiles of a quarter that size: at 4096 pairs per workgroup they would
+// leave most compute units without work, and what they move fits in L2, where the shorter runs
+// of the scatter cost nothing.
+constexpr int kSmallItems = 4;
+constexpr int64_t kSmallSortPairs = 1 << 19;      // up to this many pairs: kSmallItems per thread
+inline int sort_items(int64_t n) { return n <= kSmallSortPairs ? kSmallItems : kItems; }
 
 // Per-table scan: tables of at most this many tiles are scanned inside the scatter kernel (every
 // workgroup adds up the counts of the earlier tiles of its table itself); a batch with a larger
 // table runs radix_table_scan_kernel first.  tile_prefix[T + 1] holds the choice (1 = inside).
 constexpr int kInlineScanTiles = 64;
+// (quarter-size tiles: as many pairs per table, so that no batch of theirs of up to 2^18 pairs
+// launches the scan kernel)
+constexpr int inline_scan_tiles(int items) { return kInlineScanTiles * (kItems / items); }
 
 constexpr int kSegItems = 8;
 constexpr int kSegTile = kBlockThreads * kSegItems;  // 2048
@@ -134,6 +142,7 @@ constexpr int kScanChunk = kBlockThreads * kScanItems;  // 2048 count entries pe
 // per-table digit totals of every pass (`totals_words` words; none with the linear scan).
 // device_count (nullable): the number of pairs to sort when only the device knows it (at most n,
 // for which the launches are sized: tiles past the count find nothing to do).
+template <int ITEMS>
 __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
     const int32_t *__restrict__ offsets, int B, int num_tables, uint32_t n,
     uint32_t *__restrict__ table_starts, uint32_t *__restrict__ tile_prefix,
@@ -158,7 +167,7 @@ __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
           end = min(static_cast<uint32_t>(max(offsets[static_cast<int64_t>(t + 1) * B], 0)), n);
       }
       end = max(end, start);
-      tiles = (end - start + kTile - 1) / kTile;
+      tiles = (end - start + kBlockThreads * ITEMS - 1) / (kBlockThreads * ITEMS);
       table_starts[t] = start;
     }
     uint32_t total;
@@ -176,7 +185,7 @@ __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
     for (int w = 1; w < kWavesPerBlock; ++w) most = max(most, s_wave[w]);
     table_starts[num_tables] = n;
     tile_prefix[num_tables] = carry;
-    tile_prefix[num_tables + 1] = most <= kInlineScanTiles ? 1u : 0u;
+    tile_prefix[num_tables + 1] = most <= inline_scan_tiles(ITEMS) ? 1u : 0u;
   }
 }
 
@@ -190,7 +199,7 @@ struct TileInfo {
   int64_t tile_index;  // number of the tile among all tiles
 };
 
-template <int BITS>
+template <int BITS, int ITEMS>
 __device__ __forceinline__ TileInfo locate_tile(const uint32_t *__restrict__ table_starts,
                                                 const uint32_t *__restrict__ tile_prefix,
                                                 int num_tables, int max_tiles) {
@@ -207,9 +216,9 @@ __device__ __forceinline__ TileInfo locate_tile(const uint32_t *__restrict__ tab
   if (first_tile + tiles > static_cast<uint32_t>(max_tiles)) return info;  // inconsistent offsets
   const uint32_t j = tile - first_tile;
   info.table = lo;
-  info.begin = static_cast<int64_t>(table_starts[lo]) + static_cast<int64_t>(j) * kTile;
+  info.begin = static_cast<int64_t>(table_starts[lo]) + static_cast<int64_t>(j) * (kBlockThreads * ITEMS);
   const int64_t left = static_cast<int64_t>(table_starts[lo + 1]) - info.begin;
-  info.count = static_cast<int>(max(int64_t{0}, min(left, static_cast<int64_t>(kTile))));
+  info.count = static_cast<int>(max(int64_t{0}, min(left, static_cast<int64_t>(kBlockThreads * ITEMS))));
   info.count_base = (static_cast<int64_t>(first_tile) << BITS) + j;
   info.table_tiles = static_cast<int>(tiles);
   info.tile_index = static_cast<int64_t>(tile);
@@ -227,14 +236,14 @@ __device__ __forceinline__ int64_t count_index(const TileInfo &tile, int d) {
 
 // BITS = digit width of the pass (8, 9 or 10): 2^BITS bins, each thread owns 2^BITS / 256
 // consecutive digits in the per-digit steps.
-template <int BITS, bool LOCAL>
+template <int BITS, bool LOCAL, int ITEMS>
 __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     const uint32_t *__restrict__ keys, const uint32_t *__restrict__ table_starts,
     const uint32_t *__restrict__ tile_prefix, int num_tables, int max_tiles, int shift,
     uint32_t mask, uint32_t *__restrict__ counts, uint32_t *__restrict__ totals) {
   constexpr int kBinsT = 1 << BITS;
   __shared__ uint32_t s_hist[kBinsT];
-  const TileInfo tile = locate_tile<BITS>(table_starts, tile_prefix, num_tables, max_tiles);
+  const TileInfo tile = locate_tile<BITS, ITEMS>(table_starts, tile_prefix, num_tables, max_tiles);
   if (tile.table_tiles == 0) return;
   const int tid = threadIdx.x;
 #pragma unroll
@@ -243,12 +252,12 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
   // every thread loads all its keys first (an index past the tile's end is clamped, the key
   // dropped): straight-line loads are issued back to back, predicated ones one at a time
   if (tile.count > 0) {
-    uint32_t key[kItems];
+    uint32_t key[ITEMS];
 #pragma unroll
-    for (int k = 0; k < kItems; ++k)
+    for (int k = 0; k < ITEMS; ++k)
       key[k] = keys[tile.begin + min(k * kBlockThreads + tid, tile.count - 1)];
 #pragma unroll
-    for (int k = 0; k < kItems; ++k) {
+    for (int k = 0; k < ITEMS; ++k) {
       if (k * kBlockThreads + tid < tile.count) atomicAdd(&s_hist[(key[k] >> shift) & mask], 1u);
     }
   }
@@ -387,7 +396,7 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
 
 // key_bias (nullable): added to the keys of table t as they are written (the last pass turns
 // rows inside a table into rows of the concatenated tables).
-template <int BITS, bool LOCAL>
+template <int BITS, bool LOCAL, int ITEMS>
 __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ values_in,
     uint32_t *__restrict__ keys_out, uint32_t *__restrict__ values_out,
@@ -399,18 +408,19 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   // The per-wavefront digit counters are only needed until every key knows its slot in the
   // reordered tile.  For 10-bit digits (16 KB of counters) they share LDS with the reordered
   // keys, which keeps four workgroups on a compute unit at the price of one more barrier.
-  constexpr bool kShareCounters = BITS >= 10;
-  __shared__ uint32_t s_keys[kTile];
-  __shared__ uint32_t s_vals[kTile];
+  constexpr int kTileT = kBlockThreads * ITEMS;
+  constexpr int kWaveTileT = kWave * ITEMS;
+  constexpr bool kShareCounters = BITS >= 10 && kWavesPerBlock * kBinsT <= kTileT;
+  __shared__ uint32_t s_keys[kTileT];
+  __shared__ uint32_t s_vals[kTileT];
   __shared__ uint32_t s_own_count[kShareCounters ? 1 : kWavesPerBlock][kShareCounters ? 1 : kBinsT];
   __shared__ uint32_t s_bin_start[kBinsT];
   __shared__ uint32_t s_dest[kBinsT];
   __shared__ uint32_t s_scan[kWavesPerBlock];
-  static_assert(kWavesPerBlock * kBinsT <= kTile, "digit counters must fit the key buffer");
   uint32_t(*s_wave_count)[kBinsT] =
       kShareCounters ? reinterpret_cast<uint32_t(*)[kBinsT]>(s_keys) : reinterpret_cast<uint32_t(*)[kBinsT]>(s_own_count);
 
-  const TileInfo tile = locate_tile<BITS>(table_starts, tile_prefix, num_tables, max_tiles);
+  const TileInfo tile = locate_tile<BITS, ITEMS>(table_starts, tile_prefix, num_tables, max_tiles);
   if (tile.table_tiles == 0 || tile.count == 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -456,22 +466,22 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
 #pragma unroll
     for (int d = tid; d < kBinsT; d += kBlockThreads) s_wave_count[w][d] = 0;
 
-  uint32_t key[kItems], val[kItems];
-  const int wave_first = wave * kWaveTile;
+  uint32_t key[ITEMS], val[ITEMS];
+  const int wave_first = wave * kWaveTileT;
   // straight-line loads (an index past the tile's end is clamped, what it loads replaced)
 #pragma unroll
-  for (int k = 0; k < kItems; ++k)
+  for (int k = 0; k < ITEMS; ++k)
     key[k] = keys_in[tile.begin + min(wave_first + k * kWave + lane, tile.count - 1)];
   if (values_in) {
 #pragma unroll
-    for (int k = 0; k < kItems; ++k)
+    for (int k = 0; k < ITEMS; ++k)
       val[k] = values_in[tile.begin + min(wave_first + k * kWave + lane, tile.count - 1)];
   } else {
 #pragma unroll
-    for (int k = 0; k < kItems; ++k) val[k] = static_cast<uint32_t>(tile.begin + wave_first + k * kWave + lane);
+    for (int k = 0; k < ITEMS; ++k) val[k] = static_cast<uint32_t>(tile.begin + wave_first + k * kWave + lane);
   }
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
+  for (int k = 0; k < ITEMS; ++k) {
     const bool valid = wave_first + k * kWave + lane < tile.count;
     key[k] = valid ? key[k] : 0xffffffffu;
     val[k] = valid ? val[k] : 0u;
@@ -479,9 +489,9 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   __syncthreads();
 
   // Rank of each key among the keys of its wavefront that share its digit.
-  uint32_t rank[kItems];
+  uint32_t rank[ITEMS];
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
+  for (int k = 0; k < ITEMS; ++k) {
     const bool valid = (wave_first + k * kWave + lane) < tile.count;
     const uint32_t digit = (key[k] >> shift) & mask;
     unsigned long long peers = __ballot(valid);
@@ -548,14 +558,14 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
 
   // slot of every key in the reordered tile; the counters are dead after this
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
+  for (int k = 0; k < ITEMS; ++k) {
     const uint32_t digit = (key[k] >> shift) & mask;
     const bool valid = (wave_first + k * kWave + lane) < tile.count;
     rank[k] += valid ? s_bin_start[digit] + s_wave_count[wave][digit] : 0u;
   }
   if constexpr (kShareCounters) __syncthreads();
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
+  for (int k = 0; k < ITEMS; ++k) {
     const bool valid = (wave_first + k * kWave + lane) < tile.count;
     if (valid) {
       s_keys[rank[k]] = key[k];
@@ -566,7 +576,7 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
 
   const uint32_t bias = key_bias ? static_cast<uint32_t>(key_bias[tile.table]) : 0u;
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
+  for (int k = 0; k < ITEMS; ++k) {
     const int local = k * kBlockThreads + tid;
     if (local < tile.count) {
       const uint32_t kk = s_keys[local];
@@ -717,14 +727,15 @@ constexpr int kMaxPasses = 4;  // 32 key bits in digits of at least 8
 // The per-table scan walks a table's tiles one after the other in one workgroup: it is used when
 // the tables have few tiles each on average (the batch's lookups are spread over many tables).
 inline bool use_table_scan(int64_t n, int32_t num_tables, bool have_tables) {
-  return have_tables && num_tables >= 8 && ceil_div(n, kTile) <= static_cast<int64_t>(num_tables) * 128;
+  return have_tables && num_tables >= 8 &&
+         ceil_div(n, kBlockThreads * sort_items(n)) <= static_cast<int64_t>(num_tables) * 128 * (kItems / sort_items(n));
 }
 
 SortScratch sort_scratch(int64_t n, int32_t num_tables) {
   SortScratch s;
   const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
   const uint64_t tables = static_cast<uint64_t>(num_tables > 0 ? num_tables : 1);
-  s.max_tiles = static_cast<int>(ceil_div(nn, kTile) + tables);
+  s.max_tiles = static_cast<int>(ceil_div(nn, kBlockThreads * sort_items(n)) + tables);
   s.scan_blocks = static_cast<int>(ceil_div(static_cast<uint64_t>(s.max_tiles) * kMaxBins, kScanChunk));
   uint64_t off = 0;
   s.tmp_keys = off; off += align_up(nn * 4, 256);
@@ -752,31 +763,31 @@ struct RadixPass {
   const int32_t *key_bias;
 };
 
-template <int BITS>
+template <int BITS, int ITEMS>
 void launch_radix_pass(const RadixPass &p, hipStream_t stream) {
   const dim3 block(kBlockThreads);
   const dim3 tiles(p.max_tiles);
   if (p.totals) {
-    TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, true>), tiles, block, p.src_k,
+    TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, true, ITEMS>), tiles, block, p.src_k,
                p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, p.totals);
     // (the scatter kernel scans small tables itself, and this kernel returns at once when all
     // are small; a batch of so few pairs that they must be does not launch it)
     if (!p.tables_small)
       TBE_LAUNCH("radix_table_scan", stream, radix_table_scan_kernel<BITS>, dim3(p.num_tables), block, p.counts,
                  p.totals, p.table_starts, p.tile_prefix, p.max_tiles);
-    TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, true>), tiles, block, p.src_k, p.src_v,
+    TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, true, ITEMS>), tiles, block, p.src_k, p.src_v,
                p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
                p.counts, p.totals, p.key_bias);
     return;
   }
   const dim3 scan_blocks(static_cast<unsigned>(ceil_div(static_cast<int64_t>(p.max_tiles) << BITS, kScanChunk)));
-  TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, false>), tiles, block, p.src_k,
+  TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, false, ITEMS>), tiles, block, p.src_k,
              p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, nullptr);
   TBE_LAUNCH("radix_scan_reduce", stream, radix_scan_reduce_kernel, scan_blocks, block, p.counts,
              p.tile_prefix, p.num_tables, BITS, p.block_sums);
   TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, scan_blocks, block, p.counts, p.tile_prefix,
              p.num_tables, BITS, p.block_sums);
-  TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, false>), tiles, block, p.src_k, p.src_v,
+  TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, false, ITEMS>), tiles, block, p.src_k, p.src_v,
              p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
              p.counts, nullptr, p.key_bias);
 }
@@ -798,7 +809,8 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   uint32_t *tmp_vals = reinterpret_cast<uint32_t *>(ws + scratch.tmp_vals);
 
   RadixPass p;
-  p.tables_small = ceil_div(n, kTile) <= kInlineScanTiles;
+  const int items = sort_items(n);
+  p.tables_small = ceil_div(n, kBlockThreads * items) <= inline_scan_tiles(items);
   p.table_starts = reinterpret_cast<uint32_t *>(ws + scratch.table_starts);
   p.tile_prefix = reinterpret_cast<uint32_t *>(ws + scratch.tile_prefix);
   p.num_tables = num_tables;
@@ -809,10 +821,14 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   uint32_t *totals = reinterpret_cast<uint32_t *>(ws + scratch.totals);
   const int64_t totals_words = table_scan ? static_cast<int64_t>(num_tables) * kMaxBins * passes : 0;
   const unsigned setup_blocks = static_cast<unsigned>(1 + std::min<int64_t>(ceil_div(totals_words, kBlockThreads * 4), 255));
-  TBE_LAUNCH("sort_setup", stream, sort_setup_kernel, dim3(setup_blocks), dim3(kBlockThreads),
-             tables ? tables->offsets : nullptr, tables ? tables->bags_per_table : 0, num_tables,
-             static_cast<uint32_t>(n), const_cast<uint32_t *>(p.table_starts),
-             const_cast<uint32_t *>(p.tile_prefix), totals, totals_words, device_count);
+#define TBE_SORT_SETUP(ITEMS)                                                                          \
+  TBE_LAUNCH("sort_setup", stream, sort_setup_kernel<ITEMS>, dim3(setup_blocks), dim3(kBlockThreads),  \
+             tables ? tables->offsets : nullptr, tables ? tables->bags_per_table : 0, num_tables,      \
+             static_cast<uint32_t>(n), const_cast<uint32_t *>(p.table_starts),                         \
+             const_cast<uint32_t *>(p.tile_prefix), totals, totals_words, device_count)
+  if (items == kSmallItems) { TBE_SORT_SETUP(kSmallItems); }
+  else { TBE_SORT_SETUP(kItems); }
+#undef TBE_SORT_SETUP
 
   p.src_k = reinterpret_cast<const uint32_t *>(keys_in);
   p.src_v = reinterpret_cast<const uint32_t *>(values_in);
@@ -826,12 +842,15 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
     p.dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
     p.key_bias = (tables && pass == passes - 1) ? tables->key_bias : nullptr;
     p.totals = table_scan ? totals + static_cast<int64_t>(pass) * num_tables * kMaxBins : nullptr;
-    if (bits <= 8)
-      launch_radix_pass<8>(p, stream);
-    else if (bits == 9)
-      launch_radix_pass<9>(p, stream);
-    else
-      launch_radix_pass<10>(p, stream);
+    if (items == kSmallItems) {
+      if (bits <= 8) launch_radix_pass<8, kSmallItems>(p, stream);
+      else if (bits == 9) launch_radix_pass<9, kSmallItems>(p, stream);
+      else launch_radix_pass<10, kSmallItems>(p, stream);
+    } else {
+      if (bits <= 8) launch_radix_pass<8, kItems>(p, stream);
+      else if (bits == 9) launch_radix_pass<9, kItems>(p, stream);
+      else launch_radix_pass<10, kItems>(p, stream);
+    }
     p.src_k = p.dst_k;
     p.src_v = p.dst_v;
     p.shift += bits;

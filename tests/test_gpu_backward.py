@@ -38,7 +38,11 @@ def _vp(t):
                                           (4096, 1 << 16, 16), (4097, 1 << 23, 23), (100000, 7, 3),
                                           (250001, 1 << 25, 25), (70000, 1 << 30, 31), (5000, 1000, 0),
                                           (33333, 1 << 17, 17), (50001, 1 << 19, 19), (81920, 1 << 20, 20),
-                                          (120000, 1 << 27, 27), (60000, 1 << 29, 29), (9000, 1 << 10, 10)])
+                                          (120000, 1 << 27, 27), (60000, 1 << 29, 29), (9000, 1 << 10, 10),
+                                          # either side of the switch from quarter-size to full-size tiles
+                                          (524288, 1 << 18, 18), (524289, 1 << 18, 18), (1200000, 1 << 28, 28),
+                                          (700000, 1 << 30, 31), (900000, 1 << 20, 20), (1023, 1 << 9, 9),
+                                          (1025, 1 << 20, 20)])
 def test_sort_pairs_is_stable_and_bit_exact(oracle, n, hi, end_bit):
     rs = np.random.RandomState(n % 97)
     keys = rs.randint(0, hi, size=n).astype(np.int32)
@@ -133,7 +137,8 @@ def _plan_views(p, max_table_rows):
 
 @pytest.mark.parametrize("case", ["ragged_rows", "empty_tables", "many_small_tables", "multi_tile_tables", "one_table",
                                   "eight_tables_of_thirty_tiles", "one_large_table_among_nine",
-                                  "ten_bit_digits"])
+                                  "ten_bit_digits", "eight_tables_of_forty_small_tiles",
+                                  "one_larger_table_among_nine", "ten_bit_digits_full_tiles"])
 def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
     """The plan sorts every table's indices on their own (fewer key bits); keys_sorted,
     positions_sorted and segment_starts must equal the stable sort of table_offsets[t] + index
@@ -156,19 +161,25 @@ def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
         # scatter kernel
         p = make_problem(16, T=8, E=0, D=4, B=3000, L=40, dtype=np.float32, ragged=False, zipf=1.1,
                          rows=[70000, 300, 1 << 17, 5, 90000, 1000, 131071, 2])
-    elif case == "one_large_table_among_nine":
-        # one table of 63 tiles among small ones: the scan kernel with a workgroup per table runs
+    elif case == "eight_tables_of_forty_small_tiles":
+        # the same through the quarter-size tiles of a batch of at most 2^19 lookups
+        p = make_problem(19, T=8, E=0, D=4, B=1000, L=40, dtype=np.float32, ragged=False, zipf=1.1,
+                         rows=[70000, 300, 1 << 17, 5, 90000, 1000, 131071, 2])
+    elif case in ("one_large_table_among_nine", "one_larger_table_among_nine"):
+        # one table of more tiles than the scatter kernel scans itself, among small ones: the scan
+        # kernel with a workgroup per table runs (quarter-size tiles; full-size tiles for the larger)
         rs = np.random.RandomState(17)
         T, B = 9, 3200
         rows = [4000, 100, 50000, 1 << 17, 7, 900, 30000, 12, 65536]
         lengths = np.full((T, B), 2)
-        lengths[3] = 80
+        lengths[3] = 80 if case == "one_large_table_among_nine" else 200
         offsets = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
         indices = np.concatenate([rs.zipf(1.2, size=int(lengths[t].sum())) % rows[t] for t in range(T)])
         p = dict(T=T, B=B, rows=rows, n=int(offsets[-1]), offsets=offsets, indices=indices.astype(np.int32),
                  table_offsets=np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
-    elif case == "ten_bit_digits":
-        p = make_problem(18, T=8, E=0, D=4, B=2000, L=30, dtype=np.float32, zipf=1.05,
+    elif case in ("ten_bit_digits", "ten_bit_digits_full_tiles"):
+        p = make_problem(18, T=8, E=0, D=4, B=2000 if case == "ten_bit_digits" else 4000, L=30, dtype=np.float32,
+                         zipf=1.05,
                          rows=[1 << 20, 1000000, 999999, 1 << 19, 3, 1 << 20, 70, 524289])
     elif case == "multi_tile_tables":
         p = make_problem(14, T=3, E=0, D=4, B=1500, L=12, dtype=np.float32, zipf=1.1, rows=[1 << 17, 100, 300000])
