@@ -713,7 +713,7 @@ inline int num_seg_tiles(int64_t n) { return static_cast<int>(ceil_div(n, kSegTi
 }  // namespace
 
 // Sort workspace: [tmp keys n][tmp values n][counts 1024 * max_tiles][workgroup sums of the count
-// scan][table_starts T+1][tile_prefix T+2][digit totals 4 * 1024 * T]; max_tiles = ceil(n / 4096) + T.
+// scan][table_starts T+1][tile_prefix T+2][digit totals 4 * 1024 * T]; max_tiles = ceil(n / tile) + T.
 namespace {
 struct SortScratch {
   uint64_t tmp_keys, tmp_vals, counts, block_sums, table_starts, tile_prefix, totals, total;
@@ -736,11 +736,16 @@ SortScratch sort_scratch(int64_t n, int32_t num_tables) {
   const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
   const uint64_t tables = static_cast<uint64_t>(num_tables > 0 ? num_tables : 1);
   s.max_tiles = static_cast<int>(ceil_div(nn, kBlockThreads * sort_items(n)) + tables);
-  s.scan_blocks = static_cast<int>(ceil_div(static_cast<uint64_t>(s.max_tiles) * kMaxBins, kScanChunk));
+  // The counters are sized so that a workspace for n pairs also serves every smaller n: just above
+  // kSmallSortPairs the full-size tiles are fewer than the quarter-size tiles of kSmallSortPairs.
+  uint64_t sized_tiles = static_cast<uint64_t>(s.max_tiles);
+  if (n > kSmallSortPairs)
+    sized_tiles = std::max<uint64_t>(sized_tiles, ceil_div(kSmallSortPairs, kBlockThreads * kSmallItems) + tables);
+  s.scan_blocks = static_cast<int>(ceil_div(sized_tiles * kMaxBins, kScanChunk));
   uint64_t off = 0;
   s.tmp_keys = off; off += align_up(nn * 4, 256);
   s.tmp_vals = off; off += align_up(nn * 4, 256);
-  s.counts = off; off += align_up(static_cast<uint64_t>(s.max_tiles) * kMaxBins * 4, 256);
+  s.counts = off; off += align_up(sized_tiles * kMaxBins * 4, 256);
   s.block_sums = off; off += align_up(static_cast<uint64_t>(s.scan_blocks) * 4, 256);
   s.table_starts = off; off += align_up((tables + 1) * 4, 256);
   s.tile_prefix = off; off += align_up((tables + 2) * 4, 256);

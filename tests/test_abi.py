@@ -102,6 +102,13 @@ def test_sort_and_segment_workspace_queries():
     small, big = lib.tbe_sort_workspace_bytes(1000), lib.tbe_sort_workspace_bytes(5242880)
     assert big > small >= 2 * 1000 * 4
     assert lib.tbe_segments_workspace_bytes(5242880) >= 5242880 // 2048 * 4
+    # a workspace sized for a maximum serves every smaller batch, also across the switch of tile sizes
+    sizes = [lib.tbe_sort_workspace_bytes(n) for n in (1, 1000, 262144, 524287, 524288, 524289, 600000, 700000,
+                                                       1 << 20, 5242880)]
+    assert sizes == sorted(sizes)
+    layouts = [tbe_native.backward_workspace_layout(n, 128, tbe_native.DTYPE_F32, 64).total_bytes
+               for n in (1000, 524288, 524289, 600000, 1 << 20)]
+    assert layouts == sorted(layouts)
     assert lib.tbe_sort_pairs(_fake(), _null(), _fake(), _fake(), 10, 40, _fake(), 1 << 20, _null()) == 1
     assert lib.tbe_sort_pairs(_fake(), _null(), _fake(), _fake(), 10, 8, _fake(), 8, _null()) == 2
 

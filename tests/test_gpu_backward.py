@@ -81,6 +81,23 @@ def test_sort_pairs_carries_arbitrary_values(oracle):
     np.testing.assert_array_equal(v_out.cpu().numpy(), want_v)
 
 
+def test_sort_pairs_in_a_workspace_sized_for_a_larger_batch(oracle):
+    """One workspace, sized once for the largest batch, serves smaller ones on either tile size."""
+    lib = tbe_native.load()
+    largest = 600000
+    ws = torch.empty(lib.tbe_sort_workspace_bytes(largest), dtype=torch.uint8, device=DEV)
+    for n in (largest, 524288, 300000, 77):
+        keys = np.random.RandomState(n % 101).randint(0, 1 << 21, size=n).astype(np.int32)
+        k_in = dev(keys)
+        k_out, v_out = (torch.full((n,), -1, dtype=torch.int32, device=DEV) for _ in range(2))
+        tbe_native.check(lib.tbe_sort_pairs(_vp(k_in), _vp(None), _vp(k_out), _vp(v_out), n, 21, _vp(ws),
+                                            ws.numel(), _stream()))
+        _sync()
+        want_k, want_v = oracle.sort_pairs(keys, None, 21)
+        np.testing.assert_array_equal(k_out.cpu().numpy(), want_k)
+        np.testing.assert_array_equal(v_out.cpu().numpy(), want_v)
+
+
 @pytest.mark.parametrize("n,hi", [(0, 5), (1, 5), (2047, 3), (2048, 100000), (2049, 1), (300000, 120000),
                                   (8388608, 2000000), (8400000, 3000000)])  # 4096 tiles, and one tile count beyond
 def test_find_segments_bit_exact(oracle, n, hi):
