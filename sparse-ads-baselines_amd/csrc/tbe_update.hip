@@ -835,34 +835,43 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
 template <typename T, int VEC, int CHUNKS, bool WEIGHTED>
 void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *queue, hipStream_t stream) {
   using A = typename AccOf<T>::type;
-  const int64_t num_tiles = ceil_div(a.num_indices, tile_positions(CHUNKS));
+  const bool small = ceil_div(a.num_indices, tile_positions(CHUNKS)) < kSmallBatchTiles;
+  const int64_t num_tiles = ceil_div(a.num_indices, tile_positions(CHUNKS, small));
   const int64_t tiles_per_xcd = ceil_div(ceil_div(num_tiles, kWavesPerBlock), kNumXcd);
   const dim3 grid_short(static_cast<unsigned>(tiles_per_xcd * kNumXcd));
   if constexpr (!WEIGHTED && sizeof(T) == sizeof(A)) {
     if (queue == nullptr) {
       // fp32 / fp64 rows without per-sample weights: longer rows go to the chunk queues
-      TBE_LAUNCH("update_approx_short", stream,
-                 (update_short_kernel<T, VEC, CHUNKS, kOptAdagrad, false, kShortUnroll, true, true>), grid_short,
-                 dim3(kBlockThreads), static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),
-                 static_cast<A *>(a.optimizer_state), static_cast<const T *>(nullptr), static_cast<T *>(nullptr),
-                 a.keys_sorted, a.positions_sorted, a.grad_rows, a.segment_starts, a.segment_ids, a.counters,
-                 reinterpret_cast<LongRecord *>(a.long_segments), reinterpret_cast<ChunkRecord *>(a.chunk_segments),
-                 a.max_chunks, a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,
-                 static_cast<const int32_t *>(nullptr), static_cast<T *>(nullptr), a.stochastic_rounding,
-                 static_cast<int32_t *>(nullptr));
+#define TBE_APPROX_SUM_SHORT(SMALL)                                                                             \
+  TBE_LAUNCH("update_approx_short", stream,                                                                     \
+             (update_short_kernel<T, VEC, CHUNKS, kOptAdagrad, false, kShortUnroll, true, true, SMALL>),        \
+             grid_short, dim3(kBlockThreads), static_cast<const T *>(a.grad_output),                            \
+             static_cast<T *>(a.weights), static_cast<A *>(a.optimizer_state), static_cast<const T *>(nullptr), \
+             static_cast<T *>(nullptr), a.keys_sorted, a.positions_sorted, a.grad_rows, a.segment_starts,       \
+             a.segment_ids, a.counters, reinterpret_cast<LongRecord *>(a.long_segments),                        \
+             reinterpret_cast<ChunkRecord *>(a.chunk_segments), a.max_chunks, a.num_indices, num_tiles,         \
+             tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr),       \
+             static_cast<T *>(nullptr), a.stochastic_rounding, static_cast<int32_t *>(nullptr))
+      if (small) { TBE_APPROX_SUM_SHORT(true); }
+      else { TBE_APPROX_SUM_SHORT(false); }
+#undef TBE_APPROX_SUM_SHORT
       return;
     }
   }
-  TBE_LAUNCH("update_approx_short", stream,
-             (update_short_kernel<T, VEC, CHUNKS, kOptAdagrad, WEIGHTED, kShortUnroll, true>), grid_short,
-             dim3(kBlockThreads), static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),
-             static_cast<A *>(a.optimizer_state), static_cast<const T *>(a.per_sample_weights),
-             static_cast<T *>(a.grad_per_sample_weights), a.keys_sorted, a.positions_sorted, a.grad_rows,
-             a.segment_starts, a.segment_ids, a.counters, static_cast<LongRecord *>(nullptr),
-             static_cast<ChunkRecord *>(nullptr), kNumXcd * approx_long_queue_capacity(a.num_indices),
-             a.num_indices, num_tiles, tiles_per_xcd, a.D,
-             g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr), static_cast<T *>(nullptr),
-             a.stochastic_rounding, queue);
+#define TBE_APPROX_SHORT(SMALL)                                                                                 \
+  TBE_LAUNCH("update_approx_short", stream,                                                                     \
+             (update_short_kernel<T, VEC, CHUNKS, kOptAdagrad, WEIGHTED, kShortUnroll, true, false, SMALL>),    \
+             grid_short, dim3(kBlockThreads), static_cast<const T *>(a.grad_output),                            \
+             static_cast<T *>(a.weights), static_cast<A *>(a.optimizer_state),                                  \
+             static_cast<const T *>(a.per_sample_weights), static_cast<T *>(a.grad_per_sample_weights),         \
+             a.keys_sorted, a.positions_sorted, a.grad_rows, a.segment_starts, a.segment_ids, a.counters,       \
+             static_cast<LongRecord *>(nullptr), static_cast<ChunkRecord *>(nullptr),                           \
+             kNumXcd * approx_long_queue_capacity(a.num_indices), a.num_indices, num_tiles, tiles_per_xcd,      \
+             a.D, g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr),                      \
+             static_cast<T *>(nullptr), a.stochastic_rounding, queue)
+  if (small) { TBE_APPROX_SHORT(true); }
+  else { TBE_APPROX_SHORT(false); }
+#undef TBE_APPROX_SHORT
 }
 
 template <typename T, int VEC, bool WEIGHTED>
