@@ -66,12 +66,10 @@ int build_plan(const tbe_workspace_layout_t &l, void *workspace, const int32_t *
                int64_t total_rows, int64_t max_table_rows, hipStream_t stream) {
   char *ws = static_cast<char *>(workspace);
   int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
-  int rc = linearize(table_offsets, T, indices, offsets, B, nullptr,
-                     reinterpret_cast<int32_t *>(ws + l.grad_rows), stream);
-  if (rc) return rc;
   const int64_t largest = (max_table_rows > 0 && max_table_rows < total_rows) ? max_table_rows : total_rows;
-  const SortTables tables{offsets, B, T, table_offsets};
-  rc = sort_pairs(indices, nullptr, keys_sorted, reinterpret_cast<int32_t *>(ws + l.positions_sorted),
+  // (the gradient row of every position is recorded by the sort's first launch)
+  const SortTables tables{offsets, B, T, table_offsets, reinterpret_cast<int32_t *>(ws + l.grad_rows)};
+  int rc = sort_pairs(indices, nullptr, keys_sorted, reinterpret_cast<int32_t *>(ws + l.positions_sorted),
                   n, key_bits(largest), ws + l.sort_scratch, stream, &tables);
   if (rc) return rc;
   return find_segments(keys_sorted, n, reinterpret_cast<int32_t *>(ws + l.segment_starts),

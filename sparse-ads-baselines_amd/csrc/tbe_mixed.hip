@@ -1011,13 +1011,11 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   hipStream_t s = static_cast<hipStream_t>(stream);
   char *ws = static_cast<char *>(workspace);
   auto i32 = [&](uint64_t off) { return reinterpret_cast<int32_t *>(ws + off); };
-  // gradient row b*T + t of every position (the keys themselves are not needed: see below)
-  int rc = linearize(table_dim_offsets, T, indices, offsets, B, nullptr, i32(l.grad_rows), s);
-  if (rc) return rc;
-  // every table's indices are sorted on their own; the last pass adds the table's first row id
+  // every table's indices are sorted on their own; the last pass adds the table's first row id.
+  // The sort's first launch also records the gradient row b*T + t of every position.
   const int64_t largest = (max_table_rows > 0 && max_table_rows < total_rows) ? max_table_rows : total_rows;
-  const SortTables tables{offsets, B, T, table_dim_offsets};
-  rc = sort_pairs(indices, nullptr, i32(l.keys_sorted), i32(l.positions_sorted), num_indices,
+  const SortTables tables{offsets, B, T, table_dim_offsets, i32(l.grad_rows)};
+  int rc = sort_pairs(indices, nullptr, i32(l.keys_sorted), i32(l.positions_sorted), num_indices,
                   key_bits_for(largest), ws + l.sort_scratch, s, &tables);
   if (rc) return rc;
   rc = find_segments(i32(l.keys_sorted), num_indices, i32(l.segment_starts), i32(l.num_unique), nullptr,

@@ -108,6 +108,21 @@ __global__ __launch_bounds__(kBlockThreads) void linearize_kernel(
   }
 }
 
+// The gradient row b*T + t of every position, 8 lanes per bag, for workgroup `block` of
+// ceil(num_bags * 8 / 256): what linearize_kernel writes when it is given no keys.
+__device__ __forceinline__ void record_gradient_rows(const int32_t *__restrict__ offsets, int B,
+                                                     int num_tables, int num_bags, int64_t block,
+                                                     int32_t *__restrict__ grad_rows) {
+  const int64_t gid = block * kBlockThreads + threadIdx.x;
+  const int64_t bag64 = gid / kLinLanes;
+  if (bag64 >= num_bags) return;
+  const int bag = static_cast<int>(bag64);
+  const int t = bag / B;
+  const int32_t grow = (bag - t * B) * num_tables + t;
+  const int end = offsets[bag + 1];
+  for (int p = offsets[bag] + static_cast<int>(gid % kLinLanes); p < end; p += kLinLanes) grad_rows[p] = grow;
+}
+
 // Row numbers for tables stored interleaved, weights[row][table][D] (the layout of the older
 // sparse_embedding_cuda kernels, sparse_embedding_cuda_kernel.cu:349-379: weights[ind][t][d]).
 // Viewed as a [E*T][D] matrix, row `ind` of table t is matrix row ind*T + t; bags are numbered
@@ -138,20 +153,29 @@ __global__ __launch_bounds__(kBlockThreads) void interleaved_rows_kernel(
 constexpr int kScanItems = 8;
 constexpr int kScanChunk = kBlockThreads * kScanItems;  // 2048 count entries per workgroup
 
-// Workgroup 0 derives the tables' position ranges and tile counts; all workgroups clear the
-// per-table digit totals of every pass (`totals_words` words; none with the linear scan).
+// Workgroup 0 derives the tables' position ranges and tile counts; the first setup_blocks
+// workgroups clear the per-table digit totals of every pass (`totals_words` words; none with the
+// linear scan).  The workgroups after them, if any, record the gradient row of every position
+// (grad_rows non-null, with tables): work of the caller's that depends on nothing here and would
+// otherwise be one more launch in the chain.
 // device_count (nullable): the number of pairs to sort when only the device knows it (at most n,
 // for which the launches are sized: tiles past the count find nothing to do).
 template <int ITEMS>
 __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
     const int32_t *__restrict__ offsets, int B, int num_tables, uint32_t n,
     uint32_t *__restrict__ table_starts, uint32_t *__restrict__ tile_prefix,
-    uint32_t *__restrict__ totals, int64_t totals_words, const int32_t *__restrict__ device_count) {
+    uint32_t *__restrict__ totals, int64_t totals_words, const int32_t *__restrict__ device_count,
+    int setup_blocks, int32_t *__restrict__ grad_rows) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   const int tid = threadIdx.x;
+  if (static_cast<int>(blockIdx.x) >= setup_blocks) {
+    record_gradient_rows(offsets, B, num_tables, num_tables * B, static_cast<int64_t>(blockIdx.x) - setup_blocks,
+                         grad_rows);
+    return;
+  }
   if (device_count) n = min(n, static_cast<uint32_t>(max(*device_count, 0)));
   for (int64_t i = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + tid) * 4; i < totals_words;
-       i += static_cast<int64_t>(gridDim.x) * kBlockThreads * 4)
+       i += static_cast<int64_t>(setup_blocks) * kBlockThreads * 4)
     *reinterpret_cast<uint4 *>(totals + i) = make_uint4(0, 0, 0, 0);
   if (blockIdx.x != 0) return;
   uint32_t carry = 0;
@@ -826,11 +850,17 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   uint32_t *totals = reinterpret_cast<uint32_t *>(ws + scratch.totals);
   const int64_t totals_words = table_scan ? static_cast<int64_t>(num_tables) * kMaxBins * passes : 0;
   const unsigned setup_blocks = static_cast<unsigned>(1 + std::min<int64_t>(ceil_div(totals_words, kBlockThreads * 4), 255));
+  int32_t *grad_rows = tables ? tables->grad_rows : nullptr;
+  const unsigned row_blocks =
+      grad_rows ? static_cast<unsigned>(ceil_div(static_cast<int64_t>(num_tables) * tables->bags_per_table * kLinLanes,
+                                                 kBlockThreads))
+                : 0u;
 #define TBE_SORT_SETUP(ITEMS)                                                                          \
-  TBE_LAUNCH("sort_setup", stream, sort_setup_kernel<ITEMS>, dim3(setup_blocks), dim3(kBlockThreads),  \
-             tables ? tables->offsets : nullptr, tables ? tables->bags_per_table : 0, num_tables,      \
-             static_cast<uint32_t>(n), const_cast<uint32_t *>(p.table_starts),                         \
-             const_cast<uint32_t *>(p.tile_prefix), totals, totals_words, device_count)
+  TBE_LAUNCH("sort_setup", stream, sort_setup_kernel<ITEMS>, dim3(setup_blocks + row_blocks),          \
+             dim3(kBlockThreads), tables ? tables->offsets : nullptr,                                  \
+             tables ? tables->bags_per_table : 0, num_tables, static_cast<uint32_t>(n),                \
+             const_cast<uint32_t *>(p.table_starts), const_cast<uint32_t *>(p.tile_prefix), totals,    \
+             totals_words, device_count, static_cast<int>(setup_blocks), grad_rows)
   if (items == kSmallItems) { TBE_SORT_SETUP(kSmallItems); }
   else { TBE_SORT_SETUP(kItems); }
 #undef TBE_SORT_SETUP

@@ -18,6 +18,9 @@ struct SortTables {
   int32_t bags_per_table;   // B
   int32_t num_tables;       // T
   const int32_t *key_bias;  // [T] first row of every table
+  // nullable, [n] out: the gradient row b*T + t of every position (what linearize() records),
+  // written by the sort's set-up launch instead of a launch of its own
+  int32_t *grad_rows = nullptr;
 };
 
 uint64_t sort_workspace_bytes(int64_t n, int32_t num_tables);
