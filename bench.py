@@ -182,9 +182,10 @@ def algorithmic_bytes(w, U):
     return a_fwd, a_bwd, a_update
 
 
-def cpu_baseline(w, torch, tables=8, iters=3):
+def cpu_baseline(w, torch, tables=8, iters=3, seconds=10.0):
     """The reference's CPU path (per-table torch.nn.EmbeddingBag + Python optimizer) on a bounded
-    sample: the first `tables` tables of the same workload, all host cores."""
+    sample: the first `tables` tables of the same workload, all host cores, about `seconds` of
+    timed steps."""
     from oracle import torch_cpu_path
 
     T = min(tables, w["T"])
@@ -197,17 +198,17 @@ def cpu_baseline(w, torch, tables=8, iters=3):
     torch.set_num_threads(os.cpu_count() or 1)
     cpu = torch_cpu_path.CpuTables(weights, [E] * T, D)
     opt = w["optimizer"] or "sgd"
-    sec = torch_cpu_path.time_steps(cpu, (w["indices"][:hi], w["offsets"][:T * B + 1], B, go, opt, w["lr"],
-                                          w["eps"], psw), warmup=1, iters=iters)
+    sec, iters = torch_cpu_path.time_steps(cpu, (w["indices"][:hi], w["offsets"][:T * B + 1], B, go, opt, w["lr"],
+                                                 w["eps"], psw), warmup=1, iters=iters, seconds=seconds)
     # the same algorithmic bytes as the GPU figure, for the sample's lookups, bags and distinct rows
     keys = w["indices"][:hi].astype(np.int64) + np.repeat(np.arange(T, dtype=np.int64) * E,
                                                           np.diff(w["offsets"][:T * B + 1:B]))
     sample = dict(w, T=T, n=hi)
     a_fwd, a_bwd, _ = algorithmic_bytes(sample, int(np.unique(keys).size))
     return {"value": T * B / sec, "unit": "bags/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "first %d of %d tables of the same workload (%d bags/step), 1 warm-up + %d timed steps, "
+            "sample": "first %d of %d tables of the same workload (%d bags/step), 1 warm-up + %d timed steps (%.0f s), "
                       "per-table torch.nn.EmbeddingBag(sparse=True) forward+backward + Python %s update, fp32"
-                      % (T, w["T"], T * B, iters, opt),
+                      % (T, w["T"], T * B, iters, sec * iters, opt),
             "ms_per_step": sec * 1e3, "GBps": (a_fwd + a_bwd) / sec / 1e9,
             "algorithmic_bytes_per_step": a_fwd + a_bwd}
 

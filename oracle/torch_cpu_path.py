@@ -65,10 +65,19 @@ class CpuTables:
         return torch.stack(outs, dim=1)
 
 
-def time_steps(tables, step_args, warmup=1, iters=3, update="dense"):
+def time_steps(tables, step_args, warmup=1, iters=3, update="dense", seconds=None):
+    """Seconds per step.  With `seconds`, at least `iters` steps and as many more as that much time
+    allows (judged by the first timed steps); returns (seconds per step, steps timed)."""
     for _ in range(warmup):
         tables.step(*step_args, update=update)
     t0 = time.perf_counter()
     for _ in range(iters):
         tables.step(*step_args, update=update)
-    return (time.perf_counter() - t0) / iters
+    done = iters
+    if seconds is not None:
+        more = int((seconds - (time.perf_counter() - t0)) / ((time.perf_counter() - t0) / iters))
+        for _ in range(max(more, 0)):
+            tables.step(*step_args, update=update)
+        done += max(more, 0)
+        return (time.perf_counter() - t0) / done, done
+    return (time.perf_counter() - t0) / done
