@@ -812,9 +812,10 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
 #undef TBE_UPDATE_SHORT
 
   const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
-  // a multiple of the XCD count, so that every XCD gets as many workgroups
+  // a multiple of the XCD count, so that every XCD gets as many workgroups (a small batch, whose
+  // queues are mostly empty room, gets few: starting workgroups that find nothing is its cost)
   const dim3 grid_chunks(static_cast<unsigned>(
-      kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), 1024))));
+      kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), small ? 64 : 1024))));
   TBE_LAUNCH("update_chunks", stream,
              (update_chunks_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, (WEIGHTED && VEC == 8) ? 4 : kLongUnroll>),
              grid_chunks, block,
@@ -960,8 +961,9 @@ void launch_approx_sum_long(const UpdateArgs &a, const RowGeometry &g, const voi
     ChunkRecord *chunk_records = reinterpret_cast<ChunkRecord *>(a.chunk_segments);
     const dim3 block(kBlockThreads);
     const int64_t want_chunks = ceil_div(a.max_chunks, kWavesPerBlock);
+    const bool small = ceil_div(a.num_indices, tile_positions(CHUNKS)) < kSmallBatchTiles;
     const dim3 grid_chunks(static_cast<unsigned>(
-        kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), 1024))));
+        kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), small ? 64 : 1024))));
     TBE_LAUNCH("update_approx_chunks", stream,
                (update_chunks_kernel<T, VEC, CHUNKS, kOptSgd, false, kLongUnroll, true>), grid_chunks, block,
                static_cast<const T *>(a.grad_output), w, st, static_cast<const T *>(lookup_wss),
