@@ -20,6 +20,7 @@
 #include <map>
 #include <mutex>
 #include <iterator>
+#include <utility>
 #include <vector>
 
 #include "tbe_hip.h"
@@ -100,13 +101,15 @@ void check_state(const at::Tensor &optimizer_state, const at::Tensor &weights) {
   TORCH_CHECK(optimizer_state.device() == weights.device(), "optimizer_state must live on the weights' device");
 }
 
-// One grow-only scratch tensor per device (the reference allocates its sort buffers per call,
-// table_batched_embeddings_cuda.cu:1618-1647).
-at::Tensor &workspace(const at::Tensor &like, uint64_t bytes) {
+// One grow-only scratch tensor per (device, stream), so that calls issued on different streams
+// of a device may overlap (the reference allocates its sort buffers per call,
+// table_batched_embeddings_cuda.cu:1618-1647).  Returned by value: the caller's handle keeps the
+// memory until its launches are enqueued, whatever another thread does to the table meanwhile.
+at::Tensor workspace(const at::Tensor &like, uint64_t bytes) {
   static std::mutex mutex;
-  static std::map<int, at::Tensor> held;
+  static std::map<std::pair<int, void *>, at::Tensor> held;
   std::lock_guard<std::mutex> lock(mutex);
-  at::Tensor &ws = held[like.get_device()];
+  at::Tensor &ws = held[{static_cast<int>(like.get_device()), stream_of(like)}];
   if (!ws.defined() || static_cast<uint64_t>(ws.numel()) < bytes)
     ws = at::empty({static_cast<int64_t>(bytes + bytes / 4 + 256)}, like.options().dtype(at::kByte));
   return ws;
@@ -200,7 +203,7 @@ void backward_sgd(at::Tensor grad_output, at::Tensor weights, at::Tensor table_o
   grad_output = check_grad(grad_output, weights, s);
   const int32_t dtype = dtype_code(weights);
   c10::DeviceGuard guard(weights.device());
-  at::Tensor &ws = workspace(weights, workspace_bytes(s, dtype));
+  at::Tensor ws = workspace(weights, workspace_bytes(s, dtype));
   check(tbe_backward_sgd(grad_output.data_ptr(), weights.data_ptr(), dtype, s.rows,
                          max_table_rows(table_offsets, s.rows), s.D, table_offsets.data_ptr<int32_t>(), s.T,
                          indices.data_ptr<int32_t>(), s.n, offsets.data_ptr<int32_t>(), s.B,
@@ -236,7 +239,7 @@ c10::optional<at::Tensor> backward_exact_adagrad(at::Tensor grad_output, at::Ten
   c10::DeviceGuard guard(weights.device());
   c10::optional<at::Tensor> grad_indice_weights;
   if (indice_weights.has_value()) grad_indice_weights = at::empty_like(*indice_weights);
-  at::Tensor &ws = workspace(weights, workspace_bytes(s, dtype));
+  at::Tensor ws = workspace(weights, workspace_bytes(s, dtype));
   void *grad_psw = grad_indice_weights.has_value() ? grad_indice_weights->data_ptr() : nullptr;
   if (stochastic_rounding && weights.scalar_type() == at::kHalf) {
     const auto stream = rounding_stream(weights);
@@ -271,7 +274,7 @@ c10::optional<at::Tensor> backward_approx_adagrad(at::Tensor grad_output, at::Te
   c10::DeviceGuard guard(weights.device());
   c10::optional<at::Tensor> grad_indice_weights;
   if (indice_weights.has_value()) grad_indice_weights = at::empty_like(*indice_weights);
-  at::Tensor &ws = workspace(weights, workspace_bytes(s, dtype));
+  at::Tensor ws = workspace(weights, workspace_bytes(s, dtype));
   const bool rounds = stochastic_rounding && weights.scalar_type() == at::kHalf;
   std::pair<uint64_t, uint64_t> stream{0, 0};
   if (rounds) stream = rounding_stream(weights);
@@ -376,7 +379,7 @@ c10::optional<at::Tensor> backward_mixed(int32_t optimizer, at::Tensor grad_outp
   if (indice_weights.has_value()) grad_indice_weights = at::empty_like(*indice_weights);
   tbe_workspace_layout_t layout;
   check(tbe_backward_workspace_layout(s.n, 4, dtype, s.T, &layout));
-  at::Tensor &ws = workspace(weights, layout.total_bytes);
+  at::Tensor ws = workspace(weights, layout.total_bytes);
   const bool rounds = stochastic_rounding && weights.scalar_type() == at::kHalf;
   std::pair<uint64_t, uint64_t> stream{0, 0};
   if (rounds) stream = rounding_stream(weights);

@@ -19,7 +19,8 @@ _DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F
 # One grow-only scratch buffer per device for the backward pipeline (keys, sort
 # buffers, segment lists).  The reference allocates these per call
 # (table_batched_embeddings_cuda.cu:1618-1647).
-_workspaces = {}
+_workspaces = {}      # (device, stream handle) -> uint8 tensor
+_last_workspace = {}  # device -> the one used last
 # Owners of the host-resident allocations handed out by new_*_tensor (weak), keyed by device address.
 _host_allocations = {}
 
@@ -84,16 +85,20 @@ def _rounding_stream(device):
 
 
 def _workspace(device, nbytes):
-    ws = _workspaces.get(device)
+    """The grow-only scratch buffer of the device's current stream: one per (device, stream), so
+    that calls issued on different streams of a device may overlap."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=device)
-        _workspaces[device] = ws
+        _workspaces[key] = ws
+    _last_workspace[device] = ws
     return ws
 
 
 def backward_workspace(device):
     """The scratch buffer last used by a backward call on `device` (for inspection)."""
-    return _workspaces.get(torch.device(device))
+    return _last_workspace.get(torch.device(device))
 
 
 class BackwardPlan:
@@ -139,7 +144,7 @@ class BackwardPlan:
         stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
         seed, offset = _rounding_stream(self.device) if stochastic else (0, 0)
         torch.cuda.current_stream(self.device).wait_event(self.ready)
-        _workspaces[self.device] = self.workspace  # keep backward_workspace() pointing at the last plan
+        _last_workspace[self.device] = self.workspace  # keep backward_workspace() pointing at the last plan
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_backward_planned(
                 optimizer, _ptr(grad_output), _ptr(weights), self.code, self.total_rows, self.D, self.T, self.B,

@@ -168,3 +168,29 @@ def test_module_over_the_compiled_extension(optimizer, fp16, weighted, managed):
     assert torch.equal(results[0][1], results[1][1])
     if weighted:
         assert torch.equal(results[0][2], results[1][2])
+
+
+@pytest.mark.parametrize("module", [ext, ext_cpp], ids=["python", "cpp"])
+def test_backward_calls_on_two_streams_do_not_share_scratch(module):
+    """Each stream of a device has its own workspace, so two backward calls issued on two streams
+    without any ordering between them give what they give one after the other."""
+    problems = [make_problem(61, T=8, E=5000, D=64, B=512, L=20, dtype=np.float32, zipf=1.1),
+                make_problem(62, T=6, E=3000, D=64, B=700, L=15, dtype=np.float32, zipf=1.3)]
+    args, expect = [], []
+    for p in problems:
+        to, idx, off, go = dev(p["table_offsets"]), dev(p["indices"]), dev(p["offsets"]), dev(p["grad_output"])
+        args.append((go, to, idx, off))
+        w = dev(p["weights"])
+        module.backward_sgd(go, w, to, idx, off, 0.05, 200, 1, False)
+        expect.append(w)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+        weights = [dev(p["weights"]) for p in problems]
+        torch.cuda.synchronize()
+        for s, w, (go, to, idx, off) in zip(streams, weights, args):
+            with torch.cuda.stream(s):
+                module.backward_sgd(go, w, to, idx, off, 0.05, 200, 1, False)
+        torch.cuda.synchronize()
+        for w, want in zip(weights, expect):
+            assert torch.equal(w, want)
