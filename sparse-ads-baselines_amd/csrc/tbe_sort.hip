@@ -6,20 +6,22 @@
 // The sort is the contract of cub::DeviceRadixSort::SortPairs as the reference
 // calls it (table_batched_embeddings_cuda.cu:1639-1655): ascending, stable,
 // key bits [0, end_bit).  A pass handles a digit of 8 to 10 bits (the fewest passes that cover
-// end_bit).  Each pass is three or four kernels:
+// end_bit).  Each pass is two or four kernels:
 //   histogram  per-tile digit counts (LDS atomics)
 //   scan       turns the counts into the output position of every (table, digit, tile) run.
 //              Many tables of few tiles each (the backward's case: every table is sorted on its
-//              own): counts[tile][digit], the histogram also adds its counts to per-table digit
-//              totals, and ONE kernel with a workgroup per table scans the totals over the
-//              digits and walks the table's tiles.  Otherwise: counts[table][digit][tile] and a
-//              linear exclusive prefix sum over the whole array (workgroup sums, then the chunks)
+//              own): no kernel.  Counts are kept as counts[tile][digit], the histogram also adds
+//              its counts to per-table digit totals (and to totals of every 64 tiles), and the
+//              scatter kernel of a tile scans the table's totals over the digits and adds up the
+//              counts of the table's earlier tiles itself.  Otherwise: counts[table][digit][tile]
+//              and a linear exclusive prefix sum over the whole array (workgroup sums, then the
+//              chunks)
 //   scatter    ranks each key inside its tile with wavefront ballots (all lanes
 //              holding the same digit are found with one ballot per digit bit; the lowest lane
 //              reserves the run in a per-wavefront LDS counter), reorders the
 //              tile in LDS so every digit's keys are contiguous, and writes
 //              them out in runs.
-// A tile is 4096 pairs; position order inside a tile is (wavefront, item, lane),
+// A tile is 4096 pairs (1024 for small inputs); position order inside a tile is (wavefront, item, lane),
 // which the ranking preserves, so the sort is stable.
 
 #include <algorithm>
@@ -40,13 +42,12 @@ constexpr int kSmallItems = 4;
 constexpr int64_t kSmallSortPairs = 1 << 19;      // up to this many pairs: kSmallItems per thread
 inline int sort_items(int64_t n) { return n <= kSmallSortPairs ? kSmallItems : kItems; }
 
-// Per-table scan: tables of at most this many tiles are scanned inside the scatter kernel (every
-// workgroup adds up the counts of the earlier tiles of its table itself); a batch with a larger
-// table runs radix_table_scan_kernel first.  tile_prefix[T + 1] holds the choice (1 = inside).
-constexpr int kInlineScanTiles = 64;
-// (quarter-size tiles: as many pairs per table, so that no batch of theirs of up to 2^18 pairs
-// launches the scan kernel)
-constexpr int inline_scan_tiles(int items) { return kInlineScanTiles * (kItems / items); }
+// Per-table layout of the counts: the scatter kernel of a tile adds up the counts of the earlier
+// tiles of its table itself.  So that a table of many tiles costs it few loads, the histogram
+// kernel also collects the counts of every kGroupTiles consecutive tiles (numbered over all tables)
+// in group totals: a range of tiles is then its whole groups plus fewer than kGroupTiles tiles at
+// either end.
+constexpr int kGroupTiles = 64;
 
 constexpr int kSegItems = 8;
 constexpr int kSegTile = kBlockThreads * kSegItems;  // 2048
@@ -179,7 +180,6 @@ __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
     *reinterpret_cast<uint4 *>(totals + i) = make_uint4(0, 0, 0, 0);
   if (blockIdx.x != 0) return;
   uint32_t carry = 0;
-  uint32_t most = 0;
   for (int c0 = 0; c0 < num_tables; c0 += kBlockThreads) {
     const int t = c0 + tid;
     uint32_t tiles = 0;
@@ -198,18 +198,11 @@ __global__ __launch_bounds__(kBlockThreads) void sort_setup_kernel(
     const uint32_t incl = block_inclusive_scan(tiles, s_wave, total);
     if (t < num_tables) tile_prefix[t] = carry + incl - tiles;
     carry += total;
-    most = max(most, tiles);
     __syncthreads();
   }
-  // the table with the most tiles decides how the per-table scan is done (see radix_scatter_kernel)
-  for (int d = 1; d < kWave; d <<= 1) most = max(most, static_cast<uint32_t>(__shfl_xor(static_cast<int>(most), d, kWave)));
-  if ((tid & (kWave - 1)) == 0) s_wave[tid >> 6] = most;
-  __syncthreads();
   if (tid == 0) {
-    for (int w = 1; w < kWavesPerBlock; ++w) most = max(most, s_wave[w]);
     table_starts[num_tables] = n;
     tile_prefix[num_tables] = carry;
-    tile_prefix[num_tables + 1] = most <= inline_scan_tiles(ITEMS) ? 1u : 0u;
   }
 }
 
@@ -221,13 +214,14 @@ struct TileInfo {
   int64_t count_base;  // index of counts[table][digit 0][this tile]
   int table_tiles;     // stride between digits in counts[]
   int64_t tile_index;  // number of the tile among all tiles
+  int64_t first_tile;  // number of the table's first tile
 };
 
 template <int BITS, int ITEMS>
 __device__ __forceinline__ TileInfo locate_tile(const uint32_t *__restrict__ table_starts,
                                                 const uint32_t *__restrict__ tile_prefix,
                                                 int num_tables, int max_tiles) {
-  TileInfo info{0, 0, 0, 0, 0, 0};
+  TileInfo info{0, 0, 0, 0, 0, 0, 0};
   const uint32_t tile = blockIdx.x;
   if (tile >= tile_prefix[num_tables]) return info;
   int lo = 0, hi = num_tables;  // tile_prefix[lo] <= tile < tile_prefix[hi]
@@ -246,6 +240,7 @@ __device__ __forceinline__ TileInfo locate_tile(const uint32_t *__restrict__ tab
   info.count_base = (static_cast<int64_t>(first_tile) << BITS) + j;
   info.table_tiles = static_cast<int>(tiles);
   info.tile_index = static_cast<int64_t>(tile);
+  info.first_tile = static_cast<int64_t>(first_tile);
   return info;
 }
 
@@ -264,7 +259,8 @@ template <int BITS, bool LOCAL, int ITEMS>
 __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     const uint32_t *__restrict__ keys, const uint32_t *__restrict__ table_starts,
     const uint32_t *__restrict__ tile_prefix, int num_tables, int max_tiles, int shift,
-    uint32_t mask, uint32_t *__restrict__ counts, uint32_t *__restrict__ totals) {
+    uint32_t mask, uint32_t *__restrict__ counts, uint32_t *__restrict__ totals,
+    uint32_t *__restrict__ group_totals) {
   constexpr int kBinsT = 1 << BITS;
   __shared__ uint32_t s_hist[kBinsT];
   const TileInfo tile = locate_tile<BITS, ITEMS>(table_starts, tile_prefix, num_tables, max_tiles);
@@ -288,69 +284,16 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
   __syncthreads();
   // (linear-scan layout: one 4-byte store per digit, a tile apart -- these scattered stores are
   // most of the kernel's time there; per-table layout: coalesced stores, and the table's digit
-  // totals collect the counts with integer atomics, whose order does not matter)
+  // totals collect the counts with integer atomics, whose order does not matter; so do the group
+  // totals, which only the tiles of a table of more than kGroupTiles tiles can be asked for)
+  const bool grouped = LOCAL && tile.table_tiles > kGroupTiles;
 #pragma unroll
   for (int d = tid; d < kBinsT; d += kBlockThreads) {
     const uint32_t c = s_hist[d];
     counts[count_index<BITS, LOCAL>(tile, d)] = c;
     if constexpr (LOCAL) {
       if (c) atomicAdd(&totals[(static_cast<int64_t>(tile.table) << BITS) + d], c);
-    }
-  }
-}
-
-// Per-table scan (LOCAL layout): workgroup t turns table t's counts[tile][digit] into output
-// positions.  Thread `tid` owns 2^BITS / 256 consecutive digits: exclusive scan of the table's
-// digit totals (thread-local, then across the workgroup) gives the first output position of every
-// digit, then the thread walks the table's tiles, replacing each count by the running position.
-template <int BITS>
-__global__ __launch_bounds__(kBlockThreads) void radix_table_scan_kernel(
-    uint32_t *__restrict__ counts, const uint32_t *__restrict__ totals,
-    const uint32_t *__restrict__ table_starts, const uint32_t *__restrict__ tile_prefix,
-    int max_tiles) {
-  constexpr int kBinsT = 1 << BITS;
-  constexpr int kOwned = kBinsT / kBlockThreads;
-  constexpr int kAhead = 4;  // tiles whose counts are requested together
-  __shared__ uint32_t s_wave[kWavesPerBlock];
-  const int t = blockIdx.x;
-  if (tile_prefix[gridDim.x + 1] != 0u) return;  // every table is small: the scatter kernel scans
-  const uint32_t first_tile = tile_prefix[t];
-  const uint32_t tiles = tile_prefix[t + 1] - first_tile;
-  if (tiles == 0 || first_tile + tiles > static_cast<uint32_t>(max_tiles)) return;
-  const int d0 = threadIdx.x * kOwned;
-  uint32_t running[kOwned];
-  uint32_t mine = 0;
-#pragma unroll
-  for (int q = 0; q < kOwned; ++q) {
-    running[q] = totals[(static_cast<int64_t>(t) << BITS) + d0 + q];
-    mine += running[q];
-  }
-  uint32_t total;
-  uint32_t start = table_starts[t] + block_inclusive_scan(mine, s_wave, total) - mine;
-#pragma unroll
-  for (int q = 0; q < kOwned; ++q) {
-    const uint32_t c = running[q];
-    running[q] = start;
-    start += c;
-  }
-  uint32_t *mine_counts = counts + (static_cast<int64_t>(first_tile) << BITS) + d0;
-  for (uint32_t j0 = 0; j0 < tiles; j0 += kAhead) {
-    uint32_t c[kAhead][kOwned];
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a) {
-      const uint32_t j = min(j0 + a, tiles - 1);  // clamped: straight-line loads
-#pragma unroll
-      for (int q = 0; q < kOwned; ++q) c[a][q] = mine_counts[(static_cast<int64_t>(j) << BITS) + q];
-    }
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a) {
-      if (j0 + a < tiles) {
-#pragma unroll
-        for (int q = 0; q < kOwned; ++q) {
-          mine_counts[(static_cast<int64_t>(j0 + a) << BITS) + q] = running[q];
-          running[q] += c[a][q];
-        }
-      }
+      if (c && grouped) atomicAdd(&group_totals[((tile.tile_index / kGroupTiles) << BITS) + d], c);
     }
   }
 }
@@ -426,7 +369,8 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     uint32_t *__restrict__ keys_out, uint32_t *__restrict__ values_out,
     const uint32_t *__restrict__ table_starts, const uint32_t *__restrict__ tile_prefix,
     int num_tables, int max_tiles, int shift, uint32_t mask, const uint32_t *__restrict__ bases,
-    const uint32_t *__restrict__ totals, const int32_t *__restrict__ key_bias) {
+    const uint32_t *__restrict__ totals, const uint32_t *__restrict__ group_totals,
+    const int32_t *__restrict__ key_bias) {
   constexpr int kBinsT = 1 << BITS;
   constexpr int kOwned = kBinsT / kBlockThreads;  // consecutive digits per thread
   // The per-wavefront digit counters are only needed until every key knows its slot in the
@@ -453,32 +397,42 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   // output position of the tile's first key of every digit this thread owns (needed late;
   // fetched first so the latency hides behind the ranking)
   uint32_t digit_base[kOwned];
-  uint32_t digit_total[kOwned];  // per-table layout, scan done here: keys of the table with each digit
-  bool inline_scan = false;
-  if constexpr (LOCAL) inline_scan = tile_prefix[num_tables + 1] != 0u;
-  if (inline_scan) {
-    // bases[] still holds counts[tile][digit]: this tile's keys of digit d go behind the table's
-    // keys of smaller digits (added up further down, once the totals are here) and behind the keys
-    // of digit d in the earlier tiles of the table
-    const int j = static_cast<int>(tile.tile_index - (tile.count_base >> BITS));  // tile inside its table
-    const uint32_t *first = bases + ((tile.count_base >> BITS) << BITS) + tid * kOwned;
+  uint32_t digit_total[kOwned];  // per-table layout: keys of the table with each digit
+  if constexpr (LOCAL) {
+    // bases[] holds counts[tile][digit]: this tile's keys of digit d go behind the table's keys of
+    // smaller digits (added up further down, once the totals are here) and behind the keys of
+    // digit d in the earlier tiles of the table, [first, tile): fewer than kGroupTiles tiles up to
+    // a multiple of kGroupTiles, whole groups, and fewer than kGroupTiles tiles again.
 #pragma unroll
     for (int q = 0; q < kOwned; ++q) {
       digit_total[q] = totals[(static_cast<int64_t>(tile.table) << BITS) + tid * kOwned + q];
       digit_base[q] = 0;
     }
-    constexpr int kAhead = 8;
-    for (int j0 = 0; j0 < j; j0 += kAhead) {
-      uint32_t c[kAhead][kOwned];
+    // adds rows [from, to) of a [row][digit] array to digit_base, eight rows requested at a time
+    auto add_rows = [&](const uint32_t *__restrict__ rows, int64_t from, int64_t to) {
+      constexpr int kAhead = 8;
+      const uint32_t *mine = rows + tid * kOwned;
+      for (int64_t r0 = from; r0 < to; r0 += kAhead) {
+        uint32_t c[kAhead][kOwned];
 #pragma unroll
-      for (int a = 0; a < kAhead; ++a)
+        for (int a = 0; a < kAhead; ++a)
 #pragma unroll
-        for (int q = 0; q < kOwned; ++q)
-          c[a][q] = first[(static_cast<int64_t>(min(j0 + a, j - 1)) << BITS) + q];
+          for (int q = 0; q < kOwned; ++q) c[a][q] = mine[(min(r0 + a, to - 1) << BITS) + q];
 #pragma unroll
-      for (int a = 0; a < kAhead; ++a)
+        for (int a = 0; a < kAhead; ++a)
 #pragma unroll
-        for (int q = 0; q < kOwned; ++q) digit_base[q] += (j0 + a < j) ? c[a][q] : 0u;
+          for (int q = 0; q < kOwned; ++q) digit_base[q] += (r0 + a < to) ? c[a][q] : 0u;
+      }
+    };
+    const int64_t first = tile.first_tile;
+    const int64_t head_end = (first + kGroupTiles - 1) / kGroupTiles * kGroupTiles;
+    const int64_t tail_begin = tile.tile_index / kGroupTiles * kGroupTiles;
+    if (head_end >= tail_begin) {
+      add_rows(bases, first, tile.tile_index);  // no whole group in between
+    } else {
+      add_rows(bases, first, head_end);
+      add_rows(group_totals, head_end / kGroupTiles, tail_begin / kGroupTiles);
+      add_rows(bases, tail_begin, tile.tile_index);
     }
   } else {
 #pragma unroll
@@ -556,7 +510,7 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     }
     uint32_t total;
     uint32_t bin_start = block_inclusive_scan(mine, s_scan, total) - mine;
-    if (inline_scan) {
+    if constexpr (LOCAL) {
       // first output position of every digit inside the table: exclusive scan of the table's totals
       uint32_t table_sum = 0;
 #pragma unroll
@@ -737,19 +691,21 @@ inline int num_seg_tiles(int64_t n) { return static_cast<int>(ceil_div(n, kSegTi
 }  // namespace
 
 // Sort workspace: [tmp keys n][tmp values n][counts 1024 * max_tiles][workgroup sums of the count
-// scan][table_starts T+1][tile_prefix T+2][digit totals 4 * 1024 * T]; max_tiles = ceil(n / tile) + T.
+// scan][table_starts T+1][tile_prefix T+2][digit totals 4 * 1024 * T][group totals 4 * 1024 *
+// groups]; max_tiles = ceil(n / tile) + T, groups = ceil(max_tiles / kGroupTiles).
 namespace {
 struct SortScratch {
   uint64_t tmp_keys, tmp_vals, counts, block_sums, table_starts, tile_prefix, totals, total;
   int max_tiles;
   int scan_blocks;  // for the widest digit
-  int64_t totals_words;  // per-table digit totals of all passes (0: linear scan)
+  int64_t groups;   // groups of kGroupTiles tiles that the region behind the digit totals has room for
 };
 
 constexpr int kMaxPasses = 4;  // 32 key bits in digits of at least 8
 
-// The per-table scan walks a table's tiles one after the other in one workgroup: it is used when
-// the tables have few tiles each on average (the batch's lookups are spread over many tables).
+// The per-table layout of the counts (no scan between the histogram and the scatter kernel) is
+// used when the tables have few tiles each on average: the batch's lookups are spread over many
+// tables.
 inline bool use_table_scan(int64_t n, int32_t num_tables, bool have_tables) {
   return have_tables && num_tables >= 8 &&
          ceil_div(n, kBlockThreads * sort_items(n)) <= static_cast<int64_t>(num_tables) * 128 * (kItems / sort_items(n));
@@ -773,22 +729,24 @@ SortScratch sort_scratch(int64_t n, int32_t num_tables) {
   s.block_sums = off; off += align_up(static_cast<uint64_t>(s.scan_blocks) * 4, 256);
   s.table_starts = off; off += align_up((tables + 1) * 4, 256);
   s.tile_prefix = off; off += align_up((tables + 2) * 4, 256);
-  // (sized for every table count, so that the layout does not depend on the path taken)
-  s.totals_words = static_cast<int64_t>(tables) * kMaxBins * kMaxPasses;
-  s.totals = off; off += align_up(static_cast<uint64_t>(s.totals_words) * 4, 256);
+  // (sized for every table count, so that the layout does not depend on the path taken; the group
+  // totals follow the digit totals at once, so that one clearing loop covers both)
+  s.groups = static_cast<int64_t>(ceil_div(sized_tiles, kGroupTiles));
+  s.totals = off;
+  off += align_up((tables + static_cast<uint64_t>(s.groups)) * kMaxBins * kMaxPasses * 4, 256);
   s.total = off;
   return s;
 }
 
 struct RadixPass {
-  bool tables_small;  // known on the host: no table can have more than kInlineScanTiles tiles
   const uint32_t *src_k, *src_v;
   uint32_t *dst_k, *dst_v;
   const uint32_t *table_starts, *tile_prefix;
   int num_tables, max_tiles, shift;
   uint32_t mask;
   uint32_t *counts, *block_sums;
-  uint32_t *totals;  // this pass's per-table digit totals, zeroed; null: linear scan
+  uint32_t *totals;        // this pass's per-table digit totals, zeroed; null: linear scan
+  uint32_t *group_totals;  // this pass's digit totals of every kGroupTiles tiles, zeroed
   const int32_t *key_bias;
 };
 
@@ -798,27 +756,23 @@ void launch_radix_pass(const RadixPass &p, hipStream_t stream) {
   const dim3 tiles(p.max_tiles);
   if (p.totals) {
     TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, true, ITEMS>), tiles, block, p.src_k,
-               p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, p.totals);
-    // (the scatter kernel scans small tables itself, and this kernel returns at once when all
-    // are small; a batch of so few pairs that they must be does not launch it)
-    if (!p.tables_small)
-      TBE_LAUNCH("radix_table_scan", stream, radix_table_scan_kernel<BITS>, dim3(p.num_tables), block, p.counts,
-                 p.totals, p.table_starts, p.tile_prefix, p.max_tiles);
+               p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, p.totals,
+               p.group_totals);
     TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, true, ITEMS>), tiles, block, p.src_k, p.src_v,
                p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
-               p.counts, p.totals, p.key_bias);
+               p.counts, p.totals, p.group_totals, p.key_bias);
     return;
   }
   const dim3 scan_blocks(static_cast<unsigned>(ceil_div(static_cast<int64_t>(p.max_tiles) << BITS, kScanChunk)));
   TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, false, ITEMS>), tiles, block, p.src_k,
-             p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, nullptr);
+             p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, nullptr, nullptr);
   TBE_LAUNCH("radix_scan_reduce", stream, radix_scan_reduce_kernel, scan_blocks, block, p.counts,
              p.tile_prefix, p.num_tables, BITS, p.block_sums);
   TBE_LAUNCH("radix_scan", stream, radix_scan_kernel, scan_blocks, block, p.counts, p.tile_prefix,
              p.num_tables, BITS, p.block_sums);
   TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, false, ITEMS>), tiles, block, p.src_k, p.src_v,
              p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
-             p.counts, nullptr, p.key_bias);
+             p.counts, nullptr, nullptr, p.key_bias);
 }
 }  // namespace
 
@@ -839,7 +793,6 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
 
   RadixPass p;
   const int items = sort_items(n);
-  p.tables_small = ceil_div(n, kBlockThreads * items) <= inline_scan_tiles(items);
   p.table_starts = reinterpret_cast<uint32_t *>(ws + scratch.table_starts);
   p.tile_prefix = reinterpret_cast<uint32_t *>(ws + scratch.tile_prefix);
   p.num_tables = num_tables;
@@ -848,7 +801,10 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
   p.block_sums = reinterpret_cast<uint32_t *>(ws + scratch.block_sums);
   const bool table_scan = use_table_scan(n, num_tables, tables != nullptr) && passes <= kMaxPasses;
   uint32_t *totals = reinterpret_cast<uint32_t *>(ws + scratch.totals);
-  const int64_t totals_words = table_scan ? static_cast<int64_t>(num_tables) * kMaxBins * passes : 0;
+  // per pass: T rows of digit totals; behind those of all passes, per pass, a row per group of tiles
+  const int64_t groups = ceil_div(scratch.max_tiles, kGroupTiles);
+  const int64_t totals_words = table_scan ? (num_tables + groups) * kMaxBins * passes : 0;
+  uint32_t *group_totals = totals + static_cast<int64_t>(num_tables) * kMaxBins * passes;
   const unsigned setup_blocks = static_cast<unsigned>(1 + std::min<int64_t>(ceil_div(totals_words, kBlockThreads * 4), 255));
   int32_t *grad_rows = tables ? tables->grad_rows : nullptr;
   const unsigned row_blocks =
@@ -877,6 +833,7 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
     p.dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
     p.key_bias = (tables && pass == passes - 1) ? tables->key_bias : nullptr;
     p.totals = table_scan ? totals + static_cast<int64_t>(pass) * num_tables * kMaxBins : nullptr;
+    p.group_totals = table_scan ? group_totals + static_cast<int64_t>(pass) * groups * kMaxBins : nullptr;
     if (items == kSmallItems) {
       if (bits <= 8) launch_radix_pass<8, kSmallItems>(p, stream);
       else if (bits == 9) launch_radix_pass<9, kSmallItems>(p, stream);

@@ -155,7 +155,8 @@ def _plan_views(p, max_table_rows):
 @pytest.mark.parametrize("case", ["ragged_rows", "empty_tables", "many_small_tables", "multi_tile_tables", "one_table",
                                   "eight_tables_of_thirty_tiles", "one_large_table_among_nine",
                                   "ten_bit_digits", "eight_tables_of_forty_small_tiles",
-                                  "one_larger_table_among_nine", "ten_bit_digits_full_tiles"])
+                                  "one_larger_table_among_nine", "ten_bit_digits_full_tiles",
+                                  "two_tables_of_hundreds_of_tiles"])
 def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
     """The plan sorts every table's indices on their own (fewer key bits); keys_sorted,
     positions_sorted and segment_starts must equal the stable sort of table_offsets[t] + index
@@ -192,6 +193,19 @@ def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
         lengths[3] = 80 if case == "one_large_table_among_nine" else 200
         offsets = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
         indices = np.concatenate([rs.zipf(1.2, size=int(lengths[t].sum())) % rows[t] for t in range(T)])
+        p = dict(T=T, B=B, rows=rows, n=int(offsets[-1]), offsets=offsets, indices=indices.astype(np.int32),
+                 table_offsets=np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
+    elif case == "two_tables_of_hundreds_of_tiles":
+        # 300 and 200 tiles in two of ten tables: their later tiles add up whole groups of 64 tiles
+        # from the group totals, and the groups do not start where the tables do
+        rs = np.random.RandomState(23)
+        T, B = 10, 4100
+        rows = [4000, 100, 1 << 19, 50000, 7, 900, 30000, 700001, 12, 65536]
+        lengths = np.full((T, B), 3)
+        lengths[2] = 300
+        lengths[7] = 200
+        offsets = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
+        indices = np.concatenate([rs.zipf(1.15, size=int(lengths[t].sum())) % rows[t] for t in range(T)])
         p = dict(T=T, B=B, rows=rows, n=int(offsets[-1]), offsets=offsets, indices=indices.astype(np.int32),
                  table_offsets=np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
     elif case in ("ten_bit_digits", "ten_bit_digits_full_tiles"):
