@@ -222,8 +222,15 @@ __device__ __forceinline__ TileInfo locate_tile(const uint32_t *__restrict__ tab
                                                 const uint32_t *__restrict__ tile_prefix,
                                                 int num_tables, int max_tiles) {
   TileInfo info{0, 0, 0, 0, 0, 0, 0};
-  const uint32_t tile = blockIdx.x;
-  if (tile >= tile_prefix[num_tables]) return info;
+  // Workgroups go to the eight XCDs in turn: workgroup b takes tile (b % 8) * ceil(tiles / 8) + b / 8,
+  // so that an XCD works on consecutive tiles (mostly of one table at a time).  The runs that those
+  // tiles scatter into the same output lines then meet in one L2, and the scatter kernel finds the
+  // keys and the counts there that the histogram kernel of the same tiles left.
+  const uint32_t all_tiles = tile_prefix[num_tables];
+  const uint32_t per_xcd = (all_tiles + kNumXcd - 1) / kNumXcd;
+  const uint32_t turn = blockIdx.x / kNumXcd;
+  const uint32_t tile = (blockIdx.x % kNumXcd) * per_xcd + turn;
+  if (turn >= per_xcd || tile >= all_tiles) return info;
   int lo = 0, hi = num_tables;  // tile_prefix[lo] <= tile < tile_prefix[hi]
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -753,7 +760,7 @@ struct RadixPass {
 template <int BITS, int ITEMS>
 void launch_radix_pass(const RadixPass &p, hipStream_t stream) {
   const dim3 block(kBlockThreads);
-  const dim3 tiles(p.max_tiles);
+  const dim3 tiles(static_cast<unsigned>(ceil_div(p.max_tiles, kNumXcd) * kNumXcd));  // (whole turns of the XCDs)
   if (p.totals) {
     TBE_LAUNCH("radix_histogram", stream, (radix_histogram_kernel<BITS, true, ITEMS>), tiles, block, p.src_k,
                p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask, p.counts, p.totals,
