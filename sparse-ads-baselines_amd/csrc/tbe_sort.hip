@@ -381,11 +381,11 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
   constexpr int kBinsT = 1 << BITS;
   constexpr int kOwned = kBinsT / kBlockThreads;  // consecutive digits per thread
   // The per-wavefront digit counters are only needed until every key knows its slot in the
-  // reordered tile.  For 10-bit digits (16 KB of counters) they share LDS with the reordered
-  // keys, which keeps four workgroups on a compute unit at the price of one more barrier.
+  // reordered tile.  For 9- and 10-bit digits (8 and 16 KB of counters) they share LDS with the
+  // reordered keys, which keeps four workgroups on a compute unit at the price of one more barrier.
   constexpr int kTileT = kBlockThreads * ITEMS;
   constexpr int kWaveTileT = kWave * ITEMS;
-  constexpr bool kShareCounters = BITS >= 10 && kWavesPerBlock * kBinsT <= kTileT;
+  constexpr bool kShareCounters = BITS >= 9 && kWavesPerBlock * kBinsT <= kTileT;
   __shared__ uint32_t s_keys[kTileT];
   __shared__ uint32_t s_vals[kTileT];
   __shared__ uint32_t s_own_count[kShareCounters ? 1 : kWavesPerBlock][kShareCounters ? 1 : kBinsT];
