@@ -23,6 +23,12 @@ int key_bits(int64_t total_rows) {
   return bits;
 }
 
+// Every table is sorted on its own as long as there are at most this many: each table costs the
+// sort a (possibly nearly empty) tile and 20 KB of counters.  A batch over more tables than that
+// sorts the linearized keys in one piece, like the reference (tbe.cu:1639-1655).
+constexpr int32_t kMaxTablesSortedApart = 2048;
+inline int32_t sort_tables(int32_t T) { return T <= kMaxTablesSortedApart ? T : 1; }
+
 void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *l) {
   const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
   const uint64_t ints = align_up(nn * 4, 256);
@@ -38,7 +44,7 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspac
   l->positions_sorted = off; off += ints;
   l->segment_starts = off; off += align_up((nn + 1) * 4, 256);
   l->num_unique = off; off += 256;
-  l->sort_scratch = off; off += align_up(sort_workspace_bytes(n, T), 256);
+  l->sort_scratch = off; off += align_up(sort_workspace_bytes(n, sort_tables(T)), 256);
   l->segment_scratch = off; off += align_up(segments_workspace_bytes(n), 256);
   l->segment_ids = off; off += ints;
   l->long_segments = off; off += align_up(static_cast<uint64_t>(l->max_long_segments) * 16, 256);
@@ -56,23 +62,43 @@ void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspa
   compute_layout(n, D, dtype, T, l);
 }
 
-// gradient rows -> sort -> run boundaries (and the segment of every sorted position) into the
-// workspace regions of `l`.  The lookups of a table are consecutive, so the (table, row) order
-// of the reference's sort (tbe.cu:1639-1655) is reached by sorting every table's indices on
-// their own; the last pass adds the table's first row, and keys_sorted / positions_sorted come
-// out as the sort of the linearized keys would leave them.  The `keys` region stays unwritten.
+// sort_batch: gradient rows and the sort; build_plan: also the run boundaries (and the segment of
+// every sorted position), into the workspace regions of `l`.  The lookups of a table are
+// consecutive, so the (table, row) order of the reference's sort (tbe.cu:1639-1655) is reached by
+// sorting every table's indices on their own; the last pass adds the table's first row, and
+// keys_sorted / positions_sorted come out as the sort of the linearized keys would leave them.
+// The `keys` region stays unwritten, unless the batch has more than kMaxTablesSortedApart tables:
+// then the linearized keys are written there and sorted in one piece.
+int sort_batch(const tbe_workspace_layout_t &l, void *workspace, const int32_t *table_offsets, int32_t T,
+               const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B, int64_t total_rows,
+               int64_t max_table_rows, hipStream_t stream) {
+  char *ws = static_cast<char *>(workspace);
+  int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
+  int32_t *positions_sorted = reinterpret_cast<int32_t *>(ws + l.positions_sorted);
+  int32_t *grad_rows = reinterpret_cast<int32_t *>(ws + l.grad_rows);
+  if (sort_tables(T) != T) {
+    int32_t *keys = reinterpret_cast<int32_t *>(ws + l.keys);
+    const int rc = linearize(table_offsets, T, indices, offsets, B, keys, grad_rows, stream);
+    if (rc) return rc;
+    return sort_pairs(keys, nullptr, keys_sorted, positions_sorted, n, key_bits(total_rows), ws + l.sort_scratch,
+                      stream, nullptr);
+  }
+  const int64_t largest = (max_table_rows > 0 && max_table_rows < total_rows) ? max_table_rows : total_rows;
+  // (the gradient row of every position is recorded by the sort's first launch)
+  const SortTables tables{offsets, B, T, table_offsets, grad_rows};
+  return sort_pairs(indices, nullptr, keys_sorted, positions_sorted, n, key_bits(largest), ws + l.sort_scratch,
+                    stream, &tables);
+}
+
 int build_plan(const tbe_workspace_layout_t &l, void *workspace, const int32_t *table_offsets,
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
                int64_t total_rows, int64_t max_table_rows, hipStream_t stream) {
   char *ws = static_cast<char *>(workspace);
-  int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
-  const int64_t largest = (max_table_rows > 0 && max_table_rows < total_rows) ? max_table_rows : total_rows;
-  // (the gradient row of every position is recorded by the sort's first launch)
-  const SortTables tables{offsets, B, T, table_offsets, reinterpret_cast<int32_t *>(ws + l.grad_rows)};
-  int rc = sort_pairs(indices, nullptr, keys_sorted, reinterpret_cast<int32_t *>(ws + l.positions_sorted),
-                  n, key_bits(largest), ws + l.sort_scratch, stream, &tables);
+  const int rc = sort_batch(l, workspace, table_offsets, T, indices, n, offsets, B, total_rows, max_table_rows,
+                            stream);
   if (rc) return rc;
-  return find_segments(keys_sorted, n, reinterpret_cast<int32_t *>(ws + l.segment_starts),
+  return find_segments(reinterpret_cast<int32_t *>(ws + l.keys_sorted), n,
+                       reinterpret_cast<int32_t *>(ws + l.segment_starts),
                        reinterpret_cast<int32_t *>(ws + l.num_unique),
                        reinterpret_cast<int32_t *>(ws + l.segment_ids), ws + l.segment_scratch,
                        stream, /*clear_queue_counters=*/true);

@@ -1013,10 +1013,8 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
   auto i32 = [&](uint64_t off) { return reinterpret_cast<int32_t *>(ws + off); };
   // every table's indices are sorted on their own; the last pass adds the table's first row id.
   // The sort's first launch also records the gradient row b*T + t of every position.
-  const int64_t largest = (max_table_rows > 0 && max_table_rows < total_rows) ? max_table_rows : total_rows;
-  const SortTables tables{offsets, B, T, table_dim_offsets, i32(l.grad_rows)};
-  int rc = sort_pairs(indices, nullptr, i32(l.keys_sorted), i32(l.positions_sorted), num_indices,
-                  key_bits_for(largest), ws + l.sort_scratch, s, &tables);
+  int rc = sort_batch(l, workspace, table_dim_offsets, T, indices, num_indices, offsets, B, total_rows,
+                      max_table_rows, s);
   if (rc) return rc;
   rc = find_segments(i32(l.keys_sorted), num_indices, i32(l.segment_starts), i32(l.num_unique), nullptr,
                      ws + l.segment_scratch, s, /*clear_queue_counters=*/true);

@@ -109,6 +109,10 @@ int key_bits_for(int64_t total_rows);
 void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *layout);
 // max_table_rows: an upper bound of the rows of the largest table (0 = unknown, total_rows is
 // used); it sets how many key bits are sorted.
+// grad_rows, keys_sorted and positions_sorted of the layout (table_offsets: first row of every table)
+int sort_batch(const tbe_workspace_layout_t &layout, void *workspace, const int32_t *table_offsets, int32_t T,
+               const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B, int64_t total_rows,
+               int64_t max_table_rows, hipStream_t stream);
 int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int32_t *table_offsets,
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
                int64_t total_rows, int64_t max_table_rows, hipStream_t stream);

@@ -156,7 +156,7 @@ def _plan_views(p, max_table_rows):
                                   "eight_tables_of_thirty_tiles", "one_large_table_among_nine",
                                   "ten_bit_digits", "eight_tables_of_forty_small_tiles",
                                   "one_larger_table_among_nine", "ten_bit_digits_full_tiles",
-                                  "two_tables_of_hundreds_of_tiles"])
+                                  "two_tables_of_hundreds_of_tiles", "more_tables_than_are_sorted_apart"])
 def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
     """The plan sorts every table's indices on their own (fewer key bits); keys_sorted,
     positions_sorted and segment_starts must equal the stable sort of table_offsets[t] + index
@@ -195,6 +195,9 @@ def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
         indices = np.concatenate([rs.zipf(1.2, size=int(lengths[t].sum())) % rows[t] for t in range(T)])
         p = dict(T=T, B=B, rows=rows, n=int(offsets[-1]), offsets=offsets, indices=indices.astype(np.int32),
                  table_offsets=np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
+    elif case == "more_tables_than_are_sorted_apart":
+        # beyond 2048 tables the linearized keys are sorted in one piece
+        p = make_problem(24, T=2500, E=41, D=4, B=5, L=6, dtype=np.float32)
     elif case == "two_tables_of_hundreds_of_tiles":
         # 300 and 200 tiles in two of ten tables: their later tiles add up whole groups of 64 tiles
         # from the group totals, and the groups do not start where the tables do
@@ -228,7 +231,8 @@ def test_per_table_sort_equals_sort_of_linearized_keys(oracle, case):
 
 # --------------------------------------------------- fused backward vs oracle
 SHAPES = [(2, 1000, 32, 64, 4), (3, 50, 128, 33, 20), (1, 7, 4, 5, 3), (2, 100, 12, 17, 9), (2, 30, 520, 9, 5),
-          (4, 20, 64, 700, 40), (2, 100, 256, 50, 70), (1, 3, 8, 400, 9), (2, 64, 16, 31, 6)]
+          (4, 20, 64, 700, 40), (2, 100, 256, 50, 70), (1, 3, 8, 400, 9), (2, 64, 16, 31, 6),
+          (2100, 20, 8, 3, 4)]  # (the last: more tables than are sorted apart)
 
 
 def _run_both(oracle, p, optimizer, lr, eps):
