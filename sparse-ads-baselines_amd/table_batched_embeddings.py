@@ -85,15 +85,16 @@ def _rounding_stream(device):
 
 
 def _workspace(device, nbytes):
-    """The grow-only scratch buffer of the device's current stream: one per (device, stream), so
-    that calls issued on different streams of a device may overlap."""
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    """The grow-only scratch buffer of the device's current stream, and that stream: one buffer per
+    (device, stream), so that calls issued on different streams of a device may overlap."""
+    handle = torch.cuda.current_stream(device).cuda_stream
+    key = (device, handle)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     _last_workspace[device] = ws
-    return ws
+    return ws, ctypes.c_void_p(handle)
 
 
 def backward_workspace(device):
@@ -198,13 +199,13 @@ def backward_sgd(grad_output, weights, table_offsets, indices, offsets, learning
     D = weights.size(1)
     code = _DTYPE_CODES[weights.dtype]
     layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
-    ws = _workspace(weights.device, layout.total_bytes)
+    ws, stream = _workspace(weights.device, layout.total_bytes)
     with torch.cuda.device(weights.device):
         _native.check(_native.load().tbe_backward_sgd(
             _ptr(grad_output), _ptr(weights), code, weights.size(0),
             max_table_rows(table_offsets, weights.size(0)), D, _ptr(table_offsets), T,
             _ptr(indices), indices.numel(), _ptr(offsets), B, float(learning_rate), _ptr(ws), ws.numel(),
-            _stream(weights.device)))
+            stream))
     return None
 
 
@@ -231,7 +232,7 @@ def backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets
                  "indice_weights must be contiguous with one entry per index")
         grad_indice_weights = torch.empty(indices.shape, dtype=grad_output.dtype, device=weights.device)
     layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
-    ws = _workspace(weights.device, layout.total_bytes)
+    ws, stream = _workspace(weights.device, layout.total_bytes)
     with torch.cuda.device(weights.device):
         if stochastic_rounding and weights.dtype == torch.float16:
             seed, offset = _rounding_stream(weights.device)
@@ -240,14 +241,14 @@ def backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets
                 max_table_rows(table_offsets, weights.size(0)), D, _ptr(table_offsets), T,
                 _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state),
                 float(learning_rate), float(eps), _ptr(grad_indice_weights), seed, offset, _ptr(ws), ws.numel(),
-                _stream(weights.device)))
+                stream))
         else:  # rounding to nearest; stochastic rounding only exists for fp16 (tbe.cu:557-578)
             _native.check(_native.load().tbe_backward_exact_adagrad(
                 _ptr(grad_output), _ptr(weights), code, weights.size(0),
                 max_table_rows(table_offsets, weights.size(0)), D, _ptr(table_offsets), T,
                 _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state),
                 float(learning_rate), float(eps), _ptr(grad_indice_weights), _ptr(ws), ws.numel(),
-                _stream(weights.device)))
+                stream))
     return grad_indice_weights
 
 
@@ -284,7 +285,7 @@ def backward_approx_adagrad(grad_output, weights, table_offsets, indices, offset
     D = weights.size(1)
     code = _DTYPE_CODES[weights.dtype]
     layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
-    ws = _workspace(weights.device, layout.total_bytes)
+    ws, stream = _workspace(weights.device, layout.total_bytes)
     stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
     seed, offset = _rounding_stream(weights.device) if stochastic else (0, 0)
     with torch.cuda.device(weights.device):
@@ -292,7 +293,7 @@ def backward_approx_adagrad(grad_output, weights, table_offsets, indices, offset
             _ptr(grad_output), _ptr(weights), code, weights.size(0), max_table_rows(table_offsets, weights.size(0)),
             D, _ptr(table_offsets), T, _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights),
             _ptr(optimizer_state), float(learning_rate), float(eps), _ptr(grad_indice_weights), int(stochastic),
-            seed, offset, _ptr(ws), ws.numel(), _stream(weights.device)))
+            seed, offset, _ptr(ws), ws.numel(), stream))
     return grad_indice_weights
 
 
@@ -375,7 +376,7 @@ def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_of
     _require(optimizer_state.dtype == state_dtype and optimizer_state.is_contiguous(),
              "optimizer_state must be contiguous %s" % state_dtype)
     layout = _native.backward_workspace_layout(indices.numel(), 4, code, T)
-    ws = _workspace(weights.device, layout.total_bytes)
+    ws, stream = _workspace(weights.device, layout.total_bytes)
     stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
     seed, offset = _rounding_stream(weights.device) if stochastic else (0, 0)
     with torch.cuda.device(weights.device):
@@ -384,7 +385,7 @@ def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_of
             max_table_rows(table_dim_offsets, None), _ptr(table_offsets), _ptr(table_dim_offsets), _ptr(dim_offsets), int(total_D), T, _ptr(indices),
             indices.numel(), _ptr(offsets), B, _ptr(indice_weights), _ptr(optimizer_state), float(learning_rate),
             float(eps or 0.0), _ptr(grad_indice_weights), int(stochastic), seed, offset, _ptr(ws), ws.numel(),
-            _stream(weights.device)))
+            stream))
     return grad_indice_weights
 
 
