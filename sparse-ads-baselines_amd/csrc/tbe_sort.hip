@@ -269,12 +269,16 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
     uint32_t mask, uint32_t *__restrict__ counts, uint32_t *__restrict__ totals,
     uint32_t *__restrict__ group_totals) {
   constexpr int kBinsT = 1 << BITS;
-  __shared__ uint32_t s_hist[kBinsT];
+  // Four counters per digit, in neighbouring LDS banks, one for every fourth lane: the lanes of a
+  // wavefront that hold a hot digit (a popular row) then queue at four addresses instead of one.
+  constexpr int kCopies = 4;
+  __shared__ uint4 s_hist[kBinsT];
+  uint32_t *s_counter = reinterpret_cast<uint32_t *>(s_hist);
   const TileInfo tile = locate_tile<BITS, ITEMS>(table_starts, tile_prefix, num_tables, max_tiles);
   if (tile.table_tiles == 0) return;
   const int tid = threadIdx.x;
 #pragma unroll
-  for (int d = tid; d < kBinsT; d += kBlockThreads) s_hist[d] = 0;
+  for (int d = tid; d < kBinsT; d += kBlockThreads) s_hist[d] = make_uint4(0, 0, 0, 0);
   __syncthreads();
   // every thread loads all its keys first (an index past the tile's end is clamped, the key
   // dropped): straight-line loads are issued back to back, predicated ones one at a time
@@ -285,7 +289,8 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
       key[k] = keys[tile.begin + min(k * kBlockThreads + tid, tile.count - 1)];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
-      if (k * kBlockThreads + tid < tile.count) atomicAdd(&s_hist[(key[k] >> shift) & mask], 1u);
+      if (k * kBlockThreads + tid < tile.count)
+        atomicAdd(&s_counter[((key[k] >> shift) & mask) * kCopies + (tid & (kCopies - 1))], 1u);
     }
   }
   __syncthreads();
@@ -296,7 +301,8 @@ __global__ __launch_bounds__(kBlockThreads) void radix_histogram_kernel(
   const bool grouped = LOCAL && tile.table_tiles > kGroupTiles;
 #pragma unroll
   for (int d = tid; d < kBinsT; d += kBlockThreads) {
-    const uint32_t c = s_hist[d];
+    const uint4 four = s_hist[d];
+    const uint32_t c = four.x + four.y + four.z + four.w;
     counts[count_index<BITS, LOCAL>(tile, d)] = c;
     if constexpr (LOCAL) {
       if (c) atomicAdd(&totals[(static_cast<int64_t>(tile.table) << BITS) + d], c);
