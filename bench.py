@@ -528,14 +528,14 @@ def run_resident(args, config, steps, warmup, profile_steps, with_cpu):
         ws = ext.backward_workspace(dev)
         U = int(ws[lay.num_unique:lay.num_unique + 4].view(torch.int32)[0])
     a_fwd, a_bwd, a_update = algorithmic_bytes(w, U)
-    # The update is split over two kernels by segment length: rows with at most 16 occurrences go
+    # The update is split over two kernels by segment length: rows with at most 128 occurrences go
     # to update_short, the others to update_chunks.  Each kernel is credited with the gradient rows
     # it gathers and the weight rows it reads and writes.
     short_share = {"lookups": w["n"], "rows": U}
     if w["optimizer"] and U:
         starts = ws[lay.segment_starts:lay.segment_starts + 4 * (U + 1)].view(torch.int32).long()
         lengths = starts[1:] - starts[:-1]
-        short = lengths <= 16
+        short = lengths <= 128  # kShortSegment of csrc/tbe_stages.h
         short_share = {"lookups": int(lengths[short].sum()), "rows": int(short.sum())}
     S = 2 if w["fp16"] else 4
     extra_per_row = 8 if w["optimizer"] == "adagrad" else 0

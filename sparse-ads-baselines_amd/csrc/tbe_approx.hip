@@ -917,7 +917,7 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
   // counter block, which the segment stage left at zero
   int32_t *counters = reinterpret_cast<int32_t *>(ws + l.num_unique);
   int32_t *long_queue = reinterpret_cast<int32_t *>(ws + l.chunk_segments);
-  const int64_t most_long = a.n / (kShortSegment + 1) + 1;  // (the short-row kernel queues rows of 17 and more)
+  const int64_t most_long = a.n / (kApproxShortSegment + 1) + 1;  // (the short-row kernel queues rows of 17 and more)
   // (a multiple of the XCD count, so that every XCD has the same number of workgroups)
   const dim3 grid_long(static_cast<unsigned>(
       kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(most_long, kWavesPerBlock * kNumXcd), 256))));
@@ -965,7 +965,7 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
     if (a.psw) { TBE_APPROX(true, true); }
     else { TBE_APPROX(false, true); }
   } else if (approx_short_serves(a.dtype, a.D)) {
-    // uniform tables whose rows fit a wavefront: rows of up to kShortSegment occurrences go through
+    // uniform tables whose rows fit a wavefront: rows of up to kApproxShortSegment occurrences go through
     // the exact update's position-balanced short-row kernel in its per-lookup form, the others
     // (queued by it) get a wavefront each
     UpdateArgs ua{};

@@ -38,8 +38,14 @@ int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts
                   bool clear_queue_counters = false);
 
 // Segments of more than kShortSegment occurrences leave the lane-group path and are reduced by
-// whole wavefronts in chunks of at most kChunkLen occurrences.
-constexpr int kShortSegment = 16;
+// whole wavefronts in chunks of at most kChunkLen occurrences.  (Measured, fused forward + backward
+// of 5.2 M lookups: 64 tables of 100 k fp32 rows of 128, Zipf 1.05 / 32 tables of 1 M fp16 rows of
+// 64, Zipf 1.2, weighted Adagrad -- threshold 16: 1.118 / 0.540 ms, 32: 1.118 / 0.532, 64: 1.114 /
+// 0.525, 128: 1.105 / 0.522, 256: 1.102 / 0.525.)  The approximate (per-lookup) update, whose
+// lane groups walk a row's occurrences one after the other, hands rows over from
+// kApproxShortSegment occurrences on.
+constexpr int kShortSegment = 128;
+constexpr int kApproxShortSegment = 16;
 constexpr int kChunkLen = 256;
 // Integers kept next to the number of unique rows (all zeroed when the segments are found):
 // [1] long rows, [3] partial rows, [8..15] chunk records queued by each XCD.
@@ -53,13 +59,15 @@ constexpr int kApproxHuge = 256;   // occurrences from which on the approximate 
 // those of its eighth plus those of one segment of any length.
 inline int64_t chunk_queue_capacity(int64_t n) {
   const int64_t eighth = (n + 7) / 8 + 2048;
-  return eighth / (kShortSegment + 1) + eighth / kChunkLen + n / kChunkLen + 8;
+  // (sized for the smaller of the two thresholds: the approximate update of fp32 rows queues its
+  // chunk records here too)
+  return eighth / (kApproxShortSegment + 1) + eighth / kChunkLen + n / kChunkLen + 8;
 }
 
 // Room of one XCD's queue of rows that the approximate update's short-row kernel leaves to the
-// wavefront-per-row kernel: the rows of more than kShortSegment occurrences that start in the
+// wavefront-per-row kernel: the rows of more than kApproxShortSegment occurrences that start in the
 // XCD's eighth of the sorted positions (an eighth is rounded up to whole workgroups of tiles).
-inline int64_t approx_long_queue_capacity(int64_t n) { return (n / 8 + 8192) / (kShortSegment + 1) + 2; }
+inline int64_t approx_long_queue_capacity(int64_t n) { return (n / 8 + 8192) / (kApproxShortSegment + 1) + 2; }
 // (behind the eight queues: the rows of more than kApproxHuge occurrences, at most n / 257 + 1)
 
 enum { kOptSgd = 0, kOptAdagrad = 1 };
@@ -93,7 +101,7 @@ struct UpdateArgs {
 };
 
 int segment_update(const UpdateArgs &args, hipStream_t stream);
-// The approximate row-wise Adagrad for rows of at most kShortSegment occurrences, with the
+// The approximate row-wise Adagrad for rows of at most kApproxShortSegment occurrences, with the
 // position-balanced tiles of the exact update (rows no wider than 64 vectors: approx_short_serves);
 // longer rows are appended to `queue` as unique-row numbers, their count in args.counters[1].
 bool approx_short_serves(int32_t dtype, int32_t D);

@@ -107,7 +107,7 @@ struct LongRecord {    // 16 bytes: a segment cut into several chunks
 // (batched_embedding_backward_adagrad_approx_kernel_1, tbe.cu:648-704) instead of one update with the
 // summed gradient -- every occurrence, in position order, adds its bag's ||grad||^2 (times its
 // squared weight) to the state and moves the row by its own multiplier.  Segments longer than
-// kShortSegment are then queued as unique-row numbers for tbe_approx.hip's wavefront-per-row kernel.
+// kApproxShortSegment are then queued as unique-row numbers for tbe_approx.hip's wavefront-per-row kernel.
 // APPROX_SUM (with APPROX, rows without per-sample weights in fp32 / fp64): longer segments take the
 // chunk queue like the exact update's, for update_chunks_kernel's per-lookup form.
 template <typename T, int VEC, int CHUNKS, int OPT, bool WEIGHTED, int UNROLL, bool APPROX = false,
@@ -129,7 +129,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
   static_assert(!APPROX || OPT == kOptAdagrad, "the approximate update is a row-wise Adagrad");
 
   constexpr int kTilePositions = tile_positions(CHUNKS, SMALL);
-  constexpr int kStageCap = kTilePositions + kShortSegment;  // occurrences staged in LDS per wavefront
+  constexpr int kShort = APPROX ? kApproxShortSegment : kShortSegment;  // longest segment reduced here
+  constexpr int kStageCap = kTilePositions + kShort;  // occurrences staged in LDS per wavefront
   __shared__ int32_t s_bounds[kWavesPerBlock][kTilePositions + 1];
   __shared__ int32_t s_keys[kWavesPerBlock][kTilePositions];
   __shared__ int32_t s_grow[kWavesPerBlock][kStageCap];
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const int len = seg_end - seg_begin;
     const int32_t key = s_keys[wave][j];
     if constexpr (APPROX && !APPROX_SUM) {
-      if (len > kShortSegment) {
+      if (len > kShort) {
         // (one queue per XCD, like the chunk records: `max_chunks` is the room of all eight)
         // and one behind them for the rows of very many occurrences
         if (c == 0) {
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
         continue;
       }
     }
-    if (len > kShortSegment) {
+    if (len > kShort) {
       // Hand the segment to the chunk queue.
       const int nch = (len + kChunkLen - 1) / kChunkLen;
       int first_chunk = 0, first_partial = -1;
@@ -275,7 +276,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
       for (int q = 0; q < UNROLL; ++q) {
         const int i = i0 + q;
         if (i < seg_end) {
-          // a short segment starts inside the tile and has at most kShortSegment occurrences,
+          // a short segment starts inside the tile and has at most kShort occurrences,
           // so all of them are among the staged ones
           const int rel = i - tile_begin;
           const int64_t grow = s_grow[wave][rel];
@@ -831,7 +832,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
 }
 
 // The short-row kernel alone, in its per-lookup (approximate Adagrad) form; rows of more than
-// kShortSegment occurrences are left in `queue`: eight queues of approx_long_queue_capacity() row
+// kApproxShortSegment occurrences are left in `queue`: eight queues of approx_long_queue_capacity() row
 // numbers, one per XCD, their lengths in counters[kChunkQueueCount ...].
 template <typename T, int VEC, int CHUNKS, bool WEIGHTED>
 void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *queue, hipStream_t stream) {

@@ -290,10 +290,14 @@ def test_backward_matches_embeddingbag_fixture(name):
         assert_close(got["grad_psw"], g["expected_grad_psw"], tol)
 
 
-@pytest.mark.parametrize("dtype,D,occurrences", [(np.float32, 128, 17), (np.float16, 64, 17), (np.float32, 16, 257)])
+SHORT_SEGMENT = 128  # kShortSegment of csrc/tbe_stages.h: longer segments leave the short-row kernel
+
+
+@pytest.mark.parametrize("dtype,D,occurrences", [(np.float32, 128, SHORT_SEGMENT + 1), (np.float16, 64, SHORT_SEGMENT + 1),
+                                                 (np.float32, 16, 257)])
 def test_queues_hold_the_most_chunk_records_a_batch_can_produce(oracle, dtype, D, occurrences):
-    """Every row occurs 17 times (the most segments that leave the short-row kernel: one chunk
-    record per 17 lookups) or 257 times (two chunks and a partial-row record each): the eight
+    """Every row occurs 129 times (the most segments that leave the short-row kernel: one chunk
+    record per 129 lookups) or 257 times (two chunks and a partial-row record each): the eight
     queues together receive exactly the number of records the arithmetic predicts, and nothing
     around them is overwritten (the update still matches the oracle)."""
     rs = np.random.RandomState(11)
@@ -309,7 +313,7 @@ def test_queues_hold_the_most_chunk_records_a_batch_can_produce(oracle, dtype, D
     lengths = np.diff(ref["segment_starts"])
     assert (lengths == occurrences).sum() >= T * (rows - 1)
     counters = got["views"]["counters"]
-    assert counters[8:16].sum() == np.ceil(lengths[lengths > 16] / 256).sum()
+    assert counters[8:16].sum() == np.ceil(lengths[lengths > SHORT_SEGMENT] / 256).sum()
     assert counters[1] == (lengths > 256).sum()
     _check(p, w, st, ref, got, "sgd")
 
@@ -318,7 +322,7 @@ def test_queues_hold_the_most_chunk_records_a_batch_can_produce(oracle, dtype, D
 @pytest.mark.parametrize("mode", ["sgd", "adagrad_weighted"])
 def test_hot_rows_take_the_chunked_path(oracle, dtype, D, mode):
     """Segments far longer than one lane group handles: one row receives ~70 % of 60 k lookups,
-    others land on both sides of the 16- and 256-occurrence thresholds."""
+    others land on both sides of the 128- and 256-occurrence thresholds."""
     rs = np.random.RandomState(5)
     T, E, B, L = 2, 50, 3000, 10
     p = make_problem(9, T, E, D, B, L, dtype, ragged=False, weighted=mode.endswith("weighted"))
@@ -330,11 +334,11 @@ def test_hot_rows_take_the_chunked_path(oracle, dtype, D, mode):
     w, st, ref, got = _run_both(oracle, p, optimizer, 0.001, 0.1)
     lengths = np.diff(ref["segment_starts"])
     assert lengths.max() > 15000 and (lengths <= 256).any() and ((lengths > 256) & (lengths < 2000)).any()
-    # rows with more than 256 occurrences are reduced in several chunks, rows with more than 16 by
+    # rows with more than 256 occurrences are reduced in several chunks, rows with more than 128 by
     # whole wavefronts: counters = [U, rows in several chunks, -, partial rows, ..., chunks queued by
     # each of the eight XCDs]
     assert got["views"]["counters"][1] == (lengths > 256).sum()
-    assert got["views"]["counters"][8:16].sum() == np.ceil(lengths[lengths > 16] / 256).sum()
+    assert got["views"]["counters"][8:16].sum() == np.ceil(lengths[lengths > SHORT_SEGMENT] / 256).sum()
     np.testing.assert_array_equal(got["views"]["positions_sorted"], ref["positions_sorted"])
     np.testing.assert_array_equal(got["views"]["segment_starts"], ref["segment_starts"])
     # The truth is the update computed in fp64 from the same inputs.  The HIP path has to be within
