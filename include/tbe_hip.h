@@ -75,6 +75,16 @@ TBE_API int tbe_profile_end(void);
 TBE_API int32_t tbe_profile_count(void);
 TBE_API int tbe_profile_get(int32_t i, const char **name, float *milliseconds);
 
+/* Benchmark aid with no counterpart in the reference: the memory system's rate for the row-access
+ * pattern of the gather and update kernels, with none of their bookkeeping.  Lane groups of
+ * row_bytes / 16 lanes visit rows[row_ids[i]] (row_bytes = 64, 128, 256 or 512; eight independent
+ * rows in flight per group) in the order of row_ids.  modify = 0: the rows are read (and
+ * state[row_ids[i]], if state is not NULL); modify = 1: every row is read, changed and written
+ * back in place, and so is its state word -- row_ids must then hold no row twice.  `sink` is 16
+ * bytes of device memory that the read-only form may write. */
+TBE_API int tbe_probe_row_access(void *rows, int32_t row_bytes, const int32_t *row_ids, int64_t num_ids,
+                                 float *state, int32_t modify, void *sink, void *stream);
+
 /* ------------------------------------------------------------------ forward
  * Pooled gather-sum:  output[b][t][:] = sum_{p in bag(t,b)} (psw[p] *) weights[table_offsets[t] + indices[p]][:]
  * Replaces batched_embedding_forward_cuda (table_batched_embeddings_cuda.cu:253-316,

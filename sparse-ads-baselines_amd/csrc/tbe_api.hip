@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kBlockThreads) void construct_offsets_kernel(
 
 extern "C" const char *tbe_last_error(void) { return tbe::g_last_error; }
 
-extern "C" int32_t tbe_abi_version(void) { return 16; }
+extern "C" int32_t tbe_abi_version(void) { return 17; }
 
 extern "C" int tbe_profile_begin(void) {
   using namespace tbe;
@@ -155,6 +155,77 @@ extern "C" int tbe_stochastic_round(const float *values, const uint32_t *random_
   hipStream_t s = static_cast<hipStream_t>(stream);
   TBE_LAUNCH("stochastic_round", s, stochastic_round_kernel, grid, dim3(kBlockThreads), values, random_words, out, n);
   return check_launch("tbe_stochastic_round");
+}
+
+namespace tbe {
+namespace {
+// Row-access probe: LANES lanes (16 bytes each) own one row at a time, as in the forward and
+// update kernels, and keep kProbeRows independent rows in flight; nothing else happens, so the
+// duration is what the memory system takes for the access pattern alone.
+constexpr int kProbeRows = 8;
+template <int LANES>
+__global__ __launch_bounds__(kBlockThreads) void probe_rows_kernel(uint4 *__restrict__ rows,
+                                                                  const int32_t *__restrict__ row_ids, int64_t n,
+                                                                  float *__restrict__ state, int modify,
+                                                                  uint4 *__restrict__ sink) {
+  constexpr int kGroups = kBlockThreads / LANES;
+  const int sub = threadIdx.x % LANES;
+  const int64_t group = static_cast<int64_t>(blockIdx.x) * kGroups + threadIdx.x / LANES;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kGroups;
+  uint4 acc = make_uint4(0, 0, 0, 0);
+  for (int64_t i0 = group * kProbeRows; i0 < n; i0 += stride * kProbeRows) {
+    int64_t row[kProbeRows];
+#pragma unroll
+    for (int k = 0; k < kProbeRows; ++k) row[k] = row_ids[min(i0 + k, n - 1)];
+    uint4 v[kProbeRows];
+    float s[kProbeRows];
+#pragma unroll
+    for (int k = 0; k < kProbeRows; ++k) {
+      v[k] = rows[row[k] * LANES + sub];
+      if (state && sub == 0) s[k] = state[row[k]];
+    }
+#pragma unroll
+    for (int k = 0; k < kProbeRows; ++k) {
+      if (modify) {
+        if (i0 + k < n) {
+          v[k].x += 1u;
+          rows[row[k] * LANES + sub] = v[k];
+          if (state && sub == 0) state[row[k]] = s[k] + 1.0f;
+        }
+      } else {
+        acc.x ^= v[k].x; acc.y ^= v[k].y; acc.z ^= v[k].z; acc.w ^= v[k].w;
+        if (state && sub == 0) acc.x ^= __float_as_uint(s[k]);
+      }
+    }
+  }
+  // keeps the loads alive; the condition does not hold for the probe's data
+  if (!modify && acc.x == 0x9e3779b9u && acc.y == 0x7f4a7c15u) sink[0] = acc;
+}
+}  // namespace
+}  // namespace tbe
+
+extern "C" int tbe_probe_row_access(void *rows, int32_t row_bytes, const int32_t *row_ids, int64_t num_ids,
+                                    float *state, int32_t modify, void *sink, void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_probe_row_access";
+  TBE_REQUIRE(rows && row_ids && sink, "%s: null pointer argument", name);
+  TBE_REQUIRE(num_ids > 0 && num_ids < INT32_MAX, "%s: num_ids out of range", name);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int lanes = row_bytes / 16;
+  const int64_t groups = ceil_div(num_ids, kProbeRows);
+  const dim3 grid(static_cast<unsigned>(std::min<int64_t>(ceil_div(groups * lanes, kBlockThreads), 256 * 64)));
+#define TBE_PROBE(L)                                                                                          \
+  case L:                                                                                                     \
+    TBE_LAUNCH("probe_rows", s, probe_rows_kernel<L>, grid, dim3(kBlockThreads), static_cast<uint4 *>(rows), \
+               row_ids, num_ids, state, modify, static_cast<uint4 *>(sink));                                  \
+    break;
+  switch (lanes * (row_bytes % 16 == 0 ? 1 : 0)) {
+    TBE_PROBE(4) TBE_PROBE(8) TBE_PROBE(16) TBE_PROBE(32)
+    default:
+      return fail(TBE_ERR_UNSUPPORTED, "%s: rows of 64, 128, 256 or 512 bytes (got %d)", name, row_bytes);
+  }
+#undef TBE_PROBE
+  return check_launch(name);
 }
 
 extern "C" int tbe_construct_offsets(const int32_t *batch_offsets_per_table,

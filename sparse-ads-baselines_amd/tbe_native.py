@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -84,6 +84,7 @@ SIGNATURES = {
     "tbe_profile_end": (ctypes.c_int, []),
     "tbe_profile_count": (_i32, []),
     "tbe_profile_get": (ctypes.c_int, [_i32, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_f32)]),
+    "tbe_probe_row_access": (ctypes.c_int, [_vp, _i32, _c_i32p, _i64, _vp, _i32, _vp, _vp]),
     "tbe_forward": (ctypes.c_int, [_vp, _i32, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp, _vp, _vp]),
     "tbe_backward_workspace_layout": (ctypes.c_int, [_i64, _i32, _i32, _i32, ctypes.POINTER(WorkspaceLayout)]),
     "tbe_backward_sgd": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p,
