@@ -350,15 +350,13 @@ def run_cached(args, w):
     slots = w["cache_slots"]
     per_step, per_kernel = [], {}
     bytes_alg = 0
-    staged_before = 0
     with tbe_native.profile() as prof:
         for i in range(total):
             indices, offsets = batches[i]
             out = module(indices, offsets)
             st = cache.stats()
             U = st["unique_rows"]
-            lay, ws = cache._plan_layout, cache._plan_ws
-            starts = ws[lay.segment_starts:lay.segment_starts + 4 * (U + 1)].view(torch.int32).long()
+            starts = cache.segment_starts().long()
             occurrences = starts[1:] - starts[:-1]
             unique_slots = cache.unique_slots()
             hit = (cache.evicted_keys() == -2) & (unique_slots >= 0) & (unique_slots < slots)
@@ -366,9 +364,6 @@ def run_cached(args, w):
             st["lookups_hit"] = int(occurrences[hit].sum())
             st["hit_rate_unique_rows"] = st["hits"] / max(U, 1)
             st["hit_rate_lookups"] = st["lookups_hit"] / max(st["lookups"], 1)
-            # staged rows of the step before that this step did not take over go back to the host now
-            st["staged_written_back"] = staged_before - st["from_staging"]
-            staged_before = st["staged"]
             out.backward(grad_output)
             if i >= args.warmup:
                 per_step.append(st)
@@ -382,19 +377,19 @@ def run_cached(args, w):
                for k, v in per_kernel.items()}
     row_bytes = D * 4
     # Rows over the host link per step.  In: inserted and staged rows are fetched once, from the host
-    # table unless the step before left them in its staging area; an uncached row is read by the forward
-    # (once per lookup; counted once) and by the update.  Out: evicted rows and the rows that the step
-    # before staged and this step did not take over are written once, an uncached row is written by the
-    # update.  One launch (cache_fill) carries the fetches and both kinds of write-back.
+    # table unless an earlier step left them in a staging area; an uncached row is read by the forward
+    # (once per lookup; counted once) and by the update.  Out: the rows of the staging area that the step
+    # releases (rows staged or evicted two steps earlier that no step has fetched again since) are
+    # written once, by the same launch (cache_fill) that carries the fetches; an uncached row is
+    # written by the update, and an evicted row without a landing row by the commit launch.
     fetched = [(st["inserted"] + st["staged"] - st["from_staging"]) * row_bytes for st in per_step]
-    written = [(st["written_back"] + st["staged_written_back"]) * row_bytes for st in per_step]
+    written = [st["written_out"] * row_bytes for st in per_step]
     link_in = [f + 2 * st["uncached"] * row_bytes for f, st in zip(fetched, per_step)]
-    link_out = [o + st["uncached"] * row_bytes for o, st in zip(written, per_step)]
+    link_out = [o + (st["uncached"] + st["no_landing_row"]) * row_bytes for o, st in zip(written, per_step)]
     mean = lambda xs: sum(xs) / max(len(xs), 1)
     steady = per_step[len(per_step) // 2:]
     fill_us = kernels.get("cache_fill", {}).get("avg_us")
     fill_in, fill_out = mean(fetched), mean(written)
-    link_achieved = (mean(link_in) + mean(link_out)) / sec / 1e9
     roofline = {
         "bound": "host-link", "kernel": "cache_fill",
         "achieved": fill_in / (fill_us * 1e-6) / 1e9 if fill_us else None,
@@ -412,11 +407,12 @@ def run_cached(args, w):
         "device_to_host_achieved": fill_out / (fill_us * 1e-6) / 1e9 if fill_us else None,
         "rows_taken_from_the_staging_area_per_step": mean([st["from_staging"] for st in per_step]),
         "whole_step": {"host_link_bytes_in": mean(link_in), "host_link_bytes_out": mean(link_out),
-                       "achieved_GBps_both_directions": link_achieved,
-                       "frac_of_one_direction_peak": link_achieved * 1e9 / HOST_LINK_PEAK,
-                       "note": "fetches and write-backs share one launch, so both directions of the link are "
-                               "busy together: the step is bounded by max(in, out)/peak plus the kernels that "
-                               "work on device memory"},
+                       "in_GBps": mean(link_in) / sec / 1e9, "out_GBps": mean(link_out) / sec / 1e9,
+                       "frac_of_peak_in": mean(link_in) / sec / HOST_LINK_PEAK,
+                       "frac_of_peak_out": mean(link_out) / sec / HOST_LINK_PEAK,
+                       "note": "bytes over the host link per step in each direction over the whole step time, "
+                               "each against one direction's peak: fetches and write-backs share one launch, so "
+                               "both directions are busy together and the step is bounded by max(in, out) / peak"},
     }
     mean_lookups = mean([st["lookups"] for st in per_step])
     result = {

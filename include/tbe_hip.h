@@ -395,15 +395,25 @@ TBE_API int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void 
  *      backing table.  A staged row thus crosses the host link once in each
  *      direction per step, however many lookups hit it (an uncached row is read
  *      once per lookup in the forward and read and written once in the backward).
- * Deferred write-back (stage_of_row given): step 6 is put off to the next tbe_cache_prepare, and
- * `rows` holds TWO staging areas that take turns (a step with an odd number stages into rows
- * [num_sets * 64 + stage_slots, num_sets * 64 + 2 * stage_slots), an even one into the area before
- * it).  In step 4 of the next call a row that is fetched again is read from the staging row that
- * still holds it instead of from the backing table, and is not written back at all (its slot or new
- * staging row holds the newer copy); the staged rows that are not fetched again are written back in
- * the same launch as the fetches, so both directions of the host link are busy at once.
+ * Deferred write-back (stage_of_row given) takes the row traffic out of the step, so that the plan
+ * of the next step can be made, and most of its rows moved, while the current step computes
+ * (tbe_cache_plan / tbe_cache_commit; tbe_cache_prepare is the two in a row).  `rows` then holds
+ * THREE staging areas that take turns by the call's `sequence` number (area = sequence mod 3):
+ *   - the decisions (1-3, 5) touch no row, so they may run as soon as the previous call's have;
+ *   - a staged row is fetched into its staging row and stays there after the update; an inserted
+ *     row is fetched into a *landing row* of the same area (its slot may still serve the step
+ *     before), and tbe_cache_commit swaps slot and landing row, so the evicted row ends up in the
+ *     staging area as well;
+ *   - whatever a staging area holds two calls later, and no later step has fetched again from
+ *     there (HBM to HBM, marked in stage_keys), goes back to the backing table in that call's fill
+ *     launch, beside its fetches: both directions of the host link are busy at once, and nothing
+ *     on the link waits for a step's kernels;
+ *   - tbe_cache_commit, on the caller's stream after the update of the step before, does what
+ *     depends on that update: fetches from the staging area of the step before, the swaps, and the
+ *     rare rows that found neither slot nor staging row nor landing row (those move over the link
+ *     on the caller's stream).
  * tbe_cache_flush writes back whatever is still pending.  Until then the backing table's copy of a
- * staged row is stale, like that of a cached row.
+ * staged or evicted row is stale, like that of a cached row.
  * The resulting tags / slots are a pure function of the key sequence, so a CPU
  * model can reproduce them bit for bit (a staged row is an uncached row of the
  * model; its staging index is the rank of the miss inside its set plus the number
@@ -416,15 +426,18 @@ typedef struct tbe_cache {
   int32_t *tags;        /* [num_sets * 64] key of the row held by each slot, -1 = empty  */
   int32_t *last_used;   /* [num_sets * 64] step of the slot's last use, 0 = never        */
   int32_t *use_count;   /* [num_sets * 64] steps that used the row since it was inserted */
-  void *rows;           /* [num_sets * 64 + stage_slots][D] cached rows, then the staging area */
+  void *rows;           /* [num_sets * 64 + stage_slots][D] cached rows, then the staging area
+                         * (three areas, [num_sets * 64 + 3 * stage_slots][D], with deferred write-back) */
   void *backing_rows;   /* device-visible address of the backing table [total_rows][D]   */
   int64_t num_sets;
   int32_t policy;       /* TBE_CACHE_LRU or TBE_CACHE_LFU                                */
   int64_t stage_slots;  /* rows of the staging area (0 = none); num_sets * 64 + stage_slots < 2^31 */
-  /* deferred write-back of staged rows (all null / 0: staged rows go back right after the update) */
-  int32_t *stage_of_row;  /* [total_rows] row of `rows` that has held the row since the last step, -1 = none;
-                           * then `rows` is [num_sets * 64 + 2 * stage_slots][D]                       */
-  int32_t *stage_keys;    /* [2 * stage_slots] key held by each staging row, -1 = none                 */
+  /* deferred write-back (all null / 0: staged rows go back right after the update) */
+  int32_t *stage_of_row;  /* [total_rows] row of `rows` (a staging row) that holds the row's newest value and
+                           * owes it to the backing table, -1 = none, < -1 = none, and the backing row is
+                           * written on the caller's stream in the step with sequence -(value + 2)      */
+  int32_t *stage_keys;    /* [3 * stage_slots] key held by each staging row, -1 = none, -(key + 2) = taken
+                           * over by a later step                                                       */
   int64_t total_rows;     /* rows of the backing table                                                 */
 } tbe_cache_t;
 
@@ -439,28 +452,62 @@ typedef struct tbe_cache_workspace_layout {
   uint64_t set_counts;     /* int32 [num_sets] misses per set                                  */
   uint64_t set_fill;       /* int32 [num_sets]  (not used)                                     */
   uint64_t set_starts;     /* int32 [num_sets + 1]                                             */
-  uint64_t stats;          /* int32 [8]: unique rows, hits, misses, inserted, written back, uncached, staged,
-                            * fetched from a staging row (deferred write-back)                  */
-  uint64_t fetch_source;   /* int32 [U]  deferred write-back: row of `rows` a fetched row comes from, -1 = backing table */
+  uint64_t stats;          /* int32 [16]: unique rows, hits, misses, inserted, evicted (slots that held a row),
+                            * uncached, staged; with deferred write-back also: fetched from a staging row,
+                            * rows the fill launch writes to the backing table, fetches left to
+                            * tbe_cache_commit, inserted rows without a landing row                */
+  uint64_t fetch_source;   /* int32 [U]  deferred write-back: row of `rows` a fetched row comes from, -1 = backing
+                            * table, -3 = backing table, by tbe_cache_commit                     */
+  uint64_t landing;        /* int32 [U]  deferred write-back: landing row of an inserted row, -1 = none */
+  uint64_t write_out;      /* int32 [stage_slots]  deferred write-back: key that each row of the released
+                            * staging area owes to the backing table, -1 = none                  */
 } tbe_cache_workspace_layout_t;
 
-TBE_API int tbe_cache_workspace_layout(int64_t num_indices, int64_t num_sets,
+TBE_API int tbe_cache_workspace_layout(int64_t num_indices, int64_t num_sets, int64_t stage_slots,
                                        tbe_cache_workspace_layout_t *layout);
 
-/* Empties the cache: tags = -1, last_used = use_count = 0 (and stage_of_row = stage_keys = -1). */
+/* Empties the cache: tags = -1, last_used = use_count = 0 (and stage_of_row = stage_keys = -1: rows that
+ * still wait in a staging area are dropped, so flush first to keep them). */
 TBE_API int tbe_cache_init(const tbe_cache_t *cache, void *stream);
 
 /* Steps 1-5 above.  `workspace` is a backward workspace (tbe_backward_workspace_layout)
  * and keeps the batch's plan for tbe_backward_cached; `cache_workspace` follows
- * tbe_cache_workspace_layout.  `side_stream` must differ from `stream`. */
+ * tbe_cache_workspace_layout.  `side_stream` must differ from `stream`.  `step` stamps the recency
+ * words and only has to grow from call to call.  `sequence` selects the staging area of deferred
+ * write-back: successive calls must pass consecutive numbers (after tbe_cache_init, or a
+ * tbe_cache_flush that left no staging area listed, any number may follow); it is ignored otherwise. */
 TBE_API int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_t total_rows,
                               int64_t max_table_rows, int32_t D,
                               const int32_t *table_offsets, int32_t T,
                               const int32_t *indices, int64_t num_indices,
-                              const int32_t *offsets, int32_t B, int32_t step,
+                              const int32_t *offsets, int32_t B, int32_t step, int32_t sequence,
                               void *workspace, uint64_t workspace_bytes,
                               void *cache_workspace, uint64_t cache_workspace_bytes,
                               void *stream, void *side_stream);
+
+/* tbe_cache_prepare in two parts, for deferred write-back only, so that a batch can be planned
+ * while the batch before it still computes.  tbe_cache_plan makes the decisions on `plan_stream`
+ * and then, on `link_stream`, moves the rows that do not depend on the step before;
+ * tbe_cache_commit finishes the step on the stream that runs the forward and backward kernels.
+ * Ordering is the caller's: a plan's kernels must follow (a) the previous call's tbe_cache_plan,
+ * (b) the tbe_cache_commit of the batch two calls back and (c) the last use of the two
+ * workspaces; tbe_cache_commit of a batch must follow its tbe_cache_plan on both streams, the
+ * update of the batch before it, and precede its own forward.  With the calls of one cache issued
+ * in batch order from one host thread on one stream, that is: make `plan_stream` wait for that
+ * stream when tbe_cache_plan is called, and make that stream wait for `link_stream` before
+ * tbe_cache_commit.  The workspaces of a planned batch must stay untouched until its backward. */
+TBE_API int tbe_cache_plan(const tbe_cache_t *cache, int32_t dtype, int64_t total_rows,
+                           int64_t max_table_rows, int32_t D,
+                           const int32_t *table_offsets, int32_t T,
+                           const int32_t *indices, int64_t num_indices,
+                           const int32_t *offsets, int32_t B, int32_t step, int32_t sequence,
+                           void *workspace, uint64_t workspace_bytes,
+                           void *cache_workspace, uint64_t cache_workspace_bytes,
+                           void *plan_stream, void *link_stream);
+TBE_API int tbe_cache_commit(const tbe_cache_t *cache, int32_t dtype, int32_t D, int32_t T,
+                             int64_t num_indices, int32_t sequence,
+                             void *workspace, uint64_t workspace_bytes,
+                             void *cache_workspace, uint64_t cache_workspace_bytes, void *stream);
 
 /* tbe_forward with every row read through lookup_slots (cache slot or backing table). */
 TBE_API int tbe_forward_cached(const tbe_cache_t *cache, int32_t dtype, int32_t D,
@@ -484,8 +531,14 @@ TBE_API int tbe_backward_cached(int32_t optimizer, const void *grad_output, cons
                                 void *workspace, uint64_t workspace_bytes,
                                 const int32_t *unique_slots, void *stream);
 
-/* Writes every resident row back to the backing table (the cache stays valid). */
-TBE_API int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t D, void *stream);
+/* Writes every resident row, and every row waiting in a staging area, back to the backing table (the
+ * cache stays valid).  `stream` must be ordered behind the streams of earlier tbe_cache_plan calls, and a
+ * planned batch must have been committed.  Deferred write-back: the last `live_sequences` planned batches
+ * (sequence numbers last_sequence, last_sequence - 1, ...) have not had their update yet; their staging
+ * areas are written out as they are and stay listed, because that update changes their rows again.  With
+ * live_sequences = 0 every staging area is empty afterwards and any sequence number may follow. */
+TBE_API int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t D, uint32_t live_sequences,
+                            int32_t last_sequence, void *stream);
 
 /* ------------------------------------------------- interleaved [E][T][D] tables
  * The older sparse_embedding_cuda kernels keep all tables in one [E][T][D] array and number

@@ -5,16 +5,26 @@
 // include/tbe_hip.h.  Per step:
 //   lookup   one wavefront per unique row: ballot match -> slot, mark used; misses count per set
 //   scan     exclusive scan of the per-set miss counts
-//   group    misses written into their set's range of miss_list (integer atomics; order inside
-//            a range is irrelevant because the inserting wavefront picks the smallest row first)
+//   group    misses written into their set's range of miss_list (a stable sort by set)
 //   insert   one wavefront per set: for each missing row in ascending order, victim = lowest
 //            (priority, way) among slots not used in this step (wavefront min + ballot)
-//   fill     (side stream) write back the evicted row, fetch the new row over the host link
-//            (deferred write-back, cache->stage_of_row: or from the staging row that has held it
-//            since the step before; beside it, in the same launch, the rows staged by the step
-//            before that this step does not fetch go back to the backing table)
 //   locate   slot of every lookup position, for the forward gather
 // Every decision is a function of integers only, so the tags after a step are reproducible.
+//
+// Row traffic.  Without deferred write-back one launch on the side stream writes back each evicted
+// row and fetches each new row into its slot or staging row, and the staged rows go home after the
+// update.  With deferred write-back (cache->stage_of_row) the decisions above touch no row, so the
+// plan of step x+1 can be made, and most of its rows moved, while step x still computes:
+//   resolve  where every fetched row comes from (the backing table, or a staging row that still
+//            holds its newest value) and where it lands: a staged row in its staging row, an
+//            inserted row in a *landing* row of the same area, because its slot may still serve the
+//            step before
+//   retire   the list of rows of the oldest of the three staging areas that nobody took over
+//   fill     (link stream) the fetches whose source is final, and that list back to the host
+//   commit   (caller's stream, after the update of the step before) the fetches whose source that
+//            update wrote, and slot <-> landing row swaps: the new row enters its slot, the evicted
+//            row waits in the landing row for the fill launch two steps later
+// so nothing the host link carries waits for, or is waited for by, the kernels of a step.
 
 #include <algorithm>
 
@@ -39,7 +49,13 @@ __device__ __forceinline__ uint32_t cache_set_of(uint32_t key, uint32_t num_sets
 }
 
 enum { kStatUnique = 0, kStatHits, kStatMisses, kStatInserted, kStatWrittenBack, kStatUncached, kStatStaged,
-       kStatFromStaging };
+       kStatFromStaging, kStatWrittenOut, kStatLate, kStatNoLanding, kStatCount = 16 };
+
+// Deferred write-back: three staging areas take turns by the sequence number of the step.
+constexpr int kAreas = 3;
+__host__ __device__ inline int64_t area_of(int64_t sequence) { return ((sequence % kAreas) + kAreas) % kAreas; }
+// stage_of_row value "the backing row is written by the caller's stream during step `sequence`"
+__host__ __device__ inline int32_t host_written_mark(int32_t sequence) { return -(2 + sequence); }
 
 __global__ __launch_bounds__(kBlockThreads) void cache_fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
@@ -162,11 +178,11 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ set_starts,
     const int32_t *__restrict__ miss_list, int32_t *__restrict__ unique_slots,
     int32_t *__restrict__ evicted_keys, int32_t *__restrict__ stats, int64_t stage_slots,
-    int64_t stage_base) {
+    int64_t stage_base, int32_t *__restrict__ landing) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
-  int inserted = 0, written_back = 0, uncached = 0, staged = 0;
+  int inserted = 0, written_back = 0, uncached = 0, staged = 0, no_landing = 0;
   for (int64_t set = wave_id; set < num_sets; set += stride) {
     const int begin = set_starts[set];
     const int end = set_starts[set + 1];
@@ -204,6 +220,13 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
         if (lane == 0) {
           unique_slots[u] = static_cast<int32_t>(set * kWays + way);
           evicted_keys[u] = old_tag >= 0 ? old_tag : -1;
+          if (landing) {
+            // The set owns the staging indices [begin, end): its staged rows take the first ones (below),
+            // its inserted rows the last `takers`, as landing rows.
+            const int64_t index = static_cast<int64_t>(end) - takers + j0 + j;
+            landing[u] = index < stage_slots ? static_cast<int32_t>(stage_base + index) : -1;
+            if (index >= stage_slots) ++no_landing;
+          }
         }
         ++inserted;
         if (old_tag >= 0) ++written_back;
@@ -234,84 +257,135 @@ __global__ __launch_bounds__(kBlockThreads) void cache_insert_kernel(
     if (written_back) atomicAdd(&stats[kStatWrittenBack], written_back);
     if (uncached) atomicAdd(&stats[kStatUncached], uncached);
     if (staged) atomicAdd(&stats[kStatStaged], staged);
+    if (no_landing) atomicAdd(&stats[kStatNoLanding], no_landing);
   }
 }
 
-// Deferred write-back, after the step's slots are decided: where each row that this step fetches
-// comes from, and where the rows that it stages are.  A fetched row that the step before staged
-// is still in that step's staging row: fetch_source[u] = that row of `rows` (else -1: the backing
-// table), and the entry of the staging row is marked consumed (-(key + 2)) so that it is not
-// written back.  A row staged now is entered into stage_of_row / stage_keys.
+// ---------------------------------------------------------------- deferred write-back
+// stage_keys[3 * stage_slots]: per staging row, -1 = free, key >= 0 = the row holds the newest value
+// of that table row and has to go back to the backing table, -(key + 2) = it held that row until a
+// later step took it over.  stage_of_row[total_rows]: the row of `rows` (>= num_slots) whose
+// stage_keys entry names the table row, -1 = none (the backing table or a slot holds the newest
+// value), or host_written_mark(s): none, and the caller's stream writes the backing row in step s.
+//
+// fetch_source[u] for a row that step x fetches: -1 the backing table, read by the fill launch;
+// >= num_slots a staging row -- one of the area before last, whose rows are final, is read by the
+// fill launch, one of the last step's area by the commit launch, after that step's update; -3 the
+// backing table, read by the commit launch (the last step writes that row on the caller's stream).
+
+// After the step's slots are decided: sources and destinations of the rows it fetches.
 __global__ __launch_bounds__(kBlockThreads) void cache_resolve_kernel(
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
     const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
-    const int32_t *__restrict__ evicted_keys, int32_t *__restrict__ stage_of_row,
-    int32_t *__restrict__ stage_keys, int32_t *__restrict__ fetch_source, int64_t num_slots,
+    const int32_t *__restrict__ evicted_keys, const int32_t *__restrict__ landing,
+    int32_t *__restrict__ stage_of_row, int32_t *__restrict__ stage_keys,
+    int32_t *__restrict__ fetch_source, int64_t num_slots, int64_t stage_slots, int32_t sequence,
     int32_t *__restrict__ stats) {
   const int U = counters[0];
-  int from_staging = 0;
+  const int64_t final_area = num_slots + area_of(sequence - 2) * stage_slots;  // rows nobody updates any more
+  int from_staging = 0, late = 0;
   for (int64_t u = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; u < U;
        u += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    if (evicted_keys[u] == -2) continue;  // a hit, or a row left in the backing table
-    const int32_t key = keys_sorted[segment_starts[u]];
+    const int32_t evicted = evicted_keys[u];
     const int32_t slot = unique_slots[u];
+    if (evicted == -2 && slot >= 0) continue;  // a hit
+    const int32_t key = keys_sorted[segment_starts[u]];
     const int32_t held = stage_of_row[key];
-    fetch_source[u] = held;
-    if (held >= 0) {
-      stage_keys[held - num_slots] = -(key + 2);
-      ++from_staging;
+    const bool held_final = held >= final_area && held < final_area + stage_slots;
+    if (evicted == -2) {
+      // Left in the backing table for this step: forward and update address the backing row.  Its
+      // newest value may still sit in a staging row.  One of the oldest area goes home in this
+      // step's fill launch anyway (the entry is left as it is); one of the last step's area is
+      // copied home by the commit launch.
+      fetch_source[u] = (held >= 0 && !held_final) ? held : -1;
+      if (held >= 0 && !held_final) stage_keys[held - num_slots] = -(key + 2);
+      stage_of_row[key] = host_written_mark(sequence);
+      continue;
     }
-    if (slot >= num_slots) {
+    const bool staged = slot >= num_slots;
+    const int32_t land = staged ? slot : landing[u];
+    int32_t source = -1;
+    if (held >= 0) {
+      if (land < 0 && held_final) {
+        // an inserted row without a landing row is fetched by the commit launch; by then the oldest
+        // area may be in use again, so its row goes home with the fill launch and is read from there
+        source = -3;
+        ++late;
+      } else {
+        source = held;
+        stage_keys[held - num_slots] = -(key + 2);
+        ++from_staging;
+        if (!held_final) ++late;
+      }
+    } else if (held == host_written_mark(sequence - 1) || land < 0) {
+      source = -3;
+      ++late;
+    }
+    fetch_source[u] = source;
+    if (staged) {
       stage_of_row[key] = slot;
       stage_keys[slot - num_slots] = key;
-    } else if (held >= 0) {
+    } else {
       stage_of_row[key] = -1;  // the row lives in a slot of the cache now
+      if (evicted >= 0) {
+        if (land >= 0) {  // the commit launch moves the evicted row into the landing row
+          stage_of_row[evicted] = land;
+          stage_keys[land - num_slots] = evicted;
+        } else {          // or straight to the backing table
+          stage_of_row[evicted] = host_written_mark(sequence);
+        }
+      }
     }
   }
-  for (int m = kWave / 2; m > 0; m >>= 1) from_staging += __shfl_xor(from_staging, m, kWave);
-  if ((threadIdx.x & (kWave - 1)) == 0 && from_staging) atomicAdd(&stats[kStatFromStaging], from_staging);
+  for (int m = kWave / 2; m > 0; m >>= 1) {
+    from_staging += __shfl_xor(from_staging, m, kWave);
+    late += __shfl_xor(late, m, kWave);
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    if (from_staging) atomicAdd(&stats[kStatFromStaging], from_staging);
+    if (late) atomicAdd(&stats[kStatLate], late);
+  }
+}
+
+// The oldest staging area is released: what its rows still owe the backing table is listed for
+// the fill launch (write_out[i] = key, or -1), its entries are emptied, and stage_of_row forgets
+// the rows it held.
+__global__ __launch_bounds__(kBlockThreads) void cache_retire_stage_kernel(
+    int32_t *__restrict__ stage_of_row, int32_t *__restrict__ old_stage_keys, int64_t old_stage_base,
+    int64_t stage_slots, int32_t *__restrict__ write_out, int32_t *__restrict__ stats) {
+  int pending = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < stage_slots;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int32_t entry = old_stage_keys[i];
+    if (write_out) write_out[i] = entry >= 0 ? entry : -1;
+    if (entry == -1) continue;
+    const int32_t key = entry >= 0 ? entry : -(entry + 2);
+    if (stage_of_row[key] == old_stage_base + i) stage_of_row[key] = -1;
+    old_stage_keys[i] = -1;
+    if (entry >= 0) ++pending;
+  }
+  for (int m = kWave / 2; m > 0; m >>= 1) pending += __shfl_xor(pending, m, kWave);
+  if (stats && (threadIdx.x & (kWave - 1)) == 0 && pending) atomicAdd(&stats[kStatWrittenOut], pending);
 }
 
 // One wavefront per row; rows move as 8-byte units (row_units = D * element size / 8).
-// fetch_source (deferred write-back): per unique row, the row of `rows` to fetch it from, or -1.
-// old_stage_keys (deferred write-back): the launch also carries the write-back of the step
-// before -- the rows of that step's staging area whose entry holds a key (not consumed, not
-// empty) go to the backing table.  Every wavefront alternates between an entry of that area
-// and a unique row of this step, so that both directions of the host link are busy at once on
-// every compute unit and neither side finishes long before the other, whatever their sizes.
-// (Measured on the 35.6 GB configuration: 57 ms per launch against 65 ms when workgroups
-// with an odd index wrote back and the others fetched.)
+// Without deferred write-back: the evicted row goes to the backing table, the new row comes into
+// the slot or the staging row.
 __global__ __launch_bounds__(kBlockThreads) void cache_fill_kernel(
     uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
     const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
-    const int32_t *__restrict__ evicted_keys, const int32_t *__restrict__ fetch_source,
-    const int32_t *__restrict__ old_stage_keys, int64_t old_stage_base, int64_t stage_slots) {
+    const int32_t *__restrict__ evicted_keys) {
   const int lane = threadIdx.x & (kWave - 1);
   const int U = counters[0];
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
-  const int64_t pending = old_stage_keys ? stage_slots : 0;
-  const int64_t items = U > pending ? U : pending;
-  for (int64_t i = wave_id; i < items; i += stride) {
-    if (i < pending) {
-      const int64_t key = old_stage_keys[i];
-      if (key >= 0) {
-        const uint64_t *src = cache_rows + (old_stage_base + i) * row_units;
-        uint64_t *dst = backing_rows + key * row_units;
-        for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
-      }
-    }
-    if (i >= U) continue;
+  for (int64_t i = wave_id; i < U; i += stride) {
     const int32_t evicted = evicted_keys[i];
     if (evicted == -2) continue;
     const int64_t key = keys_sorted[segment_starts[i]];
     uint64_t *slot_row = cache_rows + static_cast<int64_t>(unique_slots[i]) * row_units;
     const uint64_t *new_row = backing_rows + key * row_units;
-    if (fetch_source) {
-      const int64_t held = fetch_source[i];
-      if (held >= 0) new_row = cache_rows + held * row_units;
-    }
     if (evicted >= 0) {
       uint64_t *old_row = backing_rows + static_cast<int64_t>(evicted) * row_units;
       for (int k = lane; k < row_units; k += kWave) old_row[k] = slot_row[k];
@@ -320,10 +394,137 @@ __global__ __launch_bounds__(kBlockThreads) void cache_fill_kernel(
   }
 }
 
-// Deferred write-back, outside a step (flush, or the check that the area a step stages into is
-// empty): the rows of a staging area that hold a key go to the backing table.  A wavefront reads
-// 64 entries at a time and copies the rows of those that hold one, so an empty area costs one
-// pass over its entries.
+// Deferred write-back, the launch on the link stream.  A wavefront takes kFillBatch rows of the
+// oldest staging area that may be owed to the backing table (write_out) and kFillBatch unique rows
+// of this step whose source may be final (the backing table, or a row of that same area) at a time:
+// one lane per row works out source and destination, then the whole wavefront moves the 2 *
+// kFillBatch rows with all loads issued before the first store.  Both directions of the host link
+// are busy at once in every wavefront, and a wavefront keeps several kilobytes in flight, so that a
+// grid of a few hundred workgroups fills the link and leaves the compute units to the kernels of
+// the step that runs beside this launch.  (A grid that occupies every wavefront slot, each
+// wavefront with one row in flight, moved the same bytes in the same time when alone, but the
+// step's own kernels then waited for its wavefronts to retire.)
+// Nothing here touches a slot or a row that the step before may still read or update.
+constexpr int kFillBatch = 4;
+__global__ __launch_bounds__(kBlockThreads) void cache_fill_deferred_kernel(
+    uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
+    const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
+    const int32_t *__restrict__ evicted_keys, const int32_t *__restrict__ landing,
+    const int32_t *__restrict__ fetch_source, const int32_t *__restrict__ write_out, int64_t old_stage_base,
+    int64_t stage_slots, int64_t num_slots) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int U = counters[0];
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  const int64_t items = U > stage_slots ? U : stage_slots;
+  for (int64_t i0 = wave_id * kFillBatch; i0 < items; i0 += stride * kFillBatch) {
+    // lanes 0 .. kFillBatch-1: a row of the released area each; the next kFillBatch lanes: a unique row each
+    const uint64_t *my_src = cache_rows;  // a harmless source for the lanes without a row to move
+    uint64_t *my_dst = nullptr;
+    if (lane < kFillBatch) {
+      const int64_t i = i0 + lane;
+      if (i < stage_slots) {
+        const int64_t key = write_out[i];
+        if (key >= 0) {
+          my_src = cache_rows + (old_stage_base + i) * row_units;
+          my_dst = backing_rows + key * row_units;
+        }
+      }
+    } else if (lane < 2 * kFillBatch) {
+      const int64_t i = i0 + lane - kFillBatch;
+      if (i < U && evicted_keys[i] != -2) {
+        const int64_t slot = unique_slots[i];
+        const int64_t land = slot >= num_slots ? slot : landing[i];
+        const int64_t source = fetch_source[i];
+        if (land >= 0) {
+          if (source == -1) {
+            my_src = backing_rows + static_cast<int64_t>(keys_sorted[segment_starts[i]]) * row_units;
+            my_dst = cache_rows + land * row_units;
+          } else if (source >= old_stage_base && source < old_stage_base + stage_slots) {
+            my_src = cache_rows + source * row_units;
+            my_dst = cache_rows + land * row_units;
+          }  // else: the commit launch fetches it
+        }
+      }
+    }
+    const uint64_t *src[2 * kFillBatch];
+    uint64_t *dst[2 * kFillBatch];
+#pragma unroll
+    for (int j = 0; j < 2 * kFillBatch; ++j) {
+      src[j] = reinterpret_cast<const uint64_t *>(__shfl(reinterpret_cast<unsigned long long>(my_src), j, kWave));
+      dst[j] = reinterpret_cast<uint64_t *>(__shfl(reinterpret_cast<unsigned long long>(my_dst), j, kWave));
+    }
+    for (int k = lane; k < row_units; k += kWave) {
+      uint64_t v[2 * kFillBatch];
+#pragma unroll
+      for (int j = 0; j < 2 * kFillBatch; ++j) v[j] = src[j][k];
+#pragma unroll
+      for (int j = 0; j < 2 * kFillBatch; ++j)
+        if (dst[j]) dst[j][k] = v[j];
+    }
+  }
+}
+
+// Deferred write-back, the launch on the caller's stream, after the fill launch and after the
+// update of the step before: the fetches that had to wait for that update, the slot <-> landing
+// row swap of every inserted row (the new row into the slot, the evicted one into the landing
+// row, or, without one, straight to the backing table), and the newest value of a row that this
+// step leaves in the backing table, if the last step's staging area still held it.
+__global__ __launch_bounds__(kBlockThreads) void cache_commit_kernel(
+    uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
+    const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
+    const int32_t *__restrict__ evicted_keys, const int32_t *__restrict__ landing,
+    const int32_t *__restrict__ fetch_source, int64_t old_stage_base, int64_t stage_slots, int64_t num_slots) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int U = counters[0];
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  for (int64_t i = wave_id; i < U; i += stride) {
+    const int32_t evicted = evicted_keys[i];
+    const int64_t slot = unique_slots[i];
+    if (evicted == -2 && slot >= 0) continue;  // a hit
+    const int64_t source = fetch_source[i];
+    const int64_t key = keys_sorted[segment_starts[i]];
+    if (evicted == -2) {
+      if (source >= 0) {
+        const uint64_t *src = cache_rows + source * row_units;
+        uint64_t *dst = backing_rows + key * row_units;
+        for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
+      }
+      continue;
+    }
+    const bool by_fill = source == -1 || (source >= old_stage_base && source < old_stage_base + stage_slots);
+    const uint64_t *late_src = source >= 0 ? cache_rows + source * row_units : backing_rows + key * row_units;
+    if (slot >= num_slots) {
+      if (!by_fill) {
+        uint64_t *dst = cache_rows + slot * row_units;
+        for (int k = lane; k < row_units; k += kWave) dst[k] = late_src[k];
+      }
+      continue;
+    }
+    const int64_t land = landing[i];
+    uint64_t *slot_row = cache_rows + slot * row_units;
+    const uint64_t *new_row = (by_fill && land >= 0) ? cache_rows + land * row_units : late_src;
+    if (evicted >= 0) {
+      uint64_t *old_row = land >= 0 ? cache_rows + land * row_units
+                                    : backing_rows + static_cast<int64_t>(evicted) * row_units;
+      for (int k = lane; k < row_units; k += kWave) {
+        const uint64_t fresh = new_row[k];
+        const uint64_t old = slot_row[k];
+        old_row[k] = old;
+        slot_row[k] = fresh;
+      }
+    } else {
+      for (int k = lane; k < row_units; k += kWave) slot_row[k] = new_row[k];
+    }
+  }
+}
+
+// Deferred write-back, outside a step (flush): the rows of the staging areas that hold a key go
+// to the backing table.  A wavefront reads 64 entries at a time and copies the rows of those that
+// hold one, so an empty area costs one pass over its entries.
 __global__ __launch_bounds__(kBlockThreads) void cache_unstage_area_kernel(
     const uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
     const int32_t *__restrict__ stage_keys, int64_t stage_base, int64_t stage_slots) {
@@ -341,21 +542,6 @@ __global__ __launch_bounds__(kBlockThreads) void cache_unstage_area_kernel(
       uint64_t *dst = backing_rows + key * row_units;
       for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
     }
-  }
-}
-
-// Deferred write-back: the staging area of the step before is released -- its entries are
-// emptied, and stage_of_row forgets the rows it held unless they have been staged again since.
-__global__ __launch_bounds__(kBlockThreads) void cache_retire_stage_kernel(
-    int32_t *__restrict__ stage_of_row, int32_t *__restrict__ old_stage_keys, int64_t old_stage_base,
-    int64_t stage_slots) {
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < stage_slots;
-       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    const int32_t entry = old_stage_keys[i];
-    if (entry == -1) continue;
-    const int32_t key = entry >= 0 ? entry : -(entry + 2);
-    if (stage_of_row[key] == old_stage_base + i) stage_of_row[key] = -1;
-    old_stage_keys[i] = -1;
   }
 }
 
@@ -402,7 +588,7 @@ __global__ __launch_bounds__(kBlockThreads) void cache_flush_kernel(
   }
 }
 
-void cache_layout(int64_t n, int64_t num_sets, tbe_cache_workspace_layout_t *l) {
+void cache_layout(int64_t n, int64_t num_sets, int64_t stage_slots, tbe_cache_workspace_layout_t *l) {
   const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
   const uint64_t ints = align_up(nn * 4, 256);
   const uint64_t sets = align_up(static_cast<uint64_t>(num_sets + 1) * 4, 256);
@@ -417,12 +603,16 @@ void cache_layout(int64_t n, int64_t num_sets, tbe_cache_workspace_layout_t *l) 
   l->set_starts = off; off += sets;
   l->stats = off; off += 256;
   l->fetch_source = off; off += ints;
+  l->landing = off; off += ints;
+  l->write_out = off; off += align_up(static_cast<uint64_t>(stage_slots > 0 ? stage_slots : 1) * 4, 256);
   l->total_bytes = off;
 }
 
 inline unsigned grid_for(int64_t work_items, int64_t per_block, int64_t cap) {
   return static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(ceil_div(work_items, per_block), cap)));
 }
+
+inline bool deferred(const tbe_cache_t *cache) { return cache->stage_of_row != nullptr && cache->stage_slots > 0; }
 
 int validate_cache(const char *name, const tbe_cache_t *cache) {
   TBE_REQUIRE(cache, "%s: null cache", name);
@@ -436,26 +626,30 @@ int validate_cache(const char *name, const tbe_cache_t *cache) {
   if (cache->stage_of_row) {
     TBE_REQUIRE(cache->stage_keys && cache->total_rows > 0 && cache->total_rows < INT32_MAX,
                 "%s: deferred write-back needs stage_keys and total_rows", name);
-    TBE_REQUIRE(cache->num_sets * kWays + 2 * cache->stage_slots < INT32_MAX, "%s: stage_slots out of range", name);
+    TBE_REQUIRE(cache->num_sets * kWays + kAreas * cache->stage_slots < INT32_MAX, "%s: stage_slots out of range",
+                name);
   }
   return TBE_OK;
 }
 
-// Deferred write-back: the rows of the staging area at `stage_base` that still wait for their
-// write-back go to the backing table, and the area is released.
-void write_back_stage(const tbe_cache_t *cache, int row_units, int64_t half, hipStream_t stream) {
-  const int64_t base = cache->num_sets * kWays + half * cache->stage_slots;
-  int32_t *keys = cache->stage_keys + half * cache->stage_slots;
+// Deferred write-back, outside a step: the rows of staging area `area` that still wait for their
+// write-back go to the backing table, and the area is released -- unless a planned batch still
+// works on it (`keep`): then its rows stay listed, since that batch's update changes them again.
+void write_back_stage(const tbe_cache_t *cache, int row_units, int64_t area, bool keep, hipStream_t stream) {
+  const int64_t base = cache->num_sets * kWays + area * cache->stage_slots;
+  int32_t *keys = cache->stage_keys + area * cache->stage_slots;
   TBE_LAUNCH("cache_unstage", stream, cache_unstage_area_kernel,
              dim3(grid_for(cache->stage_slots, kWavesPerBlock, 256 * 16)), dim3(kBlockThreads),
              static_cast<const uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units, keys,
              base, cache->stage_slots);
+  if (keep) return;
   TBE_LAUNCH("cache_retire_stage", stream, cache_retire_stage_kernel,
              dim3(grid_for(cache->stage_slots, kBlockThreads, 1024)), dim3(kBlockThreads), cache->stage_of_row, keys,
-             base, cache->stage_slots);
+             base, cache->stage_slots, static_cast<int32_t *>(nullptr), static_cast<int32_t *>(nullptr));
 }
 
-// One event per calling thread, used to order the two streams.
+// One event per calling thread and purpose, used to order two streams: it is waited for right
+// after it is recorded, so recording it again later does not disturb the earlier wait.
 hipEvent_t join_event(int which) {
   thread_local hipEvent_t events[2] = {nullptr, nullptr};
   if (!events[which]) {
@@ -464,13 +658,170 @@ hipEvent_t join_event(int which) {
   return events[which];
 }
 
+int order_after(const char *name, hipStream_t later, hipStream_t earlier, int which) {
+  if (later == earlier) return TBE_OK;
+  hipEvent_t event = join_event(which);
+  if (!event) return fail(TBE_ERR_HIP, "%s: could not create an event", name);
+  hipError_t e = hipEventRecord(event, earlier);
+  if (e == hipSuccess) e = hipStreamWaitEvent(later, event, 0);
+  if (e != hipSuccess) return fail(TBE_ERR_HIP, "%s: %s", name, hipGetErrorString(e));
+  return TBE_OK;
+}
+
+struct PlanArgs {
+  const tbe_cache_t *cache;
+  int32_t dtype;
+  int64_t total_rows, max_table_rows;
+  int32_t D;
+  const int32_t *table_offsets;
+  int32_t T;
+  const int32_t *indices;
+  int64_t num_indices;
+  const int32_t *offsets;
+  int32_t B, step, sequence;
+  void *workspace;
+  uint64_t workspace_bytes;
+  void *cache_workspace;
+  uint64_t cache_workspace_bytes;
+};
+
+int validate_plan(const char *name, const PlanArgs &a, tbe_workspace_layout_t *l, tbe_cache_workspace_layout_t *cl) {
+  if (int rc = validate_cache(name, a.cache)) return rc;
+  TBE_REQUIRE(a.T > 0 && a.B > 0, "%s: T and B must be positive (got %d, %d)", name, a.T, a.B);
+  TBE_REQUIRE(a.D > 0 && a.D % 4 == 0, "%s: D must be a positive multiple of 4 (got %d)", name, a.D);
+  TBE_REQUIRE(a.dtype >= TBE_DTYPE_F32 && a.dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, a.dtype);
+  TBE_REQUIRE(a.total_rows > 0 && a.total_rows < INT32_MAX, "%s: total_rows out of range", name);
+  TBE_REQUIRE(a.max_table_rows >= 0, "%s: max_table_rows must not be negative", name);
+  TBE_REQUIRE(a.num_indices >= 0 && a.num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(static_cast<int64_t>(a.T) * a.B < INT32_MAX, "%s: T*B out of range", name);
+  TBE_REQUIRE(a.step > 0, "%s: steps are numbered from 1 (got %d)", name, a.step);
+  TBE_REQUIRE(a.sequence >= 0 && a.sequence < INT32_MAX - 4, "%s: sequence out of range (got %d)", name, a.sequence);
+  TBE_REQUIRE(a.table_offsets && a.offsets && (a.indices || a.num_indices == 0), "%s: null pointer argument", name);
+  backward_layout(a.num_indices, a.D, a.dtype, a.T, l);
+  cache_layout(a.num_indices, a.cache->num_sets, a.cache->stage_slots, cl);
+  if (!a.workspace || a.workspace_bytes < l->total_bytes)
+    return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
+                (unsigned long long)l->total_bytes, (unsigned long long)a.workspace_bytes);
+  if (!a.cache_workspace || a.cache_workspace_bytes < cl->total_bytes)
+    return fail(TBE_ERR_WORKSPACE, "%s: cache workspace of %llu bytes needed, %llu given", name,
+                (unsigned long long)cl->total_bytes, (unsigned long long)a.cache_workspace_bytes);
+  return TBE_OK;
+}
+
+inline int32_t *i32_at(void *base, uint64_t off) { return reinterpret_cast<int32_t *>(static_cast<char *>(base) + off); }
+
+// The decisions of a step on `s` (they touch no row), then the row traffic that does not depend
+// on the step before on `link`.
+int plan_step(const char *name, const PlanArgs &a, const tbe_workspace_layout_t &l,
+              const tbe_cache_workspace_layout_t &cl, hipStream_t s, hipStream_t link) {
+  const tbe_cache_t *cache = a.cache;
+  void *ws = a.workspace, *cw = a.cache_workspace;
+  const int64_t n = a.num_indices;
+  int32_t *stats = i32_at(cw, cl.stats);
+  const dim3 block(kBlockThreads);
+  const int64_t num_sets = cache->num_sets;
+  const int64_t num_slots = num_sets * kWays;
+  const bool defer = deferred(cache);
+  const int row_units = static_cast<int>(static_cast<int64_t>(a.D) * dtype_size(a.dtype) / 8);
+  // deferred write-back: this step stages into one of three areas; the area of the step before may
+  // still be updated; the one before that is final and is released by this step
+  const int64_t stage_base = num_slots + (defer ? area_of(a.sequence) * cache->stage_slots : 0);
+  const int64_t old_area = area_of(a.sequence - 2);
+  const int64_t old_stage_base = num_slots + old_area * cache->stage_slots;
+  const int32_t *keys_sorted = i32_at(ws, l.keys_sorted);
+  const int32_t *segment_starts = i32_at(ws, l.segment_starts);
+  int32_t *counters = i32_at(ws, l.num_unique);
+
+  TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(1), block, stats, static_cast<int64_t>(kStatCount), 0);
+  if (n == 0) {
+    if (!defer) return check_launch(name);
+    TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(1), block, counters, static_cast<int64_t>(1), 0);
+  } else {
+    int rc = build_plan(l, ws, a.table_offsets, a.T, a.indices, n, a.offsets, a.B, a.total_rows, a.max_table_rows, s);
+    if (rc) return rc;
+    TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(grid_for(2 * (num_sets + 1), kBlockThreads, 1024)),
+               block, i32_at(cw, cl.set_counts), static_cast<int64_t>((cl.set_starts - cl.set_counts) / 4), 0);
+    TBE_LAUNCH("cache_lookup", s, cache_lookup_kernel, dim3(grid_for(n, kWavesPerBlock, 256 * 16)), block,
+               cache->tags, cache->last_used, cache->use_count, static_cast<uint32_t>(num_sets), a.step, keys_sorted,
+               segment_starts, counters, i32_at(cw, cl.unique_slots), i32_at(cw, cl.evicted_keys),
+               i32_at(cw, cl.miss_sets), i32_at(cw, cl.set_counts), stats);
+    TBE_LAUNCH("cache_scan_sets", s, cache_scan_sets_kernel, dim3(1), block, i32_at(cw, cl.set_counts), num_sets,
+               i32_at(cw, cl.set_starts));
+    // the missing rows grouped by set, each set's in ascending order of u: a stable sort of (set, u)
+    // over the U unique rows (hits carry the key num_sets and end up behind every set).  The
+    // sorted keys go to the slot-per-lookup array, which is written later; the sort's scratch is
+    // the plan's, free since the plan was built.
+    int bits = 1;
+    while ((int64_t{1} << bits) <= num_sets) ++bits;
+    rc = sort_pairs(i32_at(cw, cl.miss_sets), nullptr, i32_at(cw, cl.lookup_slots), i32_at(cw, cl.miss_list), n, bits,
+                    static_cast<char *>(ws) + l.sort_scratch, s, nullptr, counters);
+    if (rc) return rc;
+    TBE_LAUNCH("cache_insert", s, cache_insert_kernel, dim3(grid_for(num_sets, kWavesPerBlock, 256 * 16)), block,
+               cache->tags, cache->last_used, cache->use_count, num_sets, cache->policy, a.step, keys_sorted,
+               segment_starts, i32_at(cw, cl.set_starts), i32_at(cw, cl.miss_list), i32_at(cw, cl.unique_slots),
+               i32_at(cw, cl.evicted_keys), stats, cache->stage_slots, stage_base,
+               defer ? i32_at(cw, cl.landing) : static_cast<int32_t *>(nullptr));
+    if (defer)
+      TBE_LAUNCH("cache_resolve", s, cache_resolve_kernel, dim3(grid_for(n, kBlockThreads, 256 * 16)), block,
+                 keys_sorted, segment_starts, counters, i32_at(cw, cl.unique_slots), i32_at(cw, cl.evicted_keys),
+                 i32_at(cw, cl.landing), cache->stage_of_row, cache->stage_keys, i32_at(cw, cl.fetch_source),
+                 num_slots, cache->stage_slots, a.sequence, stats);
+  }
+  if (defer)
+    TBE_LAUNCH("cache_retire_stage", s, cache_retire_stage_kernel,
+               dim3(grid_for(cache->stage_slots, kBlockThreads, 1024)), block, cache->stage_of_row,
+               cache->stage_keys + old_area * cache->stage_slots, old_stage_base, cache->stage_slots,
+               i32_at(cw, cl.write_out), stats);
+  if (n > 0)
+    TBE_LAUNCH("cache_locate", s, cache_locate_kernel, dim3(grid_for(n, kBlockThreads, 256 * 16)), block,
+               i32_at(ws, l.positions_sorted), i32_at(ws, l.segment_ids), i32_at(cw, cl.unique_slots), n,
+               i32_at(cw, cl.lookup_slots));
+
+  // Row traffic over the host link goes to the link stream, behind the decisions.
+  if (int rc = order_after(name, link, s, 0)) return rc;
+  if (defer) {
+    const int64_t work = std::max<int64_t>(n, cache->stage_slots);
+    // One workgroup per compute unit.  Measured on 35.6 GB of host-resident tables with 6.6 M rows in and
+    // 3.9 M rows out per step: 64 / 128 / 256 / 512 / 2048 workgroups move a step's rows in 59 / 51 / 48 / 48 /
+    // 49 ms when alone, but from 384 workgroups on the kernels of the step that runs beside the launch
+    // crawl behind its outstanding host reads, and the step takes 62 / 55 / 50 / 55 / 58 ms.
+    TBE_LAUNCH("cache_fill", link, cache_fill_deferred_kernel,
+               dim3(grid_for(work, kWavesPerBlock * kFillBatch, 256)),
+               block, static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units,
+               keys_sorted, segment_starts, counters, i32_at(cw, cl.unique_slots), i32_at(cw, cl.evicted_keys),
+               i32_at(cw, cl.landing), i32_at(cw, cl.fetch_source), i32_at(cw, cl.write_out), old_stage_base,
+               cache->stage_slots, num_slots);
+  } else {
+    TBE_LAUNCH("cache_fill", link, cache_fill_kernel, dim3(grid_for(n, kWavesPerBlock, 256 * 16)), block,
+               static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units,
+               keys_sorted, segment_starts, counters, i32_at(cw, cl.unique_slots), i32_at(cw, cl.evicted_keys));
+  }
+  return check_launch(name);
+}
+
+int commit_step(const char *name, const PlanArgs &a, const tbe_workspace_layout_t &l,
+                const tbe_cache_workspace_layout_t &cl, hipStream_t s) {
+  const tbe_cache_t *cache = a.cache;
+  if (!deferred(cache) || a.num_indices == 0) return TBE_OK;
+  void *ws = a.workspace, *cw = a.cache_workspace;
+  const int64_t num_slots = cache->num_sets * kWays;
+  const int row_units = static_cast<int>(static_cast<int64_t>(a.D) * dtype_size(a.dtype) / 8);
+  TBE_LAUNCH("cache_commit", s, cache_commit_kernel, dim3(grid_for(a.num_indices, kWavesPerBlock, 256 * 16)),
+             dim3(kBlockThreads), static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows),
+             row_units, i32_at(ws, l.keys_sorted), i32_at(ws, l.segment_starts), i32_at(ws, l.num_unique),
+             i32_at(cw, cl.unique_slots), i32_at(cw, cl.evicted_keys), i32_at(cw, cl.landing),
+             i32_at(cw, cl.fetch_source), num_slots + area_of(a.sequence - 2) * cache->stage_slots, cache->stage_slots,
+             num_slots);
+  return check_launch(name);
+}
+
 }  // namespace
 
 int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int32_t *keys_sorted,
                   const int32_t *segment_starts, const int32_t *counters,
                   const int32_t *unique_slots, int64_t num_indices, hipStream_t stream) {
   if (cache->stage_slots <= 0 || num_indices == 0) return TBE_OK;
-  if (cache->stage_of_row) return TBE_OK;  // deferred: the next tbe_cache_prepare (or a flush) writes them back
+  if (cache->stage_of_row) return TBE_OK;  // deferred: a later fill launch (or a flush) writes them back
   const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
   TBE_LAUNCH("cache_unstage", stream, cache_unstage_kernel,
              dim3(grid_for(num_indices, kWavesPerBlock, 256 * 16)), dim3(kBlockThreads),
@@ -482,13 +833,14 @@ int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int3
 
 }  // namespace tbe
 
-extern "C" int tbe_cache_workspace_layout(int64_t num_indices, int64_t num_sets,
+extern "C" int tbe_cache_workspace_layout(int64_t num_indices, int64_t num_sets, int64_t stage_slots,
                                           tbe_cache_workspace_layout_t *layout) {
   using namespace tbe;
   TBE_REQUIRE(layout, "tbe_cache_workspace_layout: null layout");
   TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "tbe_cache_workspace_layout: num_indices out of range");
   TBE_REQUIRE(num_sets > 0 && num_sets * kWays < INT32_MAX, "tbe_cache_workspace_layout: num_sets out of range");
-  cache_layout(num_indices, num_sets, layout);
+  TBE_REQUIRE(stage_slots >= 0 && stage_slots < INT32_MAX, "tbe_cache_workspace_layout: stage_slots out of range");
+  cache_layout(num_indices, num_sets, stage_slots, layout);
   return TBE_OK;
 }
 
@@ -505,129 +857,76 @@ extern "C" int tbe_cache_init(const tbe_cache_t *cache, void *stream) {
     TBE_LAUNCH("cache_init", s, cache_fill_i32_kernel, dim3(grid_for(cache->total_rows, kBlockThreads, 4096)), block,
                cache->stage_of_row, cache->total_rows, -1);
     TBE_LAUNCH("cache_init", s, cache_fill_i32_kernel,
-               dim3(grid_for(2 * cache->stage_slots + 1, kBlockThreads, 4096)), block, cache->stage_keys,
-               2 * cache->stage_slots, -1);
+               dim3(grid_for(kAreas * cache->stage_slots + 1, kBlockThreads, 4096)), block, cache->stage_keys,
+               kAreas * cache->stage_slots, -1);
   }
   return check_launch("tbe_cache_init");
+}
+
+extern "C" int tbe_cache_plan(const tbe_cache_t *cache, int32_t dtype, int64_t total_rows,
+                              int64_t max_table_rows, int32_t D, const int32_t *table_offsets, int32_t T,
+                              const int32_t *indices, int64_t num_indices, const int32_t *offsets, int32_t B,
+                              int32_t step, int32_t sequence, void *workspace, uint64_t workspace_bytes,
+                              void *cache_workspace, uint64_t cache_workspace_bytes, void *plan_stream,
+                              void *link_stream) {
+  using namespace tbe;
+  const char *name = "tbe_cache_plan";
+  const PlanArgs a{cache, dtype, total_rows, max_table_rows, D, table_offsets, T, indices, num_indices, offsets, B,
+                   step, sequence, workspace, workspace_bytes, cache_workspace, cache_workspace_bytes};
+  tbe_workspace_layout_t l;
+  tbe_cache_workspace_layout_t cl;
+  if (int rc = validate_plan(name, a, &l, &cl)) return rc;
+  TBE_REQUIRE(deferred(cache), "%s: planning ahead needs deferred write-back (stage_of_row, stage_slots > 0)", name);
+  return plan_step(name, a, l, cl, static_cast<hipStream_t>(plan_stream), static_cast<hipStream_t>(link_stream));
+}
+
+extern "C" int tbe_cache_commit(const tbe_cache_t *cache, int32_t dtype, int32_t D, int32_t T,
+                                int64_t num_indices, int32_t sequence, void *workspace, uint64_t workspace_bytes,
+                                void *cache_workspace, uint64_t cache_workspace_bytes, void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_cache_commit";
+  if (int rc = validate_cache(name, cache)) return rc;
+  TBE_REQUIRE(deferred(cache), "%s: needs deferred write-back (stage_of_row, stage_slots > 0)", name);
+  TBE_REQUIRE(D > 0 && D % 4 == 0 && T > 0, "%s: bad D or T (got %d, %d)", name, D, T);
+  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(sequence >= 0, "%s: sequence out of range (got %d)", name, sequence);
+  tbe_workspace_layout_t l;
+  tbe_cache_workspace_layout_t cl;
+  backward_layout(num_indices, D, dtype, T, &l);
+  cache_layout(num_indices, cache->num_sets, cache->stage_slots, &cl);
+  TBE_REQUIRE(workspace && workspace_bytes >= l.total_bytes && cache_workspace &&
+                  cache_workspace_bytes >= cl.total_bytes,
+              "%s: the workspaces of the plan being committed are missing or too small", name);
+  const PlanArgs a{cache, dtype, 0, 0, D, nullptr, T, nullptr, num_indices, nullptr, 0, 0, sequence, workspace,
+                   workspace_bytes, cache_workspace, cache_workspace_bytes};
+  return commit_step(name, a, l, cl, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tbe_cache_prepare(const tbe_cache_t *cache, int32_t dtype, int64_t total_rows,
                                  int64_t max_table_rows, int32_t D, const int32_t *table_offsets, int32_t T,
                                  const int32_t *indices, int64_t num_indices,
-                                 const int32_t *offsets, int32_t B, int32_t step, void *workspace,
+                                 const int32_t *offsets, int32_t B, int32_t step, int32_t sequence, void *workspace,
                                  uint64_t workspace_bytes, void *cache_workspace,
                                  uint64_t cache_workspace_bytes, void *stream, void *side_stream) {
   using namespace tbe;
   const char *name = "tbe_cache_prepare";
-  if (int rc = validate_cache(name, cache)) return rc;
-  TBE_REQUIRE(T > 0 && B > 0, "%s: T and B must be positive (got %d, %d)", name, T, B);
-  TBE_REQUIRE(D > 0 && D % 4 == 0, "%s: D must be a positive multiple of 4 (got %d)", name, D);
-  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
-  TBE_REQUIRE(total_rows > 0 && total_rows < INT32_MAX, "%s: total_rows out of range", name);
-  TBE_REQUIRE(max_table_rows >= 0, "%s: max_table_rows must not be negative", name);
-  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
-  TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "%s: T*B out of range", name);
-  TBE_REQUIRE(step > 0, "%s: steps are numbered from 1 (got %d)", name, step);
-  TBE_REQUIRE(table_offsets && offsets && (indices || num_indices == 0), "%s: null pointer argument", name);
-  TBE_REQUIRE(stream != side_stream, "%s: side_stream must differ from stream", name);
+  const PlanArgs a{cache, dtype, total_rows, max_table_rows, D, table_offsets, T, indices, num_indices, offsets, B,
+                   step, sequence, workspace, workspace_bytes, cache_workspace, cache_workspace_bytes};
   tbe_workspace_layout_t l;
-  backward_layout(num_indices, D, dtype, T, &l);
   tbe_cache_workspace_layout_t cl;
-  cache_layout(num_indices, cache->num_sets, &cl);
-  if (!workspace || workspace_bytes < l.total_bytes)
-    return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
-                (unsigned long long)l.total_bytes, (unsigned long long)workspace_bytes);
-  if (!cache_workspace || cache_workspace_bytes < cl.total_bytes)
-    return fail(TBE_ERR_WORKSPACE, "%s: cache workspace of %llu bytes needed, %llu given", name,
-                (unsigned long long)cl.total_bytes, (unsigned long long)cache_workspace_bytes);
+  if (int rc = validate_plan(name, a, &l, &cl)) return rc;
+  TBE_REQUIRE(stream != side_stream, "%s: side_stream must differ from stream", name);
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipStream_t side = static_cast<hipStream_t>(side_stream);
-  char *ws = static_cast<char *>(workspace);
-  char *cw = static_cast<char *>(cache_workspace);
-  auto i32 = [](char *base, uint64_t off) { return reinterpret_cast<int32_t *>(base + off); };
-  int32_t *stats = i32(cw, cl.stats);
-  const dim3 block(kBlockThreads);
-  TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(1), block, stats, static_cast<int64_t>(8), 0);
-  const int unit_count = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
-  if (cache->stage_of_row && cache->stage_slots > 0) {
-    // deferred write-back: the area this step stages into must be empty.  It is, when steps are
-    // numbered consecutively (the step before the last released it); otherwise its rows go back now.
-    write_back_stage(cache, unit_count, step & 1, s);
-    if (num_indices == 0) write_back_stage(cache, unit_count, 1 - (step & 1), s);
-  }
-  if (num_indices == 0) return check_launch(name);
-
-  int rc = build_plan(l, workspace, table_offsets, T, indices, num_indices, offsets, B, total_rows, max_table_rows, s);
-  if (rc) return rc;
-  const int32_t *keys_sorted = i32(ws, l.keys_sorted);
-  const int32_t *segment_starts = i32(ws, l.segment_starts);
-  const int32_t *counters = i32(ws, l.num_unique);
-  const int64_t num_sets = cache->num_sets;
-  const int64_t num_slots = num_sets * kWays;
-  // deferred write-back: two staging areas take turns; this step stages into one while the rows
-  // the step before left in the other are fetched from there or written back
-  const bool deferred = cache->stage_of_row != nullptr && cache->stage_slots > 0;
-  const int64_t half = deferred ? (step & 1) : 0;
-  const int64_t stage_base = num_slots + half * cache->stage_slots;
-  const int64_t old_stage_base = num_slots + (1 - half) * cache->stage_slots;
-
-  TBE_LAUNCH("cache_zero", s, cache_fill_i32_kernel, dim3(grid_for(2 * (num_sets + 1), kBlockThreads, 1024)),
-             block, i32(cw, cl.set_counts), static_cast<int64_t>((cl.set_starts - cl.set_counts) / 4), 0);
-  TBE_LAUNCH("cache_lookup", s, cache_lookup_kernel, dim3(grid_for(num_indices, kWavesPerBlock, 256 * 16)),
-             block, cache->tags, cache->last_used, cache->use_count, static_cast<uint32_t>(num_sets), step,
-             keys_sorted, segment_starts, counters, i32(cw, cl.unique_slots), i32(cw, cl.evicted_keys),
-             i32(cw, cl.miss_sets), i32(cw, cl.set_counts), stats);
-  TBE_LAUNCH("cache_scan_sets", s, cache_scan_sets_kernel, dim3(1), block, i32(cw, cl.set_counts), num_sets,
-             i32(cw, cl.set_starts));
-  // the missing rows grouped by set, each set's in ascending order of u: a stable sort of (set, u)
-  // over the U unique rows (hits carry the key num_sets and end up behind every set).  The
-  // sorted keys go to the slot-per-lookup array, which is written later; the sort's scratch is
-  // the plan's, free since the plan was built.
-  {
-    int bits = 1;
-    while ((int64_t{1} << bits) <= num_sets) ++bits;
-    const int rc_sort = sort_pairs(i32(cw, cl.miss_sets), nullptr, i32(cw, cl.lookup_slots), i32(cw, cl.miss_list),
-                                   num_indices, bits, ws + l.sort_scratch, s, nullptr, counters);
-    if (rc_sort) return rc_sort;
-  }
-  TBE_LAUNCH("cache_insert", s, cache_insert_kernel, dim3(grid_for(num_sets, kWavesPerBlock, 256 * 16)), block,
-             cache->tags, cache->last_used, cache->use_count, num_sets, cache->policy, step, keys_sorted,
-             segment_starts, i32(cw, cl.set_starts), i32(cw, cl.miss_list), i32(cw, cl.unique_slots),
-             i32(cw, cl.evicted_keys), stats, cache->stage_slots, stage_base);
-  if (deferred)
-    TBE_LAUNCH("cache_resolve", s, cache_resolve_kernel, dim3(grid_for(num_indices, kBlockThreads, 256 * 16)), block,
-               keys_sorted, segment_starts, counters, i32(cw, cl.unique_slots), i32(cw, cl.evicted_keys),
-               cache->stage_of_row, cache->stage_keys, i32(cw, cl.fetch_source), num_slots, stats);
-
-  // Row traffic over the host link goes to the side stream while this stream builds the
-  // per-lookup slot table; the side stream is joined before anything reads the cached rows.
-  hipEvent_t ready = join_event(0), filled = join_event(1);
-  if (!ready || !filled) return fail(TBE_ERR_HIP, "%s: could not create events", name);
-  hipError_t e = hipEventRecord(ready, s);
-  if (e == hipSuccess) e = hipStreamWaitEvent(side, ready, 0);
-  if (e != hipSuccess) return fail(TBE_ERR_HIP, "%s: %s", name, hipGetErrorString(e));
-  const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
-  int32_t *old_stage_keys = deferred ? cache->stage_keys + (1 - half) * cache->stage_slots : nullptr;
-  TBE_LAUNCH("cache_fill", side, cache_fill_kernel,
-             dim3((deferred ? 2 : 1) * grid_for(num_indices, kWavesPerBlock, 256 * 16)), block,
-             static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units,
-             keys_sorted, segment_starts, counters, i32(cw, cl.unique_slots), i32(cw, cl.evicted_keys),
-             deferred ? i32(cw, cl.fetch_source) : static_cast<int32_t *>(nullptr), old_stage_keys, old_stage_base,
-             cache->stage_slots);
-  if (deferred)
-    TBE_LAUNCH("cache_retire_stage", side, cache_retire_stage_kernel,
-               dim3(grid_for(cache->stage_slots, kBlockThreads, 1024)), block, cache->stage_of_row, old_stage_keys,
-               old_stage_base, cache->stage_slots);
-  TBE_LAUNCH("cache_locate", s, cache_locate_kernel, dim3(grid_for(num_indices, kBlockThreads, 256 * 16)), block,
-             i32(ws, l.positions_sorted), i32(ws, l.segment_ids), i32(cw, cl.unique_slots), num_indices,
-             i32(cw, cl.lookup_slots));
-  e = hipEventRecord(filled, side);
-  if (e == hipSuccess) e = hipStreamWaitEvent(s, filled, 0);
-  if (e != hipSuccess) return fail(TBE_ERR_HIP, "%s: %s", name, hipGetErrorString(e));
-  return check_launch(name);
+  if (int rc = plan_step(name, a, l, cl, s, side)) return rc;
+  // the side stream is joined before anything reads the cached rows
+  if (int rc = order_after(name, s, side, 1)) return rc;
+  return commit_step(name, a, l, cl, s);
 }
 
-extern "C" int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t D, void *stream) {
+extern "C" int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t D, uint32_t live_sequences,
+                               int32_t last_sequence, void *stream) {
   using namespace tbe;
   if (int rc = validate_cache("tbe_cache_flush", cache)) return rc;
   TBE_REQUIRE(D > 0 && D % 4 == 0, "tbe_cache_flush: D must be a positive multiple of 4 (got %d)", D);
@@ -635,10 +934,12 @@ extern "C" int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t slots = cache->num_sets * kWays;
   const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
-  if (cache->stage_of_row && cache->stage_slots > 0) {
-    // the rows the last step staged (one of the two areas; the other is empty)
-    write_back_stage(cache, row_units, 0, s);
-    write_back_stage(cache, row_units, 1, s);
+  TBE_REQUIRE(live_sequences <= static_cast<uint32_t>(kAreas), "tbe_cache_flush: at most %d planned batches can be live",
+              kAreas);
+  if (deferred(cache)) {
+    bool keep[kAreas] = {false, false, false};
+    for (uint32_t back = 0; back < live_sequences; ++back) keep[area_of(static_cast<int64_t>(last_sequence) - back)] = true;
+    for (int64_t area = 0; area < kAreas; ++area) write_back_stage(cache, row_units, area, keep[area], s);
   }
   TBE_LAUNCH("cache_flush", s, cache_flush_kernel, dim3(grid_for(slots, kWavesPerBlock, 256 * 16)),
              dim3(kBlockThreads), cache->tags, static_cast<const uint64_t *>(cache->rows),

@@ -219,6 +219,17 @@ class TableBatchedEmbeddingBags(nn.Module):
         if self.row_cache is not None:
             self.row_cache.invalidate()
 
+    def prefetch(self, sharded_sparse_features, sharded_offsets):
+        """HOST_CACHED tables: plans the NEXT batch while the current one computes -- its sort, its
+        cache slots and most of its row traffic over the host link run on side streams.  Call it
+        before the current batch's forward for the most overlap; batches must then be given to
+        forward() in the order they were prefetched, and the two tensors must stay unchanged until
+        then.  Results are the same with and without it.  (No counterpart in the reference, whose
+        host-resident tables are read over the bus on every lookup.)"""
+        if self.row_cache is None:
+            raise RuntimeError("prefetch is for tables behind the row cache (managed=EmbeddingLocation.HOST_CACHED)")
+        self.row_cache.prefetch(self.table_offsets, sharded_sparse_features, sharded_offsets)
+
     def forward(self, sharded_sparse_features, sharded_offsets, per_sample_weights=None):
         if self.row_cache is not None:
             return CachedLookupFunction.apply(self.embedding_weights, self, sharded_sparse_features,

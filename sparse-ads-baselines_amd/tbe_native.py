@@ -67,7 +67,7 @@ class CacheWorkspaceLayout(ctypes.Structure):
 
     _fields_ = [(name, _u64) for name in (
         "total_bytes", "unique_slots", "lookup_slots", "evicted_keys", "miss_sets", "miss_list",
-        "set_counts", "set_fill", "set_starts", "stats", "fetch_source")]
+        "set_counts", "set_fill", "set_starts", "stats", "fetch_source", "landing", "write_out")]
 
 
 CACHE_WAYS = 64
@@ -115,15 +115,18 @@ SIGNATURES = {
     "tbe_backward_approx_adagrad": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
                                                    _c_i32p, _i32, _vp, _vp, _f32, _f32, _vp, _i32, _u64, _u64, _vp,
                                                    _u64, _vp]),
-    "tbe_cache_workspace_layout": (ctypes.c_int, [_i64, _i64, ctypes.POINTER(CacheWorkspaceLayout)]),
+    "tbe_cache_workspace_layout": (ctypes.c_int, [_i64, _i64, _i64, ctypes.POINTER(CacheWorkspaceLayout)]),
     "tbe_cache_init": (ctypes.c_int, [_cache_p, _vp]),
     "tbe_cache_prepare": (ctypes.c_int, [_cache_p, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32,
-                                         _i32, _vp, _u64, _vp, _u64, _vp, _vp]),
+                                         _i32, _i32, _vp, _u64, _vp, _u64, _vp, _vp]),
+    "tbe_cache_plan": (ctypes.c_int, [_cache_p, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32,
+                                      _i32, _i32, _vp, _u64, _vp, _u64, _vp, _vp]),
+    "tbe_cache_commit": (ctypes.c_int, [_cache_p, _i32, _i32, _i32, _i64, _i32, _vp, _u64, _vp, _u64, _vp]),
     "tbe_forward_cached": (ctypes.c_int, [_cache_p, _i32, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp,
                                           _c_i32p, _vp, _vp]),
     "tbe_backward_cached": (ctypes.c_int, [_i32, _vp, _cache_p, _i32, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _f32,
                                            _f32, _vp, _i32, _u64, _u64, _vp, _u64, _c_i32p, _vp]),
-    "tbe_cache_flush": (ctypes.c_int, [_cache_p, _i32, _i32, _vp]),
+    "tbe_cache_flush": (ctypes.c_int, [_cache_p, _i32, _i32, ctypes.c_uint32, _i32, _vp]),
     "tbe_host_mapped_alloc": (ctypes.c_int, [_u64, ctypes.POINTER(_vp), ctypes.POINTER(_vp)]),
     "tbe_host_mapped_free": (ctypes.c_int, [_vp]),
     "tbe_managed_alloc": (ctypes.c_int, [_u64, _i32, ctypes.POINTER(_vp)]),
@@ -172,9 +175,9 @@ def backward_workspace_layout(num_indices, D, dtype_code, T):
     return layout
 
 
-def cache_workspace_layout(num_indices, num_sets):
+def cache_workspace_layout(num_indices, num_sets, stage_slots=0):
     layout = CacheWorkspaceLayout()
-    check(load().tbe_cache_workspace_layout(num_indices, num_sets, ctypes.byref(layout)))
+    check(load().tbe_cache_workspace_layout(num_indices, num_sets, stage_slots, ctypes.byref(layout)))
     return layout
 
 

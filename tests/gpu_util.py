@@ -60,9 +60,25 @@ def gpu_backward(p, optimizer, lr, eps=0.0, state=None):
 
 
 def assert_close(got, want, tol, what=""):
-    """|got - want| <= tol * (|want| + max|want|): relative to the element, with the array's
-    scale as the floor for elements that cancel to near zero."""
+    """|got - want| <= tol * (|want| + scale).  For arrays of rows (two or more dimensions) `scale` is
+    the largest magnitude of the element's own row (last axis), so a small element is held to `tol`
+    of its row and not of some other, larger row of the array; elements of a row may cancel to
+    near zero, which is why the row is the floor.  For vectors (one value per row or lookup) the
+    floor is the vector's largest magnitude."""
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
-    scale = np.abs(want).max() if want.size else 0.0
-    np.testing.assert_allclose(got, want, rtol=tol, atol=tol * scale, err_msg=what)
+    assert got.shape == want.shape, "%s: shape %s, expected %s" % (what, got.shape, want.shape)
+    if want.size == 0:
+        return
+    if want.ndim >= 2:
+        scale = np.abs(want).max(axis=-1, keepdims=True)
+    else:
+        scale = np.abs(want).max()
+    err = np.abs(got - want)
+    bound = tol * (np.abs(want) + scale)
+    bad = ~(err <= bound)  # also catches NaN
+    if bad.any():
+        worst = np.unravel_index(np.argmax(np.where(bad, err / np.maximum(bound, 1e-300), 0.0)), want.shape)
+        raise AssertionError("%s: %d of %d elements differ by more than %g of (|element| + row scale); worst at %s: "
+                             "got %r, expected %r" % (what, int(bad.sum()), want.size, tol, worst, got[worst],
+                                                      want[worst]))

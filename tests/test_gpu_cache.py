@@ -49,7 +49,8 @@ def test_cache_state_matches_model_bit_exact(oracle, policy, num_sets):
         np.testing.assert_array_equal(cache.last_used.cpu().numpy(), model.last_used)
         np.testing.assert_array_equal(cache.use_count.cpu().numpy(), model.use_count)
         np.testing.assert_array_equal(cache.resident_keys().cpu().numpy(), model.resident())
-        assert list(cache.stats().values()) == stats.tolist() + [0, 0]  # nothing is staged without a staging area
+        got_stats = list(cache.stats().values())
+        assert got_stats[:6] == stats.tolist() and not any(got_stats[6:])  # nothing is staged without a staging area
         # per-lookup slots agree with per-unique slots
         all_keys = table_offsets[np.repeat(np.arange(T * B), np.diff(offsets)) // B] + indices
         np.testing.assert_array_equal(cache.lookup_slots.cpu().numpy(), slots[np.searchsorted(keys, all_keys)])
@@ -86,7 +87,8 @@ def test_many_misses_per_set(oracle, num_sets, stage_slots):
             # one staging row each, all different, inside this step's area
             rows_used = np.sort(got_slots[staged])
             assert np.unique(rows_used).size == rows_used.size
-            area = num_sets * 64 + (cache.step % 2) * stage_slots
+            area = cache.stage_area_base()
+            assert area == num_sets * 64 + (cache.sequence % 3) * stage_slots
             assert rows_used[0] >= area and rows_used[-1] < area + stage_slots
 
 
@@ -151,10 +153,11 @@ def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, sta
 
 @pytest.mark.parametrize("stage_slots", [4096, 7])
 def test_deferred_write_back_with_irregular_steps(stage_slots):
-    """Deferred write-back picks its staging area by the parity of the step number.  Step numbers
-    that skip (two steps of the same parity in a row), an empty batch and a flush in the middle
-    of the run must leave nothing behind: outputs, flushed table and state stay bit-identical to
-    the run on device memory, and after every flush the host table itself is complete."""
+    """Deferred write-back rotates its staging areas by the plan's sequence number, not by the step
+    number that stamps the recency words.  Step numbers that skip, an empty batch and a flush in
+    the middle of the run must leave nothing behind: outputs, flushed table and state stay
+    bit-identical to the run on device memory, and after every flush the host table itself is
+    complete."""
     rs = np.random.RandomState(11)
     T, rows, B, L, D = 3, [700, 90, 3000], 48, 9, 64
     table_offsets = dev(np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
@@ -259,7 +262,7 @@ def test_staging_leaves_cache_state_as_the_model_says(oracle, stage_slots, defer
     unchanged by staging; rows the model leaves uncached get distinct staging rows behind the
     slots (index = misses of the earlier sets + rank among the set's staged rows) until the
     staging area is full, the rest stay uncached.  With deferred write-back the steps stage into
-    two areas in turn, and a row staged again is fetched from the staging row it had."""
+    three areas in turn, and a row staged again is fetched from the staging row it had."""
     rs = np.random.RandomState(11)
     T, rows, B, L, D, num_sets = 3, [300, 5000, 40], 64, 12, 32, 2
     table_offsets = np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32)
@@ -276,7 +279,8 @@ def test_staging_leaves_cache_state_as_the_model_says(oracle, stage_slots, defer
         got = cache.unique_slots().cpu().numpy()
         staged = got >= num_sets * 64
         np.testing.assert_array_equal(np.where(staged, -1, got), slots)
-        area = num_sets * 64 + (stage_slots if deferred and cache.step % 2 else 0)   # first row of this step's area
+        area = cache.stage_area_base()   # first row of this step's area
+        assert area == num_sets * 64 + (stage_slots * (cache.sequence % 3) if deferred else 0)
         assert np.unique(got[staged]).size == staged.sum()
         assert (got[staged] >= area).all() and (got[staged] < area + stage_slots).all()
         got_evicted = cache.evicted_keys().cpu().numpy()

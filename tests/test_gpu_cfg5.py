@@ -61,9 +61,12 @@ def _check_cache_against_model(cache, model, keys, num_slots):
     return st
 
 
-def test_cfg5_scaled_down_every_step_against_oracle_and_cache_model(oracle):
+@pytest.mark.parametrize("prefetch", [False, True])
+def test_cfg5_scaled_down_every_step_against_oracle_and_cache_model(oracle, prefetch):
     """12 steps of the configuration-5 generator at reduced sizes: 26 tables of 100 ... 100 k rows,
-    512 bags per table, a 4096-slot LRU cache with a staging area twice its size."""
+    512 bags per table, a 4096-slot LRU cache with a staging area twice its size.  With `prefetch`
+    every batch is planned while the batch before it is between its forward and its backward, and
+    the flush after every step finds that planned batch waiting."""
     w = bench.make_cfg5_workload(seed=0, B=512, row_range=(1e2, 1e5), cache_slots=1 << 12, stage_slots=1 << 13)
     T, B, D = w["T"], w["B"], w["D"]
     assert w["stage_slots"] == 2 * w["cache_slots"]
@@ -74,8 +77,11 @@ def test_cfg5_scaled_down_every_step_against_oracle_and_cache_model(oracle):
     gen = torch.Generator(device=DEV).manual_seed(1)
     w_ref = module.embedding_weights.detach().cpu().numpy().copy()
     seen_staged = seen_hits = seen_written_back = 0
+    batches = [bench.draw_cfg5_batch(torch, w, step, DEV) for step in range(12)]
+    if prefetch:
+        module.prefetch(*batches[0])
     for step in range(12):
-        indices, offsets = bench.draw_cfg5_batch(torch, w, step, DEV)
+        indices, offsets = batches[step]
         lengths = (offsets[1:] - offsets[:-1])
         assert int(lengths.min()) >= 1 and int(lengths.max()) <= 100
         grad_output = torch.randn(B, T, D, device=DEV, generator=gen)
@@ -90,6 +96,8 @@ def test_cfg5_scaled_down_every_step_against_oracle_and_cache_model(oracle):
         scale = np.abs(want).max()
         np.testing.assert_allclose(out.detach().cpu().numpy(), want, rtol=1e-5, atol=1e-5 * scale,
                                    err_msg="pooled output, step %d" % step)
+        if prefetch and step + 1 < 12:
+            module.prefetch(*batches[step + 1])
         out.backward(grad_output)
         oracle.backward("sgd", go_np, w_ref, table_offsets, idx_np, off_np, w["lr"])
         module.flush_cache()
@@ -194,15 +202,16 @@ def test_host_tensor_is_released_with_its_storage():
 @pytest.mark.timeout(900)
 def test_cfg5_full_size_cached_run_equals_uncached_run_bit_for_bit(oracle):
     """Configuration 5 at its full size (69.6 M rows = 35.6 GB in pinned host memory, 2^22-slot
-    LRU cache + 2^23 staging rows, 65 536 bags per table, ~51 M lookups per step), 3 steps.  The
-    table also fits in HBM, so the same batches run on a plain device copy without a cache:
-    outputs of every step and the flushed table are bit-identical, and the set of resident rows
-    after every step equals the CPU model's."""
+    LRU cache + 3 x 2^23 staging rows, 65 536 bags per table, ~51 M lookups per step), 5 steps: two
+    planned inside the step, three planned one step ahead (RowCache.prefetch).  The table also fits
+    in HBM, so the same batches run on a plain device copy without a cache: outputs of every step
+    and the flushed table are bit-identical, and the set of resident rows after every batch's plan
+    equals the CPU model's."""
     free, _ = torch.cuda.mem_get_info()
     w = bench.make_cfg5_workload(seed=0)
     table_bytes = sum(w["E"]) * w["D"] * 4
-    if free < table_bytes + (16 << 30):
-        pytest.skip("needs %.0f GB of free HBM" % ((table_bytes + (16 << 30)) / 1e9))
+    if free < table_bytes + (30 << 30):
+        pytest.skip("needs %.0f GB of free HBM" % ((table_bytes + (30 << 30)) / 1e9))
     T, B, D = w["T"], w["B"], w["D"]
     print("cfg5 full size: allocating %.1f GB pinned + the same in HBM" % (table_bytes / 1e9), flush=True)
     module = _module(w)
@@ -212,21 +221,39 @@ def test_cfg5_full_size_cached_run_equals_uncached_run_bit_for_bit(oracle):
     model = oracle.CacheModel(w["cache_slots"] // 64, "lru")
     gen = torch.Generator(device=DEV).manual_seed(5)
     grad_output = torch.randn(B, T, D, device=DEV, generator=gen)
-    for step in range(3):
-        indices, offsets = bench.draw_cfg5_batch(torch, w, step, DEV)
-        print("cfg5 full size: step %d, %d lookups" % (step, indices.numel()), flush=True)
-        out = module(indices, offsets)
-        want = ext.forward(plain, module.table_offsets, indices, offsets, None, 200, 1, False)
-        assert torch.equal(out.detach(), want), "pooled output differs at step %d" % step
-        keys = _unique_keys(module.table_offsets, indices, offsets, T, B).cpu().numpy().astype(np.int32)
-        model.step(keys)
+    steps, plain_steps = 5, 2
+    batches = [bench.draw_cfg5_batch(torch, w, step, DEV) for step in range(steps)]
+    keys_of = lambda b: _unique_keys(module.table_offsets, b[0], b[1], T, B).cpu().numpy().astype(np.int32)
+
+    def check_model(step):
+        """the cache's decisions for batch `step` are made: tags and resident rows equal the model's"""
+        model.step(keys_of(batches[step]))
         np.testing.assert_array_equal(cache.resident_keys().cpu().numpy(), model.resident())
         np.testing.assert_array_equal(cache.tags.cpu().numpy(), model.tags)
+
+    for step in range(steps):
+        indices, offsets = batches[step]
+        print("cfg5 full size: step %d, %d lookups%s" % (step, indices.numel(),
+                                                         "" if step < plain_steps else ", planned ahead"), flush=True)
+        if step >= plain_steps and step + 1 < steps:
+            # from the third step on every batch is planned one step ahead, before this step's forward
+            module.prefetch(*batches[step + 1])
+        out = module(indices, offsets)
+        if step < plain_steps:
+            check_model(step)
+            if step + 1 == plain_steps:
+                module.prefetch(*batches[step + 1])
+                check_model(step + 1)
+        elif step + 1 < steps:
+            check_model(step + 1)
+        want = ext.forward(plain, module.table_offsets, indices, offsets, None, 200, 1, False)
+        assert torch.equal(out.detach(), want), "pooled output differs at step %d" % step
         st = cache.stats()
-        assert st["unique_rows"] == keys.size and st["staged"] > 0
+        assert st["unique_rows"] == keys_of(batches[step]).size and st["staged"] > 0
         # a staging row is numbered by the misses of the sets before it, so the area holds every
         # unplaced row once a step misses fewer rows than it has: from the second step on
         assert st["uncached"] == 0 or (step == 0 and st["misses"] > w["stage_slots"])
+        assert st["no_landing_row"] == 0 or step == 0
         out.backward(grad_output)
         ext.backward_sgd(grad_output, plain, module.table_offsets, indices, offsets, w["lr"], 200, 1, False)
         del out, want
