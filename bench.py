@@ -120,12 +120,12 @@ def make_workload(config, seed=0, tables=None):
         w = dict(T=T, E=E, D=D, B=B, fp16=False, weighted=False, optimizer="sgd" if config == 3 else None,
                  lr=0.01, eps=0.0)
     elif config == 4:
-        T, E, D, B = 32, 1000000, 64, 8192
+        T, E, D, B = tables or 32, 1000000, 64, 8192
         lengths = rs.randint(0, 41, size=T * B).astype(np.int64)
         n = int(lengths.sum())
         indices = rs.zipf(1.2, size=n) % E
-        name = ("cfg4 fwd + weighted exact row-wise Adagrad: T=32 E=1M D=64 fp16 B=8192 L~U[0,40] Zipf(1.2) "
-                "lr=0.01 eps=1e-8")
+        name = ("cfg4 fwd + weighted exact row-wise Adagrad: T=%d E=1M D=64 fp16 B=8192 L~U[0,40] Zipf(1.2) "
+                "lr=0.01 eps=1e-8" % T)
         w = dict(T=T, E=E, D=D, B=B, fp16=True, weighted=True, optimizer="adagrad", lr=0.01, eps=1e-8)
     elif config == 5:
         return make_cfg5_workload(seed)
@@ -871,7 +871,7 @@ def main():
     ap.add_argument("--rotate", type=int, default=4,
                     help="also time the step on this many pre-drawn batches taking turns (0 or 1: leave it out)")
     ap.add_argument("--tables", type=int, default=None,
-                    help="configurations 2 and 3 with another number of tables (experiments; the workload's name "
+                    help="configurations 2, 3 and 4 with another number of tables (experiments; the workload's name "
                          "says so and no committed counter summary applies)")
     ap.add_argument("--cfg5-steps", type=int, default=50,
                     help="steps of configuration 5 inside the default run, all timed, from a cold cache")

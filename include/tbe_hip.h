@@ -105,9 +105,10 @@ TBE_API int tbe_forward(const void *weights, int32_t dtype, int32_t D,
  * Byte offsets of the regions of the backward workspace.  After a backward call
  * the first five regions hold the intermediate results that the parity gates
  * inspect (all int32):
- *   keys              [N]   table_offsets[t] + indices[p]             (tbe.cu:1495); written by
- *                           the stage entry point tbe_linearize only -- the backward entry points
- *                           sort the indices table by table and leave this region untouched
+ *   keys              [N]   table_offsets[t] + indices[p]             (tbe.cu:1495); only for batches
+ *                           over more than 2048 tables, whose keys are sorted in one piece -- otherwise
+ *                           the backward entry points sort the indices table by table, nothing is
+ *                           written here and the region is 256 bytes
  *   keys_sorted       [N]   stable ascending sort of keys             (tbe.cu:1639-1655)
  *   positions_sorted  [N]   position p of each sorted key (IndexInfo.indices_idx, tbe.cu:1217)
  *   segment_starts    [U+1] first sorted position of each unique key, then N (tbe.cu:1523-1539)

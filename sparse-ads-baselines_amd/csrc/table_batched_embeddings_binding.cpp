@@ -18,6 +18,7 @@
 
 #include <algorithm>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <iterator>
 #include <utility>
@@ -103,16 +104,62 @@ void check_state(const at::Tensor &optimizer_state, const at::Tensor &weights) {
 
 // One grow-only scratch tensor per (device, stream), so that calls issued on different streams
 // of a device may overlap (the reference allocates its sort buffers per call,
-// table_batched_embeddings_cuda.cu:1618-1647).  Returned by value: the caller's handle keeps the
-// memory until its launches are enqueued, whatever another thread does to the table meanwhile.
-at::Tensor workspace(const at::Tensor &like, uint64_t bytes) {
-  static std::mutex mutex;
-  static std::map<std::pair<int, void *>, at::Tensor> held;
-  std::lock_guard<std::mutex> lock(mutex);
-  at::Tensor &ws = held[{static_cast<int>(like.get_device()), stream_of(like)}];
-  if (!ws.defined() || static_cast<uint64_t>(ws.numel()) < bytes)
-    ws = at::empty({static_cast<int64_t>(bytes + bytes / 4 + 256)}, like.options().dtype(at::kByte));
-  return ws;
+// table_batched_embeddings_cuda.cu:1618-1647).  The kMaxWorkspaces most recently used ones are
+// kept.  A call holds its tensor (by value: the memory stays until the launches are enqueued,
+// whatever happens to the table meanwhile) and the entry's lock until it returns, so two host
+// threads that drive one stream cannot interleave their launch sequences on one buffer.
+constexpr size_t kMaxWorkspaces = 8;
+struct HeldWorkspace {
+  at::Tensor tensor;
+  std::shared_ptr<std::mutex> busy = std::make_shared<std::mutex>();
+  uint64_t last_use = 0;
+};
+struct Scratch {
+  at::Tensor tensor;
+  std::shared_ptr<std::mutex> busy;
+  std::unique_lock<std::mutex> lock;
+  void *data() const { return tensor.data_ptr(); }
+  uint64_t bytes() const { return static_cast<uint64_t>(tensor.numel()); }
+};
+std::mutex g_workspaces_mutex;
+std::map<std::pair<int, void *>, HeldWorkspace> g_workspaces;
+uint64_t g_workspace_clock = 0;
+
+Scratch workspace(const at::Tensor &like, uint64_t bytes) {
+  const std::pair<int, void *> key{static_cast<int>(like.get_device()), stream_of(like)};
+  std::shared_ptr<std::mutex> busy;
+  {
+    std::lock_guard<std::mutex> lock(g_workspaces_mutex);
+    HeldWorkspace &held = g_workspaces[key];
+    held.last_use = ++g_workspace_clock;
+    busy = held.busy;
+    while (g_workspaces.size() > kMaxWorkspaces) {
+      auto oldest = g_workspaces.begin();
+      for (auto it = g_workspaces.begin(); it != g_workspaces.end(); ++it)
+        if (it->second.last_use < oldest->second.last_use) oldest = it;
+      g_workspaces.erase(oldest);
+    }
+  }
+  std::unique_lock<std::mutex> in_use(*busy);
+  std::lock_guard<std::mutex> lock(g_workspaces_mutex);
+  HeldWorkspace &held = g_workspaces[key];  // (back again if the eviction above or a release took it)
+  held.busy = busy;
+  if (!held.tensor.defined() || static_cast<uint64_t>(held.tensor.numel()) < bytes)
+    held.tensor = at::empty({static_cast<int64_t>(bytes + bytes / 4 + 256)}, like.options().dtype(at::kByte));
+  return Scratch{held.tensor, busy, std::move(in_use)};
+}
+
+// Sizes the current stream's scratch tensor ahead of time (before a graph capture on that stream).
+void reserve_workspace(at::Tensor like, int64_t bytes) {
+  TORCH_CHECK(like.is_cuda() && bytes >= 0, "reserve_workspace takes a GPU tensor (for its device) and a size");
+  c10::DeviceGuard guard(like.device());
+  (void)workspace(like, static_cast<uint64_t>(bytes));
+}
+
+// Drops every scratch tensor; work already enqueued keeps running on them.
+void release_workspaces() {
+  std::lock_guard<std::mutex> lock(g_workspaces_mutex);
+  g_workspaces.clear();
 }
 
 // Small int32 tensors whose values the host needs (table_offsets for the largest table's row
@@ -203,11 +250,11 @@ void backward_sgd(at::Tensor grad_output, at::Tensor weights, at::Tensor table_o
   grad_output = check_grad(grad_output, weights, s);
   const int32_t dtype = dtype_code(weights);
   c10::DeviceGuard guard(weights.device());
-  at::Tensor ws = workspace(weights, workspace_bytes(s, dtype));
+  Scratch ws = workspace(weights, workspace_bytes(s, dtype));
   check(tbe_backward_sgd(grad_output.data_ptr(), weights.data_ptr(), dtype, s.rows,
                          max_table_rows(table_offsets, s.rows), s.D, table_offsets.data_ptr<int32_t>(), s.T,
                          indices.data_ptr<int32_t>(), s.n, offsets.data_ptr<int32_t>(), s.B,
-                         static_cast<float>(learning_rate), ws.data_ptr(), static_cast<uint64_t>(ws.numel()),
+                         static_cast<float>(learning_rate), ws.data(), ws.bytes(),
                          stream_of(weights)));
 }
 
@@ -239,7 +286,7 @@ c10::optional<at::Tensor> backward_exact_adagrad(at::Tensor grad_output, at::Ten
   c10::DeviceGuard guard(weights.device());
   c10::optional<at::Tensor> grad_indice_weights;
   if (indice_weights.has_value()) grad_indice_weights = at::empty_like(*indice_weights);
-  at::Tensor ws = workspace(weights, workspace_bytes(s, dtype));
+  Scratch ws = workspace(weights, workspace_bytes(s, dtype));
   void *grad_psw = grad_indice_weights.has_value() ? grad_indice_weights->data_ptr() : nullptr;
   if (stochastic_rounding && weights.scalar_type() == at::kHalf) {
     const auto stream = rounding_stream(weights);
@@ -247,13 +294,13 @@ c10::optional<at::Tensor> backward_exact_adagrad(at::Tensor grad_output, at::Ten
         grad_output.data_ptr(), weights.data_ptr(), dtype, s.rows, max_table_rows(table_offsets, s.rows), s.D,
         table_offsets.data_ptr<int32_t>(), s.T, indices.data_ptr<int32_t>(), s.n, offsets.data_ptr<int32_t>(), s.B,
         ptr(indice_weights), optimizer_state.data_ptr(), static_cast<float>(learning_rate), static_cast<float>(eps),
-        grad_psw, stream.first, stream.second, ws.data_ptr(), static_cast<uint64_t>(ws.numel()), stream_of(weights)));
+        grad_psw, stream.first, stream.second, ws.data(), ws.bytes(), stream_of(weights)));
   } else {
     check(tbe_backward_exact_adagrad(
         grad_output.data_ptr(), weights.data_ptr(), dtype, s.rows, max_table_rows(table_offsets, s.rows), s.D,
         table_offsets.data_ptr<int32_t>(), s.T, indices.data_ptr<int32_t>(), s.n, offsets.data_ptr<int32_t>(), s.B,
         ptr(indice_weights), optimizer_state.data_ptr(), static_cast<float>(learning_rate), static_cast<float>(eps),
-        grad_psw, ws.data_ptr(), static_cast<uint64_t>(ws.numel()), stream_of(weights)));
+        grad_psw, ws.data(), ws.bytes(), stream_of(weights)));
   }
   return grad_indice_weights;
 }
@@ -274,7 +321,7 @@ c10::optional<at::Tensor> backward_approx_adagrad(at::Tensor grad_output, at::Te
   c10::DeviceGuard guard(weights.device());
   c10::optional<at::Tensor> grad_indice_weights;
   if (indice_weights.has_value()) grad_indice_weights = at::empty_like(*indice_weights);
-  at::Tensor ws = workspace(weights, workspace_bytes(s, dtype));
+  Scratch ws = workspace(weights, workspace_bytes(s, dtype));
   const bool rounds = stochastic_rounding && weights.scalar_type() == at::kHalf;
   std::pair<uint64_t, uint64_t> stream{0, 0};
   if (rounds) stream = rounding_stream(weights);
@@ -283,7 +330,7 @@ c10::optional<at::Tensor> backward_approx_adagrad(at::Tensor grad_output, at::Te
       table_offsets.data_ptr<int32_t>(), s.T, indices.data_ptr<int32_t>(), s.n, offsets.data_ptr<int32_t>(), s.B,
       ptr(indice_weights), optimizer_state.data_ptr(), static_cast<float>(learning_rate), static_cast<float>(eps),
       grad_indice_weights.has_value() ? grad_indice_weights->data_ptr() : nullptr, rounds ? 1 : 0, stream.first,
-      stream.second, ws.data_ptr(), static_cast<uint64_t>(ws.numel()), stream_of(weights)));
+      stream.second, ws.data(), ws.bytes(), stream_of(weights)));
   return grad_indice_weights;
 }
 
@@ -379,7 +426,7 @@ c10::optional<at::Tensor> backward_mixed(int32_t optimizer, at::Tensor grad_outp
   if (indice_weights.has_value()) grad_indice_weights = at::empty_like(*indice_weights);
   tbe_workspace_layout_t layout;
   check(tbe_backward_workspace_layout(s.n, 4, dtype, s.T, &layout));
-  at::Tensor ws = workspace(weights, layout.total_bytes);
+  Scratch ws = workspace(weights, layout.total_bytes);
   const bool rounds = stochastic_rounding && weights.scalar_type() == at::kHalf;
   std::pair<uint64_t, uint64_t> stream{0, 0};
   if (rounds) stream = rounding_stream(weights);
@@ -390,7 +437,7 @@ c10::optional<at::Tensor> backward_mixed(int32_t optimizer, at::Tensor grad_outp
                            indices.data_ptr<int32_t>(), s.n, offsets.data_ptr<int32_t>(), s.B, ptr(indice_weights),
                            optimizer_state.data_ptr(), static_cast<float>(learning_rate), static_cast<float>(eps),
                            grad_indice_weights.has_value() ? grad_indice_weights->data_ptr() : nullptr, rounds ? 1 : 0,
-                           stream.first, stream.second, ws.data_ptr(), static_cast<uint64_t>(ws.numel()),
+                           stream.first, stream.second, ws.data(), ws.bytes(),
                            stream_of(weights)));
   return grad_indice_weights;
 }
@@ -466,4 +513,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("new_managed_tensor", &new_managed_tensor, "new_managed_tensor");
   m.def("new_host_mapped_tensor", &new_host_mapped_tensor, "new_host_mapped_tensor");
   m.def("abi_version", []() { return tbe_abi_version(); }, "version of the C ABI the library exports");
+  m.def("reserve_workspace", &reserve_workspace, "sizes the current stream's scratch tensor ahead of time");
+  m.def("release_workspaces", &release_workspaces, "drops the scratch tensors the module holds");
 }

@@ -38,7 +38,8 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspac
   l->max_chunks = static_cast<int64_t>(kNumXcd * chunk_queue_capacity(static_cast<int64_t>(nn)));
   l->max_partial_rows = static_cast<int64_t>(nn / kChunkLen + nn / (kChunkLen + 1) + 2);
   uint64_t off = 0;
-  l->keys = off; off += ints;
+  // the linearized keys are only written (and sorted in one piece) for more tables than are sorted apart
+  l->keys = off; off += sort_tables(T) == T ? 256 : ints;
   l->grad_rows = off; off += ints;
   l->keys_sorted = off; off += ints;
   l->positions_sorted = off; off += ints;

@@ -6,7 +6,10 @@ its tensors, then hands raw device pointers and the current HIP stream to the
 C-ABI library (include/tbe_hip.h).  torch is used for device memory and streams
 only -- no arithmetic happens here.
 """
+import collections
+import contextlib
 import ctypes
+import threading
 import weakref
 
 import torch
@@ -16,10 +19,12 @@ import tbe_native as _native
 _DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F16,
                 torch.float64: _native.DTYPE_F64}
 
-# One grow-only scratch buffer per device for the backward pipeline (keys, sort
-# buffers, segment lists).  The reference allocates these per call
-# (table_batched_embeddings_cuda.cu:1618-1647).
-_workspaces = {}      # (device, stream handle) -> uint8 tensor
+# Grow-only scratch buffers for the backward pipeline (keys, sort buffers, segment lists), one per
+# (device, stream) that has run a backward, the MAX_WORKSPACES most recently used ones.  The
+# reference allocates these per call (table_batched_embeddings_cuda.cu:1618-1647).
+MAX_WORKSPACES = 8
+_workspaces = collections.OrderedDict()  # (device, stream handle) -> [uint8 tensor, lock]
+_workspaces_lock = threading.Lock()
 _last_workspace = {}  # device -> the one used last
 # Owners of the host-resident allocations handed out by new_*_tensor (weak), keyed by device address.
 _host_allocations = {}
@@ -84,17 +89,49 @@ def _rounding_stream(device):
     return seed & 0xFFFFFFFFFFFFFFFF, offset
 
 
+@contextlib.contextmanager
 def _workspace(device, nbytes):
     """The grow-only scratch buffer of the device's current stream, and that stream: one buffer per
-    (device, stream), so that calls issued on different streams of a device may overlap."""
+    (device, stream), so that calls issued on different streams of a device may overlap.  The
+    buffer is held for the duration of the `with` block (the call that enqueues a backward's
+    launches), so two host threads that drive one stream cannot interleave their launch sequences
+    on one buffer.  At most MAX_WORKSPACES buffers are kept: the one least recently used goes (its
+    memory returns to the allocator in the order of the stream it was allocated on, and a captured
+    graph keeps the pool it was captured into)."""
     handle = torch.cuda.current_stream(device).cuda_stream
     key = (device, handle)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    _last_workspace[device] = ws
-    return ws, ctypes.c_void_p(handle)
+    with _workspaces_lock:
+        entry = _workspaces.get(key)
+        if entry is None:
+            entry = _workspaces[key] = [None, threading.Lock()]
+        _workspaces.move_to_end(key)
+        while len(_workspaces) > MAX_WORKSPACES:
+            _workspaces.popitem(last=False)
+    with entry[1]:
+        if entry[0] is None or entry[0].numel() < nbytes:
+            entry[0] = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=device)
+        _last_workspace[device] = entry[0]
+        yield entry[0], ctypes.c_void_p(handle)
+
+
+def reserve_workspace(nbytes, device=None):
+    """Sizes the scratch buffer of `device`'s current stream for backward calls that need up to
+    `nbytes` (tbe_native.backward_workspace_layout(...).total_bytes), so that no later call on that
+    stream allocates -- e.g. before capturing a graph on it.  An eager step run on the same stream
+    has the same effect."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    with _workspace(device, int(nbytes)):
+        pass
+
+
+def release_workspaces(device=None):
+    """Drops the scratch buffers of `device` (all devices if None).  Work already enqueued keeps
+    running on them: the allocator hands the memory out again in stream order."""
+    with _workspaces_lock:
+        for key in [k for k in _workspaces if device is None or k[0] == torch.device(device)]:
+            del _workspaces[key]
+        for dev in [d for d in _last_workspace if device is None or d == torch.device(device)]:
+            del _last_workspace[dev]
 
 
 def backward_workspace(device):
@@ -199,8 +236,7 @@ def backward_sgd(grad_output, weights, table_offsets, indices, offsets, learning
     D = weights.size(1)
     code = _DTYPE_CODES[weights.dtype]
     layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
-    ws, stream = _workspace(weights.device, layout.total_bytes)
-    with torch.cuda.device(weights.device):
+    with _workspace(weights.device, layout.total_bytes) as (ws, stream), torch.cuda.device(weights.device):
         _native.check(_native.load().tbe_backward_sgd(
             _ptr(grad_output), _ptr(weights), code, weights.size(0),
             max_table_rows(table_offsets, weights.size(0)), D, _ptr(table_offsets), T,
@@ -232,8 +268,7 @@ def backward_exact_adagrad(grad_output, weights, table_offsets, indices, offsets
                  "indice_weights must be contiguous with one entry per index")
         grad_indice_weights = torch.empty(indices.shape, dtype=grad_output.dtype, device=weights.device)
     layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
-    ws, stream = _workspace(weights.device, layout.total_bytes)
-    with torch.cuda.device(weights.device):
+    with _workspace(weights.device, layout.total_bytes) as (ws, stream), torch.cuda.device(weights.device):
         if stochastic_rounding and weights.dtype == torch.float16:
             seed, offset = _rounding_stream(weights.device)
             _native.check(_native.load().tbe_backward_exact_adagrad_stochastic(
@@ -285,10 +320,9 @@ def backward_approx_adagrad(grad_output, weights, table_offsets, indices, offset
     D = weights.size(1)
     code = _DTYPE_CODES[weights.dtype]
     layout = _native.backward_workspace_layout(indices.numel(), D, code, T)
-    ws, stream = _workspace(weights.device, layout.total_bytes)
     stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
     seed, offset = _rounding_stream(weights.device) if stochastic else (0, 0)
-    with torch.cuda.device(weights.device):
+    with _workspace(weights.device, layout.total_bytes) as (ws, stream), torch.cuda.device(weights.device):
         _native.check(_native.load().tbe_backward_approx_adagrad(
             _ptr(grad_output), _ptr(weights), code, weights.size(0), max_table_rows(table_offsets, weights.size(0)),
             D, _ptr(table_offsets), T, _ptr(indices), indices.numel(), _ptr(offsets), B, _ptr(indice_weights),
@@ -376,10 +410,9 @@ def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_of
     _require(optimizer_state.dtype == state_dtype and optimizer_state.is_contiguous(),
              "optimizer_state must be contiguous %s" % state_dtype)
     layout = _native.backward_workspace_layout(indices.numel(), 4, code, T)
-    ws, stream = _workspace(weights.device, layout.total_bytes)
     stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
     seed, offset = _rounding_stream(weights.device) if stochastic else (0, 0)
-    with torch.cuda.device(weights.device):
+    with _workspace(weights.device, layout.total_bytes) as (ws, stream), torch.cuda.device(weights.device):
         _native.check(_native.load().tbe_backward_mixed(
             optimizer, _ptr(grad_output), _ptr(weights), code, _fp16_vector_width(dim_offsets), total_rows,
             max_table_rows(table_dim_offsets, None), _ptr(table_offsets), _ptr(table_dim_offsets), _ptr(dim_offsets), int(total_D), T, _ptr(indices),
@@ -502,7 +535,9 @@ def new_managed_tensor(self, sizes):
     _require(self.is_cuda and self.dtype in _TYPESTR, "prototype must be a floating GPU tensor")
     nbytes = self.element_size()
     for s in sizes:
+        _require(int(s) >= 0, "sizes must not be negative")
         nbytes *= int(s)
+    nbytes = max(nbytes, 1)  # an empty tensor still owns an allocation, as in the compiled binding
     lib = _native.load()
     ptr = ctypes.c_void_p()
     with torch.cuda.device(self.device):
@@ -521,7 +556,9 @@ def new_host_mapped_tensor(self, sizes):
     _require(self.is_cuda and self.dtype in _TYPESTR, "prototype must be a floating GPU tensor")
     nbytes = self.element_size()
     for s in sizes:
+        _require(int(s) >= 0, "sizes must not be negative")
         nbytes *= int(s)
+    nbytes = max(nbytes, 1)  # an empty tensor still owns an allocation, as in the compiled binding
     lib = _native.load()
     host, dev = ctypes.c_void_p(), ctypes.c_void_p()
     with torch.cuda.device(self.device):

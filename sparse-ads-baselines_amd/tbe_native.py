@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p

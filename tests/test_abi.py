@@ -47,7 +47,9 @@ def test_workspace_layout_is_ordered_and_sized():
             lay.partial_sums]
     assert offs == sorted(offs) and len(set(offs)) == len(offs)
     assert all(o % 256 == 0 for o in offs)
-    assert lay.grad_rows - lay.keys >= 5242880 * 4
+    assert lay.grad_rows - lay.keys == 256  # 64 tables are sorted apart: no linearized keys are kept
+    many = tbe_native.backward_workspace_layout(5242880, 128, tbe_native.DTYPE_F32, 4096)
+    assert many.grad_rows - many.keys >= 5242880 * 4  # more tables than are sorted apart: keys sorted in one piece
     assert lay.total_bytes >= lay.partial_sums + lay.max_partial_rows * 128 * 4
     assert lay.partial_sums - lay.chunk_segments >= lay.max_chunks * 32
     assert lay.total_bytes < 512 << 20

@@ -57,14 +57,21 @@ def test_captured_step_replays_like_eager(mode, dtype, D):
     # eager twins
     w_eager, st_eager = w.clone(), st.clone()
 
-    # warm-up outside the capture: grows the workspace, fills the host-side caches
+    # Warm-up outside the capture, on the stream the capture will use: the scratch buffer belongs
+    # to the (device, stream) pair, so this is what sizes the buffer the captured launches get, and
+    # it fills the host-side caches.  The capture itself then allocates no scratch.
+    capture_stream = torch.cuda.Stream()
+    capture_stream.wait_stream(torch.cuda.current_stream())
     warm_w, warm_st = w.clone(), st.clone()
-    step(warm_w, warm_st, idx, off, go, psw)
+    with torch.cuda.stream(capture_stream):
+        step(warm_w, warm_st, idx, off, go, psw)
     torch.cuda.synchronize()
+    scratch = ext.backward_workspace(torch.device(DEV))
 
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    with torch.cuda.graph(graph, stream=capture_stream):
         out_graph, g_graph = step(w, st, idx, off, go, psw)
+    assert ext.backward_workspace(torch.device(DEV)) is scratch, "the capture allocated a scratch buffer of its own"
     # the capture itself runs nothing: w and st are still the start values
     assert torch.equal(w, w_eager)
 

@@ -57,6 +57,47 @@ def test_static_scratch_backward_equals_workspace_backward(oracle):
         np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * scale)
 
 
+def test_static_scratch_backward_allocates_nothing():
+    """The property the entry point is named for: once the first call on the device has resolved the
+    array's address, a call neither takes device memory (free memory as the driver reports it is
+    unchanged, and so is what torch's allocator has reserved) nor does anything a stream capture
+    forbids -- the same call inside a capture region returns 0 and the captured graph, replayed,
+    gives the update of the eager call."""
+    p = make_problem(8, T=4, E=1500, D=64, B=256, L=16, dtype=np.float32, zipf=1.2)
+    lib = tbe_native.load()
+    code = tbe_native.DTYPE_F32
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+    go, toff, idx, off = dev(p["grad_output"]), dev(p["table_offsets"]), dev(p["indices"]), dev(p["offsets"])
+    T, D, B, n = p["T"], p["D"], p["B"], p["n"]
+    total_rows, largest = int(sum(p["rows"])), int(max(p["rows"]))
+
+    def call(w, stream):
+        return lib.tbe_backward_sgd_static(_p(go), _p(w), code, total_rows, largest, D, _p(toff), T, _p(idx), n,
+                                           _p(off), B, 0.05, ctypes.c_void_p(stream.cuda_stream))
+
+    w_eager, w_graph = dev(p["weights"]), dev(p["weights"])
+    warm = dev(p["weights"])
+    assert call(warm, torch.cuda.current_stream()) == 0  # resolves the symbol on this device
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    reserved_before = torch.cuda.memory_reserved()
+    assert call(w_eager, torch.cuda.current_stream()) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the call took device memory"
+    assert torch.cuda.memory_reserved() == reserved_before
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        rc = call(w_graph, torch.cuda.current_stream())
+    assert rc == 0, lib.tbe_last_error()
+    assert torch.equal(w_graph, dev(p["weights"])), "capturing must not run the update"
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(w_graph, w_eager)
+    assert torch.cuda.mem_get_info()[0] <= free_before  # (the graph object itself may hold memory)
+
+
 def test_static_scratch_backward_fp16_and_empty_batch():
     p = make_problem(7, T=4, E=2000, D=32, B=300, L=20, dtype=np.float16, zipf=1.2)
     _run_both(p, 0.01)
