@@ -542,15 +542,37 @@ TBE_API int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t D, 
                             int32_t last_sequence, void *stream);
 
 /* ------------------------------------------------- interleaved [E][T][D] tables
- * The older sparse_embedding_cuda kernels keep all tables in one [E][T][D] array and number
- * bags bag-major, b*T + t (sparse_embedding_cuda_kernel.cu:221-284, 349-379).  Viewed as an
- * [E*T][D] matrix this is a single table whose row for (ind, t) is ind*T + t; this entry point
- * writes those row numbers, after which tbe_forward / tbe_backward_sgd run with T = 1,
- * B = (real B)*(real T), table_offsets = {0}: output [B*T][1][D] is the [B][T][D] layout.
- * `offsets` is the flattened [B*T+1] array of bag starts.
+ * The older sparse_embedding_cuda kernels keep all tables in one [E][T][D] array, number bags
+ * bag-major (b*T + t) and bound bag (b, t) by two consecutive entries of an offsets array that is
+ * either flat [B*T+1] or [B][T+1] with offsets[b][T] == offsets[b+1][0]
+ * (sparse_embedding_cuda_kernel.cu:221-284 forward_offsets, :349-462 forward / forward_fast,
+ * :286-347 and :464-583 the fused updates; bound in sparse_embedding_cuda.cpp:255-322).
+ * offsets_row_stride = T for the flat form (dense [B][T][L] indices: offsets[i] = i*L), T + 1 for
+ * the [B][T+1] form.  The table-major kernels serve this layout through a row stride: the row of
+ * a lookup in the [E*T][D] view is idx*T + t, output and gradient are [B][T][D].  No index array
+ * is rewritten and nothing is allocated.
+ *
+ * tbe_forward_interleaved replaces sparse_embedding_cuda_forward_single / _fast_single / _offsets.
+ * tbe_backward_sgd_interleaved replaces sparse_embedding_cuda_backward_update_single / _fast_single /
+ * _offsets, made exact: every distinct row receives -lr * (sum of its gradients) once, where the
+ * reference's `weights[ind][t][d] -= lr * g` races on repeats (sparse_embedding_cuda_kernel.cu:493-497).
+ * Its workspace follows tbe_backward_interleaved_workspace_layout (at most 2048 tables): the lookups of a
+ * table are not consecutive positions here, so one pass first copies the indices into table-major
+ * order (kept in the layout's `keys` region); the batch is then sorted table by table and updated
+ * like a table-major one, with idx*T + t as the row of a lookup.  positions_sorted refers to that
+ * table-major order.
  */
-TBE_API int tbe_interleaved_rows(const int32_t *indices, int64_t num_indices, const int32_t *offsets,
-                                 int32_t T, int32_t B, int32_t *rows, void *stream);
+TBE_API int tbe_forward_interleaved(const void *weights, int32_t dtype, int64_t E, int32_t T, int32_t D,
+                                    const int32_t *indices, int64_t num_indices,
+                                    const int32_t *offsets, int32_t offsets_row_stride, int32_t B,
+                                    void *output, void *stream);
+TBE_API int tbe_backward_interleaved_workspace_layout(int64_t num_indices, int32_t D, int32_t dtype,
+                                                      int32_t T, int32_t B, tbe_workspace_layout_t *layout);
+TBE_API int tbe_backward_sgd_interleaved(const void *grad_output, void *weights, int32_t dtype, int64_t E,
+                                         int32_t T, int32_t D, const int32_t *indices, int64_t num_indices,
+                                         const int32_t *offsets, int32_t offsets_row_stride, int32_t B,
+                                         float learning_rate, void *workspace, uint64_t workspace_bytes,
+                                         void *stream);
 
 /* ------------------------------------------------------ host-resident tables
  * Pinned, device-mapped host memory (new_host_mapped_tensor,

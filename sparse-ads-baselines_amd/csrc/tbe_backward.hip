@@ -29,7 +29,10 @@ int key_bits(int64_t total_rows) {
 constexpr int32_t kMaxTablesSortedApart = 2048;
 inline int32_t sort_tables(int32_t T) { return T <= kMaxTablesSortedApart ? T : 1; }
 
-void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *l) {
+// interleaved_B > 0 (tables stored [E][T][D], B bags per table): the `keys` region holds the batch in
+// table-major order instead -- indices [n], offsets [T*B+1], then small scratch (interleaved_regions()).
+void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *l,
+                    int32_t interleaved_B = 0) {
   const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
   const uint64_t ints = align_up(nn * 4, 256);
   // a segment enters the chunk queue when it has more than kShortSegment occurrences and owns
@@ -39,7 +42,12 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspac
   l->max_partial_rows = static_cast<int64_t>(nn / kChunkLen + nn / (kChunkLen + 1) + 2);
   uint64_t off = 0;
   // the linearized keys are only written (and sorted in one piece) for more tables than are sorted apart
-  l->keys = off; off += sort_tables(T) == T ? 256 : ints;
+  l->keys = off;
+  if (interleaved_B > 0)
+    off += ints + align_up((static_cast<uint64_t>(T) * interleaved_B + 1) * 4, 256) + 2 * align_up(T * 4ull, 256) +
+           align_up(static_cast<uint64_t>(T) * interleaved_chunks_per_table(interleaved_B) * 4, 256);
+  else
+    off += sort_tables(T) == T ? 256 : ints;
   l->grad_rows = off; off += ints;
   l->keys_sorted = off; off += ints;
   l->positions_sorted = off; off += ints;
@@ -59,6 +67,29 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspac
 
 int key_bits_for(int64_t total_rows) { return key_bits(total_rows); }
 
+namespace {
+// The pieces of the `keys` region of an interleaved-tables layout.
+struct InterleavedRegions {
+  int32_t *indices_tm, *offsets_tm, *totals, *bias, *chunk_sums;
+};
+InterleavedRegions interleaved_regions(const tbe_workspace_layout_t &l, void *workspace, int64_t n, int32_t T,
+                                       int32_t B) {
+  char *base = static_cast<char *>(workspace) + l.keys;
+  const uint64_t nn = static_cast<uint64_t>(n > 0 ? n : 1);
+  InterleavedRegions r;
+  r.indices_tm = reinterpret_cast<int32_t *>(base);
+  base += align_up(nn * 4, 256);
+  r.offsets_tm = reinterpret_cast<int32_t *>(base);
+  base += align_up((static_cast<uint64_t>(T) * B + 1) * 4, 256);
+  r.totals = reinterpret_cast<int32_t *>(base);
+  base += align_up(T * 4ull, 256);
+  r.bias = reinterpret_cast<int32_t *>(base);
+  base += align_up(T * 4ull, 256);
+  r.chunk_sums = reinterpret_cast<int32_t *>(base);
+  return r;
+}
+}  // namespace
+
 void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspace_layout_t *l) {
   compute_layout(n, D, dtype, T, l);
 }
@@ -72,11 +103,24 @@ void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspa
 // then the linearized keys are written there and sorted in one piece.
 int sort_batch(const tbe_workspace_layout_t &l, void *workspace, const int32_t *table_offsets, int32_t T,
                const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B, int64_t total_rows,
-               int64_t max_table_rows, hipStream_t stream) {
+               int64_t max_table_rows, hipStream_t stream, int32_t interleaved_offsets_stride) {
   char *ws = static_cast<char *>(workspace);
   int32_t *keys_sorted = reinterpret_cast<int32_t *>(ws + l.keys_sorted);
   int32_t *positions_sorted = reinterpret_cast<int32_t *>(ws + l.positions_sorted);
   int32_t *grad_rows = reinterpret_cast<int32_t *>(ws + l.grad_rows);
+  if (interleaved_offsets_stride > 0) {
+    // Tables stored [E][T][D], bags b*T + t: the batch is put into table-major order first (one pass
+    // over the indices), then sorted table by table like any other; a key leaves the last pass as
+    // idx*T + t, the row of the [E*T][D] view.  Positions are those of the table-major order.
+    const InterleavedRegions r = interleaved_regions(l, workspace, n, T, B);
+    const int rc = interleaved_to_table_major(indices, offsets, interleaved_offsets_stride, T, B, r.totals, r.bias,
+                                              r.chunk_sums, r.offsets_tm, r.indices_tm, stream);
+    if (rc) return rc;
+    SortTables tables{r.offsets_tm, B, T, r.bias, grad_rows};
+    tables.key_mul = T;
+    return sort_pairs(r.indices_tm, nullptr, keys_sorted, positions_sorted, n, key_bits(total_rows / T),
+                      ws + l.sort_scratch, stream, &tables);
+  }
   if (sort_tables(T) != T) {
     int32_t *keys = reinterpret_cast<int32_t *>(ws + l.keys);
     const int rc = linearize(table_offsets, T, indices, offsets, B, keys, grad_rows, stream);
@@ -93,10 +137,11 @@ int sort_batch(const tbe_workspace_layout_t &l, void *workspace, const int32_t *
 
 int build_plan(const tbe_workspace_layout_t &l, void *workspace, const int32_t *table_offsets,
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
-               int64_t total_rows, int64_t max_table_rows, hipStream_t stream) {
+               int64_t total_rows, int64_t max_table_rows, hipStream_t stream,
+               int32_t interleaved_offsets_stride) {
   char *ws = static_cast<char *>(workspace);
   const int rc = sort_batch(l, workspace, table_offsets, T, indices, n, offsets, B, total_rows, max_table_rows,
-                            stream);
+                            stream, interleaved_offsets_stride);
   if (rc) return rc;
   return find_segments(reinterpret_cast<int32_t *>(ws + l.keys_sorted), n,
                        reinterpret_cast<int32_t *>(ws + l.segment_starts),
@@ -134,6 +179,8 @@ struct BackwardCall {
   const int32_t *unique_slots;
   void *cache_rows;
   StochasticRounding stochastic_rounding;
+  // interleaved tables [E][T][D]: entries of `offsets` per b (T or T + 1); 0 = table-major
+  int32_t interleaved_offsets_stride = 0;
 };
 
 int run_backward(const char *name, const BackwardCall &c) {
@@ -147,7 +194,8 @@ int run_backward(const char *name, const BackwardCall &c) {
   TBE_REQUIRE(c.num_indices >= 0 && c.num_indices < INT32_MAX, "%s: num_indices out of range", name);
   TBE_REQUIRE(static_cast<int64_t>(c.T) * c.B < INT32_MAX, "%s: T*B out of range", name);
   TBE_REQUIRE(c.grad_output && c.weights, "%s: null pointer argument", name);
-  TBE_REQUIRE(c.planned || (c.table_offsets && c.offsets), "%s: null pointer argument", name);
+  TBE_REQUIRE(c.planned || ((c.table_offsets || c.interleaved_offsets_stride > 0) && c.offsets),
+              "%s: null pointer argument", name);
   TBE_REQUIRE(c.planned || c.indices || c.num_indices == 0, "%s: indices is null but num_indices > 0", name);
   TBE_REQUIRE(c.optimizer == kOptSgd || c.state, "%s: optimizer_state is null", name);
   TBE_REQUIRE((c.psw == nullptr) == (c.grad_psw == nullptr),
@@ -155,7 +203,7 @@ int run_backward(const char *name, const BackwardCall &c) {
   if (c.num_indices == 0) return TBE_OK;
 
   tbe_workspace_layout_t l;
-  compute_layout(c.num_indices, c.D, c.dtype, c.T, &l);
+  compute_layout(c.num_indices, c.D, c.dtype, c.T, &l, c.interleaved_offsets_stride > 0 ? c.B : 0);
   if (!c.workspace || c.workspace_bytes < l.total_bytes)
     return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
                 (unsigned long long)l.total_bytes, (unsigned long long)c.workspace_bytes);
@@ -168,7 +216,8 @@ int run_backward(const char *name, const BackwardCall &c) {
 
   if (!c.planned) {
     const int rc = build_plan(l, c.workspace, c.table_offsets, c.T, c.indices, c.num_indices,
-                              c.offsets, c.B, c.total_rows, c.max_table_rows, c.stream);
+                              c.offsets, c.B, c.total_rows, c.max_table_rows, c.stream,
+                              c.interleaved_offsets_stride);
     if (rc) return rc;
   }
 
@@ -216,6 +265,40 @@ extern "C" int tbe_backward_workspace_layout(int64_t num_indices, int32_t D, int
   TBE_REQUIRE(T > 0, "tbe_backward_workspace_layout: T must be positive (got %d)", T);
   compute_layout(num_indices, D, dtype, T, layout);
   return TBE_OK;
+}
+
+extern "C" int tbe_backward_interleaved_workspace_layout(int64_t num_indices, int32_t D, int32_t dtype, int32_t T,
+                                                         int32_t B, tbe_workspace_layout_t *layout) {
+  using namespace tbe;
+  const char *name = "tbe_backward_interleaved_workspace_layout";
+  TBE_REQUIRE(layout, "%s: null layout", name);
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(D > 0 && D % 4 == 0, "%s: D must be a positive multiple of 4 (got %d)", name, D);
+  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
+  TBE_REQUIRE(T > 0 && B > 0 && static_cast<int64_t>(T) * B < INT32_MAX, "%s: bad T or B (got %d, %d)", name, T, B);
+  compute_layout(num_indices, D, dtype, T, layout, B);
+  return TBE_OK;
+}
+
+extern "C" int tbe_backward_sgd_interleaved(const void *grad_output, void *weights, int32_t dtype, int64_t E,
+                                            int32_t T, int32_t D, const int32_t *indices, int64_t num_indices,
+                                            const int32_t *offsets, int32_t offsets_row_stride, int32_t B,
+                                            float learning_rate, void *workspace, uint64_t workspace_bytes,
+                                            void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_backward_sgd_interleaved";
+  TBE_REQUIRE(E > 0 && T > 0 && E * T < INT32_MAX, "%s: E * T must fit a 32-bit row number", name);
+  TBE_REQUIRE(offsets_row_stride == T || offsets_row_stride == T + 1,
+              "%s: offsets_row_stride must be T (flat offsets) or T + 1 ([B][T+1] offsets), got %d", name,
+              offsets_row_stride);
+  if (T > kMaxTablesSortedApart)
+    return fail(TBE_ERR_UNSUPPORTED, "%s: at most %d interleaved tables (got %d)", name, kMaxTablesSortedApart, T);
+  // T tables of E rows: row idx*T + t of the [E*T][D] view, gradient row b*T + t of [B*T][D]
+  BackwardCall c{grad_output, weights, dtype, E * T, 0, D, nullptr, T, indices, num_indices, offsets, B, nullptr,
+                 nullptr, learning_rate, 0.0f, nullptr, workspace, workspace_bytes,
+                 static_cast<hipStream_t>(stream), kOptSgd, false, nullptr, nullptr, StochasticRounding{0, 0, 0}};
+  c.interleaved_offsets_stride = offsets_row_stride;
+  return run_backward(name, c);
 }
 
 extern "C" int tbe_backward_sgd(const void *grad_output, void *weights, int32_t dtype,

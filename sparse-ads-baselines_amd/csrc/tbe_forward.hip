@@ -14,11 +14,54 @@
 // (table_batched_embeddings_cuda.cu:193-251): bag index b_t = t*B + b,
 // output[b][t][:], empty bag -> zeros, weighted variant multiplies each row by
 // indice_weights[position] (WeightedForward, :176-191).
+//
+// Interleaved tables (the older sparse_embedding_cuda layout, sparse_embedding_cuda_kernel.cu:221-284,
+// 349-379): weights [E][T][D], bags numbered b*T + t, bag (b, t) bounded by offsets[b * stride + t]
+// and the entry after it (stride = T for one flat array, T + 1 for the [B][T+1] form).  The same
+// kernels serve it -- `table_offsets` is null then, the row of a lookup is idx * T + t and the
+// bag's output row is the bag's number -- so no index array is rewritten.
 
 #include "tbe_common.h"
 
 namespace tbe {
 namespace {
+
+// Where a bag lives.  Table-major (table_offsets given): bag = t*B + b, rows table_offsets[t] + idx.
+// Interleaved (table_offsets null): bag = b*T + t, rows idx*T + t, offsets with a row stride.
+struct BagPlace {
+  int start, end;          // the bag's lookups
+  int64_t row0;            // row of a lookup = row0 + idx * row_mul
+  int row_mul;             // (1, or T for interleaved tables, where idx * T < 2^31)
+  int64_t out_row;         // b*T + t
+};
+__device__ __forceinline__ BagPlace place_bag(int bag, bool has_end, int B, int num_tables,
+                                              const int32_t *__restrict__ table_offsets,
+                                              const int32_t *__restrict__ offsets, int offsets_stride) {
+  BagPlace p;
+  if (table_offsets) {
+    const int t = bag / B;
+    const int b = bag - t * B;
+    p.start = offsets[bag];
+    p.end = has_end ? offsets[bag + 1] : p.start;
+    p.row0 = table_offsets[t];
+    p.row_mul = 1;
+    p.out_row = static_cast<int64_t>(b) * num_tables + t;
+  } else {
+    // The wavefronts still walk the bags table by table (bag = t*B + b names the bag b*T + t), so that
+    // an XCD, which takes an eighth of the bags, works on an eighth of the tables and finds their hot
+    // rows in its own L2, as with table-major tables.  (Walking them in their own order, every XCD
+    // touches every table: 380 instead of 317 us for 64 tables of 100 k rows of 128, Zipf 1.05.)
+    const int t = bag / B;
+    const int b = bag - t * B;
+    const int64_t at = static_cast<int64_t>(b) * offsets_stride + t;
+    p.start = offsets[at];
+    p.end = has_end ? offsets[at + 1] : p.start;
+    p.row0 = t;
+    p.row_mul = num_tables;
+    p.out_row = static_cast<int64_t>(b) * num_tables + t;
+  }
+  return p;
+}
 
 // CACHED: every lookup carries a location (lookup_slots[p]); a non-negative value is a slot of
 // the HBM row cache (row at cache_rows + slot * D), a negative one means the row is read from
@@ -29,7 +72,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
     const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
     const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D,
     int chunks_rt, int num_bags, int64_t blocks_per_xcd,
-    const int32_t *__restrict__ lookup_slots, const T *__restrict__ cache_rows) {
+    const int32_t *__restrict__ lookup_slots, const T *__restrict__ cache_rows, int offsets_stride) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -39,8 +82,6 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
   const int64_t bag64 = logical * kWavesPerBlock + (threadIdx.x >> 6);
   if (bag64 >= num_bags) return;
   const int bag = static_cast<int>(bag64);
-  const int t = bag / B;
-  const int b = bag - t * B;
 
   const int chunks = CHUNKS > 0 ? CHUNKS : chunks_rt;
   const int groups = kWave / chunks;  // rows fetched per wavefront-wide load
@@ -48,9 +89,11 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
   const int c = lane - r * chunks;
   const bool active = r < groups;
 
-  const int start = offsets[bag];
-  const int end = offsets[bag + 1];
-  const int64_t table_row0 = table_offsets[t];
+  const BagPlace place = place_bag(bag, true, B, num_tables, table_offsets, offsets, offsets_stride);
+  const int start = place.start;
+  const int end = place.end;
+  const int64_t table_row0 = place.row0;
+  const int row_mul = place.row_mul;
   const T *col = weights + static_cast<int64_t>(c) * VEC;
 
   V acc;
@@ -77,7 +120,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
         const int src = ok[u] ? j : 0;
         const int idx = shfl_idx(my_idx, src);
         if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, src);
-        const T *row = col + (table_row0 + idx) * D;
+        const T *row = col + (table_row0 + idx * row_mul) * D;
         if constexpr (CACHED) {
           const int slot = shfl_idx(my_slot, src);
           if (slot >= 0) row = cache_rows + static_cast<int64_t>(slot) * D + static_cast<int64_t>(c) * VEC;
@@ -122,7 +165,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
   }
 
   if (r == 0) {
-    acc.store(output + (static_cast<int64_t>(b) * num_tables + t) * D + static_cast<int64_t>(c) * VEC);
+    acc.store(output + place.out_row * D + static_cast<int64_t>(c) * VEC);
   }
 }
 
@@ -138,7 +181,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
     const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
     const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D, int num_bags,
     int64_t blocks_per_xcd, const int32_t *__restrict__ lookup_slots,
-    const T *__restrict__ cache_rows) {
+    const T *__restrict__ cache_rows, int offsets_stride) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -156,13 +199,14 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
   const int64_t bag64 = wave_index * kGroups + r;
   const bool valid = bag64 < num_bags;
   const int bag = static_cast<int>(valid ? bag64 : num_bags - 1);
-  const int t = bag / B;
-  const int b = bag - t * B;
-  const int start = offsets[bag];
-  const int end = valid ? offsets[bag + 1] : start;
-  const int64_t table_row0 = table_offsets[t];
+  const BagPlace place = place_bag(bag, valid, B, num_tables, table_offsets, offsets, offsets_stride);
+  const int start = place.start;
+  const int end = place.end;
+  const int64_t table_row0 = place.row0;
+  const int row_mul = place.row_mul;
   const T *col = weights + static_cast<int64_t>(c) * VEC;
-  const int idle_idx = -static_cast<int>(table_row0);
+  // (interleaved tables: index 0 of the bag's own table, which exists)
+  const int idle_idx = table_offsets ? -static_cast<int>(table_row0) : 0;
 
   V acc;
   acc.zero();
@@ -204,7 +248,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
           const int src = group_base + j;
           const int i = shfl_idx(idx[q], src);
           if constexpr (WEIGHTED) ww[u] = shfl_idx(w[q], src);
-          const T *row = col + (table_row0 + i) * D;
+          const T *row = col + (table_row0 + i * row_mul) * D;
           if constexpr (CACHED) {
             const int s = shfl_idx(slot[q], src);
             if (s >= 0) row = cache_rows + static_cast<int64_t>(s) * D + static_cast<int64_t>(c) * VEC;
@@ -224,7 +268,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
       }
     }
   }
-  if (valid) acc.store(output + (static_cast<int64_t>(b) * num_tables + t) * D + static_cast<int64_t>(c) * VEC);
+  if (valid) acc.store(output + place.out_row * D + static_cast<int64_t>(c) * VEC);
 }
 
 // Rows wider than 64 vectors: the wavefront walks the row in blocks of 64
@@ -235,7 +279,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_wide_kernel(
     const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
     const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D,
     int chunks, int num_bags, int64_t blocks_per_xcd,
-    const int32_t *__restrict__ lookup_slots, const T *__restrict__ cache_rows) {
+    const int32_t *__restrict__ lookup_slots, const T *__restrict__ cache_rows, int offsets_stride) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -245,12 +289,12 @@ __global__ __launch_bounds__(kBlockThreads) void forward_wide_kernel(
   const int64_t bag64 = logical * kWavesPerBlock + (threadIdx.x >> 6);
   if (bag64 >= num_bags) return;
   const int bag = static_cast<int>(bag64);
-  const int t = bag / B;
-  const int b = bag - t * B;
-  const int start = offsets[bag];
-  const int end = offsets[bag + 1];
-  const int64_t table_row0 = table_offsets[t];
-  T *out_row = output + (static_cast<int64_t>(b) * num_tables + t) * D;
+  const BagPlace place = place_bag(bag, true, B, num_tables, table_offsets, offsets, offsets_stride);
+  const int start = place.start;
+  const int end = place.end;
+  const int64_t table_row0 = place.row0;
+  const int row_mul = place.row_mul;
+  T *out_row = output + place.out_row * D;
 
   for (int cb = 0; cb < chunks; cb += kWave) {
     const int c = cb + lane;
@@ -276,7 +320,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_wide_kernel(
           const int j = min(j0 + u, n - 1);
           const int idx = shfl_idx(my_idx, j);
           if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, j);
-          const T *row = col + (table_row0 + idx) * D;
+          const T *row = col + (table_row0 + idx * row_mul) * D;
           if constexpr (CACHED) {
             const int slot = shfl_idx(my_slot, j);
             if (slot >= 0) row = cache_rows + static_cast<int64_t>(slot) * D + static_cast<int64_t>(c) * VEC;
@@ -315,6 +359,7 @@ struct ForwardArgs {
   const int32_t *lookup_slots;  // null unless the rows are fronted by the HBM row cache
   const void *cache_rows;
   int64_t num_indices;
+  int32_t offsets_stride = 0;   // interleaved tables (table_offsets null): entries of `offsets` per b
 };
 
 template <typename T, int VEC, bool WEIGHTED, bool CACHED>
@@ -332,7 +377,7 @@ void launch_forward(const ForwardArgs &a, const RowGeometry &g, hipStream_t stre
 #define TBE_FWD(CH)                                                                            \
   TBE_LAUNCH("forward", stream, (forward_kernel<T, VEC, CH, WEIGHTED, CACHED, kUnroll>), grid, \
              block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, g.chunks,   \
-             num_bags, per_xcd, a.lookup_slots, cr)
+             num_bags, per_xcd, a.lookup_slots, cr, a.offsets_stride)
   // short bags of narrow rows: a lane group per bag instead of a wavefront per bag
   const bool grouped = !g.wide && (g.tmpl == 4 || g.tmpl == 8 || g.tmpl == 16) &&
                        a.num_indices <= static_cast<int64_t>(num_bags) * 48;
@@ -344,7 +389,7 @@ void launch_forward(const ForwardArgs &a, const RowGeometry &g, hipStream_t stre
 #define TBE_FWD_GROUPED(CH)                                                                       \
   TBE_LAUNCH("forward", stream, (forward_grouped_kernel<T, VEC, CH, WEIGHTED, CACHED>), ggrid,    \
              block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, num_bags,      \
-             gper_xcd, a.lookup_slots, cr)
+             gper_xcd, a.lookup_slots, cr, a.offsets_stride)
     if (g.tmpl == 4) TBE_FWD_GROUPED(4);
     else if (g.tmpl == 8) TBE_FWD_GROUPED(8);
     else TBE_FWD_GROUPED(16);
@@ -352,7 +397,7 @@ void launch_forward(const ForwardArgs &a, const RowGeometry &g, hipStream_t stre
   } else if (g.wide) {
     TBE_LAUNCH("forward_wide", stream, (forward_wide_kernel<T, VEC, WEIGHTED, CACHED, 4>), grid,
                block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, g.chunks,
-               num_bags, per_xcd, a.lookup_slots, cr);
+               num_bags, per_xcd, a.lookup_slots, cr, a.offsets_stride);
   } else {
     switch (g.tmpl) {
       case 64: TBE_FWD(64); break;
@@ -387,7 +432,8 @@ int validate_forward(const char *name, const ForwardArgs &a, int64_t num_indices
   TBE_REQUIRE(a.dtype >= TBE_DTYPE_F32 && a.dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, a.dtype);
   TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
   TBE_REQUIRE(static_cast<int64_t>(a.T) * a.B < INT32_MAX, "%s: T*B out of range", name);
-  TBE_REQUIRE(a.weights && a.table_offsets && a.offsets && a.output, "%s: null pointer argument", name);
+  TBE_REQUIRE(a.weights && (a.table_offsets || a.offsets_stride >= a.T) && a.offsets && a.output,
+              "%s: null pointer argument", name);
   TBE_REQUIRE(a.indices || num_indices == 0, "%s: indices is null but num_indices > 0", name);
   return TBE_OK;
 }
@@ -437,5 +483,20 @@ extern "C" int tbe_forward_cached(const tbe_cache_t *cache, int32_t dtype, int32
                             per_sample_weights, output, nullptr, nullptr, num_indices};
     return run_forward(plain, static_cast<hipStream_t>(stream));
   }
+  return run_forward(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tbe_forward_interleaved(const void *weights, int32_t dtype, int64_t E, int32_t T, int32_t D,
+                                       const int32_t *indices, int64_t num_indices, const int32_t *offsets,
+                                       int32_t offsets_row_stride, int32_t B, void *output, void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_forward_interleaved";
+  TBE_REQUIRE(E > 0 && T > 0 && E * T < INT32_MAX, "%s: E * T must fit a 32-bit row number", name);
+  TBE_REQUIRE(offsets_row_stride == T || offsets_row_stride == T + 1,
+              "%s: offsets_row_stride must be T (flat offsets) or T + 1 ([B][T+1] offsets), got %d", name,
+              offsets_row_stride);
+  ForwardArgs a{weights, dtype, D, nullptr, T, indices, offsets, B, nullptr, output, nullptr, nullptr, num_indices};
+  a.offsets_stride = offsets_row_stride;
+  if (int rc = validate_forward(name, a, num_indices)) return rc;
   return run_forward(a, static_cast<hipStream_t>(stream));
 }

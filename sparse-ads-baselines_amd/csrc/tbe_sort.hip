@@ -109,6 +109,118 @@ __global__ __launch_bounds__(kBlockThreads) void linearize_kernel(
   }
 }
 
+// ------------------------------------------------ interleaved tables -> table-major batch
+// Tables stored [E][T][D] number their bags b*T + t and bound bag (b, t) by offsets[b * stride + t]
+// and the entry after it (sparse_embedding_cuda_kernel.cu:221-284).  The backward needs the lookups
+// table by table (the sort works on one table's consecutive positions, the update walks gradient
+// rows table by table), so the batch is put into that order once: three small launches, one pass
+// over the indices.  After them `indices_tm` / `offsets_tm` are a table-major batch [T][B].
+//
+// Bags are taken kBlockThreads at a time: chunk c of table t holds bags c*256 ... of that table.
+// Launch 1, one workgroup per chunk: the chunk's lookups.
+__global__ __launch_bounds__(kBlockThreads) void interleaved_chunk_sums_kernel(
+    const int32_t *__restrict__ offsets, int offsets_stride, int B, int chunks_per_table,
+    int32_t *__restrict__ chunk_sums) {
+  __shared__ int32_t s_part[kWavesPerBlock];
+  const int t = blockIdx.x / chunks_per_table;
+  const int b = (blockIdx.x - t * chunks_per_table) * kBlockThreads + threadIdx.x;
+  int32_t sum = 0;
+  if (b < B) {
+    const int64_t at = static_cast<int64_t>(b) * offsets_stride + t;
+    sum = offsets[at + 1] - offsets[at];
+  }
+  for (int m = kWave / 2; m > 0; m >>= 1) sum += __shfl_xor(sum, m, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) s_part[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t total = 0;
+    for (int w = 0; w < kWavesPerBlock; ++w) total += s_part[w];
+    chunk_sums[blockIdx.x] = total;
+  }
+}
+
+// Launch 2, one workgroup per table: the table's lookups, and bias[t] = t for the sort's last pass.
+__global__ __launch_bounds__(kBlockThreads) void interleaved_totals_kernel(
+    const int32_t *__restrict__ chunk_sums, int chunks_per_table, int32_t *__restrict__ totals,
+    int32_t *__restrict__ bias) {
+  __shared__ int32_t s_part[kWavesPerBlock];
+  const int t = blockIdx.x;
+  int32_t sum = 0;
+  for (int c = threadIdx.x; c < chunks_per_table; c += kBlockThreads)
+    sum += chunk_sums[static_cast<int64_t>(t) * chunks_per_table + c];
+  for (int m = kWave / 2; m > 0; m >>= 1) sum += __shfl_xor(sum, m, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) s_part[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t total = 0;
+    for (int w = 0; w < kWavesPerBlock; ++w) total += s_part[w];
+    totals[t] = total;
+    bias[t] = t;
+  }
+}
+
+// Launch 3, one workgroup per chunk: offsets_tm[t*B + b] = lookups of the tables before t + of the
+// table's chunks before this one + of the chunk's bags before b; the last workgroup also writes
+// offsets_tm[T*B].
+__global__ __launch_bounds__(kBlockThreads) void interleaved_offsets_kernel(
+    const int32_t *__restrict__ offsets, int offsets_stride, int B, int num_tables, int chunks_per_table,
+    const int32_t *__restrict__ totals, const int32_t *__restrict__ chunk_sums,
+    int32_t *__restrict__ offsets_tm) {
+  __shared__ int32_t s_part[kWavesPerBlock];
+  __shared__ int32_t s_scan[kWavesPerBlock];
+  const int t = blockIdx.x / chunks_per_table;
+  const int chunk = blockIdx.x - t * chunks_per_table;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  int32_t before = 0;
+  for (int k = threadIdx.x; k < t; k += kBlockThreads) before += totals[k];
+  for (int k = threadIdx.x; k < chunk; k += kBlockThreads)
+    before += chunk_sums[static_cast<int64_t>(t) * chunks_per_table + k];
+  for (int m = kWave / 2; m > 0; m >>= 1) before += __shfl_xor(before, m, kWave);
+  const int b = chunk * kBlockThreads + threadIdx.x;
+  int32_t len = 0;
+  if (b < B) {
+    const int64_t at = static_cast<int64_t>(b) * offsets_stride + t;
+    len = offsets[at + 1] - offsets[at];
+  }
+  int32_t x = len;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int32_t y = __shfl_up(x, d, kWave);
+    if (lane >= d) x += y;
+  }
+  if (lane == 0) s_part[wave] = before;
+  if (lane == kWave - 1) s_scan[wave] = x;
+  __syncthreads();
+  int32_t carry = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) {
+    carry += s_part[w];
+    if (w < wave) carry += s_scan[w];
+    all += s_scan[w];
+  }
+  if (b < B) offsets_tm[static_cast<int64_t>(t) * B + b] = carry + x - len;
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == kBlockThreads - 1)
+    offsets_tm[static_cast<int64_t>(num_tables) * B] = carry + x;
+}
+
+// 8 lanes per bag: the bag's indices go to their place in the table-major order.
+__global__ __launch_bounds__(kBlockThreads) void interleaved_permute_kernel(
+    const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets, int offsets_stride, int B,
+    int num_tables, int num_bags, const int32_t *__restrict__ offsets_tm, int32_t *__restrict__ indices_tm) {
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t bag64 = gid / kLinLanes;
+  if (bag64 >= num_bags) return;
+  const int bag = static_cast<int>(bag64);  // t*B + b: consecutive wavefronts write consecutive memory
+  const int t = bag / B;
+  const int b = bag - t * B;
+  const int64_t at = static_cast<int64_t>(b) * offsets_stride + t;
+  const int src = offsets[at];
+  const int len = offsets[at + 1] - src;
+  const int dst = offsets_tm[bag];
+  for (int i = static_cast<int>(gid % kLinLanes); i < len; i += kLinLanes) indices_tm[dst + i] = indices[src + i];
+}
+
 // The gradient row b*T + t of every position, 8 lanes per bag, for workgroup `block` of
 // ceil(num_bags * 8 / 256): what linearize_kernel writes when it is given no keys.
 __device__ __forceinline__ void record_gradient_rows(const int32_t *__restrict__ offsets, int B,
@@ -122,22 +234,6 @@ __device__ __forceinline__ void record_gradient_rows(const int32_t *__restrict__
   const int32_t grow = (bag - t * B) * num_tables + t;
   const int end = offsets[bag + 1];
   for (int p = offsets[bag] + static_cast<int>(gid % kLinLanes); p < end; p += kLinLanes) grad_rows[p] = grow;
-}
-
-// Row numbers for tables stored interleaved, weights[row][table][D] (the layout of the older
-// sparse_embedding_cuda kernels, sparse_embedding_cuda_kernel.cu:349-379: weights[ind][t][d]).
-// Viewed as a [E*T][D] matrix, row `ind` of table t is matrix row ind*T + t; bags are numbered
-// bag-major (b*T + t), so the table of a bag is bag % T.
-__global__ __launch_bounds__(kBlockThreads) void interleaved_rows_kernel(
-    const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets, int num_tables,
-    int num_bags, int32_t *__restrict__ rows) {
-  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int64_t bag = gid / kLinLanes;
-  if (bag >= num_bags) return;
-  const int t = static_cast<int>(bag % num_tables);
-  const int end = offsets[bag + 1];
-  for (int p = offsets[bag] + static_cast<int>(gid % kLinLanes); p < end; p += kLinLanes)
-    rows[p] = indices[p] * num_tables + t;
 }
 
 // ------------------------------------------------------------------ radix sort
@@ -375,7 +471,8 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scan_kernel(
 }
 
 // key_bias (nullable): added to the keys of table t as they are written (the last pass turns
-// rows inside a table into rows of the concatenated tables).
+// rows inside a table into rows of the concatenated tables), after a multiplication by key_mul
+// (1; T for tables stored interleaved, whose row idx of table t is row idx*T + t of one array).
 template <int BITS, bool LOCAL, int ITEMS>
 __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ values_in,
@@ -383,7 +480,7 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     const uint32_t *__restrict__ table_starts, const uint32_t *__restrict__ tile_prefix,
     int num_tables, int max_tiles, int shift, uint32_t mask, const uint32_t *__restrict__ bases,
     const uint32_t *__restrict__ totals, const uint32_t *__restrict__ group_totals,
-    const int32_t *__restrict__ key_bias) {
+    const int32_t *__restrict__ key_bias, uint32_t key_mul) {
   constexpr int kBinsT = 1 << BITS;
   constexpr int kOwned = kBinsT / kBlockThreads;  // consecutive digits per thread
   // The per-wavefront digit counters are only needed until every key knows its slot in the
@@ -572,7 +669,7 @@ __global__ __launch_bounds__(kBlockThreads) void radix_scatter_kernel(
     if (local < tile.count) {
       const uint32_t kk = s_keys[local];
       const uint32_t dst = s_dest[(kk >> shift) & mask] + static_cast<uint32_t>(local);
-      keys_out[dst] = kk + bias;
+      keys_out[dst] = key_bias ? kk * key_mul + bias : kk;
       values_out[dst] = s_vals[local];
     }
   }
@@ -761,6 +858,7 @@ struct RadixPass {
   uint32_t *totals;        // this pass's per-table digit totals, zeroed; null: linear scan
   uint32_t *group_totals;  // this pass's digit totals of every kGroupTiles tiles, zeroed
   const int32_t *key_bias;
+  uint32_t key_mul;
 };
 
 template <int BITS, int ITEMS>
@@ -773,7 +871,7 @@ void launch_radix_pass(const RadixPass &p, hipStream_t stream) {
                p.group_totals);
     TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, true, ITEMS>), tiles, block, p.src_k, p.src_v,
                p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
-               p.counts, p.totals, p.group_totals, p.key_bias);
+               p.counts, p.totals, p.group_totals, p.key_bias, p.key_mul);
     return;
   }
   const dim3 scan_blocks(static_cast<unsigned>(ceil_div(static_cast<int64_t>(p.max_tiles) << BITS, kScanChunk)));
@@ -785,7 +883,7 @@ void launch_radix_pass(const RadixPass &p, hipStream_t stream) {
              p.num_tables, BITS, p.block_sums);
   TBE_LAUNCH("radix_scatter", stream, (radix_scatter_kernel<BITS, false, ITEMS>), tiles, block, p.src_k, p.src_v,
              p.dst_k, p.dst_v, p.table_starts, p.tile_prefix, p.num_tables, p.max_tiles, p.shift, p.mask,
-             p.counts, nullptr, nullptr, p.key_bias);
+             p.counts, nullptr, nullptr, p.key_bias, p.key_mul);
 }
 }  // namespace
 
@@ -845,6 +943,7 @@ int sort_pairs(const int32_t *keys_in, const int32_t *values_in, int32_t *keys_o
     p.dst_k = to_out ? reinterpret_cast<uint32_t *>(keys_out) : tmp_keys;
     p.dst_v = to_out ? reinterpret_cast<uint32_t *>(values_out) : tmp_vals;
     p.key_bias = (tables && pass == passes - 1) ? tables->key_bias : nullptr;
+    p.key_mul = tables ? static_cast<uint32_t>(tables->key_mul) : 1u;
     p.totals = table_scan ? totals + static_cast<int64_t>(pass) * num_tables * kMaxBins : nullptr;
     p.group_totals = table_scan ? group_totals + static_cast<int64_t>(pass) * groups * kMaxBins : nullptr;
     if (items == kSmallItems) {
@@ -903,6 +1002,25 @@ int linearize(const int32_t *table_offsets, int32_t T, const int32_t *indices,
   return check_launch("tbe_linearize");
 }
 
+int interleaved_to_table_major(const int32_t *indices, const int32_t *offsets, int32_t offsets_stride,
+                               int32_t T, int32_t B, int32_t *totals, int32_t *bias, int32_t *chunk_sums,
+                               int32_t *offsets_tm, int32_t *indices_tm, hipStream_t stream) {
+  const int64_t num_bags = static_cast<int64_t>(T) * B;
+  const int chunks = static_cast<int>(interleaved_chunks_per_table(B));
+  const dim3 block(kBlockThreads);
+  const dim3 per_chunk(static_cast<unsigned>(static_cast<int64_t>(T) * chunks));
+  TBE_LAUNCH("interleaved_offsets", stream, interleaved_chunk_sums_kernel, per_chunk, block, offsets, offsets_stride,
+             B, chunks, chunk_sums);
+  TBE_LAUNCH("interleaved_offsets", stream, interleaved_totals_kernel, dim3(static_cast<unsigned>(T)), block,
+             chunk_sums, chunks, totals, bias);
+  TBE_LAUNCH("interleaved_offsets", stream, interleaved_offsets_kernel, per_chunk, block, offsets, offsets_stride, B,
+             T, chunks, totals, chunk_sums, offsets_tm);
+  TBE_LAUNCH("interleaved_permute", stream, interleaved_permute_kernel,
+             dim3(static_cast<unsigned>(ceil_div(num_bags * kLinLanes, kBlockThreads))), block, indices, offsets,
+             offsets_stride, B, T, static_cast<int>(num_bags), offsets_tm, indices_tm);
+  return check_launch("tbe_backward_sgd_interleaved");
+}
+
 }  // namespace tbe
 
 extern "C" int tbe_linearize(const int32_t *table_offsets, int32_t T, const int32_t *indices,
@@ -917,24 +1035,6 @@ extern "C" int tbe_linearize(const int32_t *table_offsets, int32_t T, const int3
   TBE_REQUIRE(indices && keys && grad_rows, "tbe_linearize: null pointer argument");
   return linearize(table_offsets, T, indices, offsets, B, keys, grad_rows,
                    static_cast<hipStream_t>(stream));
-}
-
-extern "C" int tbe_interleaved_rows(const int32_t *indices, int64_t num_indices,
-                                    const int32_t *offsets, int32_t T, int32_t B, int32_t *rows,
-                                    void *stream) {
-  using namespace tbe;
-  TBE_REQUIRE(T > 0 && B > 0, "tbe_interleaved_rows: T and B must be positive (got %d, %d)", T, B);
-  TBE_REQUIRE(static_cast<int64_t>(T) * B < INT32_MAX, "tbe_interleaved_rows: T*B out of range");
-  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "tbe_interleaved_rows: num_indices out of range");
-  TBE_REQUIRE(offsets, "tbe_interleaved_rows: null offsets");
-  if (num_indices == 0) return TBE_OK;
-  TBE_REQUIRE(indices && rows, "tbe_interleaved_rows: null pointer argument");
-  const int64_t num_bags = static_cast<int64_t>(T) * B;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  TBE_LAUNCH("interleaved_rows", s, interleaved_rows_kernel,
-             dim3(static_cast<unsigned>(ceil_div(num_bags * kLinLanes, kBlockThreads))), dim3(kBlockThreads),
-             indices, offsets, T, static_cast<int>(num_bags), rows);
-  return check_launch("tbe_interleaved_rows");
 }
 
 extern "C" uint64_t tbe_sort_workspace_bytes(int64_t n) { return tbe::sort_workspace_bytes(n, 1); }

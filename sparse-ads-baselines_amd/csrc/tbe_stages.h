@@ -21,7 +21,16 @@ struct SortTables {
   // nullable, [n] out: the gradient row b*T + t of every position (what linearize() records),
   // written by the sort's set-up launch instead of a launch of its own
   int32_t *grad_rows = nullptr;
+  int32_t key_mul = 1;      // a key leaves the last pass as key * key_mul + key_bias[t]
 };
+
+// Tables stored interleaved, [E][T][D] with bags b*T + t bounded by offsets[b * stride + t] and the
+// entry after it: puts the batch into table-major order (indices_tm [n], offsets_tm [T*B+1]) and
+// writes bias[t] = t; totals [T] and chunk_sums [T * interleaved_chunks_per_table(B)] are scratch.
+inline int64_t interleaved_chunks_per_table(int32_t B) { return (static_cast<int64_t>(B) + kBlockThreads - 1) / kBlockThreads; }
+int interleaved_to_table_major(const int32_t *indices, const int32_t *offsets, int32_t offsets_stride,
+                               int32_t T, int32_t B, int32_t *totals, int32_t *bias, int32_t *chunk_sums,
+                               int32_t *offsets_tm, int32_t *indices_tm, hipStream_t stream);
 
 uint64_t sort_workspace_bytes(int64_t n, int32_t num_tables);
 // device_count (nullable): the number of pairs, read on the device (at most n; with tables == nullptr).
@@ -118,12 +127,15 @@ void backward_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspa
 // max_table_rows: an upper bound of the rows of the largest table (0 = unknown, total_rows is
 // used); it sets how many key bits are sorted.
 // grad_rows, keys_sorted and positions_sorted of the layout (table_offsets: first row of every table)
+// interleaved_offsets_stride > 0: tables stored [E][T][D] (table_offsets unused), `offsets` rows of
+// that many entries; the layout is then the one of backward_interleaved_layout().
 int sort_batch(const tbe_workspace_layout_t &layout, void *workspace, const int32_t *table_offsets, int32_t T,
                const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B, int64_t total_rows,
-               int64_t max_table_rows, hipStream_t stream);
+               int64_t max_table_rows, hipStream_t stream, int32_t interleaved_offsets_stride = 0);
 int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int32_t *table_offsets,
                int32_t T, const int32_t *indices, int64_t n, const int32_t *offsets, int32_t B,
-               int64_t total_rows, int64_t max_table_rows, hipStream_t stream);
+               int64_t total_rows, int64_t max_table_rows, hipStream_t stream,
+               int32_t interleaved_offsets_stride = 0);
 
 // The approximate row-wise Adagrad update (one lookup at a time per row, in position order) on a
 // workspace that holds the batch's plan.  Uniform tables: D > 0 and the mixed_* pointers null;

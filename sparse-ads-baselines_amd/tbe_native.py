@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -97,7 +97,12 @@ SIGNATURES = {
     "tbe_backward_planned": (ctypes.c_int, [_i32, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _f32, _f32,
                                             _vp, _i32, _u64, _u64, _vp, _u64, _vp]),
     "tbe_linearize": (ctypes.c_int, [_c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _c_i32p, _c_i32p, _vp]),
-    "tbe_interleaved_rows": (ctypes.c_int, [_c_i32p, _i64, _c_i32p, _i32, _i32, _c_i32p, _vp]),
+    "tbe_forward_interleaved": (ctypes.c_int, [_vp, _i32, _i64, _i32, _i32, _c_i32p, _i64, _c_i32p, _i32, _i32, _vp,
+                                               _vp]),
+    "tbe_backward_interleaved_workspace_layout": (ctypes.c_int, [_i64, _i32, _i32, _i32, _i32,
+                                                                 ctypes.POINTER(WorkspaceLayout)]),
+    "tbe_backward_sgd_interleaved": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i32, _i32, _c_i32p, _i64, _c_i32p, _i32,
+                                                    _i32, _f32, _vp, _u64, _vp]),
     "tbe_sort_workspace_bytes": (_u64, [_i64]),
     "tbe_sort_pairs": (ctypes.c_int, [_c_i32p, _c_i32p, _c_i32p, _c_i32p, _i64, _i32, _vp, _u64, _vp]),
     "tbe_segments_workspace_bytes": (_u64, [_i64]),
@@ -172,6 +177,12 @@ def check(code):
 def backward_workspace_layout(num_indices, D, dtype_code, T):
     layout = WorkspaceLayout()
     check(load().tbe_backward_workspace_layout(num_indices, D, dtype_code, T, ctypes.byref(layout)))
+    return layout
+
+
+def backward_interleaved_workspace_layout(num_indices, D, dtype_code, T, B):
+    layout = WorkspaceLayout()
+    check(load().tbe_backward_interleaved_workspace_layout(num_indices, D, dtype_code, T, B, ctypes.byref(layout)))
     return layout
 
 

@@ -90,3 +90,61 @@ def test_half_and_double_tables(oracle, dtype, tol):
     oracle.backward("sgd", go.reshape(B * T, 1, D), one_table, zero, one_table_rows, flat, 0.1)
     torch.cuda.synchronize()
     assert_close(w.cpu().numpy().reshape(E * T, D), one_table, tol)
+
+
+def test_large_ragged_batch_and_layout_query(oracle):
+    """More bags than one scan chunk per table (B > 256), empty bags, tables whose lookups differ a
+    lot: the pass that puts the batch into table-major order before the sort (offsets scan in
+    chunks of 256 bags, permutation of the indices) is exercised across chunk boundaries."""
+    import tbe_native
+    rs = np.random.RandomState(12)
+    E, T, D, B = 500, 7, 32, 1000
+    weights = rs.randn(E, T, D).astype(np.float32)
+    lengths = rs.randint(0, 6, size=(B, T))
+    lengths[:, 2] = 0                      # a table nobody looks up
+    lengths[300:600, 4] += 20              # and a busy stretch of another
+    flat = np.concatenate([[0], np.cumsum(lengths.reshape(-1))]).astype(np.int32)
+    indices = (rs.zipf(1.2, size=int(flat[-1])) % E).astype(np.int32)
+    merged = np.stack([flat[b * T:b * T + T + 1] for b in range(B)]).astype(np.int32)
+    go = rs.randn(B, T, D).astype(np.float32)
+    w = dev(weights)
+    got = se.forward_offsets(w, dev(indices), dev(merged))
+    assert_close(got.cpu().numpy(), oracle.forward_etd(weights, indices, flat), 1e-5)
+    se.backward_update_offsets(dev(go), w, dev(indices), dev(merged), 0.1)
+    w_ref = weights.copy()
+    oracle.backward_etd(go, w_ref, indices, flat, 0.1)
+    torch.cuda.synchronize()
+    assert_close(w.cpu().numpy(), w_ref, 1e-5)
+    lay = tbe_native.backward_interleaved_workspace_layout(indices.size, D, tbe_native.DTYPE_F32, T, B)
+    plain = tbe_native.backward_workspace_layout(indices.size, D, tbe_native.DTYPE_F32, T)
+    assert lay.grad_rows - lay.keys >= indices.size * 4 + (T * B + 1) * 4 and lay.total_bytes > plain.total_bytes
+
+
+def test_interleaved_step_in_a_graph():
+    """Forward and fused update on the interleaved layout only launch kernels (nothing is rewritten
+    or allocated besides the output), so a step can be captured and replayed with new indices."""
+    rs = np.random.RandomState(3)
+    E, T, D, B, L = 400, 5, 64, 40, 6
+    w = dev(rs.randn(E, T, D).astype(np.float32))
+    w_eager = w.clone()
+    x = dev((rs.zipf(1.3, size=(B, T, L)) % E).astype(np.int32))
+    go = dev(rs.randn(B, T, D).astype(np.float32))
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):        # sizes this stream's scratch buffer, fills the offsets cache
+        warm = w.clone()
+        se.forward_fast_single(warm, x)
+        se.backward_update_fast_single(go, warm, x, 0.05)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        out = se.forward_fast_single(w, x)
+        se.backward_update_fast_single(go, w, x, 0.05)
+    for replay in range(3):
+        if replay:
+            x.copy_(dev((rs.zipf(1.3, size=(B, T, L)) % E).astype(np.int32)))
+        graph.replay()
+        want = se.forward_fast_single(w_eager, x.clone())
+        se.backward_update_fast_single(go, w_eager, x.clone(), 0.05)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want) and torch.equal(w, w_eager)
