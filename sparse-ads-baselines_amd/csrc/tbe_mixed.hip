@@ -400,7 +400,7 @@ __device__ __forceinline__ void mixed_update_wide(
 // the table's width and offsets, optimizer state -- is fetched for the 64 rows at once, so the
 // dependent loads are paid per strip.  Rows of more than kMixedShort occurrences (the hot rows,
 // which are neighbours in key order) and rows wider than 64 vectors are not reduced here: their
-// indices go to two queues that update_mixed_long_kernel drains -- one wavefront per row of at
+// indices go to two queues that update_mixed_queued_kernel drains -- one wavefront per row of at
 // most kChunkLen occurrences, one workgroup of 16 wavefronts per longer row -- so that they
 // spread over the machine.  The other rows leave a 32-byte record in LDS (in row order), and
 // every occurrence of theirs leaves the element offset of its gradient row (and its position,
@@ -723,28 +723,29 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
 // occurrences).  The wavefronts of a row take its 64-position batches round-robin; their sums
 // meet in LDS and the row's first wavefront adds them in wavefront order and applies the
 // optimizer.  A row wider than 64 vectors is left to its first wavefront.  `queue_counter` is
-// the index of the queue's length in `counters`.
+// the index of the queue's length in `counters`.  Both kinds of row are served by ONE launch of
+// workgroups of kHugeWaves wavefronts: the first `huge_blocks` workgroups take a long row each
+// time round, the others one row per wavefront -- the two queues drain side by side instead of
+// one after the other (each is bound by the dependent loads at the head of a row, not by
+// bandwidth: 99 + 101 us one after the other for 64 tables of 100 k rows of 64..192, Zipf 1.05).
 constexpr int kHugeWaves = 16;
 template <typename T, int VEC, int OPT, bool WEIGHTED, int UNROLL, int WAVES>
-__global__ __launch_bounds__((WAVES > 1 ? WAVES : kWavesPerBlock) * kWave) void update_mixed_long_kernel(
+__device__ __forceinline__ void mixed_queued_rows(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
     T *__restrict__ grad_psw, const int64_t *__restrict__ table_offsets,
     const int32_t *__restrict__ table_dim_offsets, const int32_t *__restrict__ dim_offsets,
     int num_tables, int total_D, const int32_t *__restrict__ keys_sorted,
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
-    const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
-    int queue_counter, const int32_t *__restrict__ queue, float lr, float eps, StochasticRounding sr) {
+    const int32_t *__restrict__ segment_starts, int num_queued, const int32_t *__restrict__ queue, float lr,
+    float eps, StochasticRounding sr, int64_t first_row, int64_t row_stride,
+    typename AccOf<T>::type (*s_partial)[kWave * VEC]) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
-  constexpr int kRowsPerBlock = WAVES > 1 ? 1 : kWavesPerBlock;
-  __shared__ A s_partial[WAVES > 1 ? WAVES : 1][WAVES > 1 ? kWave * VEC : 1];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   const int wave_in_row = WAVES > 1 ? wave : 0;
-  const int num_queued = counters[queue_counter];
-  for (int64_t q = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (WAVES > 1 ? 0 : wave); q < num_queued;
-       q += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
+  for (int64_t q = first_row; q < num_queued; q += row_stride) {
     const int u = queue[q];
     MixedRow row;
     row.seg_begin = segment_starts[u];
@@ -783,6 +784,36 @@ __global__ __launch_bounds__((WAVES > 1 ? WAVES : kWavesPerBlock) * kWave) void 
     }
     if (wave_in_row == 0)
       mixed_apply_narrow<T, VEC, OPT>(weights, state, lr, eps, sr, lane, row, state_old, w_old, G);
+  }
+}
+
+template <typename T, int VEC, int OPT, bool WEIGHTED, int UNROLL>
+__global__ __launch_bounds__(kHugeWaves * kWave) void update_mixed_queued_kernel(
+    const T *__restrict__ grad_output, T *__restrict__ weights,
+    typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
+    T *__restrict__ grad_psw, const int64_t *__restrict__ table_offsets,
+    const int32_t *__restrict__ table_dim_offsets, const int32_t *__restrict__ dim_offsets,
+    int num_tables, int total_D, const int32_t *__restrict__ keys_sorted,
+    const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
+    const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
+    const int32_t *__restrict__ long_queue, const int32_t *__restrict__ huge_queue, int huge_blocks, float lr,
+    float eps, StochasticRounding sr) {
+  using A = typename AccOf<T>::type;
+  __shared__ A s_partial[kHugeWaves][kWave * VEC];
+  if (static_cast<int>(blockIdx.x) < huge_blocks) {
+    // rows of more than kChunkLen occurrences (their number is counters[1]): the workgroup per row
+    mixed_queued_rows<T, VEC, OPT, WEIGHTED, UNROLL, kHugeWaves>(
+        grad_output, weights, state, psw, grad_psw, table_offsets, table_dim_offsets, dim_offsets, num_tables, total_D,
+        keys_sorted, positions_sorted, grad_rows, segment_starts, counters[1], huge_queue, lr, eps, sr, blockIdx.x,
+        huge_blocks, s_partial);
+  } else {
+    // the other queued rows (counters[2]): a wavefront per row
+    const int64_t long_blocks = static_cast<int64_t>(gridDim.x) - huge_blocks;
+    mixed_queued_rows<T, VEC, OPT, WEIGHTED, UNROLL, 1>(
+        grad_output, weights, state, psw, grad_psw, table_offsets, table_dim_offsets, dim_offsets, num_tables, total_D,
+        keys_sorted, positions_sorted, grad_rows, segment_starts, counters[2], long_queue, lr, eps, sr,
+        (static_cast<int64_t>(blockIdx.x) - huge_blocks) * kHugeWaves + (threadIdx.x >> 6), long_blocks * kHugeWaves,
+        s_partial);
   }
 }
 
@@ -851,18 +882,15 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
              go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, bag_magic, bag_shift,
              a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
              i32(l.num_unique), long_rows, huge_rows, a.lr, a.eps, a.sr);
-  const int64_t want_long = ceil_div(a.n, kWavesPerBlock);
-  const dim3 grid_long(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 8))));
-  TBE_LAUNCH("update_mixed_long", stream, (update_mixed_long_kernel<T, VEC, OPT, WEIGHTED, 8, 1>), grid_long,
-             dim3(kBlockThreads), go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T,
-             a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
-             i32(l.num_unique), 2, long_rows, a.lr, a.eps, a.sr);
+  const int64_t want_long = ceil_div(a.n, kHugeWaves);
+  const int64_t long_blocks = std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 2));
   const int64_t want_huge = a.n / (kChunkLen + 1) + 1;
-  const dim3 grid_huge(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_huge, 256 * 2))));
-  TBE_LAUNCH("update_mixed_huge", stream, (update_mixed_long_kernel<T, VEC, OPT, WEIGHTED, 8, kHugeWaves>),
-             grid_huge, dim3(kHugeWaves * kWave), go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets,
-             a.dim_offsets, a.T, a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows),
-             i32(l.segment_starts), i32(l.num_unique), 1, huge_rows, a.lr, a.eps, a.sr);
+  const int64_t huge_blocks = std::max<int64_t>(1, std::min<int64_t>(want_huge, 256 * 2));
+  TBE_LAUNCH("update_mixed_queued", stream, (update_mixed_queued_kernel<T, VEC, OPT, WEIGHTED, 8>),
+             dim3(static_cast<unsigned>(huge_blocks + long_blocks)), dim3(kHugeWaves * kWave), go, w, st, psw, gpsw,
+             a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, a.total_D, i32(l.keys_sorted),
+             i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts), i32(l.num_unique), long_rows, huge_rows,
+             static_cast<int>(huge_blocks), a.lr, a.eps, a.sr);
 }
 
 // The approximate update's strip kernel: rows of at most 64 vectors and kMixedShort occurrences
