@@ -273,11 +273,30 @@ __device__ __forceinline__ double shfl_x(double v, int m) { return __shfl_xor(v,
 // the group gets the result.  CHUNKS > 0: power-of-two group, xor butterfly that
 // never leaves the group.  CHUNKS == 0: arbitrary group size, every lane adds the
 // group's values in lane order (`group_base` = first lane of the group).
+// Lanes exchanged inside a row of 16 by the data-parallel-primitive path of the vector ALU (no LDS
+// crossbar, no address arithmetic): 0xB1 = quad_perm [1,0,3,2] (lane ^ 1), 0x4E = quad_perm [2,3,0,1]
+// (lane ^ 2), 0x141 = row_half_mirror (lane i of a group of 8 reads lane 7 - i), 0x140 = row_mirror
+// (lane i of a row of 16 reads lane 15 - i).
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+template <int CTRL> __device__ __forceinline__ double dpp_move(double v) {
+  const long long bits = __builtin_bit_cast(long long, v);
+  const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(bits), CTRL, 0xF, 0xF, false);
+  const int hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(bits >> 32), CTRL, 0xF, 0xF, false);
+  return __builtin_bit_cast(double, (static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo));
+}
 template <int CHUNKS, typename A>
 __device__ __forceinline__ A group_sum(A v, int chunks, int group_base) {
   if constexpr (CHUNKS > 0) {
+    // pairs, quads, then -- every lane of a quad (of eight lanes) holding the same sum by then -- the mirrored
+    // quad (eight lanes); wider groups finish with lane shuffles
+    if constexpr (CHUNKS >= 2) v += dpp_move<0xB1>(v);
+    if constexpr (CHUNKS >= 4) v += dpp_move<0x4E>(v);
+    if constexpr (CHUNKS >= 8) v += dpp_move<0x141>(v);
+    if constexpr (CHUNKS >= 16) v += dpp_move<0x140>(v);
 #pragma unroll
-    for (int m = CHUNKS / 2; m > 0; m >>= 1) v += shfl_x(v, m);
+    for (int m = 16; m < CHUNKS; m <<= 1) v += shfl_x(v, m);
     return v;
   } else {
     A s = A(0);

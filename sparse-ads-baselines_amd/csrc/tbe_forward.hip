@@ -63,6 +63,23 @@ __device__ __forceinline__ BagPlace place_bag(int bag, bool has_end, int B, int 
   return p;
 }
 
+// The packed vector of a lane that holds no lookup becomes zeros, so that what follows is the same
+// multiply-add for every lane (a select on the packed words costs half of one on the converted values,
+// and leaves the conversion and the addition to one mixed-precision instruction).
+template <typename R> __device__ __forceinline__ void keep_if(R &raw, bool keep) {
+  static_assert(sizeof(R) % 4 == 0, "whole registers");
+  uint32_t words[sizeof(R) / 4];
+  __builtin_memcpy(words, &raw, sizeof(R));
+#pragma unroll
+  for (size_t i = 0; i < sizeof(R) / 4; ++i) words[i] = keep ? words[i] : 0u;
+  __builtin_memcpy(&raw, words, sizeof(R));
+}
+// Row r of a table of rows of CHUNKS 16-byte vectors (r < 2^31: one shift instead of a 64-bit multiply).
+template <typename T, int VEC, int CHUNKS>
+__device__ __forceinline__ const T *narrow_row(const T *base, uint32_t row) {
+  return base + (static_cast<uint64_t>(row) * static_cast<uint64_t>(CHUNKS * VEC));
+}
+
 // CACHED: every lookup carries a location (lookup_slots[p]); a non-negative value is a slot of
 // the HBM row cache (row at cache_rows + slot * D), a negative one means the row is read from
 // `weights` (the host-resident backing table) directly.
@@ -175,7 +192,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
 // per step, up to 8 independent row loads in flight per lane), nothing is reduced across lanes
 // and the instruction stream is shared by all the wavefront's bags.  Same sums as
 // forward_kernel in a different order (each lane adds its bag's rows in bag order).
-template <typename T, int VEC, int CHUNKS, bool WEIGHTED, bool CACHED>
+template <typename T, int VEC, int CHUNKS, bool WEIGHTED, bool CACHED, bool INTERLEAVED>
 __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
     const T *__restrict__ weights, const int32_t *__restrict__ table_offsets,
     const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
@@ -205,8 +222,10 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
   const int64_t table_row0 = place.row0;
   const int row_mul = place.row_mul;
   const T *col = weights + static_cast<int64_t>(c) * VEC;
+  const T *cache_col = cache_rows + static_cast<int64_t>(c) * VEC;
+  const uint32_t row0_32 = static_cast<uint32_t>(table_row0);  // rows are numbered below 2^31
   // (interleaved tables: index 0 of the bag's own table, which exists)
-  const int idle_idx = table_offsets ? -static_cast<int>(table_row0) : 0;
+  const int idle_idx = INTERLEAVED ? 0 : -static_cast<int>(table_row0);
 
   V acc;
   acc.zero();
@@ -246,23 +265,25 @@ __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
           const int j = j0 + u;
           ok[u] = j < left;
           const int src = group_base + j;
-          const int i = shfl_idx(idx[q], src);
+          const uint32_t i = static_cast<uint32_t>(shfl_idx(idx[q], src));
           if constexpr (WEIGHTED) ww[u] = shfl_idx(w[q], src);
-          const T *row = col + (table_row0 + i * row_mul) * D;
+          const uint32_t row32 = row0_32 + (INTERLEAVED ? i * static_cast<uint32_t>(row_mul) : i);
+          const T *row = narrow_row<T, VEC, CHUNKS>(col, row32);
           if constexpr (CACHED) {
             const int s = shfl_idx(slot[q], src);
-            if (s >= 0) row = cache_rows + static_cast<int64_t>(s) * D + static_cast<int64_t>(c) * VEC;
+            if (s >= 0) row = narrow_row<T, VEC, CHUNKS>(cache_col, static_cast<uint32_t>(s));
           }
           raw[u] = V::load_raw(row);  // every lane loads (straight-line code keeps the loads back to back)
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
+          keep_if(raw[u], ok[u]);
           V x;
           x.unpack(raw[u]);
 #pragma unroll
           for (int k = 0; k < VEC; ++k) {
-            const A term = WEIGHTED ? x.v[k] * ww[u] : x.v[k];
-            acc.v[k] += ok[u] ? term : A(0);
+            if constexpr (WEIGHTED) acc.v[k] += x.v[k] * ww[u];
+            else acc.v[k] += x.v[k];
           }
         }
       }
@@ -386,13 +407,22 @@ void launch_forward(const ForwardArgs &a, const RowGeometry &g, hipStream_t stre
     const int64_t gblocks = ceil_div(ceil_div(num_bags, groups), kWavesPerBlock);
     const int64_t gper_xcd = ceil_div(gblocks, kNumXcd);
     const dim3 ggrid(static_cast<unsigned>(gper_xcd * kNumXcd));
-#define TBE_FWD_GROUPED(CH)                                                                       \
-  TBE_LAUNCH("forward", stream, (forward_grouped_kernel<T, VEC, CH, WEIGHTED, CACHED>), ggrid,    \
-             block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, num_bags,      \
+#define TBE_FWD_GROUPED_L(CH, IL)                                                                   \
+  TBE_LAUNCH("forward", stream, (forward_grouped_kernel<T, VEC, CH, WEIGHTED, CACHED, IL>), ggrid,  \
+             block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, num_bags,        \
              gper_xcd, a.lookup_slots, cr, a.offsets_stride)
+    // (the row cache fronts table-major tables only)
+#define TBE_FWD_GROUPED(CH)                                                     \
+  do {                                                                          \
+    if constexpr (!CACHED) {                                                    \
+      if (!a.table_offsets) { TBE_FWD_GROUPED_L(CH, true); break; }             \
+    }                                                                           \
+    TBE_FWD_GROUPED_L(CH, false);                                               \
+  } while (0)
     if (g.tmpl == 4) TBE_FWD_GROUPED(4);
     else if (g.tmpl == 8) TBE_FWD_GROUPED(8);
     else TBE_FWD_GROUPED(16);
+#undef TBE_FWD_GROUPED_L
 #undef TBE_FWD_GROUPED
   } else if (g.wide) {
     TBE_LAUNCH("forward_wide", stream, (forward_wide_kernel<T, VEC, WEIGHTED, CACHED, 4>), grid,
