@@ -269,6 +269,39 @@ __device__ __forceinline__ int64_t shfl_idx(int64_t v, int src) {
 __device__ __forceinline__ float shfl_x(float v, int m) { return __shfl_xor(v, m, kWave); }
 __device__ __forceinline__ double shfl_x(double v, int m) { return __shfl_xor(v, m, kWave); }
 
+// The packed vector of a lane that holds no lookup becomes zeros, so that what follows is the same
+// multiply-add for every lane (a select on the packed words costs half of one on the converted values,
+// and leaves the conversion and the addition to one mixed-precision instruction).
+template <typename R> __device__ __forceinline__ void keep_if(R &raw, bool keep) {
+  static_assert(sizeof(R) % 4 == 0, "whole registers");
+  uint32_t words[sizeof(R) / 4];
+  __builtin_memcpy(words, &raw, sizeof(R));
+#pragma unroll
+  for (size_t i = 0; i < sizeof(R) / 4; ++i) words[i] = keep ? words[i] : 0u;
+  __builtin_memcpy(&raw, words, sizeof(R));
+}
+// <a, b> over the VEC elements a lane holds, as up to four independent partial sums that are added in a
+// fixed tree (a single chain of VEC dependent multiply-adds keeps the vector ALU waiting for itself).
+template <int VEC, typename A>
+__device__ __forceinline__ A lane_dot(const A (&a)[VEC], const A (&b)[VEC]) {
+  constexpr int kParts = VEC < 4 ? VEC : 4;
+  A part[kParts];
+#pragma unroll
+  for (int i = 0; i < kParts; ++i) part[i] = a[i] * b[i];
+#pragma unroll
+  for (int i = kParts; i < VEC; ++i) part[i % kParts] += a[i] * b[i];
+  if constexpr (kParts == 4) return (part[0] + part[1]) + (part[2] + part[3]);
+  else if constexpr (kParts == 2) return part[0] + part[1];
+  else return part[0];
+}
+// The value as the compiler must take it: a register it knows nothing about.  Used where the instruction
+// selection should convert THIS operand once instead of folding its conversion into every use.
+__device__ __forceinline__ float opaque(float x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+__device__ __forceinline__ double opaque(double x) { return x; }
+
 // Sum of `v` over the `chunks` lanes of the caller's lane group; every lane of
 // the group gets the result.  CHUNKS > 0: power-of-two group, xor butterfly that
 // never leaves the group.  CHUNKS == 0: arbitrary group size, every lane adds the

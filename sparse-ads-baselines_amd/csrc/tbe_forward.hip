@@ -63,17 +63,6 @@ __device__ __forceinline__ BagPlace place_bag(int bag, bool has_end, int B, int 
   return p;
 }
 
-// The packed vector of a lane that holds no lookup becomes zeros, so that what follows is the same
-// multiply-add for every lane (a select on the packed words costs half of one on the converted values,
-// and leaves the conversion and the addition to one mixed-precision instruction).
-template <typename R> __device__ __forceinline__ void keep_if(R &raw, bool keep) {
-  static_assert(sizeof(R) % 4 == 0, "whole registers");
-  uint32_t words[sizeof(R) / 4];
-  __builtin_memcpy(words, &raw, sizeof(R));
-#pragma unroll
-  for (size_t i = 0; i < sizeof(R) / 4; ++i) words[i] = keep ? words[i] : 0u;
-  __builtin_memcpy(&raw, words, sizeof(R));
-}
 // Row r of a table of rows of CHUNKS 16-byte vectors (r < 2^31: one shift instead of a 64-bit multiply).
 template <typename T, int VEC, int CHUNKS>
 __device__ __forceinline__ const T *narrow_row(const T *base, uint32_t row) {

@@ -309,9 +309,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
             state_old = state_old + (WEIGHTED ? gss * pw * pw : gss);
             const A mult = approx_multiplier<A>(state_old, pw, WEIGHTED, lr, eps);
             if constexpr (WEIGHTED) {
-              A dot = A(0);
-#pragma unroll
-              for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
+              A dot = lane_dot<VEC, A>(w_old.v, x.v);
               dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
               if (c == 0) grad_psw[pos[q]] = from_acc<T, A>(dot);
             }
@@ -329,10 +327,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
           V x;
           x.unpack(raw[q]);
           if constexpr (WEIGHTED) {
-            const A pw = to_acc(pw_raw[q]);
-            A dot = A(0);
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
+            const A pw = opaque(to_acc(pw_raw[q]));  // converted once; the gradient's conversions fold into the sums
+            A dot = lane_dot<VEC, A>(w_old.v, x.v);
             dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
             if (c == 0) grad_psw[pos[q]] = from_acc<T, A>(dot);
 #pragma unroll
@@ -516,17 +512,14 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
             pos = shfl_idx(my_pos, src[k]);
           }
           if constexpr (APPROX) pw = shfl_idx(my_w, src[k]);
+          keep_if(raw[k], ok[k]);
           V x;
           x.unpack(raw[k]);
-#pragma unroll
-          for (int i = 0; i < VEC; ++i) x.v[i] = ok[k] ? x.v[i] : A(0);
           if constexpr (APPROX) {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) G.v[i] += x.v[i] * pw;
           } else if constexpr (WEIGHTED) {
-            A dot = A(0);
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) dot += w_old.v[i] * x.v[i];
+            A dot = lane_dot<VEC, A>(w_old.v, x.v);
             dot = group_sum<CHUNKS, A>(dot, chunks, group_base);
             if (ok[k] && c == 0) grad_psw[pos] = from_acc<T, A>(dot);
 #pragma unroll
