@@ -63,20 +63,24 @@ __device__ __forceinline__ BagPlace place_bag(int bag, bool has_end, int B, int 
   return p;
 }
 
-// Row r of a table of rows of CHUNKS 16-byte vectors (r < 2^31: one shift instead of a 64-bit multiply).
+// Row r of a table of rows of CHUNKS 16-byte vectors (r < 2^31).  With CHUNKS known at compile time the row's
+// offset is a shift of the 32-bit row number; otherwise one 32 x 32 -> 64-bit multiply with D.  (A 64-bit row
+// number times D costs three quarter-rate 32-bit multiplies per row: the vector ALU was busy with those for a
+// fifth of the forward of 512-byte rows.)
 template <typename T, int VEC, int CHUNKS>
-__device__ __forceinline__ const T *narrow_row(const T *base, uint32_t row) {
-  return base + (static_cast<uint64_t>(row) * static_cast<uint64_t>(CHUNKS * VEC));
+__device__ __forceinline__ const T *narrow_row(const T *base, uint32_t row, int D = 0) {
+  if constexpr (CHUNKS > 0) return base + (static_cast<uint64_t>(row) * static_cast<uint64_t>(CHUNKS * VEC));
+  else return base + static_cast<uint64_t>(row) * static_cast<uint32_t>(D);
 }
 
 // CACHED: every lookup carries a location (lookup_slots[p]); a non-negative value is a slot of
 // the HBM row cache (row at cache_rows + slot * D), a negative one means the row is read from
 // `weights` (the host-resident backing table) directly.
-template <typename T, int VEC, int CHUNKS, bool WEIGHTED, bool CACHED, int UNROLL>
+template <typename T, int VEC, int CHUNKS, bool WEIGHTED, bool CACHED, int UNROLL, bool INTERLEAVED>
 __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
     const T *__restrict__ weights, const int32_t *__restrict__ table_offsets,
     const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
-    const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D,
+    const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D_rt,
     int chunks_rt, int num_bags, int64_t blocks_per_xcd,
     const int32_t *__restrict__ lookup_slots, const T *__restrict__ cache_rows, int offsets_stride) {
   using V = RowVec<T, VEC>;
@@ -90,6 +94,7 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
   const int bag = static_cast<int>(bag64);
 
   const int chunks = CHUNKS > 0 ? CHUNKS : chunks_rt;
+  const int D = CHUNKS > 0 ? CHUNKS * VEC : D_rt;
   const int groups = kWave / chunks;  // rows fetched per wavefront-wide load
   const int r = lane / chunks;
   const int c = lane - r * chunks;
@@ -98,9 +103,10 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
   const BagPlace place = place_bag(bag, true, B, num_tables, table_offsets, offsets, offsets_stride);
   const int start = place.start;
   const int end = place.end;
-  const int64_t table_row0 = place.row0;
-  const int row_mul = place.row_mul;
+  const uint32_t row0_32 = static_cast<uint32_t>(place.row0);  // rows are numbered below 2^31
+  const uint32_t row_mul = static_cast<uint32_t>(place.row_mul);
   const T *col = weights + static_cast<int64_t>(c) * VEC;
+  const T *cache_col = cache_rows + static_cast<int64_t>(c) * VEC;
 
   V acc;
   acc.zero();
@@ -124,12 +130,12 @@ __global__ __launch_bounds__(kBlockThreads) void forward_kernel(
         const int j = j0 + u * groups + r;
         ok[u] = active && j < n;
         const int src = ok[u] ? j : 0;
-        const int idx = shfl_idx(my_idx, src);
+        const uint32_t idx = static_cast<uint32_t>(shfl_idx(my_idx, src));
         if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, src);
-        const T *row = col + (table_row0 + idx * row_mul) * D;
+        const T *row = narrow_row<T, VEC, CHUNKS>(col, row0_32 + (INTERLEAVED ? idx * row_mul : idx), D);
         if constexpr (CACHED) {
           const int slot = shfl_idx(my_slot, src);
-          if (slot >= 0) row = cache_rows + static_cast<int64_t>(slot) * D + static_cast<int64_t>(c) * VEC;
+          if (slot >= 0) row = narrow_row<T, VEC, CHUNKS>(cache_col, static_cast<uint32_t>(slot), D);
         }
         if (ok[u]) raw[u] = V::load_raw(row);
       }
@@ -185,12 +191,13 @@ template <typename T, int VEC, int CHUNKS, bool WEIGHTED, bool CACHED, bool INTE
 __global__ __launch_bounds__(kBlockThreads) void forward_grouped_kernel(
     const T *__restrict__ weights, const int32_t *__restrict__ table_offsets,
     const int32_t *__restrict__ indices, const int32_t *__restrict__ offsets,
-    const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int D, int num_bags,
+    const T *__restrict__ psw, T *__restrict__ output, int B, int num_tables, int /*D*/, int num_bags,
     int64_t blocks_per_xcd, const int32_t *__restrict__ lookup_slots,
     const T *__restrict__ cache_rows, int offsets_stride) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
+  constexpr int D = CHUNKS * VEC;
   constexpr int kGroups = kWave / CHUNKS;
   constexpr int kPerLane = 32 / CHUNKS;        // indices held per lane: a step covers 32 lookups of every bag
   constexpr int kStep = kPerLane * CHUNKS;
@@ -384,10 +391,18 @@ void launch_forward(const ForwardArgs &a, const RowGeometry &g, hipStream_t stre
   const T *cr = static_cast<const T *>(a.cache_rows);
   T *o = static_cast<T *>(a.output);
   constexpr int kUnroll = 8;
-#define TBE_FWD(CH)                                                                            \
-  TBE_LAUNCH("forward", stream, (forward_kernel<T, VEC, CH, WEIGHTED, CACHED, kUnroll>), grid, \
-             block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, g.chunks,   \
+#define TBE_FWD_L(CH, IL)                                                                          \
+  TBE_LAUNCH("forward", stream, (forward_kernel<T, VEC, CH, WEIGHTED, CACHED, kUnroll, IL>), grid, \
+             block, w, a.table_offsets, a.indices, a.offsets, p, o, a.B, a.T, a.D, g.chunks,       \
              num_bags, per_xcd, a.lookup_slots, cr, a.offsets_stride)
+  // (the row cache fronts table-major tables only)
+#define TBE_FWD(CH)                                                             \
+  do {                                                                          \
+    if constexpr (!CACHED) {                                                    \
+      if (!a.table_offsets) { TBE_FWD_L(CH, true); break; }                     \
+    }                                                                           \
+    TBE_FWD_L(CH, false);                                                       \
+  } while (0)
   // short bags of narrow rows: a lane group per bag instead of a wavefront per bag
   const bool grouped = !g.wide && (g.tmpl == 4 || g.tmpl == 8 || g.tmpl == 16) &&
                        a.num_indices <= static_cast<int64_t>(num_bags) * 48;
@@ -428,6 +443,7 @@ void launch_forward(const ForwardArgs &a, const RowGeometry &g, hipStream_t stre
     }
   }
 #undef TBE_FWD
+#undef TBE_FWD_L
 }
 
 template <typename T, int VEC>

@@ -123,11 +123,13 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ segment_ids,
     int32_t *__restrict__ counters, LongRecord *__restrict__ long_records,
     ChunkRecord *__restrict__ chunk_records, int64_t max_chunks, int64_t n, int64_t num_tiles,
-    int64_t tiles_per_xcd, int D, int chunks_rt, float lr, float eps,
+    int64_t tiles_per_xcd, int D_rt, int chunks_rt, float lr, float eps,
     const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr,
     int32_t *__restrict__ approx_long_queue) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
+  // (a compile-time row width turns every row address into a shift)
+  const int D = CHUNKS > 0 ? CHUNKS * VEC : D_rt;
   using R = typename V::R;
   static_assert(!APPROX || OPT == kOptAdagrad, "the approximate update is a row-wise Adagrad");
 
@@ -375,11 +377,13 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
     T *__restrict__ grad_psw, const int32_t *__restrict__ positions_sorted,
     const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ counters,
     const ChunkRecord *__restrict__ chunk_records, int64_t max_chunks,
-    typename AccOf<T>::type *__restrict__ partial_sums, int D, int chunks_rt, float lr, float eps,
+    typename AccOf<T>::type *__restrict__ partial_sums, int D_rt, int chunks_rt, float lr, float eps,
     const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr,
     const int32_t *__restrict__ segment_starts) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
+  // (a compile-time row width turns every row address into a shift)
+  const int D = CHUNKS > 0 ? CHUNKS * VEC : D_rt;
   using R = typename V::R;
   static_assert(!APPROX || (OPT == kOptSgd && !WEIGHTED && sizeof(T) == sizeof(A)),
                 "the per-lookup form sums fp32 / fp64 rows without per-sample weights");
@@ -611,11 +615,13 @@ template <typename T, int VEC, int CHUNKS, int OPT>
 __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     T *__restrict__ weights, typename AccOf<T>::type *__restrict__ state,
     const int32_t *__restrict__ counters, const LongRecord *__restrict__ long_records,
-    const typename AccOf<T>::type *__restrict__ partial_sums, int D, int chunks_rt, float lr,
+    const typename AccOf<T>::type *__restrict__ partial_sums, int D_rt, int chunks_rt, float lr,
     float eps, const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows,
     StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
+  // (a compile-time row width turns every row address into a shift)
+  const int D = CHUNKS > 0 ? CHUNKS * VEC : D_rt;
 
   const int lane = threadIdx.x & (kWave - 1);
   const int chunks = CHUNKS > 0 ? CHUNKS : chunks_rt;
