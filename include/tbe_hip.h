@@ -532,6 +532,20 @@ TBE_API int tbe_backward_cached(int32_t optimizer, const void *grad_output, cons
                                 void *workspace, uint64_t workspace_bytes,
                                 const int32_t *unique_slots, void *stream);
 
+/* tbe_backward_approx_adagrad (the per-lookup row-wise Adagrad of
+ * batched_embedding_backward_adagrad_approx_cuda, table_batched_embeddings_cuda.cu:706-793) on the plan
+ * that tbe_cache_prepare left in `workspace`, every row updated where it lives; `offsets` are the
+ * batch's bag offsets [T*B + 1] again (the plan does not keep them).  Same result, bit for bit, as the
+ * uncached entry point on the backing table. */
+TBE_API int tbe_backward_approx_cached(const void *grad_output, const tbe_cache_t *cache, int32_t dtype,
+                                       int64_t total_rows, int32_t D, int32_t T, int32_t B,
+                                       int64_t num_indices, const int32_t *offsets,
+                                       const void *per_sample_weights, void *optimizer_state,
+                                       float learning_rate, float eps, void *grad_per_sample_weights,
+                                       int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
+                                       void *workspace, uint64_t workspace_bytes,
+                                       const int32_t *unique_slots, void *stream);
+
 /* Writes every resident row, and every row waiting in a staging area, back to the backing table (the
  * cache stays valid).  `stream` must be ordered behind the streams of earlier tbe_cache_plan calls, and a
  * planned batch must have been committed.  Deferred write-back: the last `live_sequences` planned batches

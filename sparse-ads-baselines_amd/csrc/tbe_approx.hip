@@ -115,7 +115,8 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ positions_sorted,
     const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ segment_starts,
     int32_t *__restrict__ counters, int32_t *__restrict__ long_queue, int D, int group, float lr,
-    float eps, MixedTables mt, StochasticRounding sr, const int32_t *__restrict__ only_rows) {
+    float eps, MixedTables mt, StochasticRounding sr, const int32_t *__restrict__ only_rows,
+    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -177,7 +178,13 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
       seg_end = seg_begin;  // nothing to do here
     }
     const bool handled_here = seg_end > seg_begin;
+    // (cache-fronted uniform tables: the row lives in its cache slot when it has one; its random
+    // words still go by its place in the table)
     T *wrow = weights + row_element;
+    if (unique_slots) {
+      const int slot = unique_slots[u];
+      if (slot >= 0) wrow = cache_rows + static_cast<int64_t>(slot) * D;
+    }
     A s = state_in;
     V w;
     w.zero();
@@ -456,6 +463,8 @@ template <typename T> struct LongRowArgs {
   MixedTables mt;  // (T == 0: uniform tables)
   StochasticRounding sr;
   uint64_t grad_bytes;  // size of grad_output
+  const int32_t *unique_slots;  // cache-fronted uniform tables: slot of each unique row (-1: not resident), or null
+  T *cache_rows;
 };
 
 // First element of gradient row `grad_row` for a row at `p` (mixed-D tables: mt.T > 0).
@@ -500,7 +509,8 @@ __device__ __forceinline__ P buffer_load_pack(__amdgpu_buffer_rsrc_t rsrc, uint3
 // kCoopStep occurrences.
 template <typename T, int E, bool WEIGHTED, bool STOCHASTIC, bool BIG, bool COOP = false>
 __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_begin, int seg_end, int64_t key,
-                                              const RowPlace &place, int lane, const uint16_t *words = nullptr) {
+                                              const RowPlace &place, T *storage, int lane,
+                                              const uint16_t *words = nullptr) {
   using A = typename AccOf<T>::type;
   using P = LanePack<T, E>;
   static_assert(!COOP || (STOCHASTIC && E <= 2), "the cooperative walk is for stochastic rounding of narrow rows");
@@ -513,7 +523,7 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
   constexpr int kRing = kInBlocks ? 2 * kAhead : (E * sizeof(T) <= 4 ? kWave : E * sizeof(T) <= 8 ? kWave / 2 : kWave / 4);
   const bool active = lane * E < place.row_D;
   const int lane_off = active ? lane * E : 0;  // (idle lanes shadow lane 0 and store nothing)
-  T *wrow = a.weights + place.row_element + lane_off;
+  T *wrow = storage + lane_off;  // (the row's first element where it lives: table or cache slot)
   A w[E];
   {
     const P p = *reinterpret_cast<const P *>(wrow);
@@ -761,6 +771,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     int seg_begin, seg_end;
     int64_t key;
     RowPlace place;
+    T *storage;
   };
   auto row_at = [&](int slot) {
     const int u = uniform(long_queue[slot]);
@@ -775,6 +786,11 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     r.place.row_element = uniform(r.place.row_element);
     r.place.grad_stride = uniform(r.place.grad_stride);
     r.place.grad_column = uniform(r.place.grad_column);
+    r.storage = a.weights + r.place.row_element;
+    if (a.unique_slots) {
+      const int slot = uniform(a.unique_slots[u]);
+      if (slot >= 0) r.storage = a.cache_rows + static_cast<int64_t>(slot) * D;
+    }
     return r;
   };
   int first_total = uniform(counters[1]);  // the rows every wavefront helps with first
@@ -805,9 +821,9 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
           if (wave_in_block == 0) {
             // (one barrier per step inside the walk)
             if (r.place.row_D <= kWave)
-              walk_long_row<T, 1, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, lane, s_words);
+              walk_long_row<T, 1, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane, s_words);
             else
-              walk_long_row<T, 2, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, lane, s_words);
+              walk_long_row<T, 2, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane, s_words);
           } else {
             for (int s = 1; s <= steps; ++s) {
               if (s < steps)
@@ -868,11 +884,11 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     const QueuedRow r = row_at(slot);
     // elements per lane: the row spread over the 64 lanes, in loads of at most 16 bytes
     const int per_lane = (r.place.row_D + kWave - 1) / kWave;
-    if (per_lane <= 1) walk_long_row<T, 1, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, lane);
-    else if (per_lane <= 2) walk_long_row<T, 2, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, lane);
+    if (per_lane <= 1) walk_long_row<T, 1, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane);
+    else if (per_lane <= 2) walk_long_row<T, 2, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane);
     else if constexpr (sizeof(T) <= 4) {
-      if (per_lane <= 4) walk_long_row<T, 4, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, lane);
-      else if constexpr (sizeof(T) == 2) walk_long_row<T, 8, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, lane);
+      if (per_lane <= 4) walk_long_row<T, 4, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane);
+      else if constexpr (sizeof(T) == 2) walk_long_row<T, 8, WEIGHTED, STOCHASTIC, BIG>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane);
     }
   }
 }
@@ -895,6 +911,9 @@ struct ApproxArgs {
   // mixed-D tables: the rows of at most 64 vectors and kMixedShort occurrences are done and the
   // longer ones queued (update_mixed_approx_short); this queue holds the rows wider than 64 vectors
   const int32_t *wide_rows;
+  // cache-fronted uniform tables: slot of each unique row and the cache's rows (null otherwise)
+  const int32_t *unique_slots;
+  void *cache_rows;
 };
 
 template <typename T, int VEC>
@@ -936,7 +955,8 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
   if (!mixed) long_tables.T = 0;
   LongRowArgs<T> la{static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights), static_cast<A *>(a.state),
                     static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw), i32(l.positions_sorted),
-                    i32(l.grad_rows), lookup_wss, a.lr, a.eps, long_tables, a.sr, grad_bytes};
+                    i32(l.grad_rows), lookup_wss, a.lr, a.eps, long_tables, a.sr, grad_bytes, a.unique_slots,
+                    static_cast<T *>(a.cache_rows)};
   const bool big = grad_bytes >= (1ull << 32);
   const bool stochastic = sizeof(T) == 2 && a.sr.enabled;
 #define TBE_APPROX_LONG_KERNEL(WEIGHTED, STOCHASTIC, BIG)                                              \
@@ -959,7 +979,8 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
              static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),                       \
              static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),   \
              i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),     \
-             counters, long_queue, a.D, group, a.lr, a.eps, a.mt, a.sr, a.wide_rows);                  \
+             counters, long_queue, a.D, group, a.lr, a.eps, a.mt, a.sr, a.wide_rows, a.unique_slots,   \
+             static_cast<T *>(a.cache_rows));                                                          \
   TBE_APPROX_LONG(WEIGHTED, MIXED)
   if (mixed) {
     if (a.psw) { TBE_APPROX(true, true); }
@@ -987,6 +1008,8 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
     ua.learning_rate = a.lr;
     ua.eps = a.eps;
     ua.stochastic_rounding = a.sr;
+    ua.unique_slots = a.unique_slots;
+    ua.cache_rows = a.cache_rows;
     if (approx_sums_long_rows(a.dtype, a.D, a.psw != nullptr)) {
       // fp32 / fp64 rows without per-sample weights: the update of a row is a weighted sum of its
       // gradient rows, so the longer rows are summed in chunks like the exact update's
@@ -1022,10 +1045,11 @@ int approx_update(const void *grad_output, void *weights, void *state, const voi
                   int32_t dtype, int32_t fp16_vector_width, int32_t D, int64_t n, float lr, float eps,
                   const int64_t *mixed_table_offsets, const int32_t *table_dim_offsets,
                   const int32_t *dim_offsets, int32_t total_D, int32_t T, const int32_t *offsets, int32_t B,
-                  StochasticRounding sr, const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream) {
+                  StochasticRounding sr, const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream,
+                  const int32_t *unique_slots, void *cache_rows) {
   ApproxArgs a{grad_output, weights, state, psw, grad_psw, dtype, fp16_vector_width, D, n, lr, eps,
                MixedTables{mixed_table_offsets, table_dim_offsets, dim_offsets, total_D, T}, sr, offsets, B, T,
-               D == 0 ? approx_mixed_wide_queue(l, workspace) : nullptr};
+               D == 0 ? approx_mixed_wide_queue(l, workspace) : nullptr, unique_slots, cache_rows};
   char *ws = static_cast<char *>(workspace);
   // the queues of long rows borrow the chunk records' region: eight of approx_long_queue_capacity()
   // rows and one of the rows of more than kApproxHuge occurrences, or one queue of at most n / 9 rows
@@ -1086,4 +1110,45 @@ extern "C" int tbe_backward_approx_adagrad(const void *grad_output, void *weight
                        dtype, g.vec, D, num_indices, learning_rate, eps, nullptr, nullptr, nullptr, 0, T, offsets, B,
                        StochasticRounding{seed, offset, (stochastic_rounding && dtype == TBE_DTYPE_F16) ? 1 : 0},
                        l, workspace, s);
+}
+
+extern "C" int tbe_backward_approx_cached(const void *grad_output, const tbe_cache_t *cache, int32_t dtype,
+                                          int64_t total_rows, int32_t D, int32_t T, int32_t B,
+                                          int64_t num_indices, const int32_t *offsets,
+                                          const void *per_sample_weights, void *optimizer_state,
+                                          float learning_rate, float eps, void *grad_per_sample_weights,
+                                          int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
+                                          void *workspace, uint64_t workspace_bytes,
+                                          const int32_t *unique_slots, void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_backward_approx_cached";
+  TBE_REQUIRE(cache && cache->rows && cache->backing_rows, "%s: null cache", name);
+  TBE_REQUIRE(T > 0 && B > 0, "%s: T and B must be positive (got %d, %d)", name, T, B);
+  TBE_REQUIRE(D > 0 && D % 4 == 0, "%s: D must be a positive multiple of 4 (got %d)", name, D);
+  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
+  TBE_REQUIRE(total_rows > 0 && total_rows < INT32_MAX, "%s: total_rows out of range", name);
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(grad_output && offsets && optimizer_state, "%s: null pointer argument", name);
+  TBE_REQUIRE(unique_slots || num_indices == 0, "%s: null unique_slots", name);
+  TBE_REQUIRE((per_sample_weights == nullptr) == (grad_per_sample_weights == nullptr),
+              "%s: per_sample_weights and grad_per_sample_weights must both be given or both be null", name);
+  if (num_indices == 0) return TBE_OK;
+  tbe_workspace_layout_t l;
+  backward_layout(num_indices, D, dtype, T, &l);
+  if (!workspace || workspace_bytes < l.total_bytes)
+    return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
+                (unsigned long long)l.total_bytes, (unsigned long long)workspace_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const RowGeometry g = row_geometry(dtype, D);
+  if (int rc = approx_update(grad_output, cache->backing_rows, optimizer_state, per_sample_weights,
+                             grad_per_sample_weights, dtype, g.vec, D, num_indices, learning_rate, eps, nullptr,
+                             nullptr, nullptr, 0, T, offsets, B,
+                             StochasticRounding{seed, offset, (stochastic_rounding && dtype == TBE_DTYPE_F16) ? 1 : 0},
+                             l, workspace, s, unique_slots, cache->rows))
+    return rc;
+  if (cache->stage_slots <= 0) return TBE_OK;
+  const char *ws = static_cast<const char *>(workspace);
+  return cache_unstage(cache, dtype, D, reinterpret_cast<const int32_t *>(ws + l.keys_sorted),
+                       reinterpret_cast<const int32_t *>(ws + l.segment_starts),
+                       reinterpret_cast<const int32_t *>(ws + l.num_unique), unique_slots, num_indices, s);
 }

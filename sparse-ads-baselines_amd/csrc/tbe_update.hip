@@ -854,8 +854,8 @@ void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *que
              static_cast<T *>(nullptr), a.keys_sorted, a.positions_sorted, a.grad_rows, a.segment_starts,       \
              a.segment_ids, a.counters, reinterpret_cast<LongRecord *>(a.long_segments),                        \
              reinterpret_cast<ChunkRecord *>(a.chunk_segments), a.max_chunks, a.num_indices, num_tiles,         \
-             tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr),       \
-             static_cast<T *>(nullptr), a.stochastic_rounding, static_cast<int32_t *>(nullptr))
+             tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots,                              \
+             static_cast<T *>(a.cache_rows), a.stochastic_rounding, static_cast<int32_t *>(nullptr))
       if (small) { TBE_APPROX_SUM_SHORT(true); }
       else { TBE_APPROX_SUM_SHORT(false); }
 #undef TBE_APPROX_SUM_SHORT
@@ -871,8 +871,8 @@ void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *que
              a.keys_sorted, a.positions_sorted, a.grad_rows, a.segment_starts, a.segment_ids, a.counters,       \
              static_cast<LongRecord *>(nullptr), static_cast<ChunkRecord *>(nullptr),                           \
              kNumXcd * approx_long_queue_capacity(a.num_indices), a.num_indices, num_tiles, tiles_per_xcd,      \
-             a.D, g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr),                      \
-             static_cast<T *>(nullptr), a.stochastic_rounding, queue)
+             a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, static_cast<T *>(a.cache_rows),             \
+             a.stochastic_rounding, queue)
   if (small) { TBE_APPROX_SHORT(true); }
   else { TBE_APPROX_SHORT(false); }
 #undef TBE_APPROX_SHORT
@@ -971,14 +971,14 @@ void launch_approx_sum_long(const UpdateArgs &a, const RowGeometry &g, const voi
                (update_chunks_kernel<T, VEC, CHUNKS, kOptSgd, false, kLongUnroll, true>), grid_chunks, block,
                static_cast<const T *>(a.grad_output), w, st, static_cast<const T *>(lookup_wss),
                static_cast<T *>(nullptr), a.positions_sorted, a.grad_rows, a.counters, chunk_records, a.max_chunks,
-               partial, a.D, g.chunks, a.learning_rate, a.eps, static_cast<const int32_t *>(nullptr),
-               static_cast<T *>(nullptr), a.stochastic_rounding, a.segment_starts);
+               partial, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, static_cast<T *>(a.cache_rows),
+               a.stochastic_rounding, a.segment_starts);
     const int64_t want_long = ceil_div(a.max_long, kWavesPerBlock);
     const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
     // (the partial rows already carry the multipliers: the row takes their sum as it is)
     TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, kOptSgd>), grid_finish,
-               block, w, st, a.counters, long_records, partial, a.D, g.chunks, 1.0f, a.eps,
-               static_cast<const int32_t *>(nullptr), static_cast<T *>(nullptr), a.stochastic_rounding);
+               block, w, st, a.counters, long_records, partial, a.D, g.chunks, 1.0f, a.eps, a.unique_slots,
+               static_cast<T *>(a.cache_rows), a.stochastic_rounding);
     TBE_LAUNCH("update_approx_state", stream, (approx_long_state_kernel<A>), grid_finish, block, st,
                static_cast<const A *>(lookup_wss), a.positions_sorted, a.segment_starts, a.counters, long_records);
   }

@@ -274,7 +274,8 @@ class RowCache:
 
     def backward(self, optimizer, grad_output, per_sample_weights, optimizer_state, learning_rate, eps,
                  stochastic_rounding=None, plan_id=None):
-        """optimizer: 'sgd' or 'adagrad'.  Updates rows where they live; returns the gradient
+        """optimizer: 'sgd', 'adagrad' (exact row-wise Adagrad) or 'approx_adagrad' (the reference's
+        per-lookup row-wise Adagrad, lookups of a row applied in position order).  Updates rows where they live; returns the gradient
         w.r.t. per_sample_weights or None.  stochastic_rounding: None, or the (seed, offset) of
         the random stream that rounds updated fp16 weights (Adagrad only).  plan_id: the value of
         self.plan_id after the prepare() of the batch this gradient belongs to; a later prepare()
@@ -298,8 +299,20 @@ class RowCache:
         grad_psw = None
         if per_sample_weights is not None:
             grad_psw = torch.empty(p.n, dtype=grad_output.dtype, device=self.device)
+        if optimizer not in ("sgd", "adagrad", "approx_adagrad"):
+            raise ValueError("optimizer must be 'sgd', 'adagrad' or 'approx_adagrad' (got %r)" % (optimizer,))
         code = _native.OPT_SGD if optimizer == "sgd" else _native.OPT_ROWWISE_ADAGRAD
         unique = self._view(p.cws, p.layout.unique_slots, max(p.n, 1))
+        if optimizer == "approx_adagrad":
+            with torch.cuda.device(self.device):
+                _native.check(_native.load().tbe_backward_approx_cached(
+                    _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.backing.size(0), self.D,
+                    p.T, p.B, p.n, _ptr(p.offsets), _ptr(per_sample_weights), _ptr(optimizer_state),
+                    float(learning_rate), float(eps or 0.0), _ptr(grad_psw), int(stochastic_rounding is not None),
+                    stochastic_rounding[0] if stochastic_rounding else 0,
+                    stochastic_rounding[1] if stochastic_rounding else 0, _ptr(p.ws), p.ws.numel(), _ptr(unique),
+                    self._stream()))
+            return grad_psw
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_backward_cached(
                 code, _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.backing.size(0), self.D,

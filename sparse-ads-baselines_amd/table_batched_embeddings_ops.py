@@ -138,10 +138,12 @@ class CachedLookupFunction(torch.autograd.Function):
         if module.optimizer == Optimizer.SGD:
             assert per_sample_weights is None
             kind = "sgd"
+        elif module.optimizer == Optimizer.APPROX_ROWWISE_ADAGRAD:
+            kind = "approx_adagrad"
         else:
             kind = "adagrad"
         rounding = None
-        if module.stochastic_rounding and kind == "adagrad" and weights.dtype == torch.float16:
+        if module.stochastic_rounding and kind != "sgd" and weights.dtype == torch.float16:
             rounding = table_batched_embeddings._rounding_stream(weights.device)
         grad_per_sample_weight = module.row_cache.backward(
             kind, grad_output, per_sample_weights, module.optimizer_state, module.learning_rate, module.eps,
@@ -189,8 +191,6 @@ class TableBatchedEmbeddingBags(nn.Module):
         self.row_cache = None
         if managed == EmbeddingLocation.HOST_CACHED:
             assert cache_slots is not None, "HOST_CACHED needs cache_slots"
-            if optimizer == Optimizer.APPROX_ROWWISE_ADAGRAD:
-                raise NotImplementedError("cache-fronted tables serve SGD and EXACT_ROWWISE_ADAGRAD")
             self.row_cache = table_batched_embeddings_cache.RowCache(self.embedding_weights.data, cache_slots,
                                                                      cache_policy, cache_stage_slots,
                                                                      cache_deferred_write_back)

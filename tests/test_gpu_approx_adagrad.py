@@ -471,6 +471,23 @@ def test_module_with_the_approximate_optimizer_and_repeated_rows(oracle):
         assert_close(psw.grad.cpu().numpy(), g_ref, 1e-5)
     assert_close(cc.optimizer_state.cpu().numpy(), st_ref, 1e-5)
     assert_close(cc.embedding_weights.detach().cpu().numpy(), w_ref, 1e-5)
-    with pytest.raises(NotImplementedError):
-        ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.APPROX_ROWWISE_ADAGRAD,
-                                      managed=ops.EmbeddingLocation.HOST_CACHED, cache_slots=64)
+    # behind the row cache the module follows the same trajectory, bit for bit
+    plain = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.APPROX_ROWWISE_ADAGRAD, learning_rate=0.5,
+                                          eps=0.2).cuda()
+    cached = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.APPROX_ROWWISE_ADAGRAD, learning_rate=0.5,
+                                           eps=0.2, managed=ops.EmbeddingLocation.HOST_CACHED, cache_slots=128,
+                                           cache_stage_slots=64).cuda()
+    plain.embedding_weights.data.copy_(dev(p["weights"]))
+    cached.embedding_weights.data.copy_(dev(p["weights"]))
+    for _ in range(3):
+        psw_a = dev(p["per_sample_weights"]).requires_grad_(True)
+        psw_b = dev(p["per_sample_weights"]).requires_grad_(True)
+        a = plain(dev(p["indices"]), dev(p["offsets"]), psw_a)
+        a.backward(dev(p["grad_output"]))
+        b = cached(dev(p["indices"]), dev(p["offsets"]), psw_b)
+        b.backward(dev(p["grad_output"]))
+        assert torch.equal(a, b) and torch.equal(psw_a.grad, psw_b.grad)
+    sd = cached.state_dict()
+    torch.cuda.synchronize()
+    assert torch.equal(sd["embedding_weights"], plain.embedding_weights.data)
+    assert torch.equal(sd["optimizer_state"], plain.optimizer_state)

@@ -94,7 +94,9 @@ def test_many_misses_per_set(oracle, num_sets, stage_slots):
 
 @pytest.mark.parametrize("mode,dtype,D", [("sgd", torch.float32, 128), ("adagrad", torch.float32, 64),
                                           ("adagrad_weighted", torch.float16, 64), ("sgd", torch.float32, 520),
-                                          ("sgd", torch.float64, 12)])
+                                          ("sgd", torch.float64, 12), ("approx", torch.float32, 128),
+                                          ("approx_weighted", torch.float16, 64), ("approx", torch.float16, 32),
+                                          ("approx_weighted", torch.float32, 520), ("approx", torch.float64, 12)])
 @pytest.mark.parametrize("num_sets,stage_slots,deferred", [(2, 0, False), (40, 0, False), (2, 4096, False),
                                                           (2, 7, False), (2, 4096, True), (2, 7, True),
                                                           (5, 300, True)])
@@ -105,7 +107,10 @@ def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, sta
     served straight from the backing table; with 40 most are cached.  With a staging area the rows
     that find no slot are staged in HBM for the step and copied back after the update (all of
     them with 4096 staging rows, some with 7) -- or, with deferred write-back, kept until the next
-    step, which fetches the rows it needs again from there and writes the others back."""
+    step, which fetches the rows it needs again from there and writes the others back.
+    The approximate (per-lookup) Adagrad goes through its own kernels -- tiles of short rows, chunk
+    sums or a wavefront's walk for the rows of many occurrences, the kernel for rows wider than a
+    wavefront -- each of which has to find a row where it lives."""
     rs = np.random.RandomState(3)
     T, rows, B, L = 3, [700, 90, 3000], 48, 9
     table_offsets = dev(np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
@@ -119,7 +124,7 @@ def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, sta
     cached_state = torch.zeros(total, device=DEV, dtype=st_dtype)
     cache = tc.RowCache(cached_w, num_sets * 64, "lru", stage_slots, deferred_write_back=deferred)
     weighted = mode.endswith("weighted")
-    opt = "sgd" if mode == "sgd" else "adagrad"
+    opt = "sgd" if mode == "sgd" else "approx_adagrad" if mode.startswith("approx") else "adagrad"
     served_uncached = served_staged = 0
     for step in range(6):
         indices, offsets = _draw_batch(rs, T, rows, B, L, 1.2)
@@ -130,6 +135,9 @@ def test_cached_training_equals_uncached_bit_exact(mode, dtype, D, num_sets, sta
         if opt == "sgd":
             ext.backward_sgd(go, plain_w, table_offsets, idx, off, 0.05, 200, 1, False)
             want_g = None
+        elif opt == "approx_adagrad":
+            want_g = ext.backward_approx_adagrad(go, plain_w, table_offsets, idx, off, psw, plain_state, 0.05, 0.1,
+                                                 200, False, 1)
         else:
             want_g = ext.backward_exact_adagrad(go, plain_w, table_offsets, idx, off, psw, plain_state, 0.05, 0.1,
                                                 False, 1)
@@ -339,6 +347,42 @@ def test_cached_stochastic_rounding_equals_uncached_bit_exact():
     ext.backward_exact_adagrad(go, rn_w, table_offsets, idx, off, None, torch.zeros(total, device=DEV), 0.05, 0.1,
                                False, 1)
     assert not torch.equal(rn_w, start)
+
+
+def test_cached_approx_adagrad_with_stochastic_rounding_equals_uncached_bit_exact():
+    """The approximate Adagrad with stochastic rounding behind the cache (hot rows take the walk
+    that draws a random word per element and occurrence): bit-identical to the uncached update."""
+    import ctypes
+    import tbe_native
+    rs = np.random.RandomState(9)
+    T, rows, B, L, D = 2, [900, 40], 64, 8, 64
+    table_offsets = dev(np.concatenate([[0], np.cumsum(rows[:-1])]).astype(np.int32))
+    total = sum(rows)
+    start = (torch.rand(total, D, device=DEV) * 0.02 - 0.01).half()
+    plain_w, cached_w = start.clone(), start.clone()
+    plain_state, cached_state = torch.zeros(total, device=DEV), torch.zeros(total, device=DEV)
+    cache = tc.RowCache(cached_w, 2 * 64, "lru", stage_slots=50)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    longest = 0
+    for step in range(4):
+        indices, offsets = _draw_batch(rs, T, rows, B, L, 1.2)
+        longest = max(longest, int(np.bincount(indices[offsets[B]:]).max()))
+        idx, off = dev(indices), dev(offsets)
+        go = torch.randn(B, T, D, device=DEV).half()
+        lay = tbe_native.backward_workspace_layout(indices.size, D, tbe_native.DTYPE_F16, T)
+        ws = torch.empty(lay.total_bytes, dtype=torch.uint8, device=DEV)
+        tbe_native.check(tbe_native.load().tbe_backward_approx_adagrad(
+            vp(go), vp(plain_w), tbe_native.DTYPE_F16, total, 0, D, vp(table_offsets), T, vp(idx), indices.size,
+            vp(off), B, None, vp(plain_state), 0.05, 0.1, None, 1, 99, 4 * step, vp(ws), ws.numel(),
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        cache.prepare(table_offsets, idx, off)
+        cache.backward("approx_adagrad", go, None, cached_state, 0.05, 0.1, stochastic_rounding=(99, 4 * step))
+        st = cache.stats()
+        assert st["staged"] > 0 and st["uncached"] > 0 and st["hits"] + st["inserted"] > 0
+    assert longest > 16, "no row long enough for the wavefront's walk"
+    cache.flush()
+    torch.cuda.synchronize()
+    assert torch.equal(cached_w, plain_w) and torch.equal(cached_state, plain_state)
 
 
 def test_flush_before_any_step_and_empty_batch():
