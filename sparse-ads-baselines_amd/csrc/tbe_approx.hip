@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_lookup_norms_kernel(
   using A = typename V::A;
   int queued = counters[1];  // (one queue, or one per XCD)
 #pragma unroll
-  for (int x = 0; x < kNumXcd; ++x) queued += counters[kChunkQueueCount + x];
+  for (int x = 0; x < kNumXcd; ++x) queued += counters[xcd_counter(x)];
   if (queued == 0) return;
   const int lane = threadIdx.x & (kWave - 1);
   const int r = lane / group;
@@ -758,7 +758,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int wave_in_block = uniform(static_cast<int>(threadIdx.x >> 6));
   // queue_capacity == 0: one queue, its length in counters[1].  Otherwise, as the short-row kernel
-  // leaves them: one queue per XCD (lengths in counters[kChunkQueueCount ...]) and behind them the
+  // leaves them: one queue per XCD (lengths in counters[xcd_counter(x)]) and behind them the
   // queue of the rows of more than kApproxHuge occurrences (counters[1]).  Those come first, one
   // per wavefront, so that the longest walks start when the kernel does.  Then the workgroups of
   // an XCD take their own queue in order -- it is in (table, row) order, so the gradient rows of a
@@ -849,7 +849,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
   int total = 0;
 #pragma unroll
   for (int x = 0; x < kNumXcd; ++x) {
-    queue_len[x] = queue_capacity > 0 ? uniform(counters[kChunkQueueCount + x]) : 0;
+    queue_len[x] = queue_capacity > 0 ? uniform(counters[xcd_counter(x)]) : 0;
     total += queue_len[x];
   }
   const int fair = total / kNumXcd + total / 16 + 1;

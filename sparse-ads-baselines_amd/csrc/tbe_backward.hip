@@ -37,9 +37,11 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspac
   const uint64_t ints = align_up(nn * 4, 256);
   // a segment enters the chunk queue when it has more than kShortSegment occurrences and owns
   // partial rows when it has more than kChunkLen
-  l->max_long_segments = static_cast<int64_t>(nn / (kChunkLen + 1) + 1);
+  // (one list per XCD: the segments of several chunks that start in its eighth of the sorted positions)
+  l->max_long_segments = static_cast<int64_t>(kNumXcd * long_list_capacity(static_cast<int64_t>(nn)));
   l->max_chunks = static_cast<int64_t>(kNumXcd * chunk_queue_capacity(static_cast<int64_t>(nn)));
-  l->max_partial_rows = static_cast<int64_t>(nn / kChunkLen + nn / (kChunkLen + 1) + 2);
+  // (a partial row's number follows from where its chunk lies, two per kChunkLen sorted positions)
+  l->max_partial_rows = static_cast<int64_t>(2 * (nn / kChunkLen + 1));
   uint64_t off = 0;
   // the linearized keys are only written (and sorted in one piece) for more tables than are sorted apart
   l->keys = off;
@@ -52,7 +54,7 @@ void compute_layout(int64_t n, int32_t D, int32_t dtype, int32_t T, tbe_workspac
   l->keys_sorted = off; off += ints;
   l->positions_sorted = off; off += ints;
   l->segment_starts = off; off += align_up((nn + 1) * 4, 256);
-  l->num_unique = off; off += 256;
+  l->num_unique = off; off += align_up(static_cast<uint64_t>(kNumCounters) * 4, 256);
   l->sort_scratch = off; off += align_up(sort_workspace_bytes(n, sort_tables(T)), 256);
   l->segment_scratch = off; off += align_up(segments_workspace_bytes(n), 256);
   l->segment_ids = off; off += ints;

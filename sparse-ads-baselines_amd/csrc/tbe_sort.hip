@@ -735,7 +735,10 @@ __global__ __launch_bounds__(kBlockThreads) void segment_scan_kernel(
     segment_starts[carry] = static_cast<int32_t>(n);
   }
   // the update stage keeps its queue counters next to U; starting them at zero here saves a launch
-  if (clear_queue_counters && tid >= 1 && tid < kNumCounters) num_unique[tid] = 0;
+  if (clear_queue_counters) {
+    for (int i = tid; i < kNumCounters; i += kBlockThreads)
+      if (i >= 1) num_unique[i] = 0;
+  }
 }
 
 // The heads of a tile are compacted in LDS and leave as one contiguous run; the segment of
@@ -769,7 +772,10 @@ __global__ __launch_bounds__(kBlockThreads) void segment_write_kernel(
         num_unique[0] = static_cast<int32_t>(base + total);
         segment_starts[base + total] = static_cast<int32_t>(n);
       }
-      if (clear_queue_counters && threadIdx.x >= 1 && threadIdx.x < kNumCounters) num_unique[threadIdx.x] = 0;
+      if (clear_queue_counters) {
+        for (int i = threadIdx.x; i < kNumCounters; i += kBlockThreads)
+          if (i >= 1) num_unique[i] = 0;
+      }
     }
   } else {
     base = tile_base[blockIdx.x];

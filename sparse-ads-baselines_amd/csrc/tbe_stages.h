@@ -56,10 +56,17 @@ int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts
 constexpr int kShortSegment = 128;
 constexpr int kApproxShortSegment = 16;
 constexpr int kChunkLen = 256;
-// Integers kept next to the number of unique rows (all zeroed when the segments are found):
-// [1] long rows, [3] partial rows, [8..15] chunk records queued by each XCD.
-constexpr int kNumCounters = 16;
-constexpr int kChunkQueueCount = 8;
+// Integers kept next to the number of unique rows (all zeroed when the segments are found): [1], [2]
+// queue lengths of the kernels that keep one queue (mixed-D tables, the approximate update), and from
+// word 64 on one 128-byte line per XCD: [0] chunk records (or rows) queued by the XCD's workgroups,
+// [1] its segments of several chunks.  A line of its own, because the workgroups of an XCD queue
+// with one 64-bit atomic add on those two words, and atomic adds on one line queue up behind each
+// other (with all counters of the chip on one line, a skewed batch spent 26 us of a 180 us kernel
+// waiting for them).
+constexpr int kXcdCounterBase = 64;
+constexpr int kXcdCounterStride = 32;
+constexpr int kNumCounters = kXcdCounterBase + 8 * kXcdCounterStride;
+__host__ __device__ constexpr int xcd_counter(int xcd) { return kXcdCounterBase + kXcdCounterStride * xcd; }
 constexpr int kApproxHuge = 256;   // occurrences from which on the approximate update walks a row before the others
 // The short-row kernel's workgroups of XCD x own the segments that start in the x-th eighth of
 // the sorted positions (rounded up to whole workgroups: fewer than 1200 positions more) and queue
@@ -71,6 +78,17 @@ inline int64_t chunk_queue_capacity(int64_t n) {
   // (sized for the smaller of the two thresholds: the approximate update of fp32 rows queues its
   // chunk records here too)
   return eighth / (kApproxShortSegment + 1) + eighth / kChunkLen + n / kChunkLen + 8;
+}
+
+// Room of one XCD's list of segments of several chunks (more than kChunkLen occurrences each) that
+// start in its eighth of the sorted positions.
+inline int64_t long_list_capacity(int64_t n) { return ((n + 7) / 8 + 2048) / (kChunkLen + 1) + 2; }
+// The partial row of chunk k of a segment [begin, end) of several chunks.  Every chunk but a segment's
+// last is kChunkLen positions long, so no two of them begin in the same window of kChunkLen positions;
+// and segments of several chunks end more than kChunkLen positions apart, so no two last chunks end in
+// the same window: two rows per window, no counter.
+__host__ __device__ inline int partial_row_of_chunk(int begin, int end, int k, int num_chunks) {
+  return k == num_chunks - 1 ? 2 * ((end - 1) / kChunkLen) + 1 : 2 * ((begin + k * kChunkLen) / kChunkLen);
 }
 
 // Room of one XCD's queue of rows that the approximate update's short-row kernel leaves to the
@@ -93,7 +111,7 @@ struct UpdateArgs {
   const int32_t *segment_starts;
   int32_t *counters;            // [0] = U (input), [1] = #long records, [2] = #chunk records, [3] = #partial rows
   const int32_t *segment_ids;   // [N] segment of every sorted position
-  void *long_segments;          // 16-byte records [max_long]: segments cut into several chunks
+  void *long_segments;          // 16-byte records [8][max_long / 8]: segments cut into several chunks, one list per XCD
   void *chunk_segments;         // 32-byte records [8][max_chunks / 8]: one chunk queue per XCD
   void *partial_sums;           // acc [max_partial][D]
   const int32_t *unique_slots;  // cache-fronted tables: slot of each unique row (-1 = not resident)

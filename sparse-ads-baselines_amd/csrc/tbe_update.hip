@@ -103,7 +103,7 @@ struct ChunkRecord {   // 32 bytes
   int32_t pad[3];
 };
 struct LongRecord {    // 16 bytes: a segment cut into several chunks
-  int32_t u, key, first_partial, num_chunks;
+  int32_t u, key, begin, end;  // unique-row number, row, sorted positions [begin, end)
 };
 
 // APPROX (row-wise Adagrad only): the approximate optimizer's per-lookup update
@@ -122,8 +122,8 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ segment_ids,
     int32_t *__restrict__ counters, LongRecord *__restrict__ long_records,
-    ChunkRecord *__restrict__ chunk_records, int64_t max_chunks, int64_t n, int64_t num_tiles,
-    int64_t tiles_per_xcd, int D_rt, int chunks_rt, float lr, float eps,
+    ChunkRecord *__restrict__ chunk_records, int64_t max_chunks, int64_t max_long, int64_t n,
+    int64_t num_tiles, int64_t tiles_per_xcd, int D_rt, int chunks_rt, float lr, float eps,
     const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, StochasticRounding sr,
     int32_t *__restrict__ approx_long_queue) {
   using V = RowVec<T, VEC>;
@@ -159,16 +159,16 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
   const int64_t col = static_cast<int64_t>(c) * VEC;
 
   // Segments that start in [p0, p1): the segment containing p0 belongs to this tile only if
-  // p0 is its head.
+  // p0 is its head, i.e. if the position before it lies in another segment.  Three segment
+  // numbers, fetched together, say it all: a tile inside one long row (most tiles of a skewed
+  // batch) is done after one round trip.
   const int64_t p0 = tile * kTilePositions;
   const int64_t p1 = min(n, p0 + kTilePositions);
-  const bool last_tile = p1 >= n;
+  const int id_before = segment_ids[max(p0 - 1, int64_t{0})];
   const int id0 = segment_ids[p0];
-  const int id1 = last_tile ? 0 : segment_ids[p1];
-  const int start0 = segment_starts[id0];
-  const int start1 = last_tile ? 0 : segment_starts[id1];
-  const int u_first = id0 + (start0 != p0 ? 1 : 0);
-  const int u_limit = last_tile ? counters[0] : id1 + (start1 != p1 ? 1 : 0);
+  const int id_last = segment_ids[p1 - 1];
+  const int u_first = id0 + ((p0 > 0 && id_before == id0) ? 1 : 0);
+  const int u_limit = id_last + 1;
   const int nseg = u_limit - u_first;  // <= kTilePositions
   if (nseg <= 0) return;
 
@@ -234,7 +234,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
         // and one behind them for the rows of very many occurrences
         if (c == 0) {
           if (len > kApproxHuge) approx_long_queue[max_chunks + atomicAdd(&counters[1], 1)] = u;
-          else approx_long_queue[xcd * (max_chunks / kNumXcd) + atomicAdd(&counters[kChunkQueueCount + xcd], 1)] = u;
+          else approx_long_queue[xcd * (max_chunks / kNumXcd) + atomicAdd(&counters[xcd_counter(xcd)], 1)] = u;
         }
         continue;
       }
@@ -242,23 +242,26 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
     if (len > kShort) {
       // Hand the segment to the chunk queue.
       const int nch = (len + kChunkLen - 1) / kChunkLen;
-      int first_chunk = 0, first_partial = -1;
+      int first_chunk = 0;
       if (c == 0) {
-        first_chunk = atomicAdd(&counters[kChunkQueueCount + xcd], nch);
-        if (nch > 1) {
-          first_partial = atomicAdd(&counters[3], nch);
-          long_records[atomicAdd(&counters[1], 1)] = LongRecord{u, key, first_partial, nch};
-        }
+        // one atomic add on the XCD's own line: its low word hands out the queue slots, its high
+        // word the place in the XCD's list of segments of several chunks
+        const unsigned long long taken = atomicAdd(
+            reinterpret_cast<unsigned long long *>(counters + xcd_counter(xcd)),
+            static_cast<unsigned long long>(nch) | (nch > 1 ? 1ull << 32 : 0ull));
+        first_chunk = static_cast<int>(taken & 0xffffffffull);
+        if (nch > 1)
+          long_records[xcd * (max_long / kNumXcd) + static_cast<int64_t>(taken >> 32)] =
+              LongRecord{u, key, seg_begin, seg_end};
       }
       first_chunk = shfl_idx(first_chunk, group_base);
-      first_partial = shfl_idx(first_partial, group_base);
       for (int k = c; k < nch; k += chunks) {
         ChunkRecord rec;
         rec.begin = seg_begin + k * kChunkLen;
         rec.end = min(seg_end, rec.begin + kChunkLen);
         rec.key = key;
         rec.u = u;
-        rec.partial = nch > 1 ? first_partial + k : -1;
+        rec.partial = nch > 1 ? partial_row_of_chunk(seg_begin, seg_end, k, nch) : -1;
         rec.pad[0] = rec.pad[1] = rec.pad[2] = 0;
         chunk_queue[first_chunk + k] = rec;
       }
@@ -406,7 +409,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
   int64_t total = 0;
 #pragma unroll
   for (int x = 0; x < kNumXcd; ++x) {
-    queue_len[x] = counters[kChunkQueueCount + x];
+    queue_len[x] = counters[xcd_counter(x)];
     total += queue_len[x];
   }
   const int fair = static_cast<int>(total / kNumXcd + total / 16 + 1);
@@ -575,22 +578,56 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
   }
 }
 
+// The segments of several chunks are listed per XCD (long_records[x][...], lengths in the high word
+// of each XCD's counter line).  A wavefront walks the concatenation of the eight lists.
+struct LongLists {
+  int len[kNumXcd];
+  int64_t total;
+  int64_t capacity;  // records per list
+};
+__device__ __forceinline__ LongLists long_lists(const int32_t *__restrict__ counters, int64_t max_long) {
+  LongLists l;
+  l.total = 0;
+  l.capacity = max_long / kNumXcd;
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) {
+    l.len[x] = counters[xcd_counter(x) + 1];
+    l.total += l.len[x];
+  }
+  return l;
+}
+__device__ __forceinline__ LongRecord long_record_at(const LongRecord *__restrict__ long_records, const LongLists &l,
+                                                     int64_t slot) {
+  // (straight-line: a list picked by a run-time index would put the eight lengths into scratch memory)
+  int64_t at = 0;
+  bool found = false;
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) {
+    if (!found && slot < l.len[x]) {
+      at = x * l.capacity + slot;
+      found = true;
+    }
+    slot -= l.len[x];
+  }
+  return long_records[at];
+}
+
 // The approximate Adagrad's rows that were summed in several chunks: their state takes the addends
 // of all their lookups (one wavefront per row; update_long_finish_kernel writes the row itself).
 template <typename A>
 __global__ __launch_bounds__(kBlockThreads) void approx_long_state_kernel(
     A *__restrict__ state, const A *__restrict__ lookup_wss, const int32_t *__restrict__ positions_sorted,
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
-    const LongRecord *__restrict__ long_records) {
+    const LongRecord *__restrict__ long_records, int64_t max_long) {
   constexpr int kAhead = 16;
   const int lane = threadIdx.x & (kWave - 1);
-  const int num_long = counters[1];
+  const LongLists lists = long_lists(counters, max_long);
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
-  for (int64_t slot = wave_id; slot < num_long; slot += stride) {
-    const LongRecord rec = long_records[slot];
-    const int seg_begin = segment_starts[rec.u];
-    const int seg_end = segment_starts[rec.u + 1];
+  for (int64_t slot = wave_id; slot < lists.total; slot += stride) {
+    const LongRecord rec = long_record_at(long_records, lists, slot);
+    const int seg_begin = rec.begin;
+    const int seg_end = rec.end;
     A sum = A(0);
     for (int i0 = seg_begin; i0 < seg_end; i0 += kAhead * kWave) {
       int p[kAhead];
@@ -617,7 +654,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     const int32_t *__restrict__ counters, const LongRecord *__restrict__ long_records,
     const typename AccOf<T>::type *__restrict__ partial_sums, int D_rt, int chunks_rt, float lr,
     float eps, const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows,
-    StochasticRounding sr) {
+    StochasticRounding sr, int64_t max_long) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   // (a compile-time row width turns every row address into a shift)
@@ -629,13 +666,14 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
   const int r = lane / chunks;
   const int c = lane - r * chunks;
   const bool active = r < groups;
-  const int num_long = counters[1];
+  const LongLists lists = long_lists(counters, max_long);
   const int64_t col = static_cast<int64_t>(c) * VEC;
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
 
-  for (int64_t slot = wave_id; slot < num_long; slot += stride) {
-    const LongRecord rec = long_records[slot];
+  for (int64_t slot = wave_id; slot < lists.total; slot += stride) {
+    const LongRecord rec = long_record_at(long_records, lists, slot);
+    const int num_chunks = (rec.end - rec.begin + kChunkLen - 1) / kChunkLen;
     T *wrow = resolve_row(weights, cache_rows, unique_slots, rec.u, static_cast<int64_t>(rec.key), D) + col;
     V w_old;
     w_old.zero();
@@ -647,18 +685,19 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_kernel(
     if (active) {
       // eight partial rows are requested before the first is added (same order of additions)
       constexpr int kAhead = 8;
-      for (int k0 = r; k0 < rec.num_chunks; k0 += groups * kAhead) {
+      for (int k0 = r; k0 < num_chunks; k0 += groups * kAhead) {
         A part[kAhead][VEC];
 #pragma unroll
         for (int a = 0; a < kAhead; ++a) {
-          const int k = min(k0 + a * groups, rec.num_chunks - 1);  // clamped: no branch per load
-          const A *src = partial_sums + static_cast<int64_t>(rec.first_partial + k) * D + col;
+          const int k = min(k0 + a * groups, num_chunks - 1);  // clamped: no branch per load
+          const A *src =
+              partial_sums + static_cast<int64_t>(partial_row_of_chunk(rec.begin, rec.end, k, num_chunks)) * D + col;
 #pragma unroll
           for (int i = 0; i < VEC; ++i) part[a][i] = src[i];
         }
 #pragma unroll
         for (int a = 0; a < kAhead; ++a) {
-          const bool real = k0 + a * groups < rec.num_chunks;
+          const bool real = k0 + a * groups < num_chunks;
 #pragma unroll
           for (int i = 0; i < VEC; ++i) G.v[i] += real ? part[a][i] : A(0);
         }
@@ -808,7 +847,7 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
              (update_short_kernel<T, VEC, CHUNKS, OPT, WEIGHTED, kShortUnroll, false, false, SMALL>),       \
              grid_short, block, go, w, st, psw, gpsw, a.keys_sorted, a.positions_sorted, a.grad_rows,       \
              a.segment_starts, a.segment_ids, a.counters, long_records, chunk_records, a.max_chunks,        \
-             a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,                \
+             a.max_long, a.num_indices, num_tiles, tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps,                \
              a.unique_slots, cr, a.stochastic_rounding, static_cast<int32_t *>(nullptr))
   if (small) { TBE_UPDATE_SHORT(true); }
   else { TBE_UPDATE_SHORT(false); }
@@ -830,12 +869,12 @@ void launch_narrow(const UpdateArgs &a, const RowGeometry &g, hipStream_t stream
   const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
   TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, OPT>),
              grid_finish, block, w, st, a.counters, long_records, partial, a.D, g.chunks,
-             a.learning_rate, a.eps, a.unique_slots, cr, a.stochastic_rounding);
+             a.learning_rate, a.eps, a.unique_slots, cr, a.stochastic_rounding, a.max_long);
 }
 
 // The short-row kernel alone, in its per-lookup (approximate Adagrad) form; rows of more than
 // kApproxShortSegment occurrences are left in `queue`: eight queues of approx_long_queue_capacity() row
-// numbers, one per XCD, their lengths in counters[kChunkQueueCount ...].
+// numbers, one per XCD, their lengths in counters[xcd_counter(x)].
 template <typename T, int VEC, int CHUNKS, bool WEIGHTED>
 void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *queue, hipStream_t stream) {
   using A = typename AccOf<T>::type;
@@ -853,7 +892,8 @@ void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *que
              static_cast<T *>(a.weights), static_cast<A *>(a.optimizer_state), static_cast<const T *>(nullptr), \
              static_cast<T *>(nullptr), a.keys_sorted, a.positions_sorted, a.grad_rows, a.segment_starts,       \
              a.segment_ids, a.counters, reinterpret_cast<LongRecord *>(a.long_segments),                        \
-             reinterpret_cast<ChunkRecord *>(a.chunk_segments), a.max_chunks, a.num_indices, num_tiles,         \
+             reinterpret_cast<ChunkRecord *>(a.chunk_segments), a.max_chunks, a.max_long, a.num_indices,        \
+             num_tiles,                                                                                         \
              tiles_per_xcd, a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots,                              \
              static_cast<T *>(a.cache_rows), a.stochastic_rounding, static_cast<int32_t *>(nullptr))
       if (small) { TBE_APPROX_SUM_SHORT(true); }
@@ -870,7 +910,8 @@ void launch_approx_short(const UpdateArgs &a, const RowGeometry &g, int32_t *que
              static_cast<const T *>(a.per_sample_weights), static_cast<T *>(a.grad_per_sample_weights),         \
              a.keys_sorted, a.positions_sorted, a.grad_rows, a.segment_starts, a.segment_ids, a.counters,       \
              static_cast<LongRecord *>(nullptr), static_cast<ChunkRecord *>(nullptr),                           \
-             kNumXcd * approx_long_queue_capacity(a.num_indices), a.num_indices, num_tiles, tiles_per_xcd,      \
+             kNumXcd * approx_long_queue_capacity(a.num_indices), int64_t{0}, a.num_indices, num_tiles,         \
+             tiles_per_xcd,                                                                                     \
              a.D, g.chunks, a.learning_rate, a.eps, a.unique_slots, static_cast<T *>(a.cache_rows),             \
              a.stochastic_rounding, queue)
   if (small) { TBE_APPROX_SHORT(true); }
@@ -978,9 +1019,10 @@ void launch_approx_sum_long(const UpdateArgs &a, const RowGeometry &g, const voi
     // (the partial rows already carry the multipliers: the row takes their sum as it is)
     TBE_LAUNCH("update_long_finish", stream, (update_long_finish_kernel<T, VEC, CHUNKS, kOptSgd>), grid_finish,
                block, w, st, a.counters, long_records, partial, a.D, g.chunks, 1.0f, a.eps, a.unique_slots,
-               static_cast<T *>(a.cache_rows), a.stochastic_rounding);
+               static_cast<T *>(a.cache_rows), a.stochastic_rounding, a.max_long);
     TBE_LAUNCH("update_approx_state", stream, (approx_long_state_kernel<A>), grid_finish, block, st,
-               static_cast<const A *>(lookup_wss), a.positions_sorted, a.segment_starts, a.counters, long_records);
+               static_cast<const A *>(lookup_wss), a.positions_sorted, a.segment_starts, a.counters, long_records,
+               a.max_long);
   }
 }
 

@@ -35,7 +35,7 @@ def workspace_views(n, D, dtype, T):
     U = int(view(lay.num_unique, 1)[0])
     return dict(keys_sorted=view(lay.keys_sorted, n),
                 positions_sorted=view(lay.positions_sorted, n), segment_starts=view(lay.segment_starts, U + 1),
-                num_unique=U, counters=view(lay.num_unique, 16))
+                num_unique=U, counters=view(lay.num_unique, 320))
 
 
 def gpu_backward(p, optimizer, lr, eps=0.0, state=None):

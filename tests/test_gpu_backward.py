@@ -312,9 +312,10 @@ def test_queues_hold_the_most_chunk_records_a_batch_can_produce(oracle, dtype, D
     w, st, ref, got = _run_both(oracle, p, "sgd", 0.01, 0.1)
     lengths = np.diff(ref["segment_starts"])
     assert (lengths == occurrences).sum() >= T * (rows - 1)
+    # (one 128-byte line of counters per XCD from word 64 on: [0] chunk records queued, [1] segments of several chunks)
     counters = got["views"]["counters"]
-    assert counters[8:16].sum() == np.ceil(lengths[lengths > SHORT_SEGMENT] / 256).sum()
-    assert counters[1] == (lengths > 256).sum()
+    assert counters[64:320:32].sum() == np.ceil(lengths[lengths > SHORT_SEGMENT] / 256).sum()
+    assert counters[65:320:32].sum() == (lengths > 256).sum()
     _check(p, w, st, ref, got, "sgd")
 
 
@@ -335,10 +336,10 @@ def test_hot_rows_take_the_chunked_path(oracle, dtype, D, mode):
     lengths = np.diff(ref["segment_starts"])
     assert lengths.max() > 15000 and (lengths <= 256).any() and ((lengths > 256) & (lengths < 2000)).any()
     # rows with more than 256 occurrences are reduced in several chunks, rows with more than 128 by
-    # whole wavefronts: counters = [U, rows in several chunks, -, partial rows, ..., chunks queued by
-    # each of the eight XCDs]
-    assert got["views"]["counters"][1] == (lengths > 256).sum()
-    assert got["views"]["counters"][8:16].sum() == np.ceil(lengths[lengths > SHORT_SEGMENT] / 256).sum()
+    # whole wavefronts: from word 64 on, every XCD has a 128-byte line of counters, [0] the chunk records
+    # its workgroups queued, [1] their rows of several chunks
+    assert got["views"]["counters"][65:320:32].sum() == (lengths > 256).sum()
+    assert got["views"]["counters"][64:320:32].sum() == np.ceil(lengths[lengths > SHORT_SEGMENT] / 256).sum()
     np.testing.assert_array_equal(got["views"]["positions_sorted"], ref["positions_sorted"])
     np.testing.assert_array_equal(got["views"]["segment_starts"], ref["segment_starts"])
     # The truth is the update computed in fp64 from the same inputs.  The HIP path has to be within
