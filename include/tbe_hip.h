@@ -340,7 +340,8 @@ TBE_API int tbe_stochastic_round(const float *values, const uint32_t *random_wor
  * tbe_backward_approx_adagrad), and adds exact SGD; per-sample weights as in tbe_backward_exact_adagrad;
  * stochastic_rounding / seed / offset as in tbe_backward_exact_adagrad_stochastic;
  * max_table_rows as in tbe_backward_sgd (0 = unknown).  The
- * workspace is a backward workspace sized with tbe_backward_workspace_layout(N, 4, dtype, T).
+ * workspace is a backward workspace laid out by tbe_backward_mixed_workspace_layout (its partial
+ * rows hold the widest row that is summed in chunks: 64 vectors).
  * grad_output may hold at most 2^31 - 1 elements (B * total_D), so that the element offset of a
  * gradient row fits 32 bits.
  */
@@ -350,6 +351,9 @@ TBE_API int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp16_v
                               const int32_t *indices, int64_t num_indices,
                               const int32_t *offsets, int32_t B,
                               const void *per_sample_weights, void *output, void *stream);
+
+TBE_API int tbe_backward_mixed_workspace_layout(int64_t num_indices, int32_t dtype, int32_t T,
+                                                tbe_workspace_layout_t *layout);
 
 TBE_API int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void *weights, int32_t dtype,
                                int32_t fp16_vector_width, int64_t total_rows, int64_t max_table_rows,

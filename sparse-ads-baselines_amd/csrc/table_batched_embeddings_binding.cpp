@@ -425,7 +425,7 @@ c10::optional<at::Tensor> backward_mixed(int32_t optimizer, at::Tensor grad_outp
   c10::optional<at::Tensor> grad_indice_weights;
   if (indice_weights.has_value()) grad_indice_weights = at::empty_like(*indice_weights);
   tbe_workspace_layout_t layout;
-  check(tbe_backward_workspace_layout(s.n, 4, dtype, s.T, &layout));
+  check(tbe_backward_mixed_workspace_layout(s.n, dtype, s.T, &layout));
   Scratch ws = workspace(weights, layout.total_bytes);
   const bool rounds = stochastic_rounding && weights.scalar_type() == at::kHalf;
   std::pair<uint64_t, uint64_t> stream{0, 0};

@@ -69,13 +69,6 @@ template <typename A> __device__ __forceinline__ A group_sum_pow2(A v, int group
   return v;
 }
 
-struct MixedTables {
-  const int64_t *table_offsets;      // [T+1] first element of each table
-  const int32_t *table_dim_offsets;  // [T+1] first row id of each table
-  const int32_t *dim_offsets;        // [T+1] first output column of each table
-  int32_t total_D;
-  int32_t T;
-};
 
 constexpr int kBatch = 8;  // occurrences whose gradient rows are requested together
 constexpr int kApproxLong = 64;  // a register-held row with more occurrences gets a wavefront of its own

@@ -11,13 +11,17 @@
 // (table_batched_embeddings_cuda.cu:882-943), linear_index_weight_offsets_mixed_D_kernel
 // (:1220-1247) and batched_embedding_backward_adagrad_exact_kernel_mixed_D_1 (:1249-1348).
 //
-// One wavefront owns a bag (forward) or a unique row (backward) and its lanes stride over the
-// row's 16-byte vectors, so any D_t works; these kernels are the general path and are not
-// tuned per width like the uniform-D ones.  The integer stages (sort, segments) are shared.
+// Forward: one wavefront owns a bag and its lanes stride over the row's 16-byte vectors, so any
+// D_t works.  Backward: rows of a few occurrences are updated by lane groups in strips of 64
+// unique rows (update_mixed_kernel); rows of more occurrences are summed in chunks by whole
+// wavefronts, with the chunk records, per-XCD queues and partial rows of the uniform tables'
+// update (update_chunks_mixed_kernel, update_long_finish_mixed_kernel); rows wider than 64
+// vectors are walked by one wavefront each.  The integer stages (sort, segments) are shared.
 
 #include <algorithm>
 #include <type_traits>
 
+#include "tbe_queues.h"
 #include "tbe_rowwise.h"
 #include "tbe_stages.h"
 
@@ -399,12 +403,11 @@ __device__ __forceinline__ void mixed_update_wide(
 // bounds, key, positions, bag and table of each occurrence (from the gradient row ids b*T+t),
 // the table's width and offsets, optimizer state -- is fetched for the 64 rows at once, so the
 // dependent loads are paid per strip.  Rows of more than kMixedShort occurrences (the hot rows,
-// which are neighbours in key order) and rows wider than 64 vectors are not reduced here: their
-// indices go to two queues that update_mixed_queued_kernel drains -- one wavefront per row of at
-// most kChunkLen occurrences, one workgroup of 16 wavefronts per longer row -- so that they
-// spread over the machine.  The other rows leave a 32-byte record in LDS (in row order), and
-// every occurrence of theirs leaves the element offset of its gradient row (and its position,
-// for per-sample weights).
+// which are neighbours in key order) and rows wider than 64 vectors are not reduced here: the
+// former leave chunk records for update_chunks_mixed_kernel -- one wavefront per chunk of at most
+// kChunkLen occurrences -- so that they spread over the machine, the latter their row numbers.
+// The other rows leave a 32-byte record in LDS (in row order), and every occurrence of theirs
+// leaves the element offset of its gradient row (and its position, for per-sample weights).
 //
 // Then, one row per lane *group*, 64 / group_lanes rows at a time, so the instruction stream is
 // shared by several rows.  The group size fits the widest row of the strip (a strip spans a table
@@ -424,7 +427,6 @@ template <typename X> __device__ __forceinline__ void register_fence(X &x) {
   __builtin_memcpy(&x, words, sizeof(X));
 }
 
-constexpr int kMixedShort = 8;
 // Workgroups per compute unit the strip kernel is compiled for: as many as its registers allow
 // without spilling (per-sample weights, 8-element vectors, fp64 and the per-lookup form each need more).
 constexpr int mixed_strip_blocks(bool weighted, bool wide_vectors, bool approx, bool fp64) {
@@ -436,8 +438,7 @@ constexpr int kMixedAhead = 4;
 // its bag's ||grad||^2 (times its squared weight) to the row's state and moves the row by its own
 // multiplier, one occurrence after the other in position order, the row rounded to the weights'
 // type every time (the arithmetic of approx_adagrad_kernel).  Rows of more than kMixedShort
-// occurrences then go to ONE queue (`huge_rows`, counters[1]) whatever their length, and rows wider
-// than 64 vectors to the other (`long_rows`, counters[2]).
+// occurrences then go to a queue of row numbers (`queued_rows`, counters[1]) whatever their length.
 template <typename T, int VEC, int OPT, bool WEIGHTED, bool APPROX = false>
 __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 8, APPROX, sizeof(T) == 8)) void update_mixed_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
@@ -447,8 +448,10 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
     int num_tables, uint32_t bag_magic, int bag_shift, int total_D,
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ positions_sorted,
     const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ segment_starts,
-    int32_t *__restrict__ counters, int32_t *__restrict__ long_rows,
-    int32_t *__restrict__ huge_rows, float lr, float eps, StochasticRounding sr) {
+    int32_t *__restrict__ counters, int32_t *__restrict__ wide_rows,
+    int32_t *__restrict__ queued_rows, ChunkRecord *__restrict__ chunk_records,
+    LongRecord *__restrict__ long_records, int64_t max_chunks, int64_t max_long, int positions_per_xcd,
+    float lr, float eps, StochasticRounding sr) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -494,27 +497,82 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
     A l_state = A(0);
     if constexpr (OPT == kOptAdagrad) l_state = state[l_key];
 
-    // hand the longer rows of the strip to their queues (one atomic per strip and queue);
-    // rows wider than 64 vectors count as longer rows whatever their length
+    // Rows that are not reduced here.  Rows wider than 64 vectors go to a queue of row numbers
+    // whatever their length (`wide_rows`, counters[2]; one atomic per strip).
     const bool is_wide = l_D / VEC > kWave;
-    const bool is_huge = lane < rows_here && (APPROX ? (l_end - l_begin > kMixedShort && !is_wide)
-                                                     : l_end - l_begin > kChunkLen);
     const bool is_long = lane < rows_here && (l_end - l_begin > kMixedShort || is_wide);
     const unsigned long long long_mask = __ballot(is_long);
-    const unsigned long long huge_mask = __ballot(is_huge);
-    const unsigned long long medium_mask = long_mask & ~huge_mask;
-    if (medium_mask) {
+    const unsigned long long wide_mask = __ballot(is_long && is_wide);
+    if (wide_mask) {
       int first_slot = 0;
-      if (lane == 0) first_slot = atomicAdd(&counters[2], __popcll(medium_mask));
+      if (lane == 0) first_slot = atomicAdd(&counters[2], __popcll(wide_mask));
       first_slot = shfl_idx(first_slot, 0);
-      if (is_long && !is_huge)
-        long_rows[first_slot + __popcll(medium_mask & ((1ull << lane) - 1ull))] = static_cast<int32_t>(my_u);
+      if (is_long && is_wide)
+        wide_rows[first_slot + __popcll(wide_mask & ((1ull << lane) - 1ull))] = static_cast<int32_t>(my_u);
     }
-    if (huge_mask) {
-      int first_slot = 0;
-      if (lane == 0) first_slot = atomicAdd(&counters[1], __popcll(huge_mask));
-      first_slot = shfl_idx(first_slot, 0);
-      if (is_huge) huge_rows[first_slot + __popcll(huge_mask & ((1ull << lane) - 1ull))] = static_cast<int32_t>(my_u);
+    const unsigned long long queued_mask = long_mask & ~wide_mask;
+    if constexpr (APPROX) {
+      // the per-lookup form walks a row of many occurrences in one piece: its number goes to
+      // `queued_rows` (counters[1])
+      if (queued_mask) {
+        int first_slot = 0;
+        if (lane == 0) first_slot = atomicAdd(&counters[1], __popcll(queued_mask));
+        first_slot = shfl_idx(first_slot, 0);
+        if (is_long && !is_wide)
+          queued_rows[first_slot + __popcll(queued_mask & ((1ull << lane) - 1ull))] = static_cast<int32_t>(my_u);
+      }
+    } else if (queued_mask) {
+      // The exact update sums such a row in chunks of at most kChunkLen occurrences, like the uniform
+      // tables' update: chunk records (and, for a row of several chunks, a list entry) in the queue
+      // of the XCD whose eighth of the sorted positions the strip's first such row starts in, so
+      // that update_chunks_mixed_kernel finds a table's hot rows -- and their gradient rows in L2 --
+      // on one XCD.  One atomic add per strip takes the queue slots and list entries of all its
+      // rows (atomic adds on one counter are served one after the other: one per row cost 40 us
+      // with 27 k such rows); a row's share follows from a prefix sum over the lanes.  The records
+      // of one row after the other are then written by the whole wavefront.
+      const bool chunked = is_long && !is_wide;
+      const int my_nch = chunked ? (l_end - l_begin + kChunkLen - 1) / kChunkLen : 0;
+      // (fewer than 2^23 chunks and at most 64 rows in all: both sums fit one word)
+      const int my_share = my_nch | (my_nch > 1 ? 1 << 24 : 0);
+      int before = my_share;
+#pragma unroll
+      for (int d = 1; d < kWave; d <<= 1) {
+        const int y = __shfl_up(before, d, kWave);
+        if (lane >= d) before += y;
+      }
+      const int strip_total = shfl_idx(before, kWave - 1);
+      before -= my_share;
+      const int first_lane = __ffsll(static_cast<long long>(queued_mask)) - 1;
+      const int queue_index = min(shfl_idx(l_begin, first_lane) / positions_per_xcd, kNumXcd - 1);
+      unsigned long long taken = 0ull;
+      if (lane == 0)
+        taken = atomicAdd(reinterpret_cast<unsigned long long *>(counters + xcd_counter(queue_index)),
+                          static_cast<unsigned long long>(strip_total & 0xffffff) |
+                              (static_cast<unsigned long long>(strip_total >> 24) << 32));
+      const int first_chunk_of_strip = shfl_idx(static_cast<int>(taken & 0xffffffffull), 0);
+      const int first_entry_of_strip = shfl_idx(static_cast<int>(taken >> 32), 0);
+      const int my_first_chunk = first_chunk_of_strip + (before & 0xffffff);
+      if (my_nch > 1)
+        long_records[queue_index * (max_long / kNumXcd) + first_entry_of_strip + (before >> 24)] =
+            LongRecord{l_table, l_key, l_begin, l_end};
+      ChunkRecord *queue = chunk_records + queue_index * (max_chunks / kNumXcd);
+      for (unsigned long long rest = queued_mask; rest != 0ull; rest &= rest - 1ull) {
+        const int src = __ffsll(static_cast<long long>(rest)) - 1;
+        const int seg_begin = shfl_idx(l_begin, src), seg_end = shfl_idx(l_end, src);
+        const int first_chunk = shfl_idx(my_first_chunk, src);
+        const int nch = (seg_end - seg_begin + kChunkLen - 1) / kChunkLen;
+        ChunkRecord rec;
+        rec.key = shfl_idx(l_key, src);
+        rec.u = static_cast<int32_t>(u0) + src;
+        rec.pad[0] = shfl_idx(l_table, src);
+        rec.pad[1] = rec.pad[2] = 0;
+        for (int k = lane; k < nch; k += kWave) {
+          rec.begin = seg_begin + k * kChunkLen;
+          rec.end = min(seg_end, rec.begin + kChunkLen);
+          rec.partial = nch > 1 ? partial_row_of_chunk(seg_begin, seg_end, k, nch) : -1;
+          queue[first_chunk + k] = rec;
+        }
+      }
     }
     const unsigned long long todo = ~long_mask & (rows_here == kWave ? ~0ull : ((1ull << rows_here) - 1ull));
     if (todo == 0ull) continue;
@@ -719,101 +777,174 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
   }
 }
 
-// Queued rows: WAVES wavefronts per row (1, or kHugeWaves for the rows of more than kChunkLen
-// occurrences).  The wavefronts of a row take its 64-position batches round-robin; their sums
-// meet in LDS and the row's first wavefront adds them in wavefront order and applies the
-// optimizer.  A row wider than 64 vectors is left to its first wavefront.  `queue_counter` is
-// the index of the queue's length in `counters`.  Both kinds of row are served by ONE launch of
-// workgroups of kHugeWaves wavefronts: the first `huge_blocks` workgroups take a long row each
-// time round, the others one row per wavefront -- the two queues drain side by side instead of
-// one after the other (each is bound by the dependent loads at the head of a row, not by
-// bandwidth: 99 + 101 us one after the other for 64 tables of 100 k rows of 64..192, Zipf 1.05).
-constexpr int kHugeWaves = 16;
-template <typename T, int VEC, int OPT, bool WEIGHTED, int UNROLL, int WAVES>
-__device__ __forceinline__ void mixed_queued_rows(
+// ------------------------------------------------ exact update: rows of many occurrences
+__device__ __forceinline__ int bag_of_grad_row(int grow, const MixedTables &mt) {
+  return static_cast<int>((static_cast<uint64_t>(static_cast<uint32_t>(grow)) * mt.bag_magic) >> mt.bag_shift);
+}
+
+// The chunk records of mixed-D tables: update_chunks_kernel's walk over the eight queues, each record
+// reduced with its own table's row width.  A chunk that is a whole segment is applied to its row
+// at once; a chunk of a longer segment stores its sum as a partial row of 64 vectors.
+template <typename T, int VEC, int OPT, bool WEIGHTED, int UNROLL>
+__global__ __launch_bounds__(kBlockThreads) void update_chunks_mixed_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
-    T *__restrict__ grad_psw, const int64_t *__restrict__ table_offsets,
-    const int32_t *__restrict__ table_dim_offsets, const int32_t *__restrict__ dim_offsets,
-    int num_tables, int total_D, const int32_t *__restrict__ keys_sorted,
+    T *__restrict__ grad_psw, const int32_t *__restrict__ keys_sorted,
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
-    const int32_t *__restrict__ segment_starts, int num_queued, const int32_t *__restrict__ queue, float lr,
-    float eps, StochasticRounding sr, int64_t first_row, int64_t row_stride,
-    typename AccOf<T>::type (*s_partial)[kWave * VEC]) {
+    const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
+    const ChunkRecord *__restrict__ chunk_records, int64_t max_chunks, const int32_t *__restrict__ wide_rows,
+    typename AccOf<T>::type *__restrict__ partial_sums, float lr, float eps, StochasticRounding sr,
+    MixedTables mt) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
-  const int wave_in_row = WAVES > 1 ? wave : 0;
-  for (int64_t q = first_row; q < num_queued; q += row_stride) {
-    const int u = queue[q];
+  const int xcd = blockIdx.x % kNumXcd;
+  const int64_t queue_capacity = max_chunks / kNumXcd;
+  // an XCD drains its own queue up to one and a half times the average queue length, the rest is
+  // dealt to the wavefronts of all XCDs (see update_chunks_kernel)
+  int queue_len[kNumXcd];
+  int64_t total = 0;
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) {
+    queue_len[x] = counters[xcd_counter(x)];
+    total += queue_len[x];
+  }
+  const int fair = static_cast<int>(total / kNumXcd + total / 16 + 1);
+  int64_t shared_total = 0;
+#pragma unroll
+  for (int x = 0; x < kNumXcd; ++x) shared_total += max(0, queue_len[x] - fair);
+  const int own = min(queue_len[xcd], fair);
+  int64_t q = static_cast<int64_t>(blockIdx.x / kNumXcd) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = static_cast<int64_t>(gridDim.x / kNumXcd) * kWavesPerBlock;
+  int64_t g = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t shared_stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  while (true) {
+    const ChunkRecord *next;
+    if (q < own) {
+      next = chunk_records + xcd * queue_capacity + q;
+      q += stride;
+    } else if (g < shared_total) {
+      int64_t before = 0;
+      int x = 0;
+      while (g >= before + max(0, queue_len[x] - fair)) {
+        before += max(0, queue_len[x] - fair);
+        ++x;
+      }
+      next = chunk_records + x * queue_capacity + fair + (g - before);
+      g += shared_stride;
+    } else {
+      break;
+    }
+    const ChunkRecord rec = *next;
+    const int t = rec.pad[0];
+    MixedRow row;
+    row.seg_begin = rec.begin;
+    row.seg_end = rec.end;
+    row.key = rec.key;
+    row.dim_start = mt.dim_offsets[t];
+    row.D = mt.dim_offsets[t + 1] - row.dim_start;
+    row.row_element = mt.table_offsets[t] + static_cast<int64_t>(rec.key - mt.table_dim_offsets[t]) * row.D;
+    A state_old = A(0);
+    if constexpr (OPT == kOptAdagrad) {
+      if (rec.partial < 0) state_old = state[rec.key];
+    }
+    V w_old, G;
+    mixed_accumulate_narrow<T, VEC, WEIGHTED, UNROLL>(grad_output, weights, psw, grad_psw, mt.T, mt.total_D,
+                                                      positions_sorted, grad_rows, lane, row, 0, 1, w_old, G);
+    if (rec.partial >= 0) {
+      if (lane < row.D / VEC) {
+        A *dst = partial_sums + static_cast<int64_t>(rec.partial) * (kWave * VEC) + static_cast<int64_t>(lane) * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) dst[i] = G.v[i];
+      }
+    } else {
+      mixed_apply_narrow<T, VEC, OPT>(weights, state, lr, eps, sr, lane, row, state_old, w_old, G);
+    }
+  }
+  // the rows wider than 64 vectors, a wavefront each (their number: counters[2])
+  const int num_wide = counters[2];
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6); i < num_wide; i += shared_stride) {
+    const int u = wide_rows[i];
     MixedRow row;
     row.seg_begin = segment_starts[u];
     row.seg_end = segment_starts[u + 1];
     row.key = keys_sorted[row.seg_begin];
-    const int table = grad_rows[positions_sorted[row.seg_begin]] % num_tables;
-    row.dim_start = dim_offsets[table];
-    row.D = dim_offsets[table + 1] - row.dim_start;
-    row.row_element = table_offsets[table] + static_cast<int64_t>(row.key - table_dim_offsets[table]) * row.D;
+    const int grow = grad_rows[positions_sorted[row.seg_begin]];
+    const int t = grow - bag_of_grad_row(grow, mt) * mt.T;
+    row.dim_start = mt.dim_offsets[t];
+    row.D = mt.dim_offsets[t + 1] - row.dim_start;
+    row.row_element = mt.table_offsets[t] + static_cast<int64_t>(row.key - mt.table_dim_offsets[t]) * row.D;
     A state_old = A(0);
     if constexpr (OPT == kOptAdagrad) state_old = state[row.key];
-    const int chunks = row.D / VEC;
-    if (chunks > kWave) {
-      if (wave_in_row == 0)
-        mixed_update_wide<T, VEC, OPT, WEIGHTED>(grad_output, weights, state, psw, grad_psw, num_tables, total_D,
-                                                 positions_sorted, grad_rows, lr, eps, sr, lane, row, state_old);
-      continue;
-    }
-    V w_old, G;
-    mixed_accumulate_narrow<T, VEC, WEIGHTED, UNROLL>(grad_output, weights, psw, grad_psw, num_tables, total_D,
-                                                      positions_sorted, grad_rows, lane, row, wave_in_row, WAVES,
-                                                      w_old, G);
-    if constexpr (WAVES > 1) {
-      __syncthreads();  // the previous row's partial sums have been read
-      if (lane < chunks) {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) s_partial[wave][lane * VEC + i] = G.v[i];
-      }
-      __syncthreads();
-      if (wave == 0 && lane < chunks) {
-        for (int w = 1; w < WAVES; ++w) {
-#pragma unroll
-          for (int i = 0; i < VEC; ++i) G.v[i] += s_partial[w][lane * VEC + i];
-        }
-      }
-    }
-    if (wave_in_row == 0)
-      mixed_apply_narrow<T, VEC, OPT>(weights, state, lr, eps, sr, lane, row, state_old, w_old, G);
+    mixed_update_wide<T, VEC, OPT, WEIGHTED>(grad_output, weights, state, psw, grad_psw, mt.T, mt.total_D,
+                                             positions_sorted, grad_rows, lr, eps, sr, lane, row, state_old);
   }
 }
 
-template <typename T, int VEC, int OPT, bool WEIGHTED, int UNROLL>
-__global__ __launch_bounds__(kHugeWaves * kWave) void update_mixed_queued_kernel(
-    const T *__restrict__ grad_output, T *__restrict__ weights,
-    typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
-    T *__restrict__ grad_psw, const int64_t *__restrict__ table_offsets,
-    const int32_t *__restrict__ table_dim_offsets, const int32_t *__restrict__ dim_offsets,
-    int num_tables, int total_D, const int32_t *__restrict__ keys_sorted,
-    const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows,
-    const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
-    const int32_t *__restrict__ long_queue, const int32_t *__restrict__ huge_queue, int huge_blocks, float lr,
-    float eps, StochasticRounding sr) {
-  using A = typename AccOf<T>::type;
-  __shared__ A s_partial[kHugeWaves][kWave * VEC];
-  if (static_cast<int>(blockIdx.x) < huge_blocks) {
-    // rows of more than kChunkLen occurrences (their number is counters[1]): the workgroup per row
-    mixed_queued_rows<T, VEC, OPT, WEIGHTED, UNROLL, kHugeWaves>(
-        grad_output, weights, state, psw, grad_psw, table_offsets, table_dim_offsets, dim_offsets, num_tables, total_D,
-        keys_sorted, positions_sorted, grad_rows, segment_starts, counters[1], huge_queue, lr, eps, sr, blockIdx.x,
-        huge_blocks, s_partial);
-  } else {
-    // the other queued rows (counters[2]): a wavefront per row
-    const int64_t long_blocks = static_cast<int64_t>(gridDim.x) - huge_blocks;
-    mixed_queued_rows<T, VEC, OPT, WEIGHTED, UNROLL, 1>(
-        grad_output, weights, state, psw, grad_psw, table_offsets, table_dim_offsets, dim_offsets, num_tables, total_D,
-        keys_sorted, positions_sorted, grad_rows, segment_starts, counters[2], long_queue, lr, eps, sr,
-        (static_cast<int64_t>(blockIdx.x) - huge_blocks) * kHugeWaves + (threadIdx.x >> 6), long_blocks * kHugeWaves,
-        s_partial);
+// The rows of several chunks of mixed-D tables: one wavefront per row adds its partial rows in
+// chunk order (lane group r takes partial rows r, r + groups, ..., the groups are combined in a
+// fixed tree) and applies the optimizer.  The list records carry the row's table in `u`.
+template <typename T, int VEC, int OPT>
+__global__ __launch_bounds__(kBlockThreads) void update_long_finish_mixed_kernel(
+    T *__restrict__ weights, typename AccOf<T>::type *__restrict__ state,
+    const int32_t *__restrict__ counters, const LongRecord *__restrict__ long_records,
+    const typename AccOf<T>::type *__restrict__ partial_sums, float lr, float eps, StochasticRounding sr,
+    int64_t max_long, MixedTables mt) {
+  using V = RowVec<T, VEC>;
+  using A = typename V::A;
+  const int lane = threadIdx.x & (kWave - 1);
+  const LongLists lists = long_lists(counters, max_long);
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  for (int64_t slot = wave_id; slot < lists.total; slot += stride) {
+    const LongRecord rec = long_record_at(long_records, lists, slot);
+    const int t = rec.u;
+    MixedRow row;
+    row.seg_begin = rec.begin;
+    row.seg_end = rec.end;
+    row.key = rec.key;
+    row.dim_start = mt.dim_offsets[t];
+    row.D = mt.dim_offsets[t + 1] - row.dim_start;
+    row.row_element = mt.table_offsets[t] + static_cast<int64_t>(rec.key - mt.table_dim_offsets[t]) * row.D;
+    const int chunks = row.D / VEC;
+    const int group_shift = chunks > 1 ? 32 - __builtin_clz(chunks - 1) : 0;
+    const int group_lanes = 1 << group_shift;
+    const int groups = kWave >> group_shift;
+    const int r = lane >> group_shift;
+    const int c = lane & (group_lanes - 1);
+    const bool active = c < chunks;
+    const int64_t col = active ? static_cast<int64_t>(c) * VEC : 0;
+    const int num_chunks = (rec.end - rec.begin + kChunkLen - 1) / kChunkLen;
+    V w_old;
+    w_old.zero();
+    if (lane < chunks) w_old.load(weights + row.row_element + col);
+    A state_old = A(0);
+    if constexpr (OPT == kOptAdagrad) state_old = state[rec.key];
+    V G;
+    G.zero();
+    constexpr int kAhead = 8;
+    for (int k0 = r; k0 < num_chunks; k0 += groups * kAhead) {
+      A part[kAhead][VEC];
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) {
+        const int k = min(k0 + a * groups, num_chunks - 1);  // clamped: no branch per load
+        const A *src = partial_sums +
+                       static_cast<int64_t>(partial_row_of_chunk(rec.begin, rec.end, k, num_chunks)) * (kWave * VEC) + col;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) part[a][i] = src[i];
+      }
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) {
+        const bool real = active && k0 + a * groups < num_chunks;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) G.v[i] += real ? part[a][i] : A(0);
+      }
+    }
+    for (int m = kWave >> 1; m >= group_lanes; m >>= 1) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) G.v[i] += shfl_x(G.v[i], m);
+    }
+    mixed_apply_narrow<T, VEC, OPT>(weights, state, lr, eps, sr, lane, row, state_old, w_old, G);
   }
 }
 
@@ -856,6 +987,8 @@ void launch_forward_mixed(const MixedArgs &a, hipStream_t stream) {
                a.table_offsets, a.dim_offsets, a.indices, a.offsets, p, o, a.B, a.total_D, num_bags, per_xcd);
 }
 
+// The exact update: the strip kernel for the rows of few occurrences, then one wavefront per chunk
+// record (and per row wider than 64 vectors), then the rows of several chunks.
 template <typename T, int VEC, int OPT, bool WEIGHTED>
 void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, char *ws, hipStream_t stream) {
   using A = typename AccOf<T>::type;
@@ -865,32 +998,39 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
   A *st = static_cast<A *>(a.state);
   const T *psw = static_cast<const T *>(a.psw);
   T *gpsw = static_cast<T *>(a.grad_psw);
-  // queues of row indices: rows of 9..256 occurrences or wider than 64 vectors (at most one per
-  // lookup) and rows of more occurrences (n / 257)
-  int32_t *long_rows = i32(l.segment_ids);
-  int32_t *huge_rows = i32(l.long_segments);
+  A *partial = reinterpret_cast<A *>(ws + l.partial_sums);
+  LongRecord *long_records = reinterpret_cast<LongRecord *>(ws + l.long_segments);
+  ChunkRecord *chunk_records = reinterpret_cast<ChunkRecord *>(ws + l.chunk_segments);
+  const int64_t max_chunks = static_cast<int64_t>(l.max_chunks);
+  const int64_t max_long = static_cast<int64_t>(l.max_long_segments);
+  // numbers of the rows wider than 64 vectors (at most one per lookup; the exact update of
+  // these tables does not use the segment of every position)
+  int32_t *wide_rows = i32(l.segment_ids);
+  MixedTables mt{a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.total_D, a.T};
+  set_bag_division(mt);
+  const dim3 block(kBlockThreads);
   const int64_t want = ceil_div(ceil_div(a.n, kWave), kWavesPerBlock);
   const dim3 grid(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want, 256 * 32))));
-  // b = grow / T for grow < 2^31 as a multiplication and a shift: magic = ceil(2^(31 + s) / T) with
-  // s = ceil(log2 T) fits 32 bits and gives the exact quotient
-  int log2_T = 0;
-  while ((int64_t{1} << log2_T) < a.T) ++log2_T;
-  const int bag_shift = 31 + log2_T;
-  const uint32_t bag_magic =
-      static_cast<uint32_t>(((uint64_t{1} << bag_shift) + static_cast<uint64_t>(a.T) - 1) / static_cast<uint64_t>(a.T));
-  TBE_LAUNCH("update_mixed", stream, (update_mixed_kernel<T, VEC, OPT, WEIGHTED>), grid, dim3(kBlockThreads),
-             go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, bag_magic, bag_shift,
+  TBE_LAUNCH("update_mixed", stream, (update_mixed_kernel<T, VEC, OPT, WEIGHTED>), grid, block,
+             go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, mt.bag_magic, mt.bag_shift,
              a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
-             i32(l.num_unique), long_rows, huge_rows, a.lr, a.eps, a.sr);
-  const int64_t want_long = ceil_div(a.n, kHugeWaves);
-  const int64_t long_blocks = std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 2));
-  const int64_t want_huge = a.n / (kChunkLen + 1) + 1;
-  const int64_t huge_blocks = std::max<int64_t>(1, std::min<int64_t>(want_huge, 256 * 2));
-  TBE_LAUNCH("update_mixed_queued", stream, (update_mixed_queued_kernel<T, VEC, OPT, WEIGHTED, 8>),
-             dim3(static_cast<unsigned>(huge_blocks + long_blocks)), dim3(kHugeWaves * kWave), go, w, st, psw, gpsw,
-             a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, a.total_D, i32(l.keys_sorted),
-             i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts), i32(l.num_unique), long_rows, huge_rows,
-             static_cast<int>(huge_blocks), a.lr, a.eps, a.sr);
+             i32(l.num_unique), wide_rows, static_cast<int32_t *>(nullptr), chunk_records, long_records, max_chunks,
+             max_long, static_cast<int>(ceil_div(a.n, kNumXcd)), a.lr, a.eps, a.sr);
+
+  const bool small = ceil_div(a.n, tile_positions(0)) < kSmallBatchTiles;
+  const int64_t want_chunks = ceil_div(max_chunks, kWavesPerBlock);
+  // a multiple of the XCD count, so that every XCD gets as many workgroups (few for a small batch)
+  const dim3 grid_chunks(static_cast<unsigned>(
+      kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), small ? 64 : 1024))));
+  TBE_LAUNCH("update_chunks_mixed", stream,
+             (update_chunks_mixed_kernel<T, VEC, OPT, WEIGHTED, (WEIGHTED && VEC == 8) ? 4 : 8>), grid_chunks, block,
+             go, w, st, psw, gpsw, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
+             i32(l.num_unique), chunk_records, max_chunks, wide_rows, partial, a.lr, a.eps, a.sr, mt);
+
+  const int64_t want_long = ceil_div(max_long, kWavesPerBlock);
+  const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
+  TBE_LAUNCH("update_long_finish_mixed", stream, (update_long_finish_mixed_kernel<T, VEC, OPT>), grid_finish, block,
+             w, st, i32(l.num_unique), long_records, partial, a.lr, a.eps, a.sr, max_long, mt);
 }
 
 // The approximate update's strip kernel: rows of at most 64 vectors and kMixedShort occurrences
@@ -911,7 +1051,9 @@ void launch_update_mixed_approx(const MixedArgs &a, const tbe_workspace_layout_t
              static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),
              a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, bag_magic, bag_shift, a.total_D,
              i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
-             i32(l.num_unique), approx_mixed_wide_queue(l, ws), approx_mixed_long_queue(l, ws), a.lr, a.eps, a.sr);
+             i32(l.num_unique), approx_mixed_wide_queue(l, ws), approx_mixed_long_queue(l, ws),
+             static_cast<ChunkRecord *>(nullptr), static_cast<LongRecord *>(nullptr), int64_t{0}, int64_t{0}, 1, a.lr,
+             a.eps, a.sr);
 }
 
 template <typename T, int VEC>
@@ -932,6 +1074,12 @@ void launch_update_mixed_variant(const MixedArgs &a, const tbe_workspace_layout_
     if (weighted) launch_update_mixed<T, VEC, kOptAdagrad, true>(a, l, ws, stream);
     else launch_update_mixed<T, VEC, kOptAdagrad, false>(a, l, ws, stream);
   }
+}
+
+// Row width the workspace of mixed-D tables is laid out for: its partial rows hold 64 vectors, the
+// widest row that is summed in chunks (8 elements a vector at most for fp16).
+int32_t mixed_layout_dim(int32_t dtype) {
+  return kWave * (dtype == TBE_DTYPE_F16 ? 8 : dtype == TBE_DTYPE_F32 ? 4 : 2);
 }
 
 int validate_mixed(const char *name, const MixedArgs &a) {
@@ -985,6 +1133,18 @@ extern "C" int tbe_forward_mixed(const void *weights, int32_t dtype, int32_t fp1
   return check_launch("tbe_forward_mixed");
 }
 
+extern "C" int tbe_backward_mixed_workspace_layout(int64_t num_indices, int32_t dtype, int32_t T,
+                                                   tbe_workspace_layout_t *layout) {
+  using namespace tbe;
+  const char *name = "tbe_backward_mixed_workspace_layout";
+  TBE_REQUIRE(layout, "%s: null layout", name);
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
+  TBE_REQUIRE(T > 0, "%s: T must be positive (got %d)", name, T);
+  backward_layout(num_indices, mixed_layout_dim(dtype), dtype, T, layout);
+  return TBE_OK;
+}
+
 extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, void *weights,
                                   int32_t dtype, int32_t fp16_vector_width, int64_t total_rows,
                                   int64_t max_table_rows, const int64_t *table_offsets, const int32_t *table_dim_offsets,
@@ -1032,7 +1192,7 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
               "%s: per_sample_weights and grad_per_sample_weights must both be given or both be null", name);
   if (num_indices == 0) return TBE_OK;
   tbe_workspace_layout_t l;
-  backward_layout(num_indices, 4, dtype, T, &l);  // no partial rows are used: size them for D = 4
+  backward_layout(num_indices, mixed_layout_dim(dtype), dtype, T, &l);
   if (!workspace || workspace_bytes < l.total_bytes)
     return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
                 (unsigned long long)l.total_bytes, (unsigned long long)workspace_bytes);

@@ -55,6 +55,8 @@ int find_segments(const int32_t *keys_sorted, int64_t n, int32_t *segment_starts
 // kApproxShortSegment occurrences on.
 constexpr int kShortSegment = 128;
 constexpr int kApproxShortSegment = 16;
+// (tables of different row widths: rows of more than kMixedShort occurrences are summed in chunks)
+constexpr int kMixedShort = 8;
 constexpr int kChunkLen = 256;
 // Integers kept next to the number of unique rows (all zeroed when the segments are found): [1], [2]
 // queue lengths of the kernels that keep one queue (mixed-D tables, the approximate update), and from
@@ -75,14 +77,15 @@ constexpr int kApproxHuge = 256;   // occurrences from which on the approximate 
 // those of its eighth plus those of one segment of any length.
 inline int64_t chunk_queue_capacity(int64_t n) {
   const int64_t eighth = (n + 7) / 8 + 2048;
-  // (sized for the smaller of the two thresholds: the approximate update of fp32 rows queues its
-  // chunk records here too)
-  return eighth / (kApproxShortSegment + 1) + eighth / kChunkLen + n / kChunkLen + 8;
+  // (sized for the smallest of the thresholds: the approximate update of fp32 rows and the update of
+  // tables of different row widths queue their chunk records here too)
+  return eighth / (kMixedShort + 1) + eighth / kChunkLen + n / kChunkLen + 8;
 }
 
 // Room of one XCD's list of segments of several chunks (more than kChunkLen occurrences each) that
-// start in its eighth of the sorted positions.
-inline int64_t long_list_capacity(int64_t n) { return ((n + 7) / 8 + 2048) / (kChunkLen + 1) + 2; }
+// start in its eighth of the sorted positions (and, for tables of different row widths, the up to
+// 63 rows that share a strip of 64 unique rows with the last row of the eighth).
+inline int64_t long_list_capacity(int64_t n) { return ((n + 7) / 8 + 2048) / (kChunkLen + 1) + 2 + 64; }
 // The partial row of chunk k of a segment [begin, end) of several chunks.  Every chunk but a segment's
 // last is kChunkLen positions long, so no two of them begin in the same window of kChunkLen positions;
 // and segments of several chunks end more than kChunkLen positions apart, so no two last chunks end in
@@ -155,6 +158,26 @@ int build_plan(const tbe_workspace_layout_t &layout, void *workspace, const int3
                int64_t total_rows, int64_t max_table_rows, hipStream_t stream,
                int32_t interleaved_offsets_stride = 0);
 
+// Tables of different row widths in one flat weight array (the reference's MixedDim layout,
+// table_batched_embeddings_ops.py:204-435).
+struct MixedTables {
+  const int64_t *table_offsets;      // [T+1] first element of each table
+  const int32_t *table_dim_offsets;  // [T+1] first row id of each table
+  const int32_t *dim_offsets;        // [T+1] first output column of each table
+  int32_t total_D;
+  int32_t T;
+  // b = grow / T for a gradient row number grow = b*T + t < 2^31 as a multiplication and a shift:
+  // magic = ceil(2^(31 + s) / T) with s = ceil(log2 T) fits 32 bits and gives the exact quotient
+  uint32_t bag_magic = 0;
+  int32_t bag_shift = 0;
+};
+inline void set_bag_division(MixedTables &mt) {
+  int log2_T = 0;
+  while ((int64_t{1} << log2_T) < mt.T) ++log2_T;
+  mt.bag_shift = 31 + log2_T;
+  mt.bag_magic = static_cast<uint32_t>(((uint64_t{1} << mt.bag_shift) + static_cast<uint64_t>(mt.T) - 1) /
+                                       static_cast<uint64_t>(mt.T));
+}
 // The approximate row-wise Adagrad update (one lookup at a time per row, in position order) on a
 // workspace that holds the batch's plan.  Uniform tables: D > 0 and the mixed_* pointers null;
 // mixed-D tables: D = 0, and the strip kernel of tbe_backward_mixed has already applied the rows

@@ -23,6 +23,7 @@
 
 #include <algorithm>
 
+#include "tbe_queues.h"
 #include "tbe_rowwise.h"
 #include "tbe_stages.h"
 
@@ -80,31 +81,7 @@ __device__ __forceinline__ void apply_update(T *wrow, const RowVec<T, VEC> &w_ol
 // group r walks segments r, r + groups, ...  Segments longer than kShortSegment are not
 // reduced here: the owning group appends chunk records (at most kChunkLen occurrences each)
 // to a queue that update_chunks_kernel drains with one wavefront per chunk.
-// Tile size in sorted positions: 16 per lane group, so narrow rows (many groups per wavefront)
-// get larger tiles and the per-tile bookkeeping is amortised over the same number of rows.
-// (at most 256 positions; 64 for the variant whose row width is only known at run time.  Measured
-// with segments of up to 128 occurrences reduced here: 8 / 16 / 32 / 64 positions per lane group
-// take 616 / 605 / 616 / 632 us for 64 tables of fp32 rows of 128 and 206 / 188 / 203 / 203 us for
-// 32 tables of fp16 rows of 64 with per-sample weights, 5.2 M lookups each.)
-// Small batches (fewer than kSmallBatchTiles such tiles: not enough wavefronts to fill the chip)
-// take tiles a quarter that size.
-constexpr int kSmallBatchTiles = 4096;
-constexpr int tile_positions(int chunks_template, bool small = false) {
-  if (chunks_template == 0) return small ? 16 : 64;
-  const int positions = (small ? 8 : 16) * (kWave / chunks_template);
-  return positions > 256 ? 256 : positions;
-}
-
-struct ChunkRecord {   // 32 bytes
-  int32_t begin, end;  // sorted positions [begin, end)
-  int32_t key;         // row
-  int32_t u;           // index of the unique row (for the cache slot table)
-  int32_t partial;     // index of the partial row to write, -1 = the chunk is the whole segment
-  int32_t pad[3];
-};
-struct LongRecord {    // 16 bytes: a segment cut into several chunks
-  int32_t u, key, begin, end;  // unique-row number, row, sorted positions [begin, end)
-};
+// (tile sizes: tile_positions() of tbe_queues.h)
 
 // APPROX (row-wise Adagrad only): the approximate optimizer's per-lookup update
 // (batched_embedding_backward_adagrad_approx_kernel_1, tbe.cu:648-704) instead of one update with the
@@ -172,34 +149,31 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
   const int nseg = u_limit - u_first;  // <= kTilePositions
   if (nseg <= 0) return;
 
-  // Bookkeeping into LDS.  All loads of one level are issued before the first dependent load,
-  // so a tile pays two memory round trips here however many positions it holds.
-  {
-    constexpr int kBoundIters = (kTilePositions + 1 + kWave - 1) / kWave;
-    int sb[kBoundIters];
+  // Bookkeeping into LDS.  All loads of one level are issued before the first dependent load:
+  // the segment bounds, then -- both only need the bounds -- the keys and the tile's sorted
+  // positions, then the gradient row of every position.  Three memory round trips however many
+  // positions the tile holds.  (The first and the last bound reach all lanes by lane shuffles, not
+  // through LDS, so that the positions are requested together with the keys.)
+  constexpr int kBoundIters = (kTilePositions + 1 + kWave - 1) / kWave;
+  constexpr int kStageIters = (kStageCap + kWave - 1) / kWave;
+  int sb[kBoundIters];
 #pragma unroll
-    for (int q = 0; q < kBoundIters; ++q) {
-      const int k = q * kWave + lane;
-      sb[q] = segment_starts[u_first + min(k, nseg)];  // clamped, not predicated: no branch per load
-    }
+  for (int q = 0; q < kBoundIters; ++q) {
+    const int k = q * kWave + lane;
+    sb[q] = segment_starts[u_first + min(k, nseg)];  // clamped, not predicated: no branch per load
+  }
+  const int tile_begin = shfl_idx(sb[0], 0);
+  int tile_end = 0;  // bound number nseg: where the tile's last segment ends
+#pragma unroll
+  for (int q = 0; q < kBoundIters; ++q) {
+    const int v = shfl_idx(sb[q], nseg & (kWave - 1));
+    if (q == (nseg >> 6)) tile_end = v;
+  }
+  const int staged = min(tile_end - tile_begin, kStageCap);
+  {
     int kv[kBoundIters];
 #pragma unroll
-    for (int q = 0; q < kBoundIters; ++q) {
-      const int k = q * kWave + lane;
-      kv[q] = keys_sorted[min(static_cast<int64_t>(sb[q]), n - 1)];
-    }
-#pragma unroll
-    for (int q = 0; q < kBoundIters; ++q) {
-      const int k = q * kWave + lane;
-      if (k <= nseg) s_bounds[wave][k] = sb[q];
-      if (k < nseg) s_keys[wave][k] = kv[q];
-    }
-  }
-  __builtin_amdgcn_wave_barrier();
-  const int tile_begin = s_bounds[wave][0];
-  const int staged = min(s_bounds[wave][nseg] - tile_begin, kStageCap);
-  {
-    constexpr int kStageIters = (kStageCap + kWave - 1) / kWave;
+    for (int q = 0; q < kBoundIters; ++q) kv[q] = keys_sorted[min(static_cast<int64_t>(sb[q]), n - 1)];
     int pos[kStageIters], grow[kStageIters];
 #pragma unroll
     for (int q = 0; q < kStageIters; ++q) {
@@ -207,10 +181,13 @@ __global__ __launch_bounds__(kBlockThreads) void update_short_kernel(
       pos[q] = positions_sorted[tile_begin + min(i, staged - 1)];
     }
 #pragma unroll
-    for (int q = 0; q < kStageIters; ++q) {
-      const int i = q * kWave + lane;
-      grow[q] = grad_rows[pos[q]];
+    for (int q = 0; q < kBoundIters; ++q) {
+      const int k = q * kWave + lane;
+      if (k <= nseg) s_bounds[wave][k] = sb[q];
+      if (k < nseg) s_keys[wave][k] = kv[q];
     }
+#pragma unroll
+    for (int q = 0; q < kStageIters; ++q) grow[q] = grad_rows[pos[q]];
 #pragma unroll
     for (int q = 0; q < kStageIters; ++q) {
       const int i = q * kWave + lane;
@@ -576,40 +553,6 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_kernel(
       }
     }
   }
-}
-
-// The segments of several chunks are listed per XCD (long_records[x][...], lengths in the high word
-// of each XCD's counter line).  A wavefront walks the concatenation of the eight lists.
-struct LongLists {
-  int len[kNumXcd];
-  int64_t total;
-  int64_t capacity;  // records per list
-};
-__device__ __forceinline__ LongLists long_lists(const int32_t *__restrict__ counters, int64_t max_long) {
-  LongLists l;
-  l.total = 0;
-  l.capacity = max_long / kNumXcd;
-#pragma unroll
-  for (int x = 0; x < kNumXcd; ++x) {
-    l.len[x] = counters[xcd_counter(x) + 1];
-    l.total += l.len[x];
-  }
-  return l;
-}
-__device__ __forceinline__ LongRecord long_record_at(const LongRecord *__restrict__ long_records, const LongLists &l,
-                                                     int64_t slot) {
-  // (straight-line: a list picked by a run-time index would put the eight lengths into scratch memory)
-  int64_t at = 0;
-  bool found = false;
-#pragma unroll
-  for (int x = 0; x < kNumXcd; ++x) {
-    if (!found && slot < l.len[x]) {
-      at = x * l.capacity + slot;
-      found = true;
-    }
-    slot -= l.len[x];
-  }
-  return long_records[at];
 }
 
 // The approximate Adagrad's rows that were summed in several chunks: their state takes the addends

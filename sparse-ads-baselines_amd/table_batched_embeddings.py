@@ -409,7 +409,7 @@ def _backward_mixed(optimizer, grad_output, weights, table_offsets, table_dim_of
     state_dtype = torch.float64 if weights.dtype == torch.float64 else torch.float32
     _require(optimizer_state.dtype == state_dtype and optimizer_state.is_contiguous(),
              "optimizer_state must be contiguous %s" % state_dtype)
-    layout = _native.backward_workspace_layout(indices.numel(), 4, code, T)
+    layout = _native.backward_mixed_workspace_layout(indices.numel(), code, T)
     stochastic = bool(stochastic_rounding) and weights.dtype == torch.float16
     seed, offset = _rounding_stream(weights.device) if stochastic else (0, 0)
     with _workspace(weights.device, layout.total_bytes) as (ws, stream), torch.cuda.device(weights.device):

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 20
+ABI_VERSION = 21
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -87,6 +87,7 @@ SIGNATURES = {
     "tbe_probe_row_access": (ctypes.c_int, [_vp, _i32, _c_i32p, _i64, _vp, _i32, _vp, _vp]),
     "tbe_forward": (ctypes.c_int, [_vp, _i32, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp, _vp, _vp]),
     "tbe_backward_workspace_layout": (ctypes.c_int, [_i64, _i32, _i32, _i32, ctypes.POINTER(WorkspaceLayout)]),
+    "tbe_backward_mixed_workspace_layout": (ctypes.c_int, [_i64, _i32, _i32, ctypes.POINTER(WorkspaceLayout)]),
     "tbe_backward_sgd": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64, _c_i32p,
                                         _i32, _f32, _vp, _u64, _vp]),
     "tbe_backward_sgd_static": (ctypes.c_int, [_vp, _vp, _i32, _i64, _i64, _i32, _c_i32p, _i32, _c_i32p, _i64,
@@ -179,6 +180,12 @@ def check(code):
 def backward_workspace_layout(num_indices, D, dtype_code, T):
     layout = WorkspaceLayout()
     check(load().tbe_backward_workspace_layout(num_indices, D, dtype_code, T, ctypes.byref(layout)))
+    return layout
+
+
+def backward_mixed_workspace_layout(num_indices, dtype_code, T):
+    layout = WorkspaceLayout()
+    check(load().tbe_backward_mixed_workspace_layout(num_indices, dtype_code, T, ctypes.byref(layout)))
     return layout
 
 

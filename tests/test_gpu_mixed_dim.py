@@ -51,8 +51,9 @@ def test_backward_mixed_matches_oracle(oracle, tables, mode, dtype):
 @pytest.mark.parametrize("mode", ["sgd", "adagrad", "adagrad_weighted"])
 def test_backward_mixed_hot_rows(oracle, mode, dtype):
     """Thousands of lookups per table: rows with one occurrence (strip fast path), a few (strip
-    batches), 9..256 (one wavefront per row) and more than 256 (16 wavefronts per row), also in
-    a table whose rows are wider than 64 vectors, and more than 64 unique rows per table."""
+    batches), 9..256 (one chunk record, one wavefront) and more than 256 (several chunks, partial
+    rows, the finishing kernel), also in a table whose rows are wider than 64 vectors, and more
+    than 64 unique rows per table."""
     tables = [(3, 520), (2000, 36), (5, 64), (4000, 128), (1, 8), (700, 200)]
     _check_backward_mixed(oracle, tables, mode, dtype, B=300, L=24)
 
@@ -159,7 +160,7 @@ def test_mixed_bad_arguments():
 def test_backward_mixed_random_sweep(oracle, seed):
     """Seeded random table sets: 1..12 tables, rows from 1 to thousands, widths from 4 to wider
     than a wavefront pass (power-of-two and odd vector counts), bags from a handful to hundreds,
-    so that single-occurrence rows, batches, wavefront-per-row and workgroup-per-row all occur."""
+    so that single-occurrence rows, batches, rows of one chunk and rows of several chunks all occur."""
     rs = np.random.RandomState(500 + seed)
     T = int(rs.choice([1, 2, 3, 6, 12]))
     tables = [(int(rs.choice([1, 3, 40, 600, 5000])), int(rs.choice([4, 8, 12, 20, 32, 64, 100, 128, 256, 264, 520])))
@@ -169,3 +170,36 @@ def test_backward_mixed_random_sweep(oracle, seed):
     B = int(rs.choice([1, 9, 70, 400]))
     L = int(rs.choice([1, 5, 20]))
     _check_backward_mixed(oracle, tables, mode, dtype, B=B, L=L)
+
+
+def test_backward_mixed_rows_of_many_chunks_across_queue_boundaries(oracle):
+    """Eight tables of one or two rows each, hundreds of lookups per bag: every row is summed in
+    several chunks, and the rows -- one or two per eighth of the sorted positions -- put their chunk
+    records into different per-XCD queues; widths of 1, 3, 12 and 64 vectors."""
+    tables = [(1, 4), (2, 12), (1, 48), (2, 256), (1, 8), (2, 100), (1, 64), (2, 36)]
+    for mode in ("sgd", "adagrad_weighted"):
+        _check_backward_mixed(oracle, tables, mode, np.float32, B=40, L=60)
+
+
+def test_backward_mixed_workspace_size_is_checked():
+    """The workspace must follow tbe_backward_mixed_workspace_layout: a smaller one (here the
+    layout of uniform tables of four columns) is refused, not overrun."""
+    import tbe_native
+    p = make_mixed_problem(3, [(50, 8), (20, 16), (10, 4)], B=10, L=4, dtype=np.float32)
+    n, T = p["n"], 3
+    need = tbe_native.backward_mixed_workspace_layout(n, tbe_native.DTYPE_F32, T).total_bytes
+    small = tbe_native.backward_workspace_layout(n, 4, tbe_native.DTYPE_F32, T).total_bytes
+    assert small < need
+    ws = torch.zeros(small, dtype=torch.uint8, device=DEV)
+    w, go = dev(p["weights"]), dev(p["grad_output"])
+    to, tdo, do = dev(p["table_offsets"]), dev(p["table_dim_offsets"]), dev(p["dim_offsets"])
+    idx, off = dev(p["indices"]), dev(p["offsets"])
+    vp = lambda t: t.data_ptr()
+    rc = tbe_native.load().tbe_backward_mixed(
+        tbe_native.OPT_SGD, vp(go), vp(w), tbe_native.DTYPE_F32, 4, 80, 0, vp(to), vp(tdo), vp(do),
+        int(p["dim_offsets"][-1]), 3, vp(idx), idx.numel(), vp(off), 10, None, None, 0.1, 0.0, None, 0, 0, 0,
+        vp(ws), ws.numel(), None)
+    assert rc == 2  # TBE_ERR_WORKSPACE
+    assert "workspace" in tbe_native.load().tbe_last_error().decode()
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(w.cpu().numpy(), p["weights"])
