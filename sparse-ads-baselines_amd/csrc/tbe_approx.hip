@@ -739,6 +739,214 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
   }
 }
 
+// Staged walk of a very long fp16 row without per-sample weights or stochastic rounding.  What is
+// serial in such a row is one multiply-add and one rounding per occurrence and element; fetching
+// the occurrence's gradient row and multiplier through lane reads and row requests costs the walking
+// wavefront several times that.  So a workgroup takes the row: its first wavefront only walks --
+// gradient rows and multipliers of kStageStep occurrences at a time come out of LDS, at addresses
+// known when the kernel is compiled -- while the other three wavefronts gather the next step's
+// gradient rows into the other half of the LDS buffers (requested a step before they are written
+// there), and the second wavefront also keeps the row's running state (the prefix sums over
+// batches of 64 occurrences of walk_long_row: the same additions in the same order) and forms
+// the multipliers.  One barrier per step.
+constexpr int kStageStep = 128;  // occurrences per step
+constexpr int kStageD = 64;      // widest row walked this way: one element per lane
+// (a step's gradient rows lie transposed in LDS: the kStageStep values of one element side by side,
+// so that the walking lane reads eight occurrences of its element at once; four values of padding
+// per element keep the gathering wavefronts' scattered 2-byte writes off each other's banks)
+constexpr int kStageRow = kStageStep + 4;
+template <typename T> struct StageBuffers {
+  T rows[2][kStageD][kStageRow];
+  alignas(16) float mult[2][kStageStep];
+  int64_t goff[3][kStageStep];  // first element of every occurrence's gradient row
+};
+template <typename T>
+__device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_begin, int seg_end, int64_t key,
+                                            const RowPlace &place, T *storage, StageBuffers<T> &lds) {
+  using A = typename AccOf<T>::type;
+  static_assert(sizeof(T) == 2 && sizeof(A) == 4, "fp16 rows with fp32 arithmetic");
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = static_cast<int>(threadIdx.x >> 6);
+  const int len = seg_end - seg_begin;
+  const int steps = (len + kStageStep - 1) / kStageStep;
+  const int last = seg_end - 1;
+  const bool active = lane < place.row_D;
+  const int lane_off = active ? lane : 0;  // (idle lanes shadow lane 0 and store nothing)
+
+  // ---- the second wavefront's bookkeeping: two occurrences of a step per lane
+  A running = A(0);
+  auto positions_of = [&](int step, int (&pos)[2]) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) pos[h] = a.positions_sorted[min(seg_begin + step * kStageStep + h * kWave + lane, last)];
+  };
+  // (what a step's bookkeeping reads from memory is requested first, in one go, and used after the
+  // step's gathering, so that a step costs the helpers one memory round trip)
+  struct StepLoads {
+    int grow[2];
+    A wss[2];
+  };
+  auto request_bookkeeping = [&](const int (&pos_offsets)[2], const int (&pos_multipliers)[2], StepLoads &l) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) l.grow[h] = a.grad_rows[pos_offsets[h]];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) l.wss[h] = a.lookup_wss[pos_multipliers[h]];
+  };
+  auto write_offsets = [&](int step, const StepLoads &l) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) lds.goff[step % 3][h * kWave + lane] = long_row_grad_offset(l.grow[h], place, a.mt);
+  };
+  auto write_multipliers = [&](int step, const StepLoads &l) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int nb = min(kWave, len - step * kStageStep - h * kWave);  // occurrences of this batch of 64
+      if (nb > 0) {
+        const A incl = wave_inclusive_sum<A>(lane < nb ? l.wss[h] : A(0));
+        lds.mult[step & 1][h * kWave + lane] =
+            lane < nb ? approx_multiplier<A>(running + incl, A(1), false, a.lr, a.eps) : A(0);
+        running = running + broadcast_lane(incl, nb - 1);
+      }
+    }
+  };
+  // ---- the gathering wavefronts: 8-byte pieces of the rows, `pieces` (a power of two) per row;
+  // all of a thread's pieces of a step are requested before the first is written to LDS
+  const int helper = static_cast<int>(threadIdx.x) - kWave;
+  int piece_shift = 0;
+  while ((4 << piece_shift) < place.row_D) ++piece_shift;
+  const int piece = helper & ((1 << piece_shift) - 1);
+  const int rows_per_round = (kBlockThreads - kWave) >> piece_shift;  // at least 12: rows of 16 pieces
+  constexpr int kRounds = (kStageStep + 11) / 12;
+  uint2 held[kRounds];  // the thread's pieces of the step whose rows are on their way
+  auto request_rows = [&](int step) {
+    const int count = min(kStageStep, len - step * kStageStep);
+    if (piece * 4 >= place.row_D) return;
+    const int o0 = helper >> piece_shift;
+#pragma unroll
+    for (int k = 0; k < kRounds; ++k) {
+      const int o = min(o0 + k * rows_per_round, count - 1);
+      held[k] = *reinterpret_cast<const uint2 *>(a.grad_output + lds.goff[step % 3][o] + piece * 4);
+    }
+  };
+  auto store_rows = [&](int step) {
+    const int count = min(kStageStep, len - step * kStageStep);
+    if (piece * 4 >= place.row_D) return;
+    const int o0 = helper >> piece_shift;
+#pragma unroll
+    for (int k = 0; k < kRounds; ++k) {
+      const int o = o0 + k * rows_per_round;
+      if (o < count) {
+        T four[4];
+        __builtin_memcpy(four, &held[k], 8);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) lds.rows[step & 1][piece * 4 + e][o] = four[e];
+      }
+    }
+  };
+
+  // Everything runs ahead of the walk by whole steps, so that no wavefront waits for memory inside
+  // a step: while step b is walked, the rows of step b + 1 (requested during step b - 1) are
+  // written to LDS and those of step b + 2 requested, the multipliers of step b + 1 and the row
+  // offsets of step b + 3 are formed from what was requested during step b - 1, and the state
+  // addends of step b + 2, the gradient row numbers of step b + 4 and the positions of step b + 6
+  // are requested.
+  int pos2[2] = {0, 0}, pos3[2] = {0, 0}, pos4[2] = {0, 0}, pos5[2] = {0, 0};  // positions of the steps b + 2 .. b + 5
+  StepLoads ahead{};  // requested during step b - 1: gradient rows of step b + 3, state addends of step b + 1
+  if (wave == 1) {
+    int pos0[2], pos1[2];
+    positions_of(0, pos0);
+    positions_of(1, pos1);
+    positions_of(2, pos2);
+    positions_of(3, pos3);
+    positions_of(4, pos4);
+    positions_of(5, pos5);
+    running = a.state[key];
+    StepLoads first, second, third;
+    request_bookkeeping(pos0, pos0, first);
+    request_bookkeeping(pos1, pos1, second);
+    request_bookkeeping(pos2, pos2, third);
+    write_offsets(0, first);
+    write_multipliers(0, first);
+    write_offsets(1, second);
+    write_offsets(2, third);
+    request_bookkeeping(pos3, pos1, ahead);
+  }
+  __syncthreads();
+  if (wave >= 1) {
+    request_rows(0);
+    store_rows(0);
+    if (steps > 1) request_rows(1);
+  }
+  __syncthreads();
+
+  A w = to_acc(storage[lane_off]);
+  for (int b = 0; b < steps; ++b) {
+    if (wave == 0) {
+      // eight occurrences at a time: the next eight are requested before the current eight are
+      // applied (the barrier keeps the instruction scheduler from moving the requests back down)
+      const int count = min(kStageStep, len - b * kStageStep);
+      const T *mine = lds.rows[b & 1][lane_off];
+      const float *mult = lds.mult[b & 1];
+      struct Eight {
+        T g[8];
+        float m[8];
+      };
+      auto fetch = [&](int first, Eight &e) {
+        __builtin_memcpy(&e.g[0], mine + first, 8);
+        __builtin_memcpy(&e.g[4], mine + first + 4, 8);
+        __builtin_memcpy(&e.m[0], mult + first, 16);
+        __builtin_memcpy(&e.m[4], mult + first + 4, 16);
+      };
+      auto apply = [&](const Eight &e, int limit) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          if (k < limit) {
+            w = w - to_acc(e.g[k]) * e.m[k];
+            w = __half2float(__float2half_rn(w));
+          }
+        }
+      };
+      Eight even, odd;
+      fetch(0, even);
+      if (count == kStageStep) {
+#pragma unroll
+        for (int first = 0; first < kStageStep; first += 16) {
+          fetch(first + 8, odd);
+          __builtin_amdgcn_sched_barrier(0);
+          apply(even, 8);
+          if (first + 16 < kStageStep) fetch(first + 16, even);
+          __builtin_amdgcn_sched_barrier(0);
+          apply(odd, 8);
+        }
+      } else {
+        for (int first = 0; first < count; first += 8) {
+          apply(even, count - first);
+          if (first + 8 < count) fetch(first + 8, even);
+        }
+      }
+    } else {
+      StepLoads requested{};
+      if (wave == 1) request_bookkeeping(pos4, pos2, requested);  // (clamped positions: always valid)
+      if (b + 1 < steps) store_rows(b + 1);
+      if (b + 2 < steps) request_rows(b + 2);
+      if (wave == 1) {
+        if (b + 1 < steps) write_multipliers(b + 1, ahead);
+        if (b + 3 < steps) write_offsets(b + 3, ahead);
+        ahead = requested;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          pos2[h] = pos3[h];
+          pos3[h] = pos4[h];
+          pos4[h] = pos5[h];
+        }
+        positions_of(b + 6, pos5);
+      }
+    }
+    // (the gathered rows are in LDS: a wavefront's reads have arrived before it writes them there)
+    step_barrier();
+  }
+  if (wave == 0 && active) storage[lane] = from_acc<T, A>(w);  // (already rounded: exact)
+  if (wave == 1 && lane == 0) a.state[key] = running;
+}
+
 // One wavefront per queued row (a row of at most 64 vectors with more occurrences than the kernel
 // that queued it handles itself).  BIG: grad_output has 4 GiB or more, its rows are addressed
 // with 64-bit offsets instead of through a buffer descriptor.
@@ -790,13 +998,17 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
   int block_index = static_cast<int>(blockIdx.x);
   int grid_blocks = static_cast<int>(gridDim.x);
 
-  if constexpr (STOCHASTIC) {
-    // Rows of more than kApproxHuge occurrences, at most kCoopD wide: a whole workgroup per row
-    // (see draw_step_bits).  When the grid is large enough, the first workgroups do nothing else
-    // -- as many as there are such rows, rounded up to a multiple of the XCD count, at most half
-    // the grid -- and the others share the remaining rows as if they were the whole grid.
-    __shared__ __align__(16) uint16_t s_words[2 * kCoopStep * kCoopD];
-    if (queue_capacity > 0 && a.mt.T == 0 && D <= kCoopD && first_total > 0) {
+  // Rows of more than kApproxHuge occurrences get a whole workgroup where that shortens the walk:
+  // with stochastic rounding (rows at most kCoopD wide, see draw_step_bits), and for fp16 rows at
+  // most kStageD wide without per-sample weights (see staged_walk).  When the grid is large
+  // enough, the first workgroups do nothing else -- as many as there are such rows, rounded up
+  // to a multiple of the XCD count, at most half the grid -- and the others share the remaining
+  // rows as if they were the whole grid.
+  constexpr bool kStaged = !STOCHASTIC && !WEIGHTED && sizeof(T) == 2;
+  if constexpr (STOCHASTIC || kStaged) {
+    using Shared = typename std::conditional<kStaged, StageBuffers<T>, uint16_t[2 * kCoopStep * kCoopD]>::type;
+    __shared__ __align__(16) Shared s_shared;
+    if (queue_capacity > 0 && a.mt.T == 0 && D <= (kStaged ? kStageD : kCoopD) && first_total > 0) {
       const bool dedicated = grid_blocks >= 2 * kNumXcd;
       const int coop_blocks =
           dedicated ? min((first_total + kNumXcd - 1) / kNumXcd * kNumXcd, grid_blocks / (2 * kNumXcd) * kNumXcd) : 0;
@@ -806,24 +1018,29 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
         __builtin_amdgcn_s_setprio(3);
         for (int h = block_index; h < first_total; h += dedicated ? coop_blocks : grid_blocks) {
           const QueuedRow r = row_at(kNumXcd * queue_capacity + h);
-          const int len = r.seg_end - r.seg_begin;
-          const int steps = (len + kCoopStep - 1) / kCoopStep;
-          draw_step_bits(a.sr, r.place.row_element, r.place.row_D, 0, min(kCoopStep, len), s_words,
-                         static_cast<int>(threadIdx.x), kBlockThreads);
-          __syncthreads();
-          if (wave_in_block == 0) {
-            // (one barrier per step inside the walk)
-            if (r.place.row_D <= kWave)
-              walk_long_row<T, 1, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane, s_words);
-            else
-              walk_long_row<T, 2, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane, s_words);
+          if constexpr (kStaged) {
+            staged_walk<T>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
           } else {
-            for (int s = 1; s <= steps; ++s) {
-              if (s < steps)
-                draw_step_bits(a.sr, r.place.row_element, r.place.row_D, s * kCoopStep,
-                               min(kCoopStep, len - s * kCoopStep), s_words + (s & 1) * (kCoopStep * kCoopD),
-                               static_cast<int>(threadIdx.x) - kWave, kBlockThreads - kWave);
-              step_barrier();
+            uint16_t *s_words = s_shared;
+            const int len = r.seg_end - r.seg_begin;
+            const int steps = (len + kCoopStep - 1) / kCoopStep;
+            draw_step_bits(a.sr, r.place.row_element, r.place.row_D, 0, min(kCoopStep, len), s_words,
+                           static_cast<int>(threadIdx.x), kBlockThreads);
+            __syncthreads();
+            if (wave_in_block == 0) {
+              // (one barrier per step inside the walk)
+              if (r.place.row_D <= kWave)
+                walk_long_row<T, 1, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane, s_words);
+              else
+                walk_long_row<T, 2, WEIGHTED, true, BIG, true>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, lane, s_words);
+            } else {
+              for (int s = 1; s <= steps; ++s) {
+                if (s < steps)
+                  draw_step_bits(a.sr, r.place.row_element, r.place.row_D, s * kCoopStep,
+                                 min(kCoopStep, len - s * kCoopStep), s_words + (s & 1) * (kCoopStep * kCoopD),
+                                 static_cast<int>(threadIdx.x) - kWave, kBlockThreads - kWave);
+                step_barrier();
+              }
             }
           }
           __syncthreads();  // the buffers are free for the next row

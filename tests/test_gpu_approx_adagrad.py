@@ -394,6 +394,40 @@ def test_approx_adagrad_stochastic_rounding_bit_for_bit_with_dyadic_gradients(or
     assert (w.view(np.uint16) != w_rn.view(np.uint16)).mean() > 0.05  # and it is not round-to-nearest
 
 
+@pytest.mark.parametrize("D,B", [(8, 900), (36, 900), (64, 900), (100, 900), (64, 64)])
+def test_approx_adagrad_fp16_rows_of_many_occurrences_staged_through_lds(oracle, D, B):
+    """fp16 rows of more than 256 occurrences without per-sample weights, up to 64 elements wide, are
+    walked by a workgroup whose other wavefronts stage gradient rows and multipliers in LDS, 128
+    occurrences a step (run lengths: one past two steps, exactly three steps, one more, many;
+    D = 100: a single wavefront; B = 64: a grid too small to set workgroups aside).  With
+    per-sample weights the same rows are walked by a single wavefront -- and weights of one
+    change no value of the update, so the two runs must agree bit for bit in rows and state.
+    Against the oracle: with gradient entries in {0, +-0.5, +-1} every sum of squares is exact
+    in fp32 whatever its order, so the state must be the oracle's bit for bit; the rows at the fp16
+    tolerance (the kernels' fused multiply-add rounds row - mult * grad once, the oracle, like the
+    reference, to fp32 and then to fp16, which now and then lands on the neighbouring value)."""
+    rs = np.random.RandomState(3 * D + B)
+    T, E, L = (2 if B > 100 else 1), 60, 8
+    p = make_problem(43, T=T, E=E, D=D, B=B, L=L, dtype=np.float16, ragged=False, weighted=False)
+    n_t = B * L
+    hot = [257, 384, 385, 1000, 2049] if B > 100 else [300]
+    mid = [17, 64, 65, 200, 256] if B > 100 else [40]
+    for t in range(T):
+        rows = np.concatenate([np.full(c, r, np.int32) for r, c in enumerate(hot + mid)])
+        rest = rs.randint(len(hot + mid), E, size=n_t - rows.size).astype(np.int32)
+        p["indices"][t * n_t:(t + 1) * n_t] = rs.permutation(np.concatenate([rows, rest]))
+    p["grad_output"] = rs.choice(np.array([0, 0.5, -0.5, 1, -1], np.float16), size=p["grad_output"].shape)
+    w, st, _ = _run_gpu(p, 0.02, 0.1)
+    w_ref, st_ref, _ = _run_oracle(oracle, p, 0.02, 0.1)
+    assert st.tobytes() == st_ref.tobytes()
+    assert_close(w, w_ref, 1e-2)
+    ones = dict(p, per_sample_weights=np.ones(p["n"], np.float16))
+    w_one, st_one, _ = _run_gpu(ones, 0.02, 0.1)
+    assert st_one.tobytes() == st.tobytes()
+    differing = np.flatnonzero((w.view(np.uint16) != w_one.view(np.uint16)).any(axis=1))
+    assert differing.size == 0, "rows that differ between the two walks: %s" % differing[:10]
+
+
 def test_approx_adagrad_stochastic_rounding_more_long_rows_than_workgroups_set_aside(oracle):
     """1100 rows of 300 occurrences each: more rows for the cooperative walk than the 1024
     workgroups (half the largest grid) that are set aside for them, so those take a second
