@@ -744,21 +744,17 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
 // the occurrence's gradient row and multiplier through lane reads and row requests costs the walking
 // wavefront several times that.  So a workgroup takes the row: its first wavefront only walks --
 // gradient rows and multipliers of kStageStep occurrences at a time come out of LDS, at addresses
-// known when the kernel is compiled -- while the other three wavefronts gather the next step's
-// gradient rows into the other half of the LDS buffers (requested a step before they are written
-// there), and the second wavefront also keeps the row's running state (the prefix sums over
-// batches of 64 occurrences of walk_long_row: the same additions in the same order) and forms
-// the multipliers.  One barrier per step.
+// known when the kernel is compiled -- while the third and fourth wavefront gather the next
+// step's gradient rows into the other half of the LDS buffers (requested a step before they are
+// written there) and the second wavefront keeps the row's running state (the prefix sums over
+// batches of 64 occurrences of walk_long_row: the same additions in the same order), forms the
+// multipliers and looks up where the gradient rows are.  One barrier per step.
 constexpr int kStageStep = 128;  // occurrences per step
 constexpr int kStageD = 64;      // widest row walked this way: one element per lane
-// (a step's gradient rows lie transposed in LDS: the kStageStep values of one element side by side,
-// so that the walking lane reads eight occurrences of its element at once; four values of padding
-// per element keep the gathering wavefronts' scattered 2-byte writes off each other's banks)
-constexpr int kStageRow = kStageStep + 4;
 template <typename T> struct StageBuffers {
-  T rows[2][kStageD][kStageRow];
+  alignas(16) T rows[2][kStageStep][kStageD];
   alignas(16) float mult[2][kStageStep];
-  int64_t goff[3][kStageStep];  // first element of every occurrence's gradient row
+  int64_t goff[4][kStageStep];  // first element of every occurrence's gradient row
 };
 template <typename T>
 __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_begin, int seg_end, int64_t key,
@@ -793,7 +789,7 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
   };
   auto write_offsets = [&](int step, const StepLoads &l) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) lds.goff[step % 3][h * kWave + lane] = long_row_grad_offset(l.grow[h], place, a.mt);
+    for (int h = 0; h < 2; ++h) lds.goff[step & 3][h * kWave + lane] = long_row_grad_offset(l.grow[h], place, a.mt);
   };
   auto write_multipliers = [&](int step, const StepLoads &l) {
 #pragma unroll
@@ -807,91 +803,99 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
       }
     }
   };
-  // ---- the gathering wavefronts: 8-byte pieces of the rows, `pieces` (a power of two) per row;
-  // all of a thread's pieces of a step are requested before the first is written to LDS
-  const int helper = static_cast<int>(threadIdx.x) - kWave;
+  // ---- the gathering wavefronts (the third and fourth): 8-byte pieces of the rows, `pieces` (a
+  // power of two) per row; a thread's pieces of a step are requested a step before they are
+  // written to LDS
+  constexpr int kGatherThreads = kBlockThreads - 2 * kWave;
+  const int helper = static_cast<int>(threadIdx.x) - 2 * kWave;
   int piece_shift = 0;
   while ((4 << piece_shift) < place.row_D) ++piece_shift;
   const int piece = helper & ((1 << piece_shift) - 1);
-  const int rows_per_round = (kBlockThreads - kWave) >> piece_shift;  // at least 12: rows of 16 pieces
-  constexpr int kRounds = (kStageStep + 11) / 12;
-  uint2 held[kRounds];  // the thread's pieces of the step whose rows are on their way
-  auto request_rows = [&](int step) {
+  const int rows_per_round = kGatherThreads >> piece_shift;  // at least 8: rows of 16 pieces
+  constexpr int kRounds = kStageStep / (kGatherThreads / (kStageD / 4));
+  // (two sets of registers: the pieces of the steps b + 1 and b + 2 are on their way at a time)
+  uint2 held_even[kRounds], held_odd[kRounds];
+  auto request_rows = [&](int step, uint2 (&held)[kRounds]) {
     const int count = min(kStageStep, len - step * kStageStep);
-    if (piece * 4 >= place.row_D) return;
+    if (piece * 4 >= place.row_D || count <= 0) return;
     const int o0 = helper >> piece_shift;
 #pragma unroll
     for (int k = 0; k < kRounds; ++k) {
       const int o = min(o0 + k * rows_per_round, count - 1);
-      held[k] = *reinterpret_cast<const uint2 *>(a.grad_output + lds.goff[step % 3][o] + piece * 4);
+      held[k] = *reinterpret_cast<const uint2 *>(a.grad_output + lds.goff[step & 3][o] + piece * 4);
     }
   };
-  auto store_rows = [&](int step) {
+  auto store_rows = [&](int step, const uint2 (&held)[kRounds]) {
     const int count = min(kStageStep, len - step * kStageStep);
     if (piece * 4 >= place.row_D) return;
     const int o0 = helper >> piece_shift;
 #pragma unroll
     for (int k = 0; k < kRounds; ++k) {
       const int o = o0 + k * rows_per_round;
-      if (o < count) {
-        T four[4];
-        __builtin_memcpy(four, &held[k], 8);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) lds.rows[step & 1][piece * 4 + e][o] = four[e];
-      }
+      if (o < count) *reinterpret_cast<uint2 *>(&lds.rows[step & 1][o][piece * 4]) = held[k];
     }
   };
 
-  // Everything runs ahead of the walk by whole steps, so that no wavefront waits for memory inside
-  // a step: while step b is walked, the rows of step b + 1 (requested during step b - 1) are
-  // written to LDS and those of step b + 2 requested, the multipliers of step b + 1 and the row
-  // offsets of step b + 3 are formed from what was requested during step b - 1, and the state
-  // addends of step b + 2, the gradient row numbers of step b + 4 and the positions of step b + 6
-  // are requested.
-  int pos2[2] = {0, 0}, pos3[2] = {0, 0}, pos4[2] = {0, 0}, pos5[2] = {0, 0};  // positions of the steps b + 2 .. b + 5
-  StepLoads ahead{};  // requested during step b - 1: gradient rows of step b + 3, state addends of step b + 1
+  // Everything runs ahead of the walk by whole steps, and what comes from memory is requested two
+  // steps before it is used (a step lasts about as long as one memory round trip), so that no
+  // wavefront waits for memory inside a step.  While step b is walked: the rows of step b + 1
+  // (requested during step b - 2) are written to LDS and those of step b + 3 requested; the
+  // multipliers of step b + 1 and the row offsets of step b + 4 are formed from what was requested
+  // during step b - 2; the state addends of step b + 3, the gradient row numbers of step b + 6 and
+  // the positions of step b + 8 are requested.
+  int pos3[2] = {0, 0}, pos4[2] = {0, 0}, pos5[2] = {0, 0}, pos6[2] = {0, 0}, pos7[2] = {0, 0};  // steps b + 3 .. b + 7
+  StepLoads due{}, coming{};  // requested during the steps b - 2 and b - 1
   if (wave == 1) {
-    int pos0[2], pos1[2];
+    int pos0[2], pos1[2], pos2[2];
     positions_of(0, pos0);
     positions_of(1, pos1);
     positions_of(2, pos2);
     positions_of(3, pos3);
     positions_of(4, pos4);
     positions_of(5, pos5);
+    positions_of(6, pos6);
+    positions_of(7, pos7);
     running = a.state[key];
-    StepLoads first, second, third;
+    StepLoads first, second, third, fourth;
     request_bookkeeping(pos0, pos0, first);
     request_bookkeeping(pos1, pos1, second);
     request_bookkeeping(pos2, pos2, third);
+    request_bookkeeping(pos3, pos3, fourth);
     write_offsets(0, first);
     write_multipliers(0, first);
     write_offsets(1, second);
     write_offsets(2, third);
-    request_bookkeeping(pos3, pos1, ahead);
+    write_offsets(3, fourth);
+    request_bookkeeping(pos4, pos1, due);     // (as if during step -2: offsets of step 4, multipliers of step 1)
+    request_bookkeeping(pos5, pos2, coming);  // (as if during step -1)
   }
   __syncthreads();
-  if (wave >= 1) {
-    request_rows(0);
-    store_rows(0);
-    if (steps > 1) request_rows(1);
+  if (wave >= 2) {
+    request_rows(0, held_even);
+    store_rows(0, held_even);
+    request_rows(1, held_odd);
+    request_rows(2, held_even);
   }
   __syncthreads();
 
   A w = to_acc(storage[lane_off]);
-  for (int b = 0; b < steps; ++b) {
+  // one step; `held`: the gathering threads' registers of step b + 1
+  auto step_of_walk = [&](int b, uint2 (&held)[kRounds]) {
     if (wave == 0) {
       // eight occurrences at a time: the next eight are requested before the current eight are
-      // applied (the barrier keeps the instruction scheduler from moving the requests back down)
+      // applied (the barrier keeps the instruction scheduler from moving the requests back down).
+      // The chain of dependent updates leaves the wavefront idle two thirds of the time, which is
+      // where the ten LDS reads of eight occurrences go.
       const int count = min(kStageStep, len - b * kStageStep);
-      const T *mine = lds.rows[b & 1][lane_off];
+      const T *mine = &lds.rows[b & 1][0][lane_off];
       const float *mult = lds.mult[b & 1];
       struct Eight {
         T g[8];
         float m[8];
       };
       auto fetch = [&](int first, Eight &e) {
-        __builtin_memcpy(&e.g[0], mine + first, 8);
-        __builtin_memcpy(&e.g[4], mine + first + 4, 8);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) e.g[k] = mine[(first + k) * kStageD];
         __builtin_memcpy(&e.m[0], mult + first, 16);
         __builtin_memcpy(&e.m[4], mult + first + 4, 16);
       };
@@ -923,25 +927,32 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
         }
       }
     } else {
-      StepLoads requested{};
-      if (wave == 1) request_bookkeeping(pos4, pos2, requested);  // (clamped positions: always valid)
-      if (b + 1 < steps) store_rows(b + 1);
-      if (b + 2 < steps) request_rows(b + 2);
-      if (wave == 1) {
-        if (b + 1 < steps) write_multipliers(b + 1, ahead);
-        if (b + 3 < steps) write_offsets(b + 3, ahead);
-        ahead = requested;
+      if (wave >= 2) {
+        if (b + 1 < steps) store_rows(b + 1, held);
+        request_rows(b + 3, held);
+      } else {
+        StepLoads requested{};
+        request_bookkeeping(pos6, pos3, requested);  // (clamped positions: always valid)
+        if (b + 1 < steps) write_multipliers(b + 1, due);
+        if (b + 4 < steps) write_offsets(b + 4, due);
+        due = coming;
+        coming = requested;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          pos2[h] = pos3[h];
           pos3[h] = pos4[h];
           pos4[h] = pos5[h];
+          pos5[h] = pos6[h];
+          pos6[h] = pos7[h];
         }
-        positions_of(b + 6, pos5);
+        positions_of(b + 8, pos7);
       }
     }
     // (the gathered rows are in LDS: a wavefront's reads have arrived before it writes them there)
     step_barrier();
+  };
+  for (int b = 0; b < steps; b += 2) {
+    step_of_walk(b, held_odd);
+    if (b + 1 < steps) step_of_walk(b + 1, held_even);
   }
   if (wave == 0 && active) storage[lane] = from_acc<T, A>(w);  // (already rounded: exact)
   if (wave == 1 && lane == 0) a.state[key] = running;
