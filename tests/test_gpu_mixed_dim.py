@@ -181,6 +181,38 @@ def test_backward_mixed_rows_of_many_chunks_across_queue_boundaries(oracle):
         _check_backward_mixed(oracle, tables, mode, np.float32, B=40, L=60)
 
 
+def test_backward_mixed_densest_chunk_records(oracle):
+    """Every row nine times: the most chunk records a batch can queue (one per nine lookups), in
+    every one of the eight per-XCD queues, with strips of 64 unique rows straddling the boundaries
+    between the queues' eighths of the sorted positions and between tables of different widths."""
+    rows, times = 6400, 9
+    tables = [(rows, 8), (rows, 24), (rows, 4), (rows, 12), (rows, 8), (rows, 40), (rows, 4), (rows, 16)]
+    B, L = 960, 60  # B * L = rows * times lookups per table
+    p = make_mixed_problem(11, tables, B=B, L=L, dtype=np.float32)
+    rs = np.random.RandomState(12)
+    T = len(tables)
+    p["offsets"] = np.arange(0, T * B * L + 1, L, dtype=np.int32)
+    p["indices"] = np.concatenate([rs.permutation(np.repeat(np.arange(rows, dtype=np.int32), times))
+                                   for _ in range(T)])
+    p["n"] = p["indices"].size
+    for mode in ("sgd", "adagrad"):
+        w_ref = p["weights"].copy()
+        st_ref = np.zeros(T * rows, np.float32)
+        oracle.backward_mixed(mode, p["grad_output"], w_ref, p["table_offsets"], p["table_dim_offsets"],
+                              p["dim_offsets"], p["indices"], p["offsets"], 0.05, 0.1, st_ref)
+        w, st = dev(p["weights"]), torch.zeros(T * rows, device=DEV)
+        args = (dev(p["grad_output"]), w, dev(p["table_offsets"]), dev(p["table_dim_offsets"]), dev(p["dim_offsets"]),
+                int(p["dim_offsets"][-1]), dev(p["indices"]), dev(p["offsets"]))
+        if mode == "sgd":
+            ext.backward_sgd_mixed_D(*args, st, 0.05)
+        else:
+            ext.backward_exact_adagrad_mixed_D(*args, None, st, 0.05, 0.1, False, 1)
+        torch.cuda.synchronize()
+        assert_close(w.cpu().numpy(), w_ref, 1e-5)
+        if mode == "adagrad":
+            assert_close(st.cpu().numpy(), st_ref, 1e-5)
+
+
 def test_backward_mixed_workspace_size_is_checked():
     """The workspace must follow tbe_backward_mixed_workspace_layout: a smaller one (here the
     layout of uniform tables of four columns) is refused, not overrun."""
