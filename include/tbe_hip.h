@@ -166,7 +166,7 @@ TBE_API int tbe_backward_sgd(const void *grad_output, void *weights, int32_t dty
  * results, but the workspace is an array of TBE_STATIC_SCRATCH_BYTES that the library's code
  * object holds on every device it runs on; the call makes no hipMalloc / hipFree and no other
  * allocating call.  A batch whose workspace (tbe_backward_workspace_layout(...).total_bytes)
- * exceeds TBE_STATIC_SCRATCH_BYTES is refused with TBE_ERR_WORKSPACE -- about 0.75 M lookups fit.
+ * exceeds TBE_STATIC_SCRATCH_BYTES is refused with TBE_ERR_WORKSPACE -- about 0.8 M lookups fit.
  * The first call on a device resolves the array's address there (make it outside a capture).
  * All calls on one device share the array, which keeps the previous call's contents: every
  * counter the pipeline needs at zero is cleared by its own kernels at the start of each call,
