@@ -743,58 +743,64 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
 // serial in such a row is one multiply-add and one rounding per occurrence and element; fetching
 // the occurrence's gradient row and multiplier through lane reads and row requests costs the walking
 // wavefront several times that.  So a workgroup takes the row: its first wavefront only walks --
-// gradient rows and multipliers of kStageStep occurrences at a time come out of LDS, at addresses
-// known when the kernel is compiled -- while the third and fourth wavefront gather the next
-// step's gradient rows into the other half of the LDS buffers (requested a step before they are
-// written there) and the second wavefront keeps the row's running state (the prefix sums over
-// batches of 64 occurrences of walk_long_row: the same additions in the same order), forms the
-// multipliers and looks up where the gradient rows are.  One barrier per step.
-constexpr int kStageStep = 128;  // occurrences per step
-constexpr int kStageD = 64;      // widest row walked this way: one element per lane
+// gradient rows and multipliers of a step's occurrences come out of LDS, at addresses known when
+// the kernel is compiled -- while the third and fourth wavefront gather the next step's gradient
+// rows into the other half of the LDS buffers (requested two steps before they are written
+// there) and the second wavefront keeps the row's running state (the prefix sums over batches of
+// 64 occurrences of walk_long_row: the same additions in the same order), forms the multipliers
+// and looks up where the gradient rows are.  One barrier per step.
+// Rows of up to 64 elements: one element per lane, 128 occurrences a step; rows of up to 128
+// elements: two elements per lane, 64 occurrences a step (the same 16 KB of gradient rows).
+constexpr int kStageStep = 128;  // most occurrences per step
+constexpr int kStageD = 128;     // widest row walked this way
+constexpr int kStageElements = 128 * 64;  // elements of the gradient rows of one step
 template <typename T> struct StageBuffers {
-  alignas(16) T rows[2][kStageStep][kStageD];
+  alignas(16) T rows[2][kStageElements];  // [occurrence of the step][element of the row]
   alignas(16) float mult[2][kStageStep];
   int64_t goff[4][kStageStep];  // first element of every occurrence's gradient row
 };
-template <typename T>
+template <typename T, int E>
 __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_begin, int seg_end, int64_t key,
                                             const RowPlace &place, T *storage, StageBuffers<T> &lds) {
   using A = typename AccOf<T>::type;
   static_assert(sizeof(T) == 2 && sizeof(A) == 4, "fp16 rows with fp32 arithmetic");
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = static_cast<int>(threadIdx.x >> 6);
+  constexpr int kStep = kStageStep / E;  // occurrences per step
+  constexpr int kRowD = kWave * E;       // elements of a staged row
+  constexpr int kPerLane = kStep / kWave;  // occurrences of a step per lane of the bookkeeping wavefront
   const int len = seg_end - seg_begin;
-  const int steps = (len + kStageStep - 1) / kStageStep;
+  const int steps = (len + kStep - 1) / kStep;
   const int last = seg_end - 1;
-  const bool active = lane < place.row_D;
-  const int lane_off = active ? lane : 0;  // (idle lanes shadow lane 0 and store nothing)
+  const bool active = lane * E < place.row_D;
+  const int lane_off = active ? lane * E : 0;  // (idle lanes shadow lane 0 and store nothing)
 
-  // ---- the second wavefront's bookkeeping: two occurrences of a step per lane
+  // ---- the second wavefront's bookkeeping: kPerLane occurrences of a step per lane
   A running = A(0);
-  auto positions_of = [&](int step, int (&pos)[2]) {
+  auto positions_of = [&](int step, int (&pos)[kPerLane]) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) pos[h] = a.positions_sorted[min(seg_begin + step * kStageStep + h * kWave + lane, last)];
+    for (int h = 0; h < kPerLane; ++h) pos[h] = a.positions_sorted[min(seg_begin + step * kStep + h * kWave + lane, last)];
   };
   // (what a step's bookkeeping reads from memory is requested first, in one go, and used after the
   // step's gathering, so that a step costs the helpers one memory round trip)
   struct StepLoads {
-    int grow[2];
-    A wss[2];
+    int grow[kPerLane];
+    A wss[kPerLane];
   };
-  auto request_bookkeeping = [&](const int (&pos_offsets)[2], const int (&pos_multipliers)[2], StepLoads &l) {
+  auto request_bookkeeping = [&](const int (&pos_offsets)[kPerLane], const int (&pos_multipliers)[kPerLane], StepLoads &l) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) l.grow[h] = a.grad_rows[pos_offsets[h]];
+    for (int h = 0; h < kPerLane; ++h) l.grow[h] = a.grad_rows[pos_offsets[h]];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) l.wss[h] = a.lookup_wss[pos_multipliers[h]];
+    for (int h = 0; h < kPerLane; ++h) l.wss[h] = a.lookup_wss[pos_multipliers[h]];
   };
   auto write_offsets = [&](int step, const StepLoads &l) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) lds.goff[step & 3][h * kWave + lane] = long_row_grad_offset(l.grow[h], place, a.mt);
+    for (int h = 0; h < kPerLane; ++h) lds.goff[step & 3][h * kWave + lane] = long_row_grad_offset(l.grow[h], place, a.mt);
   };
   auto write_multipliers = [&](int step, const StepLoads &l) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int nb = min(kWave, len - step * kStageStep - h * kWave);  // occurrences of this batch of 64
+    for (int h = 0; h < kPerLane; ++h) {
+      const int nb = min(kWave, len - step * kStep - h * kWave);  // occurrences of this batch of 64
       if (nb > 0) {
         const A incl = wave_inclusive_sum<A>(lane < nb ? l.wss[h] : A(0));
         lds.mult[step & 1][h * kWave + lane] =
@@ -804,19 +810,19 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
     }
   };
   // ---- the gathering wavefronts (the third and fourth): 8-byte pieces of the rows, `pieces` (a
-  // power of two) per row; a thread's pieces of a step are requested a step before they are
+  // power of two) per row; a thread's pieces of a step are requested two steps before they are
   // written to LDS
   constexpr int kGatherThreads = kBlockThreads - 2 * kWave;
   const int helper = static_cast<int>(threadIdx.x) - 2 * kWave;
   int piece_shift = 0;
   while ((4 << piece_shift) < place.row_D) ++piece_shift;
   const int piece = helper & ((1 << piece_shift) - 1);
-  const int rows_per_round = kGatherThreads >> piece_shift;  // at least 8: rows of 16 pieces
-  constexpr int kRounds = kStageStep / (kGatherThreads / (kStageD / 4));
+  const int rows_per_round = kGatherThreads >> piece_shift;  // at least 128 / (kRowD / 4)
+  constexpr int kRounds = kStep / (kGatherThreads / (kRowD / 4));
   // (two sets of registers: the pieces of the steps b + 1 and b + 2 are on their way at a time)
   uint2 held_even[kRounds], held_odd[kRounds];
   auto request_rows = [&](int step, uint2 (&held)[kRounds]) {
-    const int count = min(kStageStep, len - step * kStageStep);
+    const int count = min(kStep, len - step * kStep);
     if (piece * 4 >= place.row_D || count <= 0) return;
     const int o0 = helper >> piece_shift;
 #pragma unroll
@@ -826,13 +832,13 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
     }
   };
   auto store_rows = [&](int step, const uint2 (&held)[kRounds]) {
-    const int count = min(kStageStep, len - step * kStageStep);
+    const int count = min(kStep, len - step * kStep);
     if (piece * 4 >= place.row_D) return;
     const int o0 = helper >> piece_shift;
 #pragma unroll
     for (int k = 0; k < kRounds; ++k) {
       const int o = o0 + k * rows_per_round;
-      if (o < count) *reinterpret_cast<uint2 *>(&lds.rows[step & 1][o][piece * 4]) = held[k];
+      if (o < count) *reinterpret_cast<uint2 *>(&lds.rows[step & 1][o * kRowD + piece * 4]) = held[k];
     }
   };
 
@@ -843,10 +849,10 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
   // multipliers of step b + 1 and the row offsets of step b + 4 are formed from what was requested
   // during step b - 2; the state addends of step b + 3, the gradient row numbers of step b + 6 and
   // the positions of step b + 8 are requested.
-  int pos3[2] = {0, 0}, pos4[2] = {0, 0}, pos5[2] = {0, 0}, pos6[2] = {0, 0}, pos7[2] = {0, 0};  // steps b + 3 .. b + 7
+  int pos3[kPerLane] = {}, pos4[kPerLane] = {}, pos5[kPerLane] = {}, pos6[kPerLane] = {}, pos7[kPerLane] = {};  // steps b + 3 .. b + 7
   StepLoads due{}, coming{};  // requested during the steps b - 2 and b - 1
   if (wave == 1) {
-    int pos0[2], pos1[2], pos2[2];
+    int pos0[kPerLane], pos1[kPerLane], pos2[kPerLane];
     positions_of(0, pos0);
     positions_of(1, pos1);
     positions_of(2, pos2);
@@ -878,7 +884,9 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
   }
   __syncthreads();
 
-  A w = to_acc(storage[lane_off]);
+  A w[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) w[i] = to_acc(storage[lane_off + i]);
   // one step; `held`: the gathering threads' registers of step b + 1
   auto step_of_walk = [&](int b, uint2 (&held)[kRounds]) {
     if (wave == 0) {
@@ -886,16 +894,16 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
       // applied (the barrier keeps the instruction scheduler from moving the requests back down).
       // The chain of dependent updates leaves the wavefront idle two thirds of the time, which is
       // where the ten LDS reads of eight occurrences go.
-      const int count = min(kStageStep, len - b * kStageStep);
-      const T *mine = &lds.rows[b & 1][0][lane_off];
+      const int count = min(kStep, len - b * kStep);
+      const T *mine = &lds.rows[b & 1][lane_off];
       const float *mult = lds.mult[b & 1];
       struct Eight {
-        T g[8];
+        T g[8][E];
         float m[8];
       };
       auto fetch = [&](int first, Eight &e) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) e.g[k] = mine[(first + k) * kStageD];
+        for (int k = 0; k < 8; ++k) __builtin_memcpy(&e.g[k][0], mine + (first + k) * kRowD, sizeof(T) * E);
         __builtin_memcpy(&e.m[0], mult + first, 16);
         __builtin_memcpy(&e.m[4], mult + first + 4, 16);
       };
@@ -903,20 +911,23 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           if (k < limit) {
-            w = w - to_acc(e.g[k]) * e.m[k];
-            w = __half2float(__float2half_rn(w));
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+              w[i] = w[i] - to_acc(e.g[k][i]) * e.m[k];
+              w[i] = __half2float(__float2half_rn(w[i]));
+            }
           }
         }
       };
       Eight even, odd;
       fetch(0, even);
-      if (count == kStageStep) {
+      if (count == kStep) {
 #pragma unroll
-        for (int first = 0; first < kStageStep; first += 16) {
+        for (int first = 0; first < kStep; first += 16) {
           fetch(first + 8, odd);
           __builtin_amdgcn_sched_barrier(0);
           apply(even, 8);
-          if (first + 16 < kStageStep) fetch(first + 16, even);
+          if (first + 16 < kStep) fetch(first + 16, even);
           __builtin_amdgcn_sched_barrier(0);
           apply(odd, 8);
         }
@@ -954,7 +965,10 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
     step_of_walk(b, held_odd);
     if (b + 1 < steps) step_of_walk(b + 1, held_even);
   }
-  if (wave == 0 && active) storage[lane] = from_acc<T, A>(w);  // (already rounded: exact)
+  if (wave == 0 && active) {  // (already rounded: exact)
+#pragma unroll
+    for (int i = 0; i < E; ++i) storage[lane_off + i] = from_acc<T, A>(w[i]);
+  }
   if (wave == 1 && lane == 0) a.state[key] = running;
 }
 
@@ -1030,7 +1044,8 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
         for (int h = block_index; h < first_total; h += dedicated ? coop_blocks : grid_blocks) {
           const QueuedRow r = row_at(kNumXcd * queue_capacity + h);
           if constexpr (kStaged) {
-            staged_walk<T>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
+            if (r.place.row_D <= kWave) staged_walk<T, 1>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
+            else staged_walk<T, 2>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
           } else {
             uint16_t *s_words = s_shared;
             const int len = r.seg_end - r.seg_begin;

@@ -394,12 +394,13 @@ def test_approx_adagrad_stochastic_rounding_bit_for_bit_with_dyadic_gradients(or
     assert (w.view(np.uint16) != w_rn.view(np.uint16)).mean() > 0.05  # and it is not round-to-nearest
 
 
-@pytest.mark.parametrize("D,B", [(8, 900), (36, 900), (64, 900), (100, 900), (64, 64)])
+@pytest.mark.parametrize("D,B", [(8, 900), (36, 900), (64, 900), (100, 900), (128, 900), (256, 900), (64, 64), (128, 64)])
 def test_approx_adagrad_fp16_rows_of_many_occurrences_staged_through_lds(oracle, D, B):
-    """fp16 rows of more than 256 occurrences without per-sample weights, up to 64 elements wide, are
+    """fp16 rows of more than 256 occurrences without per-sample weights, up to 128 elements wide, are
     walked by a workgroup whose other wavefronts stage gradient rows and multipliers in LDS, 128
-    occurrences a step (run lengths: one past two steps, exactly three steps, one more, many;
-    D = 100: a single wavefront; B = 64: a grid too small to set workgroups aside).  With
+    occurrences a step (D = 100: two elements per lane, 64 occurrences a step; run lengths: one
+    past a step boundary, exactly on one, one more, many; B = 64: a grid too small to set
+    workgroups aside).  With
     per-sample weights the same rows are walked by a single wavefront -- and weights of one
     change no value of the update, so the two runs must agree bit for bit in rows and state.
     Against the oracle: with gradient entries in {0, +-0.5, +-1} every sum of squares is exact
