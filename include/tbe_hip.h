@@ -121,7 +121,8 @@ typedef struct tbe_workspace_layout {
   uint64_t keys_sorted;
   uint64_t positions_sorted;
   uint64_t segment_starts;
-  uint64_t num_unique;       /* int32 [4]: U, #long rows, #chunks, #partial rows        */
+  uint64_t num_unique;       /* int32 [320]: U, then the update stage's queue counters
+                              * (one 128-byte line per eighth of the sorted positions)   */
   uint64_t sort_scratch;
   uint64_t segment_scratch;
   uint64_t segment_ids;      /* int32 [N]: index of the unique row of each sorted position */
