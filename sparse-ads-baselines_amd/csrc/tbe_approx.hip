@@ -739,7 +739,7 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
   }
 }
 
-// Staged walk of a very long fp16 row without per-sample weights or stochastic rounding.  What is
+// Staged walk of a very long fp16 row without stochastic rounding.  What is
 // serial in such a row is one multiply-add and one rounding per occurrence and element; fetching
 // the occurrence's gradient row and multiplier through lane reads and row requests costs the walking
 // wavefront several times that.  So a workgroup takes the row: its first wavefront only walks --
@@ -748,7 +748,10 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
 // rows into the other half of the LDS buffers (requested two steps before they are written
 // there) and the second wavefront keeps the row's running state (the prefix sums over batches of
 // 64 occurrences of walk_long_row: the same additions in the same order), forms the multipliers
-// and looks up where the gradient rows are.  One barrier per step.
+// and looks up where the gradient rows are.  One barrier per step.  With per-sample weights the
+// walking wavefront also forms <row, gradient row> of every occurrence (a sum over the wavefront by
+// lane moves, off the chain of dependent updates but in its instruction stream: 75 ns per occurrence
+// instead of 7).
 // Rows of up to 64 elements: one element per lane, 128 occurrences a step; rows of up to 128
 // elements: two elements per lane, 64 occurrences a step (the same 16 KB of gradient rows).
 constexpr int kStageStep = 128;  // most occurrences per step
@@ -757,9 +760,10 @@ constexpr int kStageElements = 128 * 64;  // elements of the gradient rows of on
 template <typename T> struct StageBuffers {
   alignas(16) T rows[2][kStageElements];  // [occurrence of the step][element of the row]
   alignas(16) float mult[2][kStageStep];
+  alignas(16) int32_t pos[2][kStageStep];  // (per-sample weights) position of every occurrence: where its grad_psw goes
   int64_t goff[4][kStageStep];  // first element of every occurrence's gradient row
 };
-template <typename T, int E>
+template <typename T, int E, bool WEIGHTED>
 __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_begin, int seg_end, int64_t key,
                                             const RowPlace &place, T *storage, StageBuffers<T> &lds) {
   using A = typename AccOf<T>::type;
@@ -786,12 +790,20 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
   struct StepLoads {
     int grow[kPerLane];
     A wss[kPerLane];
+    int pos[kPerLane];  // (WEIGHTED) the positions the multipliers belong to, and their per-sample weights
+    A pw[kPerLane];
   };
   auto request_bookkeeping = [&](const int (&pos_offsets)[kPerLane], const int (&pos_multipliers)[kPerLane], StepLoads &l) {
 #pragma unroll
     for (int h = 0; h < kPerLane; ++h) l.grow[h] = a.grad_rows[pos_offsets[h]];
 #pragma unroll
     for (int h = 0; h < kPerLane; ++h) l.wss[h] = a.lookup_wss[pos_multipliers[h]];
+#pragma unroll
+    for (int h = 0; h < kPerLane; ++h) {
+      l.pos[h] = pos_multipliers[h];
+      l.pw[h] = A(1);
+      if constexpr (WEIGHTED) l.pw[h] = to_acc(a.psw[pos_multipliers[h]]);
+    }
   };
   auto write_offsets = [&](int step, const StepLoads &l) {
 #pragma unroll
@@ -804,7 +816,8 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
       if (nb > 0) {
         const A incl = wave_inclusive_sum<A>(lane < nb ? l.wss[h] : A(0));
         lds.mult[step & 1][h * kWave + lane] =
-            lane < nb ? approx_multiplier<A>(running + incl, A(1), false, a.lr, a.eps) : A(0);
+            lane < nb ? approx_multiplier<A>(running + incl, l.pw[h], WEIGHTED, a.lr, a.eps) : A(0);
+        if constexpr (WEIGHTED) lds.pos[step & 1][h * kWave + lane] = l.pos[h];
         running = running + broadcast_lane(incl, nb - 1);
       }
     }
@@ -897,24 +910,40 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
       const int count = min(kStep, len - b * kStep);
       const T *mine = &lds.rows[b & 1][lane_off];
       const float *mult = lds.mult[b & 1];
+      const int32_t *positions = lds.pos[b & 1];
       struct Eight {
         T g[8][E];
         float m[8];
+        int32_t pos[WEIGHTED ? 8 : 1];
       };
       auto fetch = [&](int first, Eight &e) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) __builtin_memcpy(&e.g[k][0], mine + (first + k) * kRowD, sizeof(T) * E);
         __builtin_memcpy(&e.m[0], mult + first, 16);
         __builtin_memcpy(&e.m[4], mult + first + 4, 16);
+        if constexpr (WEIGHTED) {
+          __builtin_memcpy(&e.pos[0], positions + first, 16);
+          __builtin_memcpy(&e.pos[4], positions + first + 4, 16);
+        }
       };
       auto apply = [&](const Eight &e, int limit) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           if (k < limit) {
+            A dot = A(0);
 #pragma unroll
             for (int i = 0; i < E; ++i) {
-              w[i] = w[i] - to_acc(e.g[k][i]) * e.m[k];
+              const A g = to_acc(e.g[k][i]);
+              if constexpr (WEIGHTED) dot += w[i] * g;  // (the row as the occurrences so far have left it)
+              w[i] = w[i] - g * e.m[k];
               w[i] = __half2float(__float2half_rn(w[i]));
+            }
+            if constexpr (WEIGHTED) {
+              // off the chain of dependent updates, and without a trip through LDS (which would wait
+              // behind the requests for the next eight occurrences): the wavefront's sum by lane
+              // moves, one store by its last lane
+              dot = wave_sum_in_last_row(active ? dot : A(0));
+              if (lane == kWave - 1) a.grad_psw[e.pos[k]] = from_acc<T, A>(dot);
             }
           }
         }
@@ -1025,11 +1054,11 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
 
   // Rows of more than kApproxHuge occurrences get a whole workgroup where that shortens the walk:
   // with stochastic rounding (rows at most kCoopD wide, see draw_step_bits), and for fp16 rows at
-  // most kStageD wide without per-sample weights (see staged_walk).  When the grid is large
+  // most kStageD wide without it (see staged_walk).  When the grid is large
   // enough, the first workgroups do nothing else -- as many as there are such rows, rounded up
   // to a multiple of the XCD count, at most half the grid -- and the others share the remaining
   // rows as if they were the whole grid.
-  constexpr bool kStaged = !STOCHASTIC && !WEIGHTED && sizeof(T) == 2;
+  constexpr bool kStaged = !STOCHASTIC && sizeof(T) == 2;
   if constexpr (STOCHASTIC || kStaged) {
     using Shared = typename std::conditional<kStaged, StageBuffers<T>, uint16_t[2 * kCoopStep * kCoopD]>::type;
     __shared__ __align__(16) Shared s_shared;
@@ -1044,8 +1073,8 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
         for (int h = block_index; h < first_total; h += dedicated ? coop_blocks : grid_blocks) {
           const QueuedRow r = row_at(kNumXcd * queue_capacity + h);
           if constexpr (kStaged) {
-            if (r.place.row_D <= kWave) staged_walk<T, 1>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
-            else staged_walk<T, 2>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
+            if (r.place.row_D <= kWave) staged_walk<T, 1, WEIGHTED>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
+            else staged_walk<T, 2, WEIGHTED>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
           } else {
             uint16_t *s_words = s_shared;
             const int len = r.seg_end - r.seg_begin;

@@ -338,6 +338,17 @@ __device__ __forceinline__ A group_sum(A v, int chunks, int group_base) {
   }
 }
 
+// Sum over the 64 lanes of a wavefront without a trip through LDS: the rows of 16 lanes as in
+// group_sum, then the sum of row 0 into row 1 and of row 2 into row 3 (0x142 = row_bcast:15: lane
+// 15 of a row to the next row), then the sum of rows 0 and 1 into rows 2 and 3 (0x143 =
+// row_bcast:31).  The total ends up in the lanes 48..63.
+__device__ __forceinline__ float wave_sum_in_last_row(float v) {
+  v = group_sum<16, float>(v, 16, 0);
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));
+  return v;
+}
+
 // Workgroups are dealt to the 8 XCDs round-robin by blockIdx.  This maps
 // blockIdx to a logical work index so that each XCD walks one contiguous
 // eighth of the work: consecutive bags / segments (same table, neighbouring
