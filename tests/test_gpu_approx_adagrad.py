@@ -394,22 +394,13 @@ def test_approx_adagrad_stochastic_rounding_bit_for_bit_with_dyadic_gradients(or
     assert (w.view(np.uint16) != w_rn.view(np.uint16)).mean() > 0.05  # and it is not round-to-nearest
 
 
-@pytest.mark.parametrize("D,B", [(8, 900), (36, 900), (64, 900), (100, 900), (128, 900), (256, 900), (64, 64), (128, 64)])
-def test_approx_adagrad_fp16_rows_of_many_occurrences_staged_through_lds(oracle, D, B):
-    """fp16 rows of more than 256 occurrences without per-sample weights, up to 128 elements wide, are
-    walked by a workgroup whose other wavefronts stage gradient rows and multipliers in LDS, 128
-    occurrences a step (D = 100: two elements per lane, 64 occurrences a step; run lengths: one
-    past a step boundary, exactly on one, one more, many; B = 64: a grid too small to set
-    workgroups aside).  With
-    per-sample weights the same rows are walked by a single wavefront -- and weights of one
-    change no value of the update, so the two runs must agree bit for bit in rows and state.
-    Against the oracle: with gradient entries in {0, +-0.5, +-1} every sum of squares is exact
-    in fp32 whatever its order, so the state must be the oracle's bit for bit; the rows at the fp16
-    tolerance (the kernels' fused multiply-add rounds row - mult * grad once, the oracle, like the
-    reference, to fp32 and then to fp16, which now and then lands on the neighbouring value)."""
-    rs = np.random.RandomState(3 * D + B)
+def _hot_row_problem(D, B, weighted, seed):
+    """fp16 tables whose first rows occur 257 ... 2049 times (and others 17 ... 256 times), gradient
+    entries in {0, +-0.5, +-1} and per-sample weights in {0.5, 1, 2}: every sum of squares and every
+    product with a multiplier is exact in fp32 whatever its order."""
+    rs = np.random.RandomState(seed)
     T, E, L = (2 if B > 100 else 1), 60, 8
-    p = make_problem(43, T=T, E=E, D=D, B=B, L=L, dtype=np.float16, ragged=False, weighted=False)
+    p = make_problem(43, T=T, E=E, D=D, B=B, L=L, dtype=np.float16, ragged=False, weighted=weighted)
     n_t = B * L
     hot = [257, 384, 385, 1000, 2049] if B > 100 else [300]
     mid = [17, 64, 65, 200, 256] if B > 100 else [40]
@@ -418,15 +409,69 @@ def test_approx_adagrad_fp16_rows_of_many_occurrences_staged_through_lds(oracle,
         rest = rs.randint(len(hot + mid), E, size=n_t - rows.size).astype(np.int32)
         p["indices"][t * n_t:(t + 1) * n_t] = rs.permutation(np.concatenate([rows, rest]))
     p["grad_output"] = rs.choice(np.array([0, 0.5, -0.5, 1, -1], np.float16), size=p["grad_output"].shape)
-    w, st, _ = _run_gpu(p, 0.02, 0.1)
-    w_ref, st_ref, _ = _run_oracle(oracle, p, 0.02, 0.1)
+    if weighted:
+        p["per_sample_weights"] = rs.choice(np.array([0.5, 1, 2], np.float16), size=p["n"])
+    return p, T, E, L
+
+
+@pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("D,B", [(8, 900), (36, 900), (64, 900), (100, 900), (128, 900), (256, 900), (64, 64), (128, 64)])
+def test_approx_adagrad_fp16_rows_of_many_occurrences_staged_through_lds(oracle, D, B, weighted):
+    """fp16 rows of more than 256 occurrences, up to 128 elements wide, are walked by a workgroup whose
+    other wavefronts stage gradient rows and multipliers in LDS, 128 occurrences a step (D = 100, 128:
+    two elements per lane, 64 occurrences a step; D = 256: a single wavefront; run lengths: one past
+    a step boundary, exactly on one, one more, many; B = 64: a grid too small to set workgroups
+    aside).  Checked against the kernels that do not stage: the same lookups fed in fifteen calls of
+    B / 15 bags each leave every row with fewer than 257 occurrences per call, i.e. to the
+    single-wavefront walk and the short-row kernel, and with exact sums (see _hot_row_problem) the
+    fifteen calls must leave the state of the one call bit for bit, and bit for bit the rows that
+    the single-wavefront walk takes in every call (it rounds like the staged walk).  Against the oracle:
+    the state bit for bit, the rows at the fp16 tolerance (the kernels' fused multiply-add rounds
+    row - mult * grad once, the oracle, like the reference, to fp32 and then to fp16, which now
+    and then lands on the neighbouring value)."""
+    p, T, E, L = _hot_row_problem(D, B, weighted, 3 * D + B)
+    w, st, g = _run_gpu(p, 0.02, 0.1)
+    w_ref, st_ref, g_ref = _run_oracle(oracle, p, 0.02, 0.1)
     assert st.tobytes() == st_ref.tobytes()
     assert_close(w, w_ref, 1e-2)
-    ones = dict(p, per_sample_weights=np.ones(p["n"], np.float16))
-    w_one, st_one, _ = _run_gpu(ones, 0.02, 0.1)
-    assert st_one.tobytes() == st.tobytes()
-    differing = np.flatnonzero((w.view(np.uint16) != w_one.view(np.uint16)).any(axis=1))
-    assert differing.size == 0, "rows that differ between the two walks: %s" % differing[:10]
+    if weighted:
+        assert_close(g, g_ref, 2e-2, "grad of per-sample weights")
+    if B % 15 == 0:
+        calls = 15
+        per = B // calls
+        idx = p["indices"].reshape(T, B, L)
+        psw = p["per_sample_weights"].reshape(T, B, L) if weighted else None
+        w_dev = dev(p["weights"])
+        st_dev = torch.zeros(w_dev.shape[0], dtype=torch.float32, device=DEV)
+        fewest = np.full(T * E, 1 << 30)
+        most = np.zeros(T * E, int)
+        for c in range(calls):
+            sub = idx[:, c * per:(c + 1) * per, :]
+            counts = np.bincount((sub + np.arange(T)[:, None, None] * E).reshape(-1), minlength=T * E)
+            fewest, most = np.minimum(fewest, counts), np.maximum(most, counts)
+            ext.backward_approx_adagrad(
+                dev(p["grad_output"][c * per:(c + 1) * per]), w_dev, dev(p["table_offsets"]),
+                dev(np.ascontiguousarray(sub).reshape(-1)),
+                dev(np.arange(0, T * per * L + 1, L, dtype=np.int32)),
+                dev(np.ascontiguousarray(psw[:, c * per:(c + 1) * per, :]).reshape(-1)) if weighted else None,
+                st_dev, 0.02, 0.1, 200, False, 1)
+        torch.cuda.synchronize()
+        assert st_dev.cpu().numpy().tobytes() == st.tobytes()
+        # the rows that the one call stages and every one of the fifteen calls gives to the single-wavefront
+        # walk (17 to 256 occurrences per call; with fewer the short-row kernel takes them, whose separate
+        # conversion rounds twice like the oracle's)
+        total = np.bincount((idx + np.arange(T)[:, None, None] * E).reshape(-1), minlength=T * E)
+        walked = np.flatnonzero((total > 256) & (fewest >= 17) & (most <= 256))
+        assert walked.size >= 2 * T
+        assert (w.view(np.uint16)[walked] == w_dev.cpu().numpy().view(np.uint16)[walked]).all(), \
+            "staged rows that differ from the single-wavefront walk's"
+        assert_close(w, w_dev.cpu().numpy(), 1e-2)
+    if not weighted:
+        # per-sample weights of one change no value of the update
+        ones = dict(p, per_sample_weights=np.ones(p["n"], np.float16))
+        w_one, st_one, _ = _run_gpu(ones, 0.02, 0.1)
+        assert st_one.tobytes() == st.tobytes()
+        assert (w.view(np.uint16) == w_one.view(np.uint16)).all()
 
 
 def test_approx_adagrad_stochastic_rounding_more_long_rows_than_workgroups_set_aside(oracle):
