@@ -633,11 +633,11 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
         round_lane_elements<T, E, false, A>(w, a.sr, place.row_element + lane_off);
       }
       if constexpr (WEIGHTED) {
-        dot = active ? dot : A(0);
-#pragma unroll
-        for (int m = kWave / 2; m > 0; m >>= 1) dot += shfl_x(dot, m);
+        // (the wavefront's sum by lane moves: lane shuffles go through LDS and would wait one round
+        // trip each, per occurrence)
+        dot = wave_sum_in_last_row<A>(active ? dot : A(0));
         const int pos = broadcast_lane(cur_pos, j);
-        if (lane == 0) a.grad_psw[pos] = from_acc<T, A>(dot);
+        if (lane == kWave - 1) a.grad_psw[pos] = from_acc<T, A>(dot);
       }
     };
 
@@ -749,23 +749,28 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
 // there) and the second wavefront keeps the row's running state (the prefix sums over batches of
 // 64 occurrences of walk_long_row: the same additions in the same order), forms the multipliers
 // and looks up where the gradient rows are.  One barrier per step.  With per-sample weights the
-// walking wavefront also forms <row, gradient row> of every occurrence (a sum over the wavefront by
-// lane moves, off the chain of dependent updates but in its instruction stream: 75 ns per occurrence
-// instead of 7).
+// walking wavefront also starts <row, gradient row> of every occurrence -- the products summed over
+// quads of lanes, off the chain of dependent updates -- and leaves the sixteen partial sums in LDS;
+// a gathering thread per occurrence finishes them during the next step.
 // Rows of up to 64 elements: one element per lane, 128 occurrences a step; rows of up to 128
 // elements: two elements per lane, 64 occurrences a step (the same 16 KB of gradient rows).
 constexpr int kStageStep = 128;  // most occurrences per step
 constexpr int kStageD = 128;     // widest row walked this way
 constexpr int kStageElements = 128 * 64;  // elements of the gradient rows of one step
-template <typename T> struct StageBuffers {
+template <typename T, bool WEIGHTED> struct StageBuffers {
   alignas(16) T rows[2][kStageElements];  // [occurrence of the step][element of the row]
   alignas(16) float mult[2][kStageStep];
-  alignas(16) int32_t pos[2][kStageStep];  // (per-sample weights) position of every occurrence: where its grad_psw goes
+  // (per-sample weights) position of every occurrence -- where its grad_psw goes -- and the sixteen
+  // sums over four lanes each of <row, gradient row>, left by the walk for the gathering wavefronts
+  // ([occurrence][quad of lanes]: a thread reads its occurrence's sixteen sums as four 16-byte
+  // pieces; measured faster than the transposed, padded layout whose reads are free of bank conflicts)
+  alignas(16) int32_t pos[3][WEIGHTED ? kStageStep : 1];
+  alignas(16) float partial[2][WEIGHTED ? kStageStep : 1][16];
   int64_t goff[4][kStageStep];  // first element of every occurrence's gradient row
 };
 template <typename T, int E, bool WEIGHTED>
 __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_begin, int seg_end, int64_t key,
-                                            const RowPlace &place, T *storage, StageBuffers<T> &lds) {
+                                            const RowPlace &place, T *storage, StageBuffers<T, WEIGHTED> &lds) {
   using A = typename AccOf<T>::type;
   static_assert(sizeof(T) == 2 && sizeof(A) == 4, "fp16 rows with fp32 arithmetic");
   const int lane = threadIdx.x & (kWave - 1);
@@ -817,7 +822,7 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
         const A incl = wave_inclusive_sum<A>(lane < nb ? l.wss[h] : A(0));
         lds.mult[step & 1][h * kWave + lane] =
             lane < nb ? approx_multiplier<A>(running + incl, l.pw[h], WEIGHTED, a.lr, a.eps) : A(0);
-        if constexpr (WEIGHTED) lds.pos[step & 1][h * kWave + lane] = l.pos[h];
+        if constexpr (WEIGHTED) lds.pos[step % 3][h * kWave + lane] = l.pos[h];
         running = running + broadcast_lane(incl, nb - 1);
       }
     }
@@ -852,6 +857,20 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
     for (int k = 0; k < kRounds; ++k) {
       const int o = o0 + k * rows_per_round;
       if (o < count) *reinterpret_cast<uint2 *>(&lds.rows[step & 1][o * kRowD + piece * 4]) = held[k];
+    }
+  };
+
+  // (per-sample weights) grad_psw of a walked step: a gathering thread per occurrence adds the sixteen
+  // partial sums in order
+  auto finish_dots = [&](int step) {
+    if constexpr (WEIGHTED) {
+      const int count = min(kStep, len - step * kStep);
+      if (helper < count) {
+        A dot = A(0);
+#pragma unroll
+        for (int q = 0; q < 16; ++q) dot += lds.partial[step & 1][helper][q];
+        a.grad_psw[lds.pos[step % 3][helper]] = from_acc<T, A>(dot);
+      }
     }
   };
 
@@ -910,23 +929,18 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
       const int count = min(kStep, len - b * kStep);
       const T *mine = &lds.rows[b & 1][lane_off];
       const float *mult = lds.mult[b & 1];
-      const int32_t *positions = lds.pos[b & 1];
+      float *my_partial = &lds.partial[b & 1][0][WEIGHTED ? lane >> 2 : 0];
       struct Eight {
         T g[8][E];
         float m[8];
-        int32_t pos[WEIGHTED ? 8 : 1];
       };
       auto fetch = [&](int first, Eight &e) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) __builtin_memcpy(&e.g[k][0], mine + (first + k) * kRowD, sizeof(T) * E);
         __builtin_memcpy(&e.m[0], mult + first, 16);
         __builtin_memcpy(&e.m[4], mult + first + 4, 16);
-        if constexpr (WEIGHTED) {
-          __builtin_memcpy(&e.pos[0], positions + first, 16);
-          __builtin_memcpy(&e.pos[4], positions + first + 4, 16);
-        }
       };
-      auto apply = [&](const Eight &e, int limit) {
+      auto apply = [&](const Eight &e, int first, int limit) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           if (k < limit) {
@@ -939,11 +953,13 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
               w[i] = __half2float(__float2half_rn(w[i]));
             }
             if constexpr (WEIGHTED) {
-              // off the chain of dependent updates, and without a trip through LDS (which would wait
-              // behind the requests for the next eight occurrences): the wavefront's sum by lane
-              // moves, one store by its last lane
-              dot = wave_sum_in_last_row(active ? dot : A(0));
-              if (lane == kWave - 1) a.grad_psw[e.pos[k]] = from_acc<T, A>(dot);
+              // off the chain of dependent updates: the sum over the lane's quad by two lane moves,
+              // left in LDS for a gathering thread to finish (the four lanes hold the same sum and
+              // all write it: cheaper than masking three of them off)
+              dot = active ? dot : A(0);
+              dot += dpp_move<0xB1>(dot);
+              dot += dpp_move<0x4E>(dot);
+              my_partial[(first + k) * 16] = dot;
             }
           }
         }
@@ -955,14 +971,14 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
         for (int first = 0; first < kStep; first += 16) {
           fetch(first + 8, odd);
           __builtin_amdgcn_sched_barrier(0);
-          apply(even, 8);
+          apply(even, first, 8);
           if (first + 16 < kStep) fetch(first + 16, even);
           __builtin_amdgcn_sched_barrier(0);
-          apply(odd, 8);
+          apply(odd, first + 8, 8);
         }
       } else {
         for (int first = 0; first < count; first += 8) {
-          apply(even, count - first);
+          apply(even, first, count - first);
           if (first + 8 < count) fetch(first + 8, even);
         }
       }
@@ -970,6 +986,7 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
       if (wave >= 2) {
         if (b + 1 < steps) store_rows(b + 1, held);
         request_rows(b + 3, held);
+        if (b > 0) finish_dots(b - 1);
       } else {
         StepLoads requested{};
         request_bookkeeping(pos6, pos3, requested);  // (clamped positions: always valid)
@@ -994,6 +1011,7 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
     step_of_walk(b, held_odd);
     if (b + 1 < steps) step_of_walk(b + 1, held_even);
   }
+  if (wave >= 2) finish_dots(steps - 1);  // (the last step's barrier is behind every wavefront)
   if (wave == 0 && active) {  // (already rounded: exact)
 #pragma unroll
     for (int i = 0; i < E; ++i) storage[lane_off + i] = from_acc<T, A>(w[i]);
@@ -1060,7 +1078,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
   // rows as if they were the whole grid.
   constexpr bool kStaged = !STOCHASTIC && sizeof(T) == 2;
   if constexpr (STOCHASTIC || kStaged) {
-    using Shared = typename std::conditional<kStaged, StageBuffers<T>, uint16_t[2 * kCoopStep * kCoopD]>::type;
+    using Shared = typename std::conditional<kStaged, StageBuffers<T, WEIGHTED>, uint16_t[2 * kCoopStep * kCoopD]>::type;
     __shared__ __align__(16) Shared s_shared;
     if (queue_capacity > 0 && a.mt.T == 0 && D <= (kStaged ? kStageD : kCoopD) && first_total > 0) {
       const bool dedicated = grid_blocks >= 2 * kNumXcd;

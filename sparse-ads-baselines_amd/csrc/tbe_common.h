@@ -342,10 +342,19 @@ __device__ __forceinline__ A group_sum(A v, int chunks, int group_base) {
 // group_sum, then the sum of row 0 into row 1 and of row 2 into row 3 (0x142 = row_bcast:15: lane
 // 15 of a row to the next row), then the sum of rows 0 and 1 into rows 2 and 3 (0x143 =
 // row_bcast:31).  The total ends up in the lanes 48..63.
-__device__ __forceinline__ float wave_sum_in_last_row(float v) {
-  v = group_sum<16, float>(v, 16, 0);
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_rows(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ double dpp_rows(double v) {
+  const long long bits = __builtin_bit_cast(long long, v);
+  const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(bits), CTRL, ROW_MASK, 0xF, false);
+  const int hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(bits >> 32), CTRL, ROW_MASK, 0xF, false);
+  return __builtin_bit_cast(double, (static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo));
+}
+template <typename A> __device__ __forceinline__ A wave_sum_in_last_row(A v) {
+  v = group_sum<16, A>(v, 16, 0);
+  v += dpp_rows<0x142, 0xA>(v);  // (rows 1 and 3 take the row before them; the others add zero)
+  v += dpp_rows<0x143, 0xC>(v);  // (rows 2 and 3 take row 1)
   return v;
 }
 
