@@ -445,6 +445,16 @@ typedef struct tbe_cache {
   int32_t *stage_keys;    /* [3 * stage_slots] key held by each staging row, -1 = none, -(key + 2) = taken
                            * over by a later step                                                       */
   int64_t total_rows;     /* rows of the backing table                                                 */
+  /* tables of different row widths (all null / 0: every row has the D elements passed to the calls).
+   * backing_rows is then the 1-D weights of tbe_forward_mixed, a row's key its global row id
+   * (mixed_table_rows[t] + index), a row of `rows` has the widest table's D_t elements -- the D passed
+   * to the calls below -- of which a narrower row uses the first D_t, and `workspace` follows
+   * tbe_backward_mixed_workspace_layout.  Forward and update: tbe_forward_mixed_cached,
+   * tbe_backward_mixed_cached. */
+  const int64_t *mixed_table_offsets;  /* [T + 1] first element of each table in backing_rows             */
+  const int32_t *mixed_table_rows;     /* [T + 1] first global row id of each table (`table_dim_offsets`) */
+  const int32_t *mixed_dim_offsets;    /* [T + 1] first output column of each table                       */
+  int32_t mixed_T;
 } tbe_cache_t;
 
 /* Byte offsets into the cache workspace (separate from the backward workspace). */
@@ -550,6 +560,28 @@ TBE_API int tbe_backward_approx_cached(const void *grad_output, const tbe_cache_
                                        int32_t stochastic_rounding, uint64_t seed, uint64_t offset,
                                        void *workspace, uint64_t workspace_bytes,
                                        const int32_t *unique_slots, void *stream);
+
+/* tbe_forward_mixed and tbe_backward_mixed (every optimizer of it) for tables of different widths
+ * behind the row cache: `cache` carries the tables (mixed_* fields), D is the width of a cache row
+ * (the widest table's), the other arguments are those of the uncached entry points; `offsets` are the
+ * batch's bag offsets [T*B + 1] again, read by TBE_OPT_APPROX_ROWWISE_ADAGRAD only (null otherwise).  The plan comes from tbe_cache_prepare / tbe_cache_plan + tbe_cache_commit called with
+ * table_offsets = mixed_table_rows, T = mixed_T and a workspace laid out by
+ * tbe_backward_mixed_workspace_layout.  Same results, bit for bit, as the uncached entry points on the
+ * backing table (stochastic rounding included: a weight's random word goes by its place in the table).
+ * The reference has no counterpart (its mixed-D tables are device or managed memory,
+ * table_batched_embeddings_ops.py:324-379). */
+TBE_API int tbe_forward_mixed_cached(const tbe_cache_t *cache, int32_t dtype, int32_t fp16_vector_width, int32_t D,
+                                     int32_t total_D, const int32_t *indices, int64_t num_indices,
+                                     const int32_t *offsets, int32_t B, const void *per_sample_weights,
+                                     const int32_t *lookup_slots, void *output, void *stream);
+TBE_API int tbe_backward_mixed_cached(int32_t optimizer, const void *grad_output, const tbe_cache_t *cache,
+                                      int32_t dtype, int32_t fp16_vector_width, int32_t D, int32_t total_D,
+                                      int32_t B, int64_t num_indices, const int32_t *offsets,
+                                      const void *per_sample_weights,
+                                      void *optimizer_state, float learning_rate, float eps,
+                                      void *grad_per_sample_weights, int32_t stochastic_rounding, uint64_t seed,
+                                      uint64_t offset, void *workspace, uint64_t workspace_bytes,
+                                      const int32_t *unique_slots, void *stream);
 
 /* Writes every resident row, and every row waiting in a staging area, back to the backing table (the
  * cache stays valid).  `stream` must be ordered behind the streams of earlier tbe_cache_plan calls, and a

@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kBlockThreads) void construct_offsets_kernel(
 
 extern "C" const char *tbe_last_error(void) { return tbe::g_last_error; }
 
-extern "C" int32_t tbe_abi_version(void) { return 21; }
+extern "C" int32_t tbe_abi_version(void) { return 22; }
 
 extern "C" int tbe_profile_begin(void) {
   using namespace tbe;

@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
     const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ segment_starts,
     int32_t *__restrict__ counters, int32_t *__restrict__ long_queue, int D, int group, float lr,
     float eps, MixedTables mt, StochasticRounding sr, const int32_t *__restrict__ only_rows,
-    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows) {
+    const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, int slot_D) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -171,12 +171,12 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_kernel(
       seg_end = seg_begin;  // nothing to do here
     }
     const bool handled_here = seg_end > seg_begin;
-    // (cache-fronted uniform tables: the row lives in its cache slot when it has one; its random
-    // words still go by its place in the table)
+    // (cache-fronted tables: the row lives in its cache slot, slot_D elements wide, when it has one;
+    // its random words still go by its place in the table)
     T *wrow = weights + row_element;
     if (unique_slots) {
       const int slot = unique_slots[u];
-      if (slot >= 0) wrow = cache_rows + static_cast<int64_t>(slot) * D;
+      if (slot >= 0) wrow = cache_rows + static_cast<int64_t>(slot) * slot_D;
     }
     A s = state_in;
     V w;
@@ -456,8 +456,9 @@ template <typename T> struct LongRowArgs {
   MixedTables mt;  // (T == 0: uniform tables)
   StochasticRounding sr;
   uint64_t grad_bytes;  // size of grad_output
-  const int32_t *unique_slots;  // cache-fronted uniform tables: slot of each unique row (-1: not resident), or null
+  const int32_t *unique_slots;  // cache-fronted tables: slot of each unique row (-1: not resident), or null
   T *cache_rows;
+  int slot_D;  // elements of a cache row
 };
 
 // First element of gradient row `grad_row` for a row at `p` (mixed-D tables: mt.T > 0).
@@ -1062,7 +1063,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     r.storage = a.weights + r.place.row_element;
     if (a.unique_slots) {
       const int slot = uniform(a.unique_slots[u]);
-      if (slot >= 0) r.storage = a.cache_rows + static_cast<int64_t>(slot) * D;
+      if (slot >= 0) r.storage = a.cache_rows + static_cast<int64_t>(slot) * a.slot_D;
     }
     return r;
   };
@@ -1194,9 +1195,10 @@ struct ApproxArgs {
   // mixed-D tables: the rows of at most 64 vectors and kMixedShort occurrences are done and the
   // longer ones queued (update_mixed_approx_short); this queue holds the rows wider than 64 vectors
   const int32_t *wide_rows;
-  // cache-fronted uniform tables: slot of each unique row and the cache's rows (null otherwise)
+  // cache-fronted tables: slot of each unique row, the cache's rows (null otherwise) and their width
   const int32_t *unique_slots;
   void *cache_rows;
+  int32_t slot_D;
 };
 
 template <typename T, int VEC>
@@ -1239,7 +1241,7 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
   LongRowArgs<T> la{static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights), static_cast<A *>(a.state),
                     static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw), i32(l.positions_sorted),
                     i32(l.grad_rows), lookup_wss, a.lr, a.eps, long_tables, a.sr, grad_bytes, a.unique_slots,
-                    static_cast<T *>(a.cache_rows)};
+                    static_cast<T *>(a.cache_rows), a.slot_D};
   const bool big = grad_bytes >= (1ull << 32);
   const bool stochastic = sizeof(T) == 2 && a.sr.enabled;
 #define TBE_APPROX_LONG_KERNEL(WEIGHTED, STOCHASTIC, BIG)                                              \
@@ -1263,7 +1265,7 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
              static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),   \
              i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),     \
              counters, long_queue, a.D, group, a.lr, a.eps, a.mt, a.sr, a.wide_rows, a.unique_slots,   \
-             static_cast<T *>(a.cache_rows));                                                          \
+             static_cast<T *>(a.cache_rows), a.slot_D);                                                \
   TBE_APPROX_LONG(WEIGHTED, MIXED)
   if (mixed) {
     if (a.psw) { TBE_APPROX(true, true); }
@@ -1329,10 +1331,11 @@ int approx_update(const void *grad_output, void *weights, void *state, const voi
                   const int64_t *mixed_table_offsets, const int32_t *table_dim_offsets,
                   const int32_t *dim_offsets, int32_t total_D, int32_t T, const int32_t *offsets, int32_t B,
                   StochasticRounding sr, const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream,
-                  const int32_t *unique_slots, void *cache_rows) {
+                  const int32_t *unique_slots, void *cache_rows, int32_t slot_D) {
   ApproxArgs a{grad_output, weights, state, psw, grad_psw, dtype, fp16_vector_width, D, n, lr, eps,
                MixedTables{mixed_table_offsets, table_dim_offsets, dim_offsets, total_D, T}, sr, offsets, B, T,
-               D == 0 ? approx_mixed_wide_queue(l, workspace) : nullptr, unique_slots, cache_rows};
+               D == 0 ? approx_mixed_wide_queue(l, workspace) : nullptr, unique_slots, cache_rows,
+               D == 0 ? slot_D : D};
   char *ws = static_cast<char *>(workspace);
   // the queues of long rows borrow the chunk records' region: eight of approx_long_queue_capacity()
   // rows and one of the rows of more than kApproxHuge occurrences, or one queue of at most n / 9 rows

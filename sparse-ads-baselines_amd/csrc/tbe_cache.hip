@@ -368,11 +368,41 @@ __global__ __launch_bounds__(kBlockThreads) void cache_retire_stage_kernel(
   if (stats && (threadIdx.x & (kWave - 1)) == 0 && pending) atomicAdd(&stats[kStatWrittenOut], pending);
 }
 
-// One wavefront per row; rows move as 8-byte units (row_units = D * element size / 8).
+// Rows move as 8-byte units.  A row of the cache (slot, staging or landing row) has row_units of
+// them: D * element size / 8, D the widest table's with tables of different widths.  Where a row
+// of the backing table lies, and how many units it has: row `key` at key * row_units with uniform
+// tables; else the table is found by bisecting the tables' first row ids.
+struct BackingMap {
+  uint64_t *rows;
+  int row_units;
+  const int64_t *table_offsets;  // tables of different widths (null otherwise): first element of each table,
+  const int32_t *table_rows;     // first row id of each table, [T + 1],
+  const int32_t *dim_offsets;    // first output column of each table, [T + 1]
+  int T;
+  int unit_shift;                // log2 of the elements per unit
+};
+struct BackingRow {
+  uint64_t *row;
+  int units;
+};
+__device__ __forceinline__ BackingRow backing_row(const BackingMap &m, int64_t key) {
+  if (!m.table_offsets) return BackingRow{m.rows + key * m.row_units, m.row_units};
+  int lo = 0, hi = m.T;  // table_rows[lo] <= key < table_rows[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (m.table_rows[mid] <= key) lo = mid;
+    else hi = mid;
+  }
+  const int64_t D = m.dim_offsets[lo + 1] - m.dim_offsets[lo];
+  const int64_t element = m.table_offsets[lo] + (key - m.table_rows[lo]) * D;
+  return BackingRow{m.rows + (element >> m.unit_shift), static_cast<int>(D >> m.unit_shift)};
+}
+
+// One wavefront per row.
 // Without deferred write-back: the evicted row goes to the backing table, the new row comes into
 // the slot or the staging row.
 __global__ __launch_bounds__(kBlockThreads) void cache_fill_kernel(
-    uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    uint64_t *__restrict__ cache_rows, BackingMap backing,
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
     const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
     const int32_t *__restrict__ evicted_keys) {
@@ -384,13 +414,13 @@ __global__ __launch_bounds__(kBlockThreads) void cache_fill_kernel(
     const int32_t evicted = evicted_keys[i];
     if (evicted == -2) continue;
     const int64_t key = keys_sorted[segment_starts[i]];
-    uint64_t *slot_row = cache_rows + static_cast<int64_t>(unique_slots[i]) * row_units;
-    const uint64_t *new_row = backing_rows + key * row_units;
+    uint64_t *slot_row = cache_rows + static_cast<int64_t>(unique_slots[i]) * backing.row_units;
+    const BackingRow fresh = backing_row(backing, key);
     if (evicted >= 0) {
-      uint64_t *old_row = backing_rows + static_cast<int64_t>(evicted) * row_units;
-      for (int k = lane; k < row_units; k += kWave) old_row[k] = slot_row[k];
+      const BackingRow old = backing_row(backing, evicted);
+      for (int k = lane; k < old.units; k += kWave) old.row[k] = slot_row[k];
     }
-    for (int k = lane; k < row_units; k += kWave) slot_row[k] = new_row[k];
+    for (int k = lane; k < fresh.units; k += kWave) slot_row[k] = fresh.row[k];
   }
 }
 
@@ -407,7 +437,7 @@ __global__ __launch_bounds__(kBlockThreads) void cache_fill_kernel(
 // Nothing here touches a slot or a row that the step before may still read or update.
 constexpr int kFillBatch = 4;
 __global__ __launch_bounds__(kBlockThreads) void cache_fill_deferred_kernel(
-    uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    uint64_t *__restrict__ cache_rows, BackingMap backing,
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
     const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
     const int32_t *__restrict__ evicted_keys, const int32_t *__restrict__ landing,
@@ -417,18 +447,22 @@ __global__ __launch_bounds__(kBlockThreads) void cache_fill_deferred_kernel(
   const int U = counters[0];
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
+  const int row_units = backing.row_units;
   const int64_t items = U > stage_slots ? U : stage_slots;
   for (int64_t i0 = wave_id * kFillBatch; i0 < items; i0 += stride * kFillBatch) {
     // lanes 0 .. kFillBatch-1: a row of the released area each; the next kFillBatch lanes: a unique row each
     const uint64_t *my_src = cache_rows;  // a harmless source for the lanes without a row to move
     uint64_t *my_dst = nullptr;
+    int my_units = 0;
     if (lane < kFillBatch) {
       const int64_t i = i0 + lane;
       if (i < stage_slots) {
         const int64_t key = write_out[i];
         if (key >= 0) {
+          const BackingRow home = backing_row(backing, key);
           my_src = cache_rows + (old_stage_base + i) * row_units;
-          my_dst = backing_rows + key * row_units;
+          my_dst = home.row;
+          my_units = home.units;
         }
       }
     } else if (lane < 2 * kFillBatch) {
@@ -438,30 +472,37 @@ __global__ __launch_bounds__(kBlockThreads) void cache_fill_deferred_kernel(
         const int64_t land = slot >= num_slots ? slot : landing[i];
         const int64_t source = fetch_source[i];
         if (land >= 0) {
+          const BackingRow home = backing_row(backing, keys_sorted[segment_starts[i]]);
           if (source == -1) {
-            my_src = backing_rows + static_cast<int64_t>(keys_sorted[segment_starts[i]]) * row_units;
+            my_src = home.row;
             my_dst = cache_rows + land * row_units;
+            my_units = home.units;
           } else if (source >= old_stage_base && source < old_stage_base + stage_slots) {
             my_src = cache_rows + source * row_units;
             my_dst = cache_rows + land * row_units;
+            my_units = home.units;
           }  // else: the commit launch fetches it
         }
       }
     }
     const uint64_t *src[2 * kFillBatch];
     uint64_t *dst[2 * kFillBatch];
+    int units[2 * kFillBatch];  // (0 for a lane without a row to move)
+    int most = 0;
 #pragma unroll
     for (int j = 0; j < 2 * kFillBatch; ++j) {
       src[j] = reinterpret_cast<const uint64_t *>(__shfl(reinterpret_cast<unsigned long long>(my_src), j, kWave));
       dst[j] = reinterpret_cast<uint64_t *>(__shfl(reinterpret_cast<unsigned long long>(my_dst), j, kWave));
+      units[j] = __shfl(my_units, j, kWave);
+      most = max(most, units[j]);
     }
-    for (int k = lane; k < row_units; k += kWave) {
+    for (int k = lane; k < most; k += kWave) {
       uint64_t v[2 * kFillBatch];
 #pragma unroll
-      for (int j = 0; j < 2 * kFillBatch; ++j) v[j] = src[j][k];
+      for (int j = 0; j < 2 * kFillBatch; ++j) v[j] = k < units[j] ? src[j][k] : 0;
 #pragma unroll
       for (int j = 0; j < 2 * kFillBatch; ++j)
-        if (dst[j]) dst[j][k] = v[j];
+        if (k < units[j]) dst[j][k] = v[j];
     }
   }
 }
@@ -472,7 +513,7 @@ __global__ __launch_bounds__(kBlockThreads) void cache_fill_deferred_kernel(
 // row, or, without one, straight to the backing table), and the newest value of a row that this
 // step leaves in the backing table, if the last step's staging area still held it.
 __global__ __launch_bounds__(kBlockThreads) void cache_commit_kernel(
-    uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    uint64_t *__restrict__ cache_rows, BackingMap backing,
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
     const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
     const int32_t *__restrict__ evicted_keys, const int32_t *__restrict__ landing,
@@ -485,22 +526,23 @@ __global__ __launch_bounds__(kBlockThreads) void cache_commit_kernel(
     const int32_t evicted = evicted_keys[i];
     const int64_t slot = unique_slots[i];
     if (evicted == -2 && slot >= 0) continue;  // a hit
+    const int row_units = backing.row_units;
     const int64_t source = fetch_source[i];
     const int64_t key = keys_sorted[segment_starts[i]];
+    const BackingRow home = backing_row(backing, key);
     if (evicted == -2) {
       if (source >= 0) {
         const uint64_t *src = cache_rows + source * row_units;
-        uint64_t *dst = backing_rows + key * row_units;
-        for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
+        for (int k = lane; k < home.units; k += kWave) home.row[k] = src[k];
       }
       continue;
     }
     const bool by_fill = source == -1 || (source >= old_stage_base && source < old_stage_base + stage_slots);
-    const uint64_t *late_src = source >= 0 ? cache_rows + source * row_units : backing_rows + key * row_units;
+    const uint64_t *late_src = source >= 0 ? cache_rows + source * row_units : home.row;
     if (slot >= num_slots) {
       if (!by_fill) {
         uint64_t *dst = cache_rows + slot * row_units;
-        for (int k = lane; k < row_units; k += kWave) dst[k] = late_src[k];
+        for (int k = lane; k < home.units; k += kWave) dst[k] = late_src[k];
       }
       continue;
     }
@@ -508,16 +550,17 @@ __global__ __launch_bounds__(kBlockThreads) void cache_commit_kernel(
     uint64_t *slot_row = cache_rows + slot * row_units;
     const uint64_t *new_row = (by_fill && land >= 0) ? cache_rows + land * row_units : late_src;
     if (evicted >= 0) {
-      uint64_t *old_row = land >= 0 ? cache_rows + land * row_units
-                                    : backing_rows + static_cast<int64_t>(evicted) * row_units;
-      for (int k = lane; k < row_units; k += kWave) {
-        const uint64_t fresh = new_row[k];
+      // (the evicted row may belong to a table of another width than the row that replaces it)
+      const BackingRow old_home = backing_row(backing, evicted);
+      uint64_t *old_row = land >= 0 ? cache_rows + land * row_units : old_home.row;
+      for (int k = lane; k < max(home.units, old_home.units); k += kWave) {
+        const uint64_t fresh = k < home.units ? new_row[k] : 0;
         const uint64_t old = slot_row[k];
-        old_row[k] = old;
-        slot_row[k] = fresh;
+        if (k < old_home.units) old_row[k] = old;
+        if (k < home.units) slot_row[k] = fresh;
       }
     } else {
-      for (int k = lane; k < row_units; k += kWave) slot_row[k] = new_row[k];
+      for (int k = lane; k < home.units; k += kWave) slot_row[k] = new_row[k];
     }
   }
 }
@@ -526,7 +569,7 @@ __global__ __launch_bounds__(kBlockThreads) void cache_commit_kernel(
 // to the backing table.  A wavefront reads 64 entries at a time and copies the rows of those that
 // hold one, so an empty area costs one pass over its entries.
 __global__ __launch_bounds__(kBlockThreads) void cache_unstage_area_kernel(
-    const uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    const uint64_t *__restrict__ cache_rows, BackingMap backing,
     const int32_t *__restrict__ stage_keys, int64_t stage_base, int64_t stage_slots) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
@@ -538,16 +581,16 @@ __global__ __launch_bounds__(kBlockThreads) void cache_unstage_area_kernel(
       const int j = __ffsll(static_cast<long long>(held)) - 1;
       held &= held - 1;
       const int64_t key = __shfl(my_key, j, kWave);
-      const uint64_t *src = cache_rows + (stage_base + i0 + j) * row_units;
-      uint64_t *dst = backing_rows + key * row_units;
-      for (int k = lane; k < row_units; k += kWave) dst[k] = src[k];
+      const uint64_t *src = cache_rows + (stage_base + i0 + j) * backing.row_units;
+      const BackingRow home = backing_row(backing, key);
+      for (int k = lane; k < home.units; k += kWave) home.row[k] = src[k];
     }
   }
 }
 
 // After the update: staged rows (slot >= first_stage_slot) go back to the backing table.
 __global__ __launch_bounds__(kBlockThreads) void cache_unstage_kernel(
-    const uint64_t *__restrict__ cache_rows, uint64_t *__restrict__ backing_rows, int row_units,
+    const uint64_t *__restrict__ cache_rows, BackingMap backing,
     const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
     const int32_t *__restrict__ counters, const int32_t *__restrict__ unique_slots,
     int64_t first_stage_slot) {
@@ -559,9 +602,9 @@ __global__ __launch_bounds__(kBlockThreads) void cache_unstage_kernel(
     const int64_t slot = unique_slots[u];
     if (slot < first_stage_slot) continue;
     const int64_t key = keys_sorted[segment_starts[u]];
-    const uint64_t *src = cache_rows + slot * row_units;
-    uint64_t *dst = backing_rows + key * row_units;
-    for (int i = lane; i < row_units; i += kWave) dst[i] = src[i];
+    const uint64_t *src = cache_rows + slot * backing.row_units;
+    const BackingRow home = backing_row(backing, key);
+    for (int i = lane; i < home.units; i += kWave) home.row[i] = src[i];
   }
 }
 
@@ -574,17 +617,17 @@ __global__ __launch_bounds__(kBlockThreads) void cache_locate_kernel(
 }
 
 __global__ __launch_bounds__(kBlockThreads) void cache_flush_kernel(
-    const int32_t *__restrict__ tags, const uint64_t *__restrict__ cache_rows,
-    uint64_t *__restrict__ backing_rows, int row_units, int64_t num_slots) {
+    const int32_t *__restrict__ tags, const uint64_t *__restrict__ cache_rows, BackingMap backing,
+    int64_t num_slots) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
   for (int64_t slot = wave_id; slot < num_slots; slot += stride) {
     const int64_t key = tags[slot];
     if (key < 0) continue;
-    const uint64_t *src = cache_rows + slot * row_units;
-    uint64_t *dst = backing_rows + key * row_units;
-    for (int i = lane; i < row_units; i += kWave) dst[i] = src[i];
+    const uint64_t *src = cache_rows + slot * backing.row_units;
+    const BackingRow home = backing_row(backing, key);
+    for (int i = lane; i < home.units; i += kWave) home.row[i] = src[i];
   }
 }
 
@@ -613,6 +656,19 @@ inline unsigned grid_for(int64_t work_items, int64_t per_block, int64_t cap) {
 }
 
 inline bool deferred(const tbe_cache_t *cache) { return cache->stage_of_row != nullptr && cache->stage_slots > 0; }
+inline bool mixed_tables(const tbe_cache_t *cache) { return cache->mixed_table_offsets != nullptr; }
+
+// D: elements of a cache row (with tables of different widths: of the widest table's rows)
+BackingMap backing_map(const tbe_cache_t *cache, int32_t D, int32_t dtype) {
+  const int element = static_cast<int>(dtype_size(dtype));
+  return BackingMap{static_cast<uint64_t *>(cache->backing_rows),
+                    static_cast<int>(static_cast<int64_t>(D) * element / 8),
+                    cache->mixed_table_offsets,
+                    cache->mixed_table_rows,
+                    cache->mixed_dim_offsets,
+                    cache->mixed_T,
+                    element == 2 ? 2 : element == 4 ? 1 : 0};
+}
 
 int validate_cache(const char *name, const tbe_cache_t *cache) {
   TBE_REQUIRE(cache, "%s: null cache", name);
@@ -629,19 +685,23 @@ int validate_cache(const char *name, const tbe_cache_t *cache) {
     TBE_REQUIRE(cache->num_sets * kWays + kAreas * cache->stage_slots < INT32_MAX, "%s: stage_slots out of range",
                 name);
   }
+  if (cache->mixed_table_offsets || cache->mixed_table_rows || cache->mixed_dim_offsets || cache->mixed_T) {
+    TBE_REQUIRE(cache->mixed_table_offsets && cache->mixed_table_rows && cache->mixed_dim_offsets && cache->mixed_T > 0,
+                "%s: tables of different widths need mixed_table_offsets, mixed_table_rows, mixed_dim_offsets and mixed_T",
+                name);
+  }
   return TBE_OK;
 }
 
 // Deferred write-back, outside a step: the rows of staging area `area` that still wait for their
 // write-back go to the backing table, and the area is released -- unless a planned batch still
 // works on it (`keep`): then its rows stay listed, since that batch's update changes them again.
-void write_back_stage(const tbe_cache_t *cache, int row_units, int64_t area, bool keep, hipStream_t stream) {
+void write_back_stage(const tbe_cache_t *cache, const BackingMap &backing, int64_t area, bool keep, hipStream_t stream) {
   const int64_t base = cache->num_sets * kWays + area * cache->stage_slots;
   int32_t *keys = cache->stage_keys + area * cache->stage_slots;
   TBE_LAUNCH("cache_unstage", stream, cache_unstage_area_kernel,
              dim3(grid_for(cache->stage_slots, kWavesPerBlock, 256 * 16)), dim3(kBlockThreads),
-             static_cast<const uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units, keys,
-             base, cache->stage_slots);
+             static_cast<const uint64_t *>(cache->rows), backing, keys, base, cache->stage_slots);
   if (keep) return;
   TBE_LAUNCH("cache_retire_stage", stream, cache_retire_stage_kernel,
              dim3(grid_for(cache->stage_slots, kBlockThreads, 1024)), dim3(kBlockThreads), cache->stage_of_row, keys,
@@ -697,7 +757,9 @@ int validate_plan(const char *name, const PlanArgs &a, tbe_workspace_layout_t *l
   TBE_REQUIRE(a.step > 0, "%s: steps are numbered from 1 (got %d)", name, a.step);
   TBE_REQUIRE(a.sequence >= 0 && a.sequence < INT32_MAX - 4, "%s: sequence out of range (got %d)", name, a.sequence);
   TBE_REQUIRE(a.table_offsets && a.offsets && (a.indices || a.num_indices == 0), "%s: null pointer argument", name);
-  backward_layout(a.num_indices, a.D, a.dtype, a.T, l);
+  TBE_REQUIRE(!mixed_tables(a.cache) || a.T == a.cache->mixed_T, "%s: T = %d, but the cache describes %d tables", name,
+              a.T, a.cache->mixed_T);
+  backward_layout(a.num_indices, mixed_tables(a.cache) ? mixed_layout_dim(a.dtype) : a.D, a.dtype, a.T, l);
   cache_layout(a.num_indices, a.cache->num_sets, a.cache->stage_slots, cl);
   if (!a.workspace || a.workspace_bytes < l->total_bytes)
     return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
@@ -722,7 +784,7 @@ int plan_step(const char *name, const PlanArgs &a, const tbe_workspace_layout_t 
   const int64_t num_sets = cache->num_sets;
   const int64_t num_slots = num_sets * kWays;
   const bool defer = deferred(cache);
-  const int row_units = static_cast<int>(static_cast<int64_t>(a.D) * dtype_size(a.dtype) / 8);
+  const BackingMap backing = backing_map(cache, a.D, a.dtype);
   // deferred write-back: this step stages into one of three areas; the area of the step before may
   // still be updated; the one before that is final and is released by this step
   const int64_t stage_base = num_slots + (defer ? area_of(a.sequence) * cache->stage_slots : 0);
@@ -787,13 +849,13 @@ int plan_step(const char *name, const PlanArgs &a, const tbe_workspace_layout_t 
     // crawl behind its outstanding host reads, and the step takes 62 / 55 / 50 / 55 / 58 ms.
     TBE_LAUNCH("cache_fill", link, cache_fill_deferred_kernel,
                dim3(grid_for(work, kWavesPerBlock * kFillBatch, 256)),
-               block, static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units,
+               block, static_cast<uint64_t *>(cache->rows), backing,
                keys_sorted, segment_starts, counters, i32_at(cw, cl.unique_slots), i32_at(cw, cl.evicted_keys),
                i32_at(cw, cl.landing), i32_at(cw, cl.fetch_source), i32_at(cw, cl.write_out), old_stage_base,
                cache->stage_slots, num_slots);
   } else {
     TBE_LAUNCH("cache_fill", link, cache_fill_kernel, dim3(grid_for(n, kWavesPerBlock, 256 * 16)), block,
-               static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows), row_units,
+               static_cast<uint64_t *>(cache->rows), backing,
                keys_sorted, segment_starts, counters, i32_at(cw, cl.unique_slots), i32_at(cw, cl.evicted_keys));
   }
   return check_launch(name);
@@ -805,10 +867,9 @@ int commit_step(const char *name, const PlanArgs &a, const tbe_workspace_layout_
   if (!deferred(cache) || a.num_indices == 0) return TBE_OK;
   void *ws = a.workspace, *cw = a.cache_workspace;
   const int64_t num_slots = cache->num_sets * kWays;
-  const int row_units = static_cast<int>(static_cast<int64_t>(a.D) * dtype_size(a.dtype) / 8);
   TBE_LAUNCH("cache_commit", s, cache_commit_kernel, dim3(grid_for(a.num_indices, kWavesPerBlock, 256 * 16)),
-             dim3(kBlockThreads), static_cast<uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows),
-             row_units, i32_at(ws, l.keys_sorted), i32_at(ws, l.segment_starts), i32_at(ws, l.num_unique),
+             dim3(kBlockThreads), static_cast<uint64_t *>(cache->rows), backing_map(cache, a.D, a.dtype),
+             i32_at(ws, l.keys_sorted), i32_at(ws, l.segment_starts), i32_at(ws, l.num_unique),
              i32_at(cw, cl.unique_slots), i32_at(cw, cl.evicted_keys), i32_at(cw, cl.landing),
              i32_at(cw, cl.fetch_source), num_slots + area_of(a.sequence - 2) * cache->stage_slots, cache->stage_slots,
              num_slots);
@@ -822,11 +883,9 @@ int cache_unstage(const tbe_cache_t *cache, int32_t dtype, int32_t D, const int3
                   const int32_t *unique_slots, int64_t num_indices, hipStream_t stream) {
   if (cache->stage_slots <= 0 || num_indices == 0) return TBE_OK;
   if (cache->stage_of_row) return TBE_OK;  // deferred: a later fill launch (or a flush) writes them back
-  const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
   TBE_LAUNCH("cache_unstage", stream, cache_unstage_kernel,
              dim3(grid_for(num_indices, kWavesPerBlock, 256 * 16)), dim3(kBlockThreads),
-             static_cast<const uint64_t *>(cache->rows), static_cast<uint64_t *>(cache->backing_rows),
-             row_units, keys_sorted, segment_starts, counters, unique_slots,
+             static_cast<const uint64_t *>(cache->rows), backing_map(cache, D, dtype), keys_sorted, segment_starts, counters, unique_slots,
              cache->num_sets * static_cast<int64_t>(kWays));
   return check_launch("tbe_backward_cached");
 }
@@ -893,7 +952,7 @@ extern "C" int tbe_cache_commit(const tbe_cache_t *cache, int32_t dtype, int32_t
   TBE_REQUIRE(sequence >= 0, "%s: sequence out of range (got %d)", name, sequence);
   tbe_workspace_layout_t l;
   tbe_cache_workspace_layout_t cl;
-  backward_layout(num_indices, D, dtype, T, &l);
+  backward_layout(num_indices, mixed_tables(cache) ? mixed_layout_dim(dtype) : D, dtype, T, &l);
   cache_layout(num_indices, cache->num_sets, cache->stage_slots, &cl);
   TBE_REQUIRE(workspace && workspace_bytes >= l.total_bytes && cache_workspace &&
                   cache_workspace_bytes >= cl.total_bytes,
@@ -933,16 +992,15 @@ extern "C" int tbe_cache_flush(const tbe_cache_t *cache, int32_t dtype, int32_t 
   TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "tbe_cache_flush: bad dtype %d", dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t slots = cache->num_sets * kWays;
-  const int row_units = static_cast<int>(static_cast<int64_t>(D) * dtype_size(dtype) / 8);
+  const BackingMap backing = backing_map(cache, D, dtype);
   TBE_REQUIRE(live_sequences <= static_cast<uint32_t>(kAreas), "tbe_cache_flush: at most %d planned batches can be live",
               kAreas);
   if (deferred(cache)) {
     bool keep[kAreas] = {false, false, false};
     for (uint32_t back = 0; back < live_sequences; ++back) keep[area_of(static_cast<int64_t>(last_sequence) - back)] = true;
-    for (int64_t area = 0; area < kAreas; ++area) write_back_stage(cache, row_units, area, keep[area], s);
+    for (int64_t area = 0; area < kAreas; ++area) write_back_stage(cache, backing, area, keep[area], s);
   }
   TBE_LAUNCH("cache_flush", s, cache_flush_kernel, dim3(grid_for(slots, kWavesPerBlock, 256 * 16)),
-             dim3(kBlockThreads), cache->tags, static_cast<const uint64_t *>(cache->rows),
-             static_cast<uint64_t *>(cache->backing_rows), row_units, slots);
+             dim3(kBlockThreads), cache->tags, static_cast<const uint64_t *>(cache->rows), backing, slots);
   return check_launch("tbe_cache_flush");
 }

@@ -42,12 +42,16 @@ template <> __device__ __forceinline__ double mixed_multiplier<double>(double s,
 // groups split the bag's rows and are combined by a butterfly at the end -- a table of 32
 // columns keeps all 64 lanes busy with 8 rows per load instruction instead of 8 lanes with one.
 // Wider rows are walked in blocks of 64 vectors, one row per load.
-template <typename T, int VEC, bool WEIGHTED, int UNROLL>
+// CACHED: every lookup carries a location (lookup_slots[p]); a non-negative value is a row of the
+// HBM row cache (at cache_rows + slot * slot_D, slot_D the widest table's width), a negative one
+// means the row is read from the table.
+template <typename T, int VEC, bool WEIGHTED, int UNROLL, bool CACHED>
 __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
     const T *__restrict__ weights, const int64_t *__restrict__ table_offsets,
     const int32_t *__restrict__ dim_offsets, const int32_t *__restrict__ indices,
     const int32_t *__restrict__ offsets, const T *__restrict__ psw, T *__restrict__ output, int B,
-    int total_D, int num_bags, int64_t blocks_per_xcd) {
+    int total_D, int num_bags, int64_t blocks_per_xcd, const int32_t *__restrict__ lookup_slots,
+    const T *__restrict__ cache_rows, int slot_D) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
@@ -75,15 +79,17 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
     const int c = lane & (group_lanes - 1);
     const bool active = c < chunks;
     // a lane beside the row's columns loads the row's last vector and drops it
-    const T *col = table + static_cast<int64_t>(min(c, chunks - 1)) * VEC;
+    const int64_t col_element = static_cast<int64_t>(min(c, chunks - 1)) * VEC;
+    const T *col = table + col_element;
     V acc;
     acc.zero();
     for (int base = start; base < end; base += kWave) {
       const int n = min(kWave, end - base);
-      int my_idx = 0;
+      int my_idx = 0, my_slot = -1;
       T my_w_raw = T(0);
       if (lane < n) {
         my_idx = __builtin_nontemporal_load(indices + base + lane);
+        if constexpr (CACHED) my_slot = __builtin_nontemporal_load(lookup_slots + base + lane);
         if constexpr (WEIGHTED) my_w_raw = psw[base + lane];
       }
       const A my_w = WEIGHTED ? to_acc(my_w_raw) : A(0);
@@ -104,7 +110,12 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
           const int src = j < n ? j : 0;
           const int64_t idx = shfl_idx(my_idx, src);
           if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, src);
-          raw[u] = V::load_raw(col + idx * D);
+          const T *row = col + idx * D;
+          if constexpr (CACHED) {
+            const int slot = shfl_idx(my_slot, src);
+            if (slot >= 0) row = cache_rows + static_cast<int64_t>(slot) * slot_D + col_element;
+          }
+          raw[u] = V::load_raw(row);
         }
 #pragma unroll
         for (int u = 0; u < kCount; ++u) {
@@ -140,10 +151,11 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
     acc.zero();
     for (int base = start; base < end; base += kWave) {
       const int n = min(kWave, end - base);
-      int my_idx = 0;
+      int my_idx = 0, my_slot = -1;
       A my_w = A(0);
       if (lane < n) {
         my_idx = indices[base + lane];
+        if constexpr (CACHED) my_slot = lookup_slots[base + lane];
         if constexpr (WEIGHTED) my_w = to_acc(psw[base + lane]);
       }
       for (int j0 = 0; j0 < n; j0 += 4) {
@@ -154,7 +166,12 @@ __global__ __launch_bounds__(kBlockThreads) void forward_mixed_kernel(
           const int j = min(j0 + u, n - 1);
           const int64_t idx = shfl_idx(my_idx, j);
           if constexpr (WEIGHTED) w[u] = shfl_idx(my_w, j);
-          if (ok_c && j0 + u < n) raw[u] = V::load_raw(col + idx * D);
+          const T *row = col + idx * D;
+          if constexpr (CACHED) {
+            const int slot = shfl_idx(my_slot, j);
+            if (slot >= 0) row = cache_rows + static_cast<int64_t>(slot) * slot_D + static_cast<int64_t>(c) * VEC;
+          }
+          if (ok_c && j0 + u < n) raw[u] = V::load_raw(row);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -179,8 +196,21 @@ struct MixedRow {
   int seg_begin, seg_end;  // sorted positions of its occurrences
   int32_t key;             // global row id (index of its optimizer state)
   int dim_start, D;        // first gradient column and width of its table
-  int64_t row_element;     // element offset of the row in `weights`
+  int64_t row_element;     // element offset of the row in `weights` (its place in the table: what the
+                           // random words of stochastic rounding go by)
+  void *where;             // the row's first element where it is stored: in `weights`, or in a row of the cache
 };
+
+// Fills in where the u-th unique row is stored.
+template <bool CACHED, typename T>
+__device__ __forceinline__ void locate_row(MixedRow &row, T *weights, const int32_t *__restrict__ unique_slots, int64_t u,
+                                           T *cache_rows, int slot_D) {
+  row.where = weights + row.row_element;
+  if constexpr (CACHED) {
+    const int slot = unique_slots[u];
+    if (slot >= 0) row.where = cache_rows + static_cast<int64_t>(slot) * slot_D;
+  }
+}
 
 // Narrow rows (at most 64 vectors): `chunks` = D / VEC consecutive lanes form a lane group, the
 // 64 / chunks groups split the occurrences of a 64-position batch (the batch's positions,
@@ -192,7 +222,7 @@ struct MixedRow {
 // w_old (valid in every group when WEIGHTED, else in group 0).
 template <typename T, int VEC, bool WEIGHTED, int UNROLL>
 __device__ __forceinline__ void mixed_accumulate_narrow(
-    const T *__restrict__ grad_output, const T *__restrict__ weights, const T *__restrict__ psw,
+    const T *__restrict__ grad_output, const T *__restrict__ psw,
     T *__restrict__ grad_psw, int num_tables, int total_D,
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows, int lane,
     const MixedRow &row, int first_batch, int batch_stride, RowVec<T, VEC> &w_old, RowVec<T, VEC> &G) {
@@ -210,7 +240,7 @@ __device__ __forceinline__ void mixed_accumulate_narrow(
   const bool active = c < chunks;
   const int64_t col = static_cast<int64_t>(c) * VEC;
   const int64_t safe_col = active ? col : 0;
-  const T *wrow = weights + row.row_element;
+  const T *wrow = static_cast<const T *>(row.where);
   const T *gcol = grad_output + row.dim_start;
   w_old.zero();
   if (active && (WEIGHTED || r == 0)) w_old.load(wrow + col);
@@ -287,8 +317,7 @@ __device__ __forceinline__ void mixed_accumulate_narrow(
 
 // Optimizer step of a narrow row whose gradient sum G sits in lane group 0.
 template <typename T, int VEC, int OPT>
-__device__ __forceinline__ void mixed_apply_narrow(T *__restrict__ weights,
-                                                   typename AccOf<T>::type *__restrict__ state,
+__device__ __forceinline__ void mixed_apply_narrow(typename AccOf<T>::type *__restrict__ state,
                                                    float lr, float eps, const StochasticRounding &sr,
                                                    int lane, const MixedRow &row,
                                                    typename AccOf<T>::type state_old,
@@ -313,8 +342,8 @@ __device__ __forceinline__ void mixed_apply_narrow(T *__restrict__ weights,
     V w;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) w.v[i] = w_old.v[i] - G.v[i] * mult;
-    const int64_t element = row.row_element + static_cast<int64_t>(lane) * VEC;
-    store_row<T, VEC, false>(weights + element, w, sr, element);
+    const int64_t col = static_cast<int64_t>(lane) * VEC;
+    store_row<T, VEC, false>(static_cast<T *>(row.where) + col, w, sr, row.row_element + col);
   }
 }
 
@@ -322,8 +351,7 @@ __device__ __forceinline__ void mixed_apply_narrow(T *__restrict__ weights,
 // squares first, then the update), one column block of 64 vectors at a time.
 template <typename T, int VEC, int OPT, bool WEIGHTED>
 __device__ __forceinline__ void mixed_update_wide(
-    const T *__restrict__ grad_output, T *__restrict__ weights,
-    typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
+    const T *__restrict__ grad_output, typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
     T *__restrict__ grad_psw, int num_tables, int total_D,
     const int32_t *__restrict__ positions_sorted, const int32_t *__restrict__ grad_rows, float lr,
     float eps, const StochasticRounding &sr, int lane, const MixedRow &row,
@@ -334,7 +362,7 @@ __device__ __forceinline__ void mixed_update_wide(
   const int32_t key = row.key;
   const int64_t row_element = row.row_element;
   const int chunks = row.D / VEC;
-  T *wrow = weights + row_element;
+  T *wrow = static_cast<T *>(row.where);
   const T *gcol = grad_output + row.dim_start;
   if constexpr (WEIGHTED) {
     for (int i = seg_begin; i < seg_end; ++i) {
@@ -439,7 +467,10 @@ constexpr int kMixedAhead = 4;
 // multiplier, one occurrence after the other in position order, the row rounded to the weights'
 // type every time (the arithmetic of approx_adagrad_kernel).  Rows of more than kMixedShort
 // occurrences then go to a queue of row numbers (`queued_rows`, counters[1]) whatever their length.
-template <typename T, int VEC, int OPT, bool WEIGHTED, bool APPROX = false>
+// CACHED: the tables are fronted by the row cache; unique_slots[u] >= 0 is the row of `cache_rows`
+// (slot_D elements each) that holds the u-th unique row, and the list records of the rows of several
+// chunks carry the row's number u instead of its table.
+template <typename T, int VEC, int OPT, bool WEIGHTED, bool APPROX = false, bool CACHED = false>
 __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 8, APPROX, sizeof(T) == 8)) void update_mixed_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
@@ -451,13 +482,23 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
     int32_t *__restrict__ counters, int32_t *__restrict__ wide_rows,
     int32_t *__restrict__ queued_rows, ChunkRecord *__restrict__ chunk_records,
     LongRecord *__restrict__ long_records, int64_t max_chunks, int64_t max_long, int positions_per_xcd,
-    float lr, float eps, StochasticRounding sr) {
+    float lr, float eps, StochasticRounding sr, const int32_t *__restrict__ unique_slots = nullptr,
+    T *__restrict__ cache_rows = nullptr, int slot_D = 0) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   using R = typename V::R;
   static_assert(sizeof(A) == 4 || sizeof(A) == 8, "optimizer state is float or double");
-  // a row's record: {occurrences, first slot, key, D}, {first element of the row (64 bits), state}
+  // a row's record: {occurrences, first slot, key, D}, {where the row is stored (64 bits), state}.
+  // Where: its first element in `weights`; CACHED: or, complemented, its first element in `cache_rows`,
+  // and s_element holds its first element in `weights` (its place in the table) beside the record.
   __shared__ int4 s_row[kWavesPerBlock][kWave][2];
+  __shared__ int64_t s_element[kWavesPerBlock][CACHED ? kWave : 1];
+  auto stored_at = [&](int64_t where) -> T * {
+    if constexpr (CACHED) {
+      if (where < 0) return cache_rows + ~where;
+    }
+    return weights + where;
+  };
   // occurrences of a strip's short rows: at most 64 rows of kMixedShort occurrences
   __shared__ int s_goff[kWavesPerBlock][kWave * kMixedShort];
   __shared__ int s_pos[kWavesPerBlock][WEIGHTED ? kWave * kMixedShort : 1];
@@ -496,6 +537,11 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
         table_offsets[l_table] + static_cast<int64_t>(l_key - table_dim_offsets[l_table]) * l_D;
     A l_state = A(0);
     if constexpr (OPT == kOptAdagrad) l_state = state[l_key];
+    int64_t l_where = l_row_element;
+    if constexpr (CACHED) {
+      const int slot = unique_slots[my_u];
+      if (slot >= 0) l_where = ~(static_cast<int64_t>(slot) * slot_D);
+    }
 
     // Rows that are not reduced here.  Rows wider than 64 vectors go to a queue of row numbers
     // whatever their length (`wide_rows`, counters[2]; one atomic per strip).
@@ -554,7 +600,7 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
       const int my_first_chunk = first_chunk_of_strip + (before & 0xffffff);
       if (my_nch > 1)
         long_records[queue_index * (max_long / kNumXcd) + first_entry_of_strip + (before >> 24)] =
-            LongRecord{l_table, l_key, l_begin, l_end};
+            LongRecord{CACHED ? static_cast<int32_t>(my_u) : l_table, l_key, l_begin, l_end};
       ChunkRecord *queue = chunk_records + queue_index * (max_chunks / kNumXcd);
       for (unsigned long long rest = queued_mask; rest != 0ull; rest &= rest - 1ull) {
         const int src = __ffsll(static_cast<long long>(rest)) - 1;
@@ -600,8 +646,8 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
       st_hi = static_cast<int>(bits >> 32);
     }
     s_row[wave][my_rank][0] = make_int4(my_len, my_offset, l_key, is_short ? l_D : 0);
-    s_row[wave][my_rank][1] =
-        make_int4(static_cast<int>(l_row_element), static_cast<int>(l_row_element >> 32), st_lo, st_hi);
+    s_row[wave][my_rank][1] = make_int4(static_cast<int>(l_where), static_cast<int>(l_where >> 32), st_lo, st_hi);
+    if constexpr (CACHED) s_element[wave][my_rank] = l_row_element;
 #pragma unroll
     for (int i = 0; i < kMixedShort; ++i) {
       if (i < my_len) {
@@ -633,9 +679,9 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
       const int4 d1 = s_row[wave][k0 + r][1];
       const int len = d0.x, slot0 = d0.y;
       const bool active = col < d0.w;
-      const int64_t row_element =
+      const int64_t where =
           (static_cast<int64_t>(d1.y) << 32) | static_cast<int64_t>(static_cast<uint32_t>(d1.x));
-      if (active) f.w = V::load_raw_streaming(weights + row_element + col);
+      if (active) f.w = V::load_raw_streaming(stored_at(where) + col);
 #pragma unroll
       for (int u = 0; u < kMixedAhead; ++u) {
         if (__ballot(u < len) == 0ull) break;
@@ -661,8 +707,10 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
       const int len = d0.x, slot0 = d0.y;
       const int32_t key = d0.z;
       const bool active = col < d0.w;
-      const int64_t row_element =
+      const int64_t where =
           (static_cast<int64_t>(d1.y) << 32) | static_cast<int64_t>(static_cast<uint32_t>(d1.x));
+      int64_t row_element = where;
+      if constexpr (CACHED) row_element = s_element[wave][k0 + r];
       A state_old;
       if constexpr (sizeof(A) == 4) {
         state_old = __builtin_bit_cast(A, d1.z);
@@ -742,7 +790,7 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
       if constexpr (APPROX) {
         if (len > 0 && c == 0) state[key] = running;
         // (fp16: the last occurrence already rounded the row to the stored type)
-        if (len > 0 && active) w_old.store_streaming(weights + row_element + col);
+        if (len > 0 && active) w_old.store_streaming(stored_at(where) + col);
         return;
       }
       A mult = static_cast<A>(lr);
@@ -759,7 +807,7 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
         V w;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) w.v[i] = w_old.v[i] - G.v[i] * mult;
-        store_row<T, VEC, true>(weights + row_element + col, w, sr, row_element + col);
+        store_row<T, VEC, true>(stored_at(where) + col, w, sr, row_element + col);
       }
     };
     Fetched fa{}, fb{};
@@ -785,7 +833,7 @@ __device__ __forceinline__ int bag_of_grad_row(int grow, const MixedTables &mt) 
 // The chunk records of mixed-D tables: update_chunks_kernel's walk over the eight queues, each record
 // reduced with its own table's row width.  A chunk that is a whole segment is applied to its row
 // at once; a chunk of a longer segment stores its sum as a partial row of 64 vectors.
-template <typename T, int VEC, int OPT, bool WEIGHTED, int UNROLL>
+template <typename T, int VEC, int OPT, bool WEIGHTED, int UNROLL, bool CACHED>
 __global__ __launch_bounds__(kBlockThreads) void update_chunks_mixed_kernel(
     const T *__restrict__ grad_output, T *__restrict__ weights,
     typename AccOf<T>::type *__restrict__ state, const T *__restrict__ psw,
@@ -794,7 +842,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_mixed_kernel(
     const int32_t *__restrict__ segment_starts, const int32_t *__restrict__ counters,
     const ChunkRecord *__restrict__ chunk_records, int64_t max_chunks, const int32_t *__restrict__ wide_rows,
     typename AccOf<T>::type *__restrict__ partial_sums, float lr, float eps, StochasticRounding sr,
-    MixedTables mt) {
+    MixedTables mt, const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows, int slot_D) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   const int lane = threadIdx.x & (kWave - 1);
@@ -844,12 +892,13 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_mixed_kernel(
     row.dim_start = mt.dim_offsets[t];
     row.D = mt.dim_offsets[t + 1] - row.dim_start;
     row.row_element = mt.table_offsets[t] + static_cast<int64_t>(rec.key - mt.table_dim_offsets[t]) * row.D;
+    locate_row<CACHED>(row, weights, unique_slots, rec.u, cache_rows, slot_D);
     A state_old = A(0);
     if constexpr (OPT == kOptAdagrad) {
       if (rec.partial < 0) state_old = state[rec.key];
     }
     V w_old, G;
-    mixed_accumulate_narrow<T, VEC, WEIGHTED, UNROLL>(grad_output, weights, psw, grad_psw, mt.T, mt.total_D,
+    mixed_accumulate_narrow<T, VEC, WEIGHTED, UNROLL>(grad_output, psw, grad_psw, mt.T, mt.total_D,
                                                       positions_sorted, grad_rows, lane, row, 0, 1, w_old, G);
     if (rec.partial >= 0) {
       if (lane < row.D / VEC) {
@@ -858,7 +907,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_mixed_kernel(
         for (int i = 0; i < VEC; ++i) dst[i] = G.v[i];
       }
     } else {
-      mixed_apply_narrow<T, VEC, OPT>(weights, state, lr, eps, sr, lane, row, state_old, w_old, G);
+      mixed_apply_narrow<T, VEC, OPT>(state, lr, eps, sr, lane, row, state_old, w_old, G);
     }
   }
   // the rows wider than 64 vectors, a wavefront each (their number: counters[2])
@@ -874,22 +923,26 @@ __global__ __launch_bounds__(kBlockThreads) void update_chunks_mixed_kernel(
     row.dim_start = mt.dim_offsets[t];
     row.D = mt.dim_offsets[t + 1] - row.dim_start;
     row.row_element = mt.table_offsets[t] + static_cast<int64_t>(row.key - mt.table_dim_offsets[t]) * row.D;
+    locate_row<CACHED>(row, weights, unique_slots, u, cache_rows, slot_D);
     A state_old = A(0);
     if constexpr (OPT == kOptAdagrad) state_old = state[row.key];
-    mixed_update_wide<T, VEC, OPT, WEIGHTED>(grad_output, weights, state, psw, grad_psw, mt.T, mt.total_D,
+    mixed_update_wide<T, VEC, OPT, WEIGHTED>(grad_output, state, psw, grad_psw, mt.T, mt.total_D,
                                              positions_sorted, grad_rows, lr, eps, sr, lane, row, state_old);
   }
 }
 
 // The rows of several chunks of mixed-D tables: one wavefront per row adds its partial rows in
 // chunk order (lane group r takes partial rows r, r + groups, ..., the groups are combined in a
-// fixed tree) and applies the optimizer.  The list records carry the row's table in `u`.
-template <typename T, int VEC, int OPT>
+// fixed tree) and applies the optimizer.  The list records carry the row's table in `u` -- or,
+// CACHED, the row's number, and the table follows from the gradient row of its first occurrence.
+template <typename T, int VEC, int OPT, bool CACHED>
 __global__ __launch_bounds__(kBlockThreads) void update_long_finish_mixed_kernel(
     T *__restrict__ weights, typename AccOf<T>::type *__restrict__ state,
     const int32_t *__restrict__ counters, const LongRecord *__restrict__ long_records,
     const typename AccOf<T>::type *__restrict__ partial_sums, float lr, float eps, StochasticRounding sr,
-    int64_t max_long, MixedTables mt) {
+    int64_t max_long, MixedTables mt, const int32_t *__restrict__ positions_sorted,
+    const int32_t *__restrict__ grad_rows, const int32_t *__restrict__ unique_slots, T *__restrict__ cache_rows,
+    int slot_D) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
   const int lane = threadIdx.x & (kWave - 1);
@@ -898,7 +951,11 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_mixed_kernel
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
   for (int64_t slot = wave_id; slot < lists.total; slot += stride) {
     const LongRecord rec = long_record_at(long_records, lists, slot);
-    const int t = rec.u;
+    int t = rec.u;
+    if constexpr (CACHED) {
+      const int grow = grad_rows[positions_sorted[rec.begin]];
+      t = grow - bag_of_grad_row(grow, mt) * mt.T;
+    }
     MixedRow row;
     row.seg_begin = rec.begin;
     row.seg_end = rec.end;
@@ -906,6 +963,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_mixed_kernel
     row.dim_start = mt.dim_offsets[t];
     row.D = mt.dim_offsets[t + 1] - row.dim_start;
     row.row_element = mt.table_offsets[t] + static_cast<int64_t>(rec.key - mt.table_dim_offsets[t]) * row.D;
+    locate_row<CACHED>(row, weights, unique_slots, rec.u, cache_rows, slot_D);
     const int chunks = row.D / VEC;
     const int group_shift = chunks > 1 ? 32 - __builtin_clz(chunks - 1) : 0;
     const int group_lanes = 1 << group_shift;
@@ -917,7 +975,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_mixed_kernel
     const int num_chunks = (rec.end - rec.begin + kChunkLen - 1) / kChunkLen;
     V w_old;
     w_old.zero();
-    if (lane < chunks) w_old.load(weights + row.row_element + col);
+    if (lane < chunks) w_old.load(static_cast<const T *>(row.where) + col);
     A state_old = A(0);
     if constexpr (OPT == kOptAdagrad) state_old = state[rec.key];
     V G;
@@ -944,7 +1002,7 @@ __global__ __launch_bounds__(kBlockThreads) void update_long_finish_mixed_kernel
 #pragma unroll
       for (int i = 0; i < VEC; ++i) G.v[i] += shfl_x(G.v[i], m);
     }
-    mixed_apply_narrow<T, VEC, OPT>(weights, state, lr, eps, sr, lane, row, state_old, w_old, G);
+    mixed_apply_narrow<T, VEC, OPT>(state, lr, eps, sr, lane, row, state_old, w_old, G);
   }
 }
 
@@ -969,6 +1027,12 @@ struct MixedArgs {
   float lr, eps;
   int optimizer;
   StochasticRounding sr;
+  // tables fronted by the row cache (null otherwise): where every lookup / every unique row lives,
+  // the cache's rows and their width
+  const int32_t *lookup_slots;
+  const int32_t *unique_slots;
+  void *cache_rows;
+  int32_t slot_D;
 };
 
 template <typename T, int VEC>
@@ -979,19 +1043,27 @@ void launch_forward_mixed(const MixedArgs &a, hipStream_t stream) {
   const T *w = static_cast<const T *>(a.weights);
   const T *p = static_cast<const T *>(a.psw);
   T *o = static_cast<T *>(a.output);
-  if (a.psw)
-    TBE_LAUNCH("forward_mixed", stream, (forward_mixed_kernel<T, VEC, true, 8>), grid, block, w,
-               a.table_offsets, a.dim_offsets, a.indices, a.offsets, p, o, a.B, a.total_D, num_bags, per_xcd);
-  else
-    TBE_LAUNCH("forward_mixed", stream, (forward_mixed_kernel<T, VEC, false, 8>), grid, block, w,
-               a.table_offsets, a.dim_offsets, a.indices, a.offsets, p, o, a.B, a.total_D, num_bags, per_xcd);
+  const T *cr = static_cast<const T *>(a.cache_rows);
+#define TBE_FORWARD_MIXED(WEIGHTED, CACHED)                                                                     \
+  TBE_LAUNCH("forward_mixed", stream, (forward_mixed_kernel<T, VEC, WEIGHTED, 8, CACHED>), grid, block, w,      \
+             a.table_offsets, a.dim_offsets, a.indices, a.offsets, p, o, a.B, a.total_D, num_bags, per_xcd,     \
+             a.lookup_slots, cr, a.slot_D)
+  if (a.lookup_slots) {
+    if (a.psw) TBE_FORWARD_MIXED(true, true);
+    else TBE_FORWARD_MIXED(false, true);
+  } else {
+    if (a.psw) TBE_FORWARD_MIXED(true, false);
+    else TBE_FORWARD_MIXED(false, false);
+  }
+#undef TBE_FORWARD_MIXED
 }
 
 // The exact update: the strip kernel for the rows of few occurrences, then one wavefront per chunk
 // record (and per row wider than 64 vectors), then the rows of several chunks.
-template <typename T, int VEC, int OPT, bool WEIGHTED>
+template <typename T, int VEC, int OPT, bool WEIGHTED, bool CACHED>
 void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, char *ws, hipStream_t stream) {
   using A = typename AccOf<T>::type;
+  T *cr = static_cast<T *>(a.cache_rows);
   auto i32 = [&](uint64_t off) { return reinterpret_cast<int32_t *>(ws + off); };
   const T *go = static_cast<const T *>(a.grad_output);
   T *w = static_cast<T *>(a.weights);
@@ -1011,11 +1083,11 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
   const dim3 block(kBlockThreads);
   const int64_t want = ceil_div(ceil_div(a.n, kWave), kWavesPerBlock);
   const dim3 grid(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want, 256 * 32))));
-  TBE_LAUNCH("update_mixed", stream, (update_mixed_kernel<T, VEC, OPT, WEIGHTED>), grid, block,
+  TBE_LAUNCH("update_mixed", stream, (update_mixed_kernel<T, VEC, OPT, WEIGHTED, false, CACHED>), grid, block,
              go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, mt.bag_magic, mt.bag_shift,
              a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
              i32(l.num_unique), wide_rows, static_cast<int32_t *>(nullptr), chunk_records, long_records, max_chunks,
-             max_long, static_cast<int>(ceil_div(a.n, kNumXcd)), a.lr, a.eps, a.sr);
+             max_long, static_cast<int>(ceil_div(a.n, kNumXcd)), a.lr, a.eps, a.sr, a.unique_slots, cr, a.slot_D);
 
   const bool small = ceil_div(a.n, tile_positions(0)) < kSmallBatchTiles;
   const int64_t want_chunks = ceil_div(max_chunks, kWavesPerBlock);
@@ -1023,19 +1095,21 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
   const dim3 grid_chunks(static_cast<unsigned>(
       kNumXcd * std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_chunks, kNumXcd), small ? 64 : 1024))));
   TBE_LAUNCH("update_chunks_mixed", stream,
-             (update_chunks_mixed_kernel<T, VEC, OPT, WEIGHTED, (WEIGHTED && VEC == 8) ? 4 : 8>), grid_chunks, block,
-             go, w, st, psw, gpsw, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
-             i32(l.num_unique), chunk_records, max_chunks, wide_rows, partial, a.lr, a.eps, a.sr, mt);
+             (update_chunks_mixed_kernel<T, VEC, OPT, WEIGHTED, (WEIGHTED && VEC == 8) ? 4 : 8, CACHED>), grid_chunks,
+             block, go, w, st, psw, gpsw, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows),
+             i32(l.segment_starts), i32(l.num_unique), chunk_records, max_chunks, wide_rows, partial, a.lr, a.eps, a.sr,
+             mt, a.unique_slots, cr, a.slot_D);
 
   const int64_t want_long = ceil_div(max_long, kWavesPerBlock);
   const dim3 grid_finish(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(want_long, 256 * 4))));
-  TBE_LAUNCH("update_long_finish_mixed", stream, (update_long_finish_mixed_kernel<T, VEC, OPT>), grid_finish, block,
-             w, st, i32(l.num_unique), long_records, partial, a.lr, a.eps, a.sr, max_long, mt);
+  TBE_LAUNCH("update_long_finish_mixed", stream, (update_long_finish_mixed_kernel<T, VEC, OPT, CACHED>), grid_finish,
+             block, w, st, i32(l.num_unique), long_records, partial, a.lr, a.eps, a.sr, max_long, mt,
+             i32(l.positions_sorted), i32(l.grad_rows), a.unique_slots, cr, a.slot_D);
 }
 
 // The approximate update's strip kernel: rows of at most 64 vectors and kMixedShort occurrences
 // are applied, the others queued for approx_update.
-template <typename T, int VEC, bool WEIGHTED>
+template <typename T, int VEC, bool WEIGHTED, bool CACHED>
 void launch_update_mixed_approx(const MixedArgs &a, const tbe_workspace_layout_t &l, char *ws, hipStream_t stream) {
   using A = typename AccOf<T>::type;
   auto i32 = [&](uint64_t off) { return reinterpret_cast<int32_t *>(ws + off); };
@@ -1046,40 +1120,49 @@ void launch_update_mixed_approx(const MixedArgs &a, const tbe_workspace_layout_t
   const int bag_shift = 31 + log2_T;
   const uint32_t bag_magic =
       static_cast<uint32_t>(((uint64_t{1} << bag_shift) + static_cast<uint64_t>(a.T) - 1) / static_cast<uint64_t>(a.T));
-  TBE_LAUNCH("update_mixed_approx", stream, (update_mixed_kernel<T, VEC, kOptAdagrad, WEIGHTED, true>), grid,
+  TBE_LAUNCH("update_mixed_approx", stream, (update_mixed_kernel<T, VEC, kOptAdagrad, WEIGHTED, true, CACHED>), grid,
              dim3(kBlockThreads), static_cast<const T *>(a.grad_output), static_cast<T *>(a.weights),
              static_cast<A *>(a.state), static_cast<const T *>(a.psw), static_cast<T *>(a.grad_psw),
              a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, bag_magic, bag_shift, a.total_D,
              i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
              i32(l.num_unique), approx_mixed_wide_queue(l, ws), approx_mixed_long_queue(l, ws),
              static_cast<ChunkRecord *>(nullptr), static_cast<LongRecord *>(nullptr), int64_t{0}, int64_t{0}, 1, a.lr,
-             a.eps, a.sr);
+             a.eps, a.sr, a.unique_slots, static_cast<T *>(a.cache_rows), a.slot_D);
 }
 
 template <typename T, int VEC>
 void launch_update_mixed_approx_variant(const MixedArgs &a, const tbe_workspace_layout_t &l, char *ws,
                                         hipStream_t stream) {
-  if (a.psw) launch_update_mixed_approx<T, VEC, true>(a, l, ws, stream);
-  else launch_update_mixed_approx<T, VEC, false>(a, l, ws, stream);
+  if (a.unique_slots) {
+    if (a.psw) launch_update_mixed_approx<T, VEC, true, true>(a, l, ws, stream);
+    else launch_update_mixed_approx<T, VEC, false, true>(a, l, ws, stream);
+  } else {
+    if (a.psw) launch_update_mixed_approx<T, VEC, true, false>(a, l, ws, stream);
+    else launch_update_mixed_approx<T, VEC, false, false>(a, l, ws, stream);
+  }
 }
 
 template <typename T, int VEC>
 void launch_update_mixed_variant(const MixedArgs &a, const tbe_workspace_layout_t &l, char *ws,
                                  hipStream_t stream) {
   const bool weighted = a.psw != nullptr;
-  if (a.optimizer == kOptSgd) {
-    if (weighted) launch_update_mixed<T, VEC, kOptSgd, true>(a, l, ws, stream);
-    else launch_update_mixed<T, VEC, kOptSgd, false>(a, l, ws, stream);
-  } else {
-    if (weighted) launch_update_mixed<T, VEC, kOptAdagrad, true>(a, l, ws, stream);
-    else launch_update_mixed<T, VEC, kOptAdagrad, false>(a, l, ws, stream);
+  if (a.unique_slots) {
+    if (a.optimizer == kOptSgd) {
+      if (weighted) launch_update_mixed<T, VEC, kOptSgd, true, true>(a, l, ws, stream);
+      else launch_update_mixed<T, VEC, kOptSgd, false, true>(a, l, ws, stream);
+    } else {
+      if (weighted) launch_update_mixed<T, VEC, kOptAdagrad, true, true>(a, l, ws, stream);
+      else launch_update_mixed<T, VEC, kOptAdagrad, false, true>(a, l, ws, stream);
+    }
+    return;
   }
-}
-
-// Row width the workspace of mixed-D tables is laid out for: its partial rows hold 64 vectors, the
-// widest row that is summed in chunks (8 elements a vector at most for fp16).
-int32_t mixed_layout_dim(int32_t dtype) {
-  return kWave * (dtype == TBE_DTYPE_F16 ? 8 : dtype == TBE_DTYPE_F32 ? 4 : 2);
+  if (a.optimizer == kOptSgd) {
+    if (weighted) launch_update_mixed<T, VEC, kOptSgd, true, false>(a, l, ws, stream);
+    else launch_update_mixed<T, VEC, kOptSgd, false, false>(a, l, ws, stream);
+  } else {
+    if (weighted) launch_update_mixed<T, VEC, kOptAdagrad, true, false>(a, l, ws, stream);
+    else launch_update_mixed<T, VEC, kOptAdagrad, false, false>(a, l, ws, stream);
+  }
 }
 
 int validate_mixed(const char *name, const MixedArgs &a) {
@@ -1230,4 +1313,147 @@ extern "C" int tbe_backward_mixed(int32_t optimizer, const void *grad_output, vo
     default: launch_update_mixed_variant<double, 2>(a, l, ws, s); break;
   }
   return check_launch(name);
+}
+
+namespace tbe {
+namespace {
+
+int validate_mixed_cache(const char *name, const tbe_cache_t *cache, int32_t D, int32_t total_D) {
+  TBE_REQUIRE(cache && cache->rows && cache->backing_rows, "%s: null cache", name);
+  TBE_REQUIRE(cache->mixed_table_offsets && cache->mixed_table_rows && cache->mixed_dim_offsets && cache->mixed_T > 0,
+              "%s: the cache does not describe tables of different widths (mixed_* fields)", name);
+  TBE_REQUIRE(D > 0 && D % 4 == 0, "%s: D, the width of a cache row, must be a positive multiple of 4 (got %d)", name, D);
+  TBE_REQUIRE(D <= total_D, "%s: a cache row of %d elements is wider than all tables together (%d)", name, D, total_D);
+  return TBE_OK;
+}
+
+}  // namespace
+}  // namespace tbe
+
+extern "C" int tbe_forward_mixed_cached(const tbe_cache_t *cache, int32_t dtype, int32_t fp16_vector_width, int32_t D,
+                                        int32_t total_D, const int32_t *indices, int64_t num_indices,
+                                        const int32_t *offsets, int32_t B, const void *per_sample_weights,
+                                        const int32_t *lookup_slots, void *output, void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_forward_mixed_cached";
+  if (int rc = validate_mixed_cache(name, cache, D, total_D)) return rc;
+  MixedArgs a{};
+  a.weights = cache->backing_rows;
+  a.dtype = dtype;
+  a.vec = fp16_vector_width;
+  a.table_offsets = cache->mixed_table_offsets;
+  a.dim_offsets = cache->mixed_dim_offsets;
+  a.total_D = total_D;
+  a.T = cache->mixed_T;
+  a.indices = indices;
+  a.n = num_indices;
+  a.offsets = offsets;
+  a.B = B;
+  a.psw = per_sample_weights;
+  a.output = output;
+  a.lookup_slots = lookup_slots;
+  a.cache_rows = cache->rows;
+  a.slot_D = D;
+  if (int rc = validate_mixed(name, a)) return rc;
+  TBE_REQUIRE(output, "%s: null output", name);
+  TBE_REQUIRE(lookup_slots || num_indices == 0, "%s: null lookup_slots", name);
+  hipStream_t s = static_cast<hipStream_t>(stream);  // (a batch without lookups reads no row: all zeros)
+  switch (dtype) {
+    case TBE_DTYPE_F32: launch_forward_mixed<float, 4>(a, s); break;
+    case TBE_DTYPE_F16:
+      if (a.vec == 8) launch_forward_mixed<__half, 8>(a, s);
+      else launch_forward_mixed<__half, 4>(a, s);
+      break;
+    default: launch_forward_mixed<double, 2>(a, s); break;
+  }
+  return check_launch(name);
+}
+
+extern "C" int tbe_backward_mixed_cached(int32_t optimizer, const void *grad_output, const tbe_cache_t *cache,
+                                         int32_t dtype, int32_t fp16_vector_width, int32_t D, int32_t total_D,
+                                         int32_t B, int64_t num_indices, const int32_t *offsets,
+                                         const void *per_sample_weights,
+                                         void *optimizer_state, float learning_rate, float eps,
+                                         void *grad_per_sample_weights, int32_t stochastic_rounding, uint64_t seed,
+                                         uint64_t offset, void *workspace, uint64_t workspace_bytes,
+                                         const int32_t *unique_slots, void *stream) {
+  using namespace tbe;
+  const char *name = "tbe_backward_mixed_cached";
+  if (int rc = validate_mixed_cache(name, cache, D, total_D)) return rc;
+  TBE_REQUIRE(optimizer == TBE_OPT_SGD || optimizer == TBE_OPT_ROWWISE_ADAGRAD ||
+                  optimizer == TBE_OPT_APPROX_ROWWISE_ADAGRAD,
+              "%s: bad optimizer %d", name, optimizer);
+  TBE_REQUIRE(optimizer != TBE_OPT_APPROX_ROWWISE_ADAGRAD || offsets,
+              "%s: the approximate update needs the batch's bag offsets", name);
+  MixedArgs a{};
+  a.grad_output = grad_output;
+  a.weights = cache->backing_rows;
+  a.dtype = dtype;
+  a.vec = fp16_vector_width;
+  a.table_offsets = cache->mixed_table_offsets;
+  a.table_dim_offsets = cache->mixed_table_rows;
+  a.dim_offsets = cache->mixed_dim_offsets;
+  a.total_D = total_D;
+  a.T = cache->mixed_T;
+  a.n = num_indices;
+  a.offsets = offsets;
+  a.B = B;
+  a.psw = per_sample_weights;
+  a.state = optimizer_state;
+  a.grad_psw = grad_per_sample_weights;
+  a.lr = learning_rate;
+  a.eps = eps;
+  a.sr = StochasticRounding{seed, offset, (stochastic_rounding && dtype == TBE_DTYPE_F16) ? 1 : 0};
+  a.optimizer = optimizer == TBE_OPT_SGD ? kOptSgd : kOptAdagrad;
+  a.unique_slots = unique_slots;
+  a.cache_rows = cache->rows;
+  a.slot_D = D;
+  TBE_REQUIRE(a.T > 0 && B > 0, "%s: T and B must be positive (got %d, %d)", name, a.T, B);
+  TBE_REQUIRE(total_D > 0 && total_D % 4 == 0, "%s: total_D must be a positive multiple of 4 (got %d)", name, total_D);
+  TBE_REQUIRE(dtype >= TBE_DTYPE_F32 && dtype <= TBE_DTYPE_F64, "%s: bad dtype %d", name, dtype);
+  TBE_REQUIRE(dtype != TBE_DTYPE_F16 || a.vec == 4 || a.vec == 8, "%s: fp16 vector width must be 4 or 8", name);
+  TBE_REQUIRE(num_indices >= 0 && num_indices < INT32_MAX, "%s: num_indices out of range", name);
+  TBE_REQUIRE(static_cast<int64_t>(B) * total_D < INT32_MAX, "%s: grad_output of B*total_D = %lld elements is too large",
+              name, static_cast<long long>(B) * total_D);
+  TBE_REQUIRE(grad_output, "%s: null grad_output", name);
+  TBE_REQUIRE(a.optimizer == kOptSgd || optimizer_state, "%s: optimizer_state is null", name);
+  TBE_REQUIRE((per_sample_weights == nullptr) == (grad_per_sample_weights == nullptr),
+              "%s: per_sample_weights and grad_per_sample_weights must both be given or both be null", name);
+  TBE_REQUIRE(unique_slots || num_indices == 0, "%s: null unique_slots", name);
+  if (num_indices == 0) return TBE_OK;
+  tbe_workspace_layout_t l;
+  backward_layout(num_indices, mixed_layout_dim(dtype), dtype, a.T, &l);
+  if (!workspace || workspace_bytes < l.total_bytes)
+    return fail(TBE_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given", name,
+                (unsigned long long)l.total_bytes, (unsigned long long)workspace_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  char *ws = static_cast<char *>(workspace);
+  if (optimizer == TBE_OPT_APPROX_ROWWISE_ADAGRAD) {
+    switch (dtype) {
+      case TBE_DTYPE_F32: launch_update_mixed_approx_variant<float, 4>(a, l, ws, s); break;
+      case TBE_DTYPE_F16:
+        if (a.vec == 8) launch_update_mixed_approx_variant<__half, 8>(a, l, ws, s);
+        else launch_update_mixed_approx_variant<__half, 4>(a, l, ws, s);
+        break;
+      default: launch_update_mixed_approx_variant<double, 2>(a, l, ws, s); break;
+    }
+    if (int rc = approx_update(grad_output, a.weights, optimizer_state, per_sample_weights, grad_per_sample_weights,
+                               dtype, dtype == TBE_DTYPE_F16 ? a.vec : (dtype == TBE_DTYPE_F32 ? 4 : 2), 0, num_indices,
+                               learning_rate, eps, a.table_offsets, a.table_dim_offsets, a.dim_offsets, total_D, a.T,
+                               offsets, B, a.sr, l, workspace, s, unique_slots, cache->rows, D))
+      return rc;
+  } else {
+    switch (dtype) {
+      case TBE_DTYPE_F32: launch_update_mixed_variant<float, 4>(a, l, ws, s); break;
+      case TBE_DTYPE_F16:
+        if (a.vec == 8) launch_update_mixed_variant<__half, 8>(a, l, ws, s);
+        else launch_update_mixed_variant<__half, 4>(a, l, ws, s);
+        break;
+      default: launch_update_mixed_variant<double, 2>(a, l, ws, s); break;
+    }
+  }
+  if (int rc = check_launch(name)) return rc;
+  return cache_unstage(cache, dtype, D, reinterpret_cast<const int32_t *>(ws + l.keys_sorted),
+                       reinterpret_cast<const int32_t *>(ws + l.segment_starts),
+                       reinterpret_cast<const int32_t *>(ws + l.num_unique), unique_slots, num_indices, s);
 }

@@ -171,6 +171,11 @@ struct MixedTables {
   uint32_t bag_magic = 0;
   int32_t bag_shift = 0;
 };
+// Row width the workspace of mixed-D tables is laid out for: its partial rows hold 64 vectors, the
+// widest row that is summed in chunks (8 elements a vector at most for fp16).
+inline int32_t mixed_layout_dim(int32_t dtype) {
+  return kWave * (dtype == TBE_DTYPE_F16 ? 8 : dtype == TBE_DTYPE_F32 ? 4 : 2);
+}
 inline void set_bag_division(MixedTables &mt) {
   int log2_T = 0;
   while ((int64_t{1} << log2_T) < mt.T) ++log2_T;
@@ -181,14 +186,15 @@ inline void set_bag_division(MixedTables &mt) {
 // The approximate row-wise Adagrad update (one lookup at a time per row, in position order) on a
 // workspace that holds the batch's plan.  Uniform tables: D > 0 and the mixed_* pointers null;
 // mixed-D tables: D = 0, and the strip kernel of tbe_backward_mixed has already applied the rows
-// of few occurrences and filled the two queues above.  unique_slots / cache_rows (uniform tables
-// behind the row cache): every row is updated where it lives, as in segment_update.
+// of few occurrences and filled the two queues above.  unique_slots / cache_rows (tables behind the
+// row cache; slot_D: the width of a cache row, for mixed-D tables): every row is updated where it
+// lives, as in segment_update.
 int approx_update(const void *grad_output, void *weights, void *state, const void *psw, void *grad_psw,
                   int32_t dtype, int32_t fp16_vector_width, int32_t D, int64_t n, float lr, float eps,
                   const int64_t *mixed_table_offsets, const int32_t *table_dim_offsets,
                   const int32_t *dim_offsets, int32_t total_D, int32_t T, const int32_t *offsets, int32_t B,
                   StochasticRounding sr, const tbe_workspace_layout_t &l, void *workspace, hipStream_t stream,
-                  const int32_t *unique_slots = nullptr, void *cache_rows = nullptr);
+                  const int32_t *unique_slots = nullptr, void *cache_rows = nullptr, int32_t slot_D = 0);
 
 // Where the approximate update of mixed-D tables keeps its two queues of unique-row indices inside
 // the backward workspace: rows of at most 64 vectors with more occurrences than the strip kernel

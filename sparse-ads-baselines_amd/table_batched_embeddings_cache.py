@@ -25,6 +25,7 @@ import torch
 
 import tbe_native as _native
 from table_batched_embeddings import max_table_rows as _max_table_rows
+from table_batched_embeddings import _fp16_vector_width
 
 _DTYPE_CODES = {torch.float32: _native.DTYPE_F32, torch.float16: _native.DTYPE_F16,
                 torch.float64: _native.DTYPE_F64}
@@ -47,11 +48,35 @@ class _Plan:
         self.__dict__.update(kw)
 
 
+class MixedTables:
+    """Tables of different widths behind one cache (the layout of MixedDimTableBatchedEmbeddingBags,
+    table_batched_embeddings_ops.py:324-379): table_offsets int64 [T+1] (first element of each table in
+    the 1-D weights), table_dim_offsets int32 [T+1] (first global row id of each table), dim_offsets
+    int32 [T+1] (first output column of each table), all on the weights' device."""
+
+    def __init__(self, table_offsets, table_dim_offsets, dim_offsets):
+        self.table_offsets = table_offsets
+        self.table_dim_offsets = table_dim_offsets
+        self.dim_offsets = dim_offsets
+        self.T = dim_offsets.numel() - 1
+        dims = dim_offsets.cpu().tolist()
+        self.total_D = dims[-1]
+        self.widest = max(b - a for a, b in zip(dims, dims[1:]))
+        self.total_rows = int(table_dim_offsets[-1])
+        # what prepare() / prefetch() / forward() take as `table_offsets`: the first row of each table
+        self.table_rows = table_dim_offsets[:self.T]
+        self.vector_width = _fp16_vector_width(dim_offsets)
+
+
 class RowCache:
-    def __init__(self, backing_weights, cache_slots, policy="lru", stage_slots=0, deferred_write_back=True):
+    def __init__(self, backing_weights, cache_slots, policy="lru", stage_slots=0, deferred_write_back=True,
+                 mixed=None):
         """backing_weights: [rows, D] tensor whose storage is device-visible host memory
         (table_batched_embeddings.new_host_mapped_tensor) -- or plain device memory, which is
-        useful for tests.  cache_slots is rounded down to a multiple of 64 (one set).
+        useful for tests.  With tables of different widths (mixed: a MixedTables) it is their 1-D
+        weights; a cache row then has the widest table's width, of which a narrower row uses the
+        front.
+        cache_slots is rounded down to a multiple of 64 (one set).
         stage_slots: rows of HBM that hold, for one step, the rows no slot could take (every way
         of their set already serves the step): they then cross the host link once per step and
         direction instead of once per lookup.  Sized for the misses of a step it stages them all.
@@ -63,11 +88,20 @@ class RowCache:
         staging areas and four bytes per row of the table in HBM."""
         if policy not in _POLICIES:
             raise ValueError("cache policy must be 'lru' or 'lfu'")
-        if not backing_weights.is_cuda or backing_weights.dim() != 2 or not backing_weights.is_contiguous():
-            raise RuntimeError("backing_weights must be a contiguous [rows, D] GPU-visible tensor")
+        self.mixed = mixed
+        if mixed is None:
+            if not backing_weights.is_cuda or backing_weights.dim() != 2 or not backing_weights.is_contiguous():
+                raise RuntimeError("backing_weights must be a contiguous [rows, D] GPU-visible tensor")
+            self.D = backing_weights.size(1)
+            self.total_rows = backing_weights.size(0)
+        else:
+            if not backing_weights.is_cuda or backing_weights.dim() != 1 or not backing_weights.is_contiguous():
+                raise RuntimeError("backing_weights of tables of different widths must be a contiguous 1-D "
+                                   "GPU-visible tensor")
+            self.D = mixed.widest
+            self.total_rows = mixed.total_rows
         self.device = backing_weights.device
         self.backing = backing_weights
-        self.D = backing_weights.size(1)
         self.dtype_code = _DTYPE_CODES[backing_weights.dtype]
         self.num_sets = int(cache_slots) // _native.CACHE_WAYS
         if self.num_sets < 1:
@@ -86,11 +120,16 @@ class RowCache:
                                 device=self.device)
         self.stage_of_row = self.stage_keys = None
         if self.deferred_write_back:
-            self.stage_of_row = torch.empty(backing_weights.size(0), dtype=torch.int32, device=self.device)
+            self.stage_of_row = torch.empty(self.total_rows, dtype=torch.int32, device=self.device)
             self.stage_keys = torch.empty(STAGE_AREAS * self.stage_slots, dtype=torch.int32, device=self.device)
         self.handle = _native.Cache(_ptr(self.tags), _ptr(self.last_used), _ptr(self.use_count), _ptr(self.rows),
                                     _ptr(self.backing), self.num_sets, _POLICIES[policy], self.stage_slots,
-                                    _ptr(self.stage_of_row), _ptr(self.stage_keys), backing_weights.size(0))
+                                    _ptr(self.stage_of_row), _ptr(self.stage_keys), self.total_rows)
+        if mixed is not None:
+            self.handle.mixed_table_offsets = _ptr(mixed.table_offsets)
+            self.handle.mixed_table_rows = _ptr(mixed.table_dim_offsets)
+            self.handle.mixed_dim_offsets = _ptr(mixed.dim_offsets)
+            self.handle.mixed_T = mixed.T
         # default priority, both: the link stream carries the row traffic over the host link, the
         # plan stream the decisions of a prefetched batch
         self.link_stream = torch.cuda.Stream(device=self.device)
@@ -137,6 +176,9 @@ class RowCache:
         T = table_offsets.numel()
         B = (offsets.numel() - 1) // T
         n = indices.numel()
+        if self.mixed is not None and T != self.mixed.T:
+            raise RuntimeError("table_offsets must be the first row of each of the cache's %d tables "
+                               "(MixedTables.table_rows)" % self.mixed.T)
         which = (self.sequence + 1) % 2
         old = self._slots[which]
         if old is not None and old.state in (_Plan.PREFETCHED, _Plan.COMMITTED):
@@ -147,7 +189,10 @@ class RowCache:
         self.step += 1
         self.sequence += 1
         self._next_plan_id += 1
-        plan_layout = _native.backward_workspace_layout(n, self.D, self.dtype_code, T)
+        if self.mixed is not None:
+            plan_layout = _native.backward_mixed_workspace_layout(n, self.dtype_code, T)
+        else:
+            plan_layout = _native.backward_workspace_layout(n, self.D, self.dtype_code, T)
         layout = _native.cache_workspace_layout(n, self.num_sets, self.stage_slots)
         self._ws[which] = self._grow(self._ws[which], plan_layout.total_bytes)
         self._cws[which] = self._grow(self._cws[which], layout.total_bytes)
@@ -157,8 +202,8 @@ class RowCache:
                      state=_Plan.PREFETCHED)
         self._slots[which] = plan
         lib = _native.load()
-        args = (ctypes.byref(self.handle), self.dtype_code, self.backing.size(0),
-                _max_table_rows(table_offsets, self.backing.size(0)), self.D, _ptr(table_offsets), T, _ptr(indices), n,
+        args = (ctypes.byref(self.handle), self.dtype_code, self.total_rows,
+                _max_table_rows(table_offsets, self.total_rows), self.D, _ptr(table_offsets), T, _ptr(indices), n,
                 _ptr(offsets), B, plan.step, plan.sequence, _ptr(plan.ws), plan.ws.numel(), _ptr(plan.cws),
                 plan.cws.numel())
         with torch.cuda.device(self.device):
@@ -264,8 +309,16 @@ class RowCache:
     # ---------------------------------------------------------------- arithmetic
     def forward(self, table_offsets, indices, offsets, per_sample_weights=None):
         p = self._require_current()
-        output = torch.empty((p.B, p.T, self.D), dtype=self.backing.dtype, device=self.device)
         slots = self.lookup_slots if p.n else None
+        if self.mixed is not None:
+            output = torch.empty((p.B, self.mixed.total_D), dtype=self.backing.dtype, device=self.device)
+            with torch.cuda.device(self.device):
+                _native.check(_native.load().tbe_forward_mixed_cached(
+                    ctypes.byref(self.handle), self.dtype_code, self.mixed.vector_width, self.D, self.mixed.total_D,
+                    _ptr(indices), p.n, _ptr(offsets), p.B, _ptr(per_sample_weights), _ptr(slots), _ptr(output),
+                    self._stream()))
+            return output
+        output = torch.empty((p.B, p.T, self.D), dtype=self.backing.dtype, device=self.device)
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_forward_cached(
                 ctypes.byref(self.handle), self.dtype_code, self.D, _ptr(table_offsets), p.T, _ptr(indices), p.n,
@@ -289,24 +342,37 @@ class RowCache:
                 "backward before the next forward" % (plan_id, self.plan_id))
         if p.state == _Plan.DONE:
             raise RuntimeError("this batch's backward has already run; its plan serves one update")
+        shape = (p.B, p.T, self.D) if self.mixed is None else (p.B, self.mixed.total_D)
         if (grad_output.dtype != self.backing.dtype or grad_output.device != self.device
-                or tuple(grad_output.shape) != (p.B, p.T, self.D)):
-            raise RuntimeError("grad_output must be [B=%d, T=%d, D=%d] of %s on %s (got %s of %s)"
-                               % (p.B, p.T, self.D, self.backing.dtype, self.device,
-                                  tuple(grad_output.shape), grad_output.dtype))
+                or tuple(grad_output.shape) != shape):
+            raise RuntimeError("grad_output must be %s of %s on %s (got %s of %s)"
+                               % (shape, self.backing.dtype, self.device, tuple(grad_output.shape), grad_output.dtype))
+        if optimizer not in ("sgd", "adagrad", "approx_adagrad"):
+            raise ValueError("optimizer must be 'sgd', 'adagrad' or 'approx_adagrad' (got %r)" % (optimizer,))
         p.state = _Plan.DONE
         grad_output = grad_output.contiguous()
         grad_psw = None
         if per_sample_weights is not None:
             grad_psw = torch.empty(p.n, dtype=grad_output.dtype, device=self.device)
-        if optimizer not in ("sgd", "adagrad", "approx_adagrad"):
-            raise ValueError("optimizer must be 'sgd', 'adagrad' or 'approx_adagrad' (got %r)" % (optimizer,))
         code = _native.OPT_SGD if optimizer == "sgd" else _native.OPT_ROWWISE_ADAGRAD
         unique = self._view(p.cws, p.layout.unique_slots, max(p.n, 1))
+        if self.mixed is not None:
+            if optimizer == "approx_adagrad":
+                code = _native.OPT_APPROX_ROWWISE_ADAGRAD
+            with torch.cuda.device(self.device):
+                _native.check(_native.load().tbe_backward_mixed_cached(
+                    code, _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.mixed.vector_width,
+                    self.D, self.mixed.total_D, p.B, p.n, _ptr(p.offsets), _ptr(per_sample_weights),
+                    _ptr(optimizer_state) if optimizer != "sgd" else ctypes.c_void_p(0), float(learning_rate),
+                    float(eps or 0.0), _ptr(grad_psw), int(stochastic_rounding is not None),
+                    stochastic_rounding[0] if stochastic_rounding else 0,
+                    stochastic_rounding[1] if stochastic_rounding else 0, _ptr(p.ws), p.ws.numel(), _ptr(unique),
+                    self._stream()))
+            return grad_psw
         if optimizer == "approx_adagrad":
             with torch.cuda.device(self.device):
                 _native.check(_native.load().tbe_backward_approx_cached(
-                    _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.backing.size(0), self.D,
+                    _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.total_rows, self.D,
                     p.T, p.B, p.n, _ptr(p.offsets), _ptr(per_sample_weights), _ptr(optimizer_state),
                     float(learning_rate), float(eps or 0.0), _ptr(grad_psw), int(stochastic_rounding is not None),
                     stochastic_rounding[0] if stochastic_rounding else 0,
@@ -315,7 +381,7 @@ class RowCache:
             return grad_psw
         with torch.cuda.device(self.device):
             _native.check(_native.load().tbe_backward_cached(
-                code, _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.backing.size(0), self.D,
+                code, _ptr(grad_output), ctypes.byref(self.handle), self.dtype_code, self.total_rows, self.D,
                 p.T, p.B, p.n, _ptr(per_sample_weights),
                 _ptr(optimizer_state) if optimizer != "sgd" else ctypes.c_void_p(0), float(learning_rate),
                 float(eps or 0.0), _ptr(grad_psw), int(stochastic_rounding is not None),

@@ -125,11 +125,12 @@ class CachedLookupFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, weights, module, indices, offsets, per_sample_weights):
         cache = module.row_cache
-        cache.prepare(module.table_offsets, indices, offsets)
+        first_rows = module.cache_table_rows()
+        cache.prepare(first_rows, indices, offsets)
         ctx.module = module
         ctx.plan_id = cache.plan_id
         ctx.save_for_backward(weights, per_sample_weights)
-        return cache.forward(module.table_offsets, indices, offsets, per_sample_weights)
+        return cache.forward(first_rows, indices, offsets, per_sample_weights)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -151,7 +152,7 @@ class CachedLookupFunction(torch.autograd.Function):
         empty_grad = None
         if ctx.needs_input_grad[0]:
             empty_grad = torch.sparse_coo_tensor(
-                torch.empty((2, 0), dtype=torch.int64, device=weights.device),
+                torch.empty((weights.dim(), 0), dtype=torch.int64, device=weights.device),
                 torch.empty((0,), dtype=weights.dtype, device=weights.device), size=tuple(weights.shape))
         return (empty_grad, None, None, None, grad_per_sample_weight)
 
@@ -208,6 +209,10 @@ class TableBatchedEmbeddingBags(nn.Module):
         self.eps = eps
         self.stochastic_rounding = stochastic_rounding
 
+    def cache_table_rows(self):
+        """First row of each table, as the row cache's calls take it."""
+        return self.table_offsets
+
     def flush_cache(self):
         """Writes the rows held by the HBM cache back to embedding_weights (no-op without a cache)."""
         if self.row_cache is not None:
@@ -228,7 +233,7 @@ class TableBatchedEmbeddingBags(nn.Module):
         host-resident tables are read over the bus on every lookup.)"""
         if self.row_cache is None:
             raise RuntimeError("prefetch is for tables behind the row cache (managed=EmbeddingLocation.HOST_CACHED)")
-        self.row_cache.prefetch(self.table_offsets, sharded_sparse_features, sharded_offsets)
+        self.row_cache.prefetch(self.cache_table_rows(), sharded_sparse_features, sharded_offsets)
 
     def forward(self, sharded_sparse_features, sharded_offsets, per_sample_weights=None):
         if self.row_cache is not None:
@@ -288,9 +293,13 @@ class MixedDimTableBatchedEmbeddingBags(nn.Module):
     `embeddings` is a list of (rows, dim) per table; weights are one flat 1-D parameter."""
 
     def __init__(self, embeddings, optimizer=Optimizer.SGD, learning_rate=0.01, eps=None,
-                 stochastic_rounding=False, fp16=False, managed=EmbeddingLocation.DEVICE):
+                 stochastic_rounding=False, fp16=False, managed=EmbeddingLocation.DEVICE, cache_slots=None,
+                 cache_policy="lru", cache_stage_slots=0, cache_deferred_write_back=True):
+        """managed=EmbeddingLocation.HOST_CACHED (an extension, like that of TableBatchedEmbeddingBags):
+        the tables live in pinned host memory behind an HBM row cache of cache_slots rows of the widest
+        table's width."""
         super(MixedDimTableBatchedEmbeddingBags, self).__init__()
-        assert managed in (EmbeddingLocation.DEVICE, EmbeddingLocation.HOST_MAPPED)
+        assert managed in (EmbeddingLocation.DEVICE, EmbeddingLocation.HOST_MAPPED, EmbeddingLocation.HOST_CACHED)
         rows, dims = zip(*embeddings)
         assert all(d > 0 and d % 4 == 0 for d in dims), "every embedding dimension must be a multiple of 4"
         numel = sum(row * dim for (row, dim) in embeddings)
@@ -299,9 +308,14 @@ class MixedDimTableBatchedEmbeddingBags(nn.Module):
         if managed == EmbeddingLocation.DEVICE:
             logging.info("Allocating device embedding bag")
             embedding_data = torch.randn(size=(numel,), device=device, dtype=dtype)
-        else:
+        elif managed == EmbeddingLocation.HOST_MAPPED:
             logging.info("Allocating host-mapped embedding bag")
             embedding_data = extension.new_managed_tensor(
+                torch.empty(1, device=device, dtype=dtype), (numel,))
+            embedding_data.normal_()
+        else:
+            logging.info("Allocating pinned host embedding bag behind an HBM row cache")
+            embedding_data = extension.new_host_mapped_tensor(
                 torch.empty(1, device=device, dtype=dtype), (numel,))
             embedding_data.normal_()
         self.embedding_weights = nn.Parameter(embedding_data)
@@ -315,8 +329,43 @@ class MixedDimTableBatchedEmbeddingBags(nn.Module):
         self.learning_rate = learning_rate
         self.eps = eps
         self.stochastic_rounding = stochastic_rounding
+        self.row_cache = None
+        if managed == EmbeddingLocation.HOST_CACHED:
+            assert cache_slots is not None, "HOST_CACHED needs cache_slots"
+            self.to(device)  # the cache keeps the addresses of the three offset buffers
+            self.row_cache = table_batched_embeddings_cache.RowCache(
+                self.embedding_weights.data, cache_slots, cache_policy, cache_stage_slots, cache_deferred_write_back,
+                mixed=table_batched_embeddings_cache.MixedTables(self.table_offsets, self.table_dim_offsets,
+                                                                 self.dim_offsets))
+            # (as for TableBatchedEmbeddingBags: checkpoints see the cached rows, a loaded one is not shadowed)
+            self.register_state_dict_pre_hook(lambda module, prefix, keep_vars: module.flush_cache())
+            self.register_load_state_dict_pre_hook(lambda module, *args: module.invalidate_cache())
+
+    def cache_table_rows(self):
+        """First row of each table, as the row cache's calls take it."""
+        return self.row_cache.mixed.table_rows
+
+    def flush_cache(self):
+        """Writes the rows held by the HBM cache back to embedding_weights (no-op without a cache)."""
+        if self.row_cache is not None:
+            self.row_cache.flush()
+
+    def invalidate_cache(self):
+        """Writes the resident rows back, then empties the cache (see TableBatchedEmbeddingBags)."""
+        if self.row_cache is not None:
+            self.row_cache.invalidate()
+
+    def prefetch(self, sharded_sparse_features, sharded_offsets):
+        """HOST_CACHED tables: plans the NEXT batch while the current one computes (see
+        TableBatchedEmbeddingBags.prefetch)."""
+        if self.row_cache is None:
+            raise RuntimeError("prefetch is for tables behind the row cache (managed=EmbeddingLocation.HOST_CACHED)")
+        self.row_cache.prefetch(self.cache_table_rows(), sharded_sparse_features, sharded_offsets)
 
     def forward(self, sharded_sparse_features, sharded_offsets, per_sample_weights=None):
+        if self.row_cache is not None:
+            return CachedLookupFunction.apply(self.embedding_weights, self, sharded_sparse_features,
+                                              sharded_offsets, per_sample_weights)
         return MixedDimLookupFunction.apply(
             self.embedding_weights, self.table_offsets, self.table_dim_offsets, self.dim_offsets, self.total_D,
             sharded_sparse_features, sharded_offsets, per_sample_weights, self.optimizer, self.optimizer_state,

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TBE_HIP_LIBRARY") or os.path.join(_HERE, "libtbe_hip.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2
-ABI_VERSION = 21
+ABI_VERSION = 22
 
 _c_i32p = ctypes.c_void_p
 _vp = ctypes.c_void_p
@@ -59,6 +59,10 @@ class Cache(ctypes.Structure):
         ("stage_of_row", _vp),
         ("stage_keys", _vp),
         ("total_rows", _i64),
+        ("mixed_table_offsets", _vp),
+        ("mixed_table_rows", _vp),
+        ("mixed_dim_offsets", _vp),
+        ("mixed_T", _i32),
     ]
 
 
@@ -135,6 +139,10 @@ SIGNATURES = {
     "tbe_backward_approx_cached": (ctypes.c_int, [_vp, _cache_p, _i32, _i64, _i32, _i32, _i32, _i64, _c_i32p, _vp, _vp,
                                                   _f32, _f32, _vp, _i32, _u64, _u64, _vp, _u64, _c_i32p, _vp]),
     "tbe_cache_flush": (ctypes.c_int, [_cache_p, _i32, _i32, ctypes.c_uint32, _i32, _vp]),
+    "tbe_forward_mixed_cached": (ctypes.c_int, [_cache_p, _i32, _i32, _i32, _i32, _c_i32p, _i64, _c_i32p, _i32, _vp,
+                                                _c_i32p, _vp, _vp]),
+    "tbe_backward_mixed_cached": (ctypes.c_int, [_i32, _vp, _cache_p, _i32, _i32, _i32, _i32, _i32, _i64, _c_i32p, _vp,
+                                                 _vp, _f32, _f32, _vp, _i32, _u64, _u64, _vp, _u64, _c_i32p, _vp]),
     "tbe_host_mapped_alloc": (ctypes.c_int, [_u64, ctypes.POINTER(_vp), ctypes.POINTER(_vp)]),
     "tbe_host_mapped_free": (ctypes.c_int, [_vp]),
     "tbe_managed_alloc": (ctypes.c_int, [_u64, _i32, ctypes.POINTER(_vp)]),

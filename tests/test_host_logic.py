@@ -95,8 +95,10 @@ def test_mixed_d_signatures_match_the_pybind_declarations():
         "offsets", "indice_weights", "optimizer_state", "learning_rate", "eps", "L_max", "stochastic_rounding",
         "BT_block_size"]
     params = inspect.signature(ops.MixedDimTableBatchedEmbeddingBags.__init__).parameters
+    # (the reference's arguments first; the row cache's, an extension, behind them with defaults)
     assert list(params)[1:] == ["embeddings", "optimizer", "learning_rate", "eps", "stochastic_rounding", "fp16",
-                                "managed"]
+                                "managed", "cache_slots", "cache_policy", "cache_stage_slots",
+                                "cache_deferred_write_back"]
     for helper in ("split_embedding_weights", "split_optimizer_state", "split_output"):
         assert callable(getattr(ops.MixedDimTableBatchedEmbeddingBags, helper))
 

@@ -95,7 +95,8 @@ def test_static_scratch_backward_allocates_nothing():
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(w_graph, w_eager)
-    assert torch.cuda.mem_get_info()[0] <= free_before  # (the graph object itself may hold memory)
+    # (free memory is not compared again here: entering torch.cuda.graph collects garbage and empties
+    # torch's cache, and the graph object itself may hold memory)
 
 
 def test_static_scratch_backward_fp16_and_empty_batch():
