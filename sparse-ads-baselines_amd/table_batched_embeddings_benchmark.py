@@ -1,13 +1,20 @@
 """Micro-benchmark CLI with the flags of the reference's table_batched_embeddings_benchmark.py
 (:360-370): --num-tables 64 --num-embeddings 10000 --embedding-dim 32 --batch-size 128
 --bag-size 32 --iters 100 [--fp16] [--managed] [--mixed] [--remote], plus --alpha / --seed / --kernels /
---compiled.
+--compiled / --cache-slots.
 
 Each operator is called directly on the extension-module mirror (not through autograd), after
 one warm-up call, `iters` times between two events on the current stream
 (table_batched_embeddings_benchmark.py:27-37).  "BW" is the reference's figure:
 elem * B * T * L * D / time for forward (:240) and twice that for backward (:356).  One JSON
 object per measurement goes to stdout.
+
+--cache-slots N (no counterpart in the reference): the tables live in pinned host memory behind an
+HBM row cache of N rows (EmbeddingLocation.HOST_CACHED) and the rows printed are the cache's plan
+for a batch (sort, slots, row traffic), the forward through it, and plan + update per optimizer
+-- a plan serves one update.  Every call sees the same batch, so from the second call on the rows
+the cache can hold are resident: with N at least the batch's unique rows this times the kernels'
+way through the slots, with fewer the host link as well.
 """
 import json
 import logging
@@ -70,18 +77,43 @@ def report(name, seconds, bytes_moved, shape):
     print(json.dumps(record))
 
 
-def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
+def run_cached(cc, indices, offsets, iters, fwd_bytes, shape):
+    """The rows of --cache-slots: plan, forward and plan + update through the module's row cache."""
+    cache = cc.row_cache
+    first_rows = cc.cache_table_rows()
+    lr, eps = 0.05, 0.01
+    plan = lambda: cache.prepare(first_rows, indices, offsets)
+    plan()
+    y0 = cache.forward(first_rows, indices, offsets)
+    go = torch.randn_like(y0)
+    report("Cached-Plan", time_calls(iters, plan), 0.0, shape)
+    report("Cached-Forward", time_calls(iters, lambda: cache.forward(first_rows, indices, offsets)), fwd_bytes, shape)
+    for name, kind in (("SGD-EXACT", "sgd"), ("ADAGRAD-nonstochastic-APPROX-NR", "approx_adagrad"),
+                       ("ADAGRAD-nonstochastic-EXACT-NR", "adagrad")):
+        def step():
+            plan()
+            cache.backward(kind, go, None, cc.optimizer_state, lr, eps)
+        report("Cached-Plan+Backward-" + name, time_calls(iters, step), 2 * fwd_bytes, shape)
+    logging.info("cache after the last plan: %s", cache.stats())
+
+
+def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed, cache_slots=0):
     rs = np.random.RandomState(seed)
     location = ops.EmbeddingLocation.HOST_MAPPED if managed else ops.EmbeddingLocation.DEVICE
+    cache_args = {}
+    if cache_slots:
+        location = ops.EmbeddingLocation.HOST_CACHED
+        cache_args = dict(cache_slots=cache_slots, cache_stage_slots=T * B * L)
     elem = 2 if fp16 else 4
     if mixed:
         dims = [int((rs.randint(int(0.5 * D), int(1.5 * D) + 1) + 3) // 4 * 4) for _ in range(T)]
         cc = ops.MixedDimTableBatchedEmbeddingBags([(E, d) for d in dims], optimizer=ops.Optimizer.EXACT_ROWWISE_ADAGRAD,
-                                                   learning_rate=0.1, eps=0.1, fp16=fp16, managed=location).cuda()
+                                                   learning_rate=0.1, eps=0.1, fp16=fp16, managed=location,
+                                                   **cache_args).cuda()
         D_eff = float(np.mean(dims))
     else:
         cc = ops.TableBatchedEmbeddingBags(T, E, D, optimizer=ops.Optimizer.EXACT_ROWWISE_ADAGRAD, learning_rate=0.1,
-                                           eps=0.1, fp16=fp16, managed=location).cuda()
+                                           eps=0.1, fp16=fp16, managed=location, **cache_args).cuda()
         D_eff = D
     logging.info("Embedding parameters: %.2fGParam", cc.embedding_weights.numel() / 1.0e9)
     indices, offsets = draw_indices(rs, T, B, L, [E] * T, alpha)
@@ -90,6 +122,9 @@ def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
     shape = dict(B=B, E=E, T=T, D=D_eff, L=L, fp16=fp16, managed=managed, mixed=mixed, alpha=alpha)
     w = cc.embedding_weights.data
     fwd_bytes = elem * B * T * L * D_eff
+    if cache_slots:
+        shape["cache_slots"] = cache_slots
+        return run_cached(cc, indices, offsets, iters, fwd_bytes, shape)
 
     if mixed:
         fwd = lambda: EXT.forward_mixed_D(
@@ -156,8 +191,9 @@ def run(B, E, T, L, D, iters, fp16, managed, mixed, alpha, seed):
 @click.option("--seed", default=42)
 @click.option("--compiled", is_flag=True, default=False,
               help="Call the kernels through the pybind11 module (table_batched_embeddings_cpp)")
+@click.option("--cache-slots", default=0, help="Host-resident tables behind an HBM row cache of this many rows")
 def cli(num_tables, num_embeddings, embedding_dim, batch_size, bag_size, iters, remote, fp16, managed, mixed, kernels,
-        alpha, seed, compiled):
+        alpha, seed, compiled, cache_slots):
     global KERNEL_TIMES, EXT
     KERNEL_TIMES = kernels
     if compiled:
@@ -167,7 +203,10 @@ def cli(num_tables, num_embeddings, embedding_dim, batch_size, bag_size, iters, 
     logging.basicConfig(level=logging.INFO, stream=sys.stderr)
     if remote:
         raise click.UsageError("--remote (cluster submission) is not available; run the benchmark locally")
-    run(batch_size, num_embeddings, num_tables, bag_size, embedding_dim, iters, fp16, managed, mixed, alpha, seed)
+    if cache_slots and (managed or compiled):
+        raise click.UsageError("--cache-slots goes with neither --managed nor --compiled")
+    run(batch_size, num_embeddings, num_tables, bag_size, embedding_dim, iters, fp16, managed, mixed, alpha, seed,
+        cache_slots)
 
 
 if __name__ == "__main__":

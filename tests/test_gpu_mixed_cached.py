@@ -342,3 +342,23 @@ def test_mixed_cached_bad_arguments_and_empty_batch():
         cache.backward("adam", torch.zeros(4, 40, device=DEV), None, torch.zeros(37, device=DEV), 0.1, 0.1)
     cache.backward("approx_adagrad", torch.zeros(4, 40, device=DEV), None, torch.zeros(37, device=DEV), 0.1, 0.1)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("mixed", [False, True])
+def test_benchmark_cli_times_the_way_through_the_cache(mixed):
+    """--cache-slots on the micro-benchmark: host-resident tables (uniform or mixed-D) behind the cache."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from conftest import PACKAGE
+    cmd = [sys.executable, os.path.join(PACKAGE, "table_batched_embeddings_benchmark.py"), "--num-tables", "4",
+           "--num-embeddings", "1000", "--embedding-dim", "32", "--batch-size", "64", "--bag-size", "8", "--iters",
+           "3", "--cache-slots", "1024"] + (["--mixed"] if mixed else [])
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=280)
+    assert out.returncode == 0, out.stderr[-2000:]
+    records = [json.loads(line) for line in out.stdout.splitlines() if line.startswith("{")]
+    assert [r["op"] for r in records] == [
+        "Cached-Plan", "Cached-Forward", "Cached-Plan+Backward-SGD-EXACT",
+        "Cached-Plan+Backward-ADAGRAD-nonstochastic-APPROX-NR", "Cached-Plan+Backward-ADAGRAD-nonstochastic-EXACT-NR"]
+    assert all(r["time_us"] > 0 and r["cache_slots"] == 1024 and r["mixed"] == mixed for r in records)
