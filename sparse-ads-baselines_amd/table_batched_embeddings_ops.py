@@ -157,7 +157,31 @@ class CachedLookupFunction(torch.autograd.Function):
         return (empty_grad, None, None, None, grad_per_sample_weight)
 
 
-class TableBatchedEmbeddingBags(nn.Module):
+class _CacheFronted:
+    """What the two modules share when their tables sit behind a row cache: the cache keeps device
+    addresses (the pinned table, and for mixed-D tables the three offset buffers), so a call that
+    moves or casts them (.to(other), .half(), .double()) is refused instead of leaving the cache
+    pointing at freed memory."""
+
+    def _cache_anchors(self):
+        cache = getattr(self, "row_cache", None)
+        if cache is None:
+            return None
+        anchors = [self.embedding_weights.data_ptr(), self.embedding_weights.dtype]
+        if cache.mixed is not None:
+            anchors += [self.table_offsets.data_ptr(), self.table_dim_offsets.data_ptr(), self.dim_offsets.data_ptr()]
+        return anchors
+
+    def _apply(self, fn, *args, **kwargs):
+        before = self._cache_anchors()
+        out = super()._apply(fn, *args, **kwargs)
+        if before is not None and before != self._cache_anchors():
+            raise RuntimeError("a module whose tables sit behind the row cache (EmbeddingLocation.HOST_CACHED) cannot "
+                               "be moved to another device or cast: the cache holds the addresses of its tensors")
+        return out
+
+
+class TableBatchedEmbeddingBags(_CacheFronted, nn.Module):
     """Mirror of TableBatchedEmbeddingBags (table_batched_embeddings_ops.py:135-201)."""
 
     def __init__(self, num_tables, num_embeddings, embedding_dim, optimizer=Optimizer.SGD,
@@ -288,7 +312,7 @@ class MixedDimLookupFunction(torch.autograd.Function):
                 None)
 
 
-class MixedDimTableBatchedEmbeddingBags(nn.Module):
+class MixedDimTableBatchedEmbeddingBags(_CacheFronted, nn.Module):
     """Mirror of MixedDimTableBatchedEmbeddingBags (table_batched_embeddings_ops.py:324-435):
     `embeddings` is a list of (rows, dim) per table; weights are one flat 1-D parameter."""
 

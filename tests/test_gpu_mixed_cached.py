@@ -362,3 +362,17 @@ def test_benchmark_cli_times_the_way_through_the_cache(mixed):
         "Cached-Plan", "Cached-Forward", "Cached-Plan+Backward-SGD-EXACT",
         "Cached-Plan+Backward-ADAGRAD-nonstochastic-APPROX-NR", "Cached-Plan+Backward-ADAGRAD-nonstochastic-EXACT-NR"]
     assert all(r["time_us"] > 0 and r["cache_slots"] == 1024 and r["mixed"] == mixed for r in records)
+
+
+def test_cache_fronted_modules_refuse_to_be_moved_or_cast():
+    """The cache keeps the addresses of the pinned table (and of the mixed-D offset buffers): .cuda() on
+    the device they are on is a no-op and fine, a cast is refused loudly."""
+    uniform = ops.TableBatchedEmbeddingBags(2, 50, 16, managed=ops.EmbeddingLocation.HOST_CACHED, cache_slots=64).cuda()
+    mixed = ops.MixedDimTableBatchedEmbeddingBags([(50, 16), (20, 8)], managed=ops.EmbeddingLocation.HOST_CACHED,
+                                                  cache_slots=64).cuda()
+    assert mixed.cuda() is mixed and uniform.cuda() is uniform
+    for module in (uniform, mixed):
+        with pytest.raises(RuntimeError, match="cannot be moved to another device or cast"):
+            module.half()
+    plain = ops.MixedDimTableBatchedEmbeddingBags([(50, 16), (20, 8)]).cuda()
+    assert plain.half().embedding_weights.dtype == torch.float16   # (tables in device memory cast as ever)
