@@ -376,3 +376,50 @@ def test_cache_fronted_modules_refuse_to_be_moved_or_cast():
             module.half()
     plain = ops.MixedDimTableBatchedEmbeddingBags([(50, 16), (20, 8)]).cuda()
     assert plain.half().embedding_weights.dtype == torch.float16   # (tables in device memory cast as ever)
+
+
+def test_cached_mixed_training_at_the_benchmark_shape_equals_uncached():
+    """64 tables of 100 000 rows, widths 64..192, 5.2 M lookups per step (the mixed-D micro-benchmark's
+    shape): three steps of exact Adagrad through a cache a sixth the size of a step's unique rows, every
+    batch planned ahead, against the same steps on tables in device memory, bit for bit."""
+    if torch.cuda.mem_get_info()[0] < 24 << 30:
+        pytest.skip("needs 24 GB of free device memory")
+    rs = np.random.RandomState(3)
+    T, E, B, L = 64, 100000, 4096, 20
+    tables = [(E, int((rs.randint(64, 193) + 3) // 4 * 4)) for _ in range(T)]
+    table_offsets, table_dim_offsets, dim_offsets = _tables_on_device(tables)
+    total_D = sum(d for _, d in tables)
+    numel = sum(r * d for r, d in tables)
+    start = torch.rand(numel, device=DEV) * 0.02 - 0.01
+    plain_w = start.clone()
+    cached_w = ext.new_host_mapped_tensor(torch.empty(1, device=DEV), (numel,))
+    cached_w.copy_(start)
+    del start
+    plain_state = torch.zeros(T * E, device=DEV)
+    cached_state = torch.zeros(T * E, device=DEV)
+    mixed = tc.MixedTables(table_offsets, table_dim_offsets, dim_offsets)
+    cache = tc.RowCache(cached_w, 1 << 19, "lru", 1 << 22, mixed=mixed)
+    offsets = dev(np.arange(0, T * B * L + 1, L, dtype=np.int32))
+    batches = [torch.from_numpy((rs.zipf(1.05, size=T * B * L) % E).astype(np.int32)).to(DEV) for _ in range(3)]
+    go = torch.randn(B, total_D, device=DEV)
+    cache.prefetch(mixed.table_rows, batches[0], offsets)
+    staged = 0
+    for i, idx in enumerate(batches):
+        if i + 1 < len(batches):
+            cache.prefetch(mixed.table_rows, batches[i + 1], offsets)
+        want = ext.forward_mixed_D(plain_w, table_offsets, dim_offsets, total_D, idx, offsets, None, 200, 1, False)
+        ext.backward_exact_adagrad_mixed_D(go, plain_w, table_offsets, table_dim_offsets, dim_offsets, total_D, idx,
+                                           offsets, None, plain_state, 0.05, 0.1, False, 1)
+        cache.prepare(mixed.table_rows, idx, offsets)
+        got = cache.forward(mixed.table_rows, idx, offsets)
+        cache.backward("adagrad", go, None, cached_state, 0.05, 0.1)
+        assert torch.equal(got, want), "forward output differs at step %d" % i
+        st = cache.stats()
+        assert st["uncached"] == 0
+        staged += st["staged"]
+    assert staged > 1 << 20
+    cache.flush()
+    torch.cuda.synchronize()
+    assert torch.equal(cached_w, plain_w)
+    assert torch.equal(cached_state, plain_state)
+    ext.free_host_tensor(cached_w)
