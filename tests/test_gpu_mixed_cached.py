@@ -423,3 +423,73 @@ def test_cached_mixed_training_at_the_benchmark_shape_equals_uncached():
     assert torch.equal(cached_w, plain_w)
     assert torch.equal(cached_state, plain_state)
     ext.free_host_tensor(cached_w)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_cached_mixed_training_random_sweep(seed):
+    """Seeded random shapes of the cached-equals-uncached property for tables of different widths:
+    1..40 tables (the bisection that finds a key's table), tables of a few rows and of thousands,
+    widths from one vector to more than 64, dtype, optimizer (approximate Adagrad included), policy,
+    cache and staging sizes from "nearly everything misses" to "everything fits", write-back deferred
+    or not, batches planned ahead or not, index skew."""
+    rs = np.random.RandomState(900 + seed)
+    T = int(rs.choice([1, 2, 7, 40]))
+    dtype = [torch.float32, torch.float16, torch.float64][seed % 3]
+    widths = [4, 8, 12, 32, 64, 100, 128, 260, 520]
+    tables = [(int(rs.choice([1, 3, 60, 900, 4000])), int(rs.choice(widths))) for _ in range(T)]
+    mode = ["sgd", "adagrad", "adagrad_weighted", "approx", "approx_weighted"][(seed // 3) % 5]
+    policy = ["lru", "lfu"][seed % 2]
+    num_sets = int(rs.choice([1, 3, 17, 200]))
+    stage_slots = int(rs.choice([0, 5, 300, 100000]))
+    deferred = bool(rs.randint(2))
+    B, L, zipf = int(rs.choice([1, 30, 200])), int(rs.choice([1, 6, 25])), float(rs.choice([1.05, 1.3, 2.0]))
+    table_offsets, table_dim_offsets, dim_offsets = _tables_on_device(tables)
+    total_D = sum(d for _, d in tables)
+    total_rows = sum(r for r, _ in tables)
+    numel = sum(r * d for r, d in tables)
+    start = (torch.rand(numel, device=DEV, dtype=torch.float64) * 0.02 - 0.01).to(dtype)
+    plain_w = start.clone()
+    cached_w = ext.new_host_mapped_tensor(torch.empty(1, device=DEV, dtype=dtype), (numel,))
+    cached_w.copy_(start)
+    st_dtype = torch.float64 if dtype == torch.float64 else torch.float32
+    plain_state = torch.zeros(total_rows, device=DEV, dtype=st_dtype)
+    cached_state = torch.zeros(total_rows, device=DEV, dtype=st_dtype)
+    mixed = tc.MixedTables(table_offsets, table_dim_offsets, dim_offsets)
+    cache = tc.RowCache(cached_w, num_sets * 64, policy, stage_slots, deferred_write_back=deferred, mixed=mixed)
+    ahead = cache.deferred_write_back and seed % 2 == 1
+    weighted = mode.endswith("weighted")
+    opt = "sgd" if mode == "sgd" else "approx_adagrad" if mode.startswith("approx") else "adagrad"
+    batches = []
+    for _ in range(5):
+        indices, offsets = _draw_batch(rs, tables, B, L, zipf)
+        batches.append((dev(indices), dev(offsets), torch.randn(B, total_D, device=DEV, dtype=torch.float64).to(dtype),
+                        torch.rand(indices.size, device=DEV, dtype=torch.float64).to(dtype) if weighted else None))
+    if ahead:
+        cache.prefetch(mixed.table_rows, batches[0][0], batches[0][1])
+    for step, (idx, off, go, psw) in enumerate(batches):
+        if ahead and step + 1 < len(batches):
+            cache.prefetch(mixed.table_rows, batches[step + 1][0], batches[step + 1][1])
+        want = ext.forward_mixed_D(plain_w, table_offsets, dim_offsets, total_D, idx, off, psw, 200, 1, False)
+        if opt == "sgd":
+            ext.backward_sgd_mixed_D(go, plain_w, table_offsets, table_dim_offsets, dim_offsets, total_D, idx, off,
+                                     plain_state, 0.05)
+            want_g = None
+        elif opt == "approx_adagrad":
+            want_g = ext.backward_approx_adagrad_mixed_D(go, plain_w, table_offsets, table_dim_offsets, dim_offsets,
+                                                         total_D, idx, off, psw, plain_state, 0.05, 0.1, 200, False, 1)
+        else:
+            want_g = ext.backward_exact_adagrad_mixed_D(go, plain_w, table_offsets, table_dim_offsets, dim_offsets,
+                                                        total_D, idx, off, psw, plain_state, 0.05, 0.1, False, 1)
+        cache.prepare(mixed.table_rows, idx, off)
+        got = cache.forward(mixed.table_rows, idx, off, psw)
+        got_g = cache.backward(opt, go, psw, cached_state, 0.05, 0.1)
+        assert torch.equal(got, want), "forward output differs at step %d" % step
+        if weighted and idx.numel():
+            assert torch.equal(got_g, want_g)
+        resident = cache.resident_keys()
+        assert resident.numel() == torch.unique(resident).numel() <= num_sets * 64
+    cache.flush()
+    torch.cuda.synchronize()
+    assert torch.equal(cached_w, plain_w)
+    assert torch.equal(cached_state, plain_state)
+    ext.free_host_tensor(cached_w)
