@@ -406,6 +406,7 @@ __device__ __forceinline__ uint4 draw_block(const StochasticRounding &sr, int64_
 // current 32.  words[2][kCoopStep][kCoopD]: the 13 random bits of every element of the row for
 // every occurrence of a step, two steps deep.
 constexpr int kCoopD = 128;    // widest row walked this way (two elements per lane)
+static_assert(kCoopD == kApproxCoopD, "the width up to which rows are listed for a workgroup's walk");
 constexpr int kCoopStep = 32;  // occurrences per step
 // The barrier between the steps of the cooperative walk: LDS traffic of the wavefront is complete
 // (the bits written, or the bits of the finished step read), but the walking wavefront's gradient
@@ -757,6 +758,7 @@ __device__ __forceinline__ void walk_long_row(const LongRowArgs<T> &a, int seg_b
 // elements: two elements per lane, 64 occurrences a step (the same 16 KB of gradient rows).
 constexpr int kStageStep = 128;  // most occurrences per step
 constexpr int kStageD = 128;     // widest row walked this way
+static_assert(kStageD == kApproxCoopD, "the width up to which rows are listed for a workgroup's walk");
 constexpr int kStageElements = 128 * 64;  // elements of the gradient rows of one step
 template <typename T, bool WEIGHTED> struct StageBuffers {
   alignas(16) T rows[2][kStageElements];  // [occurrence of the step][element of the row]
@@ -1026,12 +1028,15 @@ __device__ __forceinline__ void staged_walk(const LongRowArgs<T> &a, int seg_beg
 template <typename T, bool WEIGHTED, bool STOCHASTIC, bool BIG>
 __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
     LongRowArgs<T> a, const int32_t *__restrict__ keys_sorted, const int32_t *__restrict__ segment_starts,
-    const int32_t *__restrict__ counters, const int32_t *__restrict__ long_queue, int queue_capacity, int D) {
+    const int32_t *__restrict__ counters, const int32_t *__restrict__ long_queue, int queue_capacity, int D,
+    int mixed_huge_offset) {
   // (what is the same in every lane of the wavefront is told to the compiler, so that the walk's
   // control flow and addressing stay scalar)
   const int lane = threadIdx.x & (kWave - 1);
   const int wave_in_block = uniform(static_cast<int>(threadIdx.x >> 6));
-  // queue_capacity == 0: one queue, its length in counters[1].  Otherwise, as the short-row kernel
+  // queue_capacity == 0: one queue, its length in counters[1] (mixed-D tables: and, from
+  // mixed_huge_offset on, the rows of more than kApproxHuge occurrences that a workgroup walks, their
+  // number in counters[xcd_counter(0)]).  Otherwise, as the short-row kernel
   // leaves them: one queue per XCD (lengths in counters[xcd_counter(x)]) and behind them the
   // queue of the rows of more than kApproxHuge occurrences (counters[1]).  Those come first, one
   // per wavefront, so that the longest walks start when the kernel does.  Then the workgroups of
@@ -1081,16 +1086,20 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
   if constexpr (STOCHASTIC || kStaged) {
     using Shared = typename std::conditional<kStaged, StageBuffers<T, WEIGHTED>, uint16_t[2 * kCoopStep * kCoopD]>::type;
     __shared__ __align__(16) Shared s_shared;
-    if (queue_capacity > 0 && a.mt.T == 0 && D <= (kStaged ? kStageD : kCoopD) && first_total > 0) {
+    // (mixed-D tables: the strip kernel has listed the rows that qualify on their own)
+    const bool mixed = a.mt.T > 0;
+    const int huge_total = mixed ? uniform(counters[xcd_counter(0)]) : first_total;
+    const int huge_base = mixed ? mixed_huge_offset : kNumXcd * queue_capacity;
+    if ((mixed || (queue_capacity > 0 && D <= kApproxCoopD)) && huge_total > 0) {
       const bool dedicated = grid_blocks >= 2 * kNumXcd;
       const int coop_blocks =
-          dedicated ? min((first_total + kNumXcd - 1) / kNumXcd * kNumXcd, grid_blocks / (2 * kNumXcd) * kNumXcd) : 0;
+          dedicated ? min((huge_total + kNumXcd - 1) / kNumXcd * kNumXcd, grid_blocks / (2 * kNumXcd) * kNumXcd) : 0;
       if (!dedicated || block_index < coop_blocks) {
         // these walks are the longest chains of the launch and share their SIMDs with the
         // wavefronts of other workgroups: they go first when both have an instruction ready
         __builtin_amdgcn_s_setprio(3);
-        for (int h = block_index; h < first_total; h += dedicated ? coop_blocks : grid_blocks) {
-          const QueuedRow r = row_at(kNumXcd * queue_capacity + h);
+        for (int h = block_index; h < huge_total; h += dedicated ? coop_blocks : grid_blocks) {
+          const QueuedRow r = row_at(huge_base + h);
           if constexpr (kStaged) {
             if (r.place.row_D <= kWave) staged_walk<T, 1, WEIGHTED>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
             else staged_walk<T, 2, WEIGHTED>(a, r.seg_begin, r.seg_end, r.key, r.place, r.storage, s_shared);
@@ -1124,7 +1133,7 @@ __global__ __launch_bounds__(kBlockThreads) void approx_adagrad_long_kernel(
       }
       block_index -= coop_blocks;
       grid_blocks -= coop_blocks;
-      first_total = 0;
+      if (!mixed) first_total = 0;
     }
   }
 
@@ -1247,7 +1256,7 @@ void launch_approx(const ApproxArgs &a, const tbe_workspace_layout_t &l, char *w
 #define TBE_APPROX_LONG_KERNEL(WEIGHTED, STOCHASTIC, BIG)                                              \
   TBE_LAUNCH("update_approx_long", stream, (approx_adagrad_long_kernel<T, WEIGHTED, STOCHASTIC, BIG>), \
              grid_long, block_long, la, i32(l.keys_sorted), i32(l.segment_starts), counters,           \
-             long_queue, queue_capacity, a.D)
+             long_queue, queue_capacity, a.D, static_cast<int>(approx_mixed_huge_offset(a.n)))
 #define TBE_APPROX_LONG(WEIGHTED, MIXED)                                                               \
   TBE_LAUNCH("update_approx_norms", stream, (approx_lookup_norms_kernel<T, VEC, WEIGHTED, MIXED>),     \
              grid_norms, block, static_cast<const T *>(a.grad_output), static_cast<const T *>(a.psw),  \

@@ -482,7 +482,8 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
     int32_t *__restrict__ counters, int32_t *__restrict__ wide_rows,
     int32_t *__restrict__ queued_rows, ChunkRecord *__restrict__ chunk_records,
     LongRecord *__restrict__ long_records, int64_t max_chunks, int64_t max_long, int positions_per_xcd,
-    float lr, float eps, StochasticRounding sr, const int32_t *__restrict__ unique_slots = nullptr,
+    float lr, float eps, StochasticRounding sr, int approx_huge_offset = 0,
+    const int32_t *__restrict__ unique_slots = nullptr,
     T *__restrict__ cache_rows = nullptr, int slot_D = 0) {
   using V = RowVec<T, VEC>;
   using A = typename V::A;
@@ -559,13 +560,26 @@ __global__ __launch_bounds__(kBlockThreads, mixed_strip_blocks(WEIGHTED, VEC == 
     const unsigned long long queued_mask = long_mask & ~wide_mask;
     if constexpr (APPROX) {
       // the per-lookup form walks a row of many occurrences in one piece: its number goes to
-      // `queued_rows` (counters[1])
-      if (queued_mask) {
+      // `queued_rows` (counters[1]) -- or, an fp16 row of more than kApproxHuge occurrences that a
+      // workgroup can walk, to the list behind that queue (counters[xcd_counter(0)])
+      bool is_huge = false;
+      if constexpr (sizeof(T) == 2) is_huge = is_long && !is_wide && l_end - l_begin > kApproxHuge && l_D <= kApproxCoopD;
+      const unsigned long long huge_mask = __ballot(is_huge);
+      const unsigned long long plain_mask = queued_mask & ~huge_mask;
+      if (plain_mask) {
         int first_slot = 0;
-        if (lane == 0) first_slot = atomicAdd(&counters[1], __popcll(queued_mask));
+        if (lane == 0) first_slot = atomicAdd(&counters[1], __popcll(plain_mask));
         first_slot = shfl_idx(first_slot, 0);
-        if (is_long && !is_wide)
-          queued_rows[first_slot + __popcll(queued_mask & ((1ull << lane) - 1ull))] = static_cast<int32_t>(my_u);
+        if (is_long && !is_wide && !is_huge)
+          queued_rows[first_slot + __popcll(plain_mask & ((1ull << lane) - 1ull))] = static_cast<int32_t>(my_u);
+      }
+      if (huge_mask) {
+        int first_slot = 0;
+        if (lane == 0) first_slot = atomicAdd(&counters[xcd_counter(0)], __popcll(huge_mask));
+        first_slot = shfl_idx(first_slot, 0);
+        if (is_huge)
+          queued_rows[approx_huge_offset + first_slot + __popcll(huge_mask & ((1ull << lane) - 1ull))] =
+              static_cast<int32_t>(my_u);
       }
     } else if (queued_mask) {
       // The exact update sums such a row in chunks of at most kChunkLen occurrences, like the uniform
@@ -1087,7 +1101,7 @@ void launch_update_mixed(const MixedArgs &a, const tbe_workspace_layout_t &l, ch
              go, w, st, psw, gpsw, a.table_offsets, a.table_dim_offsets, a.dim_offsets, a.T, mt.bag_magic, mt.bag_shift,
              a.total_D, i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
              i32(l.num_unique), wide_rows, static_cast<int32_t *>(nullptr), chunk_records, long_records, max_chunks,
-             max_long, static_cast<int>(ceil_div(a.n, kNumXcd)), a.lr, a.eps, a.sr, a.unique_slots, cr, a.slot_D);
+             max_long, static_cast<int>(ceil_div(a.n, kNumXcd)), a.lr, a.eps, a.sr, 0, a.unique_slots, cr, a.slot_D);
 
   const bool small = ceil_div(a.n, tile_positions(0)) < kSmallBatchTiles;
   const int64_t want_chunks = ceil_div(max_chunks, kWavesPerBlock);
@@ -1127,7 +1141,8 @@ void launch_update_mixed_approx(const MixedArgs &a, const tbe_workspace_layout_t
              i32(l.keys_sorted), i32(l.positions_sorted), i32(l.grad_rows), i32(l.segment_starts),
              i32(l.num_unique), approx_mixed_wide_queue(l, ws), approx_mixed_long_queue(l, ws),
              static_cast<ChunkRecord *>(nullptr), static_cast<LongRecord *>(nullptr), int64_t{0}, int64_t{0}, 1, a.lr,
-             a.eps, a.sr, a.unique_slots, static_cast<T *>(a.cache_rows), a.slot_D);
+             a.eps, a.sr, static_cast<int>(approx_mixed_huge_offset(a.n)), a.unique_slots,
+             static_cast<T *>(a.cache_rows), a.slot_D);
 }
 
 template <typename T, int VEC>

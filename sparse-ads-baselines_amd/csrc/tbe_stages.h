@@ -70,6 +70,7 @@ constexpr int kXcdCounterStride = 32;
 constexpr int kNumCounters = kXcdCounterBase + 8 * kXcdCounterStride;
 __host__ __device__ constexpr int xcd_counter(int xcd) { return kXcdCounterBase + kXcdCounterStride * xcd; }
 constexpr int kApproxHuge = 256;   // occurrences from which on the approximate update walks a row before the others
+constexpr int kApproxCoopD = 128;  // widest row that a whole workgroup walks (fp16 rows of more than kApproxHuge occurrences)
 // The short-row kernel's workgroups of XCD x own the segments that start in the x-th eighth of
 // the sorted positions (rounded up to whole workgroups: fewer than 1200 positions more) and queue
 // their chunk records in a region of their own.  Segments are consecutive, so only the last
@@ -203,6 +204,9 @@ int approx_update(const void *grad_output, void *weights, void *state, const voi
 inline int32_t *approx_mixed_long_queue(const tbe_workspace_layout_t &l, void *workspace) {
   return reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + l.chunk_segments);
 }
+// (behind the first queue's room, n / (kMixedShort + 1) + 1 rows: the fp16 rows of more than kApproxHuge
+// occurrences and at most kApproxCoopD elements, which a workgroup walks; counted in counters[xcd_counter(0)])
+inline int64_t approx_mixed_huge_offset(int64_t n) { return n / (kMixedShort + 1) + 1; }
 inline int32_t *approx_mixed_wide_queue(const tbe_workspace_layout_t &l, void *workspace) {
   return reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + l.segment_ids);
 }

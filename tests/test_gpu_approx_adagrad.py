@@ -571,3 +571,72 @@ def test_module_with_the_approximate_optimizer_and_repeated_rows(oracle):
     torch.cuda.synchronize()
     assert torch.equal(sd["embedding_weights"], plain.embedding_weights.data)
     assert torch.equal(sd["optimizer_state"], plain.optimizer_state)
+
+
+@pytest.mark.parametrize("stochastic", [False, True])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_approx_adagrad_mixed_D_fp16_rows_of_many_occurrences(oracle, weighted, stochastic):
+    """Mixed-D tables: fp16 rows of more than 256 occurrences and at most 128 elements are listed by the
+    strip kernel for a workgroup's walk (staged through LDS, or with the random bits drawn by the other
+    wavefronts), wider ones and rows of 9 ... 256 occurrences for a single wavefront's.  Tables of 8, 36,
+    64, 100, 128 (a workgroup), 256 (a wavefront) and 520 elements (the wide rows' kernel), each with rows
+    of 257 ... 2049 and of 17 ... 256 occurrences; gradients and weights chosen so that every sum is exact
+    (see _hot_row_problem): the state equals the oracle's bit for bit, the rows at the fp16 tolerance --
+    and, with round to nearest, a table of 64 columns comes out bit for bit as the same table does among
+    uniform tables for the rows that a walk takes there as well (more than 16 occurrences)."""
+    rs = np.random.RandomState(77)
+    dims = [8, 36, 64, 100, 128, 256, 520]
+    E, B, L = 60, 900, 8
+    tables = [(E, d) for d in dims]
+    T = len(tables)
+    p = make_mixed_problem(44, tables, B=B, L=L, dtype=np.float16, weighted=weighted)
+    hot, mid = [257, 384, 385, 1000, 2049], [17, 64, 65, 200, 256]
+    n_t = B * L
+    p["offsets"] = np.arange(0, T * n_t + 1, L, dtype=np.int32)
+    indices = np.empty(T * n_t, np.int32)
+    for t in range(T):
+        rows = np.concatenate([np.full(c, r, np.int32) for r, c in enumerate(hot + mid)])
+        rest = rs.randint(len(hot + mid), E, size=n_t - rows.size).astype(np.int32)
+        indices[t * n_t:(t + 1) * n_t] = rs.permutation(np.concatenate([rows, rest]))
+    p["indices"] = indices
+    total_D = int(p["dim_offsets"][-1])
+    p["grad_output"] = rs.choice(np.array([0, 0.5, -0.5, 1, -1], np.float16), size=(B, total_D))
+    psw = rs.choice(np.array([0.5, 1, 2], np.float16), size=T * n_t) if weighted else None
+    w = dev(p["weights"])
+    st_np = np.zeros(T * E, np.float32)
+    st = dev(st_np)
+    g = ext.backward_approx_adagrad_mixed_D(
+        dev(p["grad_output"]), w, dev(p["table_offsets"]), dev(p["table_dim_offsets"]), dev(p["dim_offsets"]), total_D,
+        dev(p["indices"]), dev(p["offsets"]), dev(psw) if weighted else None, st, 0.02, 0.1, 200, stochastic, 1)
+    w_ref = p["weights"].copy()
+    g_ref = oracle.backward_approx_mixed(p["grad_output"], w_ref, p["table_offsets"], p["table_dim_offsets"],
+                                         p["dim_offsets"], p["indices"], p["offsets"], 0.02, 0.1, st_np, psw)
+    assert st.cpu().numpy().tobytes() == st_np.tobytes()
+    got = w.cpu().numpy()
+    if stochastic:
+        # every update lands on one of the two fp16 neighbours of its exact value, so a row drifts from the
+        # round-to-nearest trajectory like a random walk of its occurrences: unbiased, and small
+        drift = got.astype(np.float64) - w_ref.astype(np.float64)
+        assert np.isfinite(drift).all() and np.abs(drift).max() < 0.5 and abs(drift.mean()) < 2e-3
+        assert (got.view(np.uint16) != w_ref.view(np.uint16)).mean() > 0.2   # and it is not round to nearest
+        return
+    assert_close(got, w_ref, 1e-2)
+    if weighted:
+        assert_close(g.cpu().numpy(), g_ref, 2e-2, "grad of per-sample weights")
+    # the table of 64 columns alone, as a uniform table
+    t = dims.index(64)
+    lo, hi = int(p["table_offsets"][t]), int(p["table_offsets"][t + 1])
+    c0 = int(p["dim_offsets"][t])
+    w_uni = dev(p["weights"][lo:hi].reshape(E, 64))
+    st_uni = torch.zeros(E, dtype=torch.float32, device=DEV)
+    ext.backward_approx_adagrad(
+        dev(np.ascontiguousarray(p["grad_output"][:, c0:c0 + 64]).reshape(B, 1, 64)), w_uni, dev(np.zeros(1, np.int32)),
+        dev(indices[t * n_t:(t + 1) * n_t].copy()), dev(np.arange(0, n_t + 1, L, dtype=np.int32)),
+        dev(psw[t * n_t:(t + 1) * n_t].copy()) if weighted else None, st_uni, 0.02, 0.1, 200, False, 1)
+    torch.cuda.synchronize()
+    assert st_uni.cpu().numpy().tobytes() == st_np[t * E:(t + 1) * E].tobytes()
+    counts = np.bincount(indices[t * n_t:(t + 1) * n_t], minlength=E)
+    walked = np.flatnonzero(counts > 16)
+    assert walked.size >= 10
+    mixed_rows = got[lo:hi].reshape(E, 64).view(np.uint16)
+    assert (mixed_rows[walked] == w_uni.cpu().numpy().view(np.uint16)[walked]).all()
