@@ -38,7 +38,9 @@ def _draw_batch(rs, tables, B, L, zipf):
 
 
 # narrow, odd vector counts, a table wider than 64 vectors (fp32: 520 / 4 = 130), hot rows in small tables
-TABLES = [(700, 8), (90, 36), (3000, 64), (40, 520), (5, 128), (1200, 20)]
+# (the table of one row: every lookup of its bags on the same row, several hundred per step -- several
+# chunks for the exact updates, a workgroup's walk for the approximate update of fp16 rows)
+TABLES = [(700, 8), (90, 36), (3000, 64), (40, 520), (5, 128), (1200, 20), (1, 64)]
 
 
 @pytest.mark.parametrize("mode,dtype", [("sgd", torch.float32), ("adagrad", torch.float32),
