@@ -640,3 +640,36 @@ def test_approx_adagrad_mixed_D_fp16_rows_of_many_occurrences(oracle, weighted, 
     assert walked.size >= 10
     mixed_rows = got[lo:hi].reshape(E, 64).view(np.uint16)
     assert (mixed_rows[walked] == w_uni.cpu().numpy().view(np.uint16)[walked]).all()
+
+
+@pytest.mark.parametrize("seed", range(18))
+def test_approx_adagrad_mixed_D_random_sweep(oracle, seed):
+    """Seeded random mixed-D table sets for the approximate update: 1..12 tables, from one row (every
+    lookup of a bag set on it: hundreds or thousands of occurrences, the workgroup walks for fp16 rows of
+    up to 128 elements, the single wavefront's otherwise) to thousands, widths from 4 to more than 64
+    vectors, with and without per-sample weights, all three types."""
+    rs = np.random.RandomState(800 + seed)
+    T = int(rs.choice([1, 2, 3, 6, 12]))
+    tables = [(int(rs.choice([1, 3, 40, 600, 5000])), int(rs.choice([4, 8, 12, 20, 32, 64, 100, 128, 256, 264, 520])))
+              for _ in range(T)]
+    dtype = [np.float16, np.float32, np.float64][seed % 3]
+    weighted = bool((seed // 3) % 2)
+    B = int(rs.choice([9, 70, 400]))
+    L = int(rs.choice([1, 5, 20]))
+    p = make_mixed_problem(60 + seed, tables, B=B, L=L, dtype=dtype, weighted=weighted)
+    w = dev(p["weights"])
+    st_np = np.zeros(sum(r for r, _ in tables), np.float64 if dtype == np.float64 else np.float32)
+    st = dev(st_np)
+    g = ext.backward_approx_adagrad_mixed_D(
+        dev(p["grad_output"]), w, dev(p["table_offsets"]), dev(p["table_dim_offsets"]), dev(p["dim_offsets"]),
+        int(p["dim_offsets"][-1]), dev(p["indices"]), dev(p["offsets"]), dev(p["per_sample_weights"]), st, 0.05, 0.1,
+        200, False, 1)
+    w_ref = p["weights"].copy()
+    g_ref = oracle.backward_approx_mixed(p["grad_output"], w_ref, p["table_offsets"], p["table_dim_offsets"],
+                                         p["dim_offsets"], p["indices"], p["offsets"], 0.05, 0.1, st_np,
+                                         p["per_sample_weights"])
+    tol = TOL[np.dtype(dtype)]
+    assert_close(st.cpu().numpy(), st_np, 1e-5 if dtype != np.float64 else 1e-10)
+    assert_close(w.cpu().numpy(), w_ref, tol)
+    if weighted:
+        assert_close(g.cpu().numpy(), g_ref, tol if dtype != np.float16 else 2e-2)
