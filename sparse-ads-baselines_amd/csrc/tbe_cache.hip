@@ -535,58 +535,78 @@ __global__ __launch_bounds__(kBlockThreads) void cache_commit_kernel(
   const int U = counters[0];
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kWavesPerBlock;
-  // 64 unique rows at a time are screened first, one per lane (most rows of a step are hits, or were
-  // fetched by the fill launch), then the wavefront takes the rows with work one after the other
+  // 64 unique rows at a time, one per lane: most rows of a step are hits, or were fetched by the fill
+  // launch; a lane whose row has work to do here describes it as one copy, or two for a swap (the
+  // new row into the slot, the slot's old content to the landing row or the backing table).  The
+  // wavefront then moves kCommitBatch rows at a time with every load issued before the first store,
+  // which is also what makes a swap through the same landing row correct.
+  constexpr int kCommitBatch = 4;
+  const int row_units = backing.row_units;
   for (int64_t base = wave_id * kWave; base < U; base += stride * kWave) {
     const int64_t mine = min(base + lane, static_cast<int64_t>(U) - 1);
-    const int32_t my_evicted = evicted_keys[mine];
-    const int32_t my_slot = unique_slots[mine];
-    const int32_t my_source = fetch_source[mine];
-    const bool my_by_fill =
-        my_source == -1 || (my_source >= old_stage_base && my_source < old_stage_base + stage_slots);
-    const bool idle = (my_evicted == -2 && (my_slot >= 0 || my_source < 0))  // a hit, or a row left in the table
-                      || (my_evicted != -2 && my_slot >= num_slots && my_by_fill);  // staged, and fetched already
-    unsigned long long todo = __ballot(base + lane < U && !idle);
-    for (; todo != 0ull; todo &= todo - 1ull) {
-      const int which = __ffsll(static_cast<long long>(todo)) - 1;
-      const int64_t i = base + which;
-      const int32_t evicted = __shfl(my_evicted, which, kWave);
-      const int64_t slot = __shfl(my_slot, which, kWave);
-      const int row_units = backing.row_units;
-      const int64_t source = __shfl(my_source, which, kWave);
-      const int64_t key = keys_sorted[segment_starts[i]];
-      const BackingRow home = backing_row(backing, key);
+    const int32_t evicted = evicted_keys[mine];
+    const int64_t slot = unique_slots[mine];
+    const int64_t source = fetch_source[mine];
+    const bool by_fill = source == -1 || (source >= old_stage_base && source < old_stage_base + stage_slots);
+    const bool idle = (evicted == -2 && (slot >= 0 || source < 0))        // a hit, or a row left in the table
+                      || (evicted != -2 && slot >= num_slots && by_fill);  // staged, and fetched already
+    const bool busy = base + lane < U && !idle;
+    const uint64_t *src0 = cache_rows, *src1 = cache_rows;  // (harmless sources for lanes without a copy)
+    uint64_t *dst0 = nullptr, *dst1 = nullptr;
+    int units0 = 0, units1 = 0;
+    if (busy) {
+      const BackingRow home = backing_row(backing, keys_sorted[segment_starts[mine]]);
+      units0 = home.units;
       if (evicted == -2) {
-        if (source >= 0) {
-          const uint64_t *src = cache_rows + source * row_units;
-          for (int k = lane; k < home.units; k += kWave) home.row[k] = src[k];
-        }
-        continue;
-      }
-      const bool by_fill = source == -1 || (source >= old_stage_base && source < old_stage_base + stage_slots);
-      const uint64_t *late_src = source >= 0 ? cache_rows + source * row_units : home.row;
-      if (slot >= num_slots) {
-        if (!by_fill) {
-          uint64_t *dst = cache_rows + slot * row_units;
-          for (int k = lane; k < home.units; k += kWave) dst[k] = late_src[k];
-        }
-        continue;
-      }
-      const int64_t land = landing[i];
-      uint64_t *slot_row = cache_rows + slot * row_units;
-      const uint64_t *new_row = (by_fill && land >= 0) ? cache_rows + land * row_units : late_src;
-      if (evicted >= 0) {
-        // (the evicted row may belong to a table of another width than the row that replaces it)
-        const BackingRow old_home = backing_row(backing, evicted);
-        uint64_t *old_row = land >= 0 ? cache_rows + land * row_units : old_home.row;
-        for (int k = lane; k < max(home.units, old_home.units); k += kWave) {
-          const uint64_t fresh = k < home.units ? new_row[k] : 0;
-          const uint64_t old = slot_row[k];
-          if (k < old_home.units) old_row[k] = old;
-          if (k < home.units) slot_row[k] = fresh;
-        }
+        // a row that stays in the backing table, whose newest value the last step left in a staging row
+        src0 = cache_rows + source * row_units;
+        dst0 = home.row;
       } else {
-        for (int k = lane; k < home.units; k += kWave) slot_row[k] = new_row[k];
+        const uint64_t *late_src = source >= 0 ? cache_rows + source * row_units : home.row;
+        if (slot >= num_slots) {
+          src0 = late_src;  // a staged row that the fill launch could not fetch yet
+          dst0 = cache_rows + slot * row_units;
+        } else {
+          const int64_t land = landing[mine];
+          uint64_t *slot_row = cache_rows + slot * row_units;
+          src0 = (by_fill && land >= 0) ? cache_rows + land * row_units : late_src;
+          dst0 = slot_row;
+          if (evicted >= 0) {
+            // (the evicted row may belong to a table of another width than the row that replaces it)
+            const BackingRow old_home = backing_row(backing, evicted);
+            src1 = slot_row;
+            dst1 = land >= 0 ? cache_rows + land * row_units : old_home.row;
+            units1 = old_home.units;
+          }
+        }
+      }
+    }
+    unsigned long long todo = __ballot(busy);
+    while (todo != 0ull) {
+      const uint64_t *src[2 * kCommitBatch];
+      uint64_t *dst[2 * kCommitBatch];
+      int units[2 * kCommitBatch];  // (0: no copy)
+      int most = 0;
+#pragma unroll
+      for (int j = 0; j < kCommitBatch; ++j) {
+        const int which = todo ? __ffsll(static_cast<long long>(todo)) - 1 : -1;
+        todo &= todo - (todo ? 1ull : 0ull);
+        const int from = max(which, 0);
+        src[2 * j] = reinterpret_cast<const uint64_t *>(__shfl(reinterpret_cast<unsigned long long>(src0), from, kWave));
+        dst[2 * j] = reinterpret_cast<uint64_t *>(__shfl(reinterpret_cast<unsigned long long>(dst0), from, kWave));
+        units[2 * j] = which >= 0 ? __shfl(units0, from, kWave) : 0;
+        src[2 * j + 1] = reinterpret_cast<const uint64_t *>(__shfl(reinterpret_cast<unsigned long long>(src1), from, kWave));
+        dst[2 * j + 1] = reinterpret_cast<uint64_t *>(__shfl(reinterpret_cast<unsigned long long>(dst1), from, kWave));
+        units[2 * j + 1] = which >= 0 ? __shfl(units1, from, kWave) : 0;
+        most = max(most, max(units[2 * j], units[2 * j + 1]));
+      }
+      for (int k = lane; k < most; k += kWave) {
+        uint64_t v[2 * kCommitBatch];
+#pragma unroll
+        for (int j = 0; j < 2 * kCommitBatch; ++j) v[j] = k < units[j] ? src[j][k] : 0;
+#pragma unroll
+        for (int j = 0; j < 2 * kCommitBatch; ++j)
+          if (k < units[j]) dst[j][k] = v[j];
       }
     }
   }
